@@ -1,0 +1,115 @@
+/*
+ * C interface of librnnt_hip.so: the RNN-T loss hot path on one MI355X (gfx950).
+ *
+ * Every pointer is a DEVICE pointer on the current HIP device unless stated otherwise; the
+ * caller owns all inputs and outputs.  Arrays are contiguous row-major with the reference's
+ * shapes (transducer/transducer.h:3-49):
+ *     emissions   float [B, T, V]          predictions float [B, U, V]   (U = longest label + 1)
+ *     labels      int   [B, U-1]           input_lengths, label_lengths  int [B]
+ *     log_norms, alphas, lngrads  float [B, T, U]     costs float [B]
+ * `stream` is a hipStream_t (NULL = the null stream, which is what the reference uses,
+ * transducer/transducer_cuda.cu:294-387).  Calls enqueue work and return without waiting.
+ *
+ * Return value: 0 on success, otherwise one of the RNNT_* codes below with a message available
+ * from rnnt_hip_last_error() on the calling thread.
+ */
+#ifndef RNNT_HIP_H_
+#define RNNT_HIP_H_
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* rnnt_stream_t;
+
+enum {
+  RNNT_OK = 0,
+  RNNT_INVALID_ARGUMENT = 1, /* bad sizes or a missing pointer */
+  RNNT_HIP_FAILURE = 2,      /* a HIP runtime call failed; message holds "[file:line] HIP error: ..." */
+  RNNT_WORKSPACE_TOO_SMALL = 3
+};
+
+const char* rnnt_hip_last_error(void);
+int rnnt_hip_abi_version(void);
+
+/* ---- the three entry points of the reference, device side ------------------------------- */
+
+/* Replaces cuda::forward (transducer/transducer_cuda.h:14-27, transducer_cuda.cu:280-307):
+ * alpha recursion with caller-supplied log_norms.  Writes costs[B] and the alphas of the cells
+ * inside each utterance's (input_length, label_length+1) extent; other cells are untouched.
+ * An utterance with input_length 0 gets cost +inf. */
+int rnnt_hip_forward(const float* emissions, const float* predictions, float* costs,
+                     float* alphas, const float* log_norms, const int* labels,
+                     const int* input_lengths, const int* label_lengths, int B, int T, int U,
+                     int V, int blank, rnnt_stream_t stream);
+
+/* Replaces cuda::backward (transducer/transducer_cuda.h:29-44, transducer_cuda.cu:309-347):
+ * zero-fills egrads, pgrads and lngrads, then writes lngrads = d cost / d log_norms and the
+ * sparse blank/label terms of egrads and pgrads. */
+int rnnt_hip_backward(const float* emissions, const float* predictions, float* egrads,
+                      float* pgrads, float* lngrads, const float* alphas, const float* log_norms,
+                      const int* labels, const int* input_lengths, const int* label_lengths,
+                      int B, int T, int U, int V, int blank, rnnt_stream_t stream);
+
+/* Replaces cuda::viterbi (transducer/transducer_cuda.h:46-57, transducer_cuda.cu:349-388):
+ * best label sequence of the given lengths with caller-supplied log_norms.  Writes the first
+ * label_lengths[b] entries of labels[b]; the rest are untouched.  Pointers may be NULL when
+ * T == 0, labels may be NULL when U == 1 (transducer/test.cpp:229-257). */
+int rnnt_hip_viterbi(const float* emissions, const float* predictions, const float* log_norms,
+                     int* labels, const int* input_lengths, const int* label_lengths, int B,
+                     int T, int U, int V, int blank, rnnt_stream_t stream);
+
+/* ---- the parts the reference computes with torch ops ------------------------------------ */
+
+/* Replaces transducer/torch_binding.py:35-40 (and :162-167):
+ * log_norms[b,t,u] = log sum_v exp(emissions[b,t,v] + predictions[b,u,v]).
+ * input_lengths / label_lengths may be NULL (every cell is computed, as torch does); when given,
+ * cells outside an utterance's extent are written as 0 (transducer/test.h:51-80). */
+int rnnt_hip_log_norms(const float* emissions, const float* predictions, float* log_norms,
+                       const int* input_lengths, const int* label_lengths, int B, int T, int U,
+                       int V, rnnt_stream_t stream);
+
+/* Replaces transducer/torch_binding.py:85-89: adds the dense softmax part
+ * sum_u lngrads[b,t,u]*softmax(b,t,u)[v] (resp. sum_t) to what egrads / pgrads hold (the sparse
+ * terms rnnt_hip_backward left there) and multiplies the result by deltas[b].
+ * deltas may be NULL (= 1).  Frames and label positions outside an utterance stay exactly 0. */
+int rnnt_hip_dense_grads(const float* emissions, const float* predictions, float* egrads,
+                         float* pgrads, const float* lngrads, const float* log_norms,
+                         const float* deltas, const int* input_lengths, const int* label_lengths,
+                         int B, int T, int U, int V, rnnt_stream_t stream);
+
+/* ---- whole loss, as TransducerLoss uses it ---------------------------------------------- */
+
+/* Device bytes rnnt_hip_loss_forward/backward need between them; O(B*T*U) + O(B*(T+U)). */
+size_t rnnt_hip_loss_workspace_bytes(int B, int T, int U, int V);
+
+/* Replaces Transducer.forward (transducer/torch_binding.py:25-58): log-normaliser + alpha.
+ * `workspace` (>= rnnt_hip_loss_workspace_bytes, 256-byte aligned) must stay untouched until
+ * the matching rnnt_hip_loss_backward has run; it plays the role of the tensors the reference
+ * saves for backward, without any [B,T,V]-sized entry. */
+int rnnt_hip_loss_forward(const float* emissions, const float* predictions, const int* labels,
+                          const int* input_lengths, const int* label_lengths, float* costs,
+                          void* workspace, size_t workspace_bytes, int B, int T, int U, int V,
+                          int blank, rnnt_stream_t stream);
+
+/* Replaces Transducer.backward (transducer/torch_binding.py:60-90): full egrads[B,T,V] and
+ * pgrads[B,U,V] (sparse + dense parts, times deltas[b]); every element is written. */
+int rnnt_hip_loss_backward(const float* emissions, const float* predictions, const int* labels,
+                           const int* input_lengths, const int* label_lengths,
+                           const float* deltas, float* egrads, float* pgrads, void* workspace,
+                           size_t workspace_bytes, int B, int T, int U, int V, int blank,
+                           rnnt_stream_t stream);
+
+/* Replaces TransducerLoss.viterbi (transducer/torch_binding.py:130-177): log-normaliser +
+ * best path.  labels is int [B, U-1]. */
+int rnnt_hip_viterbi_decode(const float* emissions, const float* predictions,
+                            const int* input_lengths, const int* label_lengths, int* labels,
+                            int B, int T, int U, int V, int blank, rnnt_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* RNNT_HIP_H_ */

@@ -1,0 +1,340 @@
+// extern "C" entry points of librnnt_hip.so (declared in include/rnnt_hip.h): argument checks,
+// stream-ordered scratch, and the kernel sequences.  No torch types, no exceptions.
+#include <stdarg.h>
+#include <stdio.h>
+
+#include "../../include/rnnt_hip.h"
+#include "rnnt_internal.h"
+
+namespace rnnt {
+
+static thread_local char g_error[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+// Message format follows the reference's CUDA_CHECK (transducer/transducer_cuda.cu:271-278).
+int check_hip(hipError_t e, const char* what, const char* file, int line) {
+  if (e == hipSuccess) return kOk;
+  return fail(kHipError, "[%s:%d] HIP error: %s (%s)", file, line, hipGetErrorString(e), what);
+}
+
+namespace {
+
+size_t align_up(size_t x) { return (x + 255) & ~(size_t)255; }
+
+// One stream-ordered allocation carved into pieces; released on the same stream.
+class Scratch {
+ public:
+  explicit Scratch(hipStream_t s) : stream_(s) {}
+  ~Scratch() {
+    if (base_) (void)hipFreeAsync(base_, stream_);
+  }
+  int reserve(size_t bytes) {
+    if (bytes == 0) return kOk;
+    RNNT_HIP(hipMallocAsync(&base_, bytes, stream_));
+    size_ = bytes;
+    return kOk;
+  }
+  void* take(size_t bytes) {
+    void* p = static_cast<char*>(base_) + used_;
+    used_ += align_up(bytes);
+    return p;
+  }
+  size_t used() const { return used_; }
+  size_t size() const { return size_; }
+
+ private:
+  hipStream_t stream_;
+  void* base_ = nullptr;
+  size_t size_ = 0, used_ = 0;
+};
+
+int check_dims(int B, int T, int U, int V) {
+  if (B < 0 || T < 0 || U < 0 || V < 0)
+    return fail(kInvalid, "negative size (B=%d T=%d U=%d V=%d)", B, T, U, V);
+  if ((long long)T * V >= (1ll << 31) || (long long)U * V >= (1ll << 31) ||
+      (long long)T * U >= (1ll << 31))
+    return fail(kInvalid, "one utterance's T*V, U*V or T*U exceeds 2^31 elements");
+  return kOk;
+}
+
+bool nothing_to_do(int B, int T, int U) { return B == 0 || T == 0 || U == 0; }
+
+struct LossWorkspace {
+  Planes planes;
+  float *mE, *mP, *LN, *lngrads, *Wn, *Wt;
+};
+
+size_t loss_workspace_layout(const Dims& d, void* base, LossWorkspace* w) {
+  char* c = static_cast<char*>(base);
+  size_t off = 0;
+  auto take = [&](size_t bytes) {
+    float* p = base ? reinterpret_cast<float*>(c + off) : nullptr;
+    off += align_up(bytes);
+    return p;
+  };
+  const size_t pb = planes_bytes(d);
+  void* pl = take(pb);
+  if (base) carve_planes(pl, d, &w->planes);
+  const size_t btu = sizeof(float) * (size_t)d.B * d.T * d.U;
+  float* mE = take(sizeof(float) * (size_t)d.B * d.T);
+  float* mP = take(sizeof(float) * (size_t)d.B * d.U);
+  float* LN = take(btu);
+  float* lng = take(btu);
+  const size_t wb = sizeof(float) * (size_t)d.B * wplane_tw(d.T) * wplane_up(d.U);
+  float* Wn = take(wb);
+  float* Wt = take(wb);
+  if (base) { w->mE = mE; w->mP = mP; w->LN = LN; w->lngrads = lng; w->Wn = Wn; w->Wt = Wt; }
+  return off;
+}
+
+// cost = +inf for every utterance when the padded frame axis is empty (transducer_cpu.cpp:39-41)
+__global__ void fill_kernel(float* x, float v, int n) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i < n) x[i] = v;
+}
+
+int fill(float* x, float v, int n, hipStream_t s) {
+  if (n == 0) return kOk;
+  hipLaunchKernelGGL(fill_kernel, dim3((n + 255) / 256), dim3(256), 0, s, x, v, n);
+  return check_hip(hipGetLastError(), "launch fill_kernel", __FILE__, __LINE__);
+}
+
+}  // namespace
+}  // namespace rnnt
+
+using namespace rnnt;
+
+extern "C" {
+
+const char* rnnt_hip_last_error(void) { return g_error; }
+int rnnt_hip_abi_version(void) { return 1; }
+
+int rnnt_hip_forward(const float* E, const float* P, float* costs, float* alphas, const float* LN,
+                     const int* labels, const int* inLen, const int* labLen, int B, int T, int U,
+                     int V, int blank, rnnt_stream_t stream) {
+  RNNT_TRY(check_dims(B, T, U, V));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (B == 0) return kOk;
+  if (!costs || !inLen || !labLen) return fail(kInvalid, "forward: null costs or lengths");
+  if (nothing_to_do(B, T, U)) return fill(costs, __builtin_huge_valf(), B, s);
+  if (!E || !P || !alphas || !LN || (U > 1 && !labels))
+    return fail(kInvalid, "forward: null array argument");
+  const Dims d = make_dims(B, T, U, V, blank);
+  Scratch scratch(s);
+  RNNT_TRY(scratch.reserve(planes_bytes(d)));
+  Planes p;
+  carve_planes(scratch.take(planes_bytes(d)), d, &p);
+  RNNT_TRY(launch_skew(LN, p.lnS, inLen, labLen, d, s));
+  RNNT_TRY(launch_gather(E, P, labels, inLen, labLen, p, d, s));
+  RNNT_TRY(launch_alpha(p, inLen, labLen, costs, d, s));
+  RNNT_TRY(launch_unskew(p.aS, alphas, inLen, labLen, d, s));
+  return kOk;
+}
+
+int rnnt_hip_backward(const float* E, const float* P, float* egrads, float* pgrads, float* lngrads,
+                      const float* alphas, const float* LN, const int* labels, const int* inLen,
+                      const int* labLen, int B, int T, int U, int V, int blank,
+                      rnnt_stream_t stream) {
+  RNNT_TRY(check_dims(B, T, U, V));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (B == 0) return kOk;
+  // transducer_cuda.cu:326-331: the library clears all three outputs itself
+  if (egrads && (size_t)T * V) RNNT_HIP(hipMemsetAsync(egrads, 0, sizeof(float) * (size_t)B * T * V, s));
+  if (pgrads && (size_t)U * V) RNNT_HIP(hipMemsetAsync(pgrads, 0, sizeof(float) * (size_t)B * U * V, s));
+  if (lngrads && (size_t)T * U) RNNT_HIP(hipMemsetAsync(lngrads, 0, sizeof(float) * (size_t)B * T * U, s));
+  if (nothing_to_do(B, T, U) || V == 0) return kOk;
+  if (!E || !P || !egrads || !pgrads || !lngrads || !alphas || !LN || !inLen || !labLen ||
+      (U > 1 && !labels))
+    return fail(kInvalid, "backward: null array argument");
+  const Dims d = make_dims(B, T, U, V, blank);
+  Scratch scratch(s);
+  RNNT_TRY(scratch.reserve(planes_bytes(d)));
+  Planes p;
+  carve_planes(scratch.take(planes_bytes(d)), d, &p);
+  RNNT_TRY(launch_skew(LN, p.lnS, inLen, labLen, d, s));
+  RNNT_TRY(launch_skew(alphas, p.aS, inLen, labLen, d, s));
+  RNNT_TRY(launch_gather(E, P, labels, inLen, labLen, p, d, s));
+  RNNT_TRY(launch_weights(p, inLen, labLen, d, s));
+  RNNT_TRY(launch_beta(p, labels, inLen, labLen, d, s));
+  RNNT_TRY(launch_unskew(p.dS, lngrads, inLen, labLen, d, s));
+  RNNT_TRY(launch_sparse(p, egrads, pgrads, labels, inLen, labLen, nullptr, false, d, s));
+  return kOk;
+}
+
+static int viterbi_impl(const float* E, const float* P, const float* LN, int* labels,
+                        const int* inLen, const int* labLen, const Dims& d, hipStream_t s) {
+  const size_t btu = sizeof(float) * (size_t)d.B * d.T * d.U;
+  const size_t plane = sizeof(float) * (size_t)d.B * d.U * d.Dp + 64;
+  Scratch scratch(s);
+  RNNT_TRY(scratch.reserve(align_up(planes_bytes(d)) + 2 * align_up(btu) + 2 * align_up(plane) +
+                           align_up(viterbi_bits_bytes(d))));
+  Planes p;
+  carve_planes(scratch.take(planes_bytes(d)), d, &p);
+  float* best = static_cast<float*>(scratch.take(btu));
+  int* arg = static_cast<int*>(scratch.take(btu));
+  float* bestS = static_cast<float*>(scratch.take(plane));
+  float* argS = static_cast<float*>(scratch.take(plane));
+  unsigned long long* bits =
+      static_cast<unsigned long long*>(scratch.take(viterbi_bits_bytes(d)));
+  RNNT_TRY(launch_maxplus(E, P, inLen, labLen, best, arg, d, s));
+  RNNT_TRY(launch_skew(LN, p.lnS, inLen, labLen, d, s));
+  RNNT_TRY(launch_skew(best, bestS, inLen, labLen, d, s));
+  RNNT_TRY(launch_skew(reinterpret_cast<const float*>(arg), argS, inLen, labLen, d, s));
+  // blank scores only: the label planes of the gather are not needed here
+  RNNT_TRY(launch_gather(E, P, nullptr, inLen, labLen, p, d, s));
+  RNNT_TRY(launch_viterbi(p, bestS, argS, bits, inLen, labLen, labels, d, s));
+  return kOk;
+}
+
+int rnnt_hip_viterbi(const float* E, const float* P, const float* LN, int* labels,
+                     const int* inLen, const int* labLen, int B, int T, int U, int V, int blank,
+                     rnnt_stream_t stream) {
+  RNNT_TRY(check_dims(B, T, U, V));
+  if (nothing_to_do(B, T, U) || U == 1) return kOk;  // no label to emit
+  if (!E || !P || !LN || !labels || !inLen || !labLen)
+    return fail(kInvalid, "viterbi: null array argument");
+  return viterbi_impl(E, P, LN, labels, inLen, labLen, make_dims(B, T, U, V, blank),
+                      static_cast<hipStream_t>(stream));
+}
+
+int rnnt_hip_log_norms(const float* E, const float* P, float* LN, const int* inLen,
+                       const int* labLen, int B, int T, int U, int V, rnnt_stream_t stream) {
+  RNNT_TRY(check_dims(B, T, U, V));
+  if (nothing_to_do(B, T, U)) return kOk;
+  if (!E || !P || !LN) return fail(kInvalid, "log_norms: null array argument");
+  if (V == 0) return fail(kInvalid, "log_norms: empty vocabulary");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const Dims d = make_dims(B, T, U, V, 0);
+  Scratch scratch(s);
+  RNNT_TRY(scratch.reserve(align_up(sizeof(float) * (size_t)B * T) +
+                           align_up(sizeof(float) * (size_t)B * U)));
+  float* mE = static_cast<float*>(scratch.take(sizeof(float) * (size_t)B * T));
+  float* mP = static_cast<float*>(scratch.take(sizeof(float) * (size_t)B * U));
+  RNNT_TRY(launch_rowmax(E, mE, (long)B * T, V, s));
+  RNNT_TRY(launch_rowmax(P, mP, (long)B * U, V, s));
+  RNNT_TRY(launch_lse(E, P, mE, mP, LN, inLen, labLen, d, s));
+  return kOk;
+}
+
+int rnnt_hip_dense_grads(const float* E, const float* P, float* egrads, float* pgrads,
+                         const float* lngrads, const float* LN, const float* deltas,
+                         const int* inLen, const int* labLen, int B, int T, int U, int V,
+                         rnnt_stream_t stream) {
+  RNNT_TRY(check_dims(B, T, U, V));
+  if (nothing_to_do(B, T, U) || V == 0) return kOk;
+  if (!E || !P || !egrads || !pgrads || !lngrads || !LN)
+    return fail(kInvalid, "dense_grads: null array argument");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const Dims d = make_dims(B, T, U, V, 0);
+  const size_t wb = sizeof(float) * (size_t)B * wplane_tw(T) * wplane_up(U);
+  Scratch scratch(s);
+  RNNT_TRY(scratch.reserve(align_up(sizeof(float) * (size_t)B * T) +
+                           align_up(sizeof(float) * (size_t)B * U) + 2 * align_up(wb)));
+  float* mE = static_cast<float*>(scratch.take(sizeof(float) * (size_t)B * T));
+  float* mP = static_cast<float*>(scratch.take(sizeof(float) * (size_t)B * U));
+  float* Wn = static_cast<float*>(scratch.take(wb));
+  float* Wt = static_cast<float*>(scratch.take(wb));
+  RNNT_TRY(launch_rowmax(E, mE, (long)B * T, V, s));
+  RNNT_TRY(launch_rowmax(P, mP, (long)B * U, V, s));
+  RNNT_TRY(launch_wplanes(lngrads, LN, mE, mP, Wn, Wt, inLen, labLen, d, s));
+  RNNT_TRY(launch_egrads(E, P, mE, mP, Wn, deltas, egrads, inLen, labLen, d, true, s));
+  RNNT_TRY(launch_pgrads(E, P, mE, mP, Wt, deltas, pgrads, inLen, labLen, d, true, s));
+  return kOk;
+}
+
+size_t rnnt_hip_loss_workspace_bytes(int B, int T, int U, int V) {
+  if (B <= 0 || T <= 0 || U <= 0 || V <= 0) return 256;
+  const Dims d = make_dims(B, T, U, V, 0);
+  return loss_workspace_layout(d, nullptr, nullptr) + 256;
+}
+
+int rnnt_hip_loss_forward(const float* E, const float* P, const int* labels, const int* inLen,
+                          const int* labLen, float* costs, void* workspace, size_t workspace_bytes,
+                          int B, int T, int U, int V, int blank, rnnt_stream_t stream) {
+  RNNT_TRY(check_dims(B, T, U, V));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (B == 0) return kOk;
+  if (!costs || !inLen || !labLen) return fail(kInvalid, "loss_forward: null costs or lengths");
+  if (nothing_to_do(B, T, U)) return fill(costs, __builtin_huge_valf(), B, s);
+  if (V == 0) return fail(kInvalid, "loss_forward: empty vocabulary");
+  if (!E || !P || (U > 1 && !labels)) return fail(kInvalid, "loss_forward: null array argument");
+  if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & 255))
+    return fail(kInvalid, "loss_forward: workspace must be a 256-byte aligned device pointer");
+  if (workspace_bytes < rnnt_hip_loss_workspace_bytes(B, T, U, V))
+    return fail(kWorkspace, "loss_forward: workspace of %zu bytes, %zu needed", workspace_bytes,
+                rnnt_hip_loss_workspace_bytes(B, T, U, V));
+  const Dims d = make_dims(B, T, U, V, blank);
+  LossWorkspace w;
+  loss_workspace_layout(d, workspace, &w);
+  RNNT_TRY(launch_rowmax(E, w.mE, (long)B * T, V, s));
+  RNNT_TRY(launch_rowmax(P, w.mP, (long)B * U, V, s));
+  RNNT_TRY(launch_lse(E, P, w.mE, w.mP, w.LN, inLen, labLen, d, s));
+  RNNT_TRY(launch_skew(w.LN, w.planes.lnS, inLen, labLen, d, s));
+  RNNT_TRY(launch_gather(E, P, labels, inLen, labLen, w.planes, d, s));
+  RNNT_TRY(launch_alpha(w.planes, inLen, labLen, costs, d, s));
+  return kOk;
+}
+
+int rnnt_hip_loss_backward(const float* E, const float* P, const int* labels, const int* inLen,
+                           const int* labLen, const float* deltas, float* egrads, float* pgrads,
+                           void* workspace, size_t workspace_bytes, int B, int T, int U, int V,
+                           int blank, rnnt_stream_t stream) {
+  RNNT_TRY(check_dims(B, T, U, V));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (B == 0 || V == 0) return kOk;
+  if (nothing_to_do(B, T, U)) {
+    if (egrads && (size_t)T * V) RNNT_HIP(hipMemsetAsync(egrads, 0, sizeof(float) * (size_t)B * T * V, s));
+    if (pgrads && (size_t)U * V) RNNT_HIP(hipMemsetAsync(pgrads, 0, sizeof(float) * (size_t)B * U * V, s));
+    return kOk;
+  }
+  if (!E || !P || !egrads || !pgrads || !inLen || !labLen || (U > 1 && !labels))
+    return fail(kInvalid, "loss_backward: null array argument");
+  if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & 255))
+    return fail(kInvalid, "loss_backward: workspace must be a 256-byte aligned device pointer");
+  if (workspace_bytes < rnnt_hip_loss_workspace_bytes(B, T, U, V))
+    return fail(kWorkspace, "loss_backward: workspace of %zu bytes, %zu needed", workspace_bytes,
+                rnnt_hip_loss_workspace_bytes(B, T, U, V));
+  const Dims d = make_dims(B, T, U, V, blank);
+  LossWorkspace w;
+  loss_workspace_layout(d, workspace, &w);
+  RNNT_TRY(launch_weights(w.planes, inLen, labLen, d, s));
+  RNNT_TRY(launch_beta(w.planes, labels, inLen, labLen, d, s));
+  RNNT_TRY(launch_unskew(w.planes.dS, w.lngrads, inLen, labLen, d, s));
+  RNNT_TRY(launch_wplanes(w.lngrads, w.LN, w.mE, w.mP, w.Wn, w.Wt, inLen, labLen, d, s));
+  RNNT_TRY(launch_egrads(E, P, w.mE, w.mP, w.Wn, deltas, egrads, inLen, labLen, d, false, s));
+  RNNT_TRY(launch_pgrads(E, P, w.mE, w.mP, w.Wt, deltas, pgrads, inLen, labLen, d, false, s));
+  RNNT_TRY(launch_sparse(w.planes, egrads, pgrads, labels, inLen, labLen, deltas, true, d, s));
+  return kOk;
+}
+
+int rnnt_hip_viterbi_decode(const float* E, const float* P, const int* inLen, const int* labLen,
+                            int* labels, int B, int T, int U, int V, int blank,
+                            rnnt_stream_t stream) {
+  RNNT_TRY(check_dims(B, T, U, V));
+  if (nothing_to_do(B, T, U) || U == 1) return kOk;
+  if (V == 0) return fail(kInvalid, "viterbi_decode: empty vocabulary");
+  if (!E || !P || !labels || !inLen || !labLen)
+    return fail(kInvalid, "viterbi_decode: null array argument");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const Dims d = make_dims(B, T, U, V, blank);
+  Scratch scratch(s);
+  const size_t btu = sizeof(float) * (size_t)B * T * U;
+  RNNT_TRY(scratch.reserve(align_up(sizeof(float) * (size_t)B * T) +
+                           align_up(sizeof(float) * (size_t)B * U) + align_up(btu)));
+  float* mE = static_cast<float*>(scratch.take(sizeof(float) * (size_t)B * T));
+  float* mP = static_cast<float*>(scratch.take(sizeof(float) * (size_t)B * U));
+  float* LN = static_cast<float*>(scratch.take(btu));
+  RNNT_TRY(launch_rowmax(E, mE, (long)B * T, V, s));
+  RNNT_TRY(launch_rowmax(P, mP, (long)B * U, V, s));
+  RNNT_TRY(launch_lse(E, P, mE, mP, LN, inLen, labLen, d, s));
+  return viterbi_impl(E, P, LN, labels, inLen, labLen, d, s);
+}
+
+}  // extern "C"

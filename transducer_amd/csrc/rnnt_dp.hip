@@ -1,0 +1,767 @@
+// Lattice recursions of the RNN-T loss for gfx950: alpha, dalpha and the viterbi best path,
+// plus the small data-movement kernels that feed them.
+//
+// One wavefront walks one utterance's (t,u) lattice along anti-diagonals.  Lane L owns C
+// consecutive label positions u = L*C .. L*C+C-1 and, at step s, the cells (t = s-u, u).  A
+// finished cell pushes two scores forward, with the reference's exact association
+// (transducer/transducer_cpu.cpp:45-48, 61-69):
+//     stay(t,u) = ((x + E[t,blank]) + P[u,blank]) - LN[t,u]   -> consumed by (t+1,u), same lane
+//     emit(t,u) = ((x + E[t,l_u])   + P[u,l_u])   - LN[t,u]   -> consumed by (t,u+1)
+// The hand-over to the next label position stays in registers inside a lane and crosses lanes
+// with one DPP wave shift; there is no barrier and no memory access on the dependent chain.
+// Operands are read from "skewed" planes [u][t+u] so that four steps are one 16-byte load per
+// lane, prefetched a group ahead.  This file is compiled with -ffp-contract=off: the rounding
+// sequence of every cell must equal the reference's.
+#include "rnnt_internal.h"
+
+namespace rnnt {
+
+namespace {
+
+constexpr float kNegInf = -__builtin_huge_valf();
+constexpr float kPosInf = __builtin_huge_valf();
+
+// lane L receives the value of lane L-1; lane 0 receives `fill`.
+__device__ inline float wave_shr1(float x, float fill) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(fill), __float_as_int(x),
+                                                    0x138 /* wave_shr:1 */, 0xf, 0xf, false));
+}
+// lane L receives the value of lane L+1; lane 63 receives `fill`.
+__device__ inline float wave_shl1(float x, float fill) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(fill), __float_as_int(x),
+                                                    0x130 /* wave_shl:1 */, 0xf, 0xf, false));
+}
+
+// log1p(y) for y in [0,1]:  log(1+y) with the rounding error of the sum 1+y folded back in.
+// Within about one ulp of the correctly rounded value over the whole range.
+__device__ inline float log1p_unit(float y) {
+  const float w = 1.0f + y;
+  const float lost = y - (w - 1.0f);
+  return logf(w) + lost / w;
+}
+
+// transducer/transducer_cpu.cpp:16-24
+__device__ inline float lse2(float a, float b) {
+  const float hi = fmaxf(a, b);
+  float r = hi + log1p_unit(expf(-fabsf(a - b)));
+  r = (b == kNegInf) ? a : r;
+  r = (a == kNegInf) ? b : r;
+  return r;
+}
+
+__device__ inline float f4get(const float4& v, int j) {
+  return j == 0 ? v.x : (j == 1 ? v.y : (j == 2 ? v.z : v.w));
+}
+__device__ inline void f4set(float4& v, int j, float x) {
+  if (j == 0) v.x = x; else if (j == 1) v.y = x; else if (j == 2) v.z = x; else v.w = x;
+}
+
+// ------------------------------------------------------------------ skew / unskew
+// row-major [B,T,U] <-> skewed [B,U,Dp]; 64x64 tiles transposed through LDS so both sides
+// move whole cache lines.  Only cells inside the utterance's (T_b, U_b) extent are touched.
+__global__ __launch_bounds__(256) void skew_kernel(const float* __restrict__ src,
+                                                   float* __restrict__ dstS,
+                                                   const int* __restrict__ inLen,
+                                                   const int* __restrict__ labLen, Dims d) {
+  __shared__ float tile[64][65];
+  const int b = blockIdx.z, t0 = blockIdx.x * 64, u0 = blockIdx.y * 64;
+  int Tb, Ub;
+  utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
+  if (t0 >= Tb || u0 >= Ub) return;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  const float* s = src + (size_t)b * d.T * d.U;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int t = t0 + ty + 4 * i, u = u0 + tx;
+    tile[ty + 4 * i][tx] = (t < Tb && u < Ub) ? s[(size_t)t * d.U + u] : 0.0f;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int u = u0 + ty + 4 * i, t = t0 + tx;
+    if (t < Tb && u < Ub) dstS[((size_t)b * d.U + u) * d.Dp + t + u] = tile[tx][ty + 4 * i];
+  }
+}
+
+__global__ __launch_bounds__(256) void unskew_kernel(const float* __restrict__ srcS,
+                                                     float* __restrict__ dst,
+                                                     const int* __restrict__ inLen,
+                                                     const int* __restrict__ labLen, Dims d) {
+  __shared__ float tile[64][65];
+  const int b = blockIdx.z, t0 = blockIdx.x * 64, u0 = blockIdx.y * 64;
+  int Tb, Ub;
+  utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
+  if (t0 >= Tb || u0 >= Ub) return;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int u = u0 + ty + 4 * i, t = t0 + tx;
+    tile[ty + 4 * i][tx] =
+        (t < Tb && u < Ub) ? srcS[((size_t)b * d.U + u) * d.Dp + t + u] : 0.0f;
+  }
+  __syncthreads();
+  float* o = dst + (size_t)b * d.T * d.U;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int t = t0 + ty + 4 * i, u = u0 + tx;
+    if (t < Tb && u < Ub) o[(size_t)t * d.U + u] = tile[tx][ty + 4 * i];
+  }
+}
+
+// ------------------------------------------------------------------ gather
+// elS[u][t+u] = E[t, label_u]; eb[t] = E[t, blank]; pb[u] = P[u, blank]; pl[u] = P[u, label_u].
+// grid (ceil(T/256), U, B): a block serves 256 frames of one label position.
+__global__ __launch_bounds__(256) void gather_kernel(const float* __restrict__ E,
+                                                     const float* __restrict__ P,
+                                                     const int* __restrict__ labels,
+                                                     const int* __restrict__ inLen,
+                                                     const int* __restrict__ labLen, Planes p,
+                                                     Dims d) {
+  const int b = blockIdx.z, u = blockIdx.y;
+  const int t = blockIdx.x * 256 + threadIdx.x;
+  int Tb, Ub;
+  utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
+  if (u >= Ub) return;
+  const bool has_label = labels != nullptr && (u + 1 < Ub);
+  const int l = has_label ? labels[(size_t)b * (d.U - 1) + u] : d.blank;
+  const float* Eb = E + (size_t)b * d.T * d.V;
+  if (t < Tb) {
+    if (has_label) p.elS[((size_t)b * d.U + u) * d.Dp + t + u] = Eb[(size_t)t * d.V + l];
+    if (u == 0) p.eb[(size_t)b * d.Tp + t] = Eb[(size_t)t * d.V + d.blank];
+  }
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    const float* Pu = P + ((size_t)b * d.U + u) * d.V;
+    p.pb[(size_t)b * d.U + u] = Pu[d.blank];
+    p.pl[(size_t)b * d.U + u] = has_label ? Pu[l] : 0.0f;
+  }
+}
+
+// ------------------------------------------------------------------ alpha
+// transducer/transducer_cpu.cpp:30-79 (one utterance per wavefront).
+template <int C>
+__global__ __launch_bounds__(64) void alpha_kernel(Planes p, const int* __restrict__ inLen,
+                                                   const int* __restrict__ labLen,
+                                                   float* __restrict__ costs, Dims d) {
+  const int b = blockIdx.x, lane = threadIdx.x;
+  int Tb, Ub;
+  utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
+  if (Tb == 0 || Ub == 0) {  // :39-41
+    if (lane == 0) costs[b] = kPosInf;
+    return;
+  }
+  const int nsteps = Tb + Ub - 1;
+  const int ngroups = (nsteps + 3) >> 2;
+  const float* ebp = p.eb + (size_t)b * d.Tp;
+
+  float stay[C], emit[C], pbv[C], plv[C];
+  const float* lnp[C];
+  const float* elp[C];
+  float* ap[C];
+#pragma unroll
+  for (int c = 0; c < C; ++c) {
+    const int u = lane * C + c, uc = u < d.U ? u : d.U - 1;
+    const size_t row = ((size_t)b * d.U + uc) * d.Dp;
+    lnp[c] = p.lnS + row;
+    elp[c] = p.elS + row;
+    ap[c] = p.aS + row;
+    pbv[c] = p.pb[(size_t)b * d.U + uc];
+    plv[c] = p.pl[(size_t)b * d.U + uc];
+    stay[c] = kNegInf;  // "no predecessor": lse2 then returns the other operand unchanged
+    emit[c] = kNegInf;
+  }
+
+  float4 ln4[C], el4[C];
+  float eb4[C][4];
+  auto load_group = [&](int g, float4* ln, float4* el, float (*ebv)[4]) {
+#pragma unroll
+    for (int c = 0; c < C; ++c) {
+      ln[c] = *reinterpret_cast<const float4*>(lnp[c] + 4 * g);
+      el[c] = *reinterpret_cast<const float4*>(elp[c] + 4 * g);
+      const int u = lane * C + c;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) ebv[c][j] = ebp[clampi(4 * g + j - u, 0, Tb - 1)];
+    }
+  };
+  load_group(0, ln4, el4, eb4);
+
+  for (int g = 0; g < ngroups; ++g) {
+    float4 ln4n[C], el4n[C];
+    float eb4n[C][4];
+    load_group(g + 1 < ngroups ? g + 1 : g, ln4n, el4n, eb4n);
+    float4 aout[C];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int s = 4 * g + j;
+      const float from_left = wave_shr1(emit[C - 1], kNegInf);
+#pragma unroll
+      for (int c = C - 1; c >= 0; --c) {
+        const int u = lane * C + c, t = s - u;
+        const float left = (c == 0) ? from_left : emit[c - 1];
+        const bool active = (t >= 0) & (t < Tb) & (u < Ub);
+        float a = lse2(left, stay[c]);
+        a = (s == 0 && u == 0) ? 0.0f : a;  // :43
+        const float ln = f4get(ln4[c], j);
+        float sb = a + eb4[c][j];
+        sb = sb + pbv[c];
+        sb = sb - ln;
+        float se = a + f4get(el4[c], j);
+        se = se + plv[c];
+        se = se - ln;
+        stay[c] = active ? sb : stay[c];
+        emit[c] = active ? se : emit[c];
+        f4set(aout[c], j, a);
+      }
+    }
+#pragma unroll
+    for (int c = 0; c < C; ++c) {
+      if (lane * C + c < d.U) *reinterpret_cast<float4*>(ap[c] + 4 * g) = aout[c];
+      ln4[c] = ln4n[c];
+      el4[c] = el4n[c];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) eb4[c][j] = eb4n[c][j];
+    }
+  }
+  // :73-78 the blank move out of the last cell, negated
+#pragma unroll
+  for (int c = 0; c < C; ++c)
+    if (lane * C + c == Ub - 1) costs[b] = -stay[c];
+}
+
+// ------------------------------------------------------------------ transition weights
+// Everything of the dalpha recursion that does not depend on dalpha itself
+// (transducer/transducer_cpu.cpp:124-135): one thread per lattice cell.
+__global__ __launch_bounds__(256) void weights_kernel(Planes p, const int* __restrict__ inLen,
+                                                      const int* __restrict__ labLen, Dims d) {
+  const int b = blockIdx.z, u = blockIdx.y;
+  const int dg = blockIdx.x * 256 + threadIdx.x;
+  int Tb, Ub;
+  utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
+  const int t = dg - u;
+  if (u >= Ub || t < 0 || t >= Tb) return;
+  const size_t o = ((size_t)b * d.U + u) * d.Dp + dg;
+  const float a = p.aS[o], ln = p.lnS[o];
+  float wb = 0.0f, we = 0.0f;
+  if (t + 1 < Tb) {
+    float x = a + p.eb[(size_t)b * d.Tp + t];
+    x = x + p.pb[(size_t)b * d.U + u];
+    x = x - ln;
+    x = x - p.aS[o + 1];
+    wb = expf(x);
+  }
+  if (u + 1 < Ub) {
+    float x = a + p.elS[o];
+    x = x + p.pl[(size_t)b * d.U + u];
+    x = x - ln;
+    x = x - p.aS[o + d.Dp + 1];
+    we = expf(x);
+  }
+  p.wB[o] = wb;
+  p.wE[o] = we;
+}
+
+// ------------------------------------------------------------------ dalpha
+// transducer/transducer_cpu.cpp:81-143 with the exponentials already taken:
+// dalpha[t,u] = dalpha[t+1,u]*wB[t,u] + dalpha[t,u+1]*wE[t,u], walked from the last diagonal
+// back to the first.  Each lane also keeps the running sums that the reference subtracts from
+// pgrads[u,blank] and pgrads[u,l_u], in the reference's own order (t descending).
+template <int C>
+__global__ __launch_bounds__(64) void beta_kernel(Planes p, const int* __restrict__ labels,
+                                                  const int* __restrict__ inLen,
+                                                  const int* __restrict__ labLen, Dims d) {
+  const int b = blockIdx.x, lane = threadIdx.x;
+  int Tb, Ub;
+  utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
+  if (Tb == 0 || Ub == 0) return;  // :92-94
+  const int nsteps = Tb + Ub - 1;
+  const int ngroups = (nsteps + 3) >> 2;
+
+  float dcol[C], accB[C], accL[C];
+  bool fold[C];  // label of this position equals blank: both sums share one accumulator
+  const float* wbp[C];
+  const float* wep[C];
+  float* dp[C];
+#pragma unroll
+  for (int c = 0; c < C; ++c) {
+    const int u = lane * C + c, uc = u < d.U ? u : d.U - 1;
+    const size_t row = ((size_t)b * d.U + uc) * d.Dp;
+    wbp[c] = p.wB + row;
+    wep[c] = p.wE + row;
+    dp[c] = p.dS + row;
+    dcol[c] = 0.0f;
+    accB[c] = (u == Ub - 1) ? -1.0f : 0.0f;  // :97
+    accL[c] = 0.0f;
+    fold[c] = (u + 1 < Ub) && labels[(size_t)b * (d.U - 1) + u] == d.blank;
+  }
+
+  float4 wb4[C], we4[C];
+  auto load_group = [&](int g, float4* wb, float4* we) {
+#pragma unroll
+    for (int c = 0; c < C; ++c) {
+      wb[c] = *reinterpret_cast<const float4*>(wbp[c] + 4 * g);
+      we[c] = *reinterpret_cast<const float4*>(wep[c] + 4 * g);
+    }
+  };
+  load_group(ngroups - 1, wb4, we4);
+
+  for (int g = ngroups - 1; g >= 0; --g) {
+    float4 wb4n[C], we4n[C];
+    load_group(g > 0 ? g - 1 : 0, wb4n, we4n);
+    float4 dout[C];
+#pragma unroll
+    for (int j = 3; j >= 0; --j) {
+      const int s = 4 * g + j;
+      const float from_right = wave_shl1(dcol[0], 0.0f);
+#pragma unroll
+      for (int c = 0; c < C; ++c) {
+        const int u = lane * C + c, t = s - u;
+        const float right = (c == C - 1) ? from_right : dcol[c + 1];
+        const bool active = (t >= 0) & (t < Tb) & (u < Ub) & (s < nsteps);
+        const float ne = dcol[c] * f4get(wb4[c], j);
+        const float em = right * f4get(we4[c], j);
+        float dn = ne + em;
+        dn = (t == Tb - 1 && u == Ub - 1) ? 1.0f : dn;  // :95
+        const float ne_a = active ? ne : 0.0f, em_a = active ? em : 0.0f;
+        if (fold[c]) {
+          accB[c] = (accB[c] - ne_a) - em_a;
+        } else {
+          accB[c] = accB[c] - ne_a;
+          accL[c] = accL[c] - em_a;
+        }
+        dcol[c] = active ? dn : dcol[c];
+        f4set(dout[c], j, active ? dn : 0.0f);
+      }
+    }
+#pragma unroll
+    for (int c = 0; c < C; ++c) {
+      if (lane * C + c < d.U) *reinterpret_cast<float4*>(dp[c] + 4 * g) = dout[c];
+      wb4[c] = wb4n[c];
+      we4[c] = we4n[c];
+    }
+  }
+#pragma unroll
+  for (int c = 0; c < C; ++c) {
+    const int u = lane * C + c;
+    if (u < Ub) {
+      p.gB[(size_t)b * d.U + u] = accB[c];
+      p.gL[(size_t)b * d.U + u] = accL[c];
+    }
+  }
+}
+
+// ------------------------------------------------------------------ sparse gradient terms
+// The blank/label terms of transducer/transducer_cpu.cpp:95-141.  One thread per frame walks
+// the label positions from last to first, which is the order in which the reference subtracts
+// into a row of egrads, so repeated labels round the same way.  pgrads comes from the sums
+// the dalpha kernel kept.  add == 0: the terms are stored (the arrays were zero-filled);
+// add != 0: scale[b] (1 when scale is null) times the term is added to what the arrays hold.
+__global__ __launch_bounds__(256) void sparse_e_kernel(Planes p, float* __restrict__ egrads,
+                                                       const int* __restrict__ labels,
+                                                       const int* __restrict__ inLen,
+                                                       const int* __restrict__ labLen,
+                                                       const float* __restrict__ scale, int add,
+                                                       Dims d) {
+  const int b = blockIdx.y;
+  const int t = blockIdx.x * 256 + threadIdx.x;
+  int Tb, Ub;
+  utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
+  if (Ub == 0 || t >= Tb) return;
+  float* row = egrads + ((size_t)b * d.T + t) * d.V;
+  const int* lab = labels + (size_t)b * (d.U - 1);
+  const float sc = scale ? scale[b] : 1.0f;
+  float blank_acc = (t == Tb - 1) ? -1.0f : 0.0f;
+  for (int u = Ub - 1; u >= 0; --u) {
+    const size_t o = ((size_t)b * d.U + u) * d.Dp + t + u;
+    if (t + 1 < Tb) blank_acc -= p.dS[o + 1] * p.wB[o];
+    if (u + 1 < Ub) {
+      const float em = p.dS[o + d.Dp + 1] * p.wE[o];
+      const int l = lab[u];
+      if (l == d.blank) blank_acc -= em;
+      else if (add) row[l] += sc * (-em);
+      else row[l] -= em;
+    }
+  }
+  if (add) row[d.blank] += sc * blank_acc;
+  else row[d.blank] = blank_acc;
+}
+
+__global__ __launch_bounds__(256) void sparse_p_kernel(Planes p, float* __restrict__ pgrads,
+                                                       const int* __restrict__ labels,
+                                                       const int* __restrict__ inLen,
+                                                       const int* __restrict__ labLen,
+                                                       const float* __restrict__ scale, int add,
+                                                       Dims d) {
+  const int b = blockIdx.y;
+  const int u = blockIdx.x * 256 + threadIdx.x;
+  int Tb, Ub;
+  utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
+  if (Tb == 0 || u >= Ub) return;
+  float* row = pgrads + ((size_t)b * d.U + u) * d.V;
+  const float gb = p.gB[(size_t)b * d.U + u], gl = p.gL[(size_t)b * d.U + u];
+  const bool has_label = u + 1 < Ub;
+  const int l = has_label ? labels[(size_t)b * (d.U - 1) + u] : d.blank;
+  if (add) {
+    const float sc = scale ? scale[b] : 1.0f;
+    row[d.blank] += sc * gb;
+    if (has_label && l != d.blank) row[l] += sc * gl;
+  } else {
+    row[d.blank] = gb;
+    if (has_label && l != d.blank) row[l] = gl;
+  }
+}
+
+// ------------------------------------------------------------------ max-plus table
+// best[t,u] = max over v != blank of E[t,v]+P[u,v], arg = lowest such v
+// (transducer/transducer_cpu.cpp:158-171).  A block owns 32 frames x 128 label positions and
+// streams the vocabulary in chunks of 32 through LDS; a thread owns 4x4 cells.  The running
+// maximum is exact and order-free; the index is recovered afterwards by rescanning only the
+// first chunk that reached the maximum, so the inner loop is one add and one max per term.
+constexpr int kMpT = 32, kMpU = 128, kMpK = 32;
+
+__global__ __launch_bounds__(256) void maxplus_kernel(const float* __restrict__ E,
+                                                      const float* __restrict__ P,
+                                                      const int* __restrict__ inLen,
+                                                      const int* __restrict__ labLen,
+                                                      float* __restrict__ best,
+                                                      int* __restrict__ arg, Dims d) {
+  __shared__ float Es[kMpT][kMpK + 1];
+  __shared__ float Ps[kMpU][kMpK + 1];
+  const int b = blockIdx.z, t0 = blockIdx.x * kMpT, u0 = blockIdx.y * kMpU;
+  int Tb, Ub;
+  utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
+  if (t0 >= Tb || u0 >= Ub) return;
+  const int tid = threadIdx.x, tx = tid & 31, ty = tid >> 5;
+  const float* Eb = E + (size_t)b * d.T * d.V;
+  const float* Pb = P + (size_t)b * d.U * d.V;
+
+  float top[4][4];
+  int chunk[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) { top[i][j] = kNegInf; chunk[i][j] = -1; }
+
+  const int nchunks = (d.V + kMpK - 1) / kMpK;
+  for (int k = 0; k < nchunks; ++k) {
+    const int v0 = k * kMpK;
+    // stage: 32x32 of E and 128x32 of P; consecutive threads read consecutive v
+    for (int e = tid; e < kMpT * kMpK; e += 256) {
+      const int r = e / kMpK, c = e % kMpK, t = t0 + r, v = v0 + c;
+      Es[r][c] = (t < Tb && v < d.V && v != d.blank) ? Eb[(size_t)t * d.V + v] : kNegInf;
+    }
+    for (int e = tid; e < kMpU * kMpK; e += 256) {
+      const int r = e / kMpK, c = e % kMpK, u = u0 + r, v = v0 + c;
+      Ps[r][c] = (u < Ub && v < d.V) ? Pb[(size_t)u * d.V + v] : kNegInf;
+    }
+    __syncthreads();
+    float cm[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) cm[i][j] = kNegInf;
+#pragma unroll 8
+    for (int c = 0; c < kMpK; ++c) {
+      float ev[4], pv[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) ev[i] = Es[ty * 4 + i][c];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) pv[j] = Ps[tx + 32 * j][c];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) cm[i][j] = fmaxf(cm[i][j], ev[i] + pv[j]);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if (cm[i][j] > top[i][j]) { top[i][j] = cm[i][j]; chunk[i][j] = k; }
+    __syncthreads();
+  }
+  // recover the lowest index inside the winning chunk
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int t = t0 + ty * 4 + i, u = u0 + tx + 32 * j;
+      if (t >= Tb || u >= Ub) continue;
+      int at = 0;  // :160 the scan starts from index 0 and keeps it if nothing beats -inf
+      if (chunk[i][j] >= 0) {
+        const int v0 = chunk[i][j] * kMpK;
+        const float* e = Eb + (size_t)t * d.V;
+        const float* q = Pb + (size_t)u * d.V;
+        for (int v = v0; v < v0 + kMpK && v < d.V; ++v) {
+          if (v == d.blank) continue;
+          if (e[v] + q[v] == top[i][j]) { at = v; break; }
+        }
+      }
+      const size_t o = ((size_t)b * d.T + t) * d.U + u;
+      best[o] = top[i][j];
+      arg[o] = at;
+    }
+}
+
+// ------------------------------------------------------------------ viterbi
+// transducer/transducer_cpu.cpp:145-222.  Scores walk the lattice like alpha with
+// max in place of log-sum-exp: no transcendental anywhere, so given the same LN the path is
+// bit-exact.  Association: blank move ((s + e) + p) - LN (:192-195), label move
+// (s + best) - LN (:197-199); "emit > stay" takes the label, ties go to blank (:200-206).
+// The decision of every cell is one bit; each step's 64-lane ballot goes to `bits`
+// (LDS when it fits, else global), and lane 0 walks them backwards at the end (:208-219).
+template <int C, bool kLdsBits>
+__global__ __launch_bounds__(64) void viterbi_kernel(Planes p, const float* __restrict__ bestS,
+                                                     const float* __restrict__ argS,
+                                                     const int* __restrict__ inLen,
+                                                     const int* __restrict__ labLen,
+                                                     unsigned long long* __restrict__ gbits,
+                                                     int* __restrict__ labels_out, Dims d) {
+  extern __shared__ unsigned long long lbits[];
+  const int b = blockIdx.x, lane = threadIdx.x;
+  int Tb, Ub;
+  utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
+  if (Tb == 0 || Ub == 0) return;  // :152-154
+  const int nsteps = Tb + Ub - 1;
+  const int ngroups = (nsteps + 3) >> 2;
+  unsigned long long* bits =
+      kLdsBits ? lbits : gbits + (size_t)b * (size_t)(d.T + d.U + 4) * C;
+  const float* ebp = p.eb + (size_t)b * d.Tp;
+
+  float stay[C], emit[C], pbv[C];
+  const float* lnp[C];
+  const float* bsp[C];
+#pragma unroll
+  for (int c = 0; c < C; ++c) {
+    const int u = lane * C + c, uc = u < d.U ? u : d.U - 1;
+    const size_t row = ((size_t)b * d.U + uc) * d.Dp;
+    lnp[c] = p.lnS + row;
+    bsp[c] = bestS + row;
+    pbv[c] = p.pb[(size_t)b * d.U + uc];
+    stay[c] = kNegInf;
+    emit[c] = kNegInf;
+  }
+  float4 ln4[C], bs4[C];
+  float eb4[C][4];
+  auto load_group = [&](int g, float4* ln, float4* bs, float (*ebv)[4]) {
+#pragma unroll
+    for (int c = 0; c < C; ++c) {
+      ln[c] = *reinterpret_cast<const float4*>(lnp[c] + 4 * g);
+      bs[c] = *reinterpret_cast<const float4*>(bsp[c] + 4 * g);
+      const int u = lane * C + c;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) ebv[c][j] = ebp[clampi(4 * g + j - u, 0, Tb - 1)];
+    }
+  };
+  load_group(0, ln4, bs4, eb4);
+  for (int g = 0; g < ngroups; ++g) {
+    float4 ln4n[C], bs4n[C];
+    float eb4n[C][4];
+    load_group(g + 1 < ngroups ? g + 1 : g, ln4n, bs4n, eb4n);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int s = 4 * g + j;
+      const float from_left = wave_shr1(emit[C - 1], kNegInf);
+#pragma unroll
+      for (int c = C - 1; c >= 0; --c) {
+        const int u = lane * C + c, t = s - u;
+        const float left = (c == 0) ? from_left : emit[c - 1];
+        const bool active = (t >= 0) & (t < Tb) & (u < Ub);
+        const bool take = left > stay[c];
+        float x = take ? left : stay[c];
+        x = (s == 0 && u == 0) ? 0.0f : x;
+        const unsigned long long m = __ballot(take);
+        if (lane == 0) bits[(size_t)s * C + c] = m;
+        const float ln = f4get(ln4[c], j);
+        float sb = x + eb4[c][j];
+        sb = sb + pbv[c];
+        sb = sb - ln;
+        float se = x + f4get(bs4[c], j);
+        se = se - ln;
+        stay[c] = active ? sb : stay[c];
+        emit[c] = active ? se : emit[c];
+      }
+    }
+#pragma unroll
+    for (int c = 0; c < C; ++c) {
+      ln4[c] = ln4n[c];
+      bs4[c] = bs4n[c];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) eb4[c][j] = eb4n[c][j];
+    }
+  }
+  __syncthreads();
+  if (lane == 0) {
+    int* out = labels_out + (size_t)b * (d.U - 1);
+    const int* argI = reinterpret_cast<const int*>(argS);
+    int t = Tb - 1, u = Ub - 1;
+    while (u > 0 && t >= 0) {
+      const int s = t + u;
+      const unsigned long long m = bits[(size_t)s * C + (u % C)];
+      if ((m >> (u / C)) & 1ull) {
+        out[u - 1] = argI[((size_t)b * d.U + (u - 1)) * d.Dp + s - 1];
+        u -= 1;
+      } else {
+        t -= 1;
+      }
+    }
+  }
+}
+
+int cells_per_lane(int U) {
+  int c = 1;
+  while (c * 64 < U) c *= 2;
+  return c;
+}
+
+}  // namespace
+
+// ------------------------------------------------------------------ workspace layout
+static size_t align_up(size_t x) { return (x + 255) & ~(size_t)255; }
+
+size_t planes_bytes(const Dims& d) {
+  const size_t plane = align_up(sizeof(float) * (size_t)d.B * d.U * d.Dp + 64);
+  return 6 * plane + align_up(sizeof(float) * (size_t)d.B * d.Tp) +
+         4 * align_up(sizeof(float) * (size_t)d.B * d.U);
+}
+
+void carve_planes(void* base, const Dims& d, Planes* p) {
+  char* c = static_cast<char*>(base);
+  const size_t plane = align_up(sizeof(float) * (size_t)d.B * d.U * d.Dp + 64);
+  auto take = [&](size_t n) { float* r = reinterpret_cast<float*>(c); c += n; return r; };
+  p->lnS = take(plane); p->elS = take(plane); p->aS = take(plane);
+  p->wB = take(plane); p->wE = take(plane); p->dS = take(plane);
+  p->eb = take(align_up(sizeof(float) * (size_t)d.B * d.Tp));
+  const size_t bu = align_up(sizeof(float) * (size_t)d.B * d.U);
+  p->pb = take(bu); p->pl = take(bu); p->gB = take(bu); p->gL = take(bu);
+}
+
+// ------------------------------------------------------------------ launchers
+#define RNNT_LAUNCH_CHECK(name)                                                    \
+  do {                                                                             \
+    hipError_t _e = hipGetLastError();                                             \
+    if (_e != hipSuccess) return check_hip(_e, "launch " name, __FILE__, __LINE__); \
+  } while (0)
+
+static dim3 tile_grid(const Dims& d) {
+  return dim3((d.T + 63) / 64, (d.U + 63) / 64, d.B);
+}
+
+int launch_skew(const float* src, float* dstS, const int* inLen, const int* labLen, const Dims& d,
+                hipStream_t s) {
+  if (d.B == 0 || d.T == 0 || d.U == 0) return kOk;
+  hipLaunchKernelGGL(skew_kernel, tile_grid(d), dim3(256), 0, s, src, dstS, inLen, labLen, d);
+  RNNT_LAUNCH_CHECK("skew_kernel");
+  return kOk;
+}
+
+int launch_unskew(const float* srcS, float* dst, const int* inLen, const int* labLen,
+                  const Dims& d, hipStream_t s) {
+  if (d.B == 0 || d.T == 0 || d.U == 0) return kOk;
+  hipLaunchKernelGGL(unskew_kernel, tile_grid(d), dim3(256), 0, s, srcS, dst, inLen, labLen, d);
+  RNNT_LAUNCH_CHECK("unskew_kernel");
+  return kOk;
+}
+
+int launch_gather(const float* E, const float* P, const int* labels, const int* inLen,
+                  const int* labLen, const Planes& p, const Dims& d, hipStream_t s) {
+  if (d.B == 0 || d.T == 0 || d.U == 0) return kOk;
+  hipLaunchKernelGGL(gather_kernel, dim3((d.T + 255) / 256, d.U, d.B), dim3(256), 0, s, E, P,
+                     labels, inLen, labLen, p, d);
+  RNNT_LAUNCH_CHECK("gather_kernel");
+  return kOk;
+}
+
+int launch_alpha(const Planes& p, const int* inLen, const int* labLen, float* costs,
+                 const Dims& d, hipStream_t s) {
+  if (d.B == 0) return kOk;
+  switch (cells_per_lane(d.U)) {
+#define CASE(C)                                                                              \
+  case C:                                                                                    \
+    hipLaunchKernelGGL(alpha_kernel<C>, dim3(d.B), dim3(64), 0, s, p, inLen, labLen, costs, d); \
+    break;
+    CASE(1) CASE(2) CASE(4) CASE(8) CASE(16)
+#undef CASE
+    default:
+      return fail(kInvalid, "prediction length %d exceeds the supported maximum of 1024", d.U);
+  }
+  RNNT_LAUNCH_CHECK("alpha_kernel");
+  return kOk;
+}
+
+int launch_weights(const Planes& p, const int* inLen, const int* labLen, const Dims& d,
+                   hipStream_t s) {
+  if (d.B == 0 || d.T == 0 || d.U == 0) return kOk;
+  hipLaunchKernelGGL(weights_kernel, dim3((d.T + d.U + 255) / 256, d.U, d.B), dim3(256), 0, s, p,
+                     inLen, labLen, d);
+  RNNT_LAUNCH_CHECK("weights_kernel");
+  return kOk;
+}
+
+int launch_beta(const Planes& p, const int* labels, const int* inLen, const int* labLen,
+                const Dims& d, hipStream_t s) {
+  if (d.B == 0 || d.T == 0 || d.U == 0) return kOk;
+  switch (cells_per_lane(d.U)) {
+#define CASE(C)                                                                              \
+  case C:                                                                                    \
+    hipLaunchKernelGGL(beta_kernel<C>, dim3(d.B), dim3(64), 0, s, p, labels, inLen, labLen, d); \
+    break;
+    CASE(1) CASE(2) CASE(4) CASE(8) CASE(16)
+#undef CASE
+    default:
+      return fail(kInvalid, "prediction length %d exceeds the supported maximum of 1024", d.U);
+  }
+  RNNT_LAUNCH_CHECK("beta_kernel");
+  return kOk;
+}
+
+int launch_sparse(const Planes& p, float* egrads, float* pgrads, const int* labels,
+                  const int* inLen, const int* labLen, const float* scale, bool add,
+                  const Dims& d, hipStream_t s) {
+  if (d.B == 0 || d.T == 0 || d.U == 0) return kOk;
+  hipLaunchKernelGGL(sparse_e_kernel, dim3((d.T + 255) / 256, d.B), dim3(256), 0, s, p, egrads,
+                     labels, inLen, labLen, scale, add ? 1 : 0, d);
+  RNNT_LAUNCH_CHECK("sparse_e_kernel");
+  hipLaunchKernelGGL(sparse_p_kernel, dim3((d.U + 255) / 256, d.B), dim3(256), 0, s, p, pgrads,
+                     labels, inLen, labLen, scale, add ? 1 : 0, d);
+  RNNT_LAUNCH_CHECK("sparse_p_kernel");
+  return kOk;
+}
+
+int launch_maxplus(const float* E, const float* P, const int* inLen, const int* labLen,
+                   float* best, int* arg, const Dims& d, hipStream_t s) {
+  if (d.B == 0 || d.T == 0 || d.U == 0) return kOk;
+  hipLaunchKernelGGL(maxplus_kernel, dim3((d.T + kMpT - 1) / kMpT, (d.U + kMpU - 1) / kMpU, d.B),
+                     dim3(256), 0, s, E, P, inLen, labLen, best, arg, d);
+  RNNT_LAUNCH_CHECK("maxplus_kernel");
+  return kOk;
+}
+
+int launch_viterbi(const Planes& p, const float* bestS, const float* argS,
+                   unsigned long long* gbits, const int* inLen, const int* labLen,
+                   int* labels_out, const Dims& d, hipStream_t s) {
+  if (d.B == 0 || d.T == 0 || d.U <= 1) return kOk;
+  const int C = cells_per_lane(d.U);
+  const size_t lds = sizeof(unsigned long long) * (size_t)(d.T + d.U + 4) * C;
+  const bool use_lds = lds <= 60 * 1024;
+  switch (C) {
+#define CASE(C)                                                                               \
+  case C:                                                                                     \
+    if (use_lds)                                                                              \
+      hipLaunchKernelGGL((viterbi_kernel<C, true>), dim3(d.B), dim3(64), lds, s, p, bestS, argS, \
+                         inLen, labLen, gbits, labels_out, d);                                \
+    else                                                                                      \
+      hipLaunchKernelGGL((viterbi_kernel<C, false>), dim3(d.B), dim3(64), 0, s, p, bestS, argS,  \
+                         inLen, labLen, gbits, labels_out, d);                                \
+    break;
+    CASE(1) CASE(2) CASE(4) CASE(8) CASE(16)
+#undef CASE
+    default:
+      return fail(kInvalid, "prediction length %d exceeds the supported maximum of 1024", d.U);
+  }
+  RNNT_LAUNCH_CHECK("viterbi_kernel");
+  return kOk;
+}
+
+size_t viterbi_bits_bytes(const Dims& d) {
+  return sizeof(unsigned long long) * (size_t)d.B * (size_t)(d.T + d.U + 4) * cells_per_lane(d.U);
+}
+
+}  // namespace rnnt

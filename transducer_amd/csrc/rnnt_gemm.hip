@@ -1,0 +1,471 @@
+// The three vocabulary-sized contractions of the RNN-T loss on the gfx950 matrix cores, with
+// their exponentials and logarithms fused in so that nothing of size B*T*U*V -- and no copy of
+// the [B,T,V] emissions -- ever goes to memory:
+//
+//   log-normaliser (transducer/torch_binding.py:35-40)
+//       LN[t,u] = log( sum_v exp(E[t,v]-mE[t]) * exp(P[u,v]-mP[u]) ) + mE[t] + mP[u]
+//   dense gradient parts (transducer/torch_binding.py:85-89), W[t,u] = dalpha[t,u]/sum_v(...)
+//       egrads[t,v] = delta * exp(E[t,v]-mE[t]) * sum_u W[t,u] * exp(P[u,v]-mP[u])
+//       pgrads[u,v] = delta * exp(P[u,v]-mP[u]) * sum_t W[t,u] * exp(E[t,v]-mE[t])
+//
+// All three use v_mfma_f32_32x32x2_f32 (fp32 in, fp32 accumulate).  A wavefront owns 32x32
+// output blocks; for one instruction lane l supplies A[row l%32][k-slot l/32] and
+// B[k-slot l/32][col l%32] and receives D[8*(r/4) + 4*(l/32) + r%4][l%32] in register r.
+// Which element of the reduction sits in which k-slot is free as long as A and B agree, so a
+// lane takes four consecutive k of its row with one 16-byte LDS read and spends them on four
+// instructions.
+#include "rnnt_internal.h"
+
+namespace rnnt {
+
+namespace {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr float kNegInf = -__builtin_huge_valf();
+
+__device__ inline float wave_max(float m) {
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
+  return m;
+}
+
+// ------------------------------------------------------------------ row maxima
+// One wavefront per row of a [rows, V] array.
+__global__ __launch_bounds__(256) void rowmax_kernel(const float* __restrict__ X,
+                                                     float* __restrict__ out, long rows, int V,
+                                                     int vec4) {
+  const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (row >= rows) return;
+  const float* x = X + (size_t)row * V;
+  float m0 = kNegInf, m1 = kNegInf, m2 = kNegInf, m3 = kNegInf;
+  if (vec4) {
+    const float4* x4 = reinterpret_cast<const float4*>(x);
+    const int n4 = V >> 2;
+    int i = lane;
+    for (; i + 192 < n4; i += 256) {
+      const float4 a = x4[i], b = x4[i + 64], c = x4[i + 128], e = x4[i + 192];
+      m0 = fmaxf(m0, fmaxf(fmaxf(a.x, a.y), fmaxf(a.z, a.w)));
+      m1 = fmaxf(m1, fmaxf(fmaxf(b.x, b.y), fmaxf(b.z, b.w)));
+      m2 = fmaxf(m2, fmaxf(fmaxf(c.x, c.y), fmaxf(c.z, c.w)));
+      m3 = fmaxf(m3, fmaxf(fmaxf(e.x, e.y), fmaxf(e.z, e.w)));
+    }
+    for (; i < n4; i += 64) {
+      const float4 a = x4[i];
+      m0 = fmaxf(m0, fmaxf(fmaxf(a.x, a.y), fmaxf(a.z, a.w)));
+    }
+  } else {
+    for (int i = lane; i < V; i += 64) m0 = fmaxf(m0, x[i]);
+  }
+  const float m = wave_max(fmaxf(fmaxf(m0, m1), fmaxf(m2, m3)));
+  if (lane == 0) out[row] = m;
+}
+
+// ------------------------------------------------------------------ log-normaliser
+// Block tile 128 (t) x 128 (u), reduction over v in slices of 32; 4 wavefronts, each 64x64.
+// Both operands are v-contiguous in memory and are staged as S[row][v] with a 36-float pitch
+// (16-byte reads of consecutive rows then fall into distinct bank groups).
+constexpr int kLseBM = 128, kLseBN = 128, kLseBK = 32, kLsePitch = kLseBK + 4;
+
+__global__ __launch_bounds__(256, 2) void lse_kernel(const float* __restrict__ E,
+                                                     const float* __restrict__ P,
+                                                     const float* __restrict__ mE,
+                                                     const float* __restrict__ mP,
+                                                     float* __restrict__ LN,
+                                                     const int* __restrict__ inLen,
+                                                     const int* __restrict__ labLen, Dims d) {
+  __shared__ __attribute__((aligned(16))) float As[kLseBM * kLsePitch];
+  __shared__ __attribute__((aligned(16))) float Bs[kLseBN * kLsePitch];
+  const int b = blockIdx.z, t0 = blockIdx.x * kLseBM, u0 = blockIdx.y * kLseBN;
+  int Tb, Ub;
+  utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  float* LNb = LN + (size_t)b * d.T * d.U;
+
+  if (t0 >= Tb || u0 >= Ub) {
+    // nothing valid here: the array still gets defined contents (zeros, as in the torch-free
+    // reference helper transducer/test.h:58)
+    for (int e = tid; e < kLseBM * kLseBN; e += 256) {
+      const int t = t0 + e / kLseBN, u = u0 + e % kLseBN;
+      if (t < d.T && u < d.U) LNb[(size_t)t * d.U + u] = 0.0f;
+    }
+    return;
+  }
+
+  const float* Eb = E + (size_t)b * d.T * d.V;
+  const float* Pb = P + (size_t)b * d.U * d.V;
+  const float* mEb = mE + (size_t)b * d.T;
+  const float* mPb = mP + (size_t)b * d.U;
+
+  // staging assignment: element e = tid + 256*i -> row e/32, column e%32 (a wavefront reads two
+  // 128-byte row segments per load instruction)
+  const int lcol = tid & 31, lrow0 = tid >> 5;  // rows lrow0 + 8*i, i < 16
+  float ra[16], rb[16];
+  float ma[16], mb[16];
+  const float* pa[16];
+  const float* pb[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int r = lrow0 + 8 * i;
+    const int t = min(t0 + r, d.T - 1), u = min(u0 + r, d.U - 1);
+    pa[i] = Eb + (size_t)t * d.V;
+    pb[i] = Pb + (size_t)u * d.V;
+    ma[i] = mEb[t];
+    mb[i] = mPb[u];
+  }
+  auto fetch = [&](int k0) {
+    const int v = k0 + lcol;
+    const bool ok = v < d.V;
+    const int vc = ok ? v : d.V - 1;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const float x = pa[i][vc], y = pb[i][vc];
+      ra[i] = ok ? x : kNegInf;  // exp(-inf - m) = 0: past-the-end terms add nothing
+      rb[i] = ok ? y : kNegInf;
+    }
+  };
+
+  const int wm = wave >> 1, wn = wave & 1, l32 = lane & 31, h = lane >> 5;
+  floatx16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+  const int nk = (d.V + kLseBK - 1) / kLseBK;
+  fetch(0);
+  for (int kt = 0; kt < nk; ++kt) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int r = lrow0 + 8 * i;
+      As[r * kLsePitch + lcol] = __expf(ra[i] - ma[i]);
+      Bs[r * kLsePitch + lcol] = __expf(rb[i] - mb[i]);
+    }
+    __syncthreads();
+    if (kt + 1 < nk) fetch((kt + 1) * kLseBK);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      float4 a4[2], b4[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        a4[i] = *reinterpret_cast<const float4*>(
+            &As[(64 * wm + 32 * i + l32) * kLsePitch + 8 * j + 4 * h]);
+        b4[i] = *reinterpret_cast<const float4*>(
+            &Bs[(64 * wn + 32 * i + l32) * kLsePitch + 8 * j + 4 * h]);
+      }
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+          for (int jj = 0; jj < 2; ++jj) {
+            const float av = q == 0 ? a4[i].x : (q == 1 ? a4[i].y : (q == 2 ? a4[i].z : a4[i].w));
+            const float bv =
+                q == 0 ? b4[jj].x : (q == 1 ? b4[jj].y : (q == 2 ? b4[jj].z : b4[jj].w));
+            acc[i][jj] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc[i][jj], 0, 0, 0);
+          }
+      }
+    }
+    __syncthreads();
+  }
+
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int jj = 0; jj < 2; ++jj)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int t = t0 + 64 * wm + 32 * i + 8 * (r >> 2) + 4 * h + (r & 3);
+        const int u = u0 + 64 * wn + 32 * jj + l32;
+        if (t < d.T && u < d.U) {
+          float v = 0.0f;
+          if (t < Tb && u < Ub) v = (logf(acc[i][jj][r]) + mEb[t]) + mPb[u];
+          LNb[(size_t)t * d.U + u] = v;
+        }
+      }
+}
+
+// ------------------------------------------------------------------ W planes
+// W[t,u] = dalpha[t,u] / sum_v(...) = dalpha[t,u] * exp((mE[t] + mP[u]) - LN[t,u]), written
+// twice: Wn[b][t][Up] (u contiguous, feeds the egrads contraction) and Wt[b][u][Tw]
+// (t contiguous, feeds the pgrads contraction).  Cells outside the utterance are zero.
+__global__ __launch_bounds__(256) void wplanes_kernel(const float* __restrict__ lngrads,
+                                                      const float* __restrict__ LN,
+                                                      const float* __restrict__ mE,
+                                                      const float* __restrict__ mP,
+                                                      float* __restrict__ Wn,
+                                                      float* __restrict__ Wt,
+                                                      const int* __restrict__ inLen,
+                                                      const int* __restrict__ labLen, Dims d,
+                                                      int Up, int Tw) {
+  __shared__ float tile[64][65];
+  const int b = blockIdx.z, t0 = blockIdx.x * 64, u0 = blockIdx.y * 64;
+  int Tb, Ub;
+  utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int t = t0 + ty + 4 * i, u = u0 + tx;
+    float w = 0.0f;
+    if (t < Tb && u < Ub) {
+      const size_t o = ((size_t)b * d.T + t) * d.U + u;
+      w = lngrads[o] * expf((mE[(size_t)b * d.T + t] + mP[(size_t)b * d.U + u]) - LN[o]);
+    }
+    tile[ty + 4 * i][tx] = w;
+    if (t < Tw && u < Up) Wn[((size_t)b * Tw + t) * Up + u] = w;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int u = u0 + ty + 4 * i, t = t0 + tx;
+    if (t < Tw && u < Up) Wt[((size_t)b * Up + u) * Tw + t] = tile[tx][ty + 4 * i];
+  }
+}
+
+// ------------------------------------------------------------------ shared tile code
+// "A rows k-contiguous, B rows n-contiguous": As[m][k] pitch KP (16-byte reads, four k per
+// lane), Bs[k][n] pitch NP (4-byte reads, 32 consecutive n per half-wave).
+template <int KP, int NP>
+__device__ inline void mma_group(const float* As, const float* Bs, int arow, int bcol, int kbase,
+                                 int h, floatx16& acc) {
+  const float4 a4 = *reinterpret_cast<const float4*>(&As[arow * KP + kbase + 4 * h]);
+  const float b0 = Bs[(kbase + 4 * h + 0) * NP + bcol];
+  const float b1 = Bs[(kbase + 4 * h + 1) * NP + bcol];
+  const float b2 = Bs[(kbase + 4 * h + 2) * NP + bcol];
+  const float b3 = Bs[(kbase + 4 * h + 3) * NP + bcol];
+  acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a4.x, b0, acc, 0, 0, 0);
+  acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a4.y, b1, acc, 0, 0, 0);
+  acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a4.z, b2, acc, 0, 0, 0);
+  acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a4.w, b3, acc, 0, 0, 0);
+}
+
+// ------------------------------------------------------------------ egrads (dense part)
+// Block tile 64 (t) x 64 (v); the whole reduction over u (Up <= kEgMaxK) sits in LDS at once.
+constexpr int kEgMaxK = 112, kEgKP = kEgMaxK + 4, kEgNP = 64 + 4;
+
+__global__ __launch_bounds__(256, 2) void egrads_kernel(
+    const float* __restrict__ E, const float* __restrict__ P, const float* __restrict__ mE,
+    const float* __restrict__ mP, const float* __restrict__ Wn, const float* __restrict__ deltas,
+    float* __restrict__ egrads, const int* __restrict__ inLen, const int* __restrict__ labLen,
+    Dims d, int Up, int Tw, int kofs, int accumulate, int last) {
+  __shared__ __attribute__((aligned(16))) float As[64 * kEgKP];
+  __shared__ __attribute__((aligned(16))) float Bs[kEgMaxK * kEgNP];
+  const int b = blockIdx.z, v0 = blockIdx.x * 64, t0 = blockIdx.y * 64;
+  int Tb, Ub;
+  utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  float* out = egrads + (size_t)b * d.T * d.V;
+  if (t0 >= Tb) {  // padded frames: the dense part is exactly zero
+    const float dl = (deltas && last) ? deltas[b] : 1.0f;
+    for (int e = tid; e < 64 * 64; e += 256) {
+      const int t = t0 + e / 64, v = v0 + e % 64;
+      if (t < d.T && v < d.V) {
+        const size_t o = (size_t)t * d.V + v;
+        out[o] = accumulate ? dl * out[o] : 0.0f;
+      }
+    }
+    return;
+  }
+  const int K = min(Up - kofs, kEgMaxK);  // this launch's slice of the label axis
+  // A: W rows (t), k = u contiguous
+  for (int e = tid; e < 64 * K; e += 256) {
+    const int r = e / K, k = e % K;
+    As[r * kEgKP + k] = Wn[((size_t)b * Tw + t0 + r) * Up + kofs + k];
+  }
+  // B: exp(P[u,v] - mP[u]) rows (u), n = v contiguous
+  const float* Pb = P + (size_t)b * d.U * d.V;
+  for (int e = tid; e < K * 64; e += 256) {
+    const int k = e / 64, n = e % 64, u = kofs + k, v = v0 + n;
+    float y = 0.0f;
+    if (u < Ub && v < d.V) y = __expf(Pb[(size_t)u * d.V + v] - mP[(size_t)b * d.U + u]);
+    Bs[k * kEgNP + n] = y;
+  }
+  __syncthreads();
+  const int wm = wave >> 1, wn = wave & 1, l32 = lane & 31, h = lane >> 5;
+  floatx16 acc;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
+  for (int k = 0; k < K; k += 8)
+    mma_group<kEgKP, kEgNP>(As, Bs, 32 * wm + l32, 32 * wn + l32, k, h, acc);
+
+  const float delta = (deltas && last) ? deltas[b] : 1.0f;
+  const float* Eb = E + (size_t)b * d.T * d.V;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int t = t0 + 32 * wm + 8 * (r >> 2) + 4 * h + (r & 3);
+    const int v = v0 + 32 * wn + l32;
+    if (t < d.T && v < d.V) {
+      const size_t o = (size_t)t * d.V + v;
+      float g = 0.0f;
+      if (t < Tb) g = __expf(Eb[o] - mE[(size_t)b * d.T + t]) * acc[r];
+      if (accumulate) g = out[o] + g;
+      out[o] = delta * g;
+    }
+  }
+}
+
+// ------------------------------------------------------------------ pgrads (dense part)
+// Block tile 128 (u) x 64 (v), reduction over t in slices of 32.
+constexpr int kPgBK = 32, kPgKP = kPgBK + 4, kPgNP = 64 + 4;
+
+__global__ __launch_bounds__(256, 2) void pgrads_kernel(
+    const float* __restrict__ E, const float* __restrict__ P, const float* __restrict__ mE,
+    const float* __restrict__ mP, const float* __restrict__ Wt, const float* __restrict__ deltas,
+    float* __restrict__ pgrads, const int* __restrict__ inLen, const int* __restrict__ labLen,
+    Dims d, int Up, int Tw, int accumulate) {
+  __shared__ __attribute__((aligned(16))) float As[128 * kPgKP];
+  __shared__ __attribute__((aligned(16))) float Bs[kPgBK * kPgNP];
+  const int b = blockIdx.z, v0 = blockIdx.x * 64, u0 = blockIdx.y * 128;
+  int Tb, Ub;
+  utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  float* out = pgrads + (size_t)b * d.U * d.V;
+  if (u0 >= Ub || Tb == 0) {
+    const float dl = deltas ? deltas[b] : 1.0f;
+    for (int e = tid; e < 128 * 64; e += 256) {
+      const int u = u0 + e / 64, v = v0 + e % 64;
+      if (u < d.U && v < d.V) {
+        const size_t o = (size_t)u * d.V + v;
+        out[o] = accumulate ? dl * out[o] : 0.0f;
+      }
+    }
+    return;
+  }
+  const float* Eb = E + (size_t)b * d.T * d.V;
+  const float* mEb = mE + (size_t)b * d.T;
+  const int l32 = lane & 31, h = lane >> 5;
+  floatx16 acc[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[i][r] = 0.0f;
+
+  // staging: A element e -> row e/32 (u), k e%32 (t); B element e -> k e/64 (t), n e%64 (v)
+  float ra[16], rb[8];
+  auto fetch = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int e = tid + 256 * i, r = e >> 5, k = e & 31;
+      const int u = u0 + r, t = k0 + k;
+      ra[i] = (u < Up && t < Tw) ? Wt[((size_t)b * Up + u) * Tw + t] : 0.0f;
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int e = tid + 256 * i, k = e >> 6, n = e & 63;
+      const int t = k0 + k, v = v0 + n;
+      rb[i] = (t < Tb && v < d.V) ? Eb[(size_t)t * d.V + v] - mEb[t] : kNegInf;
+    }
+  };
+  const int nk = (Tb + kPgBK - 1) / kPgBK;
+  fetch(0);
+  for (int kt = 0; kt < nk; ++kt) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int e = tid + 256 * i;
+      As[(e >> 5) * kPgKP + (e & 31)] = ra[i];
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int e = tid + 256 * i;
+      Bs[(e >> 6) * kPgNP + (e & 63)] = __expf(rb[i]);
+    }
+    __syncthreads();
+    if (kt + 1 < nk) fetch((kt + 1) * kPgBK);
+    // wavefront w: u rows [32w, 32w+32), both 32-wide v blocks
+#pragma unroll
+    for (int k = 0; k < kPgBK; k += 8) {
+      mma_group<kPgKP, kPgNP>(As, Bs, 32 * wave + l32, l32, k, h, acc[0]);
+      mma_group<kPgKP, kPgNP>(As, Bs, 32 * wave + l32, 32 + l32, k, h, acc[1]);
+    }
+    __syncthreads();
+  }
+  const float delta = deltas ? deltas[b] : 1.0f;
+  const float* Pb = P + (size_t)b * d.U * d.V;
+#pragma unroll
+  for (int j = 0; j < 2; ++j)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int u = u0 + 32 * wave + 8 * (r >> 2) + 4 * h + (r & 3);
+      const int v = v0 + 32 * j + l32;
+      if (u < d.U && v < d.V) {
+        const size_t o = (size_t)u * d.V + v;
+        float g = 0.0f;
+        if (u < Ub) g = __expf(Pb[o] - mP[(size_t)b * d.U + u]) * acc[j][r];
+        if (accumulate) g = out[o] + g;
+        out[o] = delta * g;
+      }
+    }
+}
+
+}  // namespace
+
+#define RNNT_LAUNCH_CHECK(name)                                                    \
+  do {                                                                             \
+    hipError_t _e = hipGetLastError();                                             \
+    if (_e != hipSuccess) return check_hip(_e, "launch " name, __FILE__, __LINE__); \
+  } while (0)
+
+int launch_rowmax(const float* X, float* rowmax, long rows, int V, hipStream_t s) {
+  if (rows == 0) return kOk;
+  const int vec4 = (V % 4 == 0) && ((reinterpret_cast<uintptr_t>(X) & 15) == 0);
+  hipLaunchKernelGGL(rowmax_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, s, X, rowmax,
+                     rows, V, vec4);
+  RNNT_LAUNCH_CHECK("rowmax_kernel");
+  return kOk;
+}
+
+int launch_lse(const float* E, const float* P, const float* mE, const float* mP, float* LN,
+               const int* inLen, const int* labLen, const Dims& d, hipStream_t s) {
+  if (d.B == 0 || d.T == 0 || d.U == 0) return kOk;
+  hipLaunchKernelGGL(lse_kernel,
+                     dim3((d.T + kLseBM - 1) / kLseBM, (d.U + kLseBN - 1) / kLseBN, d.B),
+                     dim3(256), 0, s, E, P, mE, mP, LN, inLen, labLen, d);
+  RNNT_LAUNCH_CHECK("lse_kernel");
+  return kOk;
+}
+
+int wplane_up(int U) { return (U + 7) & ~7; }
+int wplane_tw(int T) { return (T + 63) & ~63; }
+
+int launch_wplanes(const float* lngrads, const float* LN, const float* mE, const float* mP,
+                   float* Wn, float* Wt, const int* inLen, const int* labLen, const Dims& d,
+                   hipStream_t s) {
+  if (d.B == 0 || d.T == 0 || d.U == 0) return kOk;
+  const int Up = wplane_up(d.U), Tw = wplane_tw(d.T);
+  hipLaunchKernelGGL(wplanes_kernel, dim3(Tw / 64, (Up + 63) / 64, d.B), dim3(256), 0, s, lngrads,
+                     LN, mE, mP, Wn, Wt, inLen, labLen, d, Up, Tw);
+  RNNT_LAUNCH_CHECK("wplanes_kernel");
+  return kOk;
+}
+
+int launch_egrads(const float* E, const float* P, const float* mE, const float* mP,
+                  const float* Wn, const float* deltas, float* egrads, const int* inLen,
+                  const int* labLen, const Dims& d, bool accumulate, hipStream_t s) {
+  if (d.B == 0 || d.T == 0 || d.U == 0) return kOk;
+  const int Up = wplane_up(d.U), Tw = wplane_tw(d.T);
+  // label axes longer than one LDS slice are contracted slice by slice, accumulating
+  for (int kofs = 0; kofs < Up; kofs += kEgMaxK) {
+    hipLaunchKernelGGL(egrads_kernel, dim3((d.V + 63) / 64, (d.T + 63) / 64, d.B), dim3(256), 0, s,
+                       E, P, mE, mP, Wn, deltas, egrads, inLen, labLen, d, Up, Tw, kofs,
+                       (accumulate || kofs > 0) ? 1 : 0, kofs + kEgMaxK >= Up ? 1 : 0);
+    RNNT_LAUNCH_CHECK("egrads_kernel");
+  }
+  return kOk;
+}
+
+int launch_pgrads(const float* E, const float* P, const float* mE, const float* mP,
+                  const float* Wt, const float* deltas, float* pgrads, const int* inLen,
+                  const int* labLen, const Dims& d, bool accumulate, hipStream_t s) {
+  if (d.B == 0 || d.T == 0 || d.U == 0) return kOk;
+  const int Up = wplane_up(d.U), Tw = wplane_tw(d.T);
+  hipLaunchKernelGGL(pgrads_kernel, dim3((d.V + 63) / 64, (d.U + 127) / 128, d.B), dim3(256), 0, s,
+                     E, P, mE, mP, Wt, deltas, pgrads, inLen, labLen, d, Up, Tw,
+                     accumulate ? 1 : 0);
+  RNNT_LAUNCH_CHECK("pgrads_kernel");
+  return kOk;
+}
+
+}  // namespace rnnt

@@ -1,0 +1,125 @@
+// Internal declarations shared by the HIP translation units of librnnt_hip.so.
+// Nothing here is part of the public interface (see include/rnnt_hip.h for that).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace rnnt {
+
+// ---------------------------------------------------------------- status / errors
+enum Status { kOk = 0, kInvalid = 1, kHipError = 2, kWorkspace = 3 };
+
+// Records a message for rnnt_hip_last_error() (thread-local) and returns `code`.
+int fail(int code, const char* fmt, ...);
+int check_hip(hipError_t e, const char* what, const char* file, int line);
+
+#define RNNT_HIP(call)                                                   \
+  do {                                                                   \
+    int _st = ::rnnt::check_hip((call), #call, __FILE__, __LINE__);      \
+    if (_st != ::rnnt::kOk) return _st;                                  \
+  } while (0)
+
+#define RNNT_TRY(expr)                 \
+  do {                                 \
+    int _st = (expr);                  \
+    if (_st != ::rnnt::kOk) return _st; \
+  } while (0)
+
+// ---------------------------------------------------------------- geometry
+// Problem sizes in the reference's vocabulary: U is the prediction length (longest label + 1).
+struct Dims {
+  int B, T, U, V, blank;
+  int Dp;  // row pitch of a skewed plane, in floats
+  int Tp;  // row pitch of the per-frame blank-score array
+};
+
+// A skewed plane stores cell (t,u) of utterance b at [(b*U + u)*Dp + (t+u)]: one row per label
+// position, indexed by anti-diagonal.  All lanes of the wavefront that walks the lattice then
+// read the same column index at the same step, so four consecutive steps are one aligned
+// 16-byte load per lane.  The pitch leaves room for the last partial group of four.
+__host__ __device__ inline int plane_pitch(int T, int U) { return ((T + U + 3) & ~3) + 8; }
+__host__ __device__ inline int frame_pitch(int T) { return ((T + 3) & ~3) + 8; }
+
+inline Dims make_dims(int B, int T, int U, int V, int blank) {
+  Dims d;
+  d.B = B; d.T = T; d.U = U; d.V = V; d.blank = blank;
+  d.Dp = plane_pitch(T, U);
+  d.Tp = frame_pitch(T);
+  return d;
+}
+
+__device__ inline int clampi(int x, int lo, int hi) { return x < lo ? lo : (x > hi ? hi : x); }
+
+// Per-utterance extents, clamped to the padded array so a bad length can never index past it.
+__device__ inline void utt_extent(const int* inLen, const int* labLen, int b, int T, int U,
+                                  int& Tb, int& Ub) {
+  Tb = inLen ? clampi(inLen[b], 0, T) : T;
+  Ub = labLen ? clampi(labLen[b] + 1, 0, U) : U;
+}
+
+// Buffers of the lattice recursions, all in the skewed layout except the three small vectors.
+struct Planes {
+  float* lnS;   // log-normaliser LN[t,u]
+  float* elS;   // E[t, label_u]  (label-move emission score of the cell)
+  float* aS;    // alpha
+  float* wB;    // blank-move weight exp(stay(t,u) - alpha[t+1,u])
+  float* wE;    // label-move weight exp(emit(t,u) - alpha[t,u+1])
+  float* dS;    // dalpha (= d cost / d LN)
+  float* eb;    // E[t, blank]           [B, Tp]
+  float* pb;    // P[u, blank]           [B, U]
+  float* pl;    // P[u, label_u]         [B, U]
+  float* gB;    // per-(b,u) blank-column sum of the sparse pgrads term   [B, U]
+  float* gL;    // per-(b,u) label-column sum of the sparse pgrads term   [B, U]
+};
+
+size_t planes_bytes(const Dims& d);
+void carve_planes(void* base, const Dims& d, Planes* p);
+
+// ---------------------------------------------------------------- launchers (rnnt_dp.hip)
+int launch_skew(const float* src, float* dstS, const int* inLen, const int* labLen, const Dims& d,
+                hipStream_t s);
+int launch_unskew(const float* srcS, float* dst, const int* inLen, const int* labLen,
+                  const Dims& d, hipStream_t s);
+int launch_gather(const float* E, const float* P, const int* labels, const int* inLen,
+                  const int* labLen, const Planes& p, const Dims& d, hipStream_t s);
+int launch_alpha(const Planes& p, const int* inLen, const int* labLen, float* costs,
+                 const Dims& d, hipStream_t s);
+int launch_weights(const Planes& p, const int* inLen, const int* labLen, const Dims& d,
+                   hipStream_t s);
+int launch_beta(const Planes& p, const int* labels, const int* inLen, const int* labLen,
+                const Dims& d, hipStream_t s);
+// Sparse blank/label terms.  add == false: written onto zero-filled egrads/pgrads exactly as
+// the reference's backward leaves them.  add == true: added, times scale[b] (1 when scale is
+// null), onto arrays that already hold the dense part.
+int launch_sparse(const Planes& p, float* egrads, float* pgrads, const int* labels,
+                  const int* inLen, const int* labLen, const float* scale, bool add,
+                  const Dims& d, hipStream_t s);
+int launch_maxplus(const float* E, const float* P, const int* inLen, const int* labLen,
+                   float* best, int* arg, const Dims& d, hipStream_t s);
+// bestS / argS: skewed planes of the max-plus table (argS carries int bits in float storage).
+int launch_viterbi(const Planes& p, const float* bestS, const float* argS,
+                   unsigned long long* gbits, const int* inLen, const int* labLen,
+                   int* labels_out, const Dims& d, hipStream_t s);
+size_t viterbi_bits_bytes(const Dims& d);
+
+// ---------------------------------------------------------------- launchers (rnnt_gemm.hip)
+int wplane_up(int U);  // label-axis pitch of the W planes (multiple of 8)
+int wplane_tw(int T);  // frame-axis pitch of the W planes (multiple of 64)
+int launch_rowmax(const float* X, float* rowmax, long rows, int V, hipStream_t s);
+int launch_lse(const float* E, const float* P, const float* mE, const float* mP, float* LN,
+               const int* inLen, const int* labLen, const Dims& d, hipStream_t s);
+int launch_wplanes(const float* lngrads, const float* LN, const float* mE, const float* mP,
+                   float* Wn, float* Wt, const int* inLen, const int* labLen, const Dims& d,
+                   hipStream_t s);
+// accumulate == false: out = delta * dense.   accumulate == true: out = delta * (out + dense),
+// the update of transducer/torch_binding.py:86-89.
+int launch_egrads(const float* E, const float* P, const float* mE, const float* mP,
+                  const float* Wn, const float* deltas, float* egrads, const int* inLen,
+                  const int* labLen, const Dims& d, bool accumulate, hipStream_t s);
+int launch_pgrads(const float* E, const float* P, const float* mE, const float* mP,
+                  const float* Wt, const float* deltas, float* pgrads, const int* inLen,
+                  const int* labLen, const Dims& d, bool accumulate, hipStream_t s);
+
+}  // namespace rnnt
