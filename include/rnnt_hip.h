@@ -108,6 +108,18 @@ int rnnt_hip_viterbi_decode(const float* emissions, const float* predictions,
                             const int* input_lengths, const int* label_lengths, int* labels,
                             int B, int T, int U, int V, int blank, rnnt_stream_t stream);
 
+/* ---- stage timing (diagnostic; no counterpart in the reference, whose only instrumentation
+ * is wall-clock loops in transducer/benchmark.cpp:21-34) ---------------------------------- */
+
+/* When enabled, every kernel stage of the calls above is bracketed with HIP events on the
+ * stream it runs on.  Not thread-safe; meant for one benchmarking thread. */
+int rnnt_hip_profile_enable(int on);
+int rnnt_hip_profile_stage_count(void);
+const char* rnnt_hip_profile_stage_name(int stage);
+/* Waits for the recorded events, writes per-stage total milliseconds and launch counts into
+ * the first n entries of the two HOST arrays, and clears the record. */
+int rnnt_hip_profile_read(double* total_ms, int* launches, int n);
+
 #ifdef __cplusplus
 }
 #endif

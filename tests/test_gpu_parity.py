@@ -1,0 +1,291 @@
+"""Parity of the HIP path with the CPU oracle, through the C interface of librnnt_hip.so.
+
+Boundary tests feed both sides the same log_norms (the contract of transducer.h: the
+normaliser is an input there), so the lattice recursions are compared on their own; the
+log-normaliser and the dense gradient kernels are gated separately; end-to-end runs close the
+loop.  Tolerance for costs and gradients: rel 1e-4 / abs 1e-5 in fp32; viterbi paths exact."""
+import numpy as np
+import pytest
+
+import oracle
+from transducer_amd.synthetic import CONFIGS, make_inputs, small_config
+from util import (DeviceCase, assert_close, check_close_reference, gpu_backward, gpu_dense_grads,
+                  gpu_forward, gpu_log_norms, gpu_loss, gpu_viterbi, ref_cases, reference_vectors,
+                  vector_case, violations)
+
+pytestmark = pytest.mark.gpu
+
+VEC = reference_vectors()
+CASES = ref_cases()
+KEYS = ("emissions", "predictions", "labels", "input_lengths", "label_lengths")
+
+
+def unpack(d):
+    return tuple(d[k] for k in KEYS)
+
+
+# ------------------------------------------------------------------ reference-held vectors
+@pytest.mark.parametrize("name", ["small", "big"])
+def test_golden_vectors_whole_loss(name):
+    v = VEC[name]
+    E, P, labels, il, ll = vector_case(v)
+    costs, eg, pg = gpu_loss(DeviceCase(E, P, labels, il, ll))
+    # the reference's own bar for these vectors (transducer/test.cpp:51,86-87)
+    check_close_reference(costs, v["costs"])
+    check_close_reference(eg, v["egrads"])
+    check_close_reference(pg, v["pgrads"])
+
+
+def test_tiny_closed_form_whole_loss():
+    E, P, labels, il, ll = vector_case(VEC["tiny"])
+    want = oracle.loss_and_grads(E, P, labels, il, ll, precision="f64")
+    costs, eg, pg = gpu_loss(DeviceCase(E, P, labels, il, ll))
+    check_close_reference(costs, want["costs"])
+    check_close_reference(eg, want["egrads"])
+    check_close_reference(pg, want["pgrads"])
+
+
+@pytest.mark.parametrize("name", ["viterbi_no_blanks", "viterbi_bigger"])
+def test_golden_viterbi(name):
+    v = VEC[name]
+    E, P, labels, il, ll = vector_case(v)
+    c = DeviceCase(E, P, labels, il, ll)
+    LN = oracle.log_norms_naive(E, P, il, ll)
+    assert np.array_equal(gpu_viterbi(c, LN), np.array(v["labels"], np.int32))
+
+
+def test_viterbi_empty_inputs_are_accepted():
+    # transducer/test.cpp:229-257
+    from transducer_amd import capi
+    from util import dev, ptr
+    il, ll = dev(np.array([0], np.int32)), dev(np.array([0], np.int32))
+    capi.call("rnnt_hip_viterbi", None, None, None, None, ptr(il), ptr(ll), 1, 0, 1, 2, 0, None)
+    E, P, labels, il, ll = vector_case(VEC["viterbi_empty_transcript"])
+    c = DeviceCase(E, P, labels, il, ll)
+    LN = oracle.log_norms_naive(E, P, il, ll)
+    assert gpu_viterbi(c, LN).shape == (1, 0)
+
+
+# ------------------------------------------------------------------ transducer.h boundary
+@pytest.mark.parametrize("name", sorted(CASES))
+def test_boundary_against_reference_fixture(name):
+    """forward / backward / viterbi with the fixture's log_norms against what the reference's
+    compiled CPU sources produced (ragged lengths, empty utterances, empty labels, ties)."""
+    f = CASES[name]
+    E, P, labels, il, ll = unpack(f)
+    c = DeviceCase(E, P, labels, il, ll)
+    LN = f["log_norms"]
+    costs, alphas = gpu_forward(c, LN)
+    assert np.array_equal(np.isinf(costs), np.isinf(f["costs"]))
+    assert_close(costs, f["costs"], what="costs")
+    assert np.array_equal(np.isnan(alphas), np.isnan(f["alphas"])), "cells outside must be untouched"
+    assert_close(alphas, f["alphas"], what="alphas")
+    eg, pg, lng = gpu_backward(c, f["alphas"], LN)
+    assert_close(lng, f["lngrads"], what="lngrads")
+    assert_close(eg, f["egrads_sparse"], what="egrads (sparse)")
+    assert_close(pg, f["pgrads_sparse"], what="pgrads (sparse)")
+    if "viterbi" in f:
+        got = gpu_viterbi(c, LN)
+        assert np.array_equal(got, f["viterbi"])
+
+
+def long_case(B, V, seed, sigma=1.0, ragged=True, T=2000, U=100):
+    cfg = small_config(B, T, U, V, sigma=sigma, ragged=ragged)
+    return unpack(make_inputs(cfg, seed=seed))
+
+
+@pytest.mark.parametrize("V,sigma,ragged", [(100, 1.0, False), (300, 2.0, True)])
+def test_boundary_at_T2000(V, sigma, ragged):
+    """The lattice at its real length.  alpha reaches ~1e4 here (ulp ~1e-3), so gradients only
+    agree if the rounding sequence of every cell follows the reference."""
+    E, P, labels, il, ll = long_case(2, V, seed=21, sigma=sigma, ragged=ragged)
+    LN = oracle.log_norms_naive(E, P, il, ll)
+    costs_o, alphas_o = oracle.forward(E, P, LN, labels, il, ll)
+    c = DeviceCase(E, P, labels, il, ll)
+    costs, alphas = gpu_forward(c, LN)
+    m = ~np.isnan(alphas_o)
+    exact = float((alphas[m] == alphas_o[m]).mean())
+    assert exact > 0.95, "alphas bit-exact in only %.3f of cells" % exact
+    assert_close(costs, costs_o, what="costs")
+    assert_close(alphas[m], alphas_o[m], what="alphas")
+    # backward from the device's own alphas, as a caller would chain the two calls
+    eg, pg, lng = gpu_backward(c, alphas, LN)
+    eg_o, pg_o, lng_o = oracle.backward(E, P, np.nan_to_num(alphas_o), LN, labels, il, ll)
+    assert_close(lng, lng_o, what="lngrads")
+    assert_close(eg, eg_o, what="egrads (sparse)")
+    assert_close(pg, pg_o, what="pgrads (sparse)")
+    # every path crosses each anti-diagonal exactly once
+    for b in range(E.shape[0]):
+        Tb, Ub = il[b], ll[b] + 1
+        g = lng[b, :Tb, :Ub].astype(np.float64)
+        diag = np.array([np.trace(g[::-1], offset=k) for k in range(-(Tb - 1), Ub)])
+        assert np.abs(diag - 1.0).max() < 2e-2
+
+
+@pytest.mark.parametrize("near_ties", [False, True])
+def test_viterbi_at_T2000_is_bit_exact(near_ties):
+    cfg = small_config(3, 2000, 100, 64, ragged=True)
+    d = make_inputs(cfg, seed=31, near_ties=near_ties)
+    E, P, labels, il, ll = unpack(d)
+    LN = oracle.log_norms_naive(E, P, il, ll)
+    want = oracle.viterbi(E, P, LN, il, ll)
+    got = gpu_viterbi(DeviceCase(E, P, labels, il, ll), LN)
+    assert np.array_equal(got, want)
+
+
+def test_viterbi_label_equal_to_nonzero_blank():
+    cfg = small_config(2, 40, 12, 9, ragged=True)
+    E, P, labels, il, ll = unpack(make_inputs(cfg, seed=4))
+    LN = oracle.log_norms_naive(E, P, il, ll)
+    for blank in (3, 8):
+        want = oracle.viterbi(E, P, LN, il, ll, blank=blank)
+        got = gpu_viterbi(DeviceCase(E, P, labels, il, ll), LN, blank=blank)
+        assert np.array_equal(got, want)
+
+
+def test_labels_may_repeat_and_equal_blank():
+    # transducer/benchmark.cpp:47 draws labels from [0,V): blank may appear as a label
+    cfg = small_config(3, 30, 8, 5, ragged=True)
+    E, P, labels, il, ll = unpack(make_inputs(cfg, seed=8))
+    labels = labels.copy()
+    labels[:, ::2] = 0
+    labels[:, 1::2] = 2
+    LN = oracle.log_norms_naive(E, P, il, ll)
+    costs_o, alphas_o = oracle.forward(E, P, LN, labels, il, ll)
+    eg_o, pg_o, lng_o = oracle.backward(E, P, np.nan_to_num(alphas_o), LN, labels, il, ll)
+    c = DeviceCase(E, P, labels, il, ll)
+    costs, alphas = gpu_forward(c, LN)
+    assert_close(costs, costs_o, what="costs")
+    eg, pg, lng = gpu_backward(c, alphas_o, LN)
+    assert_close(eg, eg_o, what="egrads (sparse)")
+    assert_close(pg, pg_o, what="pgrads (sparse)")
+    assert_close(lng, lng_o, what="lngrads")
+
+
+def test_long_label_axis_uses_more_cells_per_lane():
+    cfg = small_config(2, 60, 300, 11, ragged=True)
+    E, P, labels, il, ll = unpack(make_inputs(cfg, seed=12))
+    LN = oracle.log_norms_naive(E, P, il, ll)
+    costs_o, alphas_o = oracle.forward(E, P, LN, labels, il, ll)
+    c = DeviceCase(E, P, labels, il, ll)
+    costs, alphas = gpu_forward(c, LN)
+    assert_close(costs, costs_o, what="costs")
+    eg, pg, lng = gpu_backward(c, alphas_o, LN)
+    eg_o, pg_o, lng_o = oracle.backward(E, P, np.nan_to_num(alphas_o), LN, labels, il, ll)
+    assert_close(lng, lng_o, what="lngrads")
+    assert_close(eg, eg_o, what="egrads")
+    assert np.array_equal(gpu_viterbi(c, LN), oracle.viterbi(E, P, LN, il, ll))
+
+
+# ------------------------------------------------------------------ log-normaliser
+@pytest.mark.parametrize("B,T,U,V,sigma", [(2, 70, 9, 31, 1.0), (1, 200, 101, 1000, 2.0),
+                                           (3, 129, 130, 257, 1.0), (1, 64, 17, 4099, 3.0)])
+def test_log_norms_against_fp64(B, T, U, V, sigma):
+    cfg = small_config(B, T, U - 1, V, sigma=sigma, ragged=True)
+    E, P, labels, il, ll = unpack(make_inputs(cfg, seed=V))
+    c = DeviceCase(E, P, labels, il, ll)
+    truth = oracle.log_norms_truth(E, P)
+    got = gpu_log_norms(c, with_lengths=False)
+    # Bar: a few ulp of LN (|LN| ~ 10-20), and never worse than the reference's own two fp32
+    # forms (test.h naive sum, torch_binding separable sum), whose error grows when a handful
+    # of terms dominate a long sum (sigma=3 case).
+    floor = max(np.abs(oracle.log_norms_naive(E, P) - truth).max(),
+                np.abs(oracle.log_norms_sep(E, P) - truth).max())
+    tol = max(4e-6, 1.25 * floor)
+    assert np.abs(got - truth).max() < tol
+    got = gpu_log_norms(c, with_lengths=True)
+    masked = oracle.log_norms_truth(E, P, il, ll)
+    assert np.abs(got - masked).max() < tol
+    for b in range(B):
+        assert not got[b, il[b]:].any() and not got[b, :, ll[b] + 1:].any()
+
+
+def test_log_norms_wide_dynamic_range():
+    # maxima of the two operands at different v: the separable shift must not lose the sum
+    rng = np.random.default_rng(0)
+    E = rng.standard_normal((1, 40, 500)).astype(np.float32)
+    P = rng.standard_normal((1, 6, 500)).astype(np.float32)
+    E[0, :, 7] += 25.0
+    P[0, :, 300] += 30.0
+    c = DeviceCase(E, P, np.zeros((1, 5), np.int32), np.array([40], np.int32),
+                   np.array([5], np.int32))
+    got = gpu_log_norms(c, with_lengths=False)
+    truth = oracle.log_norms_truth(E, P)
+    assert np.abs(got - truth).max() < 1e-5
+
+
+# ------------------------------------------------------------------ dense gradient kernels
+@pytest.mark.parametrize("B,T,U,V", [(2, 50, 11, 32), (2, 130, 101, 333), (1, 300, 140, 64)])
+def test_dense_grads_against_oracle(B, T, U, V):
+    cfg = small_config(B, T, U - 1, V, ragged=True)
+    E, P, labels, il, ll = unpack(make_inputs(cfg, seed=T))
+    LN = oracle.log_norms_naive(E, P, il, ll)
+    _, alphas = oracle.forward(E, P, LN, labels, il, ll)
+    eg, pg, lng = oracle.backward(E, P, np.nan_to_num(alphas), LN, labels, il, ll)
+    deltas = np.linspace(0.5, 1.5, B).astype(np.float32)
+    want_e, want_p = oracle.accumulate_grads(E.astype(np.float64), P.astype(np.float64), eg, pg,
+                                             lng, LN, il, ll, precision="f64")
+    want_e *= deltas[:, None, None]
+    want_p *= deltas[:, None, None]
+    got_e, got_p = gpu_dense_grads(DeviceCase(E, P, labels, il, ll), eg, pg, lng, LN, deltas)
+    assert_close(got_e, want_e, what="egrads")
+    assert_close(got_p, want_p, what="pgrads")
+    for b in range(B):
+        assert not got_e[b, il[b]:].any() and not got_p[b, ll[b] + 1:].any()
+
+
+# ------------------------------------------------------------------ end to end
+@pytest.mark.parametrize("cfg,seed", [("cfg1", 0), ("cfg1", 1)])
+def test_whole_loss_cfg1(cfg, seed):
+    E, P, labels, il, ll = unpack(make_inputs(CONFIGS[cfg], seed=seed))
+    want = oracle.loss_and_grads(E, P, labels, il, ll)
+    costs, eg, pg = gpu_loss(DeviceCase(E, P, labels, il, ll))
+    assert_close(costs, want["costs"], what="costs")
+    assert_close(eg, want["egrads"], what="egrads")
+    assert_close(pg, want["pgrads"], what="pgrads")
+    if seed == 0:  # same inputs as the fixture the reference's compiled sources produced
+        f = CASES["cfg1"]
+        assert_close(costs, f["costs"], what="costs vs reference fixture")
+        assert_close(eg, f["egrads"], what="egrads vs reference fixture")
+        assert_close(pg, f["pgrads"], what="pgrads vs reference fixture")
+
+
+def test_whole_loss_handles_empty_utterance_and_empty_label():
+    cfg = small_config(4, 20, 6, 12, ragged=True)
+    E, P, labels, il, ll = unpack(make_inputs(cfg, seed=2))
+    il, ll = il.copy(), ll.copy()
+    il[1] = 0
+    ll[2] = 0
+    want = oracle.loss_and_grads(E, P, labels, il, ll)
+    costs, eg, pg = gpu_loss(DeviceCase(E, P, labels, il, ll))
+    assert np.isposinf(costs[1])
+    fin = np.isfinite(want["costs"])
+    assert_close(costs[fin], want["costs"][fin], what="costs")
+    assert_close(eg, want["egrads"], what="egrads")
+    assert_close(pg, want["pgrads"], what="pgrads")
+    assert not eg[1].any() and not pg[1].any()
+
+
+def test_whole_loss_at_T2000_violation_fraction():
+    """End to end at the real lattice length.  The two sides compute LN with different summation
+    orders, and the reference's gradients are sensitive to the last bits of LN (its own fp32
+    result moves by more than the tolerance when LN moves by a few ulp); so the bar here is a
+    bounded violation fraction next to the oracle's own floor between two LN orders."""
+    E, P, labels, il, ll = long_case(2, 100, seed=5)
+    a = oracle.loss_and_grads(E, P, labels, il, ll, lse="naive")
+    b = oracle.loss_and_grads(E, P, labels, il, ll, lse="sep")
+    floor_e, _ = violations(b["egrads"], a["egrads"])
+    floor_p, _ = violations(b["pgrads"], a["pgrads"])
+    costs, eg, pg = gpu_loss(DeviceCase(E, P, labels, il, ll))
+    assert_close(costs, a["costs"], rtol=1e-4, atol=1e-3, what="costs")
+    ve, worst_e = violations(eg, a["egrads"])
+    vp, worst_p = violations(pg, a["pgrads"])
+    print("violations egrads %.4f%% (oracle floor %.4f%%), pgrads %.4f%% (floor %.4f%%); "
+          "max abs err %.3g / %.3g" % (100 * ve, 100 * floor_e, 100 * vp, 100 * floor_p,
+                                       worst_e, worst_p))
+    assert ve <= max(2 * floor_e, 0.02) and vp <= max(2 * floor_p, 0.02)
+    # fp64 truth: the device result must not be further from it than the reference's fp32 is
+    t = oracle.loss_and_grads(E, P, labels, il, ll, precision="f64")
+    err_dev = np.abs(eg - t["egrads"]).max()
+    err_ref = np.abs(a["egrads"] - t["egrads"]).max()
+    assert err_dev < 4 * err_ref + 1e-5

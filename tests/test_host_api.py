@@ -1,0 +1,133 @@
+"""Host-side checks that need no GPU: the shared libraries load, export what the headers
+declare, reject bad arguments before touching the device, and the Python front end keeps the
+reference's checks and messages (transducer/torch_binding.py:180-229)."""
+import ctypes
+import os
+import re
+import subprocess
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+PKG = os.path.join(ROOT, "transducer_amd")
+
+
+def test_c_interface_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "rnnt_hip.h")).read()
+    declared = sorted(set(re.findall(r"\b(rnnt_hip_\w+)\s*\(", header)))
+    assert len(declared) >= 14
+    lib = ctypes.CDLL(os.path.join(PKG, "librnnt_hip.so"))
+    for name in declared:
+        assert hasattr(lib, name), name
+    from transducer_amd import capi
+    assert sorted(capi.SIGNATURES) == declared
+
+
+def test_cxx_interface_exports_the_three_reference_functions():
+    out = subprocess.check_output(["nm", "-DC", os.path.join(PKG, "libtransducer.so")], text=True)
+    sig = r"float const\*, float const\*"
+    assert re.search(r" T forward\(" + sig, out)
+    assert re.search(r" T backward\(" + sig, out)
+    assert re.search(r" T viterbi\(" + sig, out)
+    # and with exactly the reference's parameter lists (transducer/transducer.h:3-49)
+    assert ("forward(float const*, float const*, float*, float*, float const*, int const*, "
+            "int const*, int const*, int, int, int, int, int, bool)") in out
+    assert ("backward(float const*, float const*, float*, float*, float*, float const*, "
+            "float const*, int const*, int const*, int const*, int, int, int, int, int, bool)") in out
+    assert ("viterbi(float const*, float const*, float const*, int*, int const*, int const*, "
+            "int, int, int, int, int, bool)") in out
+
+
+def test_bad_sizes_are_rejected_before_any_device_work():
+    from transducer_amd import capi
+    lib = capi.load()
+    assert lib.rnnt_hip_forward(None, None, None, None, None, None, None, None,
+                                -1, 1, 1, 1, 0, None) == 1
+    assert b"negative size" in lib.rnnt_hip_last_error()
+    assert lib.rnnt_hip_log_norms(None, None, None, None, None, 1, 70000, 2, 70000, None) == 1
+    assert b"2^31" in lib.rnnt_hip_last_error()
+    with pytest.raises(capi.RnntHipError):
+        capi.call("rnnt_hip_backward", None, None, None, None, None, None, None, None, None, None,
+                  1, 1, -3, 1, 0, None)
+    # empty batch: nothing to do, no device needed
+    assert lib.rnnt_hip_forward(None, None, None, None, None, None, None, None,
+                                0, 5, 3, 4, 0, None) == 0
+    assert lib.rnnt_hip_loss_workspace_bytes(32, 2000, 101, 10000) < 400 * 2**20
+
+
+def test_workspace_is_order_BTU_not_BTUV():
+    from transducer_amd import capi
+    lib = capi.load()
+    small = lib.rnnt_hip_loss_workspace_bytes(8, 2000, 101, 100)
+    large = lib.rnnt_hip_loss_workspace_bytes(8, 2000, 101, 10000)
+    assert small == large
+
+
+def test_pybind_module_has_the_reference_keyword_names():
+    from transducer_amd import _transducer
+    doc = _transducer.forward.__doc__
+    for kw in ("emissions", "predictions", "costs", "alphas", "logNorms", "labels",
+               "input_lengths", "label_lengths", "batch_size", "max_input_length",
+               "max_label_length", "alphabet_size", "blank", "use_cuda"):
+        assert kw + ":" in doc
+    assert "log_norms:" in _transducer.viterbi.__doc__  # the reference spells it differently here
+    assert "lngrads:" in _transducer.backward.__doc__
+    assert isinstance(_transducer.__version__, str)
+
+
+def test_host_pointers_raise_like_a_backend_that_was_not_built():
+    from transducer_amd import _transducer
+    with pytest.raises(ValueError, match="not built with the CPU backend"):
+        _transducer.forward(0, 0, 0, 0, 0, 0, 0, 0, 1, 1, 1, 2, 0, False)
+    with pytest.raises(ValueError, match="not built with the CPU backend"):
+        _transducer.backward(0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 1, 1, 1, 2, 0, False)
+    with pytest.raises(ValueError, match="not built with the CPU backend"):
+        _transducer.viterbi(0, 0, 0, 0, 0, 0, 1, 1, 1, 2, 0, False)
+
+
+def _inputs(B=2, T=5, U=3, V=4):
+    E = torch.rand(B, T, V)
+    P = torch.rand(B, U, V)
+    labels = torch.randint(1, V, (B, U - 1), dtype=torch.int32)
+    il = torch.full((B,), T, dtype=torch.int32)
+    ll = torch.full((B,), U - 1, dtype=torch.int32)
+    return E, P, labels, il, ll
+
+
+def test_certify_inputs_messages():
+    from transducer_amd.torch_binding import certify_inputs
+    E, P, labels, il, ll = _inputs()
+    certify_inputs(E, P, labels, il, ll)
+    with pytest.raises(TypeError, match="emissions must be torch.float32"):
+        certify_inputs(E.double(), P, labels, il, ll)
+    with pytest.raises(TypeError, match="labels must be torch.int32"):
+        certify_inputs(E, P, labels.long(), il, ll)
+    with pytest.raises(TypeError, match="input_lengths must be torch.int32"):
+        certify_inputs(E, P, labels, il.long(), ll)
+    with pytest.raises(ValueError, match="labels must be contiguous"):
+        certify_inputs(E, P, labels.t().contiguous().t(), il, ll)
+    with pytest.raises(ValueError, match="vocab size mismatch."):
+        certify_inputs(E, P[:, :, :3].contiguous(), labels, il, ll)
+    with pytest.raises(ValueError, match="must have a length per example."):
+        certify_inputs(E, P, labels, il[:1], ll)
+    with pytest.raises(ValueError, match="must have a label length per example."):
+        certify_inputs(E, P, labels, il, ll[:1])
+    with pytest.raises(ValueError, match="must have a label per example."):
+        certify_inputs(E, P, labels[:1], il, ll)
+    with pytest.raises(ValueError, match="labels must be padded to maximum label length."):
+        certify_inputs(E, P, labels[:, :1].contiguous(), il, ll)
+    with pytest.raises(ValueError, match="Input length mismatch"):
+        certify_inputs(E, P, labels, il + 1, ll)
+    with pytest.raises(ValueError, match="Output length mismatch"):
+        certify_inputs(E, P, labels, il, ll + 1)
+
+
+def test_loss_on_host_tensors_fails_loudly():
+    from transducer_amd import TransducerLoss
+    E, P, labels, il, ll = _inputs()
+    with pytest.raises(ValueError, match="not built with the CPU backend"):
+        TransducerLoss()(E, P, labels, il, ll)
+    with pytest.raises(ValueError, match="not built with the CPU backend"):
+        TransducerLoss().viterbi(E, P, il, ll)
+    assert TransducerLoss(blank=3).blank == 3

@@ -23,6 +23,10 @@ SIGNATURES = {
     "rnnt_hip_loss_forward": (_I, [_F] * 7 + [_Z] + [_I] * 5 + [_F]),
     "rnnt_hip_loss_backward": (_I, [_F] * 9 + [_Z] + [_I] * 5 + [_F]),
     "rnnt_hip_viterbi_decode": (_I, [_F] * 5 + [_I] * 5 + [_F]),
+    "rnnt_hip_profile_enable": (_I, [_I]),
+    "rnnt_hip_profile_stage_count": (_I, []),
+    "rnnt_hip_profile_stage_name": (ctypes.c_char_p, [_I]),
+    "rnnt_hip_profile_read": (_I, [_F, _F, _I]),
 }
 
 _lib = None
@@ -54,3 +58,17 @@ def call(name, *args):
     if status != 0:
         raise RnntHipError("{} failed ({}): {}".format(
             name, status, lib.rnnt_hip_last_error().decode()))
+
+
+def profile_enable(on):
+    call("rnnt_hip_profile_enable", 1 if on else 0)
+
+
+def profile_read():
+    """-> {stage name: (total milliseconds, launches)} since profiling was enabled / last read."""
+    lib = load()
+    n = lib.rnnt_hip_profile_stage_count()
+    ms = (ctypes.c_double * n)()
+    cnt = (ctypes.c_int * n)()
+    call("rnnt_hip_profile_read", ctypes.cast(ms, _F), ctypes.cast(cnt, _F), n)
+    return {lib.rnnt_hip_profile_stage_name(i).decode(): (ms[i], cnt[i]) for i in range(n)}

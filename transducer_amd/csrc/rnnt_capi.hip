@@ -24,6 +24,53 @@ int check_hip(hipError_t e, const char* what, const char* file, int line) {
   return fail(kHipError, "[%s:%d] HIP error: %s (%s)", file, line, hipGetErrorString(e), what);
 }
 
+// ---------------------------------------------------------------- stage timing
+// Optional HIP-event brackets around every kernel stage, on the stream the stage runs on.
+// A single-threaded diagnostic: enable, run, read.  Off by default and free when off.
+namespace prof {
+
+enum Stage {
+  kRowmax, kLse, kSkew, kGather, kAlpha, kUnskew, kWeights, kBeta, kWplanes, kEgrads, kPgrads,
+  kSparse, kMaxplus, kViterbi, kClear, kNumStages
+};
+const char* const kNames[kNumStages] = {"rowmax", "lse", "skew", "gather", "alpha", "unskew",
+                                        "weights", "beta", "wplanes", "egrads", "pgrads",
+                                        "sparse", "maxplus", "viterbi", "clear"};
+constexpr int kMaxRecords = 8192;
+struct Record { int stage; hipEvent_t begin, end; };
+
+bool g_on = false;
+Record g_rec[kMaxRecords];
+int g_used = 0, g_created = 0;
+
+struct Scope {
+  Record* r = nullptr;
+  hipStream_t s;
+  Scope(int stage, hipStream_t stream) : s(stream) {
+    if (!g_on || g_used == kMaxRecords) return;
+    if (g_used == g_created) {
+      if (hipEventCreate(&g_rec[g_created].begin) != hipSuccess) return;
+      if (hipEventCreate(&g_rec[g_created].end) != hipSuccess) return;
+      ++g_created;
+    }
+    r = &g_rec[g_used++];
+    r->stage = stage;
+    (void)hipEventRecord(r->begin, s);
+  }
+  ~Scope() {
+    if (r) (void)hipEventRecord(r->end, s);
+  }
+};
+
+}  // namespace prof
+
+#define RNNT_STAGE(stage, expr)             \
+  do {                                      \
+    ::rnnt::prof::Scope _scope(::rnnt::prof::stage, s); \
+    int _st = (expr);                       \
+    if (_st != ::rnnt::kOk) return _st;     \
+  } while (0)
+
 namespace {
 
 size_t align_up(size_t x) { return (x + 255) & ~(size_t)255; }
@@ -116,6 +163,28 @@ extern "C" {
 const char* rnnt_hip_last_error(void) { return g_error; }
 int rnnt_hip_abi_version(void) { return 1; }
 
+int rnnt_hip_profile_enable(int on) {
+  prof::g_on = on != 0;
+  if (on) prof::g_used = 0;
+  return kOk;
+}
+int rnnt_hip_profile_stage_count(void) { return prof::kNumStages; }
+const char* rnnt_hip_profile_stage_name(int i) {
+  return (i >= 0 && i < prof::kNumStages) ? prof::kNames[i] : "";
+}
+int rnnt_hip_profile_read(double* total_ms, int* launches, int n) {
+  for (int i = 0; i < n; ++i) { total_ms[i] = 0.0; launches[i] = 0; }
+  for (int i = 0; i < prof::g_used; ++i) {
+    prof::Record& r = prof::g_rec[i];
+    RNNT_HIP(hipEventSynchronize(r.end));
+    float ms = 0.0f;
+    RNNT_HIP(hipEventElapsedTime(&ms, r.begin, r.end));
+    if (r.stage < n) { total_ms[r.stage] += ms; launches[r.stage] += 1; }
+  }
+  prof::g_used = 0;
+  return kOk;
+}
+
 int rnnt_hip_forward(const float* E, const float* P, float* costs, float* alphas, const float* LN,
                      const int* labels, const int* inLen, const int* labLen, int B, int T, int U,
                      int V, int blank, rnnt_stream_t stream) {
@@ -131,10 +200,10 @@ int rnnt_hip_forward(const float* E, const float* P, float* costs, float* alphas
   RNNT_TRY(scratch.reserve(planes_bytes(d)));
   Planes p;
   carve_planes(scratch.take(planes_bytes(d)), d, &p);
-  RNNT_TRY(launch_skew(LN, p.lnS, inLen, labLen, d, s));
-  RNNT_TRY(launch_gather(E, P, labels, inLen, labLen, p, d, s));
-  RNNT_TRY(launch_alpha(p, inLen, labLen, costs, d, s));
-  RNNT_TRY(launch_unskew(p.aS, alphas, inLen, labLen, d, s));
+  RNNT_STAGE(kSkew, launch_skew(LN, p.lnS, inLen, labLen, d, s));
+  RNNT_STAGE(kGather, launch_gather(E, P, labels, inLen, labLen, p, d, s));
+  RNNT_STAGE(kAlpha, launch_alpha(p, inLen, labLen, costs, d, s));
+  RNNT_STAGE(kUnskew, launch_unskew(p.aS, alphas, inLen, labLen, d, s));
   return kOk;
 }
 
@@ -146,9 +215,12 @@ int rnnt_hip_backward(const float* E, const float* P, float* egrads, float* pgra
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (B == 0) return kOk;
   // transducer_cuda.cu:326-331: the library clears all three outputs itself
-  if (egrads && (size_t)T * V) RNNT_HIP(hipMemsetAsync(egrads, 0, sizeof(float) * (size_t)B * T * V, s));
-  if (pgrads && (size_t)U * V) RNNT_HIP(hipMemsetAsync(pgrads, 0, sizeof(float) * (size_t)B * U * V, s));
-  if (lngrads && (size_t)T * U) RNNT_HIP(hipMemsetAsync(lngrads, 0, sizeof(float) * (size_t)B * T * U, s));
+  {
+    prof::Scope scope(prof::kClear, s);
+    if (egrads && (size_t)T * V) RNNT_HIP(hipMemsetAsync(egrads, 0, sizeof(float) * (size_t)B * T * V, s));
+    if (pgrads && (size_t)U * V) RNNT_HIP(hipMemsetAsync(pgrads, 0, sizeof(float) * (size_t)B * U * V, s));
+    if (lngrads && (size_t)T * U) RNNT_HIP(hipMemsetAsync(lngrads, 0, sizeof(float) * (size_t)B * T * U, s));
+  }
   if (nothing_to_do(B, T, U) || V == 0) return kOk;
   if (!E || !P || !egrads || !pgrads || !lngrads || !alphas || !LN || !inLen || !labLen ||
       (U > 1 && !labels))
@@ -158,13 +230,13 @@ int rnnt_hip_backward(const float* E, const float* P, float* egrads, float* pgra
   RNNT_TRY(scratch.reserve(planes_bytes(d)));
   Planes p;
   carve_planes(scratch.take(planes_bytes(d)), d, &p);
-  RNNT_TRY(launch_skew(LN, p.lnS, inLen, labLen, d, s));
-  RNNT_TRY(launch_skew(alphas, p.aS, inLen, labLen, d, s));
-  RNNT_TRY(launch_gather(E, P, labels, inLen, labLen, p, d, s));
-  RNNT_TRY(launch_weights(p, inLen, labLen, d, s));
-  RNNT_TRY(launch_beta(p, labels, inLen, labLen, d, s));
-  RNNT_TRY(launch_unskew(p.dS, lngrads, inLen, labLen, d, s));
-  RNNT_TRY(launch_sparse(p, egrads, pgrads, labels, inLen, labLen, nullptr, false, d, s));
+  RNNT_STAGE(kSkew, launch_skew(LN, p.lnS, inLen, labLen, d, s));
+  RNNT_STAGE(kSkew, launch_skew(alphas, p.aS, inLen, labLen, d, s));
+  RNNT_STAGE(kGather, launch_gather(E, P, labels, inLen, labLen, p, d, s));
+  RNNT_STAGE(kWeights, launch_weights(p, inLen, labLen, d, s));
+  RNNT_STAGE(kBeta, launch_beta(p, labels, inLen, labLen, d, s));
+  RNNT_STAGE(kUnskew, launch_unskew(p.dS, lngrads, inLen, labLen, d, s));
+  RNNT_STAGE(kSparse, launch_sparse(p, egrads, pgrads, labels, inLen, labLen, nullptr, false, d, s));
   return kOk;
 }
 
@@ -183,13 +255,13 @@ static int viterbi_impl(const float* E, const float* P, const float* LN, int* la
   float* argS = static_cast<float*>(scratch.take(plane));
   unsigned long long* bits =
       static_cast<unsigned long long*>(scratch.take(viterbi_bits_bytes(d)));
-  RNNT_TRY(launch_maxplus(E, P, inLen, labLen, best, arg, d, s));
-  RNNT_TRY(launch_skew(LN, p.lnS, inLen, labLen, d, s));
-  RNNT_TRY(launch_skew(best, bestS, inLen, labLen, d, s));
-  RNNT_TRY(launch_skew(reinterpret_cast<const float*>(arg), argS, inLen, labLen, d, s));
+  RNNT_STAGE(kMaxplus, launch_maxplus(E, P, inLen, labLen, best, arg, d, s));
+  RNNT_STAGE(kSkew, launch_skew(LN, p.lnS, inLen, labLen, d, s));
+  RNNT_STAGE(kSkew, launch_skew(best, bestS, inLen, labLen, d, s));
+  RNNT_STAGE(kSkew, launch_skew(reinterpret_cast<const float*>(arg), argS, inLen, labLen, d, s));
   // blank scores only: the label planes of the gather are not needed here
-  RNNT_TRY(launch_gather(E, P, nullptr, inLen, labLen, p, d, s));
-  RNNT_TRY(launch_viterbi(p, bestS, argS, bits, inLen, labLen, labels, d, s));
+  RNNT_STAGE(kGather, launch_gather(E, P, nullptr, inLen, labLen, p, d, s));
+  RNNT_STAGE(kViterbi, launch_viterbi(p, bestS, argS, bits, inLen, labLen, labels, d, s));
   return kOk;
 }
 
@@ -217,9 +289,9 @@ int rnnt_hip_log_norms(const float* E, const float* P, float* LN, const int* inL
                            align_up(sizeof(float) * (size_t)B * U)));
   float* mE = static_cast<float*>(scratch.take(sizeof(float) * (size_t)B * T));
   float* mP = static_cast<float*>(scratch.take(sizeof(float) * (size_t)B * U));
-  RNNT_TRY(launch_rowmax(E, mE, (long)B * T, V, s));
-  RNNT_TRY(launch_rowmax(P, mP, (long)B * U, V, s));
-  RNNT_TRY(launch_lse(E, P, mE, mP, LN, inLen, labLen, d, s));
+  RNNT_STAGE(kRowmax, launch_rowmax(E, mE, (long)B * T, V, s));
+  RNNT_STAGE(kRowmax, launch_rowmax(P, mP, (long)B * U, V, s));
+  RNNT_STAGE(kLse, launch_lse(E, P, mE, mP, LN, inLen, labLen, d, s));
   return kOk;
 }
 
@@ -241,11 +313,11 @@ int rnnt_hip_dense_grads(const float* E, const float* P, float* egrads, float* p
   float* mP = static_cast<float*>(scratch.take(sizeof(float) * (size_t)B * U));
   float* Wn = static_cast<float*>(scratch.take(wb));
   float* Wt = static_cast<float*>(scratch.take(wb));
-  RNNT_TRY(launch_rowmax(E, mE, (long)B * T, V, s));
-  RNNT_TRY(launch_rowmax(P, mP, (long)B * U, V, s));
-  RNNT_TRY(launch_wplanes(lngrads, LN, mE, mP, Wn, Wt, inLen, labLen, d, s));
-  RNNT_TRY(launch_egrads(E, P, mE, mP, Wn, deltas, egrads, inLen, labLen, d, true, s));
-  RNNT_TRY(launch_pgrads(E, P, mE, mP, Wt, deltas, pgrads, inLen, labLen, d, true, s));
+  RNNT_STAGE(kRowmax, launch_rowmax(E, mE, (long)B * T, V, s));
+  RNNT_STAGE(kRowmax, launch_rowmax(P, mP, (long)B * U, V, s));
+  RNNT_STAGE(kWplanes, launch_wplanes(lngrads, LN, mE, mP, Wn, Wt, inLen, labLen, d, s));
+  RNNT_STAGE(kEgrads, launch_egrads(E, P, mE, mP, Wn, deltas, egrads, inLen, labLen, d, true, s));
+  RNNT_STAGE(kPgrads, launch_pgrads(E, P, mE, mP, Wt, deltas, pgrads, inLen, labLen, d, true, s));
   return kOk;
 }
 
@@ -273,12 +345,12 @@ int rnnt_hip_loss_forward(const float* E, const float* P, const int* labels, con
   const Dims d = make_dims(B, T, U, V, blank);
   LossWorkspace w;
   loss_workspace_layout(d, workspace, &w);
-  RNNT_TRY(launch_rowmax(E, w.mE, (long)B * T, V, s));
-  RNNT_TRY(launch_rowmax(P, w.mP, (long)B * U, V, s));
-  RNNT_TRY(launch_lse(E, P, w.mE, w.mP, w.LN, inLen, labLen, d, s));
-  RNNT_TRY(launch_skew(w.LN, w.planes.lnS, inLen, labLen, d, s));
-  RNNT_TRY(launch_gather(E, P, labels, inLen, labLen, w.planes, d, s));
-  RNNT_TRY(launch_alpha(w.planes, inLen, labLen, costs, d, s));
+  RNNT_STAGE(kRowmax, launch_rowmax(E, w.mE, (long)B * T, V, s));
+  RNNT_STAGE(kRowmax, launch_rowmax(P, w.mP, (long)B * U, V, s));
+  RNNT_STAGE(kLse, launch_lse(E, P, w.mE, w.mP, w.LN, inLen, labLen, d, s));
+  RNNT_STAGE(kSkew, launch_skew(w.LN, w.planes.lnS, inLen, labLen, d, s));
+  RNNT_STAGE(kGather, launch_gather(E, P, labels, inLen, labLen, w.planes, d, s));
+  RNNT_STAGE(kAlpha, launch_alpha(w.planes, inLen, labLen, costs, d, s));
   return kOk;
 }
 
@@ -304,13 +376,13 @@ int rnnt_hip_loss_backward(const float* E, const float* P, const int* labels, co
   const Dims d = make_dims(B, T, U, V, blank);
   LossWorkspace w;
   loss_workspace_layout(d, workspace, &w);
-  RNNT_TRY(launch_weights(w.planes, inLen, labLen, d, s));
-  RNNT_TRY(launch_beta(w.planes, labels, inLen, labLen, d, s));
-  RNNT_TRY(launch_unskew(w.planes.dS, w.lngrads, inLen, labLen, d, s));
-  RNNT_TRY(launch_wplanes(w.lngrads, w.LN, w.mE, w.mP, w.Wn, w.Wt, inLen, labLen, d, s));
-  RNNT_TRY(launch_egrads(E, P, w.mE, w.mP, w.Wn, deltas, egrads, inLen, labLen, d, false, s));
-  RNNT_TRY(launch_pgrads(E, P, w.mE, w.mP, w.Wt, deltas, pgrads, inLen, labLen, d, false, s));
-  RNNT_TRY(launch_sparse(w.planes, egrads, pgrads, labels, inLen, labLen, deltas, true, d, s));
+  RNNT_STAGE(kWeights, launch_weights(w.planes, inLen, labLen, d, s));
+  RNNT_STAGE(kBeta, launch_beta(w.planes, labels, inLen, labLen, d, s));
+  RNNT_STAGE(kUnskew, launch_unskew(w.planes.dS, w.lngrads, inLen, labLen, d, s));
+  RNNT_STAGE(kWplanes, launch_wplanes(w.lngrads, w.LN, w.mE, w.mP, w.Wn, w.Wt, inLen, labLen, d, s));
+  RNNT_STAGE(kEgrads, launch_egrads(E, P, w.mE, w.mP, w.Wn, deltas, egrads, inLen, labLen, d, false, s));
+  RNNT_STAGE(kPgrads, launch_pgrads(E, P, w.mE, w.mP, w.Wt, deltas, pgrads, inLen, labLen, d, false, s));
+  RNNT_STAGE(kSparse, launch_sparse(w.planes, egrads, pgrads, labels, inLen, labLen, deltas, true, d, s));
   return kOk;
 }
 
@@ -331,9 +403,9 @@ int rnnt_hip_viterbi_decode(const float* E, const float* P, const int* inLen, co
   float* mE = static_cast<float*>(scratch.take(sizeof(float) * (size_t)B * T));
   float* mP = static_cast<float*>(scratch.take(sizeof(float) * (size_t)B * U));
   float* LN = static_cast<float*>(scratch.take(btu));
-  RNNT_TRY(launch_rowmax(E, mE, (long)B * T, V, s));
-  RNNT_TRY(launch_rowmax(P, mP, (long)B * U, V, s));
-  RNNT_TRY(launch_lse(E, P, mE, mP, LN, inLen, labLen, d, s));
+  RNNT_STAGE(kRowmax, launch_rowmax(E, mE, (long)B * T, V, s));
+  RNNT_STAGE(kRowmax, launch_rowmax(P, mP, (long)B * U, V, s));
+  RNNT_STAGE(kLse, launch_lse(E, P, mE, mP, LN, inLen, labLen, d, s));
   return viterbi_impl(E, P, LN, labels, inLen, labLen, d, s);
 }
 
