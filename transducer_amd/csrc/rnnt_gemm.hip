@@ -242,8 +242,9 @@ __device__ inline void mma_group(const float* As, const float* Bs, int arow, int
   acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a4.w, b3, acc, 0, 0, 0);
 }
 
-// ------------------------------------------------------------------ egrads (dense part)
-// Block tile 64 (t) x 64 (v); the whole reduction over u (Up <= kEgMaxK) sits in LDS at once.
+// ------------------------------------------------------------------ egrads, any label length
+// Fallback for label axes too long for the register-resident form in rnnt_grads.hip.
+// Block tile 64 (t) x 64 (v); a slice of the reduction over u (<= kEgMaxK) sits in LDS at once.
 constexpr int kEgMaxK = 112, kEgKP = kEgMaxK + 4, kEgNP = 64 + 4;
 
 __global__ __launch_bounds__(256, 2) void egrads_kernel(
@@ -307,99 +308,6 @@ __global__ __launch_bounds__(256, 2) void egrads_kernel(
   }
 }
 
-// ------------------------------------------------------------------ pgrads (dense part)
-// Block tile 128 (u) x 64 (v), reduction over t in slices of 32.
-constexpr int kPgBK = 32, kPgKP = kPgBK + 4, kPgNP = 64 + 4;
-
-__global__ __launch_bounds__(256, 2) void pgrads_kernel(
-    const float* __restrict__ E, const float* __restrict__ P, const float* __restrict__ mE,
-    const float* __restrict__ mP, const float* __restrict__ Wt, const float* __restrict__ deltas,
-    float* __restrict__ pgrads, const int* __restrict__ inLen, const int* __restrict__ labLen,
-    Dims d, int Up, int Tw, int accumulate) {
-  __shared__ __attribute__((aligned(16))) float As[128 * kPgKP];
-  __shared__ __attribute__((aligned(16))) float Bs[kPgBK * kPgNP];
-  const int b = blockIdx.z, v0 = blockIdx.x * 64, u0 = blockIdx.y * 128;
-  int Tb, Ub;
-  utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  float* out = pgrads + (size_t)b * d.U * d.V;
-  if (u0 >= Ub || Tb == 0) {
-    const float dl = deltas ? deltas[b] : 1.0f;
-    for (int e = tid; e < 128 * 64; e += 256) {
-      const int u = u0 + e / 64, v = v0 + e % 64;
-      if (u < d.U && v < d.V) {
-        const size_t o = (size_t)u * d.V + v;
-        out[o] = accumulate ? dl * out[o] : 0.0f;
-      }
-    }
-    return;
-  }
-  const float* Eb = E + (size_t)b * d.T * d.V;
-  const float* mEb = mE + (size_t)b * d.T;
-  const int l32 = lane & 31, h = lane >> 5;
-  floatx16 acc[2];
-#pragma unroll
-  for (int i = 0; i < 2; ++i)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) acc[i][r] = 0.0f;
-
-  // staging: A element e -> row e/32 (u), k e%32 (t); B element e -> k e/64 (t), n e%64 (v)
-  float ra[16], rb[8];
-  auto fetch = [&](int k0) {
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const int e = tid + 256 * i, r = e >> 5, k = e & 31;
-      const int u = u0 + r, t = k0 + k;
-      ra[i] = (u < Up && t < Tw) ? Wt[((size_t)b * Up + u) * Tw + t] : 0.0f;
-    }
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int e = tid + 256 * i, k = e >> 6, n = e & 63;
-      const int t = k0 + k, v = v0 + n;
-      rb[i] = (t < Tb && v < d.V) ? Eb[(size_t)t * d.V + v] - mEb[t] : kNegInf;
-    }
-  };
-  const int nk = (Tb + kPgBK - 1) / kPgBK;
-  fetch(0);
-  for (int kt = 0; kt < nk; ++kt) {
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const int e = tid + 256 * i;
-      As[(e >> 5) * kPgKP + (e & 31)] = ra[i];
-    }
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int e = tid + 256 * i;
-      Bs[(e >> 6) * kPgNP + (e & 63)] = __expf(rb[i]);
-    }
-    __syncthreads();
-    if (kt + 1 < nk) fetch((kt + 1) * kPgBK);
-    // wavefront w: u rows [32w, 32w+32), both 32-wide v blocks
-#pragma unroll
-    for (int k = 0; k < kPgBK; k += 8) {
-      mma_group<kPgKP, kPgNP>(As, Bs, 32 * wave + l32, l32, k, h, acc[0]);
-      mma_group<kPgKP, kPgNP>(As, Bs, 32 * wave + l32, 32 + l32, k, h, acc[1]);
-    }
-    __syncthreads();
-  }
-  const float delta = deltas ? deltas[b] : 1.0f;
-  const float* Pb = P + (size_t)b * d.U * d.V;
-#pragma unroll
-  for (int j = 0; j < 2; ++j)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int u = u0 + 32 * wave + 8 * (r >> 2) + 4 * h + (r & 3);
-      const int v = v0 + 32 * j + l32;
-      if (u < d.U && v < d.V) {
-        const size_t o = (size_t)u * d.V + v;
-        float g = 0.0f;
-        if (u < Ub) g = __expf(Pb[o] - mP[(size_t)b * d.U + u]) * acc[j][r];
-        if (accumulate) g = out[o] + g;
-        out[o] = delta * g;
-      }
-    }
-}
-
 }  // namespace
 
 #define RNNT_LAUNCH_CHECK(name)                                                    \
@@ -445,6 +353,8 @@ int launch_egrads(const float* E, const float* P, const float* mE, const float* 
                   const float* Wn, const float* deltas, float* egrads, const int* inLen,
                   const int* labLen, const Dims& d, bool accumulate, hipStream_t s) {
   if (d.B == 0 || d.T == 0 || d.U == 0) return kOk;
+  if (egrads_stream_supported(d))
+    return launch_egrads_stream(E, P, mE, mP, Wn, deltas, egrads, inLen, labLen, d, accumulate, s);
   const int Up = wplane_up(d.U), Tw = wplane_tw(d.T);
   // label axes longer than one LDS slice are contracted slice by slice, accumulating
   for (int kofs = 0; kofs < Up; kofs += kEgMaxK) {
@@ -460,12 +370,7 @@ int launch_pgrads(const float* E, const float* P, const float* mE, const float* 
                   const float* Wt, const float* deltas, float* pgrads, const int* inLen,
                   const int* labLen, const Dims& d, bool accumulate, hipStream_t s) {
   if (d.B == 0 || d.T == 0 || d.U == 0) return kOk;
-  const int Up = wplane_up(d.U), Tw = wplane_tw(d.T);
-  hipLaunchKernelGGL(pgrads_kernel, dim3((d.V + 63) / 64, (d.U + 127) / 128, d.B), dim3(256), 0, s,
-                     E, P, mE, mP, Wt, deltas, pgrads, inLen, labLen, d, Up, Tw,
-                     accumulate ? 1 : 0);
-  RNNT_LAUNCH_CHECK("pgrads_kernel");
-  return kOk;
+  return launch_pgrads_stream(E, P, mE, mP, Wt, deltas, pgrads, inLen, labLen, d, accumulate, s);
 }
 
 }  // namespace rnnt

@@ -122,4 +122,14 @@ int launch_pgrads(const float* E, const float* P, const float* mE, const float* 
                   const float* Wt, const float* deltas, float* pgrads, const int* inLen,
                   const int* labLen, const Dims& d, bool accumulate, hipStream_t s);
 
+
+// ---------------------------------------------------------------- launchers (rnnt_grads.hip)
+bool egrads_stream_supported(const Dims& d);
+int launch_egrads_stream(const float* E, const float* P, const float* mE, const float* mP,
+                         const float* Wn, const float* deltas, float* egrads, const int* inLen,
+                         const int* labLen, const Dims& d, bool accumulate, hipStream_t s);
+int launch_pgrads_stream(const float* E, const float* P, const float* mE, const float* mP,
+                         const float* Wt, const float* deltas, float* pgrads, const int* inLen,
+                         const int* labLen, const Dims& d, bool accumulate, hipStream_t s);
+
 }  // namespace rnnt
