@@ -4,9 +4,9 @@
 // half-wave = one 128-byte line), and pass only the small W operand through LDS:
 //
 //   egrads[t,v] = delta * exp(E[t,v]-mE[t]) * sum_u Wn[t,u] * Y[u,v]      Y = exp(P-mP)
-//       a wavefront owns 64 columns v and holds Y[:, its columns] (all label positions) in
+//       a wavefront owns 32 columns v and holds Y[:, its columns] (all label positions) in
 //       registers for its whole life; it walks the frames 32 at a time, reads the 32 x U slab
-//       of W from LDS, and multiplies the finished 32x64 block with exp(E-mE) on its way out.
+//       of W from LDS, and multiplies the finished 32x32 block with exp(E-mE) on its way out.
 //       E is read once and egrads written once, each as whole cache lines.
 //
 //   pgrads[u,v] = delta * exp(P[u,v]-mP[u]) * sum_t Wt[u,t] * X[t,v]      X = exp(E-mE)
@@ -32,18 +32,33 @@ __device__ inline float f4at(const float4& v, int q) {
 // ------------------------------------------------------------------ egrads
 constexpr int kEsMaxG = 14;              // groups of 8 label positions kept in registers
 constexpr int kEsKP = 8 * kEsMaxG + 4;   // LDS row pitch of the W slab (floats)
+constexpr int kEsSlab = 32 * kEsKP + 8;  // + a dump slot for staging lanes with nothing to do
 
+// Row of the 32x32 output block that register r of lane-half h holds.
+__device__ inline int mfma_row(int r, int h) { return 8 * (r >> 2) + 4 * h + (r & 3); }
+
+struct SlabRegs {
+  float4 v0, v1, v2, v3;
+  float m;
+};
+
+template <bool kAccumulate>
 __global__ __launch_bounds__(256, 2) void egrads_stream_kernel(
     const float* __restrict__ E, const float* __restrict__ P, const float* __restrict__ mE,
     const float* __restrict__ mP, const float* __restrict__ Wn, const float* __restrict__ deltas,
     float* __restrict__ egrads, const int* __restrict__ inLen, const int* __restrict__ labLen,
-    Dims d, int Up, int Tw, int tiles_per_chunk, int accumulate) {
-  __shared__ __attribute__((aligned(16))) float As[2][32 * kEsKP];
+    Dims d, int Up, int Tw, int tiles_per_chunk) {
+  __shared__ __attribute__((aligned(16))) float As[2][kEsSlab];
+  __shared__ __attribute__((aligned(16))) float Ms[2][32];  // mE of the slab's frames
   const int b = blockIdx.z;
   int Tb, Ub;
   utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, h = lane >> 5;
-  const int vcol = blockIdx.x * 256 + wave * 64 + l32;  // column of N-block 0; block 1 is +32
+  const int wave_col0 = blockIdx.x * 128 + wave * 32;  // this wavefront's 32 columns
+  const int vcol = wave_col0 + l32;
+  const bool vok = vcol < d.V;
+  const int vc = vok ? vcol : d.V - 1;  // always readable
+  const bool cols_full = wave_col0 + 32 <= d.V;
   const int ntiles = (d.T + 31) >> 5;
   const int tile_lo = blockIdx.y * tiles_per_chunk;
   const int tile_hi = min(tile_lo + tiles_per_chunk, ntiles);
@@ -53,11 +68,10 @@ __global__ __launch_bounds__(256, 2) void egrads_stream_kernel(
   const float* Eb = E + (size_t)b * d.T * d.V;
   float* out = egrads + (size_t)b * d.T * d.V;
   const float* mEb = mE + (size_t)b * d.T;
-  const bool vok0 = vcol < d.V, vok1 = vcol + 32 < d.V;
 
-  // Y fragments for this wavefront's 64 columns
-  float Yr[kEsMaxG][4][2];
-  {
+  // Y fragments for this wavefront's columns (branch-free: clamped address, masked value)
+  float Yr[kEsMaxG][4];
+  if (tile_lo < tile_valid) {
     const float* Pb = P + (size_t)b * d.U * d.V;
     const float* mPb = mP + (size_t)b * d.U;
 #pragma unroll
@@ -65,92 +79,111 @@ __global__ __launch_bounds__(256, 2) void egrads_stream_kernel(
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         const int u = 8 * j + 4 * h + q;
-        float y0 = 0.0f, y1 = 0.0f;
-        if (j < ngroups && u < Ub) {
-          const float m = mPb[u];
-          if (vok0) y0 = __expf(Pb[(size_t)u * d.V + vcol] - m);
-          if (vok1) y1 = __expf(Pb[(size_t)u * d.V + vcol + 32] - m);
-        }
-        Yr[j][q][0] = y0;
-        Yr[j][q][1] = y1;
+        const bool uok = u < Ub;
+        const int uc = uok ? u : 0;
+        const float y = __expf(Pb[(size_t)uc * d.V + vc] - mPb[uc]);
+        Yr[j][q] = (uok && vok) ? y : 0.0f;
       }
   }
 
   // W slab staging: the 32 x Up slab of frame tile ti is one contiguous run of 8*Up float4
   const int up4 = Up >> 2, nvec = 8 * Up;
-  int lds_off[4];
-  bool vec_ok[4];
+  int lds_off[4], src_idx[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int idx = tid + 256 * i;
-    vec_ok[i] = idx < nvec;
-    lds_off[i] = (idx / up4) * kEsKP + 4 * (idx % up4);
+    const bool ok = idx < nvec;
+    src_idx[i] = ok ? idx : nvec - 1;
+    lds_off[i] = ok ? (idx / up4) * kEsKP + 4 * (idx % up4) : 32 * kEsKP;
   }
-  float4 areg[4];
-  auto fetch_slab = [&](int ti) {
+  auto fetch_slab = [&](int ti) -> SlabRegs {
     const float4* src =
         reinterpret_cast<const float4*>(Wn + ((size_t)b * Tw + (size_t)ti * 32) * Up);
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-      if (vec_ok[i]) areg[i] = src[tid + 256 * i];
+    SlabRegs s;
+    s.v0 = src[src_idx[0]];
+    s.v1 = src[src_idx[1]];
+    s.v2 = src[src_idx[2]];
+    s.v3 = src[src_idx[3]];
+    s.m = mEb[min(ti * 32 + (tid & 31), Tb - 1)];
+    return s;
   };
-  auto store_slab = [&](int buf) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-      if (vec_ok[i]) *reinterpret_cast<float4*>(&As[buf][lds_off[i]]) = areg[i];
+  auto store_slab = [&](int buf, const SlabRegs& s) {
+    *reinterpret_cast<float4*>(&As[buf][lds_off[0]]) = s.v0;
+    *reinterpret_cast<float4*>(&As[buf][lds_off[1]]) = s.v1;
+    *reinterpret_cast<float4*>(&As[buf][lds_off[2]]) = s.v2;
+    *reinterpret_cast<float4*>(&As[buf][lds_off[3]]) = s.v3;
+    if (tid < 32) Ms[buf][tid] = s.m;
   };
 
   int cur = 0;
-  if (tile_lo < tile_valid) {
-    fetch_slab(tile_lo);
-    store_slab(0);
-  }
+  if (tile_lo < tile_valid) store_slab(0, fetch_slab(tile_lo));
   __syncthreads();
+
+  // per-lane part of the element offset inside a tile; the per-register part is r-dependent
+  // only through compile-time multiples of V
+  const unsigned lane_off = (unsigned)(4 * h) * (unsigned)d.V + (unsigned)vcol;
 
   for (int ti = tile_lo; ti < tile_valid; ++ti) {
     const int t0 = ti * 32;
     const bool has_next = ti + 1 < tile_valid;
-    if (has_next) fetch_slab(ti + 1);
+    SlabRegs nxt;
+    if (has_next) nxt = fetch_slab(ti + 1);
+    const bool interior = cols_full && (t0 + 32 <= Tb);  // no row or column needs a guard
+    const float* Etile = Eb + (size_t)t0 * d.V;
+    float* Otile = out + (size_t)t0 * d.V;
     // the emissions of this tile, requested before the matrix work so they arrive under it
-    float ev[16][2], mv[16];
+    float ev[16];
+    if (interior) {
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int t = t0 + 8 * (r >> 2) + 4 * h + (r & 3);
-      const bool tok = t < Tb;
-      const size_t o = (size_t)(tok ? t : 0) * d.V;
-      mv[r] = mEb[tok ? t : 0];
-      ev[r][0] = (tok && vok0) ? Eb[o + vcol] : kNegInf;
-      ev[r][1] = (tok && vok1) ? Eb[o + vcol + 32] : kNegInf;
+      for (int r = 0; r < 16; ++r)
+        ev[r] = Etile[lane_off + (unsigned)(8 * (r >> 2) + (r & 3)) * (unsigned)d.V];
+    } else {
+      // rows past the utterance are read from its last frame and masked on the way out
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        ev[r] = Eb[(size_t)min(t0 + mfma_row(r, h), Tb - 1) * d.V + vc];
     }
-    floatx16 acc0, acc1;
+    floatx16 acc;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) { acc0[r] = 0.0f; acc1[r] = 0.0f; }
+    for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
+    const float* arow = &As[cur][l32 * kEsKP + 4 * h];
+    float4 a_next = *reinterpret_cast<const float4*>(arow);
 #pragma unroll
     for (int j = 0; j < kEsMaxG; ++j) {
       if (j < ngroups) {
-        const float4 a4 =
-            *reinterpret_cast<const float4*>(&As[cur][l32 * kEsKP + 8 * j + 4 * h]);
+        const float4 a4 = a_next;
+        if (j + 1 < ngroups) a_next = *reinterpret_cast<const float4*>(arow + 8 * (j + 1));
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a4.x, Yr[j][0], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a4.y, Yr[j][1], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a4.z, Yr[j][2], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a4.w, Yr[j][3], acc, 0, 0, 0);
+      }
+    }
+    if (interior) {
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const float a = f4at(a4, q);
-          acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a, Yr[j][q][0], acc0, 0, 0, 0);
-          acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a, Yr[j][q][1], acc1, 0, 0, 0);
+      for (int g = 0; g < 4; ++g) {
+        const float4 m4 = *reinterpret_cast<const float4*>(&Ms[cur][8 * g + 4 * h]);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          const int r = 4 * g + k;
+          const float v = __expf(ev[r] - f4at(m4, k)) * acc[r];
+          float* o = Otile + lane_off + (unsigned)(8 * g + k) * (unsigned)d.V;
+          *o = delta * (kAccumulate ? *o + v : v);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int t = t0 + mfma_row(r, h);
+        float v = __expf(ev[r] - Ms[cur][mfma_row(r, h)]) * acc[r];
+        v = t < Tb ? v : 0.0f;
+        if (t < d.T && vok) {
+          float* o = out + (size_t)t * d.V + vcol;
+          *o = delta * (kAccumulate ? *o + v : v);
         }
       }
     }
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int t = t0 + 8 * (r >> 2) + 4 * h + (r & 3);
-      if (t < d.T) {
-        const size_t o = (size_t)t * d.V + vcol;
-        float g0 = __expf(ev[r][0] - mv[r]) * acc0[r];  // exp(-inf) = 0 on padded frames
-        float g1 = __expf(ev[r][1] - mv[r]) * acc1[r];
-        if (t >= Tb) { g0 = 0.0f; g1 = 0.0f; }
-        if (vok0) out[o] = delta * (accumulate ? out[o] + g0 : g0);
-        if (vok1) out[o + 32] = delta * (accumulate ? out[o + 32] + g1 : g1);
-      }
-    }
-    if (has_next) store_slab(cur ^ 1);
+    if (has_next) store_slab(cur ^ 1, nxt);
     __syncthreads();
     cur ^= 1;
   }
@@ -159,11 +192,10 @@ __global__ __launch_bounds__(256, 2) void egrads_stream_kernel(
   for (int ti = max(tile_lo, tile_valid); ti < tile_hi; ++ti) {
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-      const int t = ti * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
-      if (t < d.T) {
-        const size_t o = (size_t)t * d.V + vcol;
-        if (vok0) out[o] = accumulate ? delta * out[o] : 0.0f;
-        if (vok1) out[o + 32] = accumulate ? delta * out[o + 32] : 0.0f;
+      const int t = ti * 32 + mfma_row(r, h);
+      if (t < d.T && vok) {
+        float* o = out + (size_t)t * d.V + vcol;
+        *o = kAccumulate ? delta * *o : 0.0f;
       }
     }
   }
@@ -172,18 +204,21 @@ __global__ __launch_bounds__(256, 2) void egrads_stream_kernel(
 // ------------------------------------------------------------------ pgrads
 constexpr int kPsKP = 32 + 4;  // LDS row pitch of the W^T slab (floats)
 
+template <bool kAccumulate>
 __global__ __launch_bounds__(256, 2) void pgrads_stream_kernel(
     const float* __restrict__ E, const float* __restrict__ P, const float* __restrict__ mE,
     const float* __restrict__ mP, const float* __restrict__ Wt, const float* __restrict__ deltas,
     float* __restrict__ pgrads, const int* __restrict__ inLen, const int* __restrict__ labLen,
-    Dims d, int Up, int Tw, int accumulate) {
+    Dims d, int Up, int Tw) {
   __shared__ __attribute__((aligned(16))) float As[2][128 * kPsKP];
+  __shared__ __attribute__((aligned(16))) float Ms[2][32];
   const int b = blockIdx.z, u0 = blockIdx.y * 128;
   int Tb, Ub;
   utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, h = lane >> 5;
   const int vcol = blockIdx.x * 128 + wave * 32 + l32;
   const bool vok = vcol < d.V;
+  const int vc = vok ? vcol : d.V - 1;
   const float delta = deltas ? deltas[b] : 1.0f;
   float* out = pgrads + (size_t)b * d.U * d.V;
   const int nmb = (u0 < Ub && Tb > 0) ? min(4, (Ub - u0 + 31) >> 5) : 0;  // 32-row blocks in use
@@ -197,82 +232,101 @@ __global__ __launch_bounds__(256, 2) void pgrads_stream_kernel(
   if (nmb > 0) {
     const float* Eb = E + (size_t)b * d.T * d.V;
     const float* mEb = mE + (size_t)b * d.T;
-    // W^T slab staging: 128 rows (u) x 32 frames = 1024 float4, four per thread
+    // W^T slab staging: 128 rows (u) x 32 frames = 1024 float4, four per thread; rows past the
+    // padded label axis re-read its last row (their blocks are never multiplied)
     const int arow = tid >> 3, ac4 = tid & 7;  // rows arow + 32*i
-    float4 areg[4];
-    auto fetch_slab = [&](int k0) {
+    const float* asrc[4];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int u = u0 + arow + 32 * i;
-        areg[i] = (i < nmb && u < Up)
-                      ? *reinterpret_cast<const float4*>(Wt + ((size_t)b * Up + u) * Tw + k0 + 4 * ac4)
-                      : make_float4(0.f, 0.f, 0.f, 0.f);
-      }
+    for (int i = 0; i < 4; ++i)
+      asrc[i] = Wt + ((size_t)b * Up + min(u0 + arow + 32 * i, Up - 1)) * Tw + 4 * ac4;
+    struct XRegs { float v[4][4]; };
+    auto fetch_slab = [&](int k0) -> SlabRegs {
+      SlabRegs s;
+      s.v0 = *reinterpret_cast<const float4*>(asrc[0] + k0);
+      s.v1 = *reinterpret_cast<const float4*>(asrc[1] + k0);
+      s.v2 = *reinterpret_cast<const float4*>(asrc[2] + k0);
+      s.v3 = *reinterpret_cast<const float4*>(asrc[3] + k0);
+      s.m = mEb[min(k0 + (tid & 31), Tb - 1)];
+      return s;
     };
-    auto store_slab = [&](int buf) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-        *reinterpret_cast<float4*>(&As[buf][(arow + 32 * i) * kPsKP + 4 * ac4]) = areg[i];
-    };
-    float xraw[4][4], xm[4][4];
-    auto fetch_x = [&](int k0) {
+    auto fetch_x = [&](int k0) -> XRegs {
+      XRegs x;
 #pragma unroll
       for (int j = 0; j < 4; ++j)
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          const int t = k0 + 8 * j + 4 * h + q;
-          const bool tok = t < Tb;
-          xm[j][q] = mEb[tok ? t : 0];
-          xraw[j][q] = (tok && vok) ? Eb[(size_t)t * d.V + vcol] : kNegInf;
+          const int t = min(k0 + 8 * j + 4 * h + q, Tb - 1);
+          x.v[j][q] = Eb[(size_t)t * d.V + vc];
         }
+      return x;
+    };
+    auto store_slab = [&](int buf, const SlabRegs& s) {
+      float* dst = &As[buf][arow * kPsKP + 4 * ac4];
+      *reinterpret_cast<float4*>(dst) = s.v0;
+      *reinterpret_cast<float4*>(dst + 32 * kPsKP) = s.v1;
+      *reinterpret_cast<float4*>(dst + 64 * kPsKP) = s.v2;
+      *reinterpret_cast<float4*>(dst + 96 * kPsKP) = s.v3;
+      if (tid < 32) Ms[buf][tid] = s.m;
     };
 
     const int nk = (Tb + 31) >> 5;
-    fetch_slab(0);
-    fetch_x(0);
-    store_slab(0);
+    store_slab(0, fetch_slab(0));
+    XRegs xr = fetch_x(0);
     __syncthreads();
     int cur = 0;
     for (int kt = 0; kt < nk; ++kt) {
+      // X = exp(E - mE) for this slab, zero past the utterance (W is zero there as well)
       float x[4][4];
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
+      for (int j = 0; j < 4; ++j) {
+        const float4 m4 = *reinterpret_cast<const float4*>(&Ms[cur][8 * j + 4 * h]);
 #pragma unroll
-        for (int q = 0; q < 4; ++q) x[j][q] = __expf(xraw[j][q] - xm[j][q]);
-      const bool has_next = kt + 1 < nk;
-      if (has_next) {
-        fetch_slab((kt + 1) * 32);
-        fetch_x((kt + 1) * 32);
-      }
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-#pragma unroll
-        for (int mb = 0; mb < 4; ++mb) {
-          if (mb < nmb) {
-            const float4 a4 = *reinterpret_cast<const float4*>(
-                &As[cur][(32 * mb + l32) * kPsKP + 8 * j + 4 * h]);
-#pragma unroll
-            for (int q = 0; q < 4; ++q)
-              acc[mb] = __builtin_amdgcn_mfma_f32_32x32x2f32(f4at(a4, q), x[j][q], acc[mb], 0, 0, 0);
-          }
+        for (int q = 0; q < 4; ++q) {
+          const float e = __expf(xr.v[j][q] - f4at(m4, q));
+          x[j][q] = (kt * 32 + 8 * j + 4 * h + q < Tb && vok) ? e : 0.0f;
         }
-      if (has_next) store_slab(cur ^ 1);
+      }
+      const bool has_next = kt + 1 < nk;
+      SlabRegs nxt;
+      if (has_next) {
+        nxt = fetch_slab((kt + 1) * 32);
+        xr = fetch_x((kt + 1) * 32);
+      }
+      const float* abase = &As[cur][l32 * kPsKP + 4 * h];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        float4 a4[4];
+#pragma unroll
+        for (int mb = 0; mb < 4; ++mb)
+          if (mb < nmb)
+            a4[mb] = *reinterpret_cast<const float4*>(abase + 32 * mb * kPsKP + 8 * j);
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+          for (int mb = 0; mb < 4; ++mb)
+            if (mb < nmb)
+              acc[mb] = __builtin_amdgcn_mfma_f32_32x32x2f32(f4at(a4[mb], q), x[j][q], acc[mb],
+                                                              0, 0, 0);
+      }
+      if (has_next) store_slab(cur ^ 1, nxt);
       __syncthreads();
       cur ^= 1;
     }
   }
 
   const float* Pb = P + (size_t)b * d.U * d.V;
+  const float* mPb = mP + (size_t)b * d.U;
 #pragma unroll
   for (int mb = 0; mb < 4; ++mb)
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-      const int u = u0 + 32 * mb + 8 * (r >> 2) + 4 * h + (r & 3);
+      const int u = u0 + 32 * mb + mfma_row(r, h);
+      const int uc = min(u, d.U - 1);
+      const float y = __expf(Pb[(size_t)uc * d.V + vc] - mPb[uc]);
+      const float g = (mb < nmb && u < Ub) ? y * acc[mb][r] : 0.0f;
       if (u < d.U && vok) {
-        const size_t o = (size_t)u * d.V + vcol;
-        float g = 0.0f;
-        if (mb < nmb && u < Ub) g = __expf(Pb[o] - mP[(size_t)b * d.U + u]) * acc[mb][r];
-        out[o] = delta * (accumulate ? out[o] + g : g);
+        float* o = out + (size_t)u * d.V + vcol;
+        o[0] = delta * (kAccumulate ? o[0] + g : g);
       }
     }
 }
@@ -291,7 +345,7 @@ int launch_egrads_stream(const float* E, const float* P, const float* mE, const 
                          const float* Wn, const float* deltas, float* egrads, const int* inLen,
                          const int* labLen, const Dims& d, bool accumulate, hipStream_t s) {
   const int Up = wplane_up(d.U), Tw = wplane_tw(d.T);
-  const int vtiles = (d.V + 255) / 256, ntiles = (d.T + 31) / 32;
+  const int vtiles = (d.V + 127) / 128, ntiles = (d.T + 31) / 32;
   // enough workgroups to fill 256 CUs two deep several times over, but long enough runs of
   // frames per workgroup to amortise loading the Y fragments
   int chunks = (2048 + vtiles * d.B - 1) / (vtiles * d.B);
@@ -300,8 +354,12 @@ int launch_egrads_stream(const float* E, const float* P, const float* mE, const 
   if (chunks > max_chunks) chunks = max_chunks;
   const int per = (ntiles + chunks - 1) / chunks;
   chunks = (ntiles + per - 1) / per;
-  hipLaunchKernelGGL(egrads_stream_kernel, dim3(vtiles, chunks, d.B), dim3(256), 0, s, E, P, mE,
-                     mP, Wn, deltas, egrads, inLen, labLen, d, Up, Tw, per, accumulate ? 1 : 0);
+  if (accumulate)
+    hipLaunchKernelGGL(egrads_stream_kernel<true>, dim3(vtiles, chunks, d.B), dim3(256), 0, s, E,
+                       P, mE, mP, Wn, deltas, egrads, inLen, labLen, d, Up, Tw, per);
+  else
+    hipLaunchKernelGGL(egrads_stream_kernel<false>, dim3(vtiles, chunks, d.B), dim3(256), 0, s, E,
+                       P, mE, mP, Wn, deltas, egrads, inLen, labLen, d, Up, Tw, per);
   RNNT_LAUNCH_CHECK("egrads_stream_kernel");
   return kOk;
 }
@@ -310,9 +368,13 @@ int launch_pgrads_stream(const float* E, const float* P, const float* mE, const 
                          const float* Wt, const float* deltas, float* pgrads, const int* inLen,
                          const int* labLen, const Dims& d, bool accumulate, hipStream_t s) {
   const int Up = wplane_up(d.U), Tw = wplane_tw(d.T);
-  hipLaunchKernelGGL(pgrads_stream_kernel, dim3((d.V + 127) / 128, (d.U + 127) / 128, d.B),
-                     dim3(256), 0, s, E, P, mE, mP, Wt, deltas, pgrads, inLen, labLen, d, Up, Tw,
-                     accumulate ? 1 : 0);
+  const dim3 grid((d.V + 127) / 128, (d.U + 127) / 128, d.B);
+  if (accumulate)
+    hipLaunchKernelGGL(pgrads_stream_kernel<true>, grid, dim3(256), 0, s, E, P, mE, mP, Wt, deltas,
+                       pgrads, inLen, labLen, d, Up, Tw);
+  else
+    hipLaunchKernelGGL(pgrads_stream_kernel<false>, grid, dim3(256), 0, s, E, P, mE, mP, Wt,
+                       deltas, pgrads, inLen, labLen, d, Up, Tw);
   RNNT_LAUNCH_CHECK("pgrads_stream_kernel");
   return kOk;
 }
