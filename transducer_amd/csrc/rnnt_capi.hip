@@ -243,7 +243,7 @@ int rnnt_hip_backward(const float* E, const float* P, float* egrads, float* pgra
 static int viterbi_impl(const float* E, const float* P, const float* LN, int* labels,
                         const int* inLen, const int* labLen, const Dims& d, hipStream_t s) {
   const size_t btu = sizeof(float) * (size_t)d.B * d.T * d.U;
-  const size_t plane = sizeof(float) * (size_t)d.B * d.U * d.Dp + 64;
+  const size_t plane = sizeof(float) * (size_t)d.B * d.Ua * d.Dp + 64;
   Scratch scratch(s);
   RNNT_TRY(scratch.reserve(align_up(planes_bytes(d)) + 2 * align_up(btu) + 2 * align_up(plane) +
                            align_up(viterbi_bits_bytes(d))));

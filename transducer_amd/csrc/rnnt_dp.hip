@@ -32,18 +32,26 @@ __device__ inline float wave_shl1(float x, float fill) {
                                                     0x130 /* wave_shl:1 */, 0xf, 0xf, false));
 }
 
+// exp(x) for x <= 0 and log(w) for w in [1,2] straight on the hardware transcendental units
+// (v_exp_f32 / v_log_f32 work in base 2 and are good to about one ulp).  In the one place they
+// are used -- log1p(exp(-|a-b|)) below -- the rounding of x*log2(e) costs at most 2.4e-8
+// absolute in the result (it is largest where exp(x) is small), i.e. less than half an ulp of
+// the value log 2 that the result never exceeds.
+__device__ inline float exp_neg(float x) { return __builtin_amdgcn_exp2f(x * 1.44269504088896341f); }
+__device__ inline float log_1to2(float w) { return __builtin_amdgcn_logf(w) * 0.693147180559945309f; }
+
 // log1p(y) for y in [0,1]:  log(1+y) with the rounding error of the sum 1+y folded back in.
 // Within about one ulp of the correctly rounded value over the whole range.
 __device__ inline float log1p_unit(float y) {
   const float w = 1.0f + y;
   const float lost = y - (w - 1.0f);
-  return logf(w) + lost / w;
+  return log_1to2(w) + lost * __builtin_amdgcn_rcpf(w);
 }
 
 // transducer/transducer_cpu.cpp:16-24
 __device__ inline float lse2(float a, float b) {
   const float hi = fmaxf(a, b);
-  float r = hi + log1p_unit(expf(-fabsf(a - b)));
+  float r = hi + log1p_unit(exp_neg(-fabsf(a - b)));
   r = (b == kNegInf) ? a : r;
   r = (a == kNegInf) ? b : r;
   return r;
@@ -79,7 +87,7 @@ __global__ __launch_bounds__(256) void skew_kernel(const float* __restrict__ src
 #pragma unroll
   for (int i = 0; i < 16; ++i) {
     const int u = u0 + ty + 4 * i, t = t0 + tx;
-    if (t < Tb && u < Ub) dstS[((size_t)b * d.U + u) * d.Dp + t + u] = tile[tx][ty + 4 * i];
+    if (t < Tb && u < Ub) dstS[plane_row(d, b, u) + t + u] = tile[tx][ty + 4 * i];
   }
 }
 
@@ -97,7 +105,7 @@ __global__ __launch_bounds__(256) void unskew_kernel(const float* __restrict__ s
   for (int i = 0; i < 16; ++i) {
     const int u = u0 + ty + 4 * i, t = t0 + tx;
     tile[ty + 4 * i][tx] =
-        (t < Tb && u < Ub) ? srcS[((size_t)b * d.U + u) * d.Dp + t + u] : 0.0f;
+        (t < Tb && u < Ub) ? srcS[plane_row(d, b, u) + t + u] : 0.0f;
   }
   __syncthreads();
   float* o = dst + (size_t)b * d.T * d.U;
@@ -126,18 +134,22 @@ __global__ __launch_bounds__(256) void gather_kernel(const float* __restrict__ E
   const int l = has_label ? labels[(size_t)b * (d.U - 1) + u] : d.blank;
   const float* Eb = E + (size_t)b * d.T * d.V;
   if (t < Tb) {
-    if (has_label) p.elS[((size_t)b * d.U + u) * d.Dp + t + u] = Eb[(size_t)t * d.V + l];
-    if (u == 0) p.eb[(size_t)b * d.Tp + t] = Eb[(size_t)t * d.V + d.blank];
+    if (has_label) p.elS[plane_row(d, b, u) + t + u] = Eb[(size_t)t * d.V + l];
+    if (u == 0) p.eb[(size_t)b * d.Tp + d.Eo + t] = Eb[(size_t)t * d.V + d.blank];
   }
   if (blockIdx.x == 0 && threadIdx.x == 0) {
     const float* Pu = P + ((size_t)b * d.U + u) * d.V;
-    p.pb[(size_t)b * d.U + u] = Pu[d.blank];
-    p.pl[(size_t)b * d.U + u] = has_label ? Pu[l] : 0.0f;
+    p.pb[(size_t)b * d.Ua + u] = Pu[d.blank];
+    p.pl[(size_t)b * d.Ua + u] = has_label ? Pu[l] : 0.0f;
   }
 }
 
 // ------------------------------------------------------------------ alpha
 // transducer/transducer_cpu.cpp:30-79 (one utterance per wavefront).
+// A cell that has not started yet (t < 0) keeps its -inf hand-over scores, which makes lse2
+// return the other operand untouched -- exactly the reference's first-row / first-column
+// special cases.  Cells past the utterance (t >= T_b, u >= U_b) are computed on whatever the
+// planes hold there and are never read by a valid cell.
 template <int C>
 __global__ __launch_bounds__(64) void alpha_kernel(Planes p, const int* __restrict__ inLen,
                                                    const int* __restrict__ labLen,
@@ -151,7 +163,10 @@ __global__ __launch_bounds__(64) void alpha_kernel(Planes p, const int* __restri
   }
   const int nsteps = Tb + Ub - 1;
   const int ngroups = (nsteps + 3) >> 2;
-  const float* ebp = p.eb + (size_t)b * d.Tp;
+  const int u0 = lane * C;
+  // E[t,blank] for the cells of step s sits at ebp[s - u]; column c at step s = 4g+j reads
+  // ebl[4g + j - c], so one run of C+3 values serves all columns of a group
+  const float* ebl = p.eb + (size_t)b * d.Tp + d.Eo - u0;
 
   float stay[C], emit[C], pbv[C], plv[C];
   const float* lnp[C];
@@ -159,101 +174,102 @@ __global__ __launch_bounds__(64) void alpha_kernel(Planes p, const int* __restri
   float* ap[C];
 #pragma unroll
   for (int c = 0; c < C; ++c) {
-    const int u = lane * C + c, uc = u < d.U ? u : d.U - 1;
-    const size_t row = ((size_t)b * d.U + uc) * d.Dp;
+    const size_t row = plane_row(d, b, u0 + c);  // u0 + c < Ua always
     lnp[c] = p.lnS + row;
     elp[c] = p.elS + row;
     ap[c] = p.aS + row;
-    pbv[c] = p.pb[(size_t)b * d.U + uc];
-    plv[c] = p.pl[(size_t)b * d.U + uc];
-    stay[c] = kNegInf;  // "no predecessor": lse2 then returns the other operand unchanged
+    pbv[c] = p.pb[(size_t)b * d.Ua + u0 + c];
+    plv[c] = p.pl[(size_t)b * d.Ua + u0 + c];
+    stay[c] = kNegInf;
     emit[c] = kNegInf;
   }
 
-  float4 ln4[C], el4[C];
-  float eb4[C][4];
-  auto load_group = [&](int g, float4* ln, float4* el, float (*ebv)[4]) {
+  struct Group {
+    float4 ln[C], el[C];
+    float eb[C + 3];
+  };
+  auto load_group = [&](int g) -> Group {
+    Group r;
 #pragma unroll
     for (int c = 0; c < C; ++c) {
-      ln[c] = *reinterpret_cast<const float4*>(lnp[c] + 4 * g);
-      el[c] = *reinterpret_cast<const float4*>(elp[c] + 4 * g);
-      const int u = lane * C + c;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) ebv[c][j] = ebp[clampi(4 * g + j - u, 0, Tb - 1)];
+      r.ln[c] = *reinterpret_cast<const float4*>(lnp[c] + 4 * g);
+      r.el[c] = *reinterpret_cast<const float4*>(elp[c] + 4 * g);
     }
+#pragma unroll
+    for (int k = 0; k < C + 3; ++k) r.eb[k] = ebl[4 * g + k - (C - 1)];
+    return r;
   };
-  load_group(0, ln4, el4, eb4);
 
+  Group cur = load_group(0);
   for (int g = 0; g < ngroups; ++g) {
-    float4 ln4n[C], el4n[C];
-    float eb4n[C][4];
-    load_group(g + 1 < ngroups ? g + 1 : g, ln4n, el4n, eb4n);
+    const Group nxt = load_group(g + 1 < ngroups ? g + 1 : g);
     float4 aout[C];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int s = 4 * g + j;
-      const float from_left = wave_shr1(emit[C - 1], kNegInf);
+      if (s < nsteps) {  // uniform; only the last group can be partial
+        const float from_left = wave_shr1(emit[C - 1], kNegInf);
 #pragma unroll
-      for (int c = C - 1; c >= 0; --c) {
-        const int u = lane * C + c, t = s - u;
-        const float left = (c == 0) ? from_left : emit[c - 1];
-        const bool active = (t >= 0) & (t < Tb) & (u < Ub);
-        float a = lse2(left, stay[c]);
-        a = (s == 0 && u == 0) ? 0.0f : a;  // :43
-        const float ln = f4get(ln4[c], j);
-        float sb = a + eb4[c][j];
-        sb = sb + pbv[c];
-        sb = sb - ln;
-        float se = a + f4get(el4[c], j);
-        se = se + plv[c];
-        se = se - ln;
-        stay[c] = active ? sb : stay[c];
-        emit[c] = active ? se : emit[c];
-        f4set(aout[c], j, a);
+        for (int c = C - 1; c >= 0; --c) {
+          const float left = (c == 0) ? from_left : emit[c - 1];
+          float a = lse2(left, stay[c]);
+          if (j == 0 && g == 0) a = (u0 + c == 0) ? 0.0f : a;  // :43
+          const float ln = f4get(cur.ln[c], j);
+          float sb = a + cur.eb[j - c + (C - 1)];
+          sb = sb + pbv[c];
+          sb = sb - ln;
+          float se = a + f4get(cur.el[c], j);
+          se = se + plv[c];
+          se = se - ln;
+          const bool started = s >= u0 + c;
+          stay[c] = started ? sb : kNegInf;
+          emit[c] = started ? se : kNegInf;
+          f4set(aout[c], j, a);
+        }
       }
     }
 #pragma unroll
-    for (int c = 0; c < C; ++c) {
-      if (lane * C + c < d.U) *reinterpret_cast<float4*>(ap[c] + 4 * g) = aout[c];
-      ln4[c] = ln4n[c];
-      el4[c] = el4n[c];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) eb4[c][j] = eb4n[c][j];
-    }
+    for (int c = 0; c < C; ++c) *reinterpret_cast<float4*>(ap[c] + 4 * g) = aout[c];
+    cur = nxt;
   }
-  // :73-78 the blank move out of the last cell, negated
+  // :73-78 the blank move out of the last cell, negated; that cell was the last one its
+  // column processed
 #pragma unroll
   for (int c = 0; c < C; ++c)
-    if (lane * C + c == Ub - 1) costs[b] = -stay[c];
+    if (u0 + c == Ub - 1) costs[b] = -stay[c];
 }
 
 // ------------------------------------------------------------------ transition weights
 // Everything of the dalpha recursion that does not depend on dalpha itself
-// (transducer/transducer_cpu.cpp:124-135): one thread per lattice cell.
+// (transducer/transducer_cpu.cpp:124-135): one thread per lattice cell.  Every entry of the two
+// weight planes is written -- zero where there is no such move or no such cell -- so the
+// recursion below needs no bounds of its own.
 __global__ __launch_bounds__(256) void weights_kernel(Planes p, const int* __restrict__ inLen,
                                                       const int* __restrict__ labLen, Dims d) {
   const int b = blockIdx.z, u = blockIdx.y;
   const int dg = blockIdx.x * 256 + threadIdx.x;
+  if (dg >= d.Dp) return;
   int Tb, Ub;
   utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
   const int t = dg - u;
-  if (u >= Ub || t < 0 || t >= Tb) return;
-  const size_t o = ((size_t)b * d.U + u) * d.Dp + dg;
-  const float a = p.aS[o], ln = p.lnS[o];
+  const size_t o = plane_row(d, b, u) + dg;
   float wb = 0.0f, we = 0.0f;
-  if (t + 1 < Tb) {
-    float x = a + p.eb[(size_t)b * d.Tp + t];
-    x = x + p.pb[(size_t)b * d.U + u];
-    x = x - ln;
-    x = x - p.aS[o + 1];
-    wb = expf(x);
-  }
-  if (u + 1 < Ub) {
-    float x = a + p.elS[o];
-    x = x + p.pl[(size_t)b * d.U + u];
-    x = x - ln;
-    x = x - p.aS[o + d.Dp + 1];
-    we = expf(x);
+  if (u < Ub && t >= 0 && t < Tb) {
+    const float a = p.aS[o], ln = p.lnS[o];
+    if (t + 1 < Tb) {
+      float x = a + p.eb[(size_t)b * d.Tp + d.Eo + t];
+      x = x + p.pb[(size_t)b * d.Ua + u];
+      x = x - ln;
+      x = x - p.aS[o + 1];
+      wb = expf(x);
+    }
+    if (u + 1 < Ub) {
+      float x = a + p.elS[o];
+      x = x + p.pl[(size_t)b * d.Ua + u];
+      x = x - ln;
+      x = x - p.aS[o + d.Dp + 1];
+      we = expf(x);
+    }
   }
   p.wB[o] = wb;
   p.wE[o] = we;
@@ -262,8 +278,10 @@ __global__ __launch_bounds__(256) void weights_kernel(Planes p, const int* __res
 // ------------------------------------------------------------------ dalpha
 // transducer/transducer_cpu.cpp:81-143 with the exponentials already taken:
 // dalpha[t,u] = dalpha[t+1,u]*wB[t,u] + dalpha[t,u+1]*wE[t,u], walked from the last diagonal
-// back to the first.  Each lane also keeps the running sums that the reference subtracts from
-// pgrads[u,blank] and pgrads[u,l_u], in the reference's own order (t descending).
+// back to the first; the last cell is seeded with 1 (:95) before the walk.  Each lane also
+// keeps the running sums that the reference subtracts from pgrads[u,blank] and pgrads[u,l_u],
+// in the reference's own order (t descending).  Operands are prefetched two groups of four
+// steps ahead through three rotating register sets.
 template <int C>
 __global__ __launch_bounds__(64) void beta_kernel(Planes p, const int* __restrict__ labels,
                                                   const int* __restrict__ inLen,
@@ -273,7 +291,8 @@ __global__ __launch_bounds__(64) void beta_kernel(Planes p, const int* __restric
   utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
   if (Tb == 0 || Ub == 0) return;  // :92-94
   const int nsteps = Tb + Ub - 1;
-  const int ngroups = (nsteps + 3) >> 2;
+  const int last = nsteps - 1;  // diagonal of the last cell
+  const int u0 = lane * C;
 
   float dcol[C], accB[C], accL[C];
   bool fold[C];  // label of this position equals blank: both sums share one accumulator
@@ -282,68 +301,79 @@ __global__ __launch_bounds__(64) void beta_kernel(Planes p, const int* __restric
   float* dp[C];
 #pragma unroll
   for (int c = 0; c < C; ++c) {
-    const int u = lane * C + c, uc = u < d.U ? u : d.U - 1;
-    const size_t row = ((size_t)b * d.U + uc) * d.Dp;
+    const int u = u0 + c;
+    const size_t row = plane_row(d, b, u);
     wbp[c] = p.wB + row;
     wep[c] = p.wE + row;
     dp[c] = p.dS + row;
-    dcol[c] = 0.0f;
+    dcol[c] = (u == Ub - 1) ? 1.0f : 0.0f;   // :95
     accB[c] = (u == Ub - 1) ? -1.0f : 0.0f;  // :97
     accL[c] = 0.0f;
     fold[c] = (u + 1 < Ub) && labels[(size_t)b * (d.U - 1) + u] == d.blank;
   }
 
-  float4 wb4[C], we4[C];
-  auto load_group = [&](int g, float4* wb, float4* we) {
+  struct Group {
+    float4 wb[C], we[C];
+  };
+  auto load_group = [&](int g) -> Group {
+    Group r;
+    const int gc = g > 0 ? g : 0;
 #pragma unroll
     for (int c = 0; c < C; ++c) {
-      wb[c] = *reinterpret_cast<const float4*>(wbp[c] + 4 * g);
-      we[c] = *reinterpret_cast<const float4*>(wep[c] + 4 * g);
+      r.wb[c] = *reinterpret_cast<const float4*>(wbp[c] + 4 * gc);
+      r.we[c] = *reinterpret_cast<const float4*>(wep[c] + 4 * gc);
     }
+    return r;
   };
-  load_group(ngroups - 1, wb4, we4);
-
-  for (int g = ngroups - 1; g >= 0; --g) {
-    float4 wb4n[C], we4n[C];
-    load_group(g > 0 ? g - 1 : 0, wb4n, we4n);
+  // steps last-1 .. 0 are computed; the slot of step `last` receives the seed and the slots
+  // after it (same group of four) zeros
+  auto run_group = [&](int g, const Group& w) {
     float4 dout[C];
 #pragma unroll
     for (int j = 3; j >= 0; --j) {
       const int s = 4 * g + j;
-      const float from_right = wave_shl1(dcol[0], 0.0f);
+      if (s >= last) {  // uniform; only in the first group run
 #pragma unroll
-      for (int c = 0; c < C; ++c) {
-        const int u = lane * C + c, t = s - u;
-        const float right = (c == C - 1) ? from_right : dcol[c + 1];
-        const bool active = (t >= 0) & (t < Tb) & (u < Ub) & (s < nsteps);
-        const float ne = dcol[c] * f4get(wb4[c], j);
-        const float em = right * f4get(we4[c], j);
-        float dn = ne + em;
-        dn = (t == Tb - 1 && u == Ub - 1) ? 1.0f : dn;  // :95
-        const float ne_a = active ? ne : 0.0f, em_a = active ? em : 0.0f;
-        if (fold[c]) {
-          accB[c] = (accB[c] - ne_a) - em_a;
-        } else {
-          accB[c] = accB[c] - ne_a;
-          accL[c] = accL[c] - em_a;
+        for (int c = 0; c < C; ++c) f4set(dout[c], j, s == last ? dcol[c] : 0.0f);
+      } else {
+        const float from_right = wave_shl1(dcol[0], 0.0f);
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+          const float right = (c == C - 1) ? from_right : dcol[c + 1];
+          const float ne = dcol[c] * f4get(w.wb[c], j);
+          const float em = right * f4get(w.we[c], j);
+          const float dn = ne + em;
+          const float em_b = fold[c] ? em : 0.0f, em_l = fold[c] ? 0.0f : em;
+          accB[c] = (accB[c] - ne) - em_b;
+          accL[c] = accL[c] - em_l;
+          dcol[c] = dn;
+          f4set(dout[c], j, dn);
         }
-        dcol[c] = active ? dn : dcol[c];
-        f4set(dout[c], j, active ? dn : 0.0f);
       }
     }
 #pragma unroll
-    for (int c = 0; c < C; ++c) {
-      if (lane * C + c < d.U) *reinterpret_cast<float4*>(dp[c] + 4 * g) = dout[c];
-      wb4[c] = wb4n[c];
-      we4[c] = we4n[c];
-    }
+    for (int c = 0; c < C; ++c) *reinterpret_cast<float4*>(dp[c] + 4 * g) = dout[c];
+  };
+
+  int g = last >> 2;  // the group that holds the seed
+  Group x = load_group(g), y = load_group(g - 1), z = load_group(g - 2);
+  for (; g >= 2; g -= 3) {
+    run_group(g, x);
+    x = load_group(g - 3);
+    run_group(g - 1, y);
+    y = load_group(g - 4);
+    run_group(g - 2, z);
+    z = load_group(g - 5);
   }
+  if (g >= 0) run_group(g, x);
+  if (g >= 1) run_group(g - 1, y);
+
 #pragma unroll
   for (int c = 0; c < C; ++c) {
-    const int u = lane * C + c;
+    const int u = u0 + c;
     if (u < Ub) {
-      p.gB[(size_t)b * d.U + u] = accB[c];
-      p.gL[(size_t)b * d.U + u] = accL[c];
+      p.gB[(size_t)b * d.Ua + u] = accB[c];
+      p.gL[(size_t)b * d.Ua + u] = accL[c];
     }
   }
 }
@@ -370,7 +400,7 @@ __global__ __launch_bounds__(256) void sparse_e_kernel(Planes p, float* __restri
   const float sc = scale ? scale[b] : 1.0f;
   float blank_acc = (t == Tb - 1) ? -1.0f : 0.0f;
   for (int u = Ub - 1; u >= 0; --u) {
-    const size_t o = ((size_t)b * d.U + u) * d.Dp + t + u;
+    const size_t o = plane_row(d, b, u) + t + u;
     if (t + 1 < Tb) blank_acc -= p.dS[o + 1] * p.wB[o];
     if (u + 1 < Ub) {
       const float em = p.dS[o + d.Dp + 1] * p.wE[o];
@@ -396,7 +426,7 @@ __global__ __launch_bounds__(256) void sparse_p_kernel(Planes p, float* __restri
   utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
   if (Tb == 0 || u >= Ub) return;
   float* row = pgrads + ((size_t)b * d.U + u) * d.V;
-  const float gb = p.gB[(size_t)b * d.U + u], gl = p.gL[(size_t)b * d.U + u];
+  const float gb = p.gB[(size_t)b * d.Ua + u], gl = p.gL[(size_t)b * d.Ua + u];
   const bool has_label = u + 1 < Ub;
   const int l = has_label ? labels[(size_t)b * (d.U - 1) + u] : d.blank;
   if (add) {
@@ -523,7 +553,7 @@ __global__ __launch_bounds__(64) void viterbi_kernel(Planes p, const float* __re
   const int ngroups = (nsteps + 3) >> 2;
   unsigned long long* bits =
       kLdsBits ? lbits : gbits + (size_t)b * (size_t)(d.T + d.U + 4) * C;
-  const float* ebp = p.eb + (size_t)b * d.Tp;
+  const float* ebp = p.eb + (size_t)b * d.Tp + d.Eo;
 
   float stay[C], emit[C], pbv[C];
   const float* lnp[C];
@@ -531,10 +561,10 @@ __global__ __launch_bounds__(64) void viterbi_kernel(Planes p, const float* __re
 #pragma unroll
   for (int c = 0; c < C; ++c) {
     const int u = lane * C + c, uc = u < d.U ? u : d.U - 1;
-    const size_t row = ((size_t)b * d.U + uc) * d.Dp;
+    const size_t row = plane_row(d, b, uc);
     lnp[c] = p.lnS + row;
     bsp[c] = bestS + row;
-    pbv[c] = p.pb[(size_t)b * d.U + uc];
+    pbv[c] = p.pb[(size_t)b * d.Ua + uc];
     stay[c] = kNegInf;
     emit[c] = kNegInf;
   }
@@ -596,7 +626,7 @@ __global__ __launch_bounds__(64) void viterbi_kernel(Planes p, const float* __re
       const int s = t + u;
       const unsigned long long m = bits[(size_t)s * C + (u % C)];
       if ((m >> (u / C)) & 1ull) {
-        out[u - 1] = argI[((size_t)b * d.U + (u - 1)) * d.Dp + s - 1];
+        out[u - 1] = argI[plane_row(d, b, u - 1) + s - 1];
         u -= 1;
       } else {
         t -= 1;
@@ -605,31 +635,25 @@ __global__ __launch_bounds__(64) void viterbi_kernel(Planes p, const float* __re
   }
 }
 
-int cells_per_lane(int U) {
-  int c = 1;
-  while (c * 64 < U) c *= 2;
-  return c;
-}
-
 }  // namespace
 
 // ------------------------------------------------------------------ workspace layout
 static size_t align_up(size_t x) { return (x + 255) & ~(size_t)255; }
 
 size_t planes_bytes(const Dims& d) {
-  const size_t plane = align_up(sizeof(float) * (size_t)d.B * d.U * d.Dp + 64);
+  const size_t plane = align_up(sizeof(float) * (size_t)d.B * d.Ua * d.Dp + 64);
   return 6 * plane + align_up(sizeof(float) * (size_t)d.B * d.Tp) +
-         4 * align_up(sizeof(float) * (size_t)d.B * d.U);
+         4 * align_up(sizeof(float) * (size_t)d.B * d.Ua);
 }
 
 void carve_planes(void* base, const Dims& d, Planes* p) {
   char* c = static_cast<char*>(base);
-  const size_t plane = align_up(sizeof(float) * (size_t)d.B * d.U * d.Dp + 64);
+  const size_t plane = align_up(sizeof(float) * (size_t)d.B * d.Ua * d.Dp + 64);
   auto take = [&](size_t n) { float* r = reinterpret_cast<float*>(c); c += n; return r; };
   p->lnS = take(plane); p->elS = take(plane); p->aS = take(plane);
   p->wB = take(plane); p->wE = take(plane); p->dS = take(plane);
   p->eb = take(align_up(sizeof(float) * (size_t)d.B * d.Tp));
-  const size_t bu = align_up(sizeof(float) * (size_t)d.B * d.U);
+  const size_t bu = align_up(sizeof(float) * (size_t)d.B * d.Ua);
   p->pb = take(bu); p->pl = take(bu); p->gB = take(bu); p->gL = take(bu);
 }
 
@@ -689,7 +713,7 @@ int launch_alpha(const Planes& p, const int* inLen, const int* labLen, float* co
 int launch_weights(const Planes& p, const int* inLen, const int* labLen, const Dims& d,
                    hipStream_t s) {
   if (d.B == 0 || d.T == 0 || d.U == 0) return kOk;
-  hipLaunchKernelGGL(weights_kernel, dim3((d.T + d.U + 255) / 256, d.U, d.B), dim3(256), 0, s, p,
+  hipLaunchKernelGGL(weights_kernel, dim3((d.Dp + 255) / 256, d.Ua, d.B), dim3(256), 0, s, p,
                      inLen, labLen, d);
   RNNT_LAUNCH_CHECK("weights_kernel");
   return kOk;

@@ -31,8 +31,10 @@ int check_hip(hipError_t e, const char* what, const char* file, int line);
 // Problem sizes in the reference's vocabulary: U is the prediction length (longest label + 1).
 struct Dims {
   int B, T, U, V, blank;
+  int Ua;  // rows per utterance in a skewed plane: U rounded up to 64 * cells-per-lane
   int Dp;  // row pitch of a skewed plane, in floats
   int Tp;  // row pitch of the per-frame blank-score array
+  int Eo;  // index of frame 0 inside a row of that array (frames -Eo..-1 are readable padding)
 };
 
 // A skewed plane stores cell (t,u) of utterance b at [(b*U + u)*Dp + (t+u)]: one row per label
@@ -40,14 +42,27 @@ struct Dims {
 // read the same column index at the same step, so four consecutive steps are one aligned
 // 16-byte load per lane.  The pitch leaves room for the last partial group of four.
 __host__ __device__ inline int plane_pitch(int T, int U) { return ((T + U + 3) & ~3) + 8; }
-__host__ __device__ inline int frame_pitch(int T) { return ((T + 3) & ~3) + 8; }
+
+// Label positions one lane of the lattice wavefront owns: 1, 2, 4, 8 or 16 (U <= 1024).
+inline int cells_per_lane(int U) {
+  int c = 1;
+  while (c * 64 < U) c *= 2;
+  return c;
+}
 
 inline Dims make_dims(int B, int T, int U, int V, int blank) {
   Dims d;
   d.B = B; d.T = T; d.U = U; d.V = V; d.blank = blank;
+  d.Ua = 64 * cells_per_lane(U);
   d.Dp = plane_pitch(T, U);
-  d.Tp = frame_pitch(T);
+  d.Eo = d.Ua + 4;
+  d.Tp = d.Eo + ((T + U + 3) & ~3) + 8;
   return d;
+}
+
+// Offset of row u of utterance b in a skewed plane.
+__host__ __device__ inline size_t plane_row(const Dims& d, int b, int u) {
+  return ((size_t)b * d.Ua + u) * d.Dp;
 }
 
 __device__ inline int clampi(int x, int lo, int hi) { return x < lo ? lo : (x > hi ? hi : x); }
@@ -67,11 +82,11 @@ struct Planes {
   float* wB;    // blank-move weight exp(stay(t,u) - alpha[t+1,u])
   float* wE;    // label-move weight exp(emit(t,u) - alpha[t,u+1])
   float* dS;    // dalpha (= d cost / d LN)
-  float* eb;    // E[t, blank]           [B, Tp]
-  float* pb;    // P[u, blank]           [B, U]
-  float* pl;    // P[u, label_u]         [B, U]
-  float* gB;    // per-(b,u) blank-column sum of the sparse pgrads term   [B, U]
-  float* gL;    // per-(b,u) label-column sum of the sparse pgrads term   [B, U]
+  float* eb;    // E[t, blank] at [b*Tp + Eo + t]
+  float* pb;    // P[u, blank]           [B, Ua]
+  float* pl;    // P[u, label_u]         [B, Ua]
+  float* gB;    // per-(b,u) blank-column sum of the sparse pgrads term   [B, Ua]
+  float* gL;    // per-(b,u) label-column sum of the sparse pgrads term   [B, Ua]
 };
 
 size_t planes_bytes(const Dims& d);
