@@ -289,8 +289,8 @@ int rnnt_hip_log_norms(const float* E, const float* P, float* LN, const int* inL
                            align_up(sizeof(float) * (size_t)B * U)));
   float* mE = static_cast<float*>(scratch.take(sizeof(float) * (size_t)B * T));
   float* mP = static_cast<float*>(scratch.take(sizeof(float) * (size_t)B * U));
-  RNNT_STAGE(kRowmax, launch_rowmax(E, mE, (long)B * T, V, s));
-  RNNT_STAGE(kRowmax, launch_rowmax(P, mP, (long)B * U, V, s));
+  RNNT_STAGE(kRowmax, launch_rowmax(E, mE, (long)B * T, V, T, inLen, 0, s));
+  RNNT_STAGE(kRowmax, launch_rowmax(P, mP, (long)B * U, V, U, labLen, 1, s));
   RNNT_STAGE(kLse, launch_lse(E, P, mE, mP, LN, inLen, labLen, d, s));
   return kOk;
 }
@@ -313,8 +313,8 @@ int rnnt_hip_dense_grads(const float* E, const float* P, float* egrads, float* p
   float* mP = static_cast<float*>(scratch.take(sizeof(float) * (size_t)B * U));
   float* Wn = static_cast<float*>(scratch.take(wb));
   float* Wt = static_cast<float*>(scratch.take(wb));
-  RNNT_STAGE(kRowmax, launch_rowmax(E, mE, (long)B * T, V, s));
-  RNNT_STAGE(kRowmax, launch_rowmax(P, mP, (long)B * U, V, s));
+  RNNT_STAGE(kRowmax, launch_rowmax(E, mE, (long)B * T, V, T, inLen, 0, s));
+  RNNT_STAGE(kRowmax, launch_rowmax(P, mP, (long)B * U, V, U, labLen, 1, s));
   RNNT_STAGE(kWplanes, launch_wplanes(lngrads, LN, mE, mP, Wn, Wt, inLen, labLen, d, s));
   RNNT_STAGE(kEgrads, launch_egrads(E, P, mE, mP, Wn, deltas, egrads, inLen, labLen, d, true, s));
   RNNT_STAGE(kPgrads, launch_pgrads(E, P, mE, mP, Wt, deltas, pgrads, inLen, labLen, d, true, s));
@@ -345,8 +345,8 @@ int rnnt_hip_loss_forward(const float* E, const float* P, const int* labels, con
   const Dims d = make_dims(B, T, U, V, blank);
   LossWorkspace w;
   loss_workspace_layout(d, workspace, &w);
-  RNNT_STAGE(kRowmax, launch_rowmax(E, w.mE, (long)B * T, V, s));
-  RNNT_STAGE(kRowmax, launch_rowmax(P, w.mP, (long)B * U, V, s));
+  RNNT_STAGE(kRowmax, launch_rowmax(E, w.mE, (long)B * T, V, T, inLen, 0, s));
+  RNNT_STAGE(kRowmax, launch_rowmax(P, w.mP, (long)B * U, V, U, labLen, 1, s));
   RNNT_STAGE(kLse, launch_lse(E, P, w.mE, w.mP, w.LN, inLen, labLen, d, s));
   RNNT_STAGE(kSkew, launch_skew(w.LN, w.planes.lnS, inLen, labLen, d, s));
   RNNT_STAGE(kGather, launch_gather(E, P, labels, inLen, labLen, w.planes, d, s));
@@ -403,8 +403,8 @@ int rnnt_hip_viterbi_decode(const float* E, const float* P, const int* inLen, co
   float* mE = static_cast<float*>(scratch.take(sizeof(float) * (size_t)B * T));
   float* mP = static_cast<float*>(scratch.take(sizeof(float) * (size_t)B * U));
   float* LN = static_cast<float*>(scratch.take(btu));
-  RNNT_STAGE(kRowmax, launch_rowmax(E, mE, (long)B * T, V, s));
-  RNNT_STAGE(kRowmax, launch_rowmax(P, mP, (long)B * U, V, s));
+  RNNT_STAGE(kRowmax, launch_rowmax(E, mE, (long)B * T, V, T, inLen, 0, s));
+  RNNT_STAGE(kRowmax, launch_rowmax(P, mP, (long)B * U, V, U, labLen, 1, s));
   RNNT_STAGE(kLse, launch_lse(E, P, mE, mP, LN, inLen, labLen, d, s));
   return viterbi_impl(E, P, LN, labels, inLen, labLen, d, s);
 }

@@ -395,20 +395,54 @@ __global__ __launch_bounds__(256) void sparse_e_kernel(Planes p, float* __restri
   int Tb, Ub;
   utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
   if (Ub == 0 || t >= Tb) return;
-  float* row = egrads + ((size_t)b * d.T + t) * d.V;
-  const int* lab = labels + (size_t)b * (d.U - 1);
+  float* __restrict__ row = egrads + ((size_t)b * d.T + t) * d.V;
+  const int* __restrict__ lab = labels + (size_t)b * (d.U - 1);
+  const float* __restrict__ dS = p.dS;
+  const float* __restrict__ wB = p.wB;
+  const float* __restrict__ wE = p.wE;
   const float sc = scale ? scale[b] : 1.0f;
+  const bool has_stay = t + 1 < Tb;
   float blank_acc = (t == Tb - 1) ? -1.0f : 0.0f;
-  for (int u = Ub - 1; u >= 0; --u) {
-    const size_t o = plane_row(d, b, u) + t + u;
-    if (t + 1 < Tb) blank_acc -= p.dS[o + 1] * p.wB[o];
-    if (u + 1 < Ub) {
-      const float em = p.dS[o + d.Dp + 1] * p.wE[o];
-      const int l = lab[u];
-      if (l == d.blank) blank_acc -= em;
-      else if (add) row[l] += sc * (-em);
-      else row[l] -= em;
+  // Positions are taken eight at a time, last to first; the products of the next eight are
+  // requested before the current eight are folded in, so the loop runs at the rate of the
+  // memory pipe rather than one round trip per label position.
+  constexpr int kChunk = 8;
+  struct Chunk { float ne[kChunk], em[kChunk]; };
+  auto load_chunk = [&](int uhi) -> Chunk {  // positions uhi, uhi-1, ..., uhi-7 (those >= 0)
+    Chunk c;
+#pragma unroll
+    for (int k = 0; k < kChunk; ++k) {
+      const int u = uhi - k;
+      const int uc = u > 0 ? u : 0;
+      const size_t o = plane_row(d, b, uc) + t + uc;
+      // loads are unconditional (the planes are readable one past the utterance); what they
+      // return there is discarded by the selects
+      const float ne = dS[o + 1] * wB[o];
+      const float em = dS[o + d.Dp + 1] * wE[o];
+      c.ne[k] = has_stay ? ne : 0.0f;
+      c.em[k] = (u + 1 < Ub) ? em : 0.0f;
     }
+    return c;
+  };
+  Chunk cur = load_chunk(Ub - 1);
+  for (int uhi = Ub - 1; uhi >= 0; uhi -= kChunk) {
+    const Chunk nxt = load_chunk(uhi - kChunk);
+#pragma unroll
+    for (int k = 0; k < kChunk; ++k) {
+      const int u = uhi - k;
+      if (u >= 0) {
+        blank_acc -= cur.ne[k];
+        if (u + 1 < Ub) {
+          const int l = lab[u];
+          // Label columns are updated with no-return hardware adds: nothing waits on them,
+          // and since this thread alone touches row t and its requests to one address stay
+          // in order, repeated labels still accumulate in the reference's order.
+          if (l == d.blank) blank_acc -= cur.em[k];
+          else unsafeAtomicAdd(&row[l], add ? sc * (-cur.em[k]) : -cur.em[k]);
+        }
+      }
+    }
+    cur = nxt;
   }
   if (add) row[d.blank] += sc * blank_acc;
   else row[d.blank] = blank_acc;

@@ -32,12 +32,22 @@ __device__ inline float wave_max(float m) {
 
 // ------------------------------------------------------------------ row maxima
 // One wavefront per row of a [rows, V] array.
+// rows_per_item / lengths (optional): row r belongs to item r / rows_per_item and is skipped
+// (maximum reported as 0, nothing read) when its index inside the item is >= lengths[item] + extra.
 __global__ __launch_bounds__(256) void rowmax_kernel(const float* __restrict__ X,
                                                      float* __restrict__ out, long rows, int V,
-                                                     int vec4) {
+                                                     int vec4, int rows_per_item,
+                                                     const int* __restrict__ lengths, int extra) {
   const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
   if (row >= rows) return;
+  if (lengths) {
+    const long item = row / rows_per_item;
+    if (row - item * rows_per_item >= lengths[item] + extra) {
+      if (lane == 0) out[row] = 0.0f;
+      return;
+    }
+  }
   const float* x = X + (size_t)row * V;
   float m0 = kNegInf, m1 = kNegInf, m2 = kNegInf, m3 = kNegInf;
   if (vec4) {
@@ -62,7 +72,8 @@ __global__ __launch_bounds__(256) void rowmax_kernel(const float* __restrict__ X
   if (lane == 0) out[row] = m;
 }
 
-// ------------------------------------------------------------------ log-normaliser
+// ------------------------------------------------------------------ log-normaliser, any shape
+// Scalar-load form for vocabularies that are not a multiple of 4 or unaligned inputs.
 // Block tile 128 (t) x 128 (u), reduction over v in slices of 32; 4 wavefronts, each 64x64.
 // Both operands are v-contiguous in memory and are staged as S[row][v] with a 36-float pitch
 // (16-byte reads of consecutive rows then fall into distinct bank groups).
@@ -186,6 +197,160 @@ __global__ __launch_bounds__(256, 2) void lse_kernel(const float* __restrict__ E
           LNb[(size_t)t * d.U + u] = v;
         }
       }
+}
+
+// ------------------------------------------------------------------ log-normaliser, fast form
+// Same contraction for V % 4 == 0 and 16-byte aligned inputs (the usual case):
+//  * 16-byte global loads (a thread stages 16 consecutive v of one E row and one P row),
+//    double-buffered LDS, one barrier per slice of 32;
+//  * a wavefront owns 32 frames x all label positions of the tile, so 32-wide label blocks
+//    past the utterance's own length are skipped by every wavefront alike;
+//  * the running sum is flushed into a second accumulator every kLseFlush slices, which keeps
+//    the fp32 summation error near sqrt(flush length) + sqrt(number of flushes) ulp instead of
+//    sqrt(V) and stops small terms from being swamped by an early large one;
+//  * workgroups are renumbered so that all frame tiles of one utterance run on the same XCD
+//    (workgroup ids are dealt round-robin to the 8 XCDs) and share its L2 copy of P[b].
+constexpr int kLseFlush = 16;
+
+struct LseStage {
+  float4 a0, a1, a2, a3, b0, b1, b2, b3;
+};
+
+__global__ __launch_bounds__(256, 2) void lse_fast_kernel(const float* __restrict__ E,
+                                                          const float* __restrict__ P,
+                                                          const float* __restrict__ mE,
+                                                          const float* __restrict__ mP,
+                                                          float* __restrict__ LN,
+                                                          const int* __restrict__ inLen,
+                                                          const int* __restrict__ labLen, Dims d,
+                                                          int ttiles, int utiles, int total) {
+  __shared__ __attribute__((aligned(16))) float As[2][kLseBM * kLsePitch];
+  __shared__ __attribute__((aligned(16))) float Bs[2][kLseBN * kLsePitch];
+  // XCD-aware renumbering: physical id n runs on XCD n % 8
+  const int n = blockIdx.x, per_xcd = gridDim.x >> 3;
+  const int logical = (n & 7) * per_xcd + (n >> 3);
+  if (logical >= total) return;
+  const int b = logical / (ttiles * utiles);
+  const int rem = logical - b * (ttiles * utiles);
+  const int t0 = (rem % ttiles) * kLseBM, u0 = (rem / ttiles) * kLseBN;
+  int Tb, Ub;
+  utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, h = lane >> 5;
+  float* LNb = LN + (size_t)b * d.T * d.U;
+
+  if (t0 >= Tb || u0 >= Ub) {
+    for (int e = tid; e < kLseBM * kLseBN; e += 256) {
+      const int t = t0 + e / kLseBN, u = u0 + e % kLseBN;
+      if (t < d.T && u < d.U) LNb[(size_t)t * d.U + u] = 0.0f;
+    }
+    return;
+  }
+  const int nnb = min(4, (Ub - u0 + 31) >> 5);  // 32-wide label blocks in use
+
+  // staging: thread -> row tid/2 of both operands, 16 consecutive v starting at 16*(tid%2)
+  const int srow = tid >> 1, skh = (tid & 1) * 16;
+  const int ta = min(t0 + srow, Tb - 1), ub = min(u0 + srow, Ub - 1);
+  const float* pa = E + ((size_t)b * d.T + ta) * d.V + skh;
+  const float* pb = P + ((size_t)b * d.U + ub) * d.V + skh;
+  const float ma = mE[(size_t)b * d.T + ta], mb = mP[(size_t)b * d.U + ub];
+  const bool need_b = (srow >> 5) < nnb;  // uniform per wavefront
+  const int soff = srow * kLsePitch + skh;
+
+  auto ld4 = [&](const float* base, int k0, int i) -> float4 {
+    // V % 4 == 0: a group of four is either fully inside the row or fully past it
+    const int v = k0 + skh + 4 * i;
+    const float4 x = *reinterpret_cast<const float4*>(base + (v < d.V ? k0 + 4 * i : 0));
+    const float4 pad = make_float4(kNegInf, kNegInf, kNegInf, kNegInf);
+    return v < d.V ? x : pad;
+  };
+  auto fetch = [&](int k0) -> LseStage {
+    LseStage r;
+    r.a0 = ld4(pa, k0, 0); r.a1 = ld4(pa, k0, 1); r.a2 = ld4(pa, k0, 2); r.a3 = ld4(pa, k0, 3);
+    if (need_b) {
+      r.b0 = ld4(pb, k0, 0); r.b1 = ld4(pb, k0, 1); r.b2 = ld4(pb, k0, 2); r.b3 = ld4(pb, k0, 3);
+    }
+    return r;
+  };
+  auto ex4 = [](const float4& x, float m) -> float4 {
+    return make_float4(__expf(x.x - m), __expf(x.y - m), __expf(x.z - m), __expf(x.w - m));
+  };
+  auto stash = [&](int buf, const LseStage& r) {
+    float* da = &As[buf][soff];
+    *reinterpret_cast<float4*>(da) = ex4(r.a0, ma);
+    *reinterpret_cast<float4*>(da + 4) = ex4(r.a1, ma);
+    *reinterpret_cast<float4*>(da + 8) = ex4(r.a2, ma);
+    *reinterpret_cast<float4*>(da + 12) = ex4(r.a3, ma);
+    if (need_b) {
+      float* db = &Bs[buf][soff];
+      *reinterpret_cast<float4*>(db) = ex4(r.b0, mb);
+      *reinterpret_cast<float4*>(db + 4) = ex4(r.b1, mb);
+      *reinterpret_cast<float4*>(db + 8) = ex4(r.b2, mb);
+      *reinterpret_cast<float4*>(db + 12) = ex4(r.b3, mb);
+    }
+  };
+
+  floatx16 acc[4], tot[4];
+#pragma unroll
+  for (int nb = 0; nb < 4; ++nb)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) { acc[nb][r] = 0.0f; tot[nb][r] = 0.0f; }
+
+  const int nk = (d.V + kLseBK - 1) / kLseBK;
+  stash(0, fetch(0));
+  __syncthreads();
+  int cur = 0;
+  for (int kt = 0; kt < nk; ++kt) {
+    const bool has_next = kt + 1 < nk;
+    LseStage nxt;
+    if (has_next) nxt = fetch((kt + 1) * kLseBK);
+    const float* arow = &As[cur][(32 * wave + l32) * kLsePitch + 4 * h];
+    const float* brow = &Bs[cur][l32 * kLsePitch + 4 * h];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float4 a4 = *reinterpret_cast<const float4*>(arow + 8 * j);
+      float4 b4[4];
+#pragma unroll
+      for (int nb = 0; nb < 4; ++nb)
+        if (nb < nnb) b4[nb] = *reinterpret_cast<const float4*>(brow + 32 * nb * kLsePitch + 8 * j);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const float av = q == 0 ? a4.x : (q == 1 ? a4.y : (q == 2 ? a4.z : a4.w));
+#pragma unroll
+        for (int nb = 0; nb < 4; ++nb)
+          if (nb < nnb) {
+            const float bv =
+                q == 0 ? b4[nb].x : (q == 1 ? b4[nb].y : (q == 2 ? b4[nb].z : b4[nb].w));
+            acc[nb] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc[nb], 0, 0, 0);
+          }
+      }
+    }
+    if ((kt + 1) % kLseFlush == 0) {
+#pragma unroll
+      for (int nb = 0; nb < 4; ++nb)
+        if (nb < nnb) {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) { tot[nb][r] += acc[nb][r]; acc[nb][r] = 0.0f; }
+        }
+    }
+    if (has_next) stash(cur ^ 1, nxt);
+    __syncthreads();
+    cur ^= 1;
+  }
+
+  const float* mEb = mE + (size_t)b * d.T;
+  const float* mPb = mP + (size_t)b * d.U;
+#pragma unroll
+  for (int nb = 0; nb < 4; ++nb)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int t = t0 + 32 * wave + 8 * (r >> 2) + 4 * h + (r & 3);
+      const int u = u0 + 32 * nb + l32;
+      if (t < d.T && u < d.U) {
+        float v = 0.0f;
+        if (nb < nnb && t < Tb && u < Ub) v = (logf(tot[nb][r] + acc[nb][r]) + mEb[t]) + mPb[u];
+        LNb[(size_t)t * d.U + u] = v;
+      }
+    }
 }
 
 // ------------------------------------------------------------------ W planes
@@ -316,11 +481,12 @@ __global__ __launch_bounds__(256, 2) void egrads_kernel(
     if (_e != hipSuccess) return check_hip(_e, "launch " name, __FILE__, __LINE__); \
   } while (0)
 
-int launch_rowmax(const float* X, float* rowmax, long rows, int V, hipStream_t s) {
+int launch_rowmax(const float* X, float* rowmax, long rows, int V, int rows_per_item,
+                  const int* lengths, int extra, hipStream_t s) {
   if (rows == 0) return kOk;
   const int vec4 = (V % 4 == 0) && ((reinterpret_cast<uintptr_t>(X) & 15) == 0);
   hipLaunchKernelGGL(rowmax_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, s, X, rowmax,
-                     rows, V, vec4);
+                     rows, V, vec4, rows_per_item, lengths, extra);
   RNNT_LAUNCH_CHECK("rowmax_kernel");
   return kOk;
 }
@@ -328,6 +494,18 @@ int launch_rowmax(const float* X, float* rowmax, long rows, int V, hipStream_t s
 int launch_lse(const float* E, const float* P, const float* mE, const float* mP, float* LN,
                const int* inLen, const int* labLen, const Dims& d, hipStream_t s) {
   if (d.B == 0 || d.T == 0 || d.U == 0) return kOk;
+  const bool aligned = ((reinterpret_cast<uintptr_t>(E) | reinterpret_cast<uintptr_t>(P)) & 15) == 0;
+  if (d.V % 4 == 0 && aligned) {
+    const int ttiles = (d.T + kLseBM - 1) / kLseBM, utiles = (d.U + kLseBN - 1) / kLseBN;
+    const long total = (long)ttiles * utiles * d.B;
+    if (total < (1l << 30)) {
+      const int grid = (int)((total + 7) / 8 * 8);
+      hipLaunchKernelGGL(lse_fast_kernel, dim3(grid), dim3(256), 0, s, E, P, mE, mP, LN, inLen,
+                         labLen, d, ttiles, utiles, (int)total);
+      RNNT_LAUNCH_CHECK("lse_fast_kernel");
+      return kOk;
+    }
+  }
   hipLaunchKernelGGL(lse_kernel,
                      dim3((d.T + kLseBM - 1) / kLseBM, (d.U + kLseBN - 1) / kLseBN, d.B),
                      dim3(256), 0, s, E, P, mE, mP, LN, inLen, labLen, d);

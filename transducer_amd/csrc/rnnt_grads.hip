@@ -32,7 +32,7 @@ __device__ inline float f4at(const float4& v, int q) {
 // ------------------------------------------------------------------ egrads
 constexpr int kEsMaxG = 14;              // groups of 8 label positions kept in registers
 constexpr int kEsKP = 8 * kEsMaxG + 4;   // LDS row pitch of the W slab (floats)
-constexpr int kEsSlab = 32 * kEsKP + 8;  // + a dump slot for staging lanes with nothing to do
+constexpr int kEsSlab = 32 * kEsKP;
 
 // Row of the 32x32 output block that register r of lane-half h holds.
 __device__ inline int mfma_row(int r, int h) { return 8 * (r >> 2) + 4 * h + (r & 3); }
@@ -89,12 +89,13 @@ __global__ __launch_bounds__(256, 2) void egrads_stream_kernel(
   // W slab staging: the 32 x Up slab of frame tile ti is one contiguous run of 8*Up float4
   const int up4 = Up >> 2, nvec = 8 * Up;
   int lds_off[4], src_idx[4];
+  bool vec_ok[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int idx = tid + 256 * i;
-    const bool ok = idx < nvec;
-    src_idx[i] = ok ? idx : nvec - 1;
-    lds_off[i] = ok ? (idx / up4) * kEsKP + 4 * (idx % up4) : 32 * kEsKP;
+    vec_ok[i] = idx < nvec;
+    src_idx[i] = vec_ok[i] ? idx : nvec - 1;  // loads stay unconditional, stores are masked
+    lds_off[i] = vec_ok[i] ? (idx / up4) * kEsKP + 4 * (idx % up4) : 0;
   }
   auto fetch_slab = [&](int ti) -> SlabRegs {
     const float4* src =
@@ -108,10 +109,10 @@ __global__ __launch_bounds__(256, 2) void egrads_stream_kernel(
     return s;
   };
   auto store_slab = [&](int buf, const SlabRegs& s) {
-    *reinterpret_cast<float4*>(&As[buf][lds_off[0]]) = s.v0;
-    *reinterpret_cast<float4*>(&As[buf][lds_off[1]]) = s.v1;
-    *reinterpret_cast<float4*>(&As[buf][lds_off[2]]) = s.v2;
-    *reinterpret_cast<float4*>(&As[buf][lds_off[3]]) = s.v3;
+    if (vec_ok[0]) *reinterpret_cast<float4*>(&As[buf][lds_off[0]]) = s.v0;
+    if (vec_ok[1]) *reinterpret_cast<float4*>(&As[buf][lds_off[1]]) = s.v1;
+    if (vec_ok[2]) *reinterpret_cast<float4*>(&As[buf][lds_off[2]]) = s.v2;
+    if (vec_ok[3]) *reinterpret_cast<float4*>(&As[buf][lds_off[3]]) = s.v3;
     if (tid < 32) Ms[buf][tid] = s.m;
   };
 

@@ -122,7 +122,10 @@ size_t viterbi_bits_bytes(const Dims& d);
 // ---------------------------------------------------------------- launchers (rnnt_gemm.hip)
 int wplane_up(int U);  // label-axis pitch of the W planes (multiple of 8)
 int wplane_tw(int T);  // frame-axis pitch of the W planes (multiple of 64)
-int launch_rowmax(const float* X, float* rowmax, long rows, int V, hipStream_t s);
+// Row maxima of a [rows, V] array.  With `lengths`, rows at or past lengths[item] + extra inside
+// their item (rows_per_item rows each) are not read and report 0.
+int launch_rowmax(const float* X, float* rowmax, long rows, int V, int rows_per_item,
+                  const int* lengths, int extra, hipStream_t s);
 int launch_lse(const float* E, const float* P, const float* mE, const float* mP, float* LN,
                const int* inLen, const int* labLen, const Dims& d, hipStream_t s);
 int launch_wplanes(const float* lngrads, const float* LN, const float* mE, const float* mP,
