@@ -216,52 +216,32 @@ struct LseStage {
   float4 a0, a1, a2, a3, b0, b1, b2, b3;
 };
 
-__global__ __launch_bounds__(256, 2) void lse_fast_kernel(const float* __restrict__ E,
-                                                          const float* __restrict__ P,
-                                                          const float* __restrict__ mE,
-                                                          const float* __restrict__ mP,
-                                                          float* __restrict__ LN,
-                                                          const int* __restrict__ inLen,
-                                                          const int* __restrict__ labLen, Dims d,
-                                                          int ttiles, int utiles, int total) {
-  __shared__ __attribute__((aligned(16))) float As[2][kLseBM * kLsePitch];
-  __shared__ __attribute__((aligned(16))) float Bs[2][kLseBN * kLsePitch];
-  // XCD-aware renumbering: physical id n runs on XCD n % 8
-  const int n = blockIdx.x, per_xcd = gridDim.x >> 3;
-  const int logical = (n & 7) * per_xcd + (n >> 3);
-  if (logical >= total) return;
-  const int b = logical / (ttiles * utiles);
-  const int rem = logical - b * (ttiles * utiles);
-  const int t0 = (rem % ttiles) * kLseBM, u0 = (rem / ttiles) * kLseBN;
-  int Tb, Ub;
-  utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
+// One 128 x (32*NNB) tile: the whole reduction over v and the write-out.  NNB is a template
+// parameter so that the matrix instructions of a slice form one straight-line block.
+template <int NNB>
+__device__ __forceinline__ void lse_tile(const float* __restrict__ E, const float* __restrict__ P,
+                                         const float* __restrict__ mE,
+                                         const float* __restrict__ mP, float* __restrict__ LNb,
+                                         float* As0, float* Bs0, const Dims& d, int b, int t0,
+                                         int u0, int Tb, int Ub) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, h = lane >> 5;
-  float* LNb = LN + (size_t)b * d.T * d.U;
-
-  if (t0 >= Tb || u0 >= Ub) {
-    for (int e = tid; e < kLseBM * kLseBN; e += 256) {
-      const int t = t0 + e / kLseBN, u = u0 + e % kLseBN;
-      if (t < d.T && u < d.U) LNb[(size_t)t * d.U + u] = 0.0f;
-    }
-    return;
-  }
-  const int nnb = min(4, (Ub - u0 + 31) >> 5);  // 32-wide label blocks in use
-
+  constexpr int kBuf = kLseBM * kLsePitch;
   // staging: thread -> row tid/2 of both operands, 16 consecutive v starting at 16*(tid%2)
   const int srow = tid >> 1, skh = (tid & 1) * 16;
   const int ta = min(t0 + srow, Tb - 1), ub = min(u0 + srow, Ub - 1);
   const float* pa = E + ((size_t)b * d.T + ta) * d.V + skh;
   const float* pb = P + ((size_t)b * d.U + ub) * d.V + skh;
   const float ma = mE[(size_t)b * d.T + ta], mb = mP[(size_t)b * d.U + ub];
-  const bool need_b = (srow >> 5) < nnb;  // uniform per wavefront
+  const bool need_b = (srow >> 5) < NNB;  // uniform per wavefront
   const int soff = srow * kLsePitch + skh;
 
+  // Loads only: nothing may touch the loaded registers before the matrix block of the current
+  // slice has been issued, or the wavefront would sit out the memory latency first.  A group
+  // of four past the end of the row (V % 4 == 0: never partly) re-reads the row start and is
+  // zeroed when it is staged.
   auto ld4 = [&](const float* base, int k0, int i) -> float4 {
-    // V % 4 == 0: a group of four is either fully inside the row or fully past it
     const int v = k0 + skh + 4 * i;
-    const float4 x = *reinterpret_cast<const float4*>(base + (v < d.V ? k0 + 4 * i : 0));
-    const float4 pad = make_float4(kNegInf, kNegInf, kNegInf, kNegInf);
-    return v < d.V ? x : pad;
+    return *reinterpret_cast<const float4*>(base + (v < d.V ? k0 + 4 * i : 0));
   };
   auto fetch = [&](int k0) -> LseStage {
     LseStage r;
@@ -271,68 +251,70 @@ __global__ __launch_bounds__(256, 2) void lse_fast_kernel(const float* __restric
     }
     return r;
   };
-  auto ex4 = [](const float4& x, float m) -> float4 {
-    return make_float4(__expf(x.x - m), __expf(x.y - m), __expf(x.z - m), __expf(x.w - m));
+  auto ex4 = [&](const float4& x, float m, int k0, int i) -> float4 {
+    const bool in = k0 + skh + 4 * i < d.V;
+    const float4 e = make_float4(__expf(x.x - m), __expf(x.y - m), __expf(x.z - m), __expf(x.w - m));
+    return in ? e : make_float4(0.f, 0.f, 0.f, 0.f);
   };
-  auto stash = [&](int buf, const LseStage& r) {
-    float* da = &As[buf][soff];
-    *reinterpret_cast<float4*>(da) = ex4(r.a0, ma);
-    *reinterpret_cast<float4*>(da + 4) = ex4(r.a1, ma);
-    *reinterpret_cast<float4*>(da + 8) = ex4(r.a2, ma);
-    *reinterpret_cast<float4*>(da + 12) = ex4(r.a3, ma);
+  auto stash = [&](int buf, const LseStage& r, int k0) {
+    float* da = As0 + buf * kBuf + soff;
+    *reinterpret_cast<float4*>(da) = ex4(r.a0, ma, k0, 0);
+    *reinterpret_cast<float4*>(da + 4) = ex4(r.a1, ma, k0, 1);
+    *reinterpret_cast<float4*>(da + 8) = ex4(r.a2, ma, k0, 2);
+    *reinterpret_cast<float4*>(da + 12) = ex4(r.a3, ma, k0, 3);
     if (need_b) {
-      float* db = &Bs[buf][soff];
-      *reinterpret_cast<float4*>(db) = ex4(r.b0, mb);
-      *reinterpret_cast<float4*>(db + 4) = ex4(r.b1, mb);
-      *reinterpret_cast<float4*>(db + 8) = ex4(r.b2, mb);
-      *reinterpret_cast<float4*>(db + 12) = ex4(r.b3, mb);
+      float* db = Bs0 + buf * kBuf + soff;
+      *reinterpret_cast<float4*>(db) = ex4(r.b0, mb, k0, 0);
+      *reinterpret_cast<float4*>(db + 4) = ex4(r.b1, mb, k0, 1);
+      *reinterpret_cast<float4*>(db + 8) = ex4(r.b2, mb, k0, 2);
+      *reinterpret_cast<float4*>(db + 12) = ex4(r.b3, mb, k0, 3);
     }
   };
 
-  floatx16 acc[4], tot[4];
+  floatx16 acc[NNB], tot[NNB];
 #pragma unroll
-  for (int nb = 0; nb < 4; ++nb)
+  for (int nb = 0; nb < NNB; ++nb)
 #pragma unroll
     for (int r = 0; r < 16; ++r) { acc[nb][r] = 0.0f; tot[nb][r] = 0.0f; }
 
   const int nk = (d.V + kLseBK - 1) / kLseBK;
-  stash(0, fetch(0));
+  stash(0, fetch(0), 0);
   __syncthreads();
   int cur = 0;
   for (int kt = 0; kt < nk; ++kt) {
     const bool has_next = kt + 1 < nk;
     LseStage nxt;
     if (has_next) nxt = fetch((kt + 1) * kLseBK);
-    const float* arow = &As[cur][(32 * wave + l32) * kLsePitch + 4 * h];
-    const float* brow = &Bs[cur][l32 * kLsePitch + 4 * h];
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_setprio(2);  // matrix phase: take the pipe from a wavefront that is staging
+    const float* arow = As0 + cur * kBuf + (32 * wave + l32) * kLsePitch + 4 * h;
+    const float* brow = Bs0 + cur * kBuf + l32 * kLsePitch + 4 * h;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const float4 a4 = *reinterpret_cast<const float4*>(arow + 8 * j);
-      float4 b4[4];
+      float4 b4[NNB];
 #pragma unroll
-      for (int nb = 0; nb < 4; ++nb)
-        if (nb < nnb) b4[nb] = *reinterpret_cast<const float4*>(brow + 32 * nb * kLsePitch + 8 * j);
+      for (int nb = 0; nb < NNB; ++nb)
+        b4[nb] = *reinterpret_cast<const float4*>(brow + 32 * nb * kLsePitch + 8 * j);
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         const float av = q == 0 ? a4.x : (q == 1 ? a4.y : (q == 2 ? a4.z : a4.w));
 #pragma unroll
-        for (int nb = 0; nb < 4; ++nb)
-          if (nb < nnb) {
-            const float bv =
-                q == 0 ? b4[nb].x : (q == 1 ? b4[nb].y : (q == 2 ? b4[nb].z : b4[nb].w));
-            acc[nb] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc[nb], 0, 0, 0);
-          }
+        for (int nb = 0; nb < NNB; ++nb) {
+          const float bv = q == 0 ? b4[nb].x : (q == 1 ? b4[nb].y : (q == 2 ? b4[nb].z : b4[nb].w));
+          acc[nb] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc[nb], 0, 0, 0);
+        }
       }
     }
+    __builtin_amdgcn_s_setprio(0);
+    __builtin_amdgcn_sched_barrier(0);
     if ((kt + 1) % kLseFlush == 0) {
 #pragma unroll
-      for (int nb = 0; nb < 4; ++nb)
-        if (nb < nnb) {
+      for (int nb = 0; nb < NNB; ++nb)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) { tot[nb][r] += acc[nb][r]; acc[nb][r] = 0.0f; }
-        }
+        for (int r = 0; r < 16; ++r) { tot[nb][r] += acc[nb][r]; acc[nb][r] = 0.0f; }
     }
-    if (has_next) stash(cur ^ 1, nxt);
+    if (has_next) stash(cur ^ 1, nxt, (kt + 1) * kLseBK);
     __syncthreads();
     cur ^= 1;
   }
@@ -347,10 +329,49 @@ __global__ __launch_bounds__(256, 2) void lse_fast_kernel(const float* __restric
       const int u = u0 + 32 * nb + l32;
       if (t < d.T && u < d.U) {
         float v = 0.0f;
-        if (nb < nnb && t < Tb && u < Ub) v = (logf(tot[nb][r] + acc[nb][r]) + mEb[t]) + mPb[u];
+        if (nb < NNB) {
+          const int nbc = nb < NNB ? nb : 0;
+          if (t < Tb && u < Ub) v = (logf(tot[nbc][r] + acc[nbc][r]) + mEb[t]) + mPb[u];
+        }
         LNb[(size_t)t * d.U + u] = v;
       }
     }
+}
+
+__global__ __launch_bounds__(256, 2) void lse_fast_kernel(const float* __restrict__ E,
+                                                          const float* __restrict__ P,
+                                                          const float* __restrict__ mE,
+                                                          const float* __restrict__ mP,
+                                                          float* __restrict__ LN,
+                                                          const int* __restrict__ inLen,
+                                                          const int* __restrict__ labLen, Dims d,
+                                                          int ttiles, int utiles, int total) {
+  __shared__ __attribute__((aligned(16))) float As[2 * kLseBM * kLsePitch];
+  __shared__ __attribute__((aligned(16))) float Bs[2 * kLseBN * kLsePitch];
+  // XCD-aware renumbering: physical id n runs on XCD n % 8
+  const int n = blockIdx.x, per_xcd = gridDim.x >> 3;
+  const int logical = (n & 7) * per_xcd + (n >> 3);
+  if (logical >= total) return;
+  const int b = logical / (ttiles * utiles);
+  const int rem = logical - b * (ttiles * utiles);
+  const int t0 = (rem % ttiles) * kLseBM, u0 = (rem / ttiles) * kLseBN;
+  int Tb, Ub;
+  utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
+  float* LNb = LN + (size_t)b * d.T * d.U;
+
+  if (t0 >= Tb || u0 >= Ub) {
+    for (int e = threadIdx.x; e < kLseBM * kLseBN; e += 256) {
+      const int t = t0 + e / kLseBN, u = u0 + e % kLseBN;
+      if (t < d.T && u < d.U) LNb[(size_t)t * d.U + u] = 0.0f;
+    }
+    return;
+  }
+  switch (min(4, (Ub - u0 + 31) >> 5)) {  // 32-wide label blocks in use
+    case 1: lse_tile<1>(E, P, mE, mP, LNb, As, Bs, d, b, t0, u0, Tb, Ub); break;
+    case 2: lse_tile<2>(E, P, mE, mP, LNb, As, Bs, d, b, t0, u0, Tb, Ub); break;
+    case 3: lse_tile<3>(E, P, mE, mP, LNb, As, Bs, d, b, t0, u0, Tb, Ub); break;
+    default: lse_tile<4>(E, P, mE, mP, LNb, As, Bs, d, b, t0, u0, Tb, Ub); break;
+  }
 }
 
 // ------------------------------------------------------------------ W planes

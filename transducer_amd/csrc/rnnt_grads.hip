@@ -147,6 +147,8 @@ __global__ __launch_bounds__(256, 2) void egrads_stream_kernel(
     floatx16 acc;
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_setprio(2);  // matrix phase first; the other wavefronts' epilogues fill in
     const float* arow = &As[cur][l32 * kEsKP + 4 * h];
     float4 a_next = *reinterpret_cast<const float4*>(arow);
 #pragma unroll
@@ -160,6 +162,8 @@ __global__ __launch_bounds__(256, 2) void egrads_stream_kernel(
         acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a4.w, Yr[j][3], acc, 0, 0, 0);
       }
     }
+    __builtin_amdgcn_s_setprio(0);
+    __builtin_amdgcn_sched_barrier(0);
     if (interior) {
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
@@ -294,6 +298,8 @@ __global__ __launch_bounds__(256, 2) void pgrads_stream_kernel(
         xr = fetch_x((kt + 1) * 32);
       }
       const float* abase = &As[cur][l32 * kPsKP + 4 * h];
+      __builtin_amdgcn_sched_barrier(0);
+      __builtin_amdgcn_s_setprio(2);
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         float4 a4[4];
@@ -309,6 +315,8 @@ __global__ __launch_bounds__(256, 2) void pgrads_stream_kernel(
               acc[mb] = __builtin_amdgcn_mfma_f32_32x32x2f32(f4at(a4[mb], q), x[j][q], acc[mb],
                                                               0, 0, 0);
       }
+      __builtin_amdgcn_s_setprio(0);
+      __builtin_amdgcn_sched_barrier(0);
       if (has_next) store_slab(cur ^ 1, nxt);
       __syncthreads();
       cur ^= 1;
