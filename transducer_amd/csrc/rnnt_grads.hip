@@ -42,17 +42,16 @@ struct SlabRegs {
   float m;
 };
 
-template <bool kAccumulate>
-__global__ __launch_bounds__(256, 2) void egrads_stream_kernel(
+// The walk of one workgroup over its frame tiles with NG groups of eight label positions
+// (a template parameter, so the matrix instructions of a tile form one straight-line block).
+// Label positions past the utterance contribute exact zeros: their Y rows are masked and the
+// W slab is zero there.
+template <int NG, bool kAccumulate>
+__device__ __forceinline__ void egrads_walk(
     const float* __restrict__ E, const float* __restrict__ P, const float* __restrict__ mE,
     const float* __restrict__ mP, const float* __restrict__ Wn, const float* __restrict__ deltas,
-    float* __restrict__ egrads, const int* __restrict__ inLen, const int* __restrict__ labLen,
-    Dims d, int Up, int Tw, int tiles_per_chunk) {
-  __shared__ __attribute__((aligned(16))) float As[2][kEsSlab];
-  __shared__ __attribute__((aligned(16))) float Ms[2][32];  // mE of the slab's frames
-  const int b = blockIdx.z;
-  int Tb, Ub;
-  utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
+    float* __restrict__ egrads, float (*As)[kEsSlab], float (*Ms)[32], const Dims& d, int Up,
+    int Tw, int tiles_per_chunk, int b, int Tb, int Ub) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, h = lane >> 5;
   const int wave_col0 = blockIdx.x * 128 + wave * 32;  // this wavefront's 32 columns
   const int vcol = wave_col0 + l32;
@@ -63,19 +62,18 @@ __global__ __launch_bounds__(256, 2) void egrads_stream_kernel(
   const int tile_lo = blockIdx.y * tiles_per_chunk;
   const int tile_hi = min(tile_lo + tiles_per_chunk, ntiles);
   const int tile_valid = min(tile_hi, (Tb + 31) >> 5);  // tiles that hold frames of the utterance
-  const int ngroups = (Ub + 7) >> 3;
   const float delta = deltas ? deltas[b] : 1.0f;
   const float* Eb = E + (size_t)b * d.T * d.V;
   float* out = egrads + (size_t)b * d.T * d.V;
   const float* mEb = mE + (size_t)b * d.T;
 
   // Y fragments for this wavefront's columns (branch-free: clamped address, masked value)
-  float Yr[kEsMaxG][4];
+  float Yr[NG][4];
   if (tile_lo < tile_valid) {
     const float* Pb = P + (size_t)b * d.U * d.V;
     const float* mPb = mP + (size_t)b * d.U;
 #pragma unroll
-    for (int j = 0; j < kEsMaxG; ++j)
+    for (int j = 0; j < NG; ++j)
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         const int u = 8 * j + 4 * h + q;
@@ -150,17 +148,15 @@ __global__ __launch_bounds__(256, 2) void egrads_stream_kernel(
     __builtin_amdgcn_sched_barrier(0);
     __builtin_amdgcn_s_setprio(2);  // matrix phase first; the other wavefronts' epilogues fill in
     const float* arow = &As[cur][l32 * kEsKP + 4 * h];
-    float4 a_next = *reinterpret_cast<const float4*>(arow);
+    float4 a4[NG];
 #pragma unroll
-    for (int j = 0; j < kEsMaxG; ++j) {
-      if (j < ngroups) {
-        const float4 a4 = a_next;
-        if (j + 1 < ngroups) a_next = *reinterpret_cast<const float4*>(arow + 8 * (j + 1));
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a4.x, Yr[j][0], acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a4.y, Yr[j][1], acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a4.z, Yr[j][2], acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a4.w, Yr[j][3], acc, 0, 0, 0);
-      }
+    for (int j = 0; j < NG; ++j) a4[j] = *reinterpret_cast<const float4*>(arow + 8 * j);
+#pragma unroll
+    for (int j = 0; j < NG; ++j) {
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a4[j].x, Yr[j][0], acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a4[j].y, Yr[j][1], acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a4[j].z, Yr[j][2], acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a4[j].w, Yr[j][3], acc, 0, 0, 0);
     }
     __builtin_amdgcn_s_setprio(0);
     __builtin_amdgcn_sched_barrier(0);
@@ -206,31 +202,57 @@ __global__ __launch_bounds__(256, 2) void egrads_stream_kernel(
   }
 }
 
+template <bool kAccumulate>
+__global__ __launch_bounds__(256, 2) void egrads_stream_kernel(
+    const float* __restrict__ E, const float* __restrict__ P, const float* __restrict__ mE,
+    const float* __restrict__ mP, const float* __restrict__ Wn, const float* __restrict__ deltas,
+    float* __restrict__ egrads, const int* __restrict__ inLen, const int* __restrict__ labLen,
+    Dims d, int Up, int Tw, int tiles_per_chunk) {
+  __shared__ __attribute__((aligned(16))) float As[2][kEsSlab];
+  __shared__ __attribute__((aligned(16))) float Ms[2][32];  // mE of the slab's frames
+  const int b = blockIdx.z;
+  int Tb, Ub;
+  utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
+  // columns of the slab past Up are never staged; clear them once so that a walk that rounds
+  // its group count up multiplies zeros there, not whatever the LDS held
+  for (int e = threadIdx.x; e < 2 * kEsSlab; e += 256) (&As[0][0])[e] = 0.0f;
+  __syncthreads();
+  const int ngroups = (Ub + 7) >> 3;
+#define RNNT_EG_WALK(NG)                                                                      \
+  egrads_walk<NG, kAccumulate>(E, P, mE, mP, Wn, deltas, egrads, As, Ms, d, Up, Tw,          \
+                               tiles_per_chunk, b, Tb, Ub)
+  if (ngroups <= 4) RNNT_EG_WALK(4);
+  else if (ngroups <= 8) RNNT_EG_WALK(8);
+  else if (ngroups <= 10) RNNT_EG_WALK(10);
+  else if (ngroups == 11) RNNT_EG_WALK(11);
+  else if (ngroups == 12) RNNT_EG_WALK(12);
+  else if (ngroups == 13) RNNT_EG_WALK(13);
+  else RNNT_EG_WALK(14);
+#undef RNNT_EG_WALK
+}
+
 // ------------------------------------------------------------------ pgrads
 constexpr int kPsKP = 32 + 4;  // LDS row pitch of the W^T slab (floats)
 
-template <bool kAccumulate>
-__global__ __launch_bounds__(256, 2) void pgrads_stream_kernel(
+// One workgroup's 128 x 128 tile with NMB 32-row blocks of label positions in use (a template
+// parameter, so the matrix instructions of a slice form one straight-line block).
+template <int NMB, bool kAccumulate>
+__device__ __forceinline__ void pgrads_tile(
     const float* __restrict__ E, const float* __restrict__ P, const float* __restrict__ mE,
     const float* __restrict__ mP, const float* __restrict__ Wt, const float* __restrict__ deltas,
-    float* __restrict__ pgrads, const int* __restrict__ inLen, const int* __restrict__ labLen,
-    Dims d, int Up, int Tw) {
-  __shared__ __attribute__((aligned(16))) float As[2][128 * kPsKP];
-  __shared__ __attribute__((aligned(16))) float Ms[2][32];
-  const int b = blockIdx.z, u0 = blockIdx.y * 128;
-  int Tb, Ub;
-  utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
+    float* __restrict__ pgrads, float (*As)[128 * kPsKP], float (*Ms)[32], const Dims& d, int Up,
+    int Tw, int b, int u0, int Tb, int Ub) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, h = lane >> 5;
   const int vcol = blockIdx.x * 128 + wave * 32 + l32;
   const bool vok = vcol < d.V;
   const int vc = vok ? vcol : d.V - 1;
   const float delta = deltas ? deltas[b] : 1.0f;
   float* out = pgrads + (size_t)b * d.U * d.V;
-  const int nmb = (u0 < Ub && Tb > 0) ? min(4, (Ub - u0 + 31) >> 5) : 0;  // 32-row blocks in use
+  constexpr int nmb = NMB;
 
-  floatx16 acc[4];
+  floatx16 acc[NMB > 0 ? NMB : 1];
 #pragma unroll
-  for (int mb = 0; mb < 4; ++mb)
+  for (int mb = 0; mb < NMB; ++mb)
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[mb][r] = 0.0f;
 
@@ -302,18 +324,16 @@ __global__ __launch_bounds__(256, 2) void pgrads_stream_kernel(
       __builtin_amdgcn_s_setprio(2);
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        float4 a4[4];
+        float4 a4[NMB > 0 ? NMB : 1];
 #pragma unroll
-        for (int mb = 0; mb < 4; ++mb)
-          if (mb < nmb)
-            a4[mb] = *reinterpret_cast<const float4*>(abase + 32 * mb * kPsKP + 8 * j);
+        for (int mb = 0; mb < NMB; ++mb)
+          a4[mb] = *reinterpret_cast<const float4*>(abase + 32 * mb * kPsKP + 8 * j);
 #pragma unroll
         for (int q = 0; q < 4; ++q)
 #pragma unroll
-          for (int mb = 0; mb < 4; ++mb)
-            if (mb < nmb)
-              acc[mb] = __builtin_amdgcn_mfma_f32_32x32x2f32(f4at(a4[mb], q), x[j][q], acc[mb],
-                                                              0, 0, 0);
+          for (int mb = 0; mb < NMB; ++mb)
+            acc[mb] = __builtin_amdgcn_mfma_f32_32x32x2f32(f4at(a4[mb], q), x[j][q], acc[mb], 0,
+                                                            0, 0);
       }
       __builtin_amdgcn_s_setprio(0);
       __builtin_amdgcn_sched_barrier(0);
@@ -332,12 +352,37 @@ __global__ __launch_bounds__(256, 2) void pgrads_stream_kernel(
       const int u = u0 + 32 * mb + mfma_row(r, h);
       const int uc = min(u, d.U - 1);
       const float y = __expf(Pb[(size_t)uc * d.V + vc] - mPb[uc]);
-      const float g = (mb < nmb && u < Ub) ? y * acc[mb][r] : 0.0f;
+      const float g = (mb < NMB && u < Ub) ? y * acc[mb < NMB ? mb : 0][r] : 0.0f;
       if (u < d.U && vok) {
         float* o = out + (size_t)u * d.V + vcol;
         o[0] = delta * (kAccumulate ? o[0] + g : g);
       }
     }
+}
+
+template <bool kAccumulate>
+__global__ __launch_bounds__(256, 2) void pgrads_stream_kernel(
+    const float* __restrict__ E, const float* __restrict__ P, const float* __restrict__ mE,
+    const float* __restrict__ mP, const float* __restrict__ Wt, const float* __restrict__ deltas,
+    float* __restrict__ pgrads, const int* __restrict__ inLen, const int* __restrict__ labLen,
+    Dims d, int Up, int Tw) {
+  __shared__ __attribute__((aligned(16))) float As[2][128 * kPsKP];
+  __shared__ __attribute__((aligned(16))) float Ms[2][32];
+  const int b = blockIdx.z, u0 = blockIdx.y * 128;
+  int Tb, Ub;
+  utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
+  const int nmb = (u0 < Ub && Tb > 0) ? min(4, (Ub - u0 + 31) >> 5) : 0;  // 32-row blocks in use
+#define RNNT_PG_TILE(NMB)                                                                    \
+  pgrads_tile<NMB, kAccumulate>(E, P, mE, mP, Wt, deltas, pgrads, As, Ms, d, Up, Tw, b, u0, \
+                                Tb, Ub)
+  switch (nmb) {
+    case 0: RNNT_PG_TILE(0); break;
+    case 1: RNNT_PG_TILE(1); break;
+    case 2: RNNT_PG_TILE(2); break;
+    case 3: RNNT_PG_TILE(3); break;
+    default: RNNT_PG_TILE(4); break;
+  }
+#undef RNNT_PG_TILE
 }
 
 }  // namespace
