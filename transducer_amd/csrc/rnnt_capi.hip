@@ -115,7 +115,7 @@ bool nothing_to_do(int B, int T, int U) { return B == 0 || T == 0 || U == 0; }
 
 struct LossWorkspace {
   Planes planes;
-  float *mE, *mP, *LN, *lngrads, *Wn, *Wt;
+  float *mE, *mP, *LN, *lngrads, *Wn, *Wt, *bsum;
 };
 
 size_t loss_workspace_layout(const Dims& d, void* base, LossWorkspace* w) {
@@ -137,7 +137,10 @@ size_t loss_workspace_layout(const Dims& d, void* base, LossWorkspace* w) {
   const size_t wb = sizeof(float) * (size_t)d.B * wplane_tw(d.T) * wplane_up(d.U);
   float* Wn = take(wb);
   float* Wt = take(wb);
-  if (base) { w->mE = mE; w->mP = mP; w->LN = LN; w->lngrads = lng; w->Wn = Wn; w->Wt = Wt; }
+  float* bsum = take(sizeof(float) * (size_t)d.B * d.T);
+  if (base) {
+    w->mE = mE; w->mP = mP; w->LN = LN; w->lngrads = lng; w->Wn = Wn; w->Wt = Wt; w->bsum = bsum;
+  }
   return off;
 }
 
@@ -316,7 +319,8 @@ int rnnt_hip_dense_grads(const float* E, const float* P, float* egrads, float* p
   RNNT_STAGE(kRowmax, launch_rowmax(E, mE, (long)B * T, V, T, inLen, 0, s));
   RNNT_STAGE(kRowmax, launch_rowmax(P, mP, (long)B * U, V, U, labLen, 1, s));
   RNNT_STAGE(kWplanes, launch_wplanes(lngrads, LN, mE, mP, Wn, Wt, inLen, labLen, d, s));
-  RNNT_STAGE(kEgrads, launch_egrads(E, P, mE, mP, Wn, deltas, egrads, inLen, labLen, d, true, s));
+  RNNT_STAGE(kEgrads, launch_egrads(E, P, mE, mP, Wn, deltas, egrads, inLen, labLen, d, true,
+                                    SparseTerms(), s));
   RNNT_STAGE(kPgrads, launch_pgrads(E, P, mE, mP, Wt, deltas, pgrads, inLen, labLen, d, true, s));
   return kOk;
 }
@@ -380,9 +384,22 @@ int rnnt_hip_loss_backward(const float* E, const float* P, const int* labels, co
   RNNT_STAGE(kBeta, launch_beta(w.planes, labels, inLen, labLen, d, s));
   RNNT_STAGE(kUnskew, launch_unskew(w.planes.dS, w.lngrads, inLen, labLen, d, s));
   RNNT_STAGE(kWplanes, launch_wplanes(w.lngrads, w.LN, w.mE, w.mP, w.Wn, w.Wt, inLen, labLen, d, s));
-  RNNT_STAGE(kEgrads, launch_egrads(E, P, w.mE, w.mP, w.Wn, deltas, egrads, inLen, labLen, d, false, s));
+  // The blank/label terms of egrads are folded into the dense kernel's write-out (a scatter
+  // afterwards would touch one cache line of the 2.5 GB array per lattice cell); for label axes
+  // too long for that kernel they are scattered as in rnnt_hip_backward.
+  const bool fold = egrads_fusion_supported(d) && labels != nullptr;
+  SparseTerms sp;
+  if (fold) {
+    RNNT_STAGE(kSparse, launch_blank_sums(w.planes, w.bsum, labels, inLen, labLen, d, s));
+    sp.dS = w.planes.dS; sp.wE = w.planes.wE; sp.bsum = w.bsum; sp.labels = labels;
+  }
+  RNNT_STAGE(kEgrads, launch_egrads(E, P, w.mE, w.mP, w.Wn, deltas, egrads, inLen, labLen, d, false,
+                                    sp, s));
   RNNT_STAGE(kPgrads, launch_pgrads(E, P, w.mE, w.mP, w.Wt, deltas, pgrads, inLen, labLen, d, false, s));
-  RNNT_STAGE(kSparse, launch_sparse(w.planes, egrads, pgrads, labels, inLen, labLen, deltas, true, d, s));
+  if (fold)
+    RNNT_STAGE(kSparse, launch_sparse_p(w.planes, pgrads, labels, inLen, labLen, deltas, true, d, s));
+  else
+    RNNT_STAGE(kSparse, launch_sparse(w.planes, egrads, pgrads, labels, inLen, labLen, deltas, true, d, s));
   return kOk;
 }
 

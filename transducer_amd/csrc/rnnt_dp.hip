@@ -448,6 +448,34 @@ __global__ __launch_bounds__(256) void sparse_e_kernel(Planes p, float* __restri
   else row[d.blank] = blank_acc;
 }
 
+// Per-frame total of everything the reference subtracts from egrads[t, blank]
+// (transducer/transducer_cpu.cpp:96,106,138 and the label moves whose label is the blank): the
+// value sparse_e_kernel would leave in that column.  Used when the label-column terms are folded
+// into the dense egrads kernel instead of being scattered afterwards.
+__global__ __launch_bounds__(256) void blank_sums_kernel(Planes p, float* __restrict__ bsum,
+                                                         const int* __restrict__ labels,
+                                                         const int* __restrict__ inLen,
+                                                         const int* __restrict__ labLen, Dims d) {
+  const int b = blockIdx.y;
+  const int t = blockIdx.x * 256 + threadIdx.x;
+  int Tb, Ub;
+  utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
+  if (Ub == 0 || t >= Tb) return;
+  const int* __restrict__ lab = labels + (size_t)b * (d.U - 1);
+  const float* __restrict__ dS = p.dS;
+  const float* __restrict__ wB = p.wB;
+  const float* __restrict__ wE = p.wE;
+  const bool has_stay = t + 1 < Tb;
+  float acc = (t == Tb - 1) ? -1.0f : 0.0f;
+  for (int u = Ub - 1; u >= 0; --u) {
+    const size_t o = plane_row(d, b, u) + t + u;
+    const float ne = dS[o + 1] * wB[o];
+    acc -= has_stay ? ne : 0.0f;
+    if (u + 1 < Ub && lab[u] == d.blank) acc -= dS[o + d.Dp + 1] * wE[o];
+  }
+  bsum[(size_t)b * d.T + t] = acc;
+}
+
 __global__ __launch_bounds__(256) void sparse_p_kernel(Planes p, float* __restrict__ pgrads,
                                                        const int* __restrict__ labels,
                                                        const int* __restrict__ inLen,
@@ -777,6 +805,25 @@ int launch_sparse(const Planes& p, float* egrads, float* pgrads, const int* labe
   hipLaunchKernelGGL(sparse_e_kernel, dim3((d.T + 255) / 256, d.B), dim3(256), 0, s, p, egrads,
                      labels, inLen, labLen, scale, add ? 1 : 0, d);
   RNNT_LAUNCH_CHECK("sparse_e_kernel");
+  hipLaunchKernelGGL(sparse_p_kernel, dim3((d.U + 255) / 256, d.B), dim3(256), 0, s, p, pgrads,
+                     labels, inLen, labLen, scale, add ? 1 : 0, d);
+  RNNT_LAUNCH_CHECK("sparse_p_kernel");
+  return kOk;
+}
+
+int launch_blank_sums(const Planes& p, float* bsum, const int* labels, const int* inLen,
+                      const int* labLen, const Dims& d, hipStream_t s) {
+  if (d.B == 0 || d.T == 0 || d.U == 0) return kOk;
+  hipLaunchKernelGGL(blank_sums_kernel, dim3((d.T + 255) / 256, d.B), dim3(256), 0, s, p, bsum,
+                     labels, inLen, labLen, d);
+  RNNT_LAUNCH_CHECK("blank_sums_kernel");
+  return kOk;
+}
+
+int launch_sparse_p(const Planes& p, float* pgrads, const int* labels, const int* inLen,
+                    const int* labLen, const float* scale, bool add, const Dims& d,
+                    hipStream_t s) {
+  if (d.B == 0 || d.T == 0 || d.U == 0) return kOk;
   hipLaunchKernelGGL(sparse_p_kernel, dim3((d.U + 255) / 256, d.B), dim3(256), 0, s, p, pgrads,
                      labels, inLen, labLen, scale, add ? 1 : 0, d);
   RNNT_LAUNCH_CHECK("sparse_p_kernel");

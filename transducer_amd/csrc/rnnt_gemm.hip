@@ -548,12 +548,17 @@ int launch_wplanes(const float* lngrads, const float* LN, const float* mE, const
   return kOk;
 }
 
+bool egrads_fusion_supported(const Dims& d) { return egrads_stream_supported(d); }
+
 int launch_egrads(const float* E, const float* P, const float* mE, const float* mP,
                   const float* Wn, const float* deltas, float* egrads, const int* inLen,
-                  const int* labLen, const Dims& d, bool accumulate, hipStream_t s) {
+                  const int* labLen, const Dims& d, bool accumulate, const SparseTerms& sparse,
+                  hipStream_t s) {
   if (d.B == 0 || d.T == 0 || d.U == 0) return kOk;
   if (egrads_stream_supported(d))
-    return launch_egrads_stream(E, P, mE, mP, Wn, deltas, egrads, inLen, labLen, d, accumulate, s);
+    return launch_egrads_stream(E, P, mE, mP, Wn, deltas, egrads, inLen, labLen, d, accumulate,
+                                sparse, s);
+  if (sparse.labels) return fail(kInvalid, "sparse-term folding needs the streaming egrads kernel");
   const int Up = wplane_up(d.U), Tw = wplane_tw(d.T);
   // label axes longer than one LDS slice are contracted slice by slice, accumulating
   for (int kofs = 0; kofs < Up; kofs += kEgMaxK) {

@@ -33,6 +33,7 @@ __device__ inline float f4at(const float4& v, int q) {
 constexpr int kEsMaxG = 14;              // groups of 8 label positions kept in registers
 constexpr int kEsKP = 8 * kEsMaxG + 4;   // LDS row pitch of the W slab (floats)
 constexpr int kEsSlab = 32 * kEsKP;
+constexpr int kEsPrefetch = 2;          // labels per 32-column block whose sparse terms are prefetched
 
 // Row of the 32x32 output block that register r of lane-half h holds.
 __device__ inline int mfma_row(int r, int h) { return 8 * (r >> 2) + 4 * h + (r & 3); }
@@ -51,13 +52,17 @@ __device__ __forceinline__ void egrads_walk(
     const float* __restrict__ E, const float* __restrict__ P, const float* __restrict__ mE,
     const float* __restrict__ mP, const float* __restrict__ Wn, const float* __restrict__ deltas,
     float* __restrict__ egrads, float (*As)[kEsSlab], float (*Ms)[32], const Dims& d, int Up,
-    int Tw, int tiles_per_chunk, int b, int Tb, int Ub) {
+    int Tw, int tiles_per_chunk, int b, int Tb, int Ub, const SparseTerms& sp,
+    const unsigned short* match, int nmatch, float (*Sp)[32]) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, h = lane >> 5;
   const int wave_col0 = blockIdx.x * 128 + wave * 32;  // this wavefront's 32 columns
   const int vcol = wave_col0 + l32;
   const bool vok = vcol < d.V;
   const int vc = vok ? vcol : d.V - 1;  // always readable
   const bool cols_full = wave_col0 + 32 <= d.V;
+  // lane that owns the blank column, if it is one of this wavefront's and terms are folded in
+  const int blank_lane = (sp.labels && d.blank >= wave_col0 && d.blank < wave_col0 + 32)
+                             ? d.blank - wave_col0 : -1;
   const int ntiles = (d.T + 31) >> 5;
   const int tile_lo = blockIdx.y * tiles_per_chunk;
   const int tile_hi = min(tile_lo + tiles_per_chunk, ntiles);
@@ -118,6 +123,13 @@ __device__ __forceinline__ void egrads_walk(
   if (tile_lo < tile_valid) store_slab(0, fetch_slab(tile_lo));
   __syncthreads();
 
+  // the first kEsPrefetch matches, resolved once: label position and target lane
+  int mu[kEsPrefetch], mc[kEsPrefetch];
+#pragma unroll
+  for (int i = 0; i < kEsPrefetch; ++i) {
+    mu[i] = (sp.labels && i < nmatch) ? match[i] : 0;
+    mc[i] = (sp.labels && i < nmatch) ? sp.labels[(size_t)b * (d.U - 1) + mu[i]] - wave_col0 : -1;
+  }
   // per-lane part of the element offset inside a tile; the per-register part is r-dependent
   // only through compile-time multiples of V
   const unsigned lane_off = (unsigned)(4 * h) * (unsigned)d.V + (unsigned)vcol;
@@ -142,6 +154,19 @@ __device__ __forceinline__ void egrads_walk(
       for (int r = 0; r < 16; ++r)
         ev[r] = Eb[(size_t)min(t0 + mfma_row(r, h), Tb - 1) * d.V + vc];
     }
+    // sparse terms of this tile for up to kEsPrefetch labels that fall into this wavefront's
+    // columns: one coalesced load per plane, requested here so it arrives under the matrix work
+    float sd[kEsPrefetch], sw[kEsPrefetch], sbl = 0.0f;
+    if (!kAccumulate && (nmatch > 0 || blank_lane >= 0)) {
+      const int tr = min(t0 + l32, Tb - 1);
+#pragma unroll
+      for (int i = 0; i < kEsPrefetch; ++i) {
+        const size_t o = plane_row(d, b, mu[i]) + tr + mu[i];
+        sd[i] = sp.dS[o + d.Dp + 1];
+        sw[i] = sp.wE[o];
+      }
+      if (blank_lane >= 0) sbl = sp.bsum[(size_t)b * d.T + tr];
+    }
     floatx16 acc;
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
@@ -160,27 +185,60 @@ __device__ __forceinline__ void egrads_walk(
     }
     __builtin_amdgcn_s_setprio(0);
     __builtin_amdgcn_sched_barrier(0);
+    float v[16];
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const float4 m4 = *reinterpret_cast<const float4*>(&Ms[cur][8 * g + 4 * h]);
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const int r = 4 * g + k;
+        const float x = __expf(ev[r] - f4at(m4, k)) * acc[r];
+        v[r] = (interior || t0 + mfma_row(r, h) < Tb) ? x : 0.0f;
+      }
+    }
+    if (!kAccumulate && (nmatch > 0 || blank_lane >= 0)) {  // uniform per wavefront, and rare
+      // Lane l32 holds the term of frame t0+l32 (fetched before the matrix block).  The terms go
+      // through a per-wavefront LDS strip; the two lanes that own the target column read their
+      // 16 frames back as four 16-byte loads.
+      const bool row_ok = t0 + l32 < Tb;
+      float* strip = &Sp[0][0];
+      auto apply = [&](float term, int col, float sign) {
+        if (h == 0) strip[l32] = term;
+        if (l32 == col) {
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            const float4 x = *reinterpret_cast<const float4*>(&strip[8 * g + 4 * h]);
+            v[4 * g + 0] += sign * x.x;
+            v[4 * g + 1] += sign * x.y;
+            v[4 * g + 2] += sign * x.z;
+            v[4 * g + 3] += sign * x.w;
+          }
+        }
+      };
+#pragma unroll
+      for (int i = 0; i < kEsPrefetch; ++i)
+        if (i < nmatch) apply(row_ok ? sd[i] * sw[i] : 0.0f, mc[i], -1.0f);
+      for (int i = kEsPrefetch; i < nmatch; ++i) {  // more labels in one 32-column block
+        const int u = match[i];
+        const size_t o = plane_row(d, b, u) + min(t0 + l32, Tb - 1) + u;
+        apply(row_ok ? sp.dS[o + d.Dp + 1] * sp.wE[o] : 0.0f,
+              sp.labels[(size_t)b * (d.U - 1) + u] - wave_col0, -1.0f);
+      }
+      if (blank_lane >= 0) apply(row_ok ? sbl : 0.0f, blank_lane, 1.0f);
+    }
     if (interior) {
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const float4 m4 = *reinterpret_cast<const float4*>(&Ms[cur][8 * g + 4 * h]);
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-          const int r = 4 * g + k;
-          const float v = __expf(ev[r] - f4at(m4, k)) * acc[r];
-          float* o = Otile + lane_off + (unsigned)(8 * g + k) * (unsigned)d.V;
-          *o = delta * (kAccumulate ? *o + v : v);
-        }
+      for (int r = 0; r < 16; ++r) {
+        float* o = Otile + lane_off + (unsigned)(8 * (r >> 2) + (r & 3)) * (unsigned)d.V;
+        *o = delta * (kAccumulate ? *o + v[r] : v[r]);
       }
     } else {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int t = t0 + mfma_row(r, h);
-        float v = __expf(ev[r] - Ms[cur][mfma_row(r, h)]) * acc[r];
-        v = t < Tb ? v : 0.0f;
         if (t < d.T && vok) {
           float* o = out + (size_t)t * d.V + vcol;
-          *o = delta * (kAccumulate ? *o + v : v);
+          *o = delta * (kAccumulate ? *o + v[r] : v[r]);
         }
       }
     }
@@ -207,12 +265,28 @@ __global__ __launch_bounds__(256, 2) void egrads_stream_kernel(
     const float* __restrict__ E, const float* __restrict__ P, const float* __restrict__ mE,
     const float* __restrict__ mP, const float* __restrict__ Wn, const float* __restrict__ deltas,
     float* __restrict__ egrads, const int* __restrict__ inLen, const int* __restrict__ labLen,
-    Dims d, int Up, int Tw, int tiles_per_chunk) {
+    Dims d, int Up, int Tw, int tiles_per_chunk, SparseTerms sp) {
   __shared__ __attribute__((aligned(16))) float As[2][kEsSlab];
   __shared__ __attribute__((aligned(16))) float Ms[2][32];  // mE of the slab's frames
+  __shared__ __attribute__((aligned(16))) float Strip[4][32];  // per wavefront: sparse terms
+  __shared__ unsigned short Match[4][kEsMaxG * 8];  // per wavefront: label positions whose label
+                                                    // is one of its 32 columns
   const int b = blockIdx.z;
   int Tb, Ub;
   utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
+  int nmatch = 0;
+  if (sp.labels) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int col0 = blockIdx.x * 128 + wave * 32;
+    for (int u0 = 0; u0 < Ub - 1; u0 += 64) {
+      const int u = u0 + lane;
+      const int l = (u < Ub - 1) ? sp.labels[(size_t)b * (d.U - 1) + u] : -1;
+      const bool hit = l >= col0 && l < col0 + 32 && l != d.blank;
+      const unsigned long long m = __ballot(hit);
+      if (hit) Match[wave][nmatch + __popcll(m & ((1ull << lane) - 1))] = (unsigned short)u;
+      nmatch += __popcll(m);
+    }
+  }
   // columns of the slab past Up are never staged; clear them once so that a walk that rounds
   // its group count up multiplies zeros there, not whatever the LDS held
   for (int e = threadIdx.x; e < 2 * kEsSlab; e += 256) (&As[0][0])[e] = 0.0f;
@@ -220,7 +294,8 @@ __global__ __launch_bounds__(256, 2) void egrads_stream_kernel(
   const int ngroups = (Ub + 7) >> 3;
 #define RNNT_EG_WALK(NG)                                                                      \
   egrads_walk<NG, kAccumulate>(E, P, mE, mP, Wn, deltas, egrads, As, Ms, d, Up, Tw,          \
-                               tiles_per_chunk, b, Tb, Ub)
+                               tiles_per_chunk, b, Tb, Ub, sp, Match[threadIdx.x >> 6], nmatch,             \
+                               &Strip[threadIdx.x >> 6])
   if (ngroups <= 4) RNNT_EG_WALK(4);
   else if (ngroups <= 8) RNNT_EG_WALK(8);
   else if (ngroups <= 10) RNNT_EG_WALK(10);
@@ -397,7 +472,10 @@ bool egrads_stream_supported(const Dims& d) { return wplane_up(d.U) <= 8 * kEsMa
 
 int launch_egrads_stream(const float* E, const float* P, const float* mE, const float* mP,
                          const float* Wn, const float* deltas, float* egrads, const int* inLen,
-                         const int* labLen, const Dims& d, bool accumulate, hipStream_t s) {
+                         const int* labLen, const Dims& d, bool accumulate,
+                         const SparseTerms& sparse, hipStream_t s) {
+  if (sparse.labels && accumulate)
+    return fail(kInvalid, "sparse-term folding and accumulation are mutually exclusive");
   const int Up = wplane_up(d.U), Tw = wplane_tw(d.T);
   const int vtiles = (d.V + 127) / 128, ntiles = (d.T + 31) / 32;
   // enough workgroups to fill 256 CUs two deep several times over, but long enough runs of
@@ -410,10 +488,10 @@ int launch_egrads_stream(const float* E, const float* P, const float* mE, const 
   chunks = (ntiles + per - 1) / per;
   if (accumulate)
     hipLaunchKernelGGL(egrads_stream_kernel<true>, dim3(vtiles, chunks, d.B), dim3(256), 0, s, E,
-                       P, mE, mP, Wn, deltas, egrads, inLen, labLen, d, Up, Tw, per);
+                       P, mE, mP, Wn, deltas, egrads, inLen, labLen, d, Up, Tw, per, sparse);
   else
     hipLaunchKernelGGL(egrads_stream_kernel<false>, dim3(vtiles, chunks, d.B), dim3(256), 0, s, E,
-                       P, mE, mP, Wn, deltas, egrads, inLen, labLen, d, Up, Tw, per);
+                       P, mE, mP, Wn, deltas, egrads, inLen, labLen, d, Up, Tw, per, sparse);
   RNNT_LAUNCH_CHECK("egrads_stream_kernel");
   return kOk;
 }

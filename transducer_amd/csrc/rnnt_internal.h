@@ -111,6 +111,12 @@ int launch_beta(const Planes& p, const int* labels, const int* inLen, const int*
 int launch_sparse(const Planes& p, float* egrads, float* pgrads, const int* labels,
                   const int* inLen, const int* labLen, const float* scale, bool add,
                   const Dims& d, hipStream_t s);
+// bsum[b,t] = what the sparse terms leave in egrads[b,t,blank] (see blank_sums_kernel).
+int launch_blank_sums(const Planes& p, float* bsum, const int* labels, const int* inLen,
+                      const int* labLen, const Dims& d, hipStream_t s);
+int launch_sparse_p(const Planes& p, float* pgrads, const int* labels, const int* inLen,
+                    const int* labLen, const float* scale, bool add, const Dims& d,
+                    hipStream_t s);
 int launch_maxplus(const float* E, const float* P, const int* inLen, const int* labLen,
                    float* best, int* arg, const Dims& d, hipStream_t s);
 // bestS / argS: skewed planes of the max-plus table (argS carries int bits in float storage).
@@ -131,11 +137,22 @@ int launch_lse(const float* E, const float* P, const float* mE, const float* mP,
 int launch_wplanes(const float* lngrads, const float* LN, const float* mE, const float* mP,
                    float* Wn, float* Wt, const int* inLen, const int* labLen, const Dims& d,
                    hipStream_t s);
+// Sparse blank/label terms of egrads for folding into the dense kernel's write-out: with
+// labels != nullptr, out = delta * (dense + sparse) (needs accumulate == false and a label axis
+// short enough for the streaming kernel, see egrads_fusion_supported).
+struct SparseTerms {
+  const float* dS = nullptr;    // skewed dalpha plane
+  const float* wE = nullptr;    // skewed label-move weight plane
+  const float* bsum = nullptr;  // [B,T] blank-column totals
+  const int* labels = nullptr;  // [B,U-1]
+};
+bool egrads_fusion_supported(const Dims& d);
 // accumulate == false: out = delta * dense.   accumulate == true: out = delta * (out + dense),
 // the update of transducer/torch_binding.py:86-89.
 int launch_egrads(const float* E, const float* P, const float* mE, const float* mP,
                   const float* Wn, const float* deltas, float* egrads, const int* inLen,
-                  const int* labLen, const Dims& d, bool accumulate, hipStream_t s);
+                  const int* labLen, const Dims& d, bool accumulate, const SparseTerms& sparse,
+                  hipStream_t s);
 int launch_pgrads(const float* E, const float* P, const float* mE, const float* mP,
                   const float* Wt, const float* deltas, float* pgrads, const int* inLen,
                   const int* labLen, const Dims& d, bool accumulate, hipStream_t s);
@@ -145,7 +162,8 @@ int launch_pgrads(const float* E, const float* P, const float* mE, const float* 
 bool egrads_stream_supported(const Dims& d);
 int launch_egrads_stream(const float* E, const float* P, const float* mE, const float* mP,
                          const float* Wn, const float* deltas, float* egrads, const int* inLen,
-                         const int* labLen, const Dims& d, bool accumulate, hipStream_t s);
+                         const int* labLen, const Dims& d, bool accumulate,
+                         const SparseTerms& sparse, hipStream_t s);
 int launch_pgrads_stream(const float* E, const float* P, const float* mE, const float* mP,
                          const float* Wt, const float* deltas, float* pgrads, const int* inLen,
                          const int* labLen, const Dims& d, bool accumulate, hipStream_t s);
