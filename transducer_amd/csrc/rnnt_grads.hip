@@ -17,12 +17,12 @@
 // operands agree: a lane takes four consecutive k of its W row with one 16-byte LDS read
 // (k = 8j + 4*(lane/32) + q) and pairs them with the four matching register values.
 #include "rnnt_internal.h"
+#include "rnnt_split.h"
 
 namespace rnnt {
 
 namespace {
 
-typedef float floatx16 __attribute__((ext_vector_type(16)));
 constexpr float kNegInf = -__builtin_huge_valf();
 
 __device__ inline float f4at(const float4& v, int q) {
@@ -307,23 +307,26 @@ __global__ __launch_bounds__(256, 2) void egrads_stream_kernel(
 }
 
 // ------------------------------------------------------------------ pgrads
-constexpr int kPsKP = 32 + 4;  // LDS row pitch of the W^T slab (floats)
+// W^T slab in LDS: three bf16 planes of 128 rows (u) x 32 frames, row pitch 40 halfwords (80 B:
+// the 16-byte fragment reads of 8 consecutive rows fall into distinct bank groups).
+constexpr int kPsPitch = 40;
+constexpr int kPsPlane = 128 * kPsPitch;
 
 // One workgroup's 128 x 128 tile with NMB 32-row blocks of label positions in use (a template
-// parameter, so the matrix instructions of a slice form one straight-line block).
+// parameter, so the matrix instructions of a slice form one straight-line block).  Products are
+// formed on the bf16 matrix cores from exact three-way splits of both operands (rnnt_split.h).
 template <int NMB, bool kAccumulate>
 __device__ __forceinline__ void pgrads_tile(
     const float* __restrict__ E, const float* __restrict__ P, const float* __restrict__ mE,
     const float* __restrict__ mP, const float* __restrict__ Wt, const float* __restrict__ deltas,
-    float* __restrict__ pgrads, float (*As)[128 * kPsKP], float (*Ms)[32], const Dims& d, int Up,
-    int Tw, int b, int u0, int Tb, int Ub) {
+    float* __restrict__ pgrads, unsigned short (*As)[3][kPsPlane], float (*Ms)[32], const Dims& d,
+    int Up, int Tw, int b, int u0, int Tb, int Ub) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, h = lane >> 5;
   const int vcol = blockIdx.x * 128 + wave * 32 + l32;
   const bool vok = vcol < d.V;
   const int vc = vok ? vcol : d.V - 1;
   const float delta = deltas ? deltas[b] : 1.0f;
   float* out = pgrads + (size_t)b * d.U * d.V;
-  constexpr int nmb = NMB;
 
   floatx16 acc[NMB > 0 ? NMB : 1];
 #pragma unroll
@@ -331,17 +334,17 @@ __device__ __forceinline__ void pgrads_tile(
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[mb][r] = 0.0f;
 
-  if (nmb > 0) {
+  if (NMB > 0) {
     const float* Eb = E + (size_t)b * d.T * d.V;
     const float* mEb = mE + (size_t)b * d.T;
     // W^T slab staging: 128 rows (u) x 32 frames = 1024 float4, four per thread; rows past the
     // padded label axis re-read its last row (their blocks are never multiplied)
-    const int arow = tid >> 3, ac4 = tid & 7;  // rows arow + 32*i
+    const int arow = tid >> 3, ac4 = tid & 7;  // rows arow + 32*i, frames 4*ac4 .. +3
     const float* asrc[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i)
       asrc[i] = Wt + ((size_t)b * Up + min(u0 + arow + 32 * i, Up - 1)) * Tw + 4 * ac4;
-    struct XRegs { float v[4][4]; };
+    struct XRegs { float v[2][8]; };
     auto fetch_slab = [&](int k0) -> SlabRegs {
       SlabRegs s;
       s.v0 = *reinterpret_cast<const float4*>(asrc[0] + k0);
@@ -351,23 +354,30 @@ __device__ __forceinline__ void pgrads_tile(
       s.m = mEb[min(k0 + (tid & 31), Tb - 1)];
       return s;
     };
+    // frames this lane feeds to the matrix instruction of k-step s: k0 + 16 s + 8 h + i
     auto fetch_x = [&](int k0) -> XRegs {
       XRegs x;
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
+      for (int s = 0; s < 2; ++s)
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int t = min(k0 + 8 * j + 4 * h + q, Tb - 1);
-          x.v[j][q] = Eb[(size_t)t * d.V + vc];
+        for (int i = 0; i < 8; ++i) {
+          const int t = min(k0 + 16 * s + 8 * h + i, Tb - 1);
+          x.v[s][i] = Eb[(size_t)t * d.V + vc];
         }
       return x;
     };
     auto store_slab = [&](int buf, const SlabRegs& s) {
-      float* dst = &As[buf][arow * kPsKP + 4 * ac4];
-      *reinterpret_cast<float4*>(dst) = s.v0;
-      *reinterpret_cast<float4*>(dst + 32 * kPsKP) = s.v1;
-      *reinterpret_cast<float4*>(dst + 64 * kPsKP) = s.v2;
-      *reinterpret_cast<float4*>(dst + 96 * kPsKP) = s.v3;
+      const float4 v[4] = {s.v0, s.v1, s.v2, s.v3};
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        uint2 ph, pm, pl;
+        split_pair(v[i].x, v[i].y, ph.x, pm.x, pl.x);
+        split_pair(v[i].z, v[i].w, ph.y, pm.y, pl.y);
+        const int o = (arow + 32 * i) * kPsPitch + 4 * ac4;
+        *reinterpret_cast<uint2*>(&As[buf][0][o]) = ph;
+        *reinterpret_cast<uint2*>(&As[buf][1][o]) = pm;
+        *reinterpret_cast<uint2*>(&As[buf][2][o]) = pl;
+      }
       if (tid < 32) Ms[buf][tid] = s.m;
     };
 
@@ -377,16 +387,21 @@ __device__ __forceinline__ void pgrads_tile(
     __syncthreads();
     int cur = 0;
     for (int kt = 0; kt < nk; ++kt) {
-      // X = exp(E - mE) for this slab, zero past the utterance (W is zero there as well)
-      float x[4][4];
+      // X = exp(E - mE) for this slab, zero past the utterance (W is zero there as well),
+      // split into its three pieces in the instruction's operand layout
+      Frag3 xb[2];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const float4 m4 = *reinterpret_cast<const float4*>(&Ms[cur][8 * j + 4 * h]);
+      for (int s = 0; s < 2; ++s) {
+        const float4 ma = *reinterpret_cast<const float4*>(&Ms[cur][16 * s + 8 * h]);
+        const float4 mb4 = *reinterpret_cast<const float4*>(&Ms[cur][16 * s + 8 * h + 4]);
+        float x[8];
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const float e = __expf(xr.v[j][q] - f4at(m4, q));
-          x[j][q] = (kt * 32 + 8 * j + 4 * h + q < Tb && vok) ? e : 0.0f;
+        for (int i = 0; i < 8; ++i) {
+          const float m = i < 4 ? f4at(ma, i) : f4at(mb4, i - 4);
+          const float e = __expf(xr.v[s][i] - m);
+          x[i] = (kt * 32 + 16 * s + 8 * h + i < Tb && vok) ? e : 0.0f;
         }
+        xb[s] = split8(x);
       }
       const bool has_next = kt + 1 < nk;
       SlabRegs nxt;
@@ -394,24 +409,31 @@ __device__ __forceinline__ void pgrads_tile(
         nxt = fetch_slab((kt + 1) * 32);
         xr = fetch_x((kt + 1) * 32);
       }
-      const float* abase = &As[cur][l32 * kPsKP + 4 * h];
-      __builtin_amdgcn_sched_barrier(0);
-      __builtin_amdgcn_s_setprio(2);
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        float4 a4[NMB > 0 ? NMB : 1];
+      for (int s = 0; s < 2; ++s) {
+        uint4 ah[NMB > 0 ? NMB : 1], am[NMB > 0 ? NMB : 1], al[NMB > 0 ? NMB : 1];
 #pragma unroll
-        for (int mb = 0; mb < NMB; ++mb)
-          a4[mb] = *reinterpret_cast<const float4*>(abase + 32 * mb * kPsKP + 8 * j);
+        for (int mb = 0; mb < NMB; ++mb) {
+          const int o = (32 * mb + l32) * kPsPitch + 16 * s + 8 * h;
+          ah[mb] = *reinterpret_cast<const uint4*>(&As[cur][0][o]);
+          am[mb] = *reinterpret_cast<const uint4*>(&As[cur][1][o]);
+          al[mb] = *reinterpret_cast<const uint4*>(&As[cur][2][o]);
+        }
+        // six piece products per block, smallest first; blocks interleaved so that consecutive
+        // instructions never wait on each other's accumulator
 #pragma unroll
-        for (int q = 0; q < 4; ++q)
+        for (int mb = 0; mb < NMB; ++mb) acc[mb] = mfma_bf16(al[mb], xb[s].h, acc[mb]);
 #pragma unroll
-          for (int mb = 0; mb < NMB; ++mb)
-            acc[mb] = __builtin_amdgcn_mfma_f32_32x32x2f32(f4at(a4[mb], q), x[j][q], acc[mb], 0,
-                                                            0, 0);
+        for (int mb = 0; mb < NMB; ++mb) acc[mb] = mfma_bf16(ah[mb], xb[s].l, acc[mb]);
+#pragma unroll
+        for (int mb = 0; mb < NMB; ++mb) acc[mb] = mfma_bf16(am[mb], xb[s].m, acc[mb]);
+#pragma unroll
+        for (int mb = 0; mb < NMB; ++mb) acc[mb] = mfma_bf16(am[mb], xb[s].h, acc[mb]);
+#pragma unroll
+        for (int mb = 0; mb < NMB; ++mb) acc[mb] = mfma_bf16(ah[mb], xb[s].m, acc[mb]);
+#pragma unroll
+        for (int mb = 0; mb < NMB; ++mb) acc[mb] = mfma_bf16(ah[mb], xb[s].h, acc[mb]);
       }
-      __builtin_amdgcn_s_setprio(0);
-      __builtin_amdgcn_sched_barrier(0);
       if (has_next) store_slab(cur ^ 1, nxt);
       __syncthreads();
       cur ^= 1;
@@ -441,7 +463,7 @@ __global__ __launch_bounds__(256, 2) void pgrads_stream_kernel(
     const float* __restrict__ mP, const float* __restrict__ Wt, const float* __restrict__ deltas,
     float* __restrict__ pgrads, const int* __restrict__ inLen, const int* __restrict__ labLen,
     Dims d, int Up, int Tw) {
-  __shared__ __attribute__((aligned(16))) float As[2][128 * kPsKP];
+  __shared__ __attribute__((aligned(16))) unsigned short As[2][3][kPsPlane];
   __shared__ __attribute__((aligned(16))) float Ms[2][32];
   const int b = blockIdx.z, u0 = blockIdx.y * 128;
   int Tb, Ub;
