@@ -31,11 +31,11 @@ namespace prof {
 
 enum Stage {
   kRowmax, kLse, kSkew, kGather, kAlpha, kUnskew, kWeights, kBeta, kWplanes, kEgrads, kPgrads,
-  kSparse, kMaxplus, kViterbi, kClear, kNumStages
+  kSparse, kMaxplus, kViterbi, kClear, kYplanes, kNumStages
 };
 const char* const kNames[kNumStages] = {"rowmax", "lse", "skew", "gather", "alpha", "unskew",
                                         "weights", "beta", "wplanes", "egrads", "pgrads",
-                                        "sparse", "maxplus", "viterbi", "clear"};
+                                        "sparse", "maxplus", "viterbi", "clear", "yplanes"};
 constexpr int kMaxRecords = 8192;
 struct Record { int stage; hipEvent_t begin, end; };
 
@@ -113,9 +113,26 @@ int check_dims(int B, int T, int U, int V) {
 
 bool nothing_to_do(int B, int T, int U) { return B == 0 || T == 0 || U == 0; }
 
+// Row maxima of both score arrays, then the log-normaliser: the streaming kernel when the
+// shape allows it and `scratch` (lse_scratch_bytes) is given, else the general one.
+int log_norms_stages(const float* E, const float* P, float* mE, float* mP, float* LN,
+                     void* scratch, const int* inLen, const int* labLen, const Dims& d,
+                     hipStream_t s) {
+  RNNT_STAGE(kRowmax, launch_rowmax(E, mE, (long)d.B * d.T, d.V, d.T, inLen, 0, s));
+  RNNT_STAGE(kRowmax, launch_rowmax(P, mP, (long)d.B * d.U, d.V, d.U, labLen, 1, s));
+  if (scratch && lse_stream_supported(E, d)) {
+    RNNT_STAGE(kYplanes, launch_yplanes(P, mP, scratch, labLen, d, s));
+    RNNT_STAGE(kLse, launch_lse_stream(E, mE, mP, LN, scratch, inLen, labLen, d, s));
+  } else {
+    RNNT_STAGE(kLse, launch_lse(E, P, mE, mP, LN, inLen, labLen, d, s));
+  }
+  return kOk;
+}
+
 struct LossWorkspace {
   Planes planes;
   float *mE, *mP, *LN, *lngrads, *Wn, *Wt, *bsum;
+  void* lse_scratch;
 };
 
 size_t loss_workspace_layout(const Dims& d, void* base, LossWorkspace* w) {
@@ -138,8 +155,10 @@ size_t loss_workspace_layout(const Dims& d, void* base, LossWorkspace* w) {
   float* Wn = take(wb);
   float* Wt = take(wb);
   float* bsum = take(sizeof(float) * (size_t)d.B * d.T);
+  void* ys = take(lse_scratch_bytes(d));  // forward only
   if (base) {
     w->mE = mE; w->mP = mP; w->LN = LN; w->lngrads = lng; w->Wn = Wn; w->Wt = Wt; w->bsum = bsum;
+    w->lse_scratch = lse_scratch_bytes(d) ? ys : nullptr;
   }
   return off;
 }
@@ -288,14 +307,13 @@ int rnnt_hip_log_norms(const float* E, const float* P, float* LN, const int* inL
   hipStream_t s = static_cast<hipStream_t>(stream);
   const Dims d = make_dims(B, T, U, V, 0);
   Scratch scratch(s);
+  const size_t yb = lse_stream_supported(E, d) ? lse_scratch_bytes(d) : 0;
   RNNT_TRY(scratch.reserve(align_up(sizeof(float) * (size_t)B * T) +
-                           align_up(sizeof(float) * (size_t)B * U)));
+                           align_up(sizeof(float) * (size_t)B * U) + align_up(yb)));
   float* mE = static_cast<float*>(scratch.take(sizeof(float) * (size_t)B * T));
   float* mP = static_cast<float*>(scratch.take(sizeof(float) * (size_t)B * U));
-  RNNT_STAGE(kRowmax, launch_rowmax(E, mE, (long)B * T, V, T, inLen, 0, s));
-  RNNT_STAGE(kRowmax, launch_rowmax(P, mP, (long)B * U, V, U, labLen, 1, s));
-  RNNT_STAGE(kLse, launch_lse(E, P, mE, mP, LN, inLen, labLen, d, s));
-  return kOk;
+  void* ys = yb ? scratch.take(yb) : nullptr;
+  return log_norms_stages(E, P, mE, mP, LN, ys, inLen, labLen, d, s);
 }
 
 int rnnt_hip_dense_grads(const float* E, const float* P, float* egrads, float* pgrads,
@@ -349,9 +367,7 @@ int rnnt_hip_loss_forward(const float* E, const float* P, const int* labels, con
   const Dims d = make_dims(B, T, U, V, blank);
   LossWorkspace w;
   loss_workspace_layout(d, workspace, &w);
-  RNNT_STAGE(kRowmax, launch_rowmax(E, w.mE, (long)B * T, V, T, inLen, 0, s));
-  RNNT_STAGE(kRowmax, launch_rowmax(P, w.mP, (long)B * U, V, U, labLen, 1, s));
-  RNNT_STAGE(kLse, launch_lse(E, P, w.mE, w.mP, w.LN, inLen, labLen, d, s));
+  RNNT_TRY(log_norms_stages(E, P, w.mE, w.mP, w.LN, w.lse_scratch, inLen, labLen, d, s));
   RNNT_STAGE(kSkew, launch_skew(w.LN, w.planes.lnS, inLen, labLen, d, s));
   RNNT_STAGE(kGather, launch_gather(E, P, labels, inLen, labLen, w.planes, d, s));
   RNNT_STAGE(kAlpha, launch_alpha(w.planes, inLen, labLen, costs, d, s));
@@ -415,14 +431,15 @@ int rnnt_hip_viterbi_decode(const float* E, const float* P, const int* inLen, co
   const Dims d = make_dims(B, T, U, V, blank);
   Scratch scratch(s);
   const size_t btu = sizeof(float) * (size_t)B * T * U;
+  const size_t yb = lse_stream_supported(E, d) ? lse_scratch_bytes(d) : 0;
   RNNT_TRY(scratch.reserve(align_up(sizeof(float) * (size_t)B * T) +
-                           align_up(sizeof(float) * (size_t)B * U) + align_up(btu)));
+                           align_up(sizeof(float) * (size_t)B * U) + align_up(btu) +
+                           align_up(yb)));
   float* mE = static_cast<float*>(scratch.take(sizeof(float) * (size_t)B * T));
   float* mP = static_cast<float*>(scratch.take(sizeof(float) * (size_t)B * U));
   float* LN = static_cast<float*>(scratch.take(btu));
-  RNNT_STAGE(kRowmax, launch_rowmax(E, mE, (long)B * T, V, T, inLen, 0, s));
-  RNNT_STAGE(kRowmax, launch_rowmax(P, mP, (long)B * U, V, U, labLen, 1, s));
-  RNNT_STAGE(kLse, launch_lse(E, P, mE, mP, LN, inLen, labLen, d, s));
+  void* ys = yb ? scratch.take(yb) : nullptr;
+  RNNT_TRY(log_norms_stages(E, P, mE, mP, LN, ys, inLen, labLen, d, s));
   return viterbi_impl(E, P, LN, labels, inLen, labLen, d, s);
 }
 

@@ -199,181 +199,6 @@ __global__ __launch_bounds__(256, 2) void lse_kernel(const float* __restrict__ E
       }
 }
 
-// ------------------------------------------------------------------ log-normaliser, fast form
-// Same contraction for V % 4 == 0 and 16-byte aligned inputs (the usual case):
-//  * 16-byte global loads (a thread stages 16 consecutive v of one E row and one P row),
-//    double-buffered LDS, one barrier per slice of 32;
-//  * a wavefront owns 32 frames x all label positions of the tile, so 32-wide label blocks
-//    past the utterance's own length are skipped by every wavefront alike;
-//  * the running sum is flushed into a second accumulator every kLseFlush slices, which keeps
-//    the fp32 summation error near sqrt(flush length) + sqrt(number of flushes) ulp instead of
-//    sqrt(V) and stops small terms from being swamped by an early large one;
-//  * workgroups are renumbered so that all frame tiles of one utterance run on the same XCD
-//    (workgroup ids are dealt round-robin to the 8 XCDs) and share its L2 copy of P[b].
-constexpr int kLseFlush = 16;
-
-struct LseStage {
-  float4 a0, a1, a2, a3, b0, b1, b2, b3;
-};
-
-// One 128 x (32*NNB) tile: the whole reduction over v and the write-out.  NNB is a template
-// parameter so that the matrix instructions of a slice form one straight-line block.
-template <int NNB>
-__device__ __forceinline__ void lse_tile(const float* __restrict__ E, const float* __restrict__ P,
-                                         const float* __restrict__ mE,
-                                         const float* __restrict__ mP, float* __restrict__ LNb,
-                                         float* As0, float* Bs0, const Dims& d, int b, int t0,
-                                         int u0, int Tb, int Ub) {
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, h = lane >> 5;
-  constexpr int kBuf = kLseBM * kLsePitch;
-  // staging: thread -> row tid/2 of both operands, 16 consecutive v starting at 16*(tid%2)
-  const int srow = tid >> 1, skh = (tid & 1) * 16;
-  const int ta = min(t0 + srow, Tb - 1), ub = min(u0 + srow, Ub - 1);
-  const float* pa = E + ((size_t)b * d.T + ta) * d.V + skh;
-  const float* pb = P + ((size_t)b * d.U + ub) * d.V + skh;
-  const float ma = mE[(size_t)b * d.T + ta], mb = mP[(size_t)b * d.U + ub];
-  const bool need_b = (srow >> 5) < NNB;  // uniform per wavefront
-  const int soff = srow * kLsePitch + skh;
-
-  // Loads only: nothing may touch the loaded registers before the matrix block of the current
-  // slice has been issued, or the wavefront would sit out the memory latency first.  A group
-  // of four past the end of the row (V % 4 == 0: never partly) re-reads the row start and is
-  // zeroed when it is staged.
-  auto ld4 = [&](const float* base, int k0, int i) -> float4 {
-    const int v = k0 + skh + 4 * i;
-    return *reinterpret_cast<const float4*>(base + (v < d.V ? k0 + 4 * i : 0));
-  };
-  auto fetch = [&](int k0) -> LseStage {
-    LseStage r;
-    r.a0 = ld4(pa, k0, 0); r.a1 = ld4(pa, k0, 1); r.a2 = ld4(pa, k0, 2); r.a3 = ld4(pa, k0, 3);
-    if (need_b) {
-      r.b0 = ld4(pb, k0, 0); r.b1 = ld4(pb, k0, 1); r.b2 = ld4(pb, k0, 2); r.b3 = ld4(pb, k0, 3);
-    }
-    return r;
-  };
-  auto ex4 = [&](const float4& x, float m, int k0, int i) -> float4 {
-    const bool in = k0 + skh + 4 * i < d.V;
-    const float4 e = make_float4(__expf(x.x - m), __expf(x.y - m), __expf(x.z - m), __expf(x.w - m));
-    return in ? e : make_float4(0.f, 0.f, 0.f, 0.f);
-  };
-  auto stash = [&](int buf, const LseStage& r, int k0) {
-    float* da = As0 + buf * kBuf + soff;
-    *reinterpret_cast<float4*>(da) = ex4(r.a0, ma, k0, 0);
-    *reinterpret_cast<float4*>(da + 4) = ex4(r.a1, ma, k0, 1);
-    *reinterpret_cast<float4*>(da + 8) = ex4(r.a2, ma, k0, 2);
-    *reinterpret_cast<float4*>(da + 12) = ex4(r.a3, ma, k0, 3);
-    if (need_b) {
-      float* db = Bs0 + buf * kBuf + soff;
-      *reinterpret_cast<float4*>(db) = ex4(r.b0, mb, k0, 0);
-      *reinterpret_cast<float4*>(db + 4) = ex4(r.b1, mb, k0, 1);
-      *reinterpret_cast<float4*>(db + 8) = ex4(r.b2, mb, k0, 2);
-      *reinterpret_cast<float4*>(db + 12) = ex4(r.b3, mb, k0, 3);
-    }
-  };
-
-  floatx16 acc[NNB], tot[NNB];
-#pragma unroll
-  for (int nb = 0; nb < NNB; ++nb)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) { acc[nb][r] = 0.0f; tot[nb][r] = 0.0f; }
-
-  const int nk = (d.V + kLseBK - 1) / kLseBK;
-  stash(0, fetch(0), 0);
-  __syncthreads();
-  int cur = 0;
-  for (int kt = 0; kt < nk; ++kt) {
-    const bool has_next = kt + 1 < nk;
-    LseStage nxt;
-    if (has_next) nxt = fetch((kt + 1) * kLseBK);
-    __builtin_amdgcn_sched_barrier(0);
-    __builtin_amdgcn_s_setprio(2);  // matrix phase: take the pipe from a wavefront that is staging
-    const float* arow = As0 + cur * kBuf + (32 * wave + l32) * kLsePitch + 4 * h;
-    const float* brow = Bs0 + cur * kBuf + l32 * kLsePitch + 4 * h;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const float4 a4 = *reinterpret_cast<const float4*>(arow + 8 * j);
-      float4 b4[NNB];
-#pragma unroll
-      for (int nb = 0; nb < NNB; ++nb)
-        b4[nb] = *reinterpret_cast<const float4*>(brow + 32 * nb * kLsePitch + 8 * j);
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const float av = q == 0 ? a4.x : (q == 1 ? a4.y : (q == 2 ? a4.z : a4.w));
-#pragma unroll
-        for (int nb = 0; nb < NNB; ++nb) {
-          const float bv = q == 0 ? b4[nb].x : (q == 1 ? b4[nb].y : (q == 2 ? b4[nb].z : b4[nb].w));
-          acc[nb] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc[nb], 0, 0, 0);
-        }
-      }
-    }
-    __builtin_amdgcn_s_setprio(0);
-    __builtin_amdgcn_sched_barrier(0);
-    if ((kt + 1) % kLseFlush == 0) {
-#pragma unroll
-      for (int nb = 0; nb < NNB; ++nb)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) { tot[nb][r] += acc[nb][r]; acc[nb][r] = 0.0f; }
-    }
-    if (has_next) stash(cur ^ 1, nxt, (kt + 1) * kLseBK);
-    __syncthreads();
-    cur ^= 1;
-  }
-
-  const float* mEb = mE + (size_t)b * d.T;
-  const float* mPb = mP + (size_t)b * d.U;
-#pragma unroll
-  for (int nb = 0; nb < 4; ++nb)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int t = t0 + 32 * wave + 8 * (r >> 2) + 4 * h + (r & 3);
-      const int u = u0 + 32 * nb + l32;
-      if (t < d.T && u < d.U) {
-        float v = 0.0f;
-        if (nb < NNB) {
-          const int nbc = nb < NNB ? nb : 0;
-          if (t < Tb && u < Ub) v = (logf(tot[nbc][r] + acc[nbc][r]) + mEb[t]) + mPb[u];
-        }
-        LNb[(size_t)t * d.U + u] = v;
-      }
-    }
-}
-
-__global__ __launch_bounds__(256, 2) void lse_fast_kernel(const float* __restrict__ E,
-                                                          const float* __restrict__ P,
-                                                          const float* __restrict__ mE,
-                                                          const float* __restrict__ mP,
-                                                          float* __restrict__ LN,
-                                                          const int* __restrict__ inLen,
-                                                          const int* __restrict__ labLen, Dims d,
-                                                          int ttiles, int utiles, int total) {
-  __shared__ __attribute__((aligned(16))) float As[2 * kLseBM * kLsePitch];
-  __shared__ __attribute__((aligned(16))) float Bs[2 * kLseBN * kLsePitch];
-  // XCD-aware renumbering: physical id n runs on XCD n % 8
-  const int n = blockIdx.x, per_xcd = gridDim.x >> 3;
-  const int logical = (n & 7) * per_xcd + (n >> 3);
-  if (logical >= total) return;
-  const int b = logical / (ttiles * utiles);
-  const int rem = logical - b * (ttiles * utiles);
-  const int t0 = (rem % ttiles) * kLseBM, u0 = (rem / ttiles) * kLseBN;
-  int Tb, Ub;
-  utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
-  float* LNb = LN + (size_t)b * d.T * d.U;
-
-  if (t0 >= Tb || u0 >= Ub) {
-    for (int e = threadIdx.x; e < kLseBM * kLseBN; e += 256) {
-      const int t = t0 + e / kLseBN, u = u0 + e % kLseBN;
-      if (t < d.T && u < d.U) LNb[(size_t)t * d.U + u] = 0.0f;
-    }
-    return;
-  }
-  switch (min(4, (Ub - u0 + 31) >> 5)) {  // 32-wide label blocks in use
-    case 1: lse_tile<1>(E, P, mE, mP, LNb, As, Bs, d, b, t0, u0, Tb, Ub); break;
-    case 2: lse_tile<2>(E, P, mE, mP, LNb, As, Bs, d, b, t0, u0, Tb, Ub); break;
-    case 3: lse_tile<3>(E, P, mE, mP, LNb, As, Bs, d, b, t0, u0, Tb, Ub); break;
-    default: lse_tile<4>(E, P, mE, mP, LNb, As, Bs, d, b, t0, u0, Tb, Ub); break;
-  }
-}
-
 // ------------------------------------------------------------------ W planes
 // W[t,u] = dalpha[t,u] / sum_v(...) = dalpha[t,u] * exp((mE[t] + mP[u]) - LN[t,u]), written
 // twice: Wn[b][t][Up] (u contiguous, feeds the egrads contraction) and Wt[b][u][Tw]
@@ -515,18 +340,6 @@ int launch_rowmax(const float* X, float* rowmax, long rows, int V, int rows_per_
 int launch_lse(const float* E, const float* P, const float* mE, const float* mP, float* LN,
                const int* inLen, const int* labLen, const Dims& d, hipStream_t s) {
   if (d.B == 0 || d.T == 0 || d.U == 0) return kOk;
-  const bool aligned = ((reinterpret_cast<uintptr_t>(E) | reinterpret_cast<uintptr_t>(P)) & 15) == 0;
-  if (d.V % 4 == 0 && aligned) {
-    const int ttiles = (d.T + kLseBM - 1) / kLseBM, utiles = (d.U + kLseBN - 1) / kLseBN;
-    const long total = (long)ttiles * utiles * d.B;
-    if (total < (1l << 30)) {
-      const int grid = (int)((total + 7) / 8 * 8);
-      hipLaunchKernelGGL(lse_fast_kernel, dim3(grid), dim3(256), 0, s, E, P, mE, mP, LN, inLen,
-                         labLen, d, ttiles, utiles, (int)total);
-      RNNT_LAUNCH_CHECK("lse_fast_kernel");
-      return kOk;
-    }
-  }
   hipLaunchKernelGGL(lse_kernel,
                      dim3((d.T + kLseBM - 1) / kLseBM, (d.U + kLseBN - 1) / kLseBN, d.B),
                      dim3(256), 0, s, E, P, mE, mP, LN, inLen, labLen, d);

@@ -1,5 +1,6 @@
 // Streaming forms of the two dense-gradient contractions (transducer/torch_binding.py:85-89)
-// for gfx950.  Both keep the vocabulary-side operand of v_mfma_f32_32x32x2_f32 in REGISTERS,
+// for gfx950.  Products are formed on the bf16 matrix cores from exact three-way splits of the
+// fp32 operands (rnnt_split.h).  Both kernels keep the vocabulary-side operand in REGISTERS,
 // read straight from global memory in the instruction's own lane order (32 consecutive v per
 // half-wave = one 128-byte line), and pass only the small W operand through LDS:
 //
@@ -13,9 +14,8 @@
 //       a wavefront owns 32 columns v and all (up to 128) label positions; it walks the frames
 //       32 at a time, turning the 32 x 32 slab of E it just loaded into X in registers.
 //
-// Which reduction element sits in which k-slot of the instruction is free as long as both
-// operands agree: a lane takes four consecutive k of its W row with one 16-byte LDS read
-// (k = 8j + 4*(lane/32) + q) and pairs them with the four matching register values.
+// v_mfma_f32_32x32x16_bf16 takes, per lane, eight consecutive k of its row (A) or column (B):
+// k = 8*(lane/32) + i.  A lane reads them with one 16-byte LDS load per piece.
 #include "rnnt_internal.h"
 #include "rnnt_split.h"
 
@@ -30,9 +30,10 @@ __device__ inline float f4at(const float4& v, int q) {
 }
 
 // ------------------------------------------------------------------ egrads
-constexpr int kEsMaxG = 14;              // groups of 8 label positions kept in registers
-constexpr int kEsKP = 8 * kEsMaxG + 4;   // LDS row pitch of the W slab (floats)
-constexpr int kEsSlab = 32 * kEsKP;
+constexpr int kEsMaxS = 7;               // steps of 16 label positions kept in registers
+constexpr int kEsPitch = 16 * kEsMaxS + 8;  // LDS row pitch of a W-slab plane in halfwords (240 B:
+                                            // 16-byte reads of 8 consecutive rows spread over all banks)
+constexpr int kEsPlane = 32 * kEsPitch;
 constexpr int kEsPrefetch = 2;          // labels per 32-column block whose sparse terms are prefetched
 
 // Row of the 32x32 output block that register r of lane-half h holds.
@@ -43,16 +44,16 @@ struct SlabRegs {
   float m;
 };
 
-// The walk of one workgroup over its frame tiles with NG groups of eight label positions
+// The walk of one workgroup over its frame tiles with NS steps of sixteen label positions
 // (a template parameter, so the matrix instructions of a tile form one straight-line block).
 // Label positions past the utterance contribute exact zeros: their Y rows are masked and the
 // W slab is zero there.
-template <int NG, bool kAccumulate>
+template <int NS, bool kAccumulate>
 __device__ __forceinline__ void egrads_walk(
     const float* __restrict__ E, const float* __restrict__ P, const float* __restrict__ mE,
     const float* __restrict__ mP, const float* __restrict__ Wn, const float* __restrict__ deltas,
-    float* __restrict__ egrads, float (*As)[kEsSlab], float (*Ms)[32], const Dims& d, int Up,
-    int Tw, int tiles_per_chunk, int b, int Tb, int Ub, const SparseTerms& sp,
+    float* __restrict__ egrads, unsigned short (*As)[3][kEsPlane], float (*Ms)[32], const Dims& d,
+    int Up, int Tw, int tiles_per_chunk, int b, int Tb, int Ub, const SparseTerms& sp,
     const unsigned short* match, int nmatch, float (*Sp)[32]) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, h = lane >> 5;
   const int wave_col0 = blockIdx.x * 128 + wave * 32;  // this wavefront's 32 columns
@@ -72,24 +73,29 @@ __device__ __forceinline__ void egrads_walk(
   float* out = egrads + (size_t)b * d.T * d.V;
   const float* mEb = mE + (size_t)b * d.T;
 
-  // Y fragments for this wavefront's columns (branch-free: clamped address, masked value)
-  float Yr[NG][4];
+  // Y fragments for this wavefront's columns (branch-free: clamped address, masked value):
+  // step s holds label positions 16 s + 8 h + i, split into their three bf16 pieces
+  Frag3 Yf[NS];
   if (tile_lo < tile_valid) {
     const float* Pb = P + (size_t)b * d.U * d.V;
     const float* mPb = mP + (size_t)b * d.U;
 #pragma unroll
-    for (int j = 0; j < NG; ++j)
+    for (int s = 0; s < NS; ++s) {
+      float y[8];
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int u = 8 * j + 4 * h + q;
+      for (int i = 0; i < 8; ++i) {
+        const int u = 16 * s + 8 * h + i;
         const bool uok = u < Ub;
         const int uc = uok ? u : 0;
-        const float y = __expf(Pb[(size_t)uc * d.V + vc] - mPb[uc]);
-        Yr[j][q] = (uok && vok) ? y : 0.0f;
+        const float e = __expf(Pb[(size_t)uc * d.V + vc] - mPb[uc]);
+        y[i] = (uok && vok) ? e : 0.0f;
       }
+      Yf[s] = split8(y);
+    }
   }
 
-  // W slab staging: the 32 x Up slab of frame tile ti is one contiguous run of 8*Up float4
+  // W slab staging: the 32 x Up slab of frame tile ti is one contiguous run of 8*Up float4;
+  // each is split into its three pieces on the way into LDS
   const int up4 = Up >> 2, nvec = 8 * Up;
   int lds_off[4], src_idx[4];
   bool vec_ok[4];
@@ -98,7 +104,7 @@ __device__ __forceinline__ void egrads_walk(
     const int idx = tid + 256 * i;
     vec_ok[i] = idx < nvec;
     src_idx[i] = vec_ok[i] ? idx : nvec - 1;  // loads stay unconditional, stores are masked
-    lds_off[i] = vec_ok[i] ? (idx / up4) * kEsKP + 4 * (idx % up4) : 0;
+    lds_off[i] = vec_ok[i] ? (idx / up4) * kEsPitch + 4 * (idx % up4) : 0;
   }
   auto fetch_slab = [&](int ti) -> SlabRegs {
     const float4* src =
@@ -112,10 +118,18 @@ __device__ __forceinline__ void egrads_walk(
     return s;
   };
   auto store_slab = [&](int buf, const SlabRegs& s) {
-    if (vec_ok[0]) *reinterpret_cast<float4*>(&As[buf][lds_off[0]]) = s.v0;
-    if (vec_ok[1]) *reinterpret_cast<float4*>(&As[buf][lds_off[1]]) = s.v1;
-    if (vec_ok[2]) *reinterpret_cast<float4*>(&As[buf][lds_off[2]]) = s.v2;
-    if (vec_ok[3]) *reinterpret_cast<float4*>(&As[buf][lds_off[3]]) = s.v3;
+    const float4 v[4] = {s.v0, s.v1, s.v2, s.v3};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      uint2 ph, pm, pl;
+      split_pair(v[i].x, v[i].y, ph.x, pm.x, pl.x);
+      split_pair(v[i].z, v[i].w, ph.y, pm.y, pl.y);
+      if (vec_ok[i]) {
+        *reinterpret_cast<uint2*>(&As[buf][0][lds_off[i]]) = ph;
+        *reinterpret_cast<uint2*>(&As[buf][1][lds_off[i]]) = pm;
+        *reinterpret_cast<uint2*>(&As[buf][2][lds_off[i]]) = pl;
+      }
+    }
     if (tid < 32) Ms[buf][tid] = s.m;
   };
 
@@ -136,9 +150,8 @@ __device__ __forceinline__ void egrads_walk(
 
   for (int ti = tile_lo; ti < tile_valid; ++ti) {
     const int t0 = ti * 32;
-    const bool has_next = ti + 1 < tile_valid;
-    SlabRegs nxt;
-    if (has_next) nxt = fetch_slab(ti + 1);
+    // the next slab, requested now (the last tile re-reads its own: no branch around the loads)
+    const SlabRegs nxt = fetch_slab(min(ti + 1, tile_valid - 1));
     const bool interior = cols_full && (t0 + 32 <= Tb);  // no row or column needs a guard
     const float* Etile = Eb + (size_t)t0 * d.V;
     float* Otile = out + (size_t)t0 * d.V;
@@ -167,24 +180,32 @@ __device__ __forceinline__ void egrads_walk(
       }
       if (blank_lane >= 0) sbl = sp.bsum[(size_t)b * d.T + tr];
     }
-    floatx16 acc;
+    // two accumulators, so that consecutive matrix instructions never wait on each other
+    floatx16 acc, acc2;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
+    for (int r = 0; r < 16; ++r) acc[r] = acc2[r] = 0.0f;
     __builtin_amdgcn_sched_barrier(0);
-    __builtin_amdgcn_s_setprio(2);  // matrix phase first; the other wavefronts' epilogues fill in
-    const float* arow = &As[cur][l32 * kEsKP + 4 * h];
-    float4 a4[NG];
+    {
+      const unsigned short* arow = &As[cur][0][l32 * kEsPitch + 8 * h];
+      uint4 ah[NS], am[NS], al[NS];
 #pragma unroll
-    for (int j = 0; j < NG; ++j) a4[j] = *reinterpret_cast<const float4*>(arow + 8 * j);
+      for (int s = 0; s < NS; ++s) {
+        ah[s] = *reinterpret_cast<const uint4*>(arow + 16 * s);
+        am[s] = *reinterpret_cast<const uint4*>(arow + kEsPlane + 16 * s);
+        al[s] = *reinterpret_cast<const uint4*>(arow + 2 * kEsPlane + 16 * s);
+      }
 #pragma unroll
-    for (int j = 0; j < NG; ++j) {
-      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a4[j].x, Yr[j][0], acc, 0, 0, 0);
-      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a4[j].y, Yr[j][1], acc, 0, 0, 0);
-      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a4[j].z, Yr[j][2], acc, 0, 0, 0);
-      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a4[j].w, Yr[j][3], acc, 0, 0, 0);
+      for (int s = 0; s < NS; ++s) {
+        acc = mfma_bf16(al[s], Yf[s].h, acc);
+        acc2 = mfma_bf16(ah[s], Yf[s].l, acc2);
+        acc = mfma_bf16(am[s], Yf[s].m, acc);
+        acc2 = mfma_bf16(am[s], Yf[s].h, acc2);
+        acc = mfma_bf16(ah[s], Yf[s].m, acc);
+        acc2 = mfma_bf16(ah[s], Yf[s].h, acc2);
+      }
     }
-    __builtin_amdgcn_s_setprio(0);
-    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] += acc2[r];
     float v[16];
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
@@ -242,7 +263,7 @@ __device__ __forceinline__ void egrads_walk(
         }
       }
     }
-    if (has_next) store_slab(cur ^ 1, nxt);
+    store_slab(cur ^ 1, nxt);
     __syncthreads();
     cur ^= 1;
   }
@@ -266,10 +287,10 @@ __global__ __launch_bounds__(256, 2) void egrads_stream_kernel(
     const float* __restrict__ mP, const float* __restrict__ Wn, const float* __restrict__ deltas,
     float* __restrict__ egrads, const int* __restrict__ inLen, const int* __restrict__ labLen,
     Dims d, int Up, int Tw, int tiles_per_chunk, SparseTerms sp) {
-  __shared__ __attribute__((aligned(16))) float As[2][kEsSlab];
+  __shared__ __attribute__((aligned(16))) unsigned short As[2][3][kEsPlane];
   __shared__ __attribute__((aligned(16))) float Ms[2][32];  // mE of the slab's frames
   __shared__ __attribute__((aligned(16))) float Strip[4][32];  // per wavefront: sparse terms
-  __shared__ unsigned short Match[4][kEsMaxG * 8];  // per wavefront: label positions whose label
+  __shared__ unsigned short Match[4][kEsMaxS * 16];  // per wavefront: label positions whose label
                                                     // is one of its 32 columns
   const int b = blockIdx.z;
   int Tb, Ub;
@@ -288,21 +309,20 @@ __global__ __launch_bounds__(256, 2) void egrads_stream_kernel(
     }
   }
   // columns of the slab past Up are never staged; clear them once so that a walk that rounds
-  // its group count up multiplies zeros there, not whatever the LDS held
-  for (int e = threadIdx.x; e < 2 * kEsSlab; e += 256) (&As[0][0])[e] = 0.0f;
+  // its step count up multiplies zeros there, not whatever the LDS held
+  for (int e = threadIdx.x; e < 3 * kEsPlane; e += 256)
+    reinterpret_cast<unsigned*>(&As[0][0][0])[e] = 0u;
   __syncthreads();
-  const int ngroups = (Ub + 7) >> 3;
-#define RNNT_EG_WALK(NG)                                                                      \
-  egrads_walk<NG, kAccumulate>(E, P, mE, mP, Wn, deltas, egrads, As, Ms, d, Up, Tw,          \
+  const int nsteps = (Ub + 15) >> 4;
+#define RNNT_EG_WALK(NS)                                                                      \
+  egrads_walk<NS, kAccumulate>(E, P, mE, mP, Wn, deltas, egrads, As, Ms, d, Up, Tw,          \
                                tiles_per_chunk, b, Tb, Ub, sp, Match[threadIdx.x >> 6], nmatch,             \
                                &Strip[threadIdx.x >> 6])
-  if (ngroups <= 4) RNNT_EG_WALK(4);
-  else if (ngroups <= 8) RNNT_EG_WALK(8);
-  else if (ngroups <= 10) RNNT_EG_WALK(10);
-  else if (ngroups == 11) RNNT_EG_WALK(11);
-  else if (ngroups == 12) RNNT_EG_WALK(12);
-  else if (ngroups == 13) RNNT_EG_WALK(13);
-  else RNNT_EG_WALK(14);
+  if (nsteps <= 2) RNNT_EG_WALK(2);
+  else if (nsteps <= 4) RNNT_EG_WALK(4);
+  else if (nsteps == 5) RNNT_EG_WALK(5);
+  else if (nsteps == 6) RNNT_EG_WALK(6);
+  else RNNT_EG_WALK(7);
 #undef RNNT_EG_WALK
 }
 
@@ -387,8 +407,9 @@ __device__ __forceinline__ void pgrads_tile(
     __syncthreads();
     int cur = 0;
     for (int kt = 0; kt < nk; ++kt) {
-      // X = exp(E - mE) for this slab, zero past the utterance (W is zero there as well),
-      // split into its three pieces in the instruction's operand layout
+      // X = exp(E - mE) for this slab (finite everywhere; W^T is zero past the utterance and
+      // columns past V are dropped on the way out), split into its three pieces in the
+      // instruction's operand layout
       Frag3 xb[2];
 #pragma unroll
       for (int s = 0; s < 2; ++s) {
@@ -398,17 +419,14 @@ __device__ __forceinline__ void pgrads_tile(
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
           const float m = i < 4 ? f4at(ma, i) : f4at(mb4, i - 4);
-          const float e = __expf(xr.v[s][i] - m);
-          x[i] = (kt * 32 + 16 * s + 8 * h + i < Tb && vok) ? e : 0.0f;
+          x[i] = __expf(xr.v[s][i] - m);  // frames past the utterance repeat its last one
         }
         xb[s] = split8(x);
       }
-      const bool has_next = kt + 1 < nk;
-      SlabRegs nxt;
-      if (has_next) {
-        nxt = fetch_slab((kt + 1) * 32);
-        xr = fetch_x((kt + 1) * 32);
-      }
+      // the next slab, requested now (the last step re-reads its own: no branch around the loads)
+      const int knext = min(kt + 1, nk - 1) * 32;
+      const SlabRegs nxt = fetch_slab(knext);
+      xr = fetch_x(knext);
 #pragma unroll
       for (int s = 0; s < 2; ++s) {
         uint4 ah[NMB > 0 ? NMB : 1], am[NMB > 0 ? NMB : 1], al[NMB > 0 ? NMB : 1];
@@ -434,7 +452,7 @@ __device__ __forceinline__ void pgrads_tile(
 #pragma unroll
         for (int mb = 0; mb < NMB; ++mb) acc[mb] = mfma_bf16(ah[mb], xb[s].h, acc[mb]);
       }
-      if (has_next) store_slab(cur ^ 1, nxt);
+      store_slab(cur ^ 1, nxt);
       __syncthreads();
       cur ^= 1;
     }
@@ -490,7 +508,7 @@ __global__ __launch_bounds__(256, 2) void pgrads_stream_kernel(
     if (_e != hipSuccess) return check_hip(_e, "launch " name, __FILE__, __LINE__); \
   } while (0)
 
-bool egrads_stream_supported(const Dims& d) { return wplane_up(d.U) <= 8 * kEsMaxG; }
+bool egrads_stream_supported(const Dims& d) { return wplane_up(d.U) <= 16 * kEsMaxS; }
 
 int launch_egrads_stream(const float* E, const float* P, const float* mE, const float* mP,
                          const float* Wn, const float* deltas, float* egrads, const int* inLen,

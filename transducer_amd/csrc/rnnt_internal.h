@@ -132,8 +132,18 @@ int wplane_tw(int T);  // frame-axis pitch of the W planes (multiple of 64)
 // their item (rows_per_item rows each) are not read and report 0.
 int launch_rowmax(const float* X, float* rowmax, long rows, int V, int rows_per_item,
                   const int* lengths, int extra, hipStream_t s);
+// Log-normaliser, general form (any V and alignment; fp32 matrix instructions).
 int launch_lse(const float* E, const float* P, const float* mE, const float* mP, float* LN,
                const int* inLen, const int* labLen, const Dims& d, hipStream_t s);
+// Log-normaliser, streaming form (rnnt_lse.hip): V % 4 == 0 and 16-byte aligned E.  The pieces of
+// exp(P - mP) are first written to `scratch` (lse_scratch_bytes) in matrix-operand order.
+bool lse_stream_supported(const float* E, const Dims& d);
+size_t lse_scratch_bytes(const Dims& d);
+int launch_yplanes(const float* P, const float* mP, void* scratch, const int* labLen,
+                   const Dims& d, hipStream_t s);
+int launch_lse_stream(const float* E, const float* mE, const float* mP, float* LN,
+                      const void* scratch, const int* inLen, const int* labLen, const Dims& d,
+                      hipStream_t s);
 int launch_wplanes(const float* lngrads, const float* LN, const float* mE, const float* mP,
                    float* Wn, float* Wt, const int* inLen, const int* labLen, const Dims& d,
                    hipStream_t s);

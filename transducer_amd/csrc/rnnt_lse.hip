@@ -1,0 +1,291 @@
+// Log-normaliser LN[t,u] = log sum_v exp(E[t,v] + P[u,v])  (transducer/torch_binding.py:35-40,
+// transducer/test.h:51-80) for gfx950, streaming form on the bf16 matrix cores.
+//
+// With row maxima mE[t], mP[u] taken out, the sum is the contraction  sum_v X[t,v] * Y[u,v],
+// X = exp(E - mE), Y = exp(P - mP), both in (0, 1].  Each fp32 factor is split exactly into three
+// bf16 pieces and six piece products are accumulated in fp32 (rnnt_split.h), which keeps fp32
+// accuracy at 3/8 of the fp32 matrix-instruction time and leaves the vector ALUs to the exps.
+//
+//  * Y is small (B*U*V) and used by every frame tile, so it is prepared ONCE: yplanes_kernel
+//    writes its three pieces in the matrix instruction's own operand order
+//        [b][block of 32 u][step of 16 v][piece][lane 0..63][8 x bf16]
+//    and the contraction reads a fragment with one perfectly coalesced 16-byte load per lane,
+//    no LDS and no arithmetic.  Steps past V hold zeros, which also takes care of the tail of
+//    the reduction: X only has to be finite there.
+//  * X is large (B*T*V) and used once: a workgroup turns a 128 x 32 slab of E into the three
+//    pieces on its way into LDS (16-byte slots, XOR-swizzled so that the 16-byte fragment reads
+//    of eight consecutive rows and the staging writes both spread over all banks).
+//  * A wavefront owns one block of 32 label positions and all 128 frames of the tile: four
+//    accumulators, 24 matrix instructions per step of 16 v.
+//  * Workgroups are renumbered so that all frame tiles of one utterance run on the same XCD
+//    (workgroup ids are dealt round-robin to the 8 XCDs) and share its L2 copy of Y[b].
+#include "rnnt_internal.h"
+#include "rnnt_split.h"
+
+namespace rnnt {
+
+namespace {
+
+constexpr int kRows = 128;    // frames per workgroup tile
+constexpr int kSlice = 32;    // v per LDS slab (two matrix-instruction steps)
+constexpr int kSlots = kRows * 4;  // 16-byte slots per piece plane: 4 per row
+
+__device__ inline int mfma_row(int r, int h) { return 8 * (r >> 2) + 4 * h + (r & 3); }
+
+// 16-byte slot of (row, c8 = which eight of the slab's 32 v) inside a piece plane
+__device__ inline int xslot(int row, int c8) { return row * 4 + (c8 ^ ((row >> 1) & 3)); }
+
+inline int y_ublocks(const Dims& d) { return (d.U + 31) / 32; }
+inline int y_steps(const Dims& d) { return 2 * ((d.V + kSlice - 1) / kSlice); }
+
+// ------------------------------------------------------------------ Y pieces
+// One thread per (u, eight consecutive v).  vec4 = V % 4 == 0 and P 16-byte aligned.
+__global__ __launch_bounds__(256) void yplanes_kernel(const float* __restrict__ P,
+                                                      const float* __restrict__ mP,
+                                                      uint4* __restrict__ Yp,
+                                                      const int* __restrict__ labLen, Dims d,
+                                                      int nub, int nks, int vec4) {
+  const int b = blockIdx.z, ub = blockIdx.y, ks = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (ks >= nks) return;
+  const int lane = threadIdx.x & 63, l32 = lane & 31, h = lane >> 5;
+  int Ub = d.U;
+  if (labLen) Ub = min(max(labLen[b], 0) + 1, d.U);
+  const int u = 32 * ub + l32, v0 = 16 * ks + 8 * h;
+  float y[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) y[i] = 0.0f;
+  if (u < Ub) {
+    const float* row = P + ((size_t)b * d.U + u) * d.V;
+    const float m = mP[(size_t)b * d.U + u];
+    if (vec4) {
+      if (v0 < d.V) {
+        const float4 p = *reinterpret_cast<const float4*>(row + v0);
+        y[0] = __expf(p.x - m); y[1] = __expf(p.y - m); y[2] = __expf(p.z - m); y[3] = __expf(p.w - m);
+      }
+      if (v0 + 4 < d.V) {
+        const float4 p = *reinterpret_cast<const float4*>(row + v0 + 4);
+        y[4] = __expf(p.x - m); y[5] = __expf(p.y - m); y[6] = __expf(p.z - m); y[7] = __expf(p.w - m);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        if (v0 + i < d.V) y[i] = __expf(row[v0 + i] - m);
+    }
+  }
+  const Frag3 f = split8(y);
+  uint4* dst = Yp + (((size_t)b * nub + ub) * nks + ks) * 3 * 64 + lane;
+  dst[0] = f.h;
+  dst[64] = f.m;
+  dst[128] = f.l;
+}
+
+// ------------------------------------------------------------------ contraction
+struct XRegs {
+  float4 a0, a1, b0, b1;  // rows srow and srow + 64: eight consecutive v each
+};
+
+__global__ __launch_bounds__(256, 2) void lse_stream_kernel(
+    const float* __restrict__ E, const float* __restrict__ mE, const float* __restrict__ mP,
+    const uint4* __restrict__ Yp, float* __restrict__ LN, const int* __restrict__ inLen,
+    const int* __restrict__ labLen, Dims d, int ttiles, int utiles, int total, int nub, int nks) {
+  __shared__ uint4 Xs[2][3][kSlots];
+  // XCD-aware renumbering: physical id n runs on XCD n % 8
+  const int n = blockIdx.x, per_xcd = gridDim.x >> 3;
+  const int logical = (n & 7) * per_xcd + (n >> 3);
+  if (logical >= total) return;
+  const int b = logical / (ttiles * utiles);
+  const int rem = logical - b * (ttiles * utiles);
+  const int t0 = (rem % ttiles) * kRows, u0 = (rem / ttiles) * 128;
+  int Tb, Ub;
+  utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
+  float* LNb = LN + (size_t)b * d.T * d.U;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, h = lane >> 5;
+
+  if (t0 >= Tb || u0 >= Ub) {
+    for (int e = tid; e < kRows * 128; e += 256) {
+      const int t = t0 + e / 128, u = u0 + e % 128;
+      if (t < d.T && u < d.U) LNb[(size_t)t * d.U + u] = 0.0f;
+    }
+    return;
+  }
+
+  // staging: thread -> rows srow and srow + 64 of the tile, v = slab start + 8*c8 .. +7.
+  // Rows past the utterance repeat its last frame, groups of four past V repeat the row's last
+  // group (V % 4 == 0): finite values that meet zeros in Y or are dropped on the way out.
+  const int srow = tid >> 2, c8 = tid & 3;
+  const int ta = min(t0 + srow, Tb - 1), tb = min(t0 + srow + 64, Tb - 1);
+  const float* pa = E + ((size_t)b * d.T + ta) * d.V;
+  const float* pb = E + ((size_t)b * d.T + tb) * d.V;
+  const float ma = mE[(size_t)b * d.T + ta], mb = mE[(size_t)b * d.T + tb];
+  const int slot_a = xslot(srow, c8), slot_b = xslot(srow + 64, c8);
+  auto fetch = [&](int k0) -> XRegs {
+    const int v0 = min(k0 + 8 * c8, d.V - 4), v1 = min(k0 + 8 * c8 + 4, d.V - 4);
+    XRegs r;
+    r.a0 = *reinterpret_cast<const float4*>(pa + v0);
+    r.a1 = *reinterpret_cast<const float4*>(pa + v1);
+    r.b0 = *reinterpret_cast<const float4*>(pb + v0);
+    r.b1 = *reinterpret_cast<const float4*>(pb + v1);
+    return r;
+  };
+  auto stash = [&](int buf, const XRegs& r) {
+    const float xa[8] = {__expf(r.a0.x - ma), __expf(r.a0.y - ma), __expf(r.a0.z - ma),
+                         __expf(r.a0.w - ma), __expf(r.a1.x - ma), __expf(r.a1.y - ma),
+                         __expf(r.a1.z - ma), __expf(r.a1.w - ma)};
+    const Frag3 fa = split8(xa);
+    Xs[buf][0][slot_a] = fa.h;
+    Xs[buf][1][slot_a] = fa.m;
+    Xs[buf][2][slot_a] = fa.l;
+    const float xb[8] = {__expf(r.b0.x - mb), __expf(r.b0.y - mb), __expf(r.b0.z - mb),
+                         __expf(r.b0.w - mb), __expf(r.b1.x - mb), __expf(r.b1.y - mb),
+                         __expf(r.b1.z - mb), __expf(r.b1.w - mb)};
+    const Frag3 fb = split8(xb);
+    Xs[buf][0][slot_b] = fb.h;
+    Xs[buf][1][slot_b] = fb.m;
+    Xs[buf][2][slot_b] = fb.l;
+  };
+
+  // this wavefront's block of 32 label positions; a block past the utterance only helps staging
+  const int ublock = (u0 >> 5) + wave;
+  const bool active = 32 * ublock < Ub;
+  const uint4* yw = Yp + ((size_t)b * nub + (active ? ublock : 0)) * nks * 3 * 64 + lane;
+  struct YRegs { Frag3 s0, s1; };
+  auto fetch_y = [&](int kt) -> YRegs {
+    const uint4* p = yw + (size_t)kt * 2 * 3 * 64;
+    YRegs y;
+    y.s0.h = p[0]; y.s0.m = p[64]; y.s0.l = p[128];
+    y.s1.h = p[192]; y.s1.m = p[256]; y.s1.l = p[320];
+    return y;
+  };
+
+  floatx16 acc[4];
+#pragma unroll
+  for (int mb4 = 0; mb4 < 4; ++mb4)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[mb4][r] = 0.0f;
+
+  // fragment slots of this lane: row 32*m + l32, v-eights 2*s + h
+  int aslot[2][4];
+#pragma unroll
+  for (int s = 0; s < 2; ++s)
+#pragma unroll
+    for (int m = 0; m < 4; ++m) aslot[s][m] = xslot(32 * m + l32, 2 * s + h);
+
+  const int nk = (d.V + kSlice - 1) / kSlice;
+  int cur = 0;
+  // One slab: request the next slab and Y fragments (the last slice re-reads its own: no branch
+  // around the loads), multiply the current ones, stage the next.  Called with the two Y
+  // register sets swapped on alternate slices, so no set is ever copied.
+  auto slice = [&](int kt, const YRegs& yc, YRegs& yn) {
+    const int ktn = min(kt + 1, nk - 1);
+    const XRegs nxt = fetch(ktn * kSlice);
+    if (active) {
+      yn = fetch_y(ktn);
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        const Frag3& y = s == 0 ? yc.s0 : yc.s1;
+        uint4 ah[4], am[4], al[4];
+#pragma unroll
+        for (int m = 0; m < 4; ++m) {
+          ah[m] = Xs[cur][0][aslot[s][m]];
+          am[m] = Xs[cur][1][aslot[s][m]];
+          al[m] = Xs[cur][2][aslot[s][m]];
+        }
+        // six piece products per block, smallest first; blocks interleaved so that consecutive
+        // instructions never wait on each other's accumulator
+#pragma unroll
+        for (int m = 0; m < 4; ++m) acc[m] = mfma_bf16(al[m], y.h, acc[m]);
+#pragma unroll
+        for (int m = 0; m < 4; ++m) acc[m] = mfma_bf16(ah[m], y.l, acc[m]);
+#pragma unroll
+        for (int m = 0; m < 4; ++m) acc[m] = mfma_bf16(am[m], y.m, acc[m]);
+#pragma unroll
+        for (int m = 0; m < 4; ++m) acc[m] = mfma_bf16(am[m], y.h, acc[m]);
+#pragma unroll
+        for (int m = 0; m < 4; ++m) acc[m] = mfma_bf16(ah[m], y.m, acc[m]);
+#pragma unroll
+        for (int m = 0; m < 4; ++m) acc[m] = mfma_bf16(ah[m], y.h, acc[m]);
+      }
+    }
+    stash(cur ^ 1, nxt);
+    __syncthreads();
+    cur ^= 1;
+  };
+  stash(0, fetch(0));
+  YRegs y0, y1;
+  if (active) y0 = fetch_y(0);
+  __syncthreads();
+  for (int kt = 0; kt < nk; kt += 2) {
+    slice(kt, y0, y1);
+    if (kt + 1 < nk) slice(kt + 1, y1, y0);
+  }
+
+  if (!active) {
+    // label positions past the utterance (but inside U) are written as zeros
+    const int u = 32 * ublock + l32;
+    if (u < d.U)
+      for (int r = 0; r < 64; ++r) {
+        const int t = t0 + 32 * (r >> 4) + mfma_row(r & 15, h);
+        if (t < d.T) LNb[(size_t)t * d.U + u] = 0.0f;
+      }
+    return;
+  }
+  const float* mEb = mE + (size_t)b * d.T;
+  const int u = 32 * ublock + l32;
+  const float mu = mP[(size_t)b * d.U + min(u, Ub - 1)];
+#pragma unroll
+  for (int m = 0; m < 4; ++m)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int t = t0 + 32 * m + mfma_row(r, h);
+      if (t < d.T && u < d.U) {
+        float v = 0.0f;
+        if (t < Tb && u < Ub) v = (logf(acc[m][r]) + mEb[t]) + mu;
+        LNb[(size_t)t * d.U + u] = v;
+      }
+    }
+}
+
+}  // namespace
+
+#define RNNT_LAUNCH_CHECK(name)                                                    \
+  do {                                                                             \
+    hipError_t _e = hipGetLastError();                                             \
+    if (_e != hipSuccess) return check_hip(_e, "launch " name, __FILE__, __LINE__); \
+  } while (0)
+
+bool lse_stream_supported(const float* E, const Dims& d) {
+  const long total = (long)((d.T + kRows - 1) / kRows) * ((d.U + 127) / 128) * d.B;
+  return d.V % 4 == 0 && d.V >= 4 && (reinterpret_cast<uintptr_t>(E) & 15) == 0 &&
+         total < (1l << 30);
+}
+
+size_t lse_scratch_bytes(const Dims& d) {
+  if (d.B == 0 || d.T == 0 || d.U == 0 || d.V % 4 != 0) return 0;
+  return (size_t)d.B * y_ublocks(d) * y_steps(d) * 3 * 64 * sizeof(uint4);
+}
+
+int launch_yplanes(const float* P, const float* mP, void* scratch, const int* labLen,
+                   const Dims& d, hipStream_t s) {
+  const int nub = y_ublocks(d), nks = y_steps(d);
+  const int vec4 = (reinterpret_cast<uintptr_t>(P) & 15) == 0;
+  hipLaunchKernelGGL(yplanes_kernel, dim3((nks + 3) / 4, nub, d.B), dim3(256), 0, s, P, mP,
+                     static_cast<uint4*>(scratch), labLen, d, nub, nks, vec4);
+  RNNT_LAUNCH_CHECK("yplanes_kernel");
+  return kOk;
+}
+
+int launch_lse_stream(const float* E, const float* mE, const float* mP, float* LN,
+                      const void* scratch, const int* inLen, const int* labLen, const Dims& d,
+                      hipStream_t s) {
+  const int nub = y_ublocks(d), nks = y_steps(d);
+  const int ttiles = (d.T + kRows - 1) / kRows, utiles = (d.U + 127) / 128;
+  const long total = (long)ttiles * utiles * d.B;
+  const int grid = (int)((total + 7) / 8 * 8);
+  hipLaunchKernelGGL(lse_stream_kernel, dim3(grid), dim3(256), 0, s, E, mE, mP,
+                     static_cast<const uint4*>(scratch), LN, inLen, labLen, d, ttiles, utiles,
+                     (int)total, nub, nks);
+  RNNT_LAUNCH_CHECK("lse_stream_kernel");
+  return kOk;
+}
+
+}  // namespace rnnt
