@@ -53,15 +53,20 @@ def test_bad_sizes_are_rejected_before_any_device_work():
     # empty batch: nothing to do, no device needed
     assert lib.rnnt_hip_forward(None, None, None, None, None, None, None, None,
                                 0, 5, 3, 4, 0, None) == 0
-    assert lib.rnnt_hip_loss_workspace_bytes(32, 2000, 101, 10000) < 400 * 2**20
+    # far below one [B,T,V] array (2.56 GB at this shape)
+    assert lib.rnnt_hip_loss_workspace_bytes(32, 2000, 101, 10000) < 600 * 2**20
 
 
-def test_workspace_is_order_BTU_not_BTUV():
+def test_workspace_has_no_BTV_or_BTUV_term():
+    """O(B*T*U) lattice planes plus one O(B*U*V) entry (the pieces of exp(P - mP), 6 bytes per
+    element of predictions with U rounded up to 32): growing V by dV adds exactly that much, for
+    any T."""
     from transducer_amd import capi
     lib = capi.load()
-    small = lib.rnnt_hip_loss_workspace_bytes(8, 2000, 101, 100)
-    large = lib.rnnt_hip_loss_workspace_bytes(8, 2000, 101, 10000)
-    assert small == large
+    f = lib.rnnt_hip_loss_workspace_bytes
+    per_v_short = f(8, 500, 101, 10016) - f(8, 500, 101, 32)
+    per_v_long = f(8, 2000, 101, 10016) - f(8, 2000, 101, 32)
+    assert per_v_short == per_v_long == 8 * 128 * (10016 - 32) * 6
 
 
 def test_pybind_module_has_the_reference_keyword_names():
