@@ -179,7 +179,8 @@ def test_long_label_axis_uses_more_cells_per_lane():
 
 # ------------------------------------------------------------------ log-normaliser
 @pytest.mark.parametrize("B,T,U,V,sigma", [(2, 70, 9, 31, 1.0), (1, 200, 101, 1000, 2.0),
-                                           (3, 129, 130, 257, 1.0), (1, 64, 17, 4099, 3.0)])
+                                           (3, 129, 130, 257, 1.0), (1, 64, 17, 4099, 3.0),
+                                           (1, 64, 17, 4100, 3.0), (2, 150, 40, 10000, 1.0)])
 def test_log_norms_against_fp64(B, T, U, V, sigma):
     cfg = small_config(B, T, U - 1, V, sigma=sigma, ragged=True)
     E, P, labels, il, ll = unpack(make_inputs(cfg, seed=V))

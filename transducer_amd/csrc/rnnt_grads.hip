@@ -331,6 +331,7 @@ __global__ __launch_bounds__(256, 2) void egrads_stream_kernel(
 // the 16-byte fragment reads of 8 consecutive rows fall into distinct bank groups).
 constexpr int kPsPitch = 40;
 constexpr int kPsPlane = 128 * kPsPitch;
+constexpr int kPsFlush = 8;  // slabs of 32 frames between two flushes of the running sums
 
 // One workgroup's 128 x 128 tile with NMB 32-row blocks of label positions in use (a template
 // parameter, so the matrix instructions of a slice form one straight-line block).  Products are
@@ -348,11 +349,14 @@ __device__ __forceinline__ void pgrads_tile(
   const float delta = deltas ? deltas[b] : 1.0f;
   float* out = pgrads + (size_t)b * d.U * d.V;
 
-  floatx16 acc[NMB > 0 ? NMB : 1];
+  // The matrix instruction truncates what falls below its accumulator's last bit, so a long
+  // running sum drifts low; every kPsFlush slabs it is added (vector ALU, round to nearest)
+  // into a second accumulator and restarted.
+  floatx16 acc[NMB > 0 ? NMB : 1], tot[NMB > 0 ? NMB : 1];
 #pragma unroll
   for (int mb = 0; mb < NMB; ++mb)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) acc[mb][r] = 0.0f;
+    for (int r = 0; r < 16; ++r) acc[mb][r] = tot[mb][r] = 0.0f;
 
   if (NMB > 0) {
     const float* Eb = E + (size_t)b * d.T * d.V;
@@ -452,11 +456,21 @@ __device__ __forceinline__ void pgrads_tile(
 #pragma unroll
         for (int mb = 0; mb < NMB; ++mb) acc[mb] = mfma_bf16(ah[mb], xb[s].h, acc[mb]);
       }
+      if ((kt + 1) % kPsFlush == 0) {
+#pragma unroll
+        for (int mb = 0; mb < NMB; ++mb)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) { tot[mb][r] += acc[mb][r]; acc[mb][r] = 0.0f; }
+      }
       store_slab(cur ^ 1, nxt);
       __syncthreads();
       cur ^= 1;
     }
   }
+#pragma unroll
+  for (int mb = 0; mb < NMB; ++mb)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[mb][r] += tot[mb][r];
 
   const float* Pb = P + (size_t)b * d.U * d.V;
   const float* mPb = mP + (size_t)b * d.U;

@@ -17,6 +17,12 @@
 //    of eight consecutive rows and the staging writes both spread over all banks).
 //  * A wavefront owns one block of 32 label positions and all 128 frames of the tile: four
 //    accumulators, 24 matrix instructions per step of 16 v.
+//  * The matrix instruction aligns its products to the accumulator and TRUNCATES what falls
+//    below the accumulator's last bit, so a long running sum drifts low by a fraction of an ulp
+//    per instruction (3750 instructions per output at V = 10000: about 2^-16 relative, measured).
+//    Every kFlush slabs the running sums are therefore added (vector ALU, round to nearest) into
+//    a second set of accumulators and restarted: the truncation then acts on a sum that is
+//    V / (32 kFlush) times smaller.
 //  * Workgroups are renumbered so that all frame tiles of one utterance run on the same XCD
 //    (workgroup ids are dealt round-robin to the 8 XCDs) and share its L2 copy of Y[b].
 #include "rnnt_internal.h"
@@ -29,11 +35,12 @@ namespace {
 constexpr int kRows = 128;    // frames per workgroup tile
 constexpr int kSlice = 32;    // v per LDS slab (two matrix-instruction steps)
 constexpr int kSlots = kRows * 4;  // 16-byte slots per piece plane: 4 per row
+constexpr int kFlush = 8;     // slabs between two flushes of the running sums
 
 __device__ inline int mfma_row(int r, int h) { return 8 * (r >> 2) + 4 * h + (r & 3); }
 
 // 16-byte slot of (row, c8 = which eight of the slab's 32 v) inside a piece plane
-__device__ inline int xslot(int row, int c8) { return row * 4 + (c8 ^ ((row >> 1) & 3)); }
+__device__ inline int xslot(int row, int c8) { return row * 4 + (c8 ^ ((row >> 2) & 3)); }
 
 inline int y_ublocks(const Dims& d) { return (d.U + 31) / 32; }
 inline int y_steps(const Dims& d) { return 2 * ((d.V + kSlice - 1) / kSlice); }
@@ -80,14 +87,17 @@ __global__ __launch_bounds__(256) void yplanes_kernel(const float* __restrict__ 
 }
 
 // ------------------------------------------------------------------ contraction
-struct XRegs {
-  float4 a0, a1, b0, b1;  // rows srow and srow + 64: eight consecutive v each
-};
-
-__global__ __launch_bounds__(256, 2) void lse_stream_kernel(
+// kWaves = 4: a wavefront owns one block of 32 label positions and all 128 frames (four
+// accumulators).  kWaves = 8: two wavefronts share a block, 64 frames each (two accumulators,
+// half the registers, twice the wavefronts to hide each other's staging).
+template <int kWaves>
+__global__ __launch_bounds__(64 * kWaves, kWaves / 2) void lse_stream_kernel(
     const float* __restrict__ E, const float* __restrict__ mE, const float* __restrict__ mP,
     const uint4* __restrict__ Yp, float* __restrict__ LN, const int* __restrict__ inLen,
     const int* __restrict__ labLen, Dims d, int ttiles, int utiles, int total, int nub, int nks) {
+  constexpr int kThreads = 64 * kWaves;
+  constexpr int MB = 16 / kWaves;          // 32-frame blocks per wavefront
+  constexpr int NR = 512 / kThreads;       // (row, eight v) items a thread stages per slab
   __shared__ uint4 Xs[2][3][kSlots];
   // XCD-aware renumbering: physical id n runs on XCD n % 8
   const int n = blockIdx.x, per_xcd = gridDim.x >> 3;
@@ -102,144 +112,168 @@ __global__ __launch_bounds__(256, 2) void lse_stream_kernel(
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, h = lane >> 5;
 
   if (t0 >= Tb || u0 >= Ub) {
-    for (int e = tid; e < kRows * 128; e += 256) {
+    for (int e = tid; e < kRows * 128; e += kThreads) {
       const int t = t0 + e / 128, u = u0 + e % 128;
       if (t < d.T && u < d.U) LNb[(size_t)t * d.U + u] = 0.0f;
     }
     return;
   }
 
-  // staging: thread -> rows srow and srow + 64 of the tile, v = slab start + 8*c8 .. +7.
-  // Rows past the utterance repeat its last frame, groups of four past V repeat the row's last
-  // group (V % 4 == 0): finite values that meet zeros in Y or are dropped on the way out.
+  // staging: thread -> rows srow (+ 64 with four wavefronts) of the tile, v = slab start +
+  // 8*c8 .. +7.  Rows past the utterance repeat its last frame, groups of four past V repeat
+  // the row's last group (V % 4 == 0): finite values that meet zeros in Y or are dropped on
+  // the way out.
   const int srow = tid >> 2, c8 = tid & 3;
-  const int ta = min(t0 + srow, Tb - 1), tb = min(t0 + srow + 64, Tb - 1);
-  const float* pa = E + ((size_t)b * d.T + ta) * d.V;
-  const float* pb = E + ((size_t)b * d.T + tb) * d.V;
-  const float ma = mE[(size_t)b * d.T + ta], mb = mE[(size_t)b * d.T + tb];
-  const int slot_a = xslot(srow, c8), slot_b = xslot(srow + 64, c8);
+  const float* px[NR];
+  float mx[NR];
+  int slot[NR];
+#pragma unroll
+  for (int i = 0; i < NR; ++i) {
+    const int row = srow + (kThreads / 4) * i;
+    const int t = min(t0 + row, Tb - 1);
+    px[i] = E + ((size_t)b * d.T + t) * d.V;
+    mx[i] = mE[(size_t)b * d.T + t];
+    slot[i] = xslot(row, c8);
+  }
+  struct XRegs { float4 lo[NR], hi[NR]; };
   auto fetch = [&](int k0) -> XRegs {
     const int v0 = min(k0 + 8 * c8, d.V - 4), v1 = min(k0 + 8 * c8 + 4, d.V - 4);
     XRegs r;
-    r.a0 = *reinterpret_cast<const float4*>(pa + v0);
-    r.a1 = *reinterpret_cast<const float4*>(pa + v1);
-    r.b0 = *reinterpret_cast<const float4*>(pb + v0);
-    r.b1 = *reinterpret_cast<const float4*>(pb + v1);
+#pragma unroll
+    for (int i = 0; i < NR; ++i) {
+      r.lo[i] = *reinterpret_cast<const float4*>(px[i] + v0);
+      r.hi[i] = *reinterpret_cast<const float4*>(px[i] + v1);
+    }
     return r;
   };
   auto stash = [&](int buf, const XRegs& r) {
-    const float xa[8] = {__expf(r.a0.x - ma), __expf(r.a0.y - ma), __expf(r.a0.z - ma),
-                         __expf(r.a0.w - ma), __expf(r.a1.x - ma), __expf(r.a1.y - ma),
-                         __expf(r.a1.z - ma), __expf(r.a1.w - ma)};
-    const Frag3 fa = split8(xa);
-    Xs[buf][0][slot_a] = fa.h;
-    Xs[buf][1][slot_a] = fa.m;
-    Xs[buf][2][slot_a] = fa.l;
-    const float xb[8] = {__expf(r.b0.x - mb), __expf(r.b0.y - mb), __expf(r.b0.z - mb),
-                         __expf(r.b0.w - mb), __expf(r.b1.x - mb), __expf(r.b1.y - mb),
-                         __expf(r.b1.z - mb), __expf(r.b1.w - mb)};
-    const Frag3 fb = split8(xb);
-    Xs[buf][0][slot_b] = fb.h;
-    Xs[buf][1][slot_b] = fb.m;
-    Xs[buf][2][slot_b] = fb.l;
+#pragma unroll
+    for (int i = 0; i < NR; ++i) {
+      const float m = mx[i];
+      const float x[8] = {__expf(r.lo[i].x - m), __expf(r.lo[i].y - m), __expf(r.lo[i].z - m),
+                          __expf(r.lo[i].w - m), __expf(r.hi[i].x - m), __expf(r.hi[i].y - m),
+                          __expf(r.hi[i].z - m), __expf(r.hi[i].w - m)};
+      const Frag3 f = split8(x);
+      Xs[buf][0][slot[i]] = f.h;
+      Xs[buf][1][slot[i]] = f.m;
+      Xs[buf][2][slot[i]] = f.l;
+    }
   };
 
-  // this wavefront's block of 32 label positions; a block past the utterance only helps staging
-  const int ublock = (u0 >> 5) + wave;
+  // this wavefront's block of 32 label positions and first frame block; a label block past the
+  // utterance only helps staging
+  const int ublock = (u0 >> 5) + (wave & 3);
+  const int mb0 = (wave >> 2) * MB;
   const bool active = 32 * ublock < Ub;
   const uint4* yw = Yp + ((size_t)b * nub + (active ? ublock : 0)) * nks * 3 * 64 + lane;
-  struct YRegs { Frag3 s0, s1; };
-  auto fetch_y = [&](int kt) -> YRegs {
-    const uint4* p = yw + (size_t)kt * 2 * 3 * 64;
-    YRegs y;
-    y.s0.h = p[0]; y.s0.m = p[64]; y.s0.l = p[128];
-    y.s1.h = p[192]; y.s1.m = p[256]; y.s1.l = p[320];
+  // Y fragments of step `ks` (16 v): three coalesced 16-byte loads
+  auto fetch_y = [&](int ks) -> Frag3 {
+    const uint4* p = yw + (size_t)ks * 3 * 64;
+    Frag3 y;
+    y.h = p[0]; y.m = p[64]; y.l = p[128];
     return y;
   };
 
-  floatx16 acc[4];
+  floatx16 acc[MB], tot[MB];
 #pragma unroll
-  for (int mb4 = 0; mb4 < 4; ++mb4)
+  for (int m = 0; m < MB; ++m)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) acc[mb4][r] = 0.0f;
+    for (int r = 0; r < 16; ++r) acc[m][r] = tot[m][r] = 0.0f;
 
-  // fragment slots of this lane: row 32*m + l32, v-eights 2*s + h
-  int aslot[2][4];
+  // fragment slots of this lane: row 32*(mb0 + m) + l32, v-eights 2*s + h
+  int aslot[2][MB];
 #pragma unroll
   for (int s = 0; s < 2; ++s)
 #pragma unroll
-    for (int m = 0; m < 4; ++m) aslot[s][m] = xslot(32 * m + l32, 2 * s + h);
+    for (int m = 0; m < MB; ++m) aslot[s][m] = xslot(32 * (mb0 + m) + l32, 2 * s + h);
 
   const int nk = (d.V + kSlice - 1) / kSlice;
   int cur = 0;
-  // One slab: request the next slab and Y fragments (the last slice re-reads its own: no branch
-  // around the loads), multiply the current ones, stage the next.  Called with the two Y
-  // register sets swapped on alternate slices, so no set is ever copied.
-  auto slice = [&](int kt, const YRegs& yc, YRegs& yn) {
-    const int ktn = min(kt + 1, nk - 1);
-    const XRegs nxt = fetch(ktn * kSlice);
-    if (active) {
-      yn = fetch_y(ktn);
+  // One slab: request the next slab and its two Y fragments (the last slice re-reads its own:
+  // no branch around the loads), multiply the current ones, stage the next.  Called with the
+  // two Y register sets swapped on alternate slabs, so no set is ever copied.
+  struct YRegs { Frag3 s0, s1; };
+  auto step = [&](int s, const Frag3& y) {
+    uint4 ah[MB], am[MB], al[MB];
 #pragma unroll
-      for (int s = 0; s < 2; ++s) {
-        const Frag3& y = s == 0 ? yc.s0 : yc.s1;
-        uint4 ah[4], am[4], al[4];
-#pragma unroll
-        for (int m = 0; m < 4; ++m) {
-          ah[m] = Xs[cur][0][aslot[s][m]];
-          am[m] = Xs[cur][1][aslot[s][m]];
-          al[m] = Xs[cur][2][aslot[s][m]];
-        }
-        // six piece products per block, smallest first; blocks interleaved so that consecutive
-        // instructions never wait on each other's accumulator
-#pragma unroll
-        for (int m = 0; m < 4; ++m) acc[m] = mfma_bf16(al[m], y.h, acc[m]);
-#pragma unroll
-        for (int m = 0; m < 4; ++m) acc[m] = mfma_bf16(ah[m], y.l, acc[m]);
-#pragma unroll
-        for (int m = 0; m < 4; ++m) acc[m] = mfma_bf16(am[m], y.m, acc[m]);
-#pragma unroll
-        for (int m = 0; m < 4; ++m) acc[m] = mfma_bf16(am[m], y.h, acc[m]);
-#pragma unroll
-        for (int m = 0; m < 4; ++m) acc[m] = mfma_bf16(ah[m], y.m, acc[m]);
-#pragma unroll
-        for (int m = 0; m < 4; ++m) acc[m] = mfma_bf16(ah[m], y.h, acc[m]);
-      }
+    for (int m = 0; m < MB; ++m) {
+      ah[m] = Xs[cur][0][aslot[s][m]];
+      am[m] = Xs[cur][1][aslot[s][m]];
+      al[m] = Xs[cur][2][aslot[s][m]];
     }
-    stash(cur ^ 1, nxt);
+    // six piece products per block, smallest first; blocks interleaved so that consecutive
+    // instructions wait on each other's accumulator as little as possible
+#pragma unroll
+    for (int m = 0; m < MB; ++m) acc[m] = mfma_bf16(al[m], y.h, acc[m]);
+#pragma unroll
+    for (int m = 0; m < MB; ++m) acc[m] = mfma_bf16(ah[m], y.l, acc[m]);
+#pragma unroll
+    for (int m = 0; m < MB; ++m) acc[m] = mfma_bf16(am[m], y.m, acc[m]);
+#pragma unroll
+    for (int m = 0; m < MB; ++m) acc[m] = mfma_bf16(am[m], y.h, acc[m]);
+#pragma unroll
+    for (int m = 0; m < MB; ++m) acc[m] = mfma_bf16(ah[m], y.m, acc[m]);
+#pragma unroll
+    for (int m = 0; m < MB; ++m) acc[m] = mfma_bf16(ah[m], y.h, acc[m]);
+  };
+  // E is requested two slabs ahead (HBM latency under load exceeds one slab's matrix work);
+  // the slab requested one call earlier is already in registers, so its exps and splits can be
+  // scheduled among this slab's matrix instructions.
+  auto slab = [&](int kt, const YRegs& yc, YRegs& yn, const XRegs& xs, XRegs& xl) {
+    xl = fetch(min(kt + 2, nk - 1) * kSlice);
+    if (active) {
+      const int ktn = min(kt + 1, nk - 1);
+      yn.s0 = fetch_y(2 * ktn);
+      yn.s1 = fetch_y(2 * ktn + 1);
+    }
+    if (active) {
+      step(0, yc.s0);
+      step(1, yc.s1);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    stash(cur ^ 1, xs);
     __syncthreads();
     cur ^= 1;
   };
   stash(0, fetch(0));
+  XRegs xa = fetch(min(1, nk - 1) * kSlice), xb;
   YRegs y0, y1;
-  if (active) y0 = fetch_y(0);
+  if (active) {
+    y0.s0 = fetch_y(0);
+    y0.s1 = fetch_y(1);
+  }
   __syncthreads();
   for (int kt = 0; kt < nk; kt += 2) {
-    slice(kt, y0, y1);
-    if (kt + 1 < nk) slice(kt + 1, y1, y0);
+    slab(kt, y0, y1, xa, xb);
+    if (kt + 1 < nk) slab(kt + 1, y1, y0, xb, xa);
+    if (active && (kt + 2) % kFlush == 0) {
+#pragma unroll
+      for (int m = 0; m < MB; ++m)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) { tot[m][r] += acc[m][r]; acc[m][r] = 0.0f; }
+    }
   }
 
+  const int u = 32 * ublock + l32;
   if (!active) {
     // label positions past the utterance (but inside U) are written as zeros
-    const int u = 32 * ublock + l32;
     if (u < d.U)
-      for (int r = 0; r < 64; ++r) {
-        const int t = t0 + 32 * (r >> 4) + mfma_row(r & 15, h);
+      for (int r = 0; r < 16 * MB; ++r) {
+        const int t = t0 + 32 * (mb0 + (r >> 4)) + mfma_row(r & 15, h);
         if (t < d.T) LNb[(size_t)t * d.U + u] = 0.0f;
       }
     return;
   }
   const float* mEb = mE + (size_t)b * d.T;
-  const int u = 32 * ublock + l32;
   const float mu = mP[(size_t)b * d.U + min(u, Ub - 1)];
 #pragma unroll
-  for (int m = 0; m < 4; ++m)
+  for (int m = 0; m < MB; ++m)
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-      const int t = t0 + 32 * m + mfma_row(r, h);
+      const int t = t0 + 32 * (mb0 + m) + mfma_row(r, h);
       if (t < d.T && u < d.U) {
         float v = 0.0f;
-        if (t < Tb && u < Ub) v = (logf(acc[m][r]) + mEb[t]) + mu;
+        if (t < Tb && u < Ub) v = (logf(tot[m][r] + acc[m][r]) + mEb[t]) + mu;
         LNb[(size_t)t * d.U + u] = v;
       }
     }
@@ -281,7 +315,8 @@ int launch_lse_stream(const float* E, const float* mE, const float* mP, float* L
   const int ttiles = (d.T + kRows - 1) / kRows, utiles = (d.U + 127) / 128;
   const long total = (long)ttiles * utiles * d.B;
   const int grid = (int)((total + 7) / 8 * 8);
-  hipLaunchKernelGGL(lse_stream_kernel, dim3(grid), dim3(256), 0, s, E, mE, mP,
+  constexpr int kWaves = 4;
+  hipLaunchKernelGGL(lse_stream_kernel<kWaves>, dim3(grid), dim3(64 * kWaves), 0, s, E, mE, mP,
                      static_cast<const uint4*>(scratch), LN, inLen, labLen, d, ttiles, utiles,
                      (int)total, nub, nks);
   RNNT_LAUNCH_CHECK("lse_stream_kernel");
