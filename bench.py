@@ -6,10 +6,14 @@ dense + sparse gradients) on one synthetic batch that is already resident in HBM
 the C interface of librnnt_hip.so.  Prints ONE JSON line:
 
   value / ms_per_step   milliseconds per fwd+bwd at the headline shape (lower is better)
-  roofline              the slowest matrix-core kernel: algorithmic flops of one launch
+  roofline              the slowest matrix-core kernel: algorithmic fp32 flops of one launch
                         (2 * V * sum_b T_b*(U_b+1), valid lattice cells only) over its mean
                         duration, measured with HIP events on the launch stream during the
-                        timed steps, against the 157.3 TFLOP/s fp32 matrix peak
+                        timed steps, against the 157.3 TFLOP/s fp32 matrix peak (the kernels
+                        form each fp32 product from six bf16 matrix products, so this fraction
+                        may pass 1); "hbm" inside it prices the same launch against 8 TB/s with
+                        the bytes the algorithm must move (valid rows of E and P read once,
+                        the kernel's output written once)
   cpu_baseline          the CPU path (the OpenMP restatement in oracle/, which is checked bit for
                         bit against the reference's compiled sources) timed on the host cores
                         over a bounded sample of the same workload and scaled by lattice-cell
@@ -30,6 +34,7 @@ sys.path.insert(0, ROOT)
 
 METRIC = "ms per fwd+bwd RNN-T loss, B=32 T=2000 U=100 V=10000; % of roofline"
 PEAK_FP32_MATRIX_TFLOPS = 157.3
+PEAK_HBM_GBS = 8000.0
 
 WORKLOADS = {
     # BASELINE configs[3]: the shape the metric is quoted on
@@ -182,6 +187,10 @@ def main():
     dom = max(mfma_kernels, key=mfma_kernels.get)
     achieved = flops_one / (mfma_kernels[dom] * 1e-3) / 1e12
     flops_all = 3.0 * flops_one
+    # bytes each contraction must move: valid rows of E and P in, its output out
+    in_bytes = 4.0 * V * (float(il.sum()) + float((ll + 1).sum()))
+    out_bytes = {"lse": 4.0 * B * T * U1, "egrads": 4.0 * B * T * V, "pgrads": 4.0 * B * U1 * V}
+    hbm_gbs = (in_bytes + out_bytes[dom]) / (mfma_kernels[dom] * 1e-3) / 1e9
     out = {
         "metric": METRIC,
         "value": round(ms_per_step, 4),
@@ -208,7 +217,13 @@ def main():
                      "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP32_MATRIX_TFLOPS, 4),
                      "traffic": None,
                      "kernel_ms": round(mfma_kernels[dom], 4),
-                     "flops_per_launch": flops_one},
+                     "flops_per_launch": flops_one,
+                     "hbm": {"achieved": round(hbm_gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                             "frac": round(hbm_gbs / PEAK_HBM_GBS, 4),
+                             "bytes_per_launch": in_bytes + out_bytes[dom]},
+                     "all_kernels_frac_of_fp32_matrix_peak": {
+                         k: round(flops_one / (v * 1e-3) / 1e12 / PEAK_FP32_MATRIX_TFLOPS, 4)
+                         for k, v in mfma_kernels.items()}},
         "whole_step_frac_of_mfma_roofline": round(
             (flops_all / (PEAK_FP32_MATRIX_TFLOPS * 1e12)) / (ms_per_step * 1e-3), 4),
         "stage_ms_per_step": per_step,
