@@ -134,6 +134,10 @@ def main():
     ap.add_argument("--workload", default="cfg4", choices=sorted(WORKLOADS))
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run one plain elementwise copy of the emissions array (B*T*V*4 "
+                         "bytes read, as many written) so that a counter run can scale "
+                         "FETCH_SIZE / WRITE_SIZE by what they read for a known transfer")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures the one-GPU hot path; --gpus %d is not supported "
@@ -166,6 +170,9 @@ def main():
 
     for _ in range(args.warmup):
         step()
+        torch.cuda.synchronize()
+    if args.copy_calibration:
+        torch.mul(E, 1.0, out=egrads)  # vectorized_elementwise_kernel: reads E, writes egrads
         torch.cuda.synchronize()
     capi.profile_enable(True)
     torch.cuda.synchronize()
