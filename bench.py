@@ -35,6 +35,10 @@ sys.path.insert(0, ROOT)
 METRIC = "ms per fwd+bwd RNN-T loss, B=32 T=2000 U=100 V=10000; % of roofline"
 PEAK_FP32_MATRIX_TFLOPS = 157.3
 PEAK_HBM_GBS = 8000.0
+# HBM bytes per launch (fetched + written) from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this
+# file, scaled by what the counters read for a plain copy of known size
+# (profiles/cfg4_hbm_traffic_counters.md).  Recorded, not measured live: counters need rocprofv3.
+RECORDED_TRAFFIC_BYTES = {"cfg4": {"lse": 2.526e9, "egrads": 5.666e9, "pgrads": 3.126e9}}
 
 WORKLOADS = {
     # BASELINE configs[3]: the shape the metric is quoted on
@@ -222,7 +226,7 @@ def main():
                                                  "pgrads": "pgrads_stream_kernel"}[dom],
                      "achieved": round(achieved, 2), "peak": PEAK_FP32_MATRIX_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP32_MATRIX_TFLOPS, 4),
-                     "traffic": None,
+                     "traffic": RECORDED_TRAFFIC_BYTES.get(args.workload, {}).get(dom),
                      "kernel_ms": round(mfma_kernels[dom], 4),
                      "flops_per_launch": flops_one,
                      "hbm": {"achieved": round(hbm_gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
