@@ -115,11 +115,17 @@ bool nothing_to_do(int B, int T, int U) { return B == 0 || T == 0 || U == 0; }
 
 // Row maxima of both score arrays, then the log-normaliser: the streaming kernel when the
 // shape allows it and `scratch` (lse_scratch_bytes) is given, else the general one.
+// With `planes`, the row-maximum pass also extracts the blank / label scores the lattice
+// recursions need (no separate gather).
 int log_norms_stages(const float* E, const float* P, float* mE, float* mP, float* LN,
                      void* scratch, const int* inLen, const int* labLen, const Dims& d,
-                     hipStream_t s) {
-  RNNT_STAGE(kRowmax, launch_rowmax(E, mE, (long)d.B * d.T, d.V, d.T, inLen, 0, s));
-  RNNT_STAGE(kRowmax, launch_rowmax(P, mP, (long)d.B * d.U, d.V, d.U, labLen, 1, s));
+                     hipStream_t s, const Planes* planes = nullptr, const int* labels = nullptr) {
+  if (planes) {
+    RNNT_STAGE(kRowmax, launch_rowmax_pick(E, P, mE, mP, labels, inLen, labLen, *planes, d, s));
+  } else {
+    RNNT_STAGE(kRowmax, launch_rowmax(E, mE, (long)d.B * d.T, d.V, d.T, inLen, 0, s));
+    RNNT_STAGE(kRowmax, launch_rowmax(P, mP, (long)d.B * d.U, d.V, d.U, labLen, 1, s));
+  }
   if (scratch && lse_stream_supported(E, d)) {
     RNNT_STAGE(kYplanes, launch_yplanes(P, mP, scratch, labLen, d, s));
     RNNT_STAGE(kLse, launch_lse_stream(E, mE, mP, LN, scratch, inLen, labLen, d, s));
@@ -367,9 +373,9 @@ int rnnt_hip_loss_forward(const float* E, const float* P, const int* labels, con
   const Dims d = make_dims(B, T, U, V, blank);
   LossWorkspace w;
   loss_workspace_layout(d, workspace, &w);
-  RNNT_TRY(log_norms_stages(E, P, w.mE, w.mP, w.LN, w.lse_scratch, inLen, labLen, d, s));
+  RNNT_TRY(log_norms_stages(E, P, w.mE, w.mP, w.LN, w.lse_scratch, inLen, labLen, d, s,
+                            &w.planes, labels));
   RNNT_STAGE(kSkew, launch_skew(w.LN, w.planes.lnS, inLen, labLen, d, s));
-  RNNT_STAGE(kGather, launch_gather(E, P, labels, inLen, labLen, w.planes, d, s));
   RNNT_STAGE(kAlpha, launch_alpha(w.planes, inLen, labLen, costs, d, s));
   return kOk;
 }

@@ -34,21 +34,8 @@ __device__ inline float wave_max(float m) {
 // One wavefront per row of a [rows, V] array.
 // rows_per_item / lengths (optional): row r belongs to item r / rows_per_item and is skipped
 // (maximum reported as 0, nothing read) when its index inside the item is >= lengths[item] + extra.
-__global__ __launch_bounds__(256) void rowmax_kernel(const float* __restrict__ X,
-                                                     float* __restrict__ out, long rows, int V,
-                                                     int vec4, int rows_per_item,
-                                                     const int* __restrict__ lengths, int extra) {
-  const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
-  const int lane = threadIdx.x & 63;
-  if (row >= rows) return;
-  if (lengths) {
-    const long item = row / rows_per_item;
-    if (row - item * rows_per_item >= lengths[item] + extra) {
-      if (lane == 0) out[row] = 0.0f;
-      return;
-    }
-  }
-  const float* x = X + (size_t)row * V;
+// Maximum of one row, computed by one wavefront (every lane gets the result).
+__device__ inline float row_max(const float* __restrict__ x, int V, int vec4, int lane) {
   float m0 = kNegInf, m1 = kNegInf, m2 = kNegInf, m3 = kNegInf;
   if (vec4) {
     const float4* x4 = reinterpret_cast<const float4*>(x);
@@ -68,8 +55,120 @@ __global__ __launch_bounds__(256) void rowmax_kernel(const float* __restrict__ X
   } else {
     for (int i = lane; i < V; i += 64) m0 = fmaxf(m0, x[i]);
   }
-  const float m = wave_max(fmaxf(fmaxf(m0, m1), fmaxf(m2, m3)));
+  return wave_max(fmaxf(fmaxf(m0, m1), fmaxf(m2, m3)));
+}
+
+__global__ __launch_bounds__(256) void rowmax_kernel(const float* __restrict__ X,
+                                                     float* __restrict__ out, long rows, int V,
+                                                     int vec4, int rows_per_item,
+                                                     const int* __restrict__ lengths, int extra) {
+  const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (row >= rows) return;
+  if (lengths) {
+    const long item = row / rows_per_item;
+    if (row - item * rows_per_item >= lengths[item] + extra) {
+      if (lane == 0) out[row] = 0.0f;
+      return;
+    }
+  }
+  const float m = row_max(X + (size_t)row * V, V, vec4, lane);
   if (lane == 0) out[row] = m;
+}
+
+// Row maxima of the emissions plus the elements of each row that the lattice recursions need:
+// E[t, blank] and E[t, label_u] for every label position, written to the skewed planes (what
+// gather_kernel of rnnt_dp.hip does with one scattered HBM sector per element; here the sectors
+// are part of the row that is being streamed anyway).  A workgroup takes 16 consecutive frames of
+// one utterance, four per wavefront; the picked scores meet in LDS and leave as runs of 16
+// consecutive frames per label position.  Frames past the utterance are skipped.
+constexpr int kPickRows = 16, kPickU = 256;
+
+__global__ __launch_bounds__(256) void rowmax_pick_e_kernel(const float* __restrict__ E,
+                                                            float* __restrict__ mE,
+                                                            const int* __restrict__ labels,
+                                                            const int* __restrict__ inLen,
+                                                            const int* __restrict__ labLen,
+                                                            Planes p, Dims d, int vec4) {
+  __shared__ float tile[kPickRows][kPickU + 1];
+  __shared__ float blanks[kPickRows];
+  const int b = blockIdx.y, t0 = blockIdx.x * kPickRows;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int Tb, Ub;
+  utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
+  const int nlab = labels ? max(Ub - 1, 0) : 0;
+  // label columns of this lane (first kPickU label positions)
+  int col[kPickU / 64];
+#pragma unroll
+  for (int i = 0; i < kPickU / 64; ++i) {
+    const int u = lane + 64 * i;
+    col[i] = u < nlab ? labels[(size_t)b * (d.U - 1) + u] : d.blank;
+  }
+  // The picks of a frame are requested right after its row has been streamed (they hit L2) and
+  // are put away after the NEXT row's stream, so their latency is never waited for.
+  float pick[kPickU / 64], xb = 0.0f;
+  int pending = -1;  // tile row the registers belong to
+  auto put_away = [&]() {
+    if (pending < 0) return;
+#pragma unroll
+    for (int k = 0; k < kPickU / 64; ++k) tile[pending][lane + 64 * k] = pick[k];
+    if (lane == 0) blanks[pending] = xb;
+    pending = -1;
+  };
+  for (int r = 0; r < 4; ++r) {
+    const int i = 4 * wave + r, t = t0 + i;
+    if (t >= d.T) break;
+    const size_t row = (size_t)b * d.T + t;
+    if (t >= Tb) {
+      if (lane == 0) mE[row] = 0.0f;
+      continue;
+    }
+    const float* x = E + row * d.V;
+    const float m = row_max(x, d.V, vec4, lane);
+    if (lane == 0) mE[row] = m;
+    put_away();
+#pragma unroll
+    for (int k = 0; k < kPickU / 64; ++k) pick[k] = x[col[k]];
+    xb = x[d.blank];
+    pending = i;
+    // label positions past the first kPickU: straight from the row
+    for (int u = kPickU + lane; u < nlab; u += 64)
+      p.elS[plane_row(d, b, u) + t + u] = x[labels[(size_t)b * (d.U - 1) + u]];
+  }
+  put_away();
+  __syncthreads();
+  const int nrows = min(kPickRows, Tb - t0);  // may be <= 0
+  if ((int)threadIdx.x < nrows) p.eb[(size_t)b * d.Tp + d.Eo + t0 + threadIdx.x] = blanks[threadIdx.x];
+  const int nu = min(nlab, kPickU);
+  for (int idx = threadIdx.x; idx < nu * kPickRows; idx += 256) {
+    const int u = idx >> 4, i = idx & 15;
+    if (i < nrows) p.elS[plane_row(d, b, u) + t0 + i + u] = tile[i][u];
+  }
+}
+
+// The same for the predictions: P[u, blank] and P[u, label_u].
+__global__ __launch_bounds__(256) void rowmax_pick_p_kernel(const float* __restrict__ P,
+                                                            float* __restrict__ mP,
+                                                            const int* __restrict__ labels,
+                                                            const int* __restrict__ labLen,
+                                                            Planes p, Dims d, int vec4) {
+  const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (row >= (long)d.B * d.U) return;
+  const int b = (int)(row / d.U), u = (int)(row - (long)b * d.U);
+  const int Ub = min(max(labLen[b], 0) + 1, d.U);
+  if (u >= Ub) {
+    if (lane == 0) mP[row] = 0.0f;
+    return;
+  }
+  const float* x = P + (size_t)row * d.V;
+  const float m = row_max(x, d.V, vec4, lane);
+  if (lane == 0) {
+    mP[row] = m;
+    const bool has_label = labels != nullptr && (u + 1 < Ub);
+    p.pb[(size_t)b * d.Ua + u] = x[d.blank];
+    p.pl[(size_t)b * d.Ua + u] = has_label ? x[labels[(size_t)b * (d.U - 1) + u]] : 0.0f;
+  }
 }
 
 // ------------------------------------------------------------------ log-normaliser, any shape
@@ -334,6 +433,21 @@ int launch_rowmax(const float* X, float* rowmax, long rows, int V, int rows_per_
   hipLaunchKernelGGL(rowmax_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, s, X, rowmax,
                      rows, V, vec4, rows_per_item, lengths, extra);
   RNNT_LAUNCH_CHECK("rowmax_kernel");
+  return kOk;
+}
+
+int launch_rowmax_pick(const float* E, const float* P, float* mE, float* mP, const int* labels,
+                       const int* inLen, const int* labLen, const Planes& p, const Dims& d,
+                       hipStream_t s) {
+  if (d.B == 0 || d.T == 0 || d.U == 0) return kOk;
+  const int ve = (d.V % 4 == 0) && ((reinterpret_cast<uintptr_t>(E) & 15) == 0);
+  const int vp = (d.V % 4 == 0) && ((reinterpret_cast<uintptr_t>(P) & 15) == 0);
+  hipLaunchKernelGGL(rowmax_pick_e_kernel, dim3((d.T + kPickRows - 1) / kPickRows, d.B), dim3(256),
+                     0, s, E, mE, labels, inLen, labLen, p, d, ve);
+  RNNT_LAUNCH_CHECK("rowmax_pick_e_kernel");
+  hipLaunchKernelGGL(rowmax_pick_p_kernel, dim3((unsigned)(((long)d.B * d.U + 3) / 4)), dim3(256),
+                     0, s, P, mP, labels, labLen, p, d, vp);
+  RNNT_LAUNCH_CHECK("rowmax_pick_p_kernel");
   return kOk;
 }
 

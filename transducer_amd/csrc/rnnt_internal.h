@@ -132,6 +132,11 @@ int wplane_tw(int T);  // frame-axis pitch of the W planes (multiple of 64)
 // their item (rows_per_item rows each) are not read and report 0.
 int launch_rowmax(const float* X, float* rowmax, long rows, int V, int rows_per_item,
                   const int* lengths, int extra, hipStream_t s);
+// Row maxima of E and P and, in the same pass, what launch_gather extracts (E[t,blank],
+// E[t,label_u], P[u,blank], P[u,label_u] into the planes); needs inLen and labLen.
+int launch_rowmax_pick(const float* E, const float* P, float* mE, float* mP, const int* labels,
+                       const int* inLen, const int* labLen, const Planes& p, const Dims& d,
+                       hipStream_t s);
 // Log-normaliser, general form (any V and alignment; fp32 matrix instructions).
 int launch_lse(const float* E, const float* P, const float* mE, const float* mP, float* LN,
                const int* inLen, const int* labLen, const Dims& d, hipStream_t s);
