@@ -201,6 +201,28 @@ def test_log_norms_against_fp64(B, T, U, V, sigma):
         assert not got[b, il[b]:].any() and not got[b, :, ll[b] + 1:].any()
 
 
+def test_log_norms_reference_moves_late_in_the_row():
+    """Large scores far from the start of a row, rows that start with -inf, a row whose largest
+    value sits in the last column: the per-frame reference of the streaming kernel has to move
+    (and rescale what it has summed) without losing accuracy."""
+    rng = np.random.default_rng(1)
+    V = 1200
+    E = rng.standard_normal((1, 70, V)).astype(np.float32)
+    P = rng.standard_normal((1, 9, V)).astype(np.float32)
+    E[0, 0:20, 700] += 100.0          # one jump
+    E[0, 20:40, 300] += 50.0          # two jumps
+    E[0, 20:40, 900] += 120.0
+    E[0, 40:50, :64] = -np.inf        # first slabs hold nothing
+    E[0, 50:60, V - 1] += 300.0       # last column
+    E[0, 60:70, 100:1100] -= 80.0     # large early, tiny later: no jump
+    c = DeviceCase(E, P, np.zeros((1, 8), np.int32), np.array([70], np.int32),
+                   np.array([8], np.int32))
+    got = gpu_log_norms(c, with_lengths=False)
+    truth = oracle.log_norms_truth(E, P)
+    assert np.isfinite(got).all()
+    assert np.abs(got - truth).max() < 4e-6 * max(1.0, np.abs(truth).max())
+
+
 def test_log_norms_wide_dynamic_range():
     # maxima of the two operands at different v: the separable shift must not lose the sum
     rng = np.random.default_rng(0)

@@ -120,18 +120,21 @@ bool nothing_to_do(int B, int T, int U) { return B == 0 || T == 0 || U == 0; }
 int log_norms_stages(const float* E, const float* P, float* mE, float* mP, float* LN,
                      void* scratch, const int* inLen, const int* labLen, const Dims& d,
                      hipStream_t s, const Planes* planes = nullptr, const int* labels = nullptr) {
+  if (scratch && lse_stream_supported(E, d)) {
+    // one pass over E: the streaming kernel finds its own per-frame reference and leaves it in mE
+    RNNT_STAGE(kRowmax, launch_rowmax(P, mP, (long)d.B * d.U, d.V, d.U, labLen, 1, s));
+    RNNT_STAGE(kYplanes, launch_yplanes(P, mP, scratch, labLen, d, s));
+    RNNT_STAGE(kLse, launch_lse_stream(E, mE, mP, LN, scratch, inLen, labLen, d, s));
+    if (planes) RNNT_STAGE(kGather, launch_gather(E, P, labels, inLen, labLen, *planes, d, s));
+    return kOk;
+  }
   if (planes) {
     RNNT_STAGE(kRowmax, launch_rowmax_pick(E, P, mE, mP, labels, inLen, labLen, *planes, d, s));
   } else {
     RNNT_STAGE(kRowmax, launch_rowmax(E, mE, (long)d.B * d.T, d.V, d.T, inLen, 0, s));
     RNNT_STAGE(kRowmax, launch_rowmax(P, mP, (long)d.B * d.U, d.V, d.U, labLen, 1, s));
   }
-  if (scratch && lse_stream_supported(E, d)) {
-    RNNT_STAGE(kYplanes, launch_yplanes(P, mP, scratch, labLen, d, s));
-    RNNT_STAGE(kLse, launch_lse_stream(E, mE, mP, LN, scratch, inLen, labLen, d, s));
-  } else {
-    RNNT_STAGE(kLse, launch_lse(E, P, mE, mP, LN, inLen, labLen, d, s));
-  }
+  RNNT_STAGE(kLse, launch_lse(E, P, mE, mP, LN, inLen, labLen, d, s));
   return kOk;
 }
 

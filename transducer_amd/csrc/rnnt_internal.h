@@ -142,11 +142,13 @@ int launch_lse(const float* E, const float* P, const float* mE, const float* mP,
                const int* inLen, const int* labLen, const Dims& d, hipStream_t s);
 // Log-normaliser, streaming form (rnnt_lse.hip): V % 4 == 0 and 16-byte aligned E.  The pieces of
 // exp(P - mP) are first written to `scratch` (lse_scratch_bytes) in matrix-operand order.
+// launch_lse_stream needs mP only and WRITES mE (one reference value per frame, >= the row
+// maximum minus a fixed slack; what the gradient kernels need as mE).
 bool lse_stream_supported(const float* E, const Dims& d);
 size_t lse_scratch_bytes(const Dims& d);
 int launch_yplanes(const float* P, const float* mP, void* scratch, const int* labLen,
                    const Dims& d, hipStream_t s);
-int launch_lse_stream(const float* E, const float* mE, const float* mP, float* LN,
+int launch_lse_stream(const float* E, float* mE, const float* mP, float* LN,
                       const void* scratch, const int* inLen, const int* labLen, const Dims& d,
                       hipStream_t s);
 int launch_wplanes(const float* lngrads, const float* LN, const float* mE, const float* mP,

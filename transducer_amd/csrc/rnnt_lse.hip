@@ -23,6 +23,11 @@
 //    Every kFlush slabs the running sums are therefore added (vector ALU, round to nearest) into
 //    a second set of accumulators and restarted: the truncation then acts on a sum that is
 //    V / (32 kFlush) times smaller.
+//  * No separate pass over E for its row maxima: any reference m[t] works in X = exp(E - m[t]) as
+//    long as it is taken back out at the end, so a row starts with the maximum of its first 32
+//    values and keeps it unless a later value exceeds it by more than kSlack (then the sums of
+//    that row are multiplied by exp(old - new) once; rare).  The final reference is written out
+//    as mE[t] for the gradient kernels, which only need it to be consistent with LN.
 //  * Workgroups are renumbered so that all frame tiles of one utterance run on the same XCD
 //    (workgroup ids are dealt round-robin to the 8 XCDs) and share its L2 copy of Y[b].
 #include "rnnt_internal.h"
@@ -36,6 +41,8 @@ constexpr int kRows = 128;    // frames per workgroup tile
 constexpr int kSlice = 32;    // v per LDS slab (two matrix-instruction steps)
 constexpr int kSlots = kRows * 4;  // 16-byte slots per piece plane: 4 per row
 constexpr int kFlush = 8;     // slabs between two flushes of the running sums
+constexpr float kSlack = 40.0f;  // a row's reference moves when a value tops it by more than this
+constexpr float kLowest = -1.0e30f;  // stands in for a reference of -inf (a slab of -inf scores)
 
 __device__ inline int mfma_row(int r, int h) { return 8 * (r >> 2) + 4 * h + (r & 3); }
 
@@ -92,13 +99,16 @@ __global__ __launch_bounds__(256) void yplanes_kernel(const float* __restrict__ 
 // half the registers, twice the wavefronts to hide each other's staging).
 template <int kWaves>
 __global__ __launch_bounds__(64 * kWaves, kWaves / 2) void lse_stream_kernel(
-    const float* __restrict__ E, const float* __restrict__ mE, const float* __restrict__ mP,
+    const float* __restrict__ E, float* __restrict__ mE, const float* __restrict__ mP,
     const uint4* __restrict__ Yp, float* __restrict__ LN, const int* __restrict__ inLen,
     const int* __restrict__ labLen, Dims d, int ttiles, int utiles, int total, int nub, int nks) {
   constexpr int kThreads = 64 * kWaves;
   constexpr int MB = 16 / kWaves;          // 32-frame blocks per wavefront
   constexpr int NR = 512 / kThreads;       // (row, eight v) items a thread stages per slab
   __shared__ uint4 Xs[2][3][kSlots];
+  __shared__ float scale[kRows];  // pending factor for a row's sums (1 when its reference stood)
+  __shared__ float mfin[kRows];   // final references, for the write-out
+  __shared__ int moved;           // some row's reference moved while the last slab was staged
   // XCD-aware renumbering: physical id n runs on XCD n % 8
   const int n = blockIdx.x, per_xcd = gridDim.x >> 3;
   const int logical = (n & 7) * per_xcd + (n >> 3);
@@ -116,8 +126,13 @@ __global__ __launch_bounds__(64 * kWaves, kWaves / 2) void lse_stream_kernel(
       const int t = t0 + e / 128, u = u0 + e % 128;
       if (t < d.T && u < d.U) LNb[(size_t)t * d.U + u] = 0.0f;
     }
+    if (t0 >= Tb)  // frames past the utterance report a reference of 0
+      for (int r = tid; r < kRows; r += kThreads)
+        if (t0 + r < d.T) mE[(size_t)b * d.T + t0 + r] = 0.0f;
     return;
   }
+  for (int r = tid; r < kRows; r += kThreads) scale[r] = 1.0f;
+  if (tid == 0) moved = 0;
 
   // staging: thread -> rows srow (+ 64 with four wavefronts) of the tile, v = slab start +
   // 8*c8 .. +7.  Rows past the utterance repeat its last frame, groups of four past V repeat
@@ -125,14 +140,14 @@ __global__ __launch_bounds__(64 * kWaves, kWaves / 2) void lse_stream_kernel(
   // the way out.
   const int srow = tid >> 2, c8 = tid & 3;
   const float* px[NR];
-  float mx[NR];
+  float mx[NR];  // the row's reference; the four threads that share a row always agree on it
   int slot[NR];
 #pragma unroll
   for (int i = 0; i < NR; ++i) {
     const int row = srow + (kThreads / 4) * i;
     const int t = min(t0 + row, Tb - 1);
     px[i] = E + ((size_t)b * d.T + t) * d.V;
-    mx[i] = mE[(size_t)b * d.T + t];
+    mx[i] = kLowest;
     slot[i] = xslot(row, c8);
   }
   struct XRegs { float4 lo[NR], hi[NR]; };
@@ -146,9 +161,23 @@ __global__ __launch_bounds__(64 * kWaves, kWaves / 2) void lse_stream_kernel(
     }
     return r;
   };
-  auto stash = [&](int buf, const XRegs& r) {
+  auto stash = [&](int buf, const XRegs& r, bool first) {
 #pragma unroll
     for (int i = 0; i < NR; ++i) {
+      // maximum of the row's 32 values of this slab (values past V repeat earlier ones)
+      float lm = fmaxf(fmaxf(fmaxf(r.lo[i].x, r.lo[i].y), fmaxf(r.lo[i].z, r.lo[i].w)),
+                       fmaxf(fmaxf(r.hi[i].x, r.hi[i].y), fmaxf(r.hi[i].z, r.hi[i].w)));
+      lm = fmaxf(lm, __shfl_xor(lm, 1, 64));
+      lm = fmaxf(lm, __shfl_xor(lm, 2, 64));
+      lm = fmaxf(lm, kLowest);
+      if (first) {
+        mx[i] = lm;
+      } else if (lm > mx[i] + kSlack) {
+        // everything summed for this row so far shrinks by exp(old - new) (0 if old was -inf)
+        if (c8 == 0) scale[srow + (kThreads / 4) * i] = __expf(mx[i] - lm);
+        moved = 1;
+        mx[i] = lm;
+      }
       const float m = mx[i];
       const float x[8] = {__expf(r.lo[i].x - m), __expf(r.lo[i].y - m), __expf(r.lo[i].z - m),
                           __expf(r.lo[i].w - m), __expf(r.hi[i].x - m), __expf(r.hi[i].y - m),
@@ -216,11 +245,8 @@ __global__ __launch_bounds__(64 * kWaves, kWaves / 2) void lse_stream_kernel(
 #pragma unroll
     for (int m = 0; m < MB; ++m) acc[m] = mfma_bf16(ah[m], y.h, acc[m]);
   };
-  // E is requested two slabs ahead (HBM latency under load exceeds one slab's matrix work);
-  // the slab requested one call earlier is already in registers, so its exps and splits can be
-  // scheduled among this slab's matrix instructions.
-  auto slab = [&](int kt, const YRegs& yc, YRegs& yn, const XRegs& xs, XRegs& xl) {
-    xl = fetch(min(kt + 2, nk - 1) * kSlice);
+  auto slab = [&](int kt, const YRegs& yc, YRegs& yn) {
+    const XRegs xs = fetch(min(kt + 1, nk - 1) * kSlice);
     if (active) {
       const int ktn = min(kt + 1, nk - 1);
       yn.s0 = fetch_y(2 * ktn);
@@ -231,12 +257,27 @@ __global__ __launch_bounds__(64 * kWaves, kWaves / 2) void lse_stream_kernel(
       step(1, yc.s1);
     }
     __builtin_amdgcn_sched_barrier(0);
-    stash(cur ^ 1, xs);
+    stash(cur ^ 1, xs, false);
     __syncthreads();
     cur ^= 1;
+    if (moved) {  // uniform; rare: apply the factors before the re-referenced slab is multiplied
+      if (active) {
+#pragma unroll
+        for (int m = 0; m < MB; ++m)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const float f = scale[32 * (mb0 + m) + mfma_row(r, h)];
+            acc[m][r] *= f;
+            tot[m][r] *= f;
+          }
+      }
+      __syncthreads();
+      for (int r = tid; r < kRows; r += kThreads) scale[r] = 1.0f;
+      if (tid == 0) moved = 0;
+      __syncthreads();
+    }
   };
-  stash(0, fetch(0));
-  XRegs xa = fetch(min(1, nk - 1) * kSlice), xb;
+  stash(0, fetch(0), true);
   YRegs y0, y1;
   if (active) {
     y0.s0 = fetch_y(0);
@@ -244,8 +285,8 @@ __global__ __launch_bounds__(64 * kWaves, kWaves / 2) void lse_stream_kernel(
   }
   __syncthreads();
   for (int kt = 0; kt < nk; kt += 2) {
-    slab(kt, y0, y1, xa, xb);
-    if (kt + 1 < nk) slab(kt + 1, y1, y0, xb, xa);
+    slab(kt, y0, y1);
+    if (kt + 1 < nk) slab(kt + 1, y1, y0);
     if (active && (kt + 2) % kFlush == 0) {
 #pragma unroll
       for (int m = 0; m < MB; ++m)
@@ -254,6 +295,16 @@ __global__ __launch_bounds__(64 * kWaves, kWaves / 2) void lse_stream_kernel(
     }
   }
 
+  // final references: to LDS for the write-out below, to mE for the kernels that come later
+#pragma unroll
+  for (int i = 0; i < NR; ++i) {
+    const int row = srow + (kThreads / 4) * i;
+    if (c8 == 0) {
+      mfin[row] = mx[i];
+      if (t0 + row < d.T) mE[(size_t)b * d.T + t0 + row] = (t0 + row < Tb) ? mx[i] : 0.0f;
+    }
+  }
+  __syncthreads();
   const int u = 32 * ublock + l32;
   if (!active) {
     // label positions past the utterance (but inside U) are written as zeros
@@ -264,16 +315,15 @@ __global__ __launch_bounds__(64 * kWaves, kWaves / 2) void lse_stream_kernel(
       }
     return;
   }
-  const float* mEb = mE + (size_t)b * d.T;
   const float mu = mP[(size_t)b * d.U + min(u, Ub - 1)];
 #pragma unroll
   for (int m = 0; m < MB; ++m)
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-      const int t = t0 + 32 * (mb0 + m) + mfma_row(r, h);
+      const int row = 32 * (mb0 + m) + mfma_row(r, h), t = t0 + row;
       if (t < d.T && u < d.U) {
         float v = 0.0f;
-        if (t < Tb && u < Ub) v = (logf(tot[m][r] + acc[m][r]) + mEb[t]) + mu;
+        if (t < Tb && u < Ub) v = (logf(tot[m][r] + acc[m][r]) + mfin[row]) + mu;
         LNb[(size_t)t * d.U + u] = v;
       }
     }
@@ -308,7 +358,7 @@ int launch_yplanes(const float* P, const float* mP, void* scratch, const int* la
   return kOk;
 }
 
-int launch_lse_stream(const float* E, const float* mE, const float* mP, float* LN,
+int launch_lse_stream(const float* E, float* mE, const float* mP, float* LN,
                       const void* scratch, const int* inLen, const int* labLen, const Dims& d,
                       hipStream_t s) {
   const int nub = y_ublocks(d), nks = y_steps(d);
