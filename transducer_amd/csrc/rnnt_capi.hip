@@ -122,6 +122,14 @@ int log_norms_stages(const float* E, const float* P, float* mE, float* mP, float
                      hipStream_t s, const Planes* planes = nullptr, const int* labels = nullptr) {
   if (scratch && lse_stream_supported(E, d)) {
     // one pass over E: the streaming kernel finds its own per-frame reference and leaves it in mE
+    // and, with `planes`, copies the blank / label scores out of the rows as they stream by
+    if (planes && d.U - 1 <= 1024) {
+      RNNT_STAGE(kRowmax, launch_rowmax_pick_p(P, mP, labels, labLen, *planes, d, s));
+      RNNT_STAGE(kYplanes, launch_yplanes(P, mP, scratch, labLen, d, s));
+      RNNT_STAGE(kLse, launch_lse_stream(E, mE, mP, LN, scratch, inLen, labLen, d, s, labels,
+                                         planes->elS, planes->eb));
+      return kOk;
+    }
     RNNT_STAGE(kRowmax, launch_rowmax(P, mP, (long)d.B * d.U, d.V, d.U, labLen, 1, s));
     RNNT_STAGE(kYplanes, launch_yplanes(P, mP, scratch, labLen, d, s));
     RNNT_STAGE(kLse, launch_lse_stream(E, mE, mP, LN, scratch, inLen, labLen, d, s));

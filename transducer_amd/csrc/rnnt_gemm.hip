@@ -451,6 +451,16 @@ int launch_rowmax_pick(const float* E, const float* P, float* mE, float* mP, con
   return kOk;
 }
 
+int launch_rowmax_pick_p(const float* P, float* mP, const int* labels, const int* labLen,
+                         const Planes& p, const Dims& d, hipStream_t s) {
+  if (d.B == 0 || d.U == 0) return kOk;
+  const int vp = (d.V % 4 == 0) && ((reinterpret_cast<uintptr_t>(P) & 15) == 0);
+  hipLaunchKernelGGL(rowmax_pick_p_kernel, dim3((unsigned)(((long)d.B * d.U + 3) / 4)), dim3(256),
+                     0, s, P, mP, labels, labLen, p, d, vp);
+  RNNT_LAUNCH_CHECK("rowmax_pick_p_kernel");
+  return kOk;
+}
+
 int launch_lse(const float* E, const float* P, const float* mE, const float* mP, float* LN,
                const int* inLen, const int* labLen, const Dims& d, hipStream_t s) {
   if (d.B == 0 || d.T == 0 || d.U == 0) return kOk;

@@ -148,9 +148,15 @@ bool lse_stream_supported(const float* E, const Dims& d);
 size_t lse_scratch_bytes(const Dims& d);
 int launch_yplanes(const float* P, const float* mP, void* scratch, const int* labLen,
                    const Dims& d, hipStream_t s);
+// With elS / eb (skewed label-score plane and blank-score vector) it also copies E[t, label_u]
+// and E[t, blank] out of the rows it streams (what launch_gather does for the emissions).
 int launch_lse_stream(const float* E, float* mE, const float* mP, float* LN,
                       const void* scratch, const int* inLen, const int* labLen, const Dims& d,
-                      hipStream_t s);
+                      hipStream_t s, const int* labels = nullptr, float* elS = nullptr,
+                      float* eb = nullptr);
+// P[u, blank] and P[u, label_u] into the planes, with the row maxima of P (one pass).
+int launch_rowmax_pick_p(const float* P, float* mP, const int* labels, const int* labLen,
+                         const Planes& p, const Dims& d, hipStream_t s);
 int launch_wplanes(const float* lngrads, const float* LN, const float* mE, const float* mP,
                    float* Wn, float* Wt, const int* inLen, const int* labLen, const Dims& d,
                    hipStream_t s);

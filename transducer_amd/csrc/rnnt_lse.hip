@@ -101,7 +101,8 @@ template <int kWaves>
 __global__ __launch_bounds__(64 * kWaves, kWaves / 2) void lse_stream_kernel(
     const float* __restrict__ E, float* __restrict__ mE, const float* __restrict__ mP,
     const uint4* __restrict__ Yp, float* __restrict__ LN, const int* __restrict__ inLen,
-    const int* __restrict__ labLen, Dims d, int ttiles, int utiles, int total, int nub, int nks) {
+    const int* __restrict__ labLen, Dims d, int ttiles, int utiles, int total, int nub, int nks,
+    const int* __restrict__ labels, float* __restrict__ elS, float* __restrict__ ebv) {
   constexpr int kThreads = 64 * kWaves;
   constexpr int MB = 16 / kWaves;          // 32-frame blocks per wavefront
   constexpr int NR = 512 / kThreads;       // (row, eight v) items a thread stages per slab
@@ -109,6 +110,8 @@ __global__ __launch_bounds__(64 * kWaves, kWaves / 2) void lse_stream_kernel(
   __shared__ float scale[kRows];  // pending factor for a row's sums (1 when its reference stood)
   __shared__ float mfin[kRows];   // final references, for the write-out
   __shared__ int moved;           // some row's reference moved while the last slab was staged
+  __shared__ int labs[1025];      // columns to pick: the utterance's labels, then the blank
+  __shared__ short order[1025];   // their indices sorted by column
   // XCD-aware renumbering: physical id n runs on XCD n % 8
   const int n = blockIdx.x, per_xcd = gridDim.x >> 3;
   const int logical = (n & 7) * per_xcd + (n >> 3);
@@ -133,6 +136,28 @@ __global__ __launch_bounds__(64 * kWaves, kWaves / 2) void lse_stream_kernel(
   }
   for (int r = tid; r < kRows; r += kThreads) scale[r] = 1.0f;
   if (tid == 0) moved = 0;
+  // Picks: the lattice recursions need E[t, blank] and E[t, label_u] in the skewed planes.  Every
+  // element of the tile's rows passes through the staging registers exactly once, so the thread
+  // that holds a wanted column copies it out then (first label tile only; elS == nullptr: off).
+  const bool picking = elS != nullptr && u0 == 0;
+  const int nlab = (picking && labels != nullptr) ? min(Ub - 1, 1024) : 0;
+  const int npick = picking ? nlab + 1 : 0;  // entry nlab is the blank column
+  for (int u = tid; u < npick; u += kThreads)
+    labs[u] = u < nlab ? labels[(size_t)b * (d.U - 1) + u] : d.blank;
+  __syncthreads();
+  // rank every entry by (column, index): the slabs come by in column order, so one cursor into
+  // the sorted list tells each slab which columns to copy, at one LDS read per slab
+  for (int u = tid; u < npick; u += kThreads) {
+    const int c = labs[u];
+    int rank = 0;
+    for (int w = 0; w < npick; ++w) {
+      const int cw = labs[w];
+      rank += (cw < c || (cw == c && w < u)) ? 1 : 0;
+    }
+    order[rank] = (short)u;
+  }
+  int cursor = 0;      // uniform: entries before it have been copied
+  int next_slab = -1;  // slab of entry `cursor` (kept in a register: no LDS access on slabs without one)
 
   // staging: thread -> rows srow (+ 64 with four wavefronts) of the tile, v = slab start +
   // 8*c8 .. +7.  Rows past the utterance repeat its last frame, groups of four past V repeat
@@ -161,7 +186,37 @@ __global__ __launch_bounds__(64 * kWaves, kWaves / 2) void lse_stream_kernel(
     }
     return r;
   };
-  auto stash = [&](int buf, const XRegs& r, bool first) {
+  // copies column `col` (which lies in the slab held in r) of this thread's rows to dst[t]
+  auto pick = [&](const XRegs& r, int col, float* dst) {
+    if (c8 != ((col & 31) >> 3)) return;
+    const int e = col & 7;  // uniform
+#pragma unroll
+    for (int i = 0; i < NR; ++i) {
+      // element e of the eight this thread holds, selected with masks: an indexed access would
+      // send the staging registers through scratch memory on every slab
+      const unsigned k0 = e == 0 ? ~0u : 0u, k1 = e == 1 ? ~0u : 0u, k2 = e == 2 ? ~0u : 0u,
+                     k3 = e == 3 ? ~0u : 0u, k4 = e == 4 ? ~0u : 0u, k5 = e == 5 ? ~0u : 0u,
+                     k6 = e == 6 ? ~0u : 0u, k7 = e == 7 ? ~0u : 0u;
+      const float v = __uint_as_float(
+          (__float_as_uint(r.lo[i].x) & k0) | (__float_as_uint(r.lo[i].y) & k1) |
+          (__float_as_uint(r.lo[i].z) & k2) | (__float_as_uint(r.lo[i].w) & k3) |
+          (__float_as_uint(r.hi[i].x) & k4) | (__float_as_uint(r.hi[i].y) & k5) |
+          (__float_as_uint(r.hi[i].z) & k6) | (__float_as_uint(r.hi[i].w) & k7));
+      const int t = t0 + srow + (kThreads / 4) * i;
+      if (t < Tb) dst[t] = v;
+    }
+  };
+  auto picks = [&](const XRegs& r, int kslab) {
+    while (next_slab == kslab) {  // uniform
+      const int u = order[cursor], col = labs[u];
+      if (u == nlab) pick(r, col, ebv + (size_t)b * d.Tp + d.Eo);
+      else pick(r, col, elS + plane_row(d, b, u) + u);
+      ++cursor;
+      next_slab = cursor < npick ? (labs[order[cursor]] >> 5) : -1;
+    }
+  };
+  auto stash = [&](int buf, const XRegs& r, bool first, int kslab) {
+    if (picking) picks(r, kslab);
 #pragma unroll
     for (int i = 0; i < NR; ++i) {
       // maximum of the row's 32 values of this slab (values past V repeat earlier ones)
@@ -257,7 +312,7 @@ __global__ __launch_bounds__(64 * kWaves, kWaves / 2) void lse_stream_kernel(
       step(1, yc.s1);
     }
     __builtin_amdgcn_sched_barrier(0);
-    stash(cur ^ 1, xs, false);
+    stash(cur ^ 1, xs, false, min(kt + 1, nk - 1));
     __syncthreads();
     cur ^= 1;
     if (moved) {  // uniform; rare: apply the factors before the re-referenced slab is multiplied
@@ -277,7 +332,9 @@ __global__ __launch_bounds__(64 * kWaves, kWaves / 2) void lse_stream_kernel(
       __syncthreads();
     }
   };
-  stash(0, fetch(0), true);
+  __syncthreads();  // order
+  if (npick > 0) next_slab = labs[order[0]] >> 5;
+  stash(0, fetch(0), true, 0);
   YRegs y0, y1;
   if (active) {
     y0.s0 = fetch_y(0);
@@ -360,7 +417,7 @@ int launch_yplanes(const float* P, const float* mP, void* scratch, const int* la
 
 int launch_lse_stream(const float* E, float* mE, const float* mP, float* LN,
                       const void* scratch, const int* inLen, const int* labLen, const Dims& d,
-                      hipStream_t s) {
+                      hipStream_t s, const int* labels, float* elS, float* eb) {
   const int nub = y_ublocks(d), nks = y_steps(d);
   const int ttiles = (d.T + kRows - 1) / kRows, utiles = (d.U + 127) / 128;
   const long total = (long)ttiles * utiles * d.B;
@@ -368,7 +425,7 @@ int launch_lse_stream(const float* E, float* mE, const float* mP, float* LN,
   constexpr int kWaves = 4;
   hipLaunchKernelGGL(lse_stream_kernel<kWaves>, dim3(grid), dim3(64 * kWaves), 0, s, E, mE, mP,
                      static_cast<const uint4*>(scratch), LN, inLen, labLen, d, ttiles, utiles,
-                     (int)total, nub, nks);
+                     (int)total, nub, nks, labels, elS, eb);
   RNNT_LAUNCH_CHECK("lse_stream_kernel");
   return kOk;
 }
