@@ -50,11 +50,11 @@ __device__ inline float log1p_unit(float y) {
 
 // transducer/transducer_cpu.cpp:16-24
 __device__ inline float lse2(float a, float b) {
+  // One operand -inf: |a - b| = inf, exp gives 0, log1p(0) = 0 and the sum is the other operand
+  // exactly, as the reference's early returns have it; only both -inf (inf - inf) needs a guard.
   const float hi = fmaxf(a, b);
-  float r = hi + log1p_unit(exp_neg(-fabsf(a - b)));
-  r = (b == kNegInf) ? a : r;
-  r = (a == kNegInf) ? b : r;
-  return r;
+  const float r = hi + log1p_unit(exp_neg(-fabsf(a - b)));
+  return (hi == kNegInf) ? kNegInf : r;
 }
 
 __device__ inline float f4get(const float4& v, int j) {
