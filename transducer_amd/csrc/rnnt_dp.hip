@@ -200,9 +200,7 @@ __global__ __launch_bounds__(64) void alpha_kernel(Planes p, const int* __restri
     return r;
   };
 
-  Group cur = load_group(0);
-  for (int g = 0; g < ngroups; ++g) {
-    const Group nxt = load_group(g + 1 < ngroups ? g + 1 : g);
+  auto run_group = [&](int g, const Group& cur) {
     float4 aout[C];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -230,7 +228,15 @@ __global__ __launch_bounds__(64) void alpha_kernel(Planes p, const int* __restri
     }
 #pragma unroll
     for (int c = 0; c < C; ++c) *reinterpret_cast<float4*>(ap[c] + 4 * g) = aout[c];
-    cur = nxt;
+  };
+  // two register sets alternate (no copies): a group's loads are requested two groups ahead
+  auto clamp_g = [&](int g) { return g < ngroups ? g : ngroups - 1; };
+  Group x = load_group(0), y = load_group(clamp_g(1));
+  for (int g = 0; g < ngroups; g += 2) {
+    run_group(g, x);
+    x = load_group(clamp_g(g + 2));
+    if (g + 1 < ngroups) run_group(g + 1, y);
+    y = load_group(clamp_g(g + 3));
   }
   // :73-78 the blank move out of the last cell, negated; that cell was the last one its
   // column processed
