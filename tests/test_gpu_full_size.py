@@ -1,0 +1,192 @@
+"""The benchmark configurations at their full sizes (B=8/32, T=2000, U=100, V up to 10000).
+
+The CPU oracle needs minutes for the largest one, so there the device result is held to
+properties that do not depend on size -- rows of a gradient sum to zero, padding stays exactly
+zero, the upstream factor is linear, an utterance's result does not depend on what else is in
+the batch (bit for bit) -- and to the oracle on ONE utterance cut out of the batch.  The smaller
+configurations go through the oracle whole."""
+import numpy as np
+import pytest
+
+from util import RTOL, ATOL, DeviceCase, assert_close, dev, gpu_loss, ptr, violations
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+import oracle  # noqa: E402
+from transducer_amd import capi  # noqa: E402
+from transducer_amd.synthetic import CONFIGS, lengths, make_inputs  # noqa: E402
+
+
+def unpack(d):
+    return tuple(d[k] for k in ("emissions", "predictions", "labels", "input_lengths",
+                                "label_lengths"))
+
+
+class DeviceBatch(object):
+    """Inputs of one configuration drawn on the device (torch's generator: these tests check
+    properties and cut-outs, not fixtures, so the host generator's minutes are not needed)."""
+
+    def __init__(self, cfg, seed, near_ties=False):
+        g = torch.Generator(device="cuda:0")
+        g.manual_seed(seed)
+        self.B, self.T, self.U, self.V = cfg.B, cfg.T, cfg.U + 1, cfg.V
+        self.E = torch.randn((cfg.B, cfg.T, cfg.V), generator=g, device="cuda:0") * cfg.sigma
+        self.P = torch.randn((cfg.B, cfg.U + 1, cfg.V), generator=g, device="cuda:0") * cfg.sigma
+        self.labels = torch.randint(1, cfg.V, (cfg.B, cfg.U), generator=g, device="cuda:0",
+                                    dtype=torch.int32)
+        il, ll = lengths(cfg, np.random.Generator(np.random.Philox(key=seed)))
+        self.il_h, self.ll_h = il, ll
+        self.il, self.ll = dev(il), dev(ll)
+        if near_ties:  # a tenth of the entries of every frame repeat another column's value
+            k = cfg.V // 10
+            for b in range(cfg.B):
+                dst = torch.randint(1, cfg.V, (cfg.T, k), generator=g, device="cuda:0")
+                src = torch.randint(1, cfg.V, (cfg.T, k), generator=g, device="cuda:0")
+                self.E[b].scatter_(1, dst, self.E[b].gather(1, src))
+
+    @property
+    def dims(self):
+        return (self.B, self.T, self.U, self.V)
+
+    def cut(self, b):
+        """Utterance b as a batch of one with the same padded sizes."""
+        c = DeviceBatch.__new__(DeviceBatch)
+        c.B, c.T, c.U, c.V = 1, self.T, self.U, self.V
+        c.E, c.P = self.E[b:b + 1].contiguous(), self.P[b:b + 1].contiguous()
+        c.labels = self.labels[b:b + 1].contiguous()
+        c.il_h, c.ll_h = self.il_h[b:b + 1].copy(), self.ll_h[b:b + 1].copy()
+        c.il, c.ll = dev(c.il_h), dev(c.ll_h)
+        return c
+
+    def host(self):
+        return (self.E.cpu().numpy(), self.P.cpu().numpy(), self.labels.cpu().numpy(),
+                self.il_h, self.ll_h)
+
+
+def loss_on_device(c, deltas=None, blank=0):
+    """Whole loss through the C interface; results stay on the device."""
+    B, T, U, V = c.dims
+    nbytes = capi.load().rnnt_hip_loss_workspace_bytes(B, T, U, V)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device="cuda:0")
+    costs = torch.full((B,), float("nan"), device="cuda:0")
+    eg = torch.full_like(c.E, float("nan"))
+    pg = torch.full_like(c.P, float("nan"))
+    capi.call("rnnt_hip_loss_forward", ptr(c.E), ptr(c.P), ptr(c.labels), ptr(c.il), ptr(c.ll),
+              ptr(costs), ptr(ws), nbytes, B, T, U, V, blank, None)
+    capi.call("rnnt_hip_loss_backward", ptr(c.E), ptr(c.P), ptr(c.labels), ptr(c.il), ptr(c.ll),
+              ptr(deltas), ptr(eg), ptr(pg), ptr(ws), nbytes, B, T, U, V, blank, None)
+    torch.cuda.synchronize()
+    return costs, eg, pg
+
+
+def log_norms_on_device(c):
+    B, T, U, V = c.dims
+    LN = torch.full((B, T, U), float("nan"), device="cuda:0")
+    capi.call("rnnt_hip_log_norms", ptr(c.E), ptr(c.P), ptr(LN), ptr(c.il), ptr(c.ll),
+              B, T, U, V, None)
+    return LN
+
+
+def viterbi_on_device(c, LN, blank=0):
+    B, T, U, V = c.dims
+    out = torch.full((B, U - 1), -1, dtype=torch.int32, device="cuda:0")
+    capi.call("rnnt_hip_viterbi", ptr(c.E), ptr(c.P), ptr(LN), ptr(out), ptr(c.il), ptr(c.ll),
+              B, T, U, V, blank, None)
+    torch.cuda.synchronize()
+    return out
+
+
+# ------------------------------------------------------------------ headline configuration
+def test_headline_configuration_properties_and_one_utterance_against_the_oracle():
+    c = DeviceBatch(CONFIGS["cfg4"], seed=3)
+    B, T, U, V = c.dims
+    costs, eg, pg = loss_on_device(c)
+    assert torch.isfinite(costs).all() and (costs > 0).all()
+    assert torch.isfinite(eg).all() and torch.isfinite(pg).all()
+
+    # padding: frames past an utterance and label positions past it hold exact zeros
+    tmask = torch.arange(T, device="cuda:0")[None, :] >= c.il[:, None]
+    umask = torch.arange(U, device="cuda:0")[None, :] > c.ll[:, None]
+    assert not eg[tmask].any() and not pg[umask].any()
+
+    # every row of a gradient sums to zero: sum_v softmax = 1 and the occupancy of a node equals
+    # the sum of its two outgoing moves
+    # (relative to the row's size: with T >> U nearly all of an utterance's waiting happens at
+    # one label position, whose blank entry reaches ~ -T_b as a sequential fp32 sum)
+    se = eg.double().sum(-1).abs()
+    sp = pg.double().sum(-1).abs()
+    ae = eg.double().abs().sum(-1)
+    ap = pg.double().abs().sum(-1)
+    assert float(ae[~tmask].min()) > 1e-3  # the rows are not trivially zero
+    print("largest |row sum| / sum |row|: egrads %.3g, pgrads %.3g"
+          % (float((se / (ae + 1e-30)).max()), float((sp / (ap + 1e-30)).max())))
+    assert bool((se <= 1e-5 + 2e-5 * ae).all())
+    assert bool((sp <= 1e-5 + 2e-5 * ap).all())
+
+    # the upstream factor: exact doubling
+    two = torch.full((B,), 2.0, device="cuda:0")
+    costs2, eg2, pg2 = loss_on_device(c, deltas=two)
+    assert torch.equal(costs2, costs)
+    assert torch.equal(eg2, 2.0 * eg) and torch.equal(pg2, 2.0 * pg)
+    del eg2, pg2
+
+    # an utterance alone gives the same bits as inside the batch
+    shortest = int(np.argmin(c.il_h.astype(np.int64) * (c.ll_h + 1)))
+    for b in (0, shortest):
+        one = c.cut(b)
+        c1, e1, p1 = loss_on_device(one)
+        assert torch.equal(c1[0], costs[b])
+        assert torch.equal(e1[0], eg[b]) and torch.equal(p1[0], pg[b])
+
+    # the shortest utterance against the oracle (18 s of one host core)
+    one = c.cut(shortest)
+    E, P, labels, il, ll = one.host()
+    want = oracle.loss_and_grads(E, P, labels, il, ll)
+    assert_close(costs[shortest:shortest + 1].cpu().numpy(), want["costs"], what="costs")
+    ve, worst_e = violations(eg[shortest].cpu().numpy(), want["egrads"][0])
+    vp, worst_p = violations(pg[shortest].cpu().numpy(), want["pgrads"][0])
+    print("cfg4 utterance %d (T=%d, U=%d): violations egrads %.4f%%, pgrads %.4f%%; max abs err "
+          "%.3g / %.3g" % (shortest, il[0], ll[0], 100 * ve, 100 * vp, worst_e, worst_p))
+    # the reference's own fp32 gradients move by more than the tolerance when LN moves by a few
+    # ulp at this lattice length; the bar is a bounded violation fraction
+    assert ve <= 0.02 and vp <= 0.02
+
+
+@pytest.mark.parametrize("near_ties", [False, True])
+def test_headline_viterbi_one_utterance_bit_exact_and_batch_independent(near_ties):
+    c = DeviceBatch(CONFIGS["cfg5"], seed=5, near_ties=near_ties)
+    LN = log_norms_on_device(c)
+    paths = viterbi_on_device(c, LN)
+    U = c.U
+    written = torch.arange(U - 1, device="cuda:0")[None, :] < c.ll[:, None]
+    assert ((paths >= 1) & (paths < c.V))[written].all()
+    assert (paths[~written] == -1).all()  # only the first label_lengths[b] entries are written
+    shortest = int(np.argmin(c.il_h.astype(np.int64) * (c.ll_h + 1)))
+    one = c.cut(shortest)
+    LN1 = LN[shortest:shortest + 1].contiguous()
+    alone = viterbi_on_device(one, LN1)
+    assert torch.equal(alone[0], paths[shortest])
+    E, P, _, il, ll = one.host()
+    want = oracle.viterbi(E, P, LN1.cpu().numpy(), il, ll)
+    assert np.array_equal(alone.cpu().numpy()[:, :ll[0]], want[:, :ll[0]])
+
+
+# ------------------------------------------------------------------ the smaller configurations, whole
+@pytest.mark.parametrize("name", ["cfg2", "cfg3a", "cfg3b"])
+def test_configuration_whole_against_the_oracle(name):
+    E, P, labels, il, ll = unpack(make_inputs(CONFIGS[name], seed=0))
+    a = oracle.loss_and_grads(E, P, labels, il, ll, lse="naive")
+    b = oracle.loss_and_grads(E, P, labels, il, ll, lse="sep")
+    floor_e, _ = violations(b["egrads"], a["egrads"])
+    floor_p, _ = violations(b["pgrads"], a["pgrads"])
+    costs, eg, pg = gpu_loss(DeviceCase(E, P, labels, il, ll))
+    assert_close(costs, a["costs"], rtol=RTOL, atol=max(ATOL, 1e-3), what="costs")
+    ve, worst_e = violations(eg, a["egrads"])
+    vp, worst_p = violations(pg, a["pgrads"])
+    print("%s: violations egrads %.4f%% (oracle floor between two LN orders %.4f%%), pgrads "
+          "%.4f%% (floor %.4f%%); max abs err %.3g / %.3g"
+          % (name, 100 * ve, 100 * floor_e, 100 * vp, 100 * floor_p, worst_e, worst_p))
+    assert ve <= max(2 * floor_e, 0.02) and vp <= max(2 * floor_p, 0.02)
+    for i in range(E.shape[0]):
+        assert not eg[i, il[i]:].any() and not pg[i, ll[i] + 1:].any()
