@@ -94,6 +94,47 @@ def long_case(B, V, seed, sigma=1.0, ragged=True, T=2000, U=100):
     return unpack(make_inputs(cfg, seed=seed))
 
 
+@pytest.mark.parametrize("B", [1, 10])
+@pytest.mark.parametrize("T", [1, 10, 100])
+def test_reference_stress_grid(B, T):
+    """The grid of the reference's CPU-against-GPU stress test at its own sizes
+    (transducer/test_cuda.cu:323-378: uniform [0,1) scores, input lengths in [0,T], label
+    lengths in [0,U-1], host-computed log_norms, forward + backward + dense accumulation), at
+    this build's tolerance instead of the reference's 1e-3 / 1e-4 where both sides are given the
+    same log_norms."""
+    rng = np.random.Generator(np.random.Philox(key=1000 * B + T))
+    for U in (1, 10, 100):
+        for V in (8, 20, 32, 101, 128):
+            print("stress case B=%d T=%d U=%d V=%d" % (B, T, U, V), flush=True)
+            E = rng.random((B, T, V), dtype=np.float32)
+            P = rng.random((B, U, V), dtype=np.float32)
+            il = rng.integers(0, T + 1, B).astype(np.int32)
+            ll = rng.integers(0, U, B).astype(np.int32)
+            labels = rng.integers(1, V, (B, U - 1)).astype(np.int32)
+            LN = oracle.log_norms_naive(E, P, il, ll)
+            costs_o, alphas_o = oracle.forward(E, P, LN, labels, il, ll)
+            eg_o, pg_o, lng_o = oracle.backward(E, P, np.nan_to_num(alphas_o), LN, labels, il, ll)
+            ed_o, pd_o = oracle.accumulate_grads(E, P, eg_o, pg_o, lng_o, LN, il, ll)
+            c = DeviceCase(E, P, labels, il, ll)
+            costs, alphas = gpu_forward(c, LN)
+            assert np.array_equal(np.isinf(costs), np.isinf(costs_o))
+            assert_close(costs, costs_o, what="costs")
+            eg, pg, lng = gpu_backward(c, alphas, LN)
+            assert_close(lng, lng_o, what="lngrads")
+            ed, pd = gpu_dense_grads(c, eg, pg, lng, LN)
+            assert_close(ed, ed_o, what="egrads")
+            assert_close(pd, pd_o, what="pgrads")
+            # and the fused path, which computes log_norms itself (a last-bit difference there
+            # moves a rounding in alpha, ~6e-5 at |alpha| ~ 1e3): held to the reference's own
+            # bar for this test (test_cuda.cu:373-375)
+            costs_f, ed_f, pd_f = gpu_loss(c)
+            fin = np.isfinite(costs_o)
+            assert np.array_equal(np.isinf(costs_f), np.isinf(costs_o))
+            assert_close(costs_f[fin], costs_o[fin], what="costs (fused)")
+            assert_close(ed_f, ed_o, rtol=1e-3, atol=1e-4, what="egrads (fused)")
+            assert_close(pd_f, pd_o, rtol=1e-3, atol=1e-4, what="pgrads (fused)")
+
+
 @pytest.mark.parametrize("V,sigma,ragged", [(100, 1.0, False), (300, 2.0, True)])
 def test_boundary_at_T2000(V, sigma, ragged):
     """The lattice at its real length.  alpha reaches ~1e4 here (ulp ~1e-3), so gradients only
