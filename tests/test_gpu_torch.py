@@ -135,3 +135,22 @@ def test_nonzero_blank_and_noncontiguous_scores():
     want = oracle.loss_and_grads(d["emissions"], d["predictions"], labels_np, d["input_lengths"],
                                  d["label_lengths"], blank=blank)
     assert_close(costs.cpu().numpy(), want["costs"], what="costs")
+
+
+def test_backward_twice_on_one_forward_gives_the_same_gradients():
+    """benchmarks/torch_benchmarks.py:76-82 repeats loss.backward(retain_graph=True): the state
+    the forward pass leaves behind must survive a backward pass."""
+    d = make_inputs(small_config(3, 90, 12, 40, ragged=True), seed=17)
+    dev = torch.device("cuda")
+    E = torch.tensor(d["emissions"], device=dev, requires_grad=True)
+    P = torch.tensor(d["predictions"], device=dev, requires_grad=True)
+    labels = torch.tensor(d["labels"], device=dev)
+    il = torch.tensor(d["input_lengths"], device=dev)
+    ll = torch.tensor(d["label_lengths"], device=dev)
+    loss = TransducerLoss()(E, P, labels, il, ll).sum()
+    loss.backward(retain_graph=True)
+    e1, p1 = E.grad.clone(), P.grad.clone()
+    E.grad = None
+    P.grad = None
+    loss.backward(retain_graph=True)
+    assert torch.equal(E.grad, e1) and torch.equal(P.grad, p1)
