@@ -46,7 +46,17 @@ WORKLOADS = {
     "cfg2": dict(B=8, T=2000, U=100, V=100, sigma=1.0, ragged_T=None, ragged_U=None),
     "cfg3a": dict(B=8, T=2000, U=100, V=1000, sigma=2.0, ragged_T=(1000, 2000), ragged_U=(50, 100)),
     "cfg3b": dict(B=8, T=2000, U=100, V=2000, sigma=2.0, ragged_T=(1000, 2000), ragged_U=(50, 100)),
+    # BASELINE configs[4]: teacher-forced best path (log-normaliser + max-plus + lattice + backtrace)
+    "cfg5": dict(B=32, T=2000, U=100, V=10000, sigma=1.0, ragged_T=(1500, 2000), ragged_U=(75, 100),
+                 kind="viterbi"),
+    "cfg5ties": dict(B=32, T=2000, U=100, V=10000, sigma=1.0, ragged_T=(1500, 2000),
+                     ragged_U=(75, 100), kind="viterbi", near_ties=True),
+    # the inputs of the reference's own benchmark script at the shape its README quotes 223.33 ms
+    # for on an A100 (benchmarks/torch_benchmarks.py:26-35: uniform [0,1) scores, full lengths)
+    "readme": dict(B=32, T=2000, U=100, V=10000, sigma=1.0, ragged_T=None, ragged_U=None,
+                   uniform=True, published_ms=223.33),
 }
+PEAK_VALU_TLANEOPS = 256 * 64 * 2.4e9 / 1e12  # 256 CUs x 64 fp32 lanes x 2.4 GHz, one op per lane
 
 
 def make_device_inputs(w, seed, device):
@@ -54,8 +64,14 @@ def make_device_inputs(w, seed, device):
     g = torch.Generator(device=device)
     g.manual_seed(seed)
     B, T, U, V = w["B"], w["T"], w["U"], w["V"]
-    E = torch.randn((B, T, V), generator=g, device=device, dtype=torch.float32) * w["sigma"]
-    P = torch.randn((B, U + 1, V), generator=g, device=device, dtype=torch.float32) * w["sigma"]
+    draw = torch.rand if w.get("uniform") else torch.randn
+    E = draw((B, T, V), generator=g, device=device, dtype=torch.float32) * w["sigma"]
+    P = draw((B, U + 1, V), generator=g, device=device, dtype=torch.float32) * w["sigma"]
+    if w.get("near_ties"):  # a tenth of every frame's entries repeat another column's value
+        for b in range(B):
+            dst = torch.randint(1, V, (T, V // 10), generator=g, device=device)
+            src = torch.randint(1, V, (T, V // 10), generator=g, device=device)
+            E[b].scatter_(1, dst, E[b].gather(1, src))
     labels = torch.randint(1, V, (B, U), generator=g, device=device, dtype=torch.int32)
     rng = np.random.Generator(np.random.Philox(key=seed))
     il = np.full(B, T, np.int32)
@@ -130,6 +146,59 @@ def cpu_baseline(w, il, ll, seconds_budget=15.0):
     return out
 
 
+def viterbi_main(args, w, capi, E, P, d_il, d_ll, il, ll):
+    """--workload cfg5: one step = rnnt_hip_viterbi_decode (log-normaliser, best label per cell,
+    best-path lattice, backtrace).  The dominant kernel is the max-plus scan, which has no
+    matrix form: it is priced in vector lane-operations (one add and one compare/select per
+    (t, u, v) of the valid lattice) against 256 CUs x 64 lanes x 2.4 GHz."""
+    import torch
+    B, T, U1, V = w["B"], w["T"], w["U"] + 1, w["V"]
+    out_labels = torch.empty((B, U1 - 1), dtype=torch.int32, device=E.device)
+    stream = ctypes.c_void_p(torch.cuda.current_stream(E.device).cuda_stream)
+    p = lambda t: ctypes.c_void_p(t.data_ptr())
+
+    def step():
+        capi.call("rnnt_hip_viterbi_decode", p(E), p(P), p(d_il), p(d_ll), p(out_labels), B, T, U1,
+                  V, 0, stream)
+
+    for _ in range(args.warmup):
+        step()
+        torch.cuda.synchronize()
+    capi.profile_enable(True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+        torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    stages = capi.profile_read()
+    capi.profile_enable(False)
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    per_launch = {k: (ms / n) for k, (ms, n) in stages.items() if n}
+    per_step = {k: round(ms / args.steps, 4) for k, (ms, n) in stages.items() if n}
+    cells = float(np.sum(il.astype(np.int64) * (ll.astype(np.int64) + 1)))
+    lane_ops = 2.0 * (V - 1) * cells
+    achieved = lane_ops / (per_launch["maxplus"] * 1e-3) / 1e12
+    out = {
+        "metric": "ms per teacher-forced viterbi decode, B=%d T=%d U=%d V=%d" % (B, T, w["U"], V),
+        "value": round(ms_per_step, 4), "unit": "ms", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": False,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "%s: B=%d T=%d U=%d V=%d blank=0, N(0,1) scores%s, input_lengths "
+                               "U[%d,%d], label_lengths U[%d,%d]"
+                               % ((args.workload, B, T, w["U"], V,
+                                   ", a tenth of each frame's entries duplicated"
+                                   if w.get("near_ties") else "") + w["ragged_T"] + w["ragged_U"]),
+                   "seed": args.seed, "valid_lattice_cells": int(cells)},
+        "roofline": {"bound": "valu", "kernel": "maxplus_kernel", "achieved": round(achieved, 2),
+                     "peak": round(PEAK_VALU_TLANEOPS, 2), "unit": "Tlane-op/s",
+                     "frac": round(achieved / PEAK_VALU_TLANEOPS, 4), "traffic": None,
+                     "kernel_ms": round(per_launch["maxplus"], 4), "lane_ops_per_launch": lane_ops},
+        "stage_ms_per_step": per_step,
+    }
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -157,6 +226,8 @@ def main():
     w = WORKLOADS[args.workload]
     B, T, U1, V = w["B"], w["T"], w["U"] + 1, w["V"]
     E, P, labels, d_il, d_ll, il, ll = make_device_inputs(w, args.seed, device)
+    if w.get("kind") == "viterbi":
+        return viterbi_main(args, w, capi, E, P, d_il, d_ll, il, ll)
     costs = torch.empty(B, device=device)
     egrads = torch.empty_like(E)
     pgrads = torch.empty_like(P)
@@ -212,16 +283,18 @@ def main():
         "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": False,
         "scaling": "weak",
-        "vs_baseline": None,
+        "vs_baseline": (round(ms_per_step / w["published_ms"], 5) if w.get("published_ms")
+                        else None),
         "dtype": "f32",
         "data": "synthetic",
-        "config": {"workload": "%s: B=%d T=%d U=%d V=%d blank=0, N(0,%g) scores, input_lengths "
+        "config": {"workload": "%s: B=%d T=%d U=%d V=%d blank=0, %s scores, input_lengths "
                                "%s, label_lengths %s, deltas=1" %
-                               (args.workload, B, T, w["U"], V, w["sigma"],
+                               (args.workload, B, T, w["U"], V,
+                                "uniform [0,1)" if w.get("uniform") else "N(0,%g)" % w["sigma"],
                                 "U[%d,%d]" % w["ragged_T"] if w["ragged_T"] else "=T",
                                 "U[%d,%d]" % w["ragged_U"] if w["ragged_U"] else "=U"),
                    "seed": args.seed, "valid_lattice_cells": int(cells)},
-        "roofline": {"bound": "mfma", "kernel": {"lse": "lse_fast_kernel",
+        "roofline": {"bound": "mfma", "kernel": {"lse": "lse_stream_kernel",
                                                  "egrads": "egrads_stream_kernel",
                                                  "pgrads": "pgrads_stream_kernel"}[dom],
                      "achieved": round(achieved, 2), "peak": PEAK_FP32_MATRIX_TFLOPS,

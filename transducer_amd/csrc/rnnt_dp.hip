@@ -509,91 +509,152 @@ __global__ __launch_bounds__(256) void sparse_p_kernel(Planes p, float* __restri
 
 // ------------------------------------------------------------------ max-plus table
 // best[t,u] = max over v != blank of E[t,v]+P[u,v], arg = lowest such v
-// (transducer/transducer_cpu.cpp:158-171).  A block owns 32 frames x 128 label positions and
-// streams the vocabulary in chunks of 32 through LDS; a thread owns 4x4 cells.  The running
-// maximum is exact and order-free; the index is recovered afterwards by rescanning only the
-// first chunk that reached the maximum, so the inner loop is one add and one max per term.
-constexpr int kMpT = 32, kMpU = 128, kMpK = 32;
+// (transducer/transducer_cpu.cpp:158-171).  Pure vector-ALU work (max-plus has no matrix form),
+// so the kernel is laid out to spend its instructions on the add and the max:
+//   * a workgroup of 16 wavefronts owns 128 frames x 128 label positions; a wavefront owns 8 label
+//     positions, a lane two frames (lane, lane+64): 16 cells per lane;
+//   * E and P stream through LDS in chunks of 32 columns (double-buffered, one barrier per
+//     chunk); E is staged with the blank column, columns past V and frames past the utterance at
+//     -inf; a lane reads its two rows of E 16 bytes at a time (row pitch 36 floats:
+//     conflict-free), and the P values of the wavefront's 8 rows, which are the same for all its
+//     lanes, with broadcast reads (one address per wavefront).  Scalar loads would bring them in
+//     as scalar operands, but they return out of order, so only one row could be in flight and
+//     the L2 latency of every row showed: measured 5.5 ms against 6.8 ms for a 4x4-cells
+//     LDS-tiled first version;
+//   * the running maximum is exact and order-free; per chunk a cell only notes whether the
+//     chunk raised it, and the index is recovered afterwards by rescanning the first chunk that
+//     reached the maximum.
+// Wavefronts whose label positions lie past the utterance only help staging.
+constexpr int kMpT = 128, kMpU = 128, kMpK = 32, kMpPitch = 36, kMpRows = 8;
 
-__global__ __launch_bounds__(256) void maxplus_kernel(const float* __restrict__ E,
-                                                      const float* __restrict__ P,
-                                                      const int* __restrict__ inLen,
-                                                      const int* __restrict__ labLen,
-                                                      float* __restrict__ best,
-                                                      int* __restrict__ arg, Dims d) {
-  __shared__ float Es[kMpT][kMpK + 1];
-  __shared__ float Ps[kMpU][kMpK + 1];
+// kVec: V is a multiple of 4, so every row of E starts on a 16-byte boundary.
+template <bool kVec>
+__global__ __launch_bounds__(1024) void maxplus_kernel(const float* __restrict__ E,
+                                                       const float* __restrict__ P,
+                                                       const int* __restrict__ inLen,
+                                                       const int* __restrict__ labLen,
+                                                       float* __restrict__ best,
+                                                       int* __restrict__ arg, Dims d) {
+  __shared__ __attribute__((aligned(16))) float Es[2][kMpT * kMpPitch];
+  __shared__ __attribute__((aligned(16))) float Ps[2][kMpU * kMpK];
   const int b = blockIdx.z, t0 = blockIdx.x * kMpT, u0 = blockIdx.y * kMpU;
   int Tb, Ub;
   utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
   if (t0 >= Tb || u0 >= Ub) return;
-  const int tid = threadIdx.x, tx = tid & 31, ty = tid >> 5;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const float* Eb = E + (size_t)b * d.T * d.V;
   const float* Pb = P + (size_t)b * d.U * d.V;
+  const int ur0 = u0 + wave * kMpRows;  // first label position of this wavefront
+  const bool active = ur0 < Ub;
 
-  float top[4][4];
-  int chunk[4][4];
+  // staging role: thread -> (row srow of the E tile and of the P tile, four columns from sc4)
+  const int srow = tid >> 3, sc4 = (tid & 7) * 4;
+  const bool srow_ok = t0 + srow < Tb;
+  const float* esrc = Eb + (size_t)min(t0 + srow, Tb - 1) * d.V;
+  const float* psrc = Pb + (size_t)min(u0 + srow, Ub - 1) * d.V;  // rows past the utterance are
+                                                                  // computed and dropped
+  // the raw values are requested before a chunk's arithmetic and stored after it, so the wait
+  // for them falls behind the arithmetic
+  auto fetch = [&](const float* src, int k) -> float4 {
+    const int v = k * kMpK + sc4;
+    float4 x;
+    if (kVec) {  // columns past V are re-read from the row's last four (E: masked below; P: any
+                 // finite value will do there, E is -inf)
+      x = *reinterpret_cast<const float4*>(src + min(v, d.V - 4));
+    } else {
+      x.x = src[min(v, d.V - 1)];
+      x.y = src[min(v + 1, d.V - 1)];
+      x.z = src[min(v + 2, d.V - 1)];
+      x.w = src[min(v + 3, d.V - 1)];
+    }
+    return x;
+  };
+  auto stash = [&](int buf, int k, float4 x, const float4& y) {
+    const int v = k * kMpK + sc4;
+    x.x = (srow_ok && v < d.V && v != d.blank) ? x.x : kNegInf;
+    x.y = (srow_ok && v + 1 < d.V && v + 1 != d.blank) ? x.y : kNegInf;
+    x.z = (srow_ok && v + 2 < d.V && v + 2 != d.blank) ? x.z : kNegInf;
+    x.w = (srow_ok && v + 3 < d.V && v + 3 != d.blank) ? x.w : kNegInf;
+    *reinterpret_cast<float4*>(&Es[buf][srow * kMpPitch + sc4]) = x;
+    *reinterpret_cast<float4*>(&Ps[buf][srow * kMpK + sc4]) = y;
+  };
+
+  float top[2][kMpRows];
+  int chunk[2][kMpRows];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < 2; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) { top[i][j] = kNegInf; chunk[i][j] = -1; }
+    for (int r = 0; r < kMpRows; ++r) { top[i][r] = kNegInf; chunk[i][r] = -1; }
 
   const int nchunks = (d.V + kMpK - 1) / kMpK;
+  int cur = 0;
+  stash(0, 0, fetch(esrc, 0), fetch(psrc, 0));
+  __syncthreads();
   for (int k = 0; k < nchunks; ++k) {
-    const int v0 = k * kMpK;
-    // stage: 32x32 of E and 128x32 of P; consecutive threads read consecutive v
-    for (int e = tid; e < kMpT * kMpK; e += 256) {
-      const int r = e / kMpK, c = e % kMpK, t = t0 + r, v = v0 + c;
-      Es[r][c] = (t < Tb && v < d.V && v != d.blank) ? Eb[(size_t)t * d.V + v] : kNegInf;
+    const int kn = min(k + 1, nchunks - 1);  // the last chunk re-reads its own
+    const float4 nxt = fetch(esrc, kn), nxp = fetch(psrc, kn);
+    if (active) {
+      float cm[2][kMpRows];
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int r = 0; r < kMpRows; ++r) cm[i][r] = kNegInf;
+#pragma unroll
+      for (int sub = 0; sub < kMpK / 8; ++sub) {
+        float e[2][8];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+          const float4 lo =
+              *reinterpret_cast<const float4*>(&Es[cur][(lane + 64 * i) * kMpPitch + sub * 8]);
+          const float4 hi =
+              *reinterpret_cast<const float4*>(&Es[cur][(lane + 64 * i) * kMpPitch + sub * 8 + 4]);
+          e[i][0] = lo.x; e[i][1] = lo.y; e[i][2] = lo.z; e[i][3] = lo.w;
+          e[i][4] = hi.x; e[i][5] = hi.y; e[i][6] = hi.z; e[i][7] = hi.w;
+        }
+        const float* pw = &Ps[cur][wave * kMpRows * kMpK + sub * 8];
+#pragma unroll
+        for (int r = 0; r < kMpRows; ++r) {
+          const float4 plo = *reinterpret_cast<const float4*>(pw + r * kMpK);
+          const float4 phi = *reinterpret_cast<const float4*>(pw + r * kMpK + 4);
+          const float pv[8] = {plo.x, plo.y, plo.z, plo.w, phi.x, phi.y, phi.z, phi.w};
+#pragma unroll
+          for (int c = 0; c < 8; c += 2) {
+            cm[0][r] = fmaxf(fmaxf(cm[0][r], e[0][c] + pv[c]), e[0][c + 1] + pv[c + 1]);
+            cm[1][r] = fmaxf(fmaxf(cm[1][r], e[1][c] + pv[c]), e[1][c + 1] + pv[c + 1]);
+          }
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int r = 0; r < kMpRows; ++r)
+          if (cm[i][r] > top[i][r]) { top[i][r] = cm[i][r]; chunk[i][r] = k; }
     }
-    for (int e = tid; e < kMpU * kMpK; e += 256) {
-      const int r = e / kMpK, c = e % kMpK, u = u0 + r, v = v0 + c;
-      Ps[r][c] = (u < Ub && v < d.V) ? Pb[(size_t)u * d.V + v] : kNegInf;
-    }
+    stash(cur ^ 1, kn, nxt, nxp);
     __syncthreads();
-    float cm[4][4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) cm[i][j] = kNegInf;
-#pragma unroll 8
-    for (int c = 0; c < kMpK; ++c) {
-      float ev[4], pv[4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) ev[i] = Es[ty * 4 + i][c];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) pv[j] = Ps[tx + 32 * j][c];
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) cm[i][j] = fmaxf(cm[i][j], ev[i] + pv[j]);
-    }
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-        if (cm[i][j] > top[i][j]) { top[i][j] = cm[i][j]; chunk[i][j] = k; }
-    __syncthreads();
+    cur ^= 1;
   }
+  if (!active) return;
   // recover the lowest index inside the winning chunk
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < 2; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int t = t0 + ty * 4 + i, u = u0 + tx + 32 * j;
+    for (int r = 0; r < kMpRows; ++r) {
+      const int t = t0 + lane + 64 * i, u = ur0 + r;
       if (t >= Tb || u >= Ub) continue;
       int at = 0;  // :160 the scan starts from index 0 and keeps it if nothing beats -inf
-      if (chunk[i][j] >= 0) {
-        const int v0 = chunk[i][j] * kMpK;
+      if (chunk[i][r] >= 0) {
+        const int v0 = chunk[i][r] * kMpK;
         const float* e = Eb + (size_t)t * d.V;
         const float* q = Pb + (size_t)u * d.V;
         for (int v = v0; v < v0 + kMpK && v < d.V; ++v) {
           if (v == d.blank) continue;
-          if (e[v] + q[v] == top[i][j]) { at = v; break; }
+          if (e[v] + q[v] == top[i][r]) { at = v; break; }
         }
       }
       const size_t o = ((size_t)b * d.T + t) * d.U + u;
-      best[o] = top[i][j];
+      best[o] = top[i][r];
       arg[o] = at;
     }
 }
@@ -839,8 +900,13 @@ int launch_sparse_p(const Planes& p, float* pgrads, const int* labels, const int
 int launch_maxplus(const float* E, const float* P, const int* inLen, const int* labLen,
                    float* best, int* arg, const Dims& d, hipStream_t s) {
   if (d.B == 0 || d.T == 0 || d.U == 0) return kOk;
-  hipLaunchKernelGGL(maxplus_kernel, dim3((d.T + kMpT - 1) / kMpT, (d.U + kMpU - 1) / kMpU, d.B),
-                     dim3(256), 0, s, E, P, inLen, labLen, best, arg, d);
+  const dim3 grid((d.T + kMpT - 1) / kMpT, (d.U + kMpU - 1) / kMpU, d.B);
+  if (d.V % 4 == 0)
+    hipLaunchKernelGGL(maxplus_kernel<true>, grid, dim3(1024), 0, s, E, P, inLen, labLen, best, arg,
+                       d);
+  else
+    hipLaunchKernelGGL(maxplus_kernel<false>, grid, dim3(1024), 0, s, E, P, inLen, labLen, best,
+                       arg, d);
   RNNT_LAUNCH_CHECK("maxplus_kernel");
   return kOk;
 }
