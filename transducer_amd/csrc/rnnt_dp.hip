@@ -682,14 +682,17 @@ __global__ __launch_bounds__(64) void viterbi_kernel(Planes p, const float* __re
   const int ngroups = (nsteps + 3) >> 2;
   unsigned long long* bits =
       kLdsBits ? lbits : gbits + (size_t)b * (size_t)(d.T + d.U + 4) * C;
-  const float* ebp = p.eb + (size_t)b * d.Tp + d.Eo;
+  const int u0 = lane * C;
+  // E[t,blank] for the cells of step s sits at ebl[s - u]; column c at step 4g+j reads
+  // ebl[4g + j - c], so one run of C+3 values serves all columns of a group
+  const float* ebl = p.eb + (size_t)b * d.Tp + d.Eo - u0;
 
   float stay[C], emit[C], pbv[C];
   const float* lnp[C];
   const float* bsp[C];
 #pragma unroll
   for (int c = 0; c < C; ++c) {
-    const int u = lane * C + c, uc = u < d.U ? u : d.U - 1;
+    const int u = u0 + c, uc = u < d.U ? u : d.U - 1;
     const size_t row = plane_row(d, b, uc);
     lnp[c] = p.lnS + row;
     bsp[c] = bestS + row;
@@ -697,57 +700,112 @@ __global__ __launch_bounds__(64) void viterbi_kernel(Planes p, const float* __re
     stay[c] = kNegInf;
     emit[c] = kNegInf;
   }
-  float4 ln4[C], bs4[C];
-  float eb4[C][4];
-  auto load_group = [&](int g, float4* ln, float4* bs, float (*ebv)[4]) {
+  struct Group {
+    float4 ln[C], bs[C];
+    float eb[C + 3];
+  };
+  auto load_group = [&](int g) -> Group {
+    Group r;
 #pragma unroll
     for (int c = 0; c < C; ++c) {
-      ln[c] = *reinterpret_cast<const float4*>(lnp[c] + 4 * g);
-      bs[c] = *reinterpret_cast<const float4*>(bsp[c] + 4 * g);
-      const int u = lane * C + c;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) ebv[c][j] = ebp[clampi(4 * g + j - u, 0, Tb - 1)];
+      r.ln[c] = *reinterpret_cast<const float4*>(lnp[c] + 4 * g);
+      r.bs[c] = *reinterpret_cast<const float4*>(bsp[c] + 4 * g);
     }
+#pragma unroll
+    for (int k = 0; k < C + 3; ++k) r.eb[k] = ebl[4 * g + k - (C - 1)];
+    return r;
   };
-  load_group(0, ln4, bs4, eb4);
-  for (int g = 0; g < ngroups; ++g) {
-    float4 ln4n[C], bs4n[C];
-    float eb4n[C][4];
-    load_group(g + 1 < ngroups ? g + 1 : g, ln4n, bs4n, eb4n);
+  // A cell that has not started (t < 0) keeps -inf scores and never takes a label; cells past
+  // the utterance run on whatever the planes hold and are never consulted by the backtrace.
+  auto run_group = [&](int g, const Group& cur) {
+    unsigned long long mw[4][C];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int s = 4 * g + j;
       const float from_left = wave_shr1(emit[C - 1], kNegInf);
 #pragma unroll
       for (int c = C - 1; c >= 0; --c) {
-        const int u = lane * C + c, t = s - u;
         const float left = (c == 0) ? from_left : emit[c - 1];
-        const bool active = (t >= 0) & (t < Tb) & (u < Ub);
-        const bool take = left > stay[c];
+        const bool take = left > stay[c];  // :200-206 ties go to blank
         float x = take ? left : stay[c];
-        x = (s == 0 && u == 0) ? 0.0f : x;
-        const unsigned long long m = __ballot(take);
-        if (lane == 0) bits[(size_t)s * C + c] = m;
-        const float ln = f4get(ln4[c], j);
-        float sb = x + eb4[c][j];
+        if (j == 0 && g == 0) x = (u0 + c == 0) ? 0.0f : x;
+        mw[j][c] = __ballot(take);
+        const float ln = f4get(cur.ln[c], j);
+        float sb = x + cur.eb[j - c + (C - 1)];
         sb = sb + pbv[c];
         sb = sb - ln;
-        float se = x + f4get(bs4[c], j);
+        float se = x + f4get(cur.bs[c], j);
         se = se - ln;
-        stay[c] = active ? sb : stay[c];
-        emit[c] = active ? se : emit[c];
+        const bool started = s >= u0 + c;
+        stay[c] = started ? sb : kNegInf;
+        emit[c] = started ? se : kNegInf;
       }
     }
+    if (lane == 0) {  // the group's ballots in one go: 4*C consecutive words
 #pragma unroll
-    for (int c = 0; c < C; ++c) {
-      ln4[c] = ln4n[c];
-      bs4[c] = bs4n[c];
+      for (int j = 0; j < 4; ++j)
 #pragma unroll
-      for (int j = 0; j < 4; ++j) eb4[c][j] = eb4n[c][j];
+        for (int c = 0; c < C; ++c) bits[(size_t)(4 * g + j) * C + c] = mw[j][c];
     }
+  };
+  // two register sets alternate (no copies): a group's loads are requested two groups ahead
+  auto clamp_g = [&](int g) { return g < ngroups ? g : ngroups - 1; };
+  Group x = load_group(0), y = load_group(clamp_g(1));
+  for (int g = 0; g < ngroups; g += 2) {
+    run_group(g, x);
+    x = load_group(clamp_g(g + 2));
+    if (g + 1 < ngroups) run_group(g + 1, y);
+    y = load_group(clamp_g(g + 3));
   }
   __syncthreads();
-  if (lane == 0) {
+  // Backtrace (:208-219).  Every move lowers t + u by one, so the words the walk will need are
+  // known ahead of the decisions: lane 0 keeps the next kAhead steps' ballots in registers and
+  // only notes, per label position, the step at which the label was taken; the labels
+  // themselves are fetched by all lanes afterwards (a fetch inside the walk would put a global
+  // round trip on every label).
+  int* taken = reinterpret_cast<int*>(kLdsBits ? lbits + (size_t)(d.T + d.U + 4) * C
+                                               : nullptr);  // [U] steps, -1 = not reached
+  constexpr int kAhead = 4;
+  if (kLdsBits) {
+    for (int u = lane; u < Ub; u += 64) taken[u] = -1;
+    __syncthreads();
+    if (lane == 0) {
+      int t = Tb - 1, u = Ub - 1, s = t + u;
+      unsigned long long w[kAhead][C];
+#pragma unroll
+      for (int i = 0; i < kAhead; ++i)
+#pragma unroll
+        for (int c = 0; c < C; ++c) w[i][c] = bits[(size_t)max(s - i, 0) * C + c];
+      bool done = !(u > 0 && t >= 0);
+      while (!done) {
+#pragma unroll
+        for (int i = 0; i < kAhead; ++i) {
+          if (!done) {
+            unsigned long long m = w[i][0];
+#pragma unroll
+            for (int c = 1; c < C; ++c) m = (u % C == c) ? w[i][c] : m;
+            if ((m >> (u / C)) & 1ull) {
+              taken[u - 1] = s;
+              u -= 1;
+            } else {
+              t -= 1;
+            }
+            s -= 1;
+            done = !(u > 0 && t >= 0);
+          }
+#pragma unroll
+          for (int c = 0; c < C; ++c) w[i][c] = bits[(size_t)max(s - kAhead + 1, 0) * C + c];
+        }
+      }
+    }
+    __syncthreads();
+    int* out = labels_out + (size_t)b * (d.U - 1);
+    const int* argI = reinterpret_cast<const int*>(argS);
+    for (int u1 = lane; u1 < Ub - 1; u1 += 64) {
+      const int st = taken[u1];
+      if (st >= 0) out[u1] = argI[plane_row(d, b, u1) + st - 1];
+    }
+  } else if (lane == 0) {
     int* out = labels_out + (size_t)b * (d.U - 1);
     const int* argI = reinterpret_cast<const int*>(argS);
     int t = Tb - 1, u = Ub - 1;
@@ -916,7 +974,8 @@ int launch_viterbi(const Planes& p, const float* bestS, const float* argS,
                    int* labels_out, const Dims& d, hipStream_t s) {
   if (d.B == 0 || d.T == 0 || d.U <= 1) return kOk;
   const int C = cells_per_lane(d.U);
-  const size_t lds = sizeof(unsigned long long) * (size_t)(d.T + d.U + 4) * C;
+  // the ballots of every step, then one int per label position for the backtrace
+  const size_t lds = sizeof(unsigned long long) * (size_t)(d.T + d.U + 4) * C + sizeof(int) * d.U;
   const bool use_lds = lds <= 60 * 1024;
   switch (C) {
 #define CASE(C)                                                                               \
