@@ -511,8 +511,10 @@ __global__ __launch_bounds__(256) void sparse_p_kernel(Planes p, float* __restri
 // best[t,u] = max over v != blank of E[t,v]+P[u,v], arg = lowest such v
 // (transducer/transducer_cpu.cpp:158-171).  Pure vector-ALU work (max-plus has no matrix form),
 // so the kernel is laid out to spend its instructions on the add and the max:
-//   * a workgroup of 16 wavefronts owns 128 frames x 128 label positions; a wavefront owns 8 label
-//     positions, a lane two frames (lane, lane+64): 16 cells per lane;
+//   * a workgroup of 8 wavefronts owns 128 frames x 64 label positions; a wavefront owns 8 label
+//     positions, a lane two frames (lane, lane+64): 16 cells per lane (two workgroups share a
+//     CU; with 16 wavefronts and 128 label positions per workgroup only one fits, and the
+//     wavefronts idling past a short utterance's last label cost a whole slot);
 //   * E and P stream through LDS in chunks of 32 columns (double-buffered, one barrier per
 //     chunk); E is staged with the blank column, columns past V and frames past the utterance at
 //     -inf; a lane reads its two rows of E 16 bytes at a time (row pitch 36 floats:
@@ -525,11 +527,13 @@ __global__ __launch_bounds__(256) void sparse_p_kernel(Planes p, float* __restri
 //     chunk raised it, and the index is recovered afterwards by rescanning the first chunk that
 //     reached the maximum.
 // Wavefronts whose label positions lie past the utterance only help staging.
-constexpr int kMpT = 128, kMpU = 128, kMpK = 32, kMpPitch = 36, kMpRows = 8;
+constexpr int kMpT = 128, kMpK = 32, kMpPitch = 36, kMpRows = 8;
+constexpr int kMpWaves = 8, kMpU = kMpWaves * kMpRows, kMpThreads = 64 * kMpWaves;
+constexpr int kMpEPasses = kMpT * (kMpK / 4) / kMpThreads;  // 16-byte pieces of the E chunk per thread
 
 // kVec: V is a multiple of 4, so every row of E starts on a 16-byte boundary.
 template <bool kVec>
-__global__ __launch_bounds__(1024) void maxplus_kernel(const float* __restrict__ E,
+__global__ __launch_bounds__(kMpThreads) void maxplus_kernel(const float* __restrict__ E,
                                                        const float* __restrict__ P,
                                                        const int* __restrict__ inLen,
                                                        const int* __restrict__ labLen,
@@ -548,10 +552,17 @@ __global__ __launch_bounds__(1024) void maxplus_kernel(const float* __restrict__
   const int ur0 = u0 + wave * kMpRows;  // first label position of this wavefront
   const bool active = ur0 < Ub;
 
-  // staging role: thread -> (row srow of the E tile and of the P tile, four columns from sc4)
+  // staging role: thread -> row srow of the P tile and rows srow + (kMpThreads/8) * i of the E
+  // tile, four columns from sc4
   const int srow = tid >> 3, sc4 = (tid & 7) * 4;
-  const bool srow_ok = t0 + srow < Tb;
-  const float* esrc = Eb + (size_t)min(t0 + srow, Tb - 1) * d.V;
+  const float* esrc[kMpEPasses];
+  bool erow_ok[kMpEPasses];
+#pragma unroll
+  for (int i = 0; i < kMpEPasses; ++i) {
+    const int t = t0 + srow + (kMpThreads / 8) * i;
+    erow_ok[i] = t < Tb;
+    esrc[i] = Eb + (size_t)min(t, Tb - 1) * d.V;
+  }
   const float* psrc = Pb + (size_t)min(u0 + srow, Ub - 1) * d.V;  // rows past the utterance are
                                                                   // computed and dropped
   // the raw values are requested before a chunk's arithmetic and stored after it, so the wait
@@ -570,14 +581,28 @@ __global__ __launch_bounds__(1024) void maxplus_kernel(const float* __restrict__
     }
     return x;
   };
-  auto stash = [&](int buf, int k, float4 x, const float4& y) {
+  struct Staged {
+    float4 e[kMpEPasses], p;
+  };
+  auto fetch_all = [&](int k) -> Staged {
+    Staged r;
+#pragma unroll
+    for (int i = 0; i < kMpEPasses; ++i) r.e[i] = fetch(esrc[i], k);
+    r.p = fetch(psrc, k);
+    return r;
+  };
+  auto stash = [&](int buf, int k, const Staged& r) {
     const int v = k * kMpK + sc4;
-    x.x = (srow_ok && v < d.V && v != d.blank) ? x.x : kNegInf;
-    x.y = (srow_ok && v + 1 < d.V && v + 1 != d.blank) ? x.y : kNegInf;
-    x.z = (srow_ok && v + 2 < d.V && v + 2 != d.blank) ? x.z : kNegInf;
-    x.w = (srow_ok && v + 3 < d.V && v + 3 != d.blank) ? x.w : kNegInf;
-    *reinterpret_cast<float4*>(&Es[buf][srow * kMpPitch + sc4]) = x;
-    *reinterpret_cast<float4*>(&Ps[buf][srow * kMpK + sc4]) = y;
+#pragma unroll
+    for (int i = 0; i < kMpEPasses; ++i) {
+      float4 x = r.e[i];
+      x.x = (erow_ok[i] && v < d.V && v != d.blank) ? x.x : kNegInf;
+      x.y = (erow_ok[i] && v + 1 < d.V && v + 1 != d.blank) ? x.y : kNegInf;
+      x.z = (erow_ok[i] && v + 2 < d.V && v + 2 != d.blank) ? x.z : kNegInf;
+      x.w = (erow_ok[i] && v + 3 < d.V && v + 3 != d.blank) ? x.w : kNegInf;
+      *reinterpret_cast<float4*>(&Es[buf][(srow + (kMpThreads / 8) * i) * kMpPitch + sc4]) = x;
+    }
+    *reinterpret_cast<float4*>(&Ps[buf][srow * kMpK + sc4]) = r.p;
   };
 
   float top[2][kMpRows];
@@ -589,11 +614,11 @@ __global__ __launch_bounds__(1024) void maxplus_kernel(const float* __restrict__
 
   const int nchunks = (d.V + kMpK - 1) / kMpK;
   int cur = 0;
-  stash(0, 0, fetch(esrc, 0), fetch(psrc, 0));
+  stash(0, 0, fetch_all(0));
   __syncthreads();
   for (int k = 0; k < nchunks; ++k) {
     const int kn = min(k + 1, nchunks - 1);  // the last chunk re-reads its own
-    const float4 nxt = fetch(esrc, kn), nxp = fetch(psrc, kn);
+    const Staged nxt = fetch_all(kn);
     if (active) {
       float cm[2][kMpRows];
 #pragma unroll
@@ -631,7 +656,7 @@ __global__ __launch_bounds__(1024) void maxplus_kernel(const float* __restrict__
         for (int r = 0; r < kMpRows; ++r)
           if (cm[i][r] > top[i][r]) { top[i][r] = cm[i][r]; chunk[i][r] = k; }
     }
-    stash(cur ^ 1, kn, nxt, nxp);
+    stash(cur ^ 1, kn, nxt);
     __syncthreads();
     cur ^= 1;
   }
@@ -960,11 +985,11 @@ int launch_maxplus(const float* E, const float* P, const int* inLen, const int* 
   if (d.B == 0 || d.T == 0 || d.U == 0) return kOk;
   const dim3 grid((d.T + kMpT - 1) / kMpT, (d.U + kMpU - 1) / kMpU, d.B);
   if (d.V % 4 == 0)
-    hipLaunchKernelGGL(maxplus_kernel<true>, grid, dim3(1024), 0, s, E, P, inLen, labLen, best, arg,
-                       d);
+    hipLaunchKernelGGL(maxplus_kernel<true>, grid, dim3(kMpThreads), 0, s, E, P, inLen, labLen,
+                       best, arg, d);
   else
-    hipLaunchKernelGGL(maxplus_kernel<false>, grid, dim3(1024), 0, s, E, P, inLen, labLen, best,
-                       arg, d);
+    hipLaunchKernelGGL(maxplus_kernel<false>, grid, dim3(kMpThreads), 0, s, E, P, inLen, labLen,
+                       best, arg, d);
   RNNT_LAUNCH_CHECK("maxplus_kernel");
   return kOk;
 }
