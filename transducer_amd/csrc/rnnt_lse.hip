@@ -46,6 +46,14 @@ constexpr float kLowest = -1.0e30f;  // stands in for a reference of -inf (a sla
 
 __device__ inline int mfma_row(int r, int h) { return 8 * (r >> 2) + 4 * h + (r & 3); }
 
+// Value of lane ^ 1 / lane ^ 2 within each group of four lanes: a DPP move, no LDS round trip.
+__device__ inline float quad_xor1(float x) {
+  return __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(x), 0xB1, 0xf, 0xf, true));
+}
+__device__ inline float quad_xor2(float x) {
+  return __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(x), 0x4E, 0xf, 0xf, true));
+}
+
 // 16-byte slot of (row, c8 = which eight of the slab's 32 v) inside a piece plane
 __device__ inline int xslot(int row, int c8) { return row * 4 + (c8 ^ ((row >> 2) & 3)); }
 
@@ -222,8 +230,8 @@ __global__ __launch_bounds__(64 * kWaves, kWaves / 2) void lse_stream_kernel(
       // maximum of the row's 32 values of this slab (values past V repeat earlier ones)
       float lm = fmaxf(fmaxf(fmaxf(r.lo[i].x, r.lo[i].y), fmaxf(r.lo[i].z, r.lo[i].w)),
                        fmaxf(fmaxf(r.hi[i].x, r.hi[i].y), fmaxf(r.hi[i].z, r.hi[i].w)));
-      lm = fmaxf(lm, __shfl_xor(lm, 1, 64));
-      lm = fmaxf(lm, __shfl_xor(lm, 2, 64));
+      lm = fmaxf(lm, quad_xor1(lm));  // the four threads of a row are one quad of lanes
+      lm = fmaxf(lm, quad_xor2(lm));
       lm = fmaxf(lm, kLowest);
       if (first) {
         mx[i] = lm;
@@ -273,43 +281,65 @@ __global__ __launch_bounds__(64 * kWaves, kWaves / 2) void lse_stream_kernel(
 
   const int nk = (d.V + kSlice - 1) / kSlice;
   int cur = 0;
-  // One slab: request the next slab and its two Y fragments (the last slice re-reads its own:
-  // no branch around the loads), multiply the current ones, stage the next.  Called with the
-  // two Y register sets swapped on alternate slabs, so no set is ever copied.
+  // One slab: request the next slab's emissions, multiply the current one, stage the next.
+  // Inside the matrix part the order is pinned with scheduling fences: the fragments of the
+  // second step are read from LDS while the first step is multiplied, each piece as soon as the
+  // first step's copy of it is no longer needed (so one set of fragment registers serves), and a
+  // step's Y fragments are re-requested for the next slab right after their last use (one set
+  // again).  Left to itself the compiler reads every fragment just before its first use and the
+  // matrix instructions wait for LDS one by one.
   struct YRegs { Frag3 s0, s1; };
-  auto step = [&](int s, const Frag3& y) {
-    uint4 ah[MB], am[MB], al[MB];
-#pragma unroll
-    for (int m = 0; m < MB; ++m) {
-      ah[m] = Xs[cur][0][aslot[s][m]];
-      am[m] = Xs[cur][1][aslot[s][m]];
-      al[m] = Xs[cur][2][aslot[s][m]];
-    }
-    // six piece products per block, smallest first; blocks interleaved so that consecutive
-    // instructions wait on each other's accumulator as little as possible
-#pragma unroll
-    for (int m = 0; m < MB; ++m) acc[m] = mfma_bf16(al[m], y.h, acc[m]);
-#pragma unroll
-    for (int m = 0; m < MB; ++m) acc[m] = mfma_bf16(ah[m], y.l, acc[m]);
-#pragma unroll
-    for (int m = 0; m < MB; ++m) acc[m] = mfma_bf16(am[m], y.m, acc[m]);
-#pragma unroll
-    for (int m = 0; m < MB; ++m) acc[m] = mfma_bf16(am[m], y.h, acc[m]);
-#pragma unroll
-    for (int m = 0; m < MB; ++m) acc[m] = mfma_bf16(ah[m], y.m, acc[m]);
-#pragma unroll
-    for (int m = 0; m < MB; ++m) acc[m] = mfma_bf16(ah[m], y.h, acc[m]);
-  };
-  auto slab = [&](int kt, const YRegs& yc, YRegs& yn) {
-    const XRegs xs = fetch(min(kt + 1, nk - 1) * kSlice);
+  auto slab = [&](int kt, YRegs& y) {
+    const int ktn = min(kt + 1, nk - 1);
+    const XRegs xs = fetch(ktn * kSlice);
     if (active) {
-      const int ktn = min(kt + 1, nk - 1);
-      yn.s0 = fetch_y(2 * ktn);
-      yn.s1 = fetch_y(2 * ktn + 1);
-    }
-    if (active) {
-      step(0, yc.s0);
-      step(1, yc.s1);
+      uint4 ah[MB], am[MB], al[MB];
+#pragma unroll
+      for (int m = 0; m < MB; ++m) al[m] = Xs[cur][2][aslot[0][m]];
+#pragma unroll
+      for (int m = 0; m < MB; ++m) ah[m] = Xs[cur][0][aslot[0][m]];
+#pragma unroll
+      for (int m = 0; m < MB; ++m) am[m] = Xs[cur][1][aslot[0][m]];
+      __builtin_amdgcn_sched_barrier(0);
+      // six piece products per block, smallest first; blocks interleaved so that consecutive
+      // instructions do not wait on each other's accumulator
+#pragma unroll
+      for (int m = 0; m < MB; ++m) acc[m] = mfma_bf16(al[m], y.s0.h, acc[m]);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int m = 0; m < MB; ++m) al[m] = Xs[cur][2][aslot[1][m]];
+#pragma unroll
+      for (int m = 0; m < MB; ++m) acc[m] = mfma_bf16(ah[m], y.s0.l, acc[m]);
+#pragma unroll
+      for (int m = 0; m < MB; ++m) acc[m] = mfma_bf16(am[m], y.s0.m, acc[m]);
+#pragma unroll
+      for (int m = 0; m < MB; ++m) acc[m] = mfma_bf16(am[m], y.s0.h, acc[m]);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int m = 0; m < MB; ++m) am[m] = Xs[cur][1][aslot[1][m]];
+#pragma unroll
+      for (int m = 0; m < MB; ++m) acc[m] = mfma_bf16(ah[m], y.s0.m, acc[m]);
+#pragma unroll
+      for (int m = 0; m < MB; ++m) acc[m] = mfma_bf16(ah[m], y.s0.h, acc[m]);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int m = 0; m < MB; ++m) ah[m] = Xs[cur][0][aslot[1][m]];
+      y.s0 = fetch_y(2 * ktn);
+#pragma unroll
+      for (int m = 0; m < MB; ++m) acc[m] = mfma_bf16(al[m], y.s1.h, acc[m]);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int m = 0; m < MB; ++m) acc[m] = mfma_bf16(ah[m], y.s1.l, acc[m]);
+#pragma unroll
+      for (int m = 0; m < MB; ++m) acc[m] = mfma_bf16(am[m], y.s1.m, acc[m]);
+#pragma unroll
+      for (int m = 0; m < MB; ++m) acc[m] = mfma_bf16(am[m], y.s1.h, acc[m]);
+#pragma unroll
+      for (int m = 0; m < MB; ++m) acc[m] = mfma_bf16(ah[m], y.s1.m, acc[m]);
+#pragma unroll
+      for (int m = 0; m < MB; ++m) acc[m] = mfma_bf16(ah[m], y.s1.h, acc[m]);
+      __builtin_amdgcn_sched_barrier(0);
+      y.s1 = fetch_y(2 * ktn + 1);
     }
     __builtin_amdgcn_sched_barrier(0);
     stash(cur ^ 1, xs, false, min(kt + 1, nk - 1));
@@ -335,16 +365,15 @@ __global__ __launch_bounds__(64 * kWaves, kWaves / 2) void lse_stream_kernel(
   __syncthreads();  // order
   if (npick > 0) next_slab = labs[order[0]] >> 5;
   stash(0, fetch(0), true, 0);
-  YRegs y0, y1;
+  YRegs y0;
   if (active) {
     y0.s0 = fetch_y(0);
     y0.s1 = fetch_y(1);
   }
   __syncthreads();
-  for (int kt = 0; kt < nk; kt += 2) {
-    slab(kt, y0, y1);
-    if (kt + 1 < nk) slab(kt + 1, y1, y0);
-    if (active && (kt + 2) % kFlush == 0) {
+  for (int kt = 0; kt < nk; ++kt) {
+    slab(kt, y0);
+    if (active && (kt + 1) % kFlush == 0) {
 #pragma unroll
       for (int m = 0; m < MB; ++m)
 #pragma unroll
