@@ -150,20 +150,40 @@ __global__ __launch_bounds__(256) void gather_kernel(const float* __restrict__ E
 // return the other operand untouched -- exactly the reference's first-row / first-column
 // special cases.  Cells past the utterance (t >= T_b, u >= U_b) are computed on whatever the
 // planes hold there and are never read by a valid cell.
-template <int C>
-__global__ __launch_bounds__(64) void alpha_kernel(Planes p, const int* __restrict__ inLen,
-                                                   const int* __restrict__ labLen,
-                                                   float* __restrict__ costs, Dims d) {
-  const int b = blockIdx.x, lane = threadIdx.x;
+// W > 1: the label positions are dealt to W wavefronts of one workgroup (wavefront w owns
+// positions [64 C w, 64 C (w+1))), because the walk is bound by how fast ONE wavefront issues
+// the ~22 instructions of a cell: a step costs about 30 + 65 C ns.  The only value that crosses
+// a wavefront boundary is the label-move score of the boundary cell, one float per step: the
+// lower wavefront leaves it in an LDS array indexed by step and then publishes how far it has
+// got; the upper one runs a few groups behind, so it finds its inputs there without waiting and
+// re-reads the progress counter only once every few groups.  The lowest
+// wavefront waits for nobody and every wavefront runs all groups, so the waits are bounded.
+template <int C, int W>
+__global__ __launch_bounds__(64 * W) void alpha_kernel(Planes p, const int* __restrict__ inLen,
+                                                       const int* __restrict__ labLen,
+                                                       float* __restrict__ costs, Dims d,
+                                                       int hand_stride) {
+  extern __shared__ __attribute__((aligned(16))) float hand[];  // [W-1][hand_stride]: entry s =
+                                                                // score handed to step s
+  __shared__ int done[W];          // steps a wavefront has published
+  const int b = blockIdx.x, lane = threadIdx.x & 63;
+  const int wave = W > 1 ? __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) : 0;
   int Tb, Ub;
   utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
   if (Tb == 0 || Ub == 0) {  // :39-41
-    if (lane == 0) costs[b] = kPosInf;
+    if (threadIdx.x == 0) costs[b] = kPosInf;
     return;
   }
   const int nsteps = Tb + Ub - 1;
   const int ngroups = (nsteps + 3) >> 2;
-  const int u0 = lane * C;
+  const int u0 = (wave * 64 + lane) * C;
+  if (W > 1) {
+    if (threadIdx.x < W) done[threadIdx.x] = 0;
+    if (threadIdx.x < W - 1) hand[threadIdx.x * hand_stride] = kNegInf;  // nothing enters step 0
+    __syncthreads();
+  }
+  float* hand_out = hand + wave * hand_stride;                     // wave < W-1
+  const float* hand_in = hand + (wave > 0 ? wave - 1 : 0) * hand_stride;  // wave > 0
   // E[t,blank] for the cells of step s sits at ebp[s - u]; column c at step s = 4g+j reads
   // ebl[4g + j - c], so one run of C+3 values serves all columns of a group
   const float* ebl = p.eb + (size_t)b * d.Tp + d.Eo - u0;
@@ -200,13 +220,31 @@ __global__ __launch_bounds__(64) void alpha_kernel(Planes p, const int* __restri
     return r;
   };
 
+  int avail = 0;  // steps the wavefront below is known to have published
+  auto wait_for = [&](int need) {
+    // LDS serves a wavefront's requests in order, so no hardware fence is needed on either
+    // side (a release/acquire pair would also wait for the global prefetches in flight);
+    // the empty asm statements only keep the compiler from moving LDS accesses across
+    while (avail < need) {
+      avail = __hip_atomic_load(&done[wave - 1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      asm volatile("" ::: "memory");
+      if (avail < need) __builtin_amdgcn_s_sleep(1);
+    }
+  };
   auto run_group = [&](int g, const Group& cur) {
     float4 aout[C];
+    float4 hin = {kNegInf, kNegInf, kNegInf, kNegInf};
+    if (W > 1 && wave > 0) {
+      wait_for(4 * g + 3);  // the scores entering steps 4g .. 4g+3 left steps 4g-1 .. 4g+2
+      hin = *reinterpret_cast<const float4*>(hand_in + 4 * g);
+    }
+    float hout[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int s = 4 * g + j;
       if (s < nsteps) {  // uniform; only the last group can be partial
-        const float from_left = wave_shr1(emit[C - 1], kNegInf);
+        float from_left = wave_shr1(emit[C - 1], kNegInf);
+        if (W > 1) from_left = (lane == 0) ? f4get(hin, j) : from_left;
 #pragma unroll
         for (int c = C - 1; c >= 0; --c) {
           const float left = (c == 0) ? from_left : emit[c - 1];
@@ -225,18 +263,33 @@ __global__ __launch_bounds__(64) void alpha_kernel(Planes p, const int* __restri
           f4set(aout[c], j, a);
         }
       }
+      if (W > 1)
+        hout[j] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(emit[C - 1]), 63));
     }
 #pragma unroll
     for (int c = 0; c < C; ++c) *reinterpret_cast<float4*>(ap[c] + 4 * g) = aout[c];
+    if (W > 1 && wave < W - 1 && lane == 0) {  // entries 4g+1 .. 4g+4, then the progress
+#pragma unroll
+      for (int j = 0; j < 4; ++j) hand_out[4 * g + 1 + j] = hout[j];
+      asm volatile("" ::: "memory");
+      __hip_atomic_store(&done[wave], 4 * g + 4, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
   };
-  // two register sets alternate (no copies): a group's loads are requested two groups ahead
+  // four register sets rotate (no copies): a group's loads are requested four groups (16
+  // steps, more than a microsecond) ahead -- the planes of a long batch do not fit L2
   auto clamp_g = [&](int g) { return g < ngroups ? g : ngroups - 1; };
-  Group x = load_group(0), y = load_group(clamp_g(1));
-  for (int g = 0; g < ngroups; g += 2) {
-    run_group(g, x);
-    x = load_group(clamp_g(g + 2));
-    if (g + 1 < ngroups) run_group(g + 1, y);
-    y = load_group(clamp_g(g + 3));
+  Group q0 = load_group(0), q1 = load_group(clamp_g(1)), q2 = load_group(clamp_g(2)),
+        q3 = load_group(clamp_g(3));
+  if (W > 1 && wave > 0) wait_for(min(4 * ngroups, 4 * 8 * wave));  // fall a few groups behind
+  for (int g = 0; g < ngroups; g += 4) {
+    run_group(g, q0);
+    q0 = load_group(clamp_g(g + 4));
+    if (g + 1 < ngroups) run_group(g + 1, q1);
+    q1 = load_group(clamp_g(g + 5));
+    if (g + 2 < ngroups) run_group(g + 2, q2);
+    q2 = load_group(clamp_g(g + 6));
+    if (g + 3 < ngroups) run_group(g + 3, q3);
+    q3 = load_group(clamp_g(g + 7));
   }
   // :73-78 the blank move out of the last cell, negated; that cell was the last one its
   // column processed
@@ -908,12 +961,22 @@ int launch_gather(const float* E, const float* P, const int* labels, const int* 
 int launch_alpha(const Planes& p, const int* inLen, const int* labLen, float* costs,
                  const Dims& d, hipStream_t s) {
   if (d.B == 0) return kOk;
-  switch (cells_per_lane(d.U)) {
-#define CASE(C)                                                                              \
-  case C:                                                                                    \
-    hipLaunchKernelGGL(alpha_kernel<C>, dim3(d.B), dim3(64), 0, s, p, inLen, labLen, costs, d); \
+  // cells per lane of a single wavefront; split over two wavefronts when the hand-over
+  // array (one float per step and boundary) fits LDS
+  const int cpl = cells_per_lane(d.U);
+  const int stride = ((d.T + d.U + 3) & ~3) + 8;
+  // (two wavefronts, not four: every lane reads its own plane row, 64 cache lines per load
+  // instruction, and with four wavefronts the CU's vector memory pipeline becomes the limit)
+  const int W = (cpl >= 2 && stride * sizeof(float) <= 48 * 1024) ? 2 : 1;
+  const size_t lds = W > 1 ? sizeof(float) * (size_t)(W - 1) * stride : 0;
+  switch (cpl / W * 100 + W) {
+#define CASE(C, W)                                                                          \
+  case C * 100 + W:                                                                         \
+    hipLaunchKernelGGL((alpha_kernel<C, W>), dim3(d.B), dim3(64 * W), lds, s, p, inLen,    \
+                       labLen, costs, d, stride);                                           \
     break;
-    CASE(1) CASE(2) CASE(4) CASE(8) CASE(16)
+    CASE(1, 1) CASE(2, 1) CASE(4, 1) CASE(8, 1) CASE(16, 1)
+    CASE(1, 2) CASE(2, 2) CASE(4, 2) CASE(8, 2)
 #undef CASE
     default:
       return fail(kInvalid, "prediction length %d exceeds the supported maximum of 1024", d.U);
