@@ -174,6 +174,20 @@ def test_viterbi_at_T2000_is_bit_exact(near_ties):
     assert np.array_equal(got, want)
 
 
+def test_viterbi_decision_table_in_global_memory():
+    """T large enough that the table of decision bits (and the hand-over array of the two
+    wavefronts) no longer fits LDS: the kernel's other code paths."""
+    cfg = small_config(2, 9000, 100, 12, ragged=True)
+    E, P, labels, il, ll = unpack(make_inputs(cfg, seed=33))
+    LN = oracle.log_norms_naive(E, P, il, ll)
+    want = oracle.viterbi(E, P, LN, il, ll)
+    c = DeviceCase(E, P, labels, il, ll)
+    assert np.array_equal(gpu_viterbi(c, LN), want)
+    costs_o, alphas_o = oracle.forward(E, P, LN, labels, il, ll)
+    costs, alphas = gpu_forward(c, LN)
+    assert_close(costs, costs_o, rtol=1e-4, atol=1e-2, what="costs")
+
+
 def test_viterbi_label_equal_to_nonzero_blank():
     cfg = small_config(2, 40, 12, 9, ragged=True)
     E, P, labels, il, ll = unpack(make_inputs(cfg, seed=4))

@@ -744,28 +744,54 @@ __global__ __launch_bounds__(kMpThreads) void maxplus_kernel(const float* __rest
 // (s + best) - LN (:197-199); "emit > stay" takes the label, ties go to blank (:200-206).
 // The decision of every cell is one bit; each step's 64-lane ballot goes to `bits`
 // (LDS when it fits, else global), and lane 0 walks them backwards at the end (:208-219).
-template <int C, bool kLdsBits>
-__global__ __launch_bounds__(64) void viterbi_kernel(Planes p, const float* __restrict__ bestS,
-                                                     const float* __restrict__ argS,
-                                                     const int* __restrict__ inLen,
-                                                     const int* __restrict__ labLen,
-                                                     unsigned long long* __restrict__ gbits,
-                                                     int* __restrict__ labels_out, Dims d) {
-  extern __shared__ unsigned long long lbits[];
-  const int b = blockIdx.x, lane = threadIdx.x;
+// C cells per lane, W wavefronts (the label positions dealt to them as in alpha_kernel, with
+// the same hand-over of the boundary score).
+// The decision of a cell is one bit.  A lane keeps the bits of its own cells, 32 steps to a
+// word, and stores a word when it is full: column u of the table `cols` holds the decisions of
+// label position u over all steps.  The backtrace then does not walk the ~T+U moves one by one:
+// at position u, reached at step s, the move that entered u is the highest set bit at or below
+// s in column u (everything above it is blank moves), found with one or two word reads and a
+// count-leading-zeros; U-1 such searches, by one lane, and the labels are fetched by all lanes
+// afterwards.
+// Dynamic LDS: one int per label position (steps at which labels were taken), the hand-over
+// array (W > 1), the columns (kLdsBits; else they live in global memory).
+template <int C, int W, bool kLdsBits>
+__global__ __launch_bounds__(64 * W) void viterbi_kernel(Planes p, const float* __restrict__ bestS,
+                                                         const float* __restrict__ argS,
+                                                         const int* __restrict__ inLen,
+                                                         const int* __restrict__ labLen,
+                                                         unsigned* __restrict__ gcols,
+                                                         int* __restrict__ labels_out, Dims d,
+                                                         int hand_stride, int nw) {
+  extern __shared__ __attribute__((aligned(16))) int dyn[];
+  __shared__ int done[W];  // steps a wavefront has published
+  const int b = blockIdx.x, lane = threadIdx.x & 63, tidx = threadIdx.x;
+  const int wave = W > 1 ? __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) : 0;
   int Tb, Ub;
   utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
   if (Tb == 0 || Ub == 0) return;  // :152-154
   const int nsteps = Tb + Ub - 1;
   const int ngroups = (nsteps + 3) >> 2;
-  unsigned long long* bits =
-      kLdsBits ? lbits : gbits + (size_t)b * (size_t)(d.T + d.U + 4) * C;
-  const int u0 = lane * C;
+  int* taken = dyn;                                                   // [U rounded up to 4]
+  float* hand = reinterpret_cast<float*>(dyn + ((d.U + 3) & ~3));     // [W-1][hand_stride]
+  unsigned* cols = kLdsBits
+      ? reinterpret_cast<unsigned*>(hand + (W - 1) * hand_stride)     // [64 C W][nw]
+      : gcols + (size_t)b * (64 * C * W) * nw;
+  if (W > 1) {
+    if (tidx < W) done[tidx] = 0;
+    if (tidx < W - 1) hand[tidx * hand_stride] = kNegInf;  // nothing enters step 0
+  }
+  for (int u = tidx; u < Ub; u += 64 * W) taken[u] = -1;
+  __syncthreads();
+  float* hand_out = hand + wave * hand_stride;                            // wave < W-1
+  const float* hand_in = hand + (wave > 0 ? wave - 1 : 0) * hand_stride;  // wave > 0
+  const int u0 = (wave * 64 + lane) * C;
   // E[t,blank] for the cells of step s sits at ebl[s - u]; column c at step 4g+j reads
   // ebl[4g + j - c], so one run of C+3 values serves all columns of a group
   const float* ebl = p.eb + (size_t)b * d.Tp + d.Eo - u0;
 
   float stay[C], emit[C], pbv[C];
+  unsigned wbits[C];
   const float* lnp[C];
   const float* bsp[C];
 #pragma unroll
@@ -777,6 +803,7 @@ __global__ __launch_bounds__(64) void viterbi_kernel(Planes p, const float* __re
     pbv[c] = p.pb[(size_t)b * d.Ua + uc];
     stay[c] = kNegInf;
     emit[c] = kNegInf;
+    wbits[c] = 0u;
   }
   struct Group {
     float4 ln[C], bs[C];
@@ -793,21 +820,36 @@ __global__ __launch_bounds__(64) void viterbi_kernel(Planes p, const float* __re
     for (int k = 0; k < C + 3; ++k) r.eb[k] = ebl[4 * g + k - (C - 1)];
     return r;
   };
+  int avail = 0;  // steps the wavefront below is known to have published (see alpha_kernel)
+  auto wait_for = [&](int need) {
+    while (avail < need) {
+      avail = __hip_atomic_load(&done[wave - 1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      asm volatile("" ::: "memory");
+      if (avail < need) __builtin_amdgcn_s_sleep(1);
+    }
+  };
   // A cell that has not started (t < 0) keeps -inf scores and never takes a label; cells past
   // the utterance run on whatever the planes hold and are never consulted by the backtrace.
   auto run_group = [&](int g, const Group& cur) {
-    unsigned long long mw[4][C];
+    float4 hin = {kNegInf, kNegInf, kNegInf, kNegInf};
+    if (W > 1 && wave > 0) {
+      wait_for(4 * g + 3);
+      hin = *reinterpret_cast<const float4*>(hand_in + 4 * g);
+    }
+    float hout[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int s = 4 * g + j;
-      const float from_left = wave_shr1(emit[C - 1], kNegInf);
+      const unsigned sbit = 1u << (s & 31);  // uniform
+      float from_left = wave_shr1(emit[C - 1], kNegInf);
+      if (W > 1) from_left = (lane == 0) ? f4get(hin, j) : from_left;
 #pragma unroll
       for (int c = C - 1; c >= 0; --c) {
         const float left = (c == 0) ? from_left : emit[c - 1];
         const bool take = left > stay[c];  // :200-206 ties go to blank
         float x = take ? left : stay[c];
         if (j == 0 && g == 0) x = (u0 + c == 0) ? 0.0f : x;
-        mw[j][c] = __ballot(take);
+        wbits[c] |= take ? sbit : 0u;
         const float ln = f4get(cur.ln[c], j);
         float sb = x + cur.eb[j - c + (C - 1)];
         sb = sb + pbv[c];
@@ -818,85 +860,64 @@ __global__ __launch_bounds__(64) void viterbi_kernel(Planes p, const float* __re
         stay[c] = started ? sb : kNegInf;
         emit[c] = started ? se : kNegInf;
       }
+      if (W > 1)
+        hout[j] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(emit[C - 1]), 63));
     }
-    if (lane == 0) {  // the group's ballots in one go: 4*C consecutive words
+    if ((g & 7) == 7 || g == ngroups - 1) {  // uniform: a word of 32 steps is complete
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
+      for (int c = 0; c < C; ++c) {
+        cols[(size_t)(u0 + c) * nw + (g >> 3)] = wbits[c];
+        wbits[c] = 0u;
+      }
+    }
+    if (W > 1 && wave < W - 1 && lane == 0) {  // entries 4g+1 .. 4g+4, then the progress
 #pragma unroll
-        for (int c = 0; c < C; ++c) bits[(size_t)(4 * g + j) * C + c] = mw[j][c];
+      for (int j = 0; j < 4; ++j) hand_out[4 * g + 1 + j] = hout[j];
+      asm volatile("" ::: "memory");
+      __hip_atomic_store(&done[wave], 4 * g + 4, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
   };
-  // two register sets alternate (no copies): a group's loads are requested two groups ahead
+  // four register sets rotate (no copies): a group's loads are requested four groups ahead
   auto clamp_g = [&](int g) { return g < ngroups ? g : ngroups - 1; };
-  Group x = load_group(0), y = load_group(clamp_g(1));
-  for (int g = 0; g < ngroups; g += 2) {
-    run_group(g, x);
-    x = load_group(clamp_g(g + 2));
-    if (g + 1 < ngroups) run_group(g + 1, y);
-    y = load_group(clamp_g(g + 3));
+  Group q0 = load_group(0), q1 = load_group(clamp_g(1)), q2 = load_group(clamp_g(2)),
+        q3 = load_group(clamp_g(3));
+  if (W > 1 && wave > 0) wait_for(min(4 * ngroups, 4 * 8 * wave));  // fall a few groups behind
+  for (int g = 0; g < ngroups; g += 4) {
+    run_group(g, q0);
+    q0 = load_group(clamp_g(g + 4));
+    if (g + 1 < ngroups) run_group(g + 1, q1);
+    q1 = load_group(clamp_g(g + 5));
+    if (g + 2 < ngroups) run_group(g + 2, q2);
+    q2 = load_group(clamp_g(g + 6));
+    if (g + 3 < ngroups) run_group(g + 3, q3);
+    q3 = load_group(clamp_g(g + 7));
+  }
+  if (!kLdsBits) __threadfence();  // the columns in global memory, before another lane reads them
+  __syncthreads();
+  // Backtrace (:208-219): from (T_b - 1, U_b - 1); a set bit at (step, u) means "entered from
+  // u - 1 with a label", a clear one "entered from t - 1 with a blank".
+  if (tidx == 0) {
+    int u = Ub - 1, s = nsteps - 1;
+    while (u > 0) {
+      int wi = s >> 5;
+      unsigned m = cols[(size_t)u * nw + wi] & (0xFFFFFFFFu >> (31 - (s & 31)));
+      while (m == 0u && wi > 0) {
+        --wi;
+        m = cols[(size_t)u * nw + wi];
+      }
+      if (m == 0u) break;  // ran out of frames: cannot happen on a lattice that was walked
+      const int st = 32 * wi + 31 - __clz(m);
+      taken[u - 1] = st;
+      u -= 1;
+      s = st - 1;
+    }
   }
   __syncthreads();
-  // Backtrace (:208-219).  Every move lowers t + u by one, so the words the walk will need are
-  // known ahead of the decisions: lane 0 keeps the next kAhead steps' ballots in registers and
-  // only notes, per label position, the step at which the label was taken; the labels
-  // themselves are fetched by all lanes afterwards (a fetch inside the walk would put a global
-  // round trip on every label).
-  int* taken = reinterpret_cast<int*>(kLdsBits ? lbits + (size_t)(d.T + d.U + 4) * C
-                                               : nullptr);  // [U] steps, -1 = not reached
-  constexpr int kAhead = 4;
-  if (kLdsBits) {
-    for (int u = lane; u < Ub; u += 64) taken[u] = -1;
-    __syncthreads();
-    if (lane == 0) {
-      int t = Tb - 1, u = Ub - 1, s = t + u;
-      unsigned long long w[kAhead][C];
-#pragma unroll
-      for (int i = 0; i < kAhead; ++i)
-#pragma unroll
-        for (int c = 0; c < C; ++c) w[i][c] = bits[(size_t)max(s - i, 0) * C + c];
-      bool done = !(u > 0 && t >= 0);
-      while (!done) {
-#pragma unroll
-        for (int i = 0; i < kAhead; ++i) {
-          if (!done) {
-            unsigned long long m = w[i][0];
-#pragma unroll
-            for (int c = 1; c < C; ++c) m = (u % C == c) ? w[i][c] : m;
-            if ((m >> (u / C)) & 1ull) {
-              taken[u - 1] = s;
-              u -= 1;
-            } else {
-              t -= 1;
-            }
-            s -= 1;
-            done = !(u > 0 && t >= 0);
-          }
-#pragma unroll
-          for (int c = 0; c < C; ++c) w[i][c] = bits[(size_t)max(s - kAhead + 1, 0) * C + c];
-        }
-      }
-    }
-    __syncthreads();
-    int* out = labels_out + (size_t)b * (d.U - 1);
-    const int* argI = reinterpret_cast<const int*>(argS);
-    for (int u1 = lane; u1 < Ub - 1; u1 += 64) {
-      const int st = taken[u1];
-      if (st >= 0) out[u1] = argI[plane_row(d, b, u1) + st - 1];
-    }
-  } else if (lane == 0) {
-    int* out = labels_out + (size_t)b * (d.U - 1);
-    const int* argI = reinterpret_cast<const int*>(argS);
-    int t = Tb - 1, u = Ub - 1;
-    while (u > 0 && t >= 0) {
-      const int s = t + u;
-      const unsigned long long m = bits[(size_t)s * C + (u % C)];
-      if ((m >> (u / C)) & 1ull) {
-        out[u - 1] = argI[plane_row(d, b, u - 1) + s - 1];
-        u -= 1;
-      } else {
-        t -= 1;
-      }
-    }
+  int* out = labels_out + (size_t)b * (d.U - 1);
+  const int* argI = reinterpret_cast<const int*>(argS);
+  for (int u1 = tidx; u1 < Ub - 1; u1 += 64 * W) {
+    const int st = taken[u1];
+    if (st >= 0) out[u1] = argI[plane_row(d, b, u1) + st - 1];
   }
 }
 
@@ -1057,25 +1078,37 @@ int launch_maxplus(const float* E, const float* P, const int* inLen, const int* 
   return kOk;
 }
 
+// 32-step words per column of the decision table (one spare)
+static int viterbi_words(const Dims& d) { return (d.T + d.U + 31) / 32 + 1; }
+
 int launch_viterbi(const Planes& p, const float* bestS, const float* argS,
                    unsigned long long* gbits, const int* inLen, const int* labLen,
                    int* labels_out, const Dims& d, hipStream_t s) {
   if (d.B == 0 || d.T == 0 || d.U <= 1) return kOk;
-  const int C = cells_per_lane(d.U);
-  // the ballots of every step, then one int per label position for the backtrace
-  const size_t lds = sizeof(unsigned long long) * (size_t)(d.T + d.U + 4) * C + sizeof(int) * d.U;
-  const bool use_lds = lds <= 60 * 1024;
-  switch (C) {
-#define CASE(C)                                                                               \
-  case C:                                                                                     \
-    if (use_lds)                                                                              \
-      hipLaunchKernelGGL((viterbi_kernel<C, true>), dim3(d.B), dim3(64), lds, s, p, bestS, argS, \
-                         inLen, labLen, gbits, labels_out, d);                                \
-    else                                                                                      \
-      hipLaunchKernelGGL((viterbi_kernel<C, false>), dim3(d.B), dim3(64), 0, s, p, bestS, argS,  \
-                         inLen, labLen, gbits, labels_out, d);                                \
+  unsigned* gcols = reinterpret_cast<unsigned*>(gbits);
+  const int cpl = cells_per_lane(d.U);
+  const int stride = ((d.T + d.U + 3) & ~3) + 8;
+  const int nw = viterbi_words(d);
+  const int W = (cpl >= 2 && stride * sizeof(float) <= 16 * 1024) ? 2 : 1;
+  // dynamic LDS: one int per label position, the hand-over array between the two wavefronts,
+  // and the decision columns when they fit
+  const size_t base_lds = sizeof(int) * (size_t)((d.U + 3) & ~3) +
+                          (W > 1 ? sizeof(float) * (size_t)(W - 1) * stride : 0);
+  const size_t cols_lds = sizeof(unsigned) * (size_t)64 * cpl * nw;
+  const bool use_lds = base_lds + cols_lds <= 60 * 1024;
+  const size_t lds = base_lds + (use_lds ? cols_lds : 0);
+  switch (cpl / W * 100 + W) {
+#define CASE(C, W)                                                                             \
+  case C * 100 + W:                                                                            \
+    if (use_lds)                                                                               \
+      hipLaunchKernelGGL((viterbi_kernel<C, W, true>), dim3(d.B), dim3(64 * W), lds, s, p,    \
+                         bestS, argS, inLen, labLen, gcols, labels_out, d, stride, nw);        \
+    else                                                                                       \
+      hipLaunchKernelGGL((viterbi_kernel<C, W, false>), dim3(d.B), dim3(64 * W), lds, s, p,   \
+                         bestS, argS, inLen, labLen, gcols, labels_out, d, stride, nw);        \
     break;
-    CASE(1) CASE(2) CASE(4) CASE(8) CASE(16)
+    CASE(1, 1) CASE(2, 1) CASE(4, 1) CASE(8, 1) CASE(16, 1)
+    CASE(1, 2) CASE(2, 2) CASE(4, 2) CASE(8, 2)
 #undef CASE
     default:
       return fail(kInvalid, "prediction length %d exceeds the supported maximum of 1024", d.U);
@@ -1085,7 +1118,7 @@ int launch_viterbi(const Planes& p, const float* bestS, const float* argS,
 }
 
 size_t viterbi_bits_bytes(const Dims& d) {
-  return sizeof(unsigned long long) * (size_t)d.B * (size_t)(d.T + d.U + 4) * cells_per_lane(d.U);
+  return sizeof(unsigned) * (size_t)d.B * 64 * cells_per_lane(d.U) * viterbi_words(d);
 }
 
 }  // namespace rnnt
