@@ -420,10 +420,10 @@ int rnnt_hip_loss_backward(const float* E, const float* P, const int* labels, co
   // The blank/label terms of egrads are folded into the dense kernel's write-out (a scatter
   // afterwards would touch one cache line of the 2.5 GB array per lattice cell); for label axes
   // too long for that kernel they are scattered as in rnnt_hip_backward.
-  // (folding pays when the array is large; with a small vocabulary many labels fall into one
-  // wavefront's 32 columns and their terms queue up in the dense kernel: B=8 V=100 0.17 ms folded,
-  // 0.03 + 0.04 ms scattered; even at V=2000)
-  const bool fold = egrads_fusion_supported(d) && labels != nullptr && d.V >= 1536;
+  // (not with a small vocabulary: many labels then fall into one wavefront's 32 columns and
+  // their terms queue up in the dense kernel -- B=8 V=100: 0.17 ms folded, 0.03 + 0.04 ms
+  // scattered; from V=1000 on folding is level or ahead)
+  const bool fold = egrads_fusion_supported(d) && labels != nullptr && d.V >= 512;
   SparseTerms sp;
   if (fold) {
     RNNT_STAGE(kSparse, launch_blank_sums(w.planes, w.bsum, labels, inLen, labLen, d, s));
