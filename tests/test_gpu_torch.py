@@ -154,3 +154,65 @@ def test_backward_twice_on_one_forward_gives_the_same_gradients():
     P.grad = None
     loss.backward(retain_graph=True)
     assert torch.equal(E.grad, e1) and torch.equal(P.grad, p1)
+
+
+def _small_problem(seed=23):
+    d = make_inputs(small_config(3, 150, 20, 260, ragged=True), seed=seed)
+    dev = torch.device("cuda")
+    return (torch.tensor(d["emissions"], device=dev), torch.tensor(d["predictions"], device=dev),
+            torch.tensor(d["labels"], device=dev), torch.tensor(d["input_lengths"], device=dev),
+            torch.tensor(d["label_lengths"], device=dev))
+
+
+def test_loss_on_a_side_stream_matches_the_default_stream():
+    """The C interface takes the stream to enqueue on (the reference is wired to stream 0,
+    transducer_cuda.cu:326-331); the torch front end passes torch's current stream."""
+    E, P, labels, il, ll = _small_problem()
+    E1, P1 = E.clone().requires_grad_(), P.clone().requires_grad_()
+    TransducerLoss()(E1, P1, labels, il, ll).sum().backward()
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()  # default priority
+    E2, P2 = E.clone().requires_grad_(), P.clone().requires_grad_()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        costs = TransducerLoss()(E2, P2, labels, il, ll)
+        costs.sum().backward()
+        paths = TransducerLoss().viterbi(E, P, il, ll)
+    side.synchronize()
+    assert torch.equal(E1.grad, E2.grad) and torch.equal(P1.grad, P2.grad)
+    assert torch.equal(paths, TransducerLoss().viterbi(E, P, il, ll))
+
+
+def test_fused_entry_points_replay_from_a_captured_graph():
+    """rnnt_hip_loss_forward / rnnt_hip_loss_backward allocate nothing and use kernels only, so
+    a caller may capture them; every replay (with eager work and synchronisation in between)
+    must reproduce the eager result bit for bit."""
+    import ctypes
+    from transducer_amd import capi
+    E, P, labels, il, ll = _small_problem(seed=29)
+    B, T, V = E.shape
+    U = P.shape[1]
+    p = lambda t: ctypes.c_void_p(t.data_ptr())
+    nbytes = capi.load().rnnt_hip_loss_workspace_bytes(B, T, U, V)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=E.device)
+    costs, eg, pg = torch.empty(B, device=E.device), torch.empty_like(E), torch.empty_like(P)
+
+    def run(stream):
+        capi.call("rnnt_hip_loss_forward", p(E), p(P), p(labels), p(il), p(ll), p(costs), p(ws),
+                  nbytes, B, T, U, V, 0, stream)
+        capi.call("rnnt_hip_loss_backward", p(E), p(P), p(labels), p(il), p(ll), None, p(eg), p(pg),
+                  p(ws), nbytes, B, T, U, V, 0, stream)
+
+    run(None)
+    torch.cuda.synchronize()
+    want = (costs.clone(), eg.clone(), pg.clone())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        run(ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    for _ in range(3):
+        costs.fill_(float("nan")); eg.fill_(float("nan")); pg.fill_(float("nan"))
+        ws.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(costs, want[0]) and torch.equal(eg, want[1]) and torch.equal(pg, want[2])
