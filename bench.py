@@ -55,6 +55,10 @@ WORKLOADS = {
     # for on an A100 (benchmarks/torch_benchmarks.py:26-35: uniform [0,1) scores, full lengths)
     "readme": dict(B=32, T=2000, U=100, V=10000, sigma=1.0, ragged_T=None, ragged_U=None,
                    uniform=True, published_ms=223.33),
+    # the headline shape with bf16 scores and gradients (rnnt_hip_loss_*_bf16; not a reference
+    # configuration: the reference takes float32 only)
+    "cfg4bf16": dict(B=32, T=2000, U=100, V=10000, sigma=1.0, ragged_T=(1500, 2000),
+                     ragged_U=(75, 100), io="bf16"),
 }
 PEAK_VALU_TLANEOPS = 256 * 64 * 2.4e9 / 1e12  # 256 CUs x 64 fp32 lanes x 2.4 GHz, one op per lane
 
@@ -228,6 +232,10 @@ def main():
     E, P, labels, d_il, d_ll, il, ll = make_device_inputs(w, args.seed, device)
     if w.get("kind") == "viterbi":
         return viterbi_main(args, w, capi, E, P, d_il, d_ll, il, ll)
+    bf16 = w.get("io") == "bf16"
+    if bf16:
+        E, P = E.to(torch.bfloat16), P.to(torch.bfloat16)
+    suffix, esize = ("_bf16", 2.0) if bf16 else ("", 4.0)
     costs = torch.empty(B, device=device)
     egrads = torch.empty_like(E)
     pgrads = torch.empty_like(P)
@@ -238,10 +246,10 @@ def main():
     p = lambda t: ctypes.c_void_p(t.data_ptr())
 
     def step():
-        capi.call("rnnt_hip_loss_forward", p(E), p(P), p(labels), p(d_il), p(d_ll), p(costs),
-                  p(ws), nbytes, B, T, U1, V, 0, stream)
-        capi.call("rnnt_hip_loss_backward", p(E), p(P), p(labels), p(d_il), p(d_ll), p(deltas),
-                  p(egrads), p(pgrads), p(ws), nbytes, B, T, U1, V, 0, stream)
+        capi.call("rnnt_hip_loss_forward" + suffix, p(E), p(P), p(labels), p(d_il), p(d_ll),
+                  p(costs), p(ws), nbytes, B, T, U1, V, 0, stream)
+        capi.call("rnnt_hip_loss_backward" + suffix, p(E), p(P), p(labels), p(d_il), p(d_ll),
+                  p(deltas), p(egrads), p(pgrads), p(ws), nbytes, B, T, U1, V, 0, stream)
 
     for _ in range(args.warmup):
         step()
@@ -270,11 +278,12 @@ def main():
     achieved = flops_one / (mfma_kernels[dom] * 1e-3) / 1e12
     flops_all = 3.0 * flops_one
     # bytes each contraction must move: valid rows of E and P in, its output out
-    in_bytes = 4.0 * V * (float(il.sum()) + float((ll + 1).sum()))
-    out_bytes = {"lse": 4.0 * B * T * U1, "egrads": 4.0 * B * T * V, "pgrads": 4.0 * B * U1 * V}
+    in_bytes = esize * V * (float(il.sum()) + float((ll + 1).sum()))
+    out_bytes = {"lse": 4.0 * B * T * U1, "egrads": esize * B * T * V,
+                 "pgrads": esize * B * U1 * V}
     hbm_gbs = (in_bytes + out_bytes[dom]) / (mfma_kernels[dom] * 1e-3) / 1e9
     out = {
-        "metric": METRIC,
+        "metric": METRIC + (" (bf16 scores and gradients)" if bf16 else ""),
         "value": round(ms_per_step, 4),
         "unit": "ms",
         "n_gpus": 1,
@@ -285,7 +294,7 @@ def main():
         "scaling": "weak",
         "vs_baseline": (round(ms_per_step / w["published_ms"], 5) if w.get("published_ms")
                         else None),
-        "dtype": "f32",
+        "dtype": "f32 arithmetic on bf16 scores, bf16 gradients" if bf16 else "f32",
         "data": "synthetic",
         "config": {"workload": "%s: B=%d T=%d U=%d V=%d blank=0, %s scores, input_lengths "
                                "%s, label_lengths %s, deltas=1" %
@@ -312,7 +321,7 @@ def main():
             (flops_all / (PEAK_FP32_MATRIX_TFLOPS * 1e12)) / (ms_per_step * 1e-3), 4),
         "stage_ms_per_step": per_step,
     }
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline and not bf16:  # the CPU path has no bf16 form
         out["cpu_baseline"] = cpu_baseline(w, il, ll)
     print(json.dumps(out))
 

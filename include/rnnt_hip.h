@@ -17,6 +17,7 @@
 #define RNNT_HIP_H_
 
 #include <stddef.h>
+#include <stdint.h>
 
 #ifdef __cplusplus
 extern "C" {
@@ -101,6 +102,25 @@ int rnnt_hip_loss_backward(const float* emissions, const float* predictions, con
                            const float* deltas, float* egrads, float* pgrads, void* workspace,
                            size_t workspace_bytes, int B, int T, int U, int V, int blank,
                            rnnt_stream_t stream);
+
+/* The same two calls for bf16 scores (the 16 high bits of an fp32, as torch.bfloat16 stores
+ * them) and bf16 gradients.  No counterpart in the reference, which refuses anything but
+ * float32 (transducer/torch_binding.py:195-201): this is for a caller whose projection layers
+ * emit bf16 logits, and it halves the traffic of the two [B,T,V] arrays.  A score converts to
+ * fp32 exactly and all arithmetic is the fp32 path's; each gradient element is the fp32 result
+ * (dense + blank/label terms, times deltas[b]) rounded once to nearest-even.  Shapes: V a
+ * multiple of 8, at most 112 label positions (U <= 112), 16-byte aligned score arrays; anything
+ * else is refused with an error.  Workspace as for the fp32 calls. */
+int rnnt_hip_loss_forward_bf16(const uint16_t* emissions, const uint16_t* predictions,
+                               const int* labels, const int* input_lengths,
+                               const int* label_lengths, float* costs, void* workspace,
+                               size_t workspace_bytes, int B, int T, int U, int V, int blank,
+                               rnnt_stream_t stream);
+int rnnt_hip_loss_backward_bf16(const uint16_t* emissions, const uint16_t* predictions,
+                                const int* labels, const int* input_lengths,
+                                const int* label_lengths, const float* deltas, uint16_t* egrads,
+                                uint16_t* pgrads, void* workspace, size_t workspace_bytes, int B,
+                                int T, int U, int V, int blank, rnnt_stream_t stream);
 
 /* Replaces TransducerLoss.viterbi (transducer/torch_binding.py:130-177): log-normaliser +
  * best path.  labels is int [B, U-1]. */

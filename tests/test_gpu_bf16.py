@@ -1,0 +1,248 @@
+"""bf16 scores and gradients through rnnt_hip_loss_forward_bf16 / rnnt_hip_loss_backward_bf16.
+
+The reference takes float32 only (transducer/torch_binding.py:195-201), so there is no reference
+output to match.  What pins these entry points:
+
+* a bf16 score converts to fp32 exactly, and the kernels are the fp32 ones with other loads and
+  stores, so the costs must EQUAL the fp32 entry points' costs on the upcast inputs, and each
+  gradient element must be the fp32 entry points' element rounded once to bf16 (allowing one bf16
+  unit where the two paths order an addition differently: the blank/label terms are always folded
+  into the dense kernels here, the fp32 path scatters them when the vocabulary is small);
+* against the CPU oracle on the upcast inputs the tolerance is the fp32 one plus half a unit of
+  bf16: |got - want| <= 1e-5 + (1e-4 + 2**-8) * |want|.
+"""
+import numpy as np
+import pytest
+
+from util import ATOL, RTOL, dev, ptr, violations
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+import oracle  # noqa: E402
+from transducer_amd import capi  # noqa: E402
+from transducer_amd.synthetic import CONFIGS  # noqa: E402
+
+BF16_RTOL = RTOL + 2.0 ** -8
+
+
+def draw(B, T, U, V, seed, sigma=1.0, ragged=True):
+    g = torch.Generator(device="cuda:0")
+    g.manual_seed(seed)
+    E = (torch.randn((B, T, V), generator=g, device="cuda:0") * sigma).to(torch.bfloat16)
+    P = (torch.randn((B, U, V), generator=g, device="cuda:0") * sigma).to(torch.bfloat16)
+    labels = torch.randint(1, V, (B, max(U - 1, 0)), generator=g, device="cuda:0",
+                           dtype=torch.int32)
+    rng = np.random.default_rng(seed)
+    il = np.full(B, T, np.int32)
+    ll = np.full(B, U - 1, np.int32)
+    if ragged and B > 1:
+        il[1:] = rng.integers(max(T // 2, 1), T + 1, B - 1)
+        ll[:-1] = rng.integers(0, U, B - 1)
+    return E, P, labels, il, ll
+
+
+def loss_bf16(E, P, labels, il, ll, deltas=None, blank=0):
+    B, T, V = E.shape
+    U = P.shape[1]
+    d_il, d_ll = dev(il), dev(ll)
+    nbytes = capi.load().rnnt_hip_loss_workspace_bytes(B, T, U, V)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device="cuda:0")
+    costs = torch.full((B,), float("nan"), device="cuda:0")
+    eg = torch.full_like(E, float("nan"))
+    pg = torch.full_like(P, float("nan"))
+    capi.call("rnnt_hip_loss_forward_bf16", ptr(E), ptr(P), ptr(labels), ptr(d_il), ptr(d_ll),
+              ptr(costs), ptr(ws), nbytes, B, T, U, V, blank, None)
+    capi.call("rnnt_hip_loss_backward_bf16", ptr(E), ptr(P), ptr(labels), ptr(d_il), ptr(d_ll),
+              ptr(deltas), ptr(eg), ptr(pg), ptr(ws), nbytes, B, T, U, V, blank, None)
+    torch.cuda.synchronize()
+    return costs, eg, pg
+
+
+def loss_fp32(E, P, labels, il, ll, deltas=None, blank=0):
+    """The fp32 entry points on the same values."""
+    E, P = E.float().contiguous(), P.float().contiguous()
+    B, T, V = E.shape
+    U = P.shape[1]
+    d_il, d_ll = dev(il), dev(ll)
+    nbytes = capi.load().rnnt_hip_loss_workspace_bytes(B, T, U, V)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device="cuda:0")
+    costs = torch.full((B,), float("nan"), device="cuda:0")
+    eg = torch.full_like(E, float("nan"))
+    pg = torch.full_like(P, float("nan"))
+    capi.call("rnnt_hip_loss_forward", ptr(E), ptr(P), ptr(labels), ptr(d_il), ptr(d_ll),
+              ptr(costs), ptr(ws), nbytes, B, T, U, V, blank, None)
+    capi.call("rnnt_hip_loss_backward", ptr(E), ptr(P), ptr(labels), ptr(d_il), ptr(d_ll),
+              ptr(deltas), ptr(eg), ptr(pg), ptr(ws), nbytes, B, T, U, V, blank, None)
+    torch.cuda.synchronize()
+    return costs, eg, pg
+
+
+def bf16_units_apart(got, want_fp32):
+    """|got - round_bf16(want)| in units of bf16 at want's magnitude, elementwise (device)."""
+    want = want_fp32.to(torch.bfloat16)
+    gi = got.view(torch.int16).to(torch.int32)
+    wi = want.view(torch.int16).to(torch.int32)
+    # sign-magnitude -> monotone integers
+    gi = torch.where(gi < 0, -(gi & 0x7FFF), gi)
+    wi = torch.where(wi < 0, -(wi & 0x7FFF), wi)
+    return (gi - wi).abs()
+
+
+def assert_rounds_the_fp32_result(got, want_fp32, what, exact_fraction):
+    assert got.dtype is torch.bfloat16
+    apart = bf16_units_apart(got, want_fp32)
+    # around zero one unit of the integer view is a denormal step: judge those by value
+    small = want_fp32.abs() < 1e-30
+    assert bool((got.float()[small].abs() < 1e-30).all())
+    apart = apart[~small]
+    worst = int(apart.max()) if apart.numel() else 0
+    same = float((apart == 0).float().mean()) if apart.numel() else 1.0
+    print("%s: %.5f%% of elements are the rounded fp32 result, worst %d unit(s)"
+          % (what, 100 * same, worst))
+    assert worst <= 1 and same >= exact_fraction
+
+
+SHAPES = [
+    # B, T, U, V
+    (1, 1, 1, 8),
+    (2, 5, 1, 16),
+    (3, 37, 9, 64),
+    (2, 64, 33, 128),
+    (4, 50, 11, 32),
+    (2, 130, 112, 520),
+    (3, 96, 20, 1000),
+]
+
+
+@pytest.mark.parametrize("B,T,U,V", SHAPES)
+def test_bf16_against_the_fp32_entry_points_and_the_oracle(B, T, U, V):
+    E, P, labels, il, ll = draw(B, T, U, V, seed=B * 1000 + T + U + V)
+    deltas = torch.linspace(0.5, 2.0, B, device="cuda:0")
+    costs, eg, pg = loss_bf16(E, P, labels, il, ll, deltas)
+    c32, e32, p32 = loss_fp32(E, P, labels, il, ll, deltas)
+    assert torch.equal(costs, c32)
+    assert_rounds_the_fp32_result(eg, e32, "egrads", 0.999)
+    assert_rounds_the_fp32_result(pg, p32, "pgrads", 0.999)
+    # padding is exact zero
+    for b in range(B):
+        assert not eg[b, il[b]:].any() and not pg[b, ll[b] + 1:].any()
+    want = oracle.loss_and_grads(E.float().cpu().numpy(), P.float().cpu().numpy(),
+                                 labels.cpu().numpy(), il, ll)
+    d = deltas.cpu().numpy()
+    ve, _ = violations(costs.cpu().numpy(), want["costs"])
+    assert ve == 0.0
+    for got, ref, what in ((eg, want["egrads"], "egrads"), (pg, want["pgrads"], "pgrads")):
+        ref = ref * d[:, None, None]
+        frac, worst = violations(got.float().cpu().numpy(), ref, rtol=BF16_RTOL, atol=ATOL)
+        assert frac == 0.0, "%s: %.4g%% outside rtol=%g atol=%g (max abs err %g)" % (
+            what, 100 * frac, BF16_RTOL, ATOL, worst)
+
+
+def test_bf16_blank_not_zero_and_repeated_labels():
+    B, T, U, V = 2, 40, 7, 24
+    E, P, labels, il, ll = draw(B, T, U, V, seed=11, ragged=False)
+    labels[:] = torch.tensor([[3, 3, 5, 5, 5, 0], [1, 1, 1, 2, 0, 0]], dtype=torch.int32)
+    blank = 4
+    costs, eg, pg = loss_bf16(E, P, labels, il, ll, blank=blank)
+    c32, e32, p32 = loss_fp32(E, P, labels, il, ll, blank=blank)
+    assert torch.equal(costs, c32)
+    assert_rounds_the_fp32_result(eg, e32, "egrads", 0.999)
+    assert_rounds_the_fp32_result(pg, p32, "pgrads", 0.999)
+    want = oracle.loss_and_grads(E.float().cpu().numpy(), P.float().cpu().numpy(),
+                                 labels.cpu().numpy(), il, ll, blank=blank)
+    for got, ref in ((eg, want["egrads"]), (pg, want["pgrads"])):
+        frac, _ = violations(got.float().cpu().numpy(), ref, rtol=BF16_RTOL, atol=ATOL)
+        assert frac == 0.0
+
+
+def test_bf16_empty_utterances_and_empty_batch():
+    B, T, U, V = 3, 12, 4, 16
+    E, P, labels, il, ll = draw(B, T, U, V, seed=5)
+    il[1] = 0   # no frames: cost +inf, zero gradients (transducer_cpu.cpp:39-41)
+    ll[2] = 0   # no labels
+    costs, eg, pg = loss_bf16(E, P, labels, il, ll)
+    c32, e32, p32 = loss_fp32(E, P, labels, il, ll)
+    assert torch.equal(costs, c32) and bool(torch.isinf(costs[1]))
+    assert not eg[1].any() and not pg[1].any()
+    assert_rounds_the_fp32_result(eg, e32, "egrads", 0.999)
+    assert_rounds_the_fp32_result(pg, p32, "pgrads", 0.999)
+    # B == 0 and T == 0 are legal and touch nothing / clear the outputs
+    capi.call("rnnt_hip_loss_forward_bf16", None, None, None, None, None, None, None, 0,
+              0, T, U, V, 0, None)
+    eg0 = torch.full((2, 0, V), 1.0, device="cuda:0", dtype=torch.bfloat16)
+    pg0 = torch.full((2, U, V), 1.0, device="cuda:0", dtype=torch.bfloat16)
+    d_il, d_ll = dev(np.zeros(2, np.int32)), dev(np.zeros(2, np.int32))
+    capi.call("rnnt_hip_loss_backward_bf16", None, None, None, ptr(d_il), ptr(d_ll), None,
+              ptr(eg0), ptr(pg0), None, 0, 2, 0, U, V, 0, None)
+    torch.cuda.synchronize()
+    assert not pg0.any()
+
+
+@pytest.mark.parametrize("B,T,U,V,needle", [
+    (1, 8, 3, 12, "multiple of 8"),
+    (1, 8, 3, 4, "multiple of 8"),
+    (1, 8, 113, 16, "112 label positions"),
+])
+def test_bf16_shapes_outside_the_streaming_kernels_are_refused(B, T, U, V, needle):
+    E = torch.zeros((B, T, V), device="cuda:0", dtype=torch.bfloat16)
+    P = torch.zeros((B, U, V), device="cuda:0", dtype=torch.bfloat16)
+    labels = torch.ones((B, U - 1), device="cuda:0", dtype=torch.int32)
+    il, ll = dev(np.full(B, T, np.int32)), dev(np.full(B, U - 1, np.int32))
+    nbytes = capi.load().rnnt_hip_loss_workspace_bytes(B, T, U, V)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device="cuda:0")
+    costs = torch.zeros((B,), device="cuda:0")
+    with pytest.raises(capi.RnntHipError, match=needle):
+        capi.call("rnnt_hip_loss_forward_bf16", ptr(E), ptr(P), ptr(labels), ptr(il), ptr(ll),
+                  ptr(costs), ptr(ws), nbytes, B, T, U, V, 0, None)
+    eg, pg = torch.zeros_like(E), torch.zeros_like(P)
+    with pytest.raises(capi.RnntHipError, match=needle):
+        capi.call("rnnt_hip_loss_backward_bf16", ptr(E), ptr(P), ptr(labels), ptr(il), ptr(ll),
+                  None, ptr(eg), ptr(pg), ptr(ws), nbytes, B, T, U, V, 0, None)
+
+
+def test_bf16_through_the_torch_module():
+    from transducer_amd import TransducerLoss
+    B, T, U, V = 3, 30, 6, 40
+    E, P, labels, il, ll = draw(B, T, U, V, seed=21)
+    d_il, d_ll = dev(il), dev(ll)
+    with pytest.raises(TypeError, match="emissions must be torch.float32"):
+        TransducerLoss()(E, P, labels, d_il, d_ll)  # the reference's behaviour stays the default
+    crit = TransducerLoss(allow_bf16=True)
+    with pytest.raises(TypeError, match="predictions must be torch.bfloat16"):
+        crit(E, P.float(), labels, d_il, d_ll)
+    Et, Pt = E.clone().requires_grad_(True), P.clone().requires_grad_(True)
+    costs = crit(Et, Pt, labels, d_il, d_ll)
+    assert costs.dtype is torch.float32
+    w = torch.linspace(1.0, 2.0, B, device="cuda:0")
+    (costs * w).sum().backward()
+    c, eg, pg = loss_bf16(E, P, labels, il, ll, w)
+    assert torch.equal(costs.detach(), c)
+    assert Et.grad.dtype is torch.bfloat16 and torch.equal(Et.grad, eg)
+    assert torch.equal(Pt.grad, pg)
+    # float32 tensors still take the fp32 path under allow_bf16
+    c32 = crit(E.float(), P.float(), labels, d_il, d_ll)
+    assert torch.equal(c32, c)
+
+
+def test_bf16_headline_configuration_against_the_fp32_path():
+    cfg = CONFIGS["cfg4"]
+    from transducer_amd.synthetic import lengths
+    g = torch.Generator(device="cuda:0")
+    g.manual_seed(17)
+    B, T, U, V = cfg.B, cfg.T, cfg.U + 1, cfg.V
+    E = torch.randn((B, T, V), generator=g, device="cuda:0").to(torch.bfloat16)
+    P = torch.randn((B, U, V), generator=g, device="cuda:0").to(torch.bfloat16)
+    labels = torch.randint(1, V, (B, U - 1), generator=g, device="cuda:0", dtype=torch.int32)
+    il, ll = lengths(cfg, np.random.Generator(np.random.Philox(key=17)))
+    costs, eg, pg = loss_bf16(E, P, labels, il, ll)
+    assert torch.isfinite(costs).all() and torch.isfinite(eg.float()).all()
+    d_il, d_ll = dev(il), dev(ll)
+    tmask = torch.arange(T, device="cuda:0")[None, :] >= d_il[:, None]
+    umask = torch.arange(U, device="cuda:0")[None, :] > d_ll[:, None]
+    assert not eg[tmask].any() and not pg[umask].any()
+    c32, e32, p32 = loss_fp32(E, P, labels, il, ll)
+    assert torch.equal(costs, c32)
+    # both paths fold the sparse terms of egrads at this vocabulary: the same fp32 value, rounded
+    assert torch.equal(eg, e32.to(torch.bfloat16))
+    assert_rounds_the_fp32_result(pg, p32, "pgrads", 0.9999)

@@ -356,7 +356,8 @@ int rnnt_hip_dense_grads(const float* E, const float* P, float* egrads, float* p
   RNNT_STAGE(kWplanes, launch_wplanes(lngrads, LN, mE, mP, Wn, Wt, inLen, labLen, d, s));
   RNNT_STAGE(kEgrads, launch_egrads(E, P, mE, mP, Wn, deltas, egrads, inLen, labLen, d, true,
                                     SparseTerms(), s));
-  RNNT_STAGE(kPgrads, launch_pgrads(E, P, mE, mP, Wt, deltas, pgrads, inLen, labLen, d, true, s));
+  RNNT_STAGE(kPgrads, launch_pgrads(E, P, mE, mP, Wt, deltas, pgrads, inLen, labLen, d, true,
+                                    SparsePTerms(), s));
   return kOk;
 }
 
@@ -431,11 +432,115 @@ int rnnt_hip_loss_backward(const float* E, const float* P, const int* labels, co
   }
   RNNT_STAGE(kEgrads, launch_egrads(E, P, w.mE, w.mP, w.Wn, deltas, egrads, inLen, labLen, d, false,
                                     sp, s));
-  RNNT_STAGE(kPgrads, launch_pgrads(E, P, w.mE, w.mP, w.Wt, deltas, pgrads, inLen, labLen, d, false, s));
-  if (fold)
-    RNNT_STAGE(kSparse, launch_sparse_p(w.planes, pgrads, labels, inLen, labLen, deltas, true, d, s));
-  else
+  // pgrads takes its blank / label totals in its write-out too (the same two fp32 operations
+  // the scatter kernel would do afterwards, so the same bits)
+  SparsePTerms spp;
+  if (fold) { spp.gB = w.planes.gB; spp.gL = w.planes.gL; spp.labels = labels; }
+  RNNT_STAGE(kPgrads, launch_pgrads(E, P, w.mE, w.mP, w.Wt, deltas, pgrads, inLen, labLen, d, false,
+                                    spp, s));
+  if (!fold)
     RNNT_STAGE(kSparse, launch_sparse(w.planes, egrads, pgrads, labels, inLen, labLen, deltas, true, d, s));
+  return kOk;
+}
+
+// bf16 scores: the shapes the streaming kernels take (every launcher below exists for both
+// element types; the general-shape fallbacks are fp32 only).
+static int check_bf16_shape(const void* E, const void* P, const Dims& d, const char* who) {
+  if (d.V % 8 != 0)
+    return fail(kInvalid, "%s: bf16 scores need a vocabulary that is a multiple of 8 (V=%d)", who,
+                d.V);
+  if ((reinterpret_cast<uintptr_t>(E) | reinterpret_cast<uintptr_t>(P)) & 15)
+    return fail(kInvalid, "%s: bf16 scores must be 16-byte aligned", who);
+  if (!egrads_stream_supported(d) || d.U > 128)
+    return fail(kInvalid, "%s: bf16 scores take at most 112 label positions (U=%d)", who, d.U);
+  if (!lse_stream_supported(static_cast<const bf16_t*>(E), d))
+    return fail(kInvalid, "%s: B*T*U too large for the bf16 path", who);
+  return kOk;
+}
+
+int rnnt_hip_loss_forward_bf16(const uint16_t* E16, const uint16_t* P16, const int* labels,
+                               const int* inLen, const int* labLen, float* costs, void* workspace,
+                               size_t workspace_bytes, int B, int T, int U, int V, int blank,
+                               rnnt_stream_t stream) {
+  RNNT_TRY(check_dims(B, T, U, V));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (B == 0) return kOk;
+  if (!costs || !inLen || !labLen)
+    return fail(kInvalid, "loss_forward_bf16: null costs or lengths");
+  if (nothing_to_do(B, T, U)) return fill(costs, __builtin_huge_valf(), B, s);
+  if (V == 0) return fail(kInvalid, "loss_forward_bf16: empty vocabulary");
+  if (!E16 || !P16 || (U > 1 && !labels))
+    return fail(kInvalid, "loss_forward_bf16: null array argument");
+  if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & 255))
+    return fail(kInvalid, "loss_forward_bf16: workspace must be a 256-byte aligned device pointer");
+  if (workspace_bytes < rnnt_hip_loss_workspace_bytes(B, T, U, V))
+    return fail(kWorkspace, "loss_forward_bf16: workspace of %zu bytes, %zu needed",
+                workspace_bytes, rnnt_hip_loss_workspace_bytes(B, T, U, V));
+  const Dims d = make_dims(B, T, U, V, blank);
+  RNNT_TRY(check_bf16_shape(E16, P16, d, "loss_forward_bf16"));
+  const bf16_t* E = reinterpret_cast<const bf16_t*>(E16);
+  const bf16_t* P = reinterpret_cast<const bf16_t*>(P16);
+  LossWorkspace w;
+  loss_workspace_layout(d, workspace, &w);
+  RNNT_STAGE(kRowmax, launch_rowmax_pick_p(P, w.mP, labels, labLen, w.planes, d, s));
+  RNNT_STAGE(kYplanes, launch_yplanes(P, w.mP, w.lse_scratch, labLen, d, s));
+  RNNT_STAGE(kLse, launch_lse_stream(E, w.mE, w.mP, w.LN, w.lse_scratch, inLen, labLen, d, s,
+                                     labels, w.planes.elS, w.planes.eb));
+  RNNT_STAGE(kSkew, launch_skew(w.LN, w.planes.lnS, inLen, labLen, d, s));
+  RNNT_STAGE(kAlpha, launch_alpha(w.planes, inLen, labLen, costs, d, s));
+  return kOk;
+}
+
+int rnnt_hip_loss_backward_bf16(const uint16_t* E16, const uint16_t* P16, const int* labels,
+                                const int* inLen, const int* labLen, const float* deltas,
+                                uint16_t* egrads16, uint16_t* pgrads16, void* workspace,
+                                size_t workspace_bytes, int B, int T, int U, int V, int blank,
+                                rnnt_stream_t stream) {
+  RNNT_TRY(check_dims(B, T, U, V));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (B == 0 || V == 0) return kOk;
+  if (nothing_to_do(B, T, U)) {
+    if (egrads16 && (size_t)T * V)
+      RNNT_HIP(hipMemsetAsync(egrads16, 0, sizeof(uint16_t) * (size_t)B * T * V, s));
+    if (pgrads16 && (size_t)U * V)
+      RNNT_HIP(hipMemsetAsync(pgrads16, 0, sizeof(uint16_t) * (size_t)B * U * V, s));
+    return kOk;
+  }
+  if (!E16 || !P16 || !egrads16 || !pgrads16 || !inLen || !labLen || (U > 1 && !labels))
+    return fail(kInvalid, "loss_backward_bf16: null array argument");
+  if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & 255))
+    return fail(kInvalid, "loss_backward_bf16: workspace must be a 256-byte aligned device pointer");
+  if (workspace_bytes < rnnt_hip_loss_workspace_bytes(B, T, U, V))
+    return fail(kWorkspace, "loss_backward_bf16: workspace of %zu bytes, %zu needed",
+                workspace_bytes, rnnt_hip_loss_workspace_bytes(B, T, U, V));
+  const Dims d = make_dims(B, T, U, V, blank);
+  RNNT_TRY(check_bf16_shape(E16, P16, d, "loss_backward_bf16"));
+  if ((reinterpret_cast<uintptr_t>(egrads16) | reinterpret_cast<uintptr_t>(pgrads16)) & 1)
+    return fail(kInvalid, "loss_backward_bf16: misaligned gradient arrays");
+  const bf16_t* E = reinterpret_cast<const bf16_t*>(E16);
+  const bf16_t* P = reinterpret_cast<const bf16_t*>(P16);
+  LossWorkspace w;
+  loss_workspace_layout(d, workspace, &w);
+  RNNT_STAGE(kWeights, launch_weights(w.planes, inLen, labLen, d, s));
+  RNNT_STAGE(kBeta, launch_beta(w.planes, labels, inLen, labLen, d, s));
+  RNNT_STAGE(kUnskew, launch_unskew(w.planes.dS, w.lngrads, inLen, labLen, d, s));
+  RNNT_STAGE(kWplanes, launch_wplanes(w.lngrads, w.LN, w.mE, w.mP, w.Wn, w.Wt, inLen, labLen, d, s));
+  // Both gradients are rounded to bf16 once, from the complete fp32 value: the blank / label
+  // terms are always folded into the dense kernels' write-outs here, whatever the vocabulary.
+  // With U == 1 there are no labels; the kernels then never read the list, but its pointer is
+  // what switches the folding on, so any valid device pointer serves.
+  const int* lab = labels ? labels : inLen;
+  RNNT_STAGE(kSparse, launch_blank_sums(w.planes, w.bsum, lab, inLen, labLen, d, s));
+  SparseTerms sp;
+  sp.dS = w.planes.dS; sp.wE = w.planes.wE; sp.bsum = w.bsum; sp.labels = lab;
+  SparsePTerms spp;
+  spp.gB = w.planes.gB; spp.gL = w.planes.gL; spp.labels = lab;
+  RNNT_STAGE(kEgrads, launch_egrads_stream(E, P, w.mE, w.mP, w.Wn, deltas,
+                                           reinterpret_cast<bf16_t*>(egrads16), inLen, labLen, d,
+                                           false, sp, s));
+  RNNT_STAGE(kPgrads, launch_pgrads_stream(E, P, w.mE, w.mP, w.Wt, deltas,
+                                           reinterpret_cast<bf16_t*>(pgrads16), inLen, labLen, d,
+                                           false, spp, s));
   return kOk;
 }
 

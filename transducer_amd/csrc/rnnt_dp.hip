@@ -1054,16 +1054,6 @@ int launch_blank_sums(const Planes& p, float* bsum, const int* labels, const int
   return kOk;
 }
 
-int launch_sparse_p(const Planes& p, float* pgrads, const int* labels, const int* inLen,
-                    const int* labLen, const float* scale, bool add, const Dims& d,
-                    hipStream_t s) {
-  if (d.B == 0 || d.T == 0 || d.U == 0) return kOk;
-  hipLaunchKernelGGL(sparse_p_kernel, dim3((d.U + 255) / 256, d.B), dim3(256), 0, s, p, pgrads,
-                     labels, inLen, labLen, scale, add ? 1 : 0, d);
-  RNNT_LAUNCH_CHECK("sparse_p_kernel");
-  return kOk;
-}
-
 int launch_maxplus(const float* E, const float* P, const int* inLen, const int* labLen,
                    float* best, int* arg, const Dims& d, hipStream_t s) {
   if (d.B == 0 || d.T == 0 || d.U == 0) return kOk;

@@ -31,6 +31,22 @@ __device__ inline float wave_max(float m) {
 }
 
 // ------------------------------------------------------------------ row maxima
+// bf16 rows (V % 8 == 0 and 16-byte aligned when vec is set): eight elements per load.
+__device__ inline float row_max(const bf16_t* __restrict__ x, int V, int vec, int lane) {
+  float m0 = kNegInf, m1 = kNegInf;
+  if (vec) {
+    for (int i = lane; i < (V >> 3); i += 64) {
+      float e[8];
+      expand(load8(x, 8 * i, V), e);
+      m0 = fmaxf(m0, fmaxf(fmaxf(e[0], e[1]), fmaxf(e[2], e[3])));
+      m1 = fmaxf(m1, fmaxf(fmaxf(e[4], e[5]), fmaxf(e[6], e[7])));
+    }
+  } else {
+    for (int i = lane; i < V; i += 64) m0 = fmaxf(m0, ldf(x + i));
+  }
+  return wave_max(fmaxf(m0, m1));
+}
+
 // One wavefront per row of a [rows, V] array.
 // rows_per_item / lengths (optional): row r belongs to item r / rows_per_item and is skipped
 // (maximum reported as 0, nothing read) when its index inside the item is >= lengths[item] + extra.
@@ -147,7 +163,8 @@ __global__ __launch_bounds__(256) void rowmax_pick_e_kernel(const float* __restr
 }
 
 // The same for the predictions: P[u, blank] and P[u, label_u].
-__global__ __launch_bounds__(256) void rowmax_pick_p_kernel(const float* __restrict__ P,
+template <typename TIO>
+__global__ __launch_bounds__(256) void rowmax_pick_p_kernel(const TIO* __restrict__ P,
                                                             float* __restrict__ mP,
                                                             const int* __restrict__ labels,
                                                             const int* __restrict__ labLen,
@@ -161,13 +178,13 @@ __global__ __launch_bounds__(256) void rowmax_pick_p_kernel(const float* __restr
     if (lane == 0) mP[row] = 0.0f;
     return;
   }
-  const float* x = P + (size_t)row * d.V;
+  const TIO* x = P + (size_t)row * d.V;
   const float m = row_max(x, d.V, vec4, lane);
   if (lane == 0) {
     mP[row] = m;
     const bool has_label = labels != nullptr && (u + 1 < Ub);
-    p.pb[(size_t)b * d.Ua + u] = x[d.blank];
-    p.pl[(size_t)b * d.Ua + u] = has_label ? x[labels[(size_t)b * (d.U - 1) + u]] : 0.0f;
+    p.pb[(size_t)b * d.Ua + u] = ldf(x + d.blank);
+    p.pl[(size_t)b * d.Ua + u] = has_label ? ldf(x + labels[(size_t)b * (d.U - 1) + u]) : 0.0f;
   }
 }
 
@@ -445,20 +462,29 @@ int launch_rowmax_pick(const float* E, const float* P, float* mE, float* mP, con
   hipLaunchKernelGGL(rowmax_pick_e_kernel, dim3((d.T + kPickRows - 1) / kPickRows, d.B), dim3(256),
                      0, s, E, mE, labels, inLen, labLen, p, d, ve);
   RNNT_LAUNCH_CHECK("rowmax_pick_e_kernel");
-  hipLaunchKernelGGL(rowmax_pick_p_kernel, dim3((unsigned)(((long)d.B * d.U + 3) / 4)), dim3(256),
-                     0, s, P, mP, labels, labLen, p, d, vp);
+  hipLaunchKernelGGL(rowmax_pick_p_kernel<float>, dim3((unsigned)(((long)d.B * d.U + 3) / 4)),
+                     dim3(256), 0, s, P, mP, labels, labLen, p, d, vp);
   RNNT_LAUNCH_CHECK("rowmax_pick_p_kernel");
   return kOk;
 }
 
-int launch_rowmax_pick_p(const float* P, float* mP, const int* labels, const int* labLen,
-                         const Planes& p, const Dims& d, hipStream_t s) {
+template <typename TIO>
+static int rowmax_pick_p_any(const TIO* P, float* mP, const int* labels, const int* labLen,
+                             const Planes& p, const Dims& d, hipStream_t s) {
   if (d.B == 0 || d.U == 0) return kOk;
-  const int vp = (d.V % 4 == 0) && ((reinterpret_cast<uintptr_t>(P) & 15) == 0);
-  hipLaunchKernelGGL(rowmax_pick_p_kernel, dim3((unsigned)(((long)d.B * d.U + 3) / 4)), dim3(256),
-                     0, s, P, mP, labels, labLen, p, d, vp);
+  const int vp = (d.V % RowAlign<TIO>::kElems == 0) && ((reinterpret_cast<uintptr_t>(P) & 15) == 0);
+  hipLaunchKernelGGL(rowmax_pick_p_kernel<TIO>, dim3((unsigned)(((long)d.B * d.U + 3) / 4)),
+                     dim3(256), 0, s, P, mP, labels, labLen, p, d, vp);
   RNNT_LAUNCH_CHECK("rowmax_pick_p_kernel");
   return kOk;
+}
+int launch_rowmax_pick_p(const float* P, float* mP, const int* labels, const int* labLen,
+                         const Planes& p, const Dims& d, hipStream_t s) {
+  return rowmax_pick_p_any(P, mP, labels, labLen, p, d, s);
+}
+int launch_rowmax_pick_p(const bf16_t* P, float* mP, const int* labels, const int* labLen,
+                         const Planes& p, const Dims& d, hipStream_t s) {
+  return rowmax_pick_p_any(P, mP, labels, labLen, p, d, s);
 }
 
 int launch_lse(const float* E, const float* P, const float* mE, const float* mP, float* LN,
@@ -509,9 +535,11 @@ int launch_egrads(const float* E, const float* P, const float* mE, const float* 
 
 int launch_pgrads(const float* E, const float* P, const float* mE, const float* mP,
                   const float* Wt, const float* deltas, float* pgrads, const int* inLen,
-                  const int* labLen, const Dims& d, bool accumulate, hipStream_t s) {
+                  const int* labLen, const Dims& d, bool accumulate, const SparsePTerms& sparse,
+                  hipStream_t s) {
   if (d.B == 0 || d.T == 0 || d.U == 0) return kOk;
-  return launch_pgrads_stream(E, P, mE, mP, Wt, deltas, pgrads, inLen, labLen, d, accumulate, s);
+  return launch_pgrads_stream(E, P, mE, mP, Wt, deltas, pgrads, inLen, labLen, d, accumulate,
+                              sparse, s);
 }
 
 }  // namespace rnnt

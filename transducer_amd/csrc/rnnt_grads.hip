@@ -17,6 +17,7 @@
 // v_mfma_f32_32x32x16_bf16 takes, per lane, eight consecutive k of its row (A) or column (B):
 // k = 8*(lane/32) + i.  A lane reads them with one 16-byte LDS load per piece.
 #include "rnnt_internal.h"
+#include "rnnt_io.h"
 #include "rnnt_split.h"
 
 namespace rnnt {
@@ -24,6 +25,7 @@ namespace rnnt {
 namespace {
 
 constexpr float kNegInf = -__builtin_huge_valf();
+
 
 __device__ inline float f4at(const float4& v, int q) {
   return q == 0 ? v.x : (q == 1 ? v.y : (q == 2 ? v.z : v.w));
@@ -48,11 +50,11 @@ struct SlabRegs {
 // (a template parameter, so the matrix instructions of a tile form one straight-line block).
 // Label positions past the utterance contribute exact zeros: their Y rows are masked and the
 // W slab is zero there.
-template <int NS, bool kAccumulate>
+template <int NS, bool kAccumulate, typename TIO>
 __device__ __forceinline__ void egrads_walk(
-    const float* __restrict__ E, const float* __restrict__ P, const float* __restrict__ mE,
+    const TIO* __restrict__ E, const TIO* __restrict__ P, const float* __restrict__ mE,
     const float* __restrict__ mP, const float* __restrict__ Wn, const float* __restrict__ deltas,
-    float* __restrict__ egrads, unsigned short (*As)[3][kEsPlane], float (*Ms)[32], const Dims& d,
+    TIO* __restrict__ egrads, unsigned short (*As)[3][kEsPlane], float (*Ms)[32], const Dims& d,
     int Up, int Tw, int tiles_per_chunk, int b, int Tb, int Ub, const SparseTerms& sp,
     const unsigned short* match, int nmatch, float (*Sp)[32]) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, h = lane >> 5;
@@ -69,15 +71,15 @@ __device__ __forceinline__ void egrads_walk(
   const int tile_hi = min(tile_lo + tiles_per_chunk, ntiles);
   const int tile_valid = min(tile_hi, (Tb + 31) >> 5);  // tiles that hold frames of the utterance
   const float delta = deltas ? deltas[b] : 1.0f;
-  const float* Eb = E + (size_t)b * d.T * d.V;
-  float* out = egrads + (size_t)b * d.T * d.V;
+  const TIO* Eb = E + (size_t)b * d.T * d.V;
+  TIO* out = egrads + (size_t)b * d.T * d.V;
   const float* mEb = mE + (size_t)b * d.T;
 
   // Y fragments for this wavefront's columns (branch-free: clamped address, masked value):
   // step s holds label positions 16 s + 8 h + i, split into their three bf16 pieces
   Frag3 Yf[NS];
   if (tile_lo < tile_valid) {
-    const float* Pb = P + (size_t)b * d.U * d.V;
+    const TIO* Pb = P + (size_t)b * d.U * d.V;
     const float* mPb = mP + (size_t)b * d.U;
 #pragma unroll
     for (int s = 0; s < NS; ++s) {
@@ -87,7 +89,7 @@ __device__ __forceinline__ void egrads_walk(
         const int u = 16 * s + 8 * h + i;
         const bool uok = u < Ub;
         const int uc = uok ? u : 0;
-        const float e = __expf(Pb[(size_t)uc * d.V + vc] - mPb[uc]);
+        const float e = __expf(ldf(Pb + (size_t)uc * d.V + vc) - mPb[uc]);
         y[i] = (uok && vok) ? e : 0.0f;
       }
       Yf[s] = split8(y);
@@ -106,6 +108,9 @@ __device__ __forceinline__ void egrads_walk(
     src_idx[i] = vec_ok[i] ? idx : nvec - 1;  // loads stay unconditional, stores are masked
     lds_off[i] = vec_ok[i] ? (idx / up4) * kEsPitch + 4 * (idx % up4) : 0;
   }
+  // per-lane part of the element offset inside a tile; the per-register part is r-dependent
+  // only through compile-time multiples of V
+  const unsigned lane_off = (unsigned)(4 * h) * (unsigned)d.V + (unsigned)vcol;
   auto fetch_slab = [&](int ti) -> SlabRegs {
     const float4* src =
         reinterpret_cast<const float4*>(Wn + ((size_t)b * Tw + (size_t)ti * 32) * Up);
@@ -144,28 +149,25 @@ __device__ __forceinline__ void egrads_walk(
     mu[i] = (sp.labels && i < nmatch) ? match[i] : 0;
     mc[i] = (sp.labels && i < nmatch) ? sp.labels[(size_t)b * (d.U - 1) + mu[i]] - wave_col0 : -1;
   }
-  // per-lane part of the element offset inside a tile; the per-register part is r-dependent
-  // only through compile-time multiples of V
-  const unsigned lane_off = (unsigned)(4 * h) * (unsigned)d.V + (unsigned)vcol;
 
   for (int ti = tile_lo; ti < tile_valid; ++ti) {
     const int t0 = ti * 32;
     // the next slab, requested now (the last tile re-reads its own: no branch around the loads)
     const SlabRegs nxt = fetch_slab(min(ti + 1, tile_valid - 1));
     const bool interior = cols_full && (t0 + 32 <= Tb);  // no row or column needs a guard
-    const float* Etile = Eb + (size_t)t0 * d.V;
-    float* Otile = out + (size_t)t0 * d.V;
+    const TIO* Etile = Eb + (size_t)t0 * d.V;
+    TIO* Otile = out + (size_t)t0 * d.V;
     // the emissions of this tile, requested before the matrix work so they arrive under it
     float ev[16];
     if (interior) {
 #pragma unroll
       for (int r = 0; r < 16; ++r)
-        ev[r] = Etile[lane_off + (unsigned)(8 * (r >> 2) + (r & 3)) * (unsigned)d.V];
+        ev[r] = ldf(Etile + (lane_off + (unsigned)(8 * (r >> 2) + (r & 3)) * (unsigned)d.V));
     } else {
       // rows past the utterance are read from its last frame and masked on the way out
 #pragma unroll
       for (int r = 0; r < 16; ++r)
-        ev[r] = Eb[(size_t)min(t0 + mfma_row(r, h), Tb - 1) * d.V + vc];
+        ev[r] = ldf(Eb + (size_t)min(t0 + mfma_row(r, h), Tb - 1) * d.V + vc);
     }
     // sparse terms of this tile for up to kEsPrefetch labels that fall into this wavefront's
     // columns: one coalesced load per plane, requested here so it arrives under the matrix work
@@ -250,16 +252,16 @@ __device__ __forceinline__ void egrads_walk(
     if (interior) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        float* o = Otile + lane_off + (unsigned)(8 * (r >> 2) + (r & 3)) * (unsigned)d.V;
-        *o = delta * (kAccumulate ? *o + v[r] : v[r]);
+        TIO* o = Otile + (lane_off + (unsigned)(8 * (r >> 2) + (r & 3)) * (unsigned)d.V);
+        stf(o, delta * (kAccumulate ? ldf(o) + v[r] : v[r]));
       }
     } else {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int t = t0 + mfma_row(r, h);
         if (t < d.T && vok) {
-          float* o = out + (size_t)t * d.V + vcol;
-          *o = delta * (kAccumulate ? *o + v[r] : v[r]);
+          TIO* o = out + (size_t)t * d.V + vcol;
+          stf(o, delta * (kAccumulate ? ldf(o) + v[r] : v[r]));
         }
       }
     }
@@ -274,18 +276,18 @@ __device__ __forceinline__ void egrads_walk(
     for (int r = 0; r < 16; ++r) {
       const int t = ti * 32 + mfma_row(r, h);
       if (t < d.T && vok) {
-        float* o = out + (size_t)t * d.V + vcol;
-        *o = kAccumulate ? delta * *o : 0.0f;
+        TIO* o = out + (size_t)t * d.V + vcol;
+        stf(o, kAccumulate ? delta * ldf(o) : 0.0f);
       }
     }
   }
 }
 
-template <bool kAccumulate>
+template <bool kAccumulate, typename TIO>
 __global__ __launch_bounds__(256, 2) void egrads_stream_kernel(
-    const float* __restrict__ E, const float* __restrict__ P, const float* __restrict__ mE,
+    const TIO* __restrict__ E, const TIO* __restrict__ P, const float* __restrict__ mE,
     const float* __restrict__ mP, const float* __restrict__ Wn, const float* __restrict__ deltas,
-    float* __restrict__ egrads, const int* __restrict__ inLen, const int* __restrict__ labLen,
+    TIO* __restrict__ egrads, const int* __restrict__ inLen, const int* __restrict__ labLen,
     Dims d, int Up, int Tw, int tiles_per_chunk, SparseTerms sp) {
   __shared__ __attribute__((aligned(16))) unsigned short As[2][3][kEsPlane];
   __shared__ __attribute__((aligned(16))) float Ms[2][32];  // mE of the slab's frames
@@ -333,21 +335,27 @@ constexpr int kPsPitch = 40;
 constexpr int kPsPlane = 128 * kPsPitch;
 constexpr int kPsFlush = 8;  // slabs of 32 frames between two flushes of the running sums
 
+// Blank / label terms of the 128 rows of one tile, staged in LDS for the write-out.
+struct PRowTerms {
+  float gB[128], gL[128];
+  int label[128];
+};
+
 // One workgroup's 128 x 128 tile with NMB 32-row blocks of label positions in use (a template
 // parameter, so the matrix instructions of a slice form one straight-line block).  Products are
 // formed on the bf16 matrix cores from exact three-way splits of both operands (rnnt_split.h).
-template <int NMB, bool kAccumulate>
+template <int NMB, bool kAccumulate, typename TIO>
 __device__ __forceinline__ void pgrads_tile(
-    const float* __restrict__ E, const float* __restrict__ P, const float* __restrict__ mE,
+    const TIO* __restrict__ E, const TIO* __restrict__ P, const float* __restrict__ mE,
     const float* __restrict__ mP, const float* __restrict__ Wt, const float* __restrict__ deltas,
-    float* __restrict__ pgrads, unsigned short (*As)[3][kPsPlane], float (*Ms)[32], const Dims& d,
-    int Up, int Tw, int b, int u0, int Tb, int Ub) {
+    TIO* __restrict__ pgrads, unsigned short (*As)[3][kPsPlane], float (*Ms)[32], const Dims& d,
+    int Up, int Tw, int b, int u0, int Tb, int Ub, const PRowTerms* rt) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, h = lane >> 5;
   const int vcol = blockIdx.x * 128 + wave * 32 + l32;
   const bool vok = vcol < d.V;
   const int vc = vok ? vcol : d.V - 1;
   const float delta = deltas ? deltas[b] : 1.0f;
-  float* out = pgrads + (size_t)b * d.U * d.V;
+  TIO* out = pgrads + (size_t)b * d.U * d.V;
 
   // The matrix instruction truncates what falls below its accumulator's last bit, so a long
   // running sum drifts low; every kPsFlush slabs it is added (vector ALU, round to nearest)
@@ -359,7 +367,7 @@ __device__ __forceinline__ void pgrads_tile(
     for (int r = 0; r < 16; ++r) acc[mb][r] = tot[mb][r] = 0.0f;
 
   if (NMB > 0) {
-    const float* Eb = E + (size_t)b * d.T * d.V;
+    const TIO* Eb = E + (size_t)b * d.T * d.V;
     const float* mEb = mE + (size_t)b * d.T;
     // W^T slab staging: 128 rows (u) x 32 frames = 1024 float4, four per thread; rows past the
     // padded label axis re-read its last row (their blocks are never multiplied)
@@ -386,7 +394,7 @@ __device__ __forceinline__ void pgrads_tile(
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
           const int t = min(k0 + 16 * s + 8 * h + i, Tb - 1);
-          x.v[s][i] = Eb[(size_t)t * d.V + vc];
+          x.v[s][i] = ldf(Eb + (size_t)t * d.V + vc);
         }
       return x;
     };
@@ -472,7 +480,7 @@ __device__ __forceinline__ void pgrads_tile(
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[mb][r] += tot[mb][r];
 
-  const float* Pb = P + (size_t)b * d.U * d.V;
+  const TIO* Pb = P + (size_t)b * d.U * d.V;
   const float* mPb = mP + (size_t)b * d.U;
 #pragma unroll
   for (int mb = 0; mb < 4; ++mb)
@@ -480,30 +488,52 @@ __device__ __forceinline__ void pgrads_tile(
     for (int r = 0; r < 16; ++r) {
       const int u = u0 + 32 * mb + mfma_row(r, h);
       const int uc = min(u, d.U - 1);
-      const float y = __expf(Pb[(size_t)uc * d.V + vc] - mPb[uc]);
+      const float y = __expf(ldf(Pb + (size_t)uc * d.V + vc) - mPb[uc]);
       const float g = (mb < NMB && u < Ub) ? y * acc[mb < NMB ? mb : 0][r] : 0.0f;
       if (u < d.U && vok) {
-        float* o = out + (size_t)u * d.V + vcol;
-        o[0] = delta * (kAccumulate ? o[0] + g : g);
+        TIO* o = out + (size_t)u * d.V + vcol;
+        float res = delta * (kAccumulate ? ldf(o) + g : g);
+        if (!kAccumulate && rt != nullptr) {
+          // the blank / label terms of this row (what sparse_p_kernel adds), same arithmetic:
+          // delta * dense, then + delta * term.  Read from LDS with one address per half-wave.
+          const int k = 32 * mb + mfma_row(r, h);
+          if (vcol == d.blank) res += delta * rt->gB[k];
+          else if (vcol == rt->label[k]) res += delta * rt->gL[k];
+        }
+        stf(o, res);
       }
     }
 }
 
-template <bool kAccumulate>
+template <bool kAccumulate, typename TIO>
 __global__ __launch_bounds__(256, 2) void pgrads_stream_kernel(
-    const float* __restrict__ E, const float* __restrict__ P, const float* __restrict__ mE,
+    const TIO* __restrict__ E, const TIO* __restrict__ P, const float* __restrict__ mE,
     const float* __restrict__ mP, const float* __restrict__ Wt, const float* __restrict__ deltas,
-    float* __restrict__ pgrads, const int* __restrict__ inLen, const int* __restrict__ labLen,
-    Dims d, int Up, int Tw) {
+    TIO* __restrict__ pgrads, const int* __restrict__ inLen, const int* __restrict__ labLen,
+    Dims d, int Up, int Tw, SparsePTerms sp) {
   __shared__ __attribute__((aligned(16))) unsigned short As[2][3][kPsPlane];
   __shared__ __attribute__((aligned(16))) float Ms[2][32];
+  __shared__ PRowTerms Rt;
   const int b = blockIdx.z, u0 = blockIdx.y * 128;
   int Tb, Ub;
   utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
+  const bool folding = !kAccumulate && sp.gB != nullptr;
+  if (folding && threadIdx.x < 128) {
+    // this tile's rows: blank total, label and label total; rows without one get a label that
+    // matches no column.  Visible to all after the barriers of the walk (or the one below).
+    const int k = threadIdx.x, u = u0 + k;
+    const bool valid = Tb > 0 && u < Ub, has_label = valid && u + 1 < Ub;
+    const int l = has_label ? sp.labels[(size_t)b * (d.U - 1) + u] : d.blank;
+    Rt.gB[k] = valid ? sp.gB[(size_t)b * d.Ua + u] : 0.0f;
+    Rt.gL[k] = has_label ? sp.gL[(size_t)b * d.Ua + u] : 0.0f;
+    Rt.label[k] = (has_label && l != d.blank) ? l : -1;
+  }
+  if (folding) __syncthreads();
+  const PRowTerms* rt = folding ? &Rt : nullptr;
   const int nmb = (u0 < Ub && Tb > 0) ? min(4, (Ub - u0 + 31) >> 5) : 0;  // 32-row blocks in use
 #define RNNT_PG_TILE(NMB)                                                                    \
   pgrads_tile<NMB, kAccumulate>(E, P, mE, mP, Wt, deltas, pgrads, As, Ms, d, Up, Tw, b, u0, \
-                                Tb, Ub)
+                                Tb, Ub, rt)
   switch (nmb) {
     case 0: RNNT_PG_TILE(0); break;
     case 1: RNNT_PG_TILE(1); break;
@@ -524,10 +554,11 @@ __global__ __launch_bounds__(256, 2) void pgrads_stream_kernel(
 
 bool egrads_stream_supported(const Dims& d) { return wplane_up(d.U) <= 16 * kEsMaxS; }
 
-int launch_egrads_stream(const float* E, const float* P, const float* mE, const float* mP,
-                         const float* Wn, const float* deltas, float* egrads, const int* inLen,
-                         const int* labLen, const Dims& d, bool accumulate,
-                         const SparseTerms& sparse, hipStream_t s) {
+template <typename TIO>
+static int egrads_stream_any(const TIO* E, const TIO* P, const float* mE, const float* mP,
+                             const float* Wn, const float* deltas, TIO* egrads, const int* inLen,
+                             const int* labLen, const Dims& d, bool accumulate,
+                             const SparseTerms& sparse, hipStream_t s) {
   if (sparse.labels && accumulate)
     return fail(kInvalid, "sparse-term folding and accumulation are mutually exclusive");
   const int Up = wplane_up(d.U), Tw = wplane_tw(d.T);
@@ -541,28 +572,58 @@ int launch_egrads_stream(const float* E, const float* P, const float* mE, const 
   const int per = (ntiles + chunks - 1) / chunks;
   chunks = (ntiles + per - 1) / per;
   if (accumulate)
-    hipLaunchKernelGGL(egrads_stream_kernel<true>, dim3(vtiles, chunks, d.B), dim3(256), 0, s, E,
+    hipLaunchKernelGGL((egrads_stream_kernel<true, TIO>), dim3(vtiles, chunks, d.B), dim3(256), 0, s, E,
                        P, mE, mP, Wn, deltas, egrads, inLen, labLen, d, Up, Tw, per, sparse);
   else
-    hipLaunchKernelGGL(egrads_stream_kernel<false>, dim3(vtiles, chunks, d.B), dim3(256), 0, s, E,
+    hipLaunchKernelGGL((egrads_stream_kernel<false, TIO>), dim3(vtiles, chunks, d.B), dim3(256), 0, s, E,
                        P, mE, mP, Wn, deltas, egrads, inLen, labLen, d, Up, Tw, per, sparse);
   RNNT_LAUNCH_CHECK("egrads_stream_kernel");
   return kOk;
 }
+int launch_egrads_stream(const float* E, const float* P, const float* mE, const float* mP,
+                         const float* Wn, const float* deltas, float* egrads, const int* inLen,
+                         const int* labLen, const Dims& d, bool accumulate,
+                         const SparseTerms& sparse, hipStream_t s) {
+  return egrads_stream_any(E, P, mE, mP, Wn, deltas, egrads, inLen, labLen, d, accumulate, sparse,
+                           s);
+}
+int launch_egrads_stream(const bf16_t* E, const bf16_t* P, const float* mE, const float* mP,
+                         const float* Wn, const float* deltas, bf16_t* egrads, const int* inLen,
+                         const int* labLen, const Dims& d, bool accumulate,
+                         const SparseTerms& sparse, hipStream_t s) {
+  return egrads_stream_any(E, P, mE, mP, Wn, deltas, egrads, inLen, labLen, d, accumulate, sparse,
+                           s);
+}
 
-int launch_pgrads_stream(const float* E, const float* P, const float* mE, const float* mP,
-                         const float* Wt, const float* deltas, float* pgrads, const int* inLen,
-                         const int* labLen, const Dims& d, bool accumulate, hipStream_t s) {
+template <typename TIO>
+static int pgrads_stream_any(const TIO* E, const TIO* P, const float* mE, const float* mP,
+                             const float* Wt, const float* deltas, TIO* pgrads, const int* inLen,
+                             const int* labLen, const Dims& d, bool accumulate,
+                             const SparsePTerms& sp, hipStream_t s) {
+  if (sp.gB && accumulate)
+    return fail(kInvalid, "sparse-term folding and accumulation are mutually exclusive");
   const int Up = wplane_up(d.U), Tw = wplane_tw(d.T);
   const dim3 grid((d.V + 127) / 128, (d.U + 127) / 128, d.B);
   if (accumulate)
-    hipLaunchKernelGGL(pgrads_stream_kernel<true>, grid, dim3(256), 0, s, E, P, mE, mP, Wt, deltas,
-                       pgrads, inLen, labLen, d, Up, Tw);
+    hipLaunchKernelGGL((pgrads_stream_kernel<true, TIO>), grid, dim3(256), 0, s, E, P, mE, mP, Wt,
+                       deltas, pgrads, inLen, labLen, d, Up, Tw, sp);
   else
-    hipLaunchKernelGGL(pgrads_stream_kernel<false>, grid, dim3(256), 0, s, E, P, mE, mP, Wt,
-                       deltas, pgrads, inLen, labLen, d, Up, Tw);
+    hipLaunchKernelGGL((pgrads_stream_kernel<false, TIO>), grid, dim3(256), 0, s, E, P, mE, mP, Wt,
+                       deltas, pgrads, inLen, labLen, d, Up, Tw, sp);
   RNNT_LAUNCH_CHECK("pgrads_stream_kernel");
   return kOk;
+}
+int launch_pgrads_stream(const float* E, const float* P, const float* mE, const float* mP,
+                         const float* Wt, const float* deltas, float* pgrads, const int* inLen,
+                         const int* labLen, const Dims& d, bool accumulate,
+                         const SparsePTerms& sp, hipStream_t s) {
+  return pgrads_stream_any(E, P, mE, mP, Wt, deltas, pgrads, inLen, labLen, d, accumulate, sp, s);
+}
+int launch_pgrads_stream(const bf16_t* E, const bf16_t* P, const float* mE, const float* mP,
+                         const float* Wt, const float* deltas, bf16_t* pgrads, const int* inLen,
+                         const int* labLen, const Dims& d, bool accumulate,
+                         const SparsePTerms& sp, hipStream_t s) {
+  return pgrads_stream_any(E, P, mE, mP, Wt, deltas, pgrads, inLen, labLen, d, accumulate, sp, s);
 }
 
 }  // namespace rnnt

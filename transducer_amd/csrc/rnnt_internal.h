@@ -6,6 +6,8 @@
 #include <stddef.h>
 #include <stdint.h>
 
+#include "rnnt_io.h"
+
 namespace rnnt {
 
 // ---------------------------------------------------------------- status / errors
@@ -114,9 +116,6 @@ int launch_sparse(const Planes& p, float* egrads, float* pgrads, const int* labe
 // bsum[b,t] = what the sparse terms leave in egrads[b,t,blank] (see blank_sums_kernel).
 int launch_blank_sums(const Planes& p, float* bsum, const int* labels, const int* inLen,
                       const int* labLen, const Dims& d, hipStream_t s);
-int launch_sparse_p(const Planes& p, float* pgrads, const int* labels, const int* inLen,
-                    const int* labLen, const float* scale, bool add, const Dims& d,
-                    hipStream_t s);
 int launch_maxplus(const float* E, const float* P, const int* inLen, const int* labLen,
                    float* best, int* arg, const Dims& d, hipStream_t s);
 // bestS / argS: skewed planes of the max-plus table (argS carries int bits in float storage).
@@ -144,9 +143,14 @@ int launch_lse(const float* E, const float* P, const float* mE, const float* mP,
 // exp(P - mP) are first written to `scratch` (lse_scratch_bytes) in matrix-operand order.
 // launch_lse_stream needs mP only and WRITES mE (one reference value per frame, >= the row
 // maximum minus a fixed slack; what the gradient kernels need as mE).
+// Each launcher that reads the scores or writes their gradients exists for fp32 and for bf16
+// arrays (rnnt_io.h); the bf16 forms need V % 8 == 0.
 bool lse_stream_supported(const float* E, const Dims& d);
+bool lse_stream_supported(const bf16_t* E, const Dims& d);
 size_t lse_scratch_bytes(const Dims& d);
 int launch_yplanes(const float* P, const float* mP, void* scratch, const int* labLen,
+                   const Dims& d, hipStream_t s);
+int launch_yplanes(const bf16_t* P, const float* mP, void* scratch, const int* labLen,
                    const Dims& d, hipStream_t s);
 // With elS / eb (skewed label-score plane and blank-score vector) it also copies E[t, label_u]
 // and E[t, blank] out of the rows it streams (what launch_gather does for the emissions).
@@ -154,8 +158,14 @@ int launch_lse_stream(const float* E, float* mE, const float* mP, float* LN,
                       const void* scratch, const int* inLen, const int* labLen, const Dims& d,
                       hipStream_t s, const int* labels = nullptr, float* elS = nullptr,
                       float* eb = nullptr);
+int launch_lse_stream(const bf16_t* E, float* mE, const float* mP, float* LN,
+                      const void* scratch, const int* inLen, const int* labLen, const Dims& d,
+                      hipStream_t s, const int* labels = nullptr, float* elS = nullptr,
+                      float* eb = nullptr);
 // P[u, blank] and P[u, label_u] into the planes, with the row maxima of P (one pass).
 int launch_rowmax_pick_p(const float* P, float* mP, const int* labels, const int* labLen,
+                         const Planes& p, const Dims& d, hipStream_t s);
+int launch_rowmax_pick_p(const bf16_t* P, float* mP, const int* labels, const int* labLen,
                          const Planes& p, const Dims& d, hipStream_t s);
 int launch_wplanes(const float* lngrads, const float* LN, const float* mE, const float* mP,
                    float* Wn, float* Wt, const int* inLen, const int* labLen, const Dims& d,
@@ -169,6 +179,13 @@ struct SparseTerms {
   const float* bsum = nullptr;  // [B,T] blank-column totals
   const int* labels = nullptr;  // [B,U-1]
 };
+// The same for pgrads: per-(b,u) totals of the blank and the label column (Planes::gB, gL), added
+// in the dense kernel's write-out exactly as sparse_p_kernel would add them afterwards.
+struct SparsePTerms {
+  const float* gB = nullptr;
+  const float* gL = nullptr;
+  const int* labels = nullptr;  // [B,U-1]; may be null when U == 1
+};
 bool egrads_fusion_supported(const Dims& d);
 // accumulate == false: out = delta * dense.   accumulate == true: out = delta * (out + dense),
 // the update of transducer/torch_binding.py:86-89.
@@ -178,7 +195,8 @@ int launch_egrads(const float* E, const float* P, const float* mE, const float* 
                   hipStream_t s);
 int launch_pgrads(const float* E, const float* P, const float* mE, const float* mP,
                   const float* Wt, const float* deltas, float* pgrads, const int* inLen,
-                  const int* labLen, const Dims& d, bool accumulate, hipStream_t s);
+                  const int* labLen, const Dims& d, bool accumulate, const SparsePTerms& sparse,
+                  hipStream_t s);
 
 
 // ---------------------------------------------------------------- launchers (rnnt_grads.hip)
@@ -187,8 +205,17 @@ int launch_egrads_stream(const float* E, const float* P, const float* mE, const 
                          const float* Wn, const float* deltas, float* egrads, const int* inLen,
                          const int* labLen, const Dims& d, bool accumulate,
                          const SparseTerms& sparse, hipStream_t s);
+int launch_egrads_stream(const bf16_t* E, const bf16_t* P, const float* mE, const float* mP,
+                         const float* Wn, const float* deltas, bf16_t* egrads, const int* inLen,
+                         const int* labLen, const Dims& d, bool accumulate,
+                         const SparseTerms& sparse, hipStream_t s);
 int launch_pgrads_stream(const float* E, const float* P, const float* mE, const float* mP,
                          const float* Wt, const float* deltas, float* pgrads, const int* inLen,
-                         const int* labLen, const Dims& d, bool accumulate, hipStream_t s);
+                         const int* labLen, const Dims& d, bool accumulate,
+                         const SparsePTerms& sparse, hipStream_t s);
+int launch_pgrads_stream(const bf16_t* E, const bf16_t* P, const float* mE, const float* mP,
+                         const float* Wt, const float* deltas, bf16_t* pgrads, const int* inLen,
+                         const int* labLen, const Dims& d, bool accumulate,
+                         const SparsePTerms& sparse, hipStream_t s);
 
 }  // namespace rnnt

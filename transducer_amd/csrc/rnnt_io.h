@@ -1,0 +1,78 @@
+// Element types of the score arrays (emissions, predictions) and of their gradients at the
+// library's interface: fp32, as in the reference, or bf16 for a caller whose projection layers
+// produce bf16 logits.  The kernels are written once over these helpers; all arithmetic stays
+// fp32 (a bf16 score converts exactly), only the loads and the final stores differ.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+namespace rnnt {
+
+struct bf16_t {
+  unsigned short bits;
+};
+
+__device__ inline float bf16_to_float(unsigned short b) {
+  return __uint_as_float((unsigned)b << 16);
+}
+// round to nearest even (one v_cvt_pk_bf16_f32)
+__device__ inline unsigned short float_to_bf16(float v) {
+  return __builtin_bit_cast(unsigned short, (__bf16)v);
+}
+
+__device__ inline float ldf(const float* p) { return *p; }
+__device__ inline float ldf(const bf16_t* p) { return bf16_to_float(p->bits); }
+__device__ inline void stf(float* p, float v) { *p = v; }
+__device__ inline void stf(bf16_t* p, float v) { p->bits = float_to_bf16(v); }
+
+// Eight consecutive elements of a row as they sit in registers after the load.
+template <typename T>
+struct Raw8;
+template <>
+struct Raw8<float> {
+  float4 lo, hi;
+};
+template <>
+struct Raw8<bf16_t> {
+  uint4 w;
+};
+
+// Elements v .. v+7 of `row`, with the start clamped so that the load stays inside a row of V
+// elements: fp32 rows (V % 4 == 0) clamp each group of four to the last group, bf16 rows
+// (V % 8 == 0) the whole eight to the last eight.  Both are 16-byte loads.
+__device__ inline Raw8<float> load8(const float* row, int v, int V) {
+  Raw8<float> r;
+  r.lo = *reinterpret_cast<const float4*>(row + min(v, V - 4));
+  r.hi = *reinterpret_cast<const float4*>(row + min(v + 4, V - 4));
+  return r;
+}
+__device__ inline Raw8<bf16_t> load8(const bf16_t* row, int v, int V) {
+  Raw8<bf16_t> r;
+  r.w = *reinterpret_cast<const uint4*>(row + min(v, V - 8));
+  return r;
+}
+
+__device__ inline void expand(const Raw8<float>& r, float (&e)[8]) {
+  e[0] = r.lo.x; e[1] = r.lo.y; e[2] = r.lo.z; e[3] = r.lo.w;
+  e[4] = r.hi.x; e[5] = r.hi.y; e[6] = r.hi.z; e[7] = r.hi.w;
+}
+__device__ inline void expand(const Raw8<bf16_t>& r, float (&e)[8]) {
+  e[0] = __uint_as_float(r.w.x << 16); e[1] = __uint_as_float(r.w.x & 0xffff0000u);
+  e[2] = __uint_as_float(r.w.y << 16); e[3] = __uint_as_float(r.w.y & 0xffff0000u);
+  e[4] = __uint_as_float(r.w.z << 16); e[5] = __uint_as_float(r.w.z & 0xffff0000u);
+  e[6] = __uint_as_float(r.w.w << 16); e[7] = __uint_as_float(r.w.w & 0xffff0000u);
+}
+
+// Vector width (elements) that makes a row start 16-byte aligned.
+template <typename T>
+struct RowAlign;
+template <>
+struct RowAlign<float> {
+  static constexpr int kElems = 4;
+};
+template <>
+struct RowAlign<bf16_t> {
+  static constexpr int kElems = 8;
+};
+
+}  // namespace rnnt

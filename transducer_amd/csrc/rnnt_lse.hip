@@ -31,6 +31,7 @@
 //  * Workgroups are renumbered so that all frame tiles of one utterance run on the same XCD
 //    (workgroup ids are dealt round-robin to the 8 XCDs) and share its L2 copy of Y[b].
 #include "rnnt_internal.h"
+#include "rnnt_io.h"
 #include "rnnt_split.h"
 
 namespace rnnt {
@@ -61,8 +62,10 @@ inline int y_ublocks(const Dims& d) { return (d.U + 31) / 32; }
 inline int y_steps(const Dims& d) { return 2 * ((d.V + kSlice - 1) / kSlice); }
 
 // ------------------------------------------------------------------ Y pieces
-// One thread per (u, eight consecutive v).  vec4 = V % 4 == 0 and P 16-byte aligned.
-__global__ __launch_bounds__(256) void yplanes_kernel(const float* __restrict__ P,
+// One thread per (u, eight consecutive v).  vec = rows of P start 16-byte aligned (V a multiple
+// of 4 for fp32, of 8 for bf16, and P aligned).
+template <typename TIO>
+__global__ __launch_bounds__(256) void yplanes_kernel(const TIO* __restrict__ P,
                                                       const float* __restrict__ mP,
                                                       uint4* __restrict__ Yp,
                                                       const int* __restrict__ labLen, Dims d,
@@ -77,21 +80,20 @@ __global__ __launch_bounds__(256) void yplanes_kernel(const float* __restrict__ 
 #pragma unroll
   for (int i = 0; i < 8; ++i) y[i] = 0.0f;
   if (u < Ub) {
-    const float* row = P + ((size_t)b * d.U + u) * d.V;
+    const TIO* row = P + ((size_t)b * d.U + u) * d.V;
     const float m = mP[(size_t)b * d.U + u];
     if (vec4) {
       if (v0 < d.V) {
-        const float4 p = *reinterpret_cast<const float4*>(row + v0);
-        y[0] = __expf(p.x - m); y[1] = __expf(p.y - m); y[2] = __expf(p.z - m); y[3] = __expf(p.w - m);
-      }
-      if (v0 + 4 < d.V) {
-        const float4 p = *reinterpret_cast<const float4*>(row + v0 + 4);
-        y[4] = __expf(p.x - m); y[5] = __expf(p.y - m); y[6] = __expf(p.z - m); y[7] = __expf(p.w - m);
+        float e[8];
+        expand(load8(row, v0, d.V), e);  // a clamped group repeats values; masked below
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+          if (v0 + i < d.V) y[i] = __expf(e[i] - m);
       }
     } else {
 #pragma unroll
       for (int i = 0; i < 8; ++i)
-        if (v0 + i < d.V) y[i] = __expf(row[v0 + i] - m);
+        if (v0 + i < d.V) y[i] = __expf(ldf(row + v0 + i) - m);
     }
   }
   const Frag3 f = split8(y);
@@ -105,9 +107,9 @@ __global__ __launch_bounds__(256) void yplanes_kernel(const float* __restrict__ 
 // kWaves = 4: a wavefront owns one block of 32 label positions and all 128 frames (four
 // accumulators).  kWaves = 8: two wavefronts share a block, 64 frames each (two accumulators,
 // half the registers, twice the wavefronts to hide each other's staging).
-template <int kWaves>
+template <int kWaves, typename TIO>
 __global__ __launch_bounds__(64 * kWaves, kWaves / 2) void lse_stream_kernel(
-    const float* __restrict__ E, float* __restrict__ mE, const float* __restrict__ mP,
+    const TIO* __restrict__ E, float* __restrict__ mE, const float* __restrict__ mP,
     const uint4* __restrict__ Yp, float* __restrict__ LN, const int* __restrict__ inLen,
     const int* __restrict__ labLen, Dims d, int ttiles, int utiles, int total, int nub, int nks,
     const int* __restrict__ labels, float* __restrict__ elS, float* __restrict__ ebv) {
@@ -172,7 +174,7 @@ __global__ __launch_bounds__(64 * kWaves, kWaves / 2) void lse_stream_kernel(
   // the row's last group (V % 4 == 0): finite values that meet zeros in Y or are dropped on
   // the way out.
   const int srow = tid >> 2, c8 = tid & 3;
-  const float* px[NR];
+  const TIO* px[NR];
   float mx[NR];  // the row's reference; the four threads that share a row always agree on it
   int slot[NR];
 #pragma unroll
@@ -183,15 +185,11 @@ __global__ __launch_bounds__(64 * kWaves, kWaves / 2) void lse_stream_kernel(
     mx[i] = kLowest;
     slot[i] = xslot(row, c8);
   }
-  struct XRegs { float4 lo[NR], hi[NR]; };
+  struct XRegs { Raw8<TIO> x[NR]; };
   auto fetch = [&](int k0) -> XRegs {
-    const int v0 = min(k0 + 8 * c8, d.V - 4), v1 = min(k0 + 8 * c8 + 4, d.V - 4);
     XRegs r;
 #pragma unroll
-    for (int i = 0; i < NR; ++i) {
-      r.lo[i] = *reinterpret_cast<const float4*>(px[i] + v0);
-      r.hi[i] = *reinterpret_cast<const float4*>(px[i] + v1);
-    }
+    for (int i = 0; i < NR; ++i) r.x[i] = load8(px[i], k0 + 8 * c8, d.V);
     return r;
   };
   // copies column `col` (which lies in the slab held in r) of this thread's rows to dst[t]
@@ -205,11 +203,13 @@ __global__ __launch_bounds__(64 * kWaves, kWaves / 2) void lse_stream_kernel(
       const unsigned k0 = e == 0 ? ~0u : 0u, k1 = e == 1 ? ~0u : 0u, k2 = e == 2 ? ~0u : 0u,
                      k3 = e == 3 ? ~0u : 0u, k4 = e == 4 ? ~0u : 0u, k5 = e == 5 ? ~0u : 0u,
                      k6 = e == 6 ? ~0u : 0u, k7 = e == 7 ? ~0u : 0u;
+      float x[8];
+      expand(r.x[i], x);
       const float v = __uint_as_float(
-          (__float_as_uint(r.lo[i].x) & k0) | (__float_as_uint(r.lo[i].y) & k1) |
-          (__float_as_uint(r.lo[i].z) & k2) | (__float_as_uint(r.lo[i].w) & k3) |
-          (__float_as_uint(r.hi[i].x) & k4) | (__float_as_uint(r.hi[i].y) & k5) |
-          (__float_as_uint(r.hi[i].z) & k6) | (__float_as_uint(r.hi[i].w) & k7));
+          (__float_as_uint(x[0]) & k0) | (__float_as_uint(x[1]) & k1) |
+          (__float_as_uint(x[2]) & k2) | (__float_as_uint(x[3]) & k3) |
+          (__float_as_uint(x[4]) & k4) | (__float_as_uint(x[5]) & k5) |
+          (__float_as_uint(x[6]) & k6) | (__float_as_uint(x[7]) & k7));
       const int t = t0 + srow + (kThreads / 4) * i;
       if (t < Tb) dst[t] = v;
     }
@@ -228,8 +228,10 @@ __global__ __launch_bounds__(64 * kWaves, kWaves / 2) void lse_stream_kernel(
 #pragma unroll
     for (int i = 0; i < NR; ++i) {
       // maximum of the row's 32 values of this slab (values past V repeat earlier ones)
-      float lm = fmaxf(fmaxf(fmaxf(r.lo[i].x, r.lo[i].y), fmaxf(r.lo[i].z, r.lo[i].w)),
-                       fmaxf(fmaxf(r.hi[i].x, r.hi[i].y), fmaxf(r.hi[i].z, r.hi[i].w)));
+      float e[8];
+      expand(r.x[i], e);
+      float lm = fmaxf(fmaxf(fmaxf(e[0], e[1]), fmaxf(e[2], e[3])),
+                       fmaxf(fmaxf(e[4], e[5]), fmaxf(e[6], e[7])));
       lm = fmaxf(lm, quad_xor1(lm));  // the four threads of a row are one quad of lanes
       lm = fmaxf(lm, quad_xor2(lm));
       lm = fmaxf(lm, kLowest);
@@ -242,9 +244,8 @@ __global__ __launch_bounds__(64 * kWaves, kWaves / 2) void lse_stream_kernel(
         mx[i] = lm;
       }
       const float m = mx[i];
-      const float x[8] = {__expf(r.lo[i].x - m), __expf(r.lo[i].y - m), __expf(r.lo[i].z - m),
-                          __expf(r.lo[i].w - m), __expf(r.hi[i].x - m), __expf(r.hi[i].y - m),
-                          __expf(r.hi[i].z - m), __expf(r.hi[i].w - m)};
+      const float x[8] = {__expf(e[0] - m), __expf(e[1] - m), __expf(e[2] - m), __expf(e[3] - m),
+                          __expf(e[4] - m), __expf(e[5] - m), __expf(e[6] - m), __expf(e[7] - m)};
       const Frag3 f = split8(x);
       Xs[buf][0][slot[i]] = f.h;
       Xs[buf][1][slot[i]] = f.m;
@@ -423,40 +424,65 @@ __global__ __launch_bounds__(64 * kWaves, kWaves / 2) void lse_stream_kernel(
     if (_e != hipSuccess) return check_hip(_e, "launch " name, __FILE__, __LINE__); \
   } while (0)
 
-bool lse_stream_supported(const float* E, const Dims& d) {
+template <typename TIO>
+static bool lse_stream_ok(const TIO* E, const Dims& d) {
+  constexpr int kA = RowAlign<TIO>::kElems;
   const long total = (long)((d.T + kRows - 1) / kRows) * ((d.U + 127) / 128) * d.B;
-  return d.V % 4 == 0 && d.V >= 4 && (reinterpret_cast<uintptr_t>(E) & 15) == 0 &&
+  return d.V % kA == 0 && d.V >= kA && (reinterpret_cast<uintptr_t>(E) & 15) == 0 &&
          total < (1l << 30);
 }
+bool lse_stream_supported(const float* E, const Dims& d) { return lse_stream_ok(E, d); }
+bool lse_stream_supported(const bf16_t* E, const Dims& d) { return lse_stream_ok(E, d); }
 
 size_t lse_scratch_bytes(const Dims& d) {
   if (d.B == 0 || d.T == 0 || d.U == 0 || d.V % 4 != 0) return 0;
   return (size_t)d.B * y_ublocks(d) * y_steps(d) * 3 * 64 * sizeof(uint4);
 }
 
-int launch_yplanes(const float* P, const float* mP, void* scratch, const int* labLen,
-                   const Dims& d, hipStream_t s) {
+template <typename TIO>
+static int yplanes_any(const TIO* P, const float* mP, void* scratch, const int* labLen,
+                       const Dims& d, hipStream_t s) {
   const int nub = y_ublocks(d), nks = y_steps(d);
-  const int vec4 = (reinterpret_cast<uintptr_t>(P) & 15) == 0;
-  hipLaunchKernelGGL(yplanes_kernel, dim3((nks + 3) / 4, nub, d.B), dim3(256), 0, s, P, mP,
+  const int vec4 = (reinterpret_cast<uintptr_t>(P) & 15) == 0 && d.V % RowAlign<TIO>::kElems == 0;
+  hipLaunchKernelGGL(yplanes_kernel<TIO>, dim3((nks + 3) / 4, nub, d.B), dim3(256), 0, s, P, mP,
                      static_cast<uint4*>(scratch), labLen, d, nub, nks, vec4);
   RNNT_LAUNCH_CHECK("yplanes_kernel");
   return kOk;
 }
+int launch_yplanes(const float* P, const float* mP, void* scratch, const int* labLen,
+                   const Dims& d, hipStream_t s) {
+  return yplanes_any(P, mP, scratch, labLen, d, s);
+}
+int launch_yplanes(const bf16_t* P, const float* mP, void* scratch, const int* labLen,
+                   const Dims& d, hipStream_t s) {
+  return yplanes_any(P, mP, scratch, labLen, d, s);
+}
 
-int launch_lse_stream(const float* E, float* mE, const float* mP, float* LN,
-                      const void* scratch, const int* inLen, const int* labLen, const Dims& d,
-                      hipStream_t s, const int* labels, float* elS, float* eb) {
+template <typename TIO>
+static int lse_stream_any(const TIO* E, float* mE, const float* mP, float* LN,
+                          const void* scratch, const int* inLen, const int* labLen,
+                          const Dims& d, hipStream_t s, const int* labels, float* elS,
+                          float* eb) {
   const int nub = y_ublocks(d), nks = y_steps(d);
   const int ttiles = (d.T + kRows - 1) / kRows, utiles = (d.U + 127) / 128;
   const long total = (long)ttiles * utiles * d.B;
   const int grid = (int)((total + 7) / 8 * 8);
   constexpr int kWaves = 4;
-  hipLaunchKernelGGL(lse_stream_kernel<kWaves>, dim3(grid), dim3(64 * kWaves), 0, s, E, mE, mP,
+  hipLaunchKernelGGL((lse_stream_kernel<kWaves, TIO>), dim3(grid), dim3(64 * kWaves), 0, s, E, mE, mP,
                      static_cast<const uint4*>(scratch), LN, inLen, labLen, d, ttiles, utiles,
                      (int)total, nub, nks, labels, elS, eb);
   RNNT_LAUNCH_CHECK("lse_stream_kernel");
   return kOk;
+}
+int launch_lse_stream(const float* E, float* mE, const float* mP, float* LN,
+                      const void* scratch, const int* inLen, const int* labLen, const Dims& d,
+                      hipStream_t s, const int* labels, float* elS, float* eb) {
+  return lse_stream_any(E, mE, mP, LN, scratch, inLen, labLen, d, s, labels, elS, eb);
+}
+int launch_lse_stream(const bf16_t* E, float* mE, const float* mP, float* LN,
+                      const void* scratch, const int* inLen, const int* labLen, const Dims& d,
+                      hipStream_t s, const int* labels, float* elS, float* eb) {
+  return lse_stream_any(E, mE, mP, LN, scratch, inLen, labLen, d, s, labels, elS, eb);
 }
 
 }  // namespace rnnt

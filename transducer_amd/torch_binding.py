@@ -45,8 +45,11 @@ class Transducer(torch.autograd.Function):
     """costs[B] = -log p(labels | emissions, predictions); reference: torch_binding.py:23-90."""
 
     @staticmethod
-    def forward(ctx, emissions, predictions, labels, input_lengths, label_lengths, blank=0):
-        certify_inputs(emissions, predictions, labels, input_lengths, label_lengths)
+    def forward(ctx, emissions, predictions, labels, input_lengths, label_lengths, blank=0,
+                allow_bf16=False):
+        bf16 = allow_bf16 and emissions.dtype is torch.bfloat16
+        certify_inputs(emissions, predictions, labels, input_lengths, label_lengths,
+                       score_dtype=torch.bfloat16 if bf16 else torch.float32)
         _require_device(emissions)
         device = emissions.device
         # the library reads raw pointers: dense row-major storage is required
@@ -54,17 +57,18 @@ class Transducer(torch.autograd.Function):
         predictions = predictions.contiguous()
         B, T, V = emissions.shape
         U = predictions.shape[1]
-        costs = torch.empty(size=(B,), device=device, dtype=emissions.dtype)
+        costs = torch.empty(size=(B,), device=device, dtype=torch.float32)
         nbytes = _transducer.loss_workspace_bytes(B, T, U, V)
         workspace = torch.empty(size=(nbytes,), device=device, dtype=torch.uint8)
         with DeviceManager(device):
-            _transducer.loss_forward(
+            (_transducer.loss_forward_bf16 if bf16 else _transducer.loss_forward)(
                 emissions.data_ptr(), predictions.data_ptr(), labels.data_ptr(),
                 input_lengths.data_ptr(), label_lengths.data_ptr(), costs.data_ptr(),
                 workspace.data_ptr(), nbytes, B, T, U, V, blank, _stream(device))
         ctx.save_for_backward(
             emissions, predictions, labels, input_lengths, label_lengths, workspace)
         ctx.blank = blank
+        ctx.bf16 = bf16
         return costs
 
     @staticmethod
@@ -78,12 +82,12 @@ class Transducer(torch.autograd.Function):
         egrads = torch.empty(size=(B, T, V), device=device, dtype=emissions.dtype)
         pgrads = torch.empty(size=(B, U, V), device=device, dtype=emissions.dtype)
         with DeviceManager(device):
-            _transducer.loss_backward(
+            (_transducer.loss_backward_bf16 if ctx.bf16 else _transducer.loss_backward)(
                 emissions.data_ptr(), predictions.data_ptr(), labels.data_ptr(),
                 input_lengths.data_ptr(), label_lengths.data_ptr(), deltas.data_ptr(),
                 egrads.data_ptr(), pgrads.data_ptr(), workspace.data_ptr(), workspace.numel(),
                 B, T, U, V, ctx.blank, _stream(device))
-        return egrads, pgrads, None, None, None, None
+        return egrads, pgrads, None, None, None, None, None
 
 
 class TransducerLoss(torch.nn.Module):
@@ -94,11 +98,16 @@ class TransducerLoss(torch.nn.Module):
 
     Arguments:
         blank (int, optional): Integer id of blank label (default is 0).
+        allow_bf16 (bool, optional): also accept ``torch.bfloat16`` emissions and predictions
+            (both), returning float32 costs and bfloat16 gradients.  Not in the reference, which
+            raises ``TypeError`` for anything but float32 -- and so does this module by default.
+            Needs a vocabulary that is a multiple of 8 and at most 112 label positions.
     """
 
-    def __init__(self, blank=0):
+    def __init__(self, blank=0, allow_bf16=False):
         super(TransducerLoss, self).__init__()
         self.blank = blank
+        self.allow_bf16 = allow_bf16
 
     def forward(self, emissions, predictions, labels, input_lengths, label_lengths):
         """
@@ -115,7 +124,8 @@ class TransducerLoss(torch.nn.Module):
           costs (FloatTensor): (minibatch,) negative log-likelihood of each example.
         """
         return Transducer.apply(
-            emissions, predictions, labels, input_lengths, label_lengths, self.blank)
+            emissions, predictions, labels, input_lengths, label_lengths, self.blank,
+            self.allow_bf16)
 
     @torch.no_grad()
     def viterbi(self, emissions, predictions, input_lengths, label_lengths):
@@ -158,10 +168,11 @@ def check_dim(var, dim, name):
         raise ValueError("{} must be {}D".format(name, dim))
 
 
-def certify_inputs(emissions, predictions, labels, input_lengths, label_lengths):
+def certify_inputs(emissions, predictions, labels, input_lengths, label_lengths,
+                   score_dtype=torch.float32):
     """Same checks, order and messages as the reference (torch_binding.py:195-229)."""
-    check_type(emissions, torch.float32, "emissions")
-    check_type(predictions, torch.float32, "predictions")
+    check_type(emissions, score_dtype, "emissions")
+    check_type(predictions, score_dtype, "predictions")
     check_type(labels, torch.int32, "labels")
     check_type(input_lengths, torch.int32, "input_lengths")
     check_type(label_lengths, torch.int32, "label_lengths")
