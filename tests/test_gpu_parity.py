@@ -328,6 +328,22 @@ def test_whole_loss_cfg1(cfg, seed):
         assert_close(pg, f["pgrads"], what="pgrads vs reference fixture")
 
 
+@pytest.mark.parametrize("T,U,V", [(60, 150, 36), (60, 150, 37), (40, 260, 16), (33, 113, 520)])
+def test_whole_loss_with_a_label_axis_past_the_streaming_kernels(T, U, V):
+    """More than 112 label positions: egrads falls back to the general kernel (slice by slice
+    over the label axis) and the blank/label terms are scattered; odd V also takes the general
+    log-normaliser.  Same entry points, same bar."""
+    cfg = small_config(2, T, U, V, ragged=True)
+    E, P, labels, il, ll = unpack(make_inputs(cfg, seed=T + U + V))
+    want = oracle.loss_and_grads(E, P, labels, il, ll)
+    costs, eg, pg = gpu_loss(DeviceCase(E, P, labels, il, ll))
+    assert_close(costs, want["costs"], what="costs")
+    assert_close(eg, want["egrads"], what="egrads")
+    assert_close(pg, want["pgrads"], what="pgrads")
+    for b in range(2):
+        assert not eg[b, il[b]:].any() and not pg[b, ll[b] + 1:].any()
+
+
 def test_whole_loss_handles_empty_utterance_and_empty_label():
     cfg = small_config(4, 20, 6, 12, ragged=True)
     E, P, labels, il, ll = unpack(make_inputs(cfg, seed=2))
