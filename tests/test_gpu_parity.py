@@ -126,7 +126,7 @@ def test_reference_stress_grid(B, T):
             assert_close(pd, pd_o, what="pgrads")
             # and the fused path, which computes log_norms itself (a last-bit difference there
             # moves a rounding in alpha, ~6e-5 at |alpha| ~ 1e3): held to the reference's own
-            # bar for this test (test_cuda.cu:373-375)
+            # bar for this test (test_cuda.cu:371-373)
             costs_f, ed_f, pd_f = gpu_loss(c)
             fin = np.isfinite(costs_o)
             assert np.array_equal(np.isinf(costs_f), np.isinf(costs_o))
@@ -335,11 +335,20 @@ def test_whole_loss_with_a_label_axis_past_the_streaming_kernels(T, U, V):
     log-normaliser.  Same entry points, same bar."""
     cfg = small_config(2, T, U, V, ragged=True)
     E, P, labels, il, ll = unpack(make_inputs(cfg, seed=T + U + V))
-    want = oracle.loss_and_grads(E, P, labels, il, ll)
+    want = oracle.loss_and_grads(E, P, labels, il, ll, lse="naive")
+    other = oracle.loss_and_grads(E, P, labels, il, ll, lse="sep")
     costs, eg, pg = gpu_loss(DeviceCase(E, P, labels, il, ll))
     assert_close(costs, want["costs"], what="costs")
-    assert_close(eg, want["egrads"], what="egrads")
-    assert_close(pg, want["pgrads"], what="pgrads")
+    # a lattice this long along the label axis moves by more than the tolerance when LN moves in
+    # its last bits: the bar is the oracle's own spread between its two summation orders of LN
+    for got, name in ((eg, "egrads"), (pg, "pgrads")):
+        floor, _ = violations(other[name], want[name])
+        frac, worst = violations(got, want[name])
+        print("%s: %.4f%% outside (oracle's own two LN orders: %.4f%%), max abs err %.3g"
+              % (name, 100 * frac, 100 * floor, worst))
+        assert frac <= max(2 * floor, 1e-3)
+        # and nothing is far off: the reference's own CPU/GPU bar (test_cuda.cu:371-373)
+        assert violations(got, want[name], rtol=1e-3, atol=1e-4)[0] == 0.0
     for b in range(2):
         assert not eg[b, il[b]:].any() and not pg[b, ll[b] + 1:].any()
 
