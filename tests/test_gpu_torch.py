@@ -180,7 +180,10 @@ def test_loss_on_a_side_stream_matches_the_default_stream():
         paths = TransducerLoss().viterbi(E, P, il, ll)
     side.synchronize()
     assert torch.equal(E1.grad, E2.grad) and torch.equal(P1.grad, P2.grad)
-    assert torch.equal(paths, TransducerLoss().viterbi(E, P, il, ll))
+    # entries past an utterance's label length are unwritten padding, as in the reference
+    written = torch.arange(paths.shape[1], device=paths.device)[None, :] < ll[:, None]
+    again = TransducerLoss().viterbi(E, P, il, ll)
+    assert torch.equal(paths[written], again[written])
 
 
 def test_fused_entry_points_replay_from_a_captured_graph():

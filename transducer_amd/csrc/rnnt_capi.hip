@@ -148,7 +148,7 @@ int log_norms_stages(const float* E, const float* P, float* mE, float* mP, float
 
 struct LossWorkspace {
   Planes planes;
-  float *mE, *mP, *LN, *lngrads, *Wn, *Wt, *bsum;
+  float *mE, *mP, *LN, *Wn, *Wt, *bsum;
   void* lse_scratch;
 };
 
@@ -167,14 +167,13 @@ size_t loss_workspace_layout(const Dims& d, void* base, LossWorkspace* w) {
   float* mE = take(sizeof(float) * (size_t)d.B * d.T);
   float* mP = take(sizeof(float) * (size_t)d.B * d.U);
   float* LN = take(btu);
-  float* lng = take(btu);
   const size_t wb = sizeof(float) * (size_t)d.B * wplane_tw(d.T) * wplane_up(d.U);
   float* Wn = take(wb);
   float* Wt = take(wb);
   float* bsum = take(sizeof(float) * (size_t)d.B * d.T);
   void* ys = take(lse_scratch_bytes(d));  // forward only
   if (base) {
-    w->mE = mE; w->mP = mP; w->LN = LN; w->lngrads = lng; w->Wn = Wn; w->Wt = Wt; w->bsum = bsum;
+    w->mE = mE; w->mP = mP; w->LN = LN; w->Wn = Wn; w->Wt = Wt; w->bsum = bsum;
     w->lse_scratch = lse_scratch_bytes(d) ? ys : nullptr;
   }
   return off;
@@ -416,8 +415,8 @@ int rnnt_hip_loss_backward(const float* E, const float* P, const int* labels, co
   loss_workspace_layout(d, workspace, &w);
   RNNT_STAGE(kWeights, launch_weights(w.planes, inLen, labLen, d, s));
   RNNT_STAGE(kBeta, launch_beta(w.planes, labels, inLen, labLen, d, s));
-  RNNT_STAGE(kUnskew, launch_unskew(w.planes.dS, w.lngrads, inLen, labLen, d, s));
-  RNNT_STAGE(kWplanes, launch_wplanes(w.lngrads, w.LN, w.mE, w.mP, w.Wn, w.Wt, inLen, labLen, d, s));
+  RNNT_STAGE(kWplanes, launch_wplanes_skewed(w.planes.dS, w.planes.lnS, w.mE, w.mP, w.Wn, w.Wt,
+                                             inLen, labLen, d, s));
   // The blank/label terms of egrads are folded into the dense kernel's write-out (a scatter
   // afterwards would touch one cache line of the 2.5 GB array per lattice cell); for label axes
   // too long for that kernel they are scattered as in rnnt_hip_backward.
@@ -523,8 +522,8 @@ int rnnt_hip_loss_backward_bf16(const uint16_t* E16, const uint16_t* P16, const 
   loss_workspace_layout(d, workspace, &w);
   RNNT_STAGE(kWeights, launch_weights(w.planes, inLen, labLen, d, s));
   RNNT_STAGE(kBeta, launch_beta(w.planes, labels, inLen, labLen, d, s));
-  RNNT_STAGE(kUnskew, launch_unskew(w.planes.dS, w.lngrads, inLen, labLen, d, s));
-  RNNT_STAGE(kWplanes, launch_wplanes(w.lngrads, w.LN, w.mE, w.mP, w.Wn, w.Wt, inLen, labLen, d, s));
+  RNNT_STAGE(kWplanes, launch_wplanes_skewed(w.planes.dS, w.planes.lnS, w.mE, w.mP, w.Wn, w.Wt,
+                                             inLen, labLen, d, s));
   // Both gradients are rounded to bf16 once, from the complete fp32 value: the blank / label
   // terms are always folded into the dense kernels' write-outs here, whatever the vocabulary.
   // With U == 1 there are no labels; the kernels then never read the list, but its pointer is

@@ -170,6 +170,10 @@ int launch_rowmax_pick_p(const bf16_t* P, float* mP, const int* labels, const in
 int launch_wplanes(const float* lngrads, const float* LN, const float* mE, const float* mP,
                    float* Wn, float* Wt, const int* inLen, const int* labLen, const Dims& d,
                    hipStream_t s);
+// The same from the skewed dalpha and LN planes of the lattice kernels.
+int launch_wplanes_skewed(const float* dS, const float* lnS, const float* mE, const float* mP,
+                          float* Wn, float* Wt, const int* inLen, const int* labLen,
+                          const Dims& d, hipStream_t s);
 // Sparse blank/label terms of egrads for folding into the dense kernel's write-out: with
 // labels != nullptr, out = delta * (dense + sparse) (needs accumulate == false and a label axis
 // short enough for the streaming kernel, see egrads_fusion_supported).
