@@ -57,6 +57,8 @@ WORKLOADS = {
                    uniform=True, published_ms=223.33),
     # the headline shape with bf16 scores and gradients (rnnt_hip_loss_*_bf16; not a reference
     # configuration: the reference takes float32 only)
+    "cfg5bf16": dict(B=32, T=2000, U=100, V=10000, sigma=1.0, ragged_T=(1500, 2000),
+                     ragged_U=(75, 100), kind="viterbi", io="bf16"),
     "cfg4bf16": dict(B=32, T=2000, U=100, V=10000, sigma=1.0, ragged_T=(1500, 2000),
                      ragged_U=(75, 100), io="bf16"),
 }
@@ -160,10 +162,13 @@ def viterbi_main(args, w, capi, E, P, d_il, d_ll, il, ll):
     out_labels = torch.empty((B, U1 - 1), dtype=torch.int32, device=E.device)
     stream = ctypes.c_void_p(torch.cuda.current_stream(E.device).cuda_stream)
     p = lambda t: ctypes.c_void_p(t.data_ptr())
+    bf16 = w.get("io") == "bf16"
+    if bf16:
+        E, P = E.to(torch.bfloat16), P.to(torch.bfloat16)
+    entry = "rnnt_hip_viterbi_decode" + ("_bf16" if bf16 else "")
 
     def step():
-        capi.call("rnnt_hip_viterbi_decode", p(E), p(P), p(d_il), p(d_ll), p(out_labels), B, T, U1,
-                  V, 0, stream)
+        capi.call(entry, p(E), p(P), p(d_il), p(d_ll), p(out_labels), B, T, U1, V, 0, stream)
 
     for _ in range(args.warmup):
         step()
@@ -187,7 +192,8 @@ def viterbi_main(args, w, capi, E, P, d_il, d_ll, il, ll):
         "metric": "ms per teacher-forced viterbi decode, B=%d T=%d U=%d V=%d" % (B, T, w["U"], V),
         "value": round(ms_per_step, 4), "unit": "ms", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": False,
-        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32 arithmetic on bf16 scores" if bf16 else "f32", "data": "synthetic",
         "config": {"workload": "%s: B=%d T=%d U=%d V=%d blank=0, N(0,1) scores%s, input_lengths "
                                "U[%d,%d], label_lengths U[%d,%d]"
                                % ((args.workload, B, T, w["U"], V,

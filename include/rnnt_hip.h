@@ -122,6 +122,12 @@ int rnnt_hip_loss_backward_bf16(const uint16_t* emissions, const uint16_t* predi
                                 uint16_t* pgrads, void* workspace, size_t workspace_bytes, int B,
                                 int T, int U, int V, int blank, rnnt_stream_t stream);
 
+/* rnnt_hip_viterbi_decode for bf16 scores (V a multiple of 8, 16-byte aligned arrays; any U up
+ * to 1024).  The path is the one rnnt_hip_viterbi_decode finds on the same values in fp32. */
+int rnnt_hip_viterbi_decode_bf16(const uint16_t* emissions, const uint16_t* predictions,
+                                 const int* input_lengths, const int* label_lengths, int* labels,
+                                 int B, int T, int U, int V, int blank, rnnt_stream_t stream);
+
 /* Replaces TransducerLoss.viterbi (transducer/torch_binding.py:130-177): log-normaliser +
  * best path.  labels is int [B, U-1]. */
 int rnnt_hip_viterbi_decode(const float* emissions, const float* predictions,

@@ -1,4 +1,5 @@
-"""bf16 scores and gradients through rnnt_hip_loss_forward_bf16 / rnnt_hip_loss_backward_bf16.
+"""bf16 scores and gradients through rnnt_hip_loss_forward_bf16 / rnnt_hip_loss_backward_bf16,
+and the best path through rnnt_hip_viterbi_decode_bf16.
 
 The reference takes float32 only (transducer/torch_binding.py:195-201), so there is no reference
 output to match.  What pins these entry points:
@@ -246,3 +247,64 @@ def test_bf16_headline_configuration_against_the_fp32_path():
     # both paths fold the sparse terms of egrads at this vocabulary: the same fp32 value, rounded
     assert torch.equal(eg, e32.to(torch.bfloat16))
     assert_rounds_the_fp32_result(pg, p32, "pgrads", 0.9999)
+
+
+# ------------------------------------------------------------------ best path
+def decode_bf16(E, P, il, ll, blank=0):
+    B, T, V = E.shape
+    U = P.shape[1]
+    out = torch.full((B, U - 1), -1, dtype=torch.int32, device="cuda:0")
+    d_il, d_ll = dev(il), dev(ll)
+    capi.call("rnnt_hip_viterbi_decode_bf16", ptr(E), ptr(P), ptr(d_il), ptr(d_ll), ptr(out),
+              B, T, U, V, blank, None)
+    torch.cuda.synchronize()
+    return out
+
+
+def decode_fp32(E, P, il, ll, blank=0):
+    E, P = E.float().contiguous(), P.float().contiguous()
+    B, T, V = E.shape
+    U = P.shape[1]
+    out = torch.full((B, U - 1), -1, dtype=torch.int32, device="cuda:0")
+    d_il, d_ll = dev(il), dev(ll)
+    capi.call("rnnt_hip_viterbi_decode", ptr(E), ptr(P), ptr(d_il), ptr(d_ll), ptr(out),
+              B, T, U, V, blank, None)
+    torch.cuda.synchronize()
+    return out
+
+
+@pytest.mark.parametrize("B,T,U,V,blank", [(3, 37, 9, 64, 0), (2, 64, 33, 128, 5),
+                                           (2, 300, 130, 40, 0), (4, 50, 11, 32, 31)])
+def test_bf16_best_path_is_the_fp32_path_and_the_oracles(B, T, U, V, blank):
+    """bf16 scores are exact in fp32 and the decode has no rounding step of its own, so the
+    path must be the fp32 decode's on the upcast scores, label for label; the oracle is fed the
+    device's log-normaliser, as in the fp32 tests (the path is bit-exact GIVEN LN)."""
+    E, P, _, il, ll = draw(B, T, U, V, seed=7 * B + T + U + V)
+    ll = np.maximum(ll, 1).astype(np.int32)
+    got = decode_bf16(E, P, il, ll, blank)
+    ref = decode_fp32(E, P, il, ll, blank)
+    assert torch.equal(got, ref)
+    E32, P32 = E.float().contiguous(), P.float().contiguous()
+    LN = torch.empty((B, T, U), device="cuda:0")
+    d_il, d_ll = dev(il), dev(ll)
+    capi.call("rnnt_hip_log_norms", ptr(E32), ptr(P32), ptr(LN), ptr(d_il), ptr(d_ll),
+              B, T, U, V, None)
+    want = oracle.viterbi(E32.cpu().numpy(), P32.cpu().numpy(), LN.cpu().numpy(), il, ll,
+                          blank=blank)
+    g = got.cpu().numpy()
+    for b in range(B):
+        assert np.array_equal(g[b, :ll[b]], want[b, :ll[b]])
+        assert (g[b, ll[b]:] == -1).all()
+
+
+def test_bf16_best_path_through_the_torch_module():
+    from transducer_amd import TransducerLoss
+    B, T, U, V = 3, 40, 8, 48
+    E, P, _, il, ll = draw(B, T, U, V, seed=3)
+    d_il, d_ll = dev(il), dev(ll)
+    with pytest.raises(TypeError, match="emissions must be torch.float32"):
+        TransducerLoss().viterbi(E, P, d_il, d_ll)
+    paths = TransducerLoss(allow_bf16=True).viterbi(E, P, d_il, d_ll)
+    ref = decode_bf16(E, P, il, ll)
+    for b in range(B):
+        assert torch.equal(paths[b, :ll[b]], ref[b, :ll[b]])

@@ -185,6 +185,20 @@ PYBIND11_MODULE(_transducer, m) {
         "batch_size"_a, "max_input_length"_a, "max_label_length"_a, "alphabet_size"_a, "blank"_a,
         "stream"_a = 0);
 
+  m.def("viterbi_decode_bf16",
+        [](ptr_t emissions, ptr_t predictions, ptr_t input_lengths, ptr_t label_lengths,
+           ptr_t labels, int batch_size, int max_input_length, int max_label_length,
+           int alphabet_size, int blank, ptr_t stream) {
+          raise_on(rnnt_hip_viterbi_decode_bf16(
+              as<const uint16_t>(emissions), as<const uint16_t>(predictions),
+              as<const int>(input_lengths), as<const int>(label_lengths), as<int>(labels),
+              batch_size, max_input_length, max_label_length, alphabet_size, blank,
+              as<void>(stream)));
+        },
+        "emissions"_a, "predictions"_a, "input_lengths"_a, "label_lengths"_a, "labels"_a,
+        "batch_size"_a, "max_input_length"_a, "max_label_length"_a, "alphabet_size"_a, "blank"_a,
+        "stream"_a = 0);
+
 #ifdef VERSION_INFO
   m.attr("__version__") = VERSION_INFO;
 #else

@@ -191,6 +191,32 @@ int fill(float* x, float v, int n, hipStream_t s) {
   return check_hip(hipGetLastError(), "launch fill_kernel", __FILE__, __LINE__);
 }
 
+template <typename TIO>
+int viterbi_impl(const TIO* E, const TIO* P, const float* LN, int* labels,
+                        const int* inLen, const int* labLen, const Dims& d, hipStream_t s) {
+  const size_t btu = sizeof(float) * (size_t)d.B * d.T * d.U;
+  const size_t plane = sizeof(float) * (size_t)d.B * d.Ua * d.Dp + 64;
+  Scratch scratch(s);
+  RNNT_TRY(scratch.reserve(align_up(planes_bytes(d)) + 2 * align_up(btu) + 2 * align_up(plane) +
+                           align_up(viterbi_bits_bytes(d))));
+  Planes p;
+  carve_planes(scratch.take(planes_bytes(d)), d, &p);
+  float* best = static_cast<float*>(scratch.take(btu));
+  int* arg = static_cast<int*>(scratch.take(btu));
+  float* bestS = static_cast<float*>(scratch.take(plane));
+  float* argS = static_cast<float*>(scratch.take(plane));
+  unsigned long long* bits =
+      static_cast<unsigned long long*>(scratch.take(viterbi_bits_bytes(d)));
+  RNNT_STAGE(kMaxplus, launch_maxplus(E, P, inLen, labLen, best, arg, d, s));
+  RNNT_STAGE(kSkew, launch_skew(LN, p.lnS, inLen, labLen, d, s));
+  RNNT_STAGE(kSkew, launch_skew(best, bestS, inLen, labLen, d, s));
+  RNNT_STAGE(kSkew, launch_skew(reinterpret_cast<const float*>(arg), argS, inLen, labLen, d, s));
+  // blank scores only: the label planes of the gather are not needed here
+  RNNT_STAGE(kGather, launch_gather(E, P, nullptr, inLen, labLen, p, d, s));
+  RNNT_STAGE(kViterbi, launch_viterbi(p, bestS, argS, bits, inLen, labLen, labels, d, s));
+  return kOk;
+}
+
 }  // namespace
 }  // namespace rnnt
 
@@ -275,31 +301,6 @@ int rnnt_hip_backward(const float* E, const float* P, float* egrads, float* pgra
   RNNT_STAGE(kBeta, launch_beta(p, labels, inLen, labLen, d, s));
   RNNT_STAGE(kUnskew, launch_unskew(p.dS, lngrads, inLen, labLen, d, s));
   RNNT_STAGE(kSparse, launch_sparse(p, egrads, pgrads, labels, inLen, labLen, nullptr, false, d, s));
-  return kOk;
-}
-
-static int viterbi_impl(const float* E, const float* P, const float* LN, int* labels,
-                        const int* inLen, const int* labLen, const Dims& d, hipStream_t s) {
-  const size_t btu = sizeof(float) * (size_t)d.B * d.T * d.U;
-  const size_t plane = sizeof(float) * (size_t)d.B * d.Ua * d.Dp + 64;
-  Scratch scratch(s);
-  RNNT_TRY(scratch.reserve(align_up(planes_bytes(d)) + 2 * align_up(btu) + 2 * align_up(plane) +
-                           align_up(viterbi_bits_bytes(d))));
-  Planes p;
-  carve_planes(scratch.take(planes_bytes(d)), d, &p);
-  float* best = static_cast<float*>(scratch.take(btu));
-  int* arg = static_cast<int*>(scratch.take(btu));
-  float* bestS = static_cast<float*>(scratch.take(plane));
-  float* argS = static_cast<float*>(scratch.take(plane));
-  unsigned long long* bits =
-      static_cast<unsigned long long*>(scratch.take(viterbi_bits_bytes(d)));
-  RNNT_STAGE(kMaxplus, launch_maxplus(E, P, inLen, labLen, best, arg, d, s));
-  RNNT_STAGE(kSkew, launch_skew(LN, p.lnS, inLen, labLen, d, s));
-  RNNT_STAGE(kSkew, launch_skew(best, bestS, inLen, labLen, d, s));
-  RNNT_STAGE(kSkew, launch_skew(reinterpret_cast<const float*>(arg), argS, inLen, labLen, d, s));
-  // blank scores only: the label planes of the gather are not needed here
-  RNNT_STAGE(kGather, launch_gather(E, P, nullptr, inLen, labLen, p, d, s));
-  RNNT_STAGE(kViterbi, launch_viterbi(p, bestS, argS, bits, inLen, labLen, labels, d, s));
   return kOk;
 }
 
@@ -541,6 +542,41 @@ int rnnt_hip_loss_backward_bf16(const uint16_t* E16, const uint16_t* P16, const 
                                            reinterpret_cast<bf16_t*>(pgrads16), inLen, labLen, d,
                                            false, spp, s));
   return kOk;
+}
+
+int rnnt_hip_viterbi_decode_bf16(const uint16_t* E16, const uint16_t* P16, const int* inLen,
+                                 const int* labLen, int* labels, int B, int T, int U, int V,
+                                 int blank, rnnt_stream_t stream) {
+  RNNT_TRY(check_dims(B, T, U, V));
+  if (nothing_to_do(B, T, U) || U == 1) return kOk;  // no label to emit
+  if (V == 0) return fail(kInvalid, "viterbi_decode_bf16: empty vocabulary");
+  if (!E16 || !P16 || !labels || !inLen || !labLen)
+    return fail(kInvalid, "viterbi_decode_bf16: null array argument");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const Dims d = make_dims(B, T, U, V, blank);
+  if (d.V % 8 != 0)
+    return fail(kInvalid, "viterbi_decode_bf16: bf16 scores need a vocabulary that is a "
+                          "multiple of 8 (V=%d)", d.V);
+  if ((reinterpret_cast<uintptr_t>(E16) | reinterpret_cast<uintptr_t>(P16)) & 15)
+    return fail(kInvalid, "viterbi_decode_bf16: bf16 scores must be 16-byte aligned");
+  const bf16_t* E = reinterpret_cast<const bf16_t*>(E16);
+  const bf16_t* P = reinterpret_cast<const bf16_t*>(P16);
+  if (!lse_stream_supported(E, d))
+    return fail(kInvalid, "viterbi_decode_bf16: B*T*U too large for the bf16 path");
+  Scratch scratch(s);
+  const size_t btu = sizeof(float) * (size_t)B * T * U;
+  const size_t yb = lse_scratch_bytes(d);
+  RNNT_TRY(scratch.reserve(align_up(sizeof(float) * (size_t)B * T) +
+                           align_up(sizeof(float) * (size_t)B * U) + align_up(btu) +
+                           align_up(yb)));
+  float* mE = static_cast<float*>(scratch.take(sizeof(float) * (size_t)B * T));
+  float* mP = static_cast<float*>(scratch.take(sizeof(float) * (size_t)B * U));
+  float* LN = static_cast<float*>(scratch.take(btu));
+  void* ys = scratch.take(yb);
+  RNNT_STAGE(kRowmax, launch_rowmax(P, mP, (long)B * U, V, U, labLen, 1, s));
+  RNNT_STAGE(kYplanes, launch_yplanes(P, mP, ys, labLen, d, s));
+  RNNT_STAGE(kLse, launch_lse_stream(E, mE, mP, LN, ys, inLen, labLen, d, s));
+  return viterbi_impl(E, P, LN, labels, inLen, labLen, d, s);
 }
 
 int rnnt_hip_viterbi_decode(const float* E, const float* P, const int* inLen, const int* labLen,

@@ -119,8 +119,9 @@ __global__ __launch_bounds__(256) void unskew_kernel(const float* __restrict__ s
 // ------------------------------------------------------------------ gather
 // elS[u][t+u] = E[t, label_u]; eb[t] = E[t, blank]; pb[u] = P[u, blank]; pl[u] = P[u, label_u].
 // grid (ceil(T/256), U, B): a block serves 256 frames of one label position.
-__global__ __launch_bounds__(256) void gather_kernel(const float* __restrict__ E,
-                                                     const float* __restrict__ P,
+template <typename TIO>
+__global__ __launch_bounds__(256) void gather_kernel(const TIO* __restrict__ E,
+                                                     const TIO* __restrict__ P,
                                                      const int* __restrict__ labels,
                                                      const int* __restrict__ inLen,
                                                      const int* __restrict__ labLen, Planes p,
@@ -132,15 +133,15 @@ __global__ __launch_bounds__(256) void gather_kernel(const float* __restrict__ E
   if (u >= Ub) return;
   const bool has_label = labels != nullptr && (u + 1 < Ub);
   const int l = has_label ? labels[(size_t)b * (d.U - 1) + u] : d.blank;
-  const float* Eb = E + (size_t)b * d.T * d.V;
+  const TIO* Eb = E + (size_t)b * d.T * d.V;
   if (t < Tb) {
-    if (has_label) p.elS[plane_row(d, b, u) + t + u] = Eb[(size_t)t * d.V + l];
-    if (u == 0) p.eb[(size_t)b * d.Tp + d.Eo + t] = Eb[(size_t)t * d.V + d.blank];
+    if (has_label) p.elS[plane_row(d, b, u) + t + u] = ldf(Eb + (size_t)t * d.V + l);
+    if (u == 0) p.eb[(size_t)b * d.Tp + d.Eo + t] = ldf(Eb + (size_t)t * d.V + d.blank);
   }
   if (blockIdx.x == 0 && threadIdx.x == 0) {
-    const float* Pu = P + ((size_t)b * d.U + u) * d.V;
-    p.pb[(size_t)b * d.Ua + u] = Pu[d.blank];
-    p.pl[(size_t)b * d.Ua + u] = has_label ? Pu[l] : 0.0f;
+    const TIO* Pu = P + ((size_t)b * d.U + u) * d.V;
+    p.pb[(size_t)b * d.Ua + u] = ldf(Pu + d.blank);
+    p.pl[(size_t)b * d.Ua + u] = has_label ? ldf(Pu + l) : 0.0f;
   }
 }
 
@@ -584,10 +585,11 @@ constexpr int kMpT = 128, kMpK = 32, kMpPitch = 36, kMpRows = 8;
 constexpr int kMpWaves = 8, kMpU = kMpWaves * kMpRows, kMpThreads = 64 * kMpWaves;
 constexpr int kMpEPasses = kMpT * (kMpK / 4) / kMpThreads;  // 16-byte pieces of the E chunk per thread
 
-// kVec: V is a multiple of 4, so every row of E starts on a 16-byte boundary.
-template <bool kVec>
-__global__ __launch_bounds__(kMpThreads) void maxplus_kernel(const float* __restrict__ E,
-                                                       const float* __restrict__ P,
+// kVec: V is a multiple of 4, so four consecutive elements never straddle a row's end and every
+// group of four is naturally aligned (16 bytes in fp32, 8 in bf16).
+template <bool kVec, typename TIO>
+__global__ __launch_bounds__(kMpThreads) void maxplus_kernel(const TIO* __restrict__ E,
+                                                       const TIO* __restrict__ P,
                                                        const int* __restrict__ inLen,
                                                        const int* __restrict__ labLen,
                                                        float* __restrict__ best,
@@ -600,15 +602,15 @@ __global__ __launch_bounds__(kMpThreads) void maxplus_kernel(const float* __rest
   if (t0 >= Tb || u0 >= Ub) return;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const float* Eb = E + (size_t)b * d.T * d.V;
-  const float* Pb = P + (size_t)b * d.U * d.V;
+  const TIO* Eb = E + (size_t)b * d.T * d.V;
+  const TIO* Pb = P + (size_t)b * d.U * d.V;
   const int ur0 = u0 + wave * kMpRows;  // first label position of this wavefront
   const bool active = ur0 < Ub;
 
   // staging role: thread -> row srow of the P tile and rows srow + (kMpThreads/8) * i of the E
   // tile, four columns from sc4
   const int srow = tid >> 3, sc4 = (tid & 7) * 4;
-  const float* esrc[kMpEPasses];
+  const TIO* esrc[kMpEPasses];
   bool erow_ok[kMpEPasses];
 #pragma unroll
   for (int i = 0; i < kMpEPasses; ++i) {
@@ -616,21 +618,21 @@ __global__ __launch_bounds__(kMpThreads) void maxplus_kernel(const float* __rest
     erow_ok[i] = t < Tb;
     esrc[i] = Eb + (size_t)min(t, Tb - 1) * d.V;
   }
-  const float* psrc = Pb + (size_t)min(u0 + srow, Ub - 1) * d.V;  // rows past the utterance are
+  const TIO* psrc = Pb + (size_t)min(u0 + srow, Ub - 1) * d.V;  // rows past the utterance are
                                                                   // computed and dropped
   // the raw values are requested before a chunk's arithmetic and stored after it, so the wait
   // for them falls behind the arithmetic
-  auto fetch = [&](const float* src, int k) -> float4 {
+  auto fetch = [&](const TIO* src, int k) -> float4 {
     const int v = k * kMpK + sc4;
     float4 x;
     if (kVec) {  // columns past V are re-read from the row's last four (E: masked below; P: any
                  // finite value will do there, E is -inf)
-      x = *reinterpret_cast<const float4*>(src + min(v, d.V - 4));
+      x = load4(src + min(v, d.V - 4));
     } else {
-      x.x = src[min(v, d.V - 1)];
-      x.y = src[min(v + 1, d.V - 1)];
-      x.z = src[min(v + 2, d.V - 1)];
-      x.w = src[min(v + 3, d.V - 1)];
+      x.x = ldf(src + min(v, d.V - 1));
+      x.y = ldf(src + min(v + 1, d.V - 1));
+      x.z = ldf(src + min(v + 2, d.V - 1));
+      x.w = ldf(src + min(v + 3, d.V - 1));
     }
     return x;
   };
@@ -724,11 +726,11 @@ __global__ __launch_bounds__(kMpThreads) void maxplus_kernel(const float* __rest
       int at = 0;  // :160 the scan starts from index 0 and keeps it if nothing beats -inf
       if (chunk[i][r] >= 0) {
         const int v0 = chunk[i][r] * kMpK;
-        const float* e = Eb + (size_t)t * d.V;
-        const float* q = Pb + (size_t)u * d.V;
+        const TIO* e = Eb + (size_t)t * d.V;
+        const TIO* q = Pb + (size_t)u * d.V;
         for (int v = v0; v < v0 + kMpK && v < d.V; ++v) {
           if (v == d.blank) continue;
-          if (e[v] + q[v] == top[i][r]) { at = v; break; }
+          if (ldf(e + v) + ldf(q + v) == top[i][r]) { at = v; break; }
         }
       }
       const size_t o = ((size_t)b * d.T + t) * d.U + u;
@@ -970,13 +972,22 @@ int launch_unskew(const float* srcS, float* dst, const int* inLen, const int* la
   return kOk;
 }
 
-int launch_gather(const float* E, const float* P, const int* labels, const int* inLen,
-                  const int* labLen, const Planes& p, const Dims& d, hipStream_t s) {
+template <typename TIO>
+static int gather_any(const TIO* E, const TIO* P, const int* labels, const int* inLen,
+                      const int* labLen, const Planes& p, const Dims& d, hipStream_t s) {
   if (d.B == 0 || d.T == 0 || d.U == 0) return kOk;
-  hipLaunchKernelGGL(gather_kernel, dim3((d.T + 255) / 256, d.U, d.B), dim3(256), 0, s, E, P,
+  hipLaunchKernelGGL(gather_kernel<TIO>, dim3((d.T + 255) / 256, d.U, d.B), dim3(256), 0, s, E, P,
                      labels, inLen, labLen, p, d);
   RNNT_LAUNCH_CHECK("gather_kernel");
   return kOk;
+}
+int launch_gather(const float* E, const float* P, const int* labels, const int* inLen,
+                  const int* labLen, const Planes& p, const Dims& d, hipStream_t s) {
+  return gather_any(E, P, labels, inLen, labLen, p, d, s);
+}
+int launch_gather(const bf16_t* E, const bf16_t* P, const int* labels, const int* inLen,
+                  const int* labLen, const Planes& p, const Dims& d, hipStream_t s) {
+  return gather_any(E, P, labels, inLen, labLen, p, d, s);
 }
 
 int launch_alpha(const Planes& p, const int* inLen, const int* labLen, float* costs,
@@ -1054,18 +1065,30 @@ int launch_blank_sums(const Planes& p, float* bsum, const int* labels, const int
   return kOk;
 }
 
-int launch_maxplus(const float* E, const float* P, const int* inLen, const int* labLen,
-                   float* best, int* arg, const Dims& d, hipStream_t s) {
+template <typename TIO>
+static int maxplus_any(const TIO* E, const TIO* P, const int* inLen, const int* labLen,
+                       float* best, int* arg, const Dims& d, hipStream_t s) {
   if (d.B == 0 || d.T == 0 || d.U == 0) return kOk;
   const dim3 grid((d.T + kMpT - 1) / kMpT, (d.U + kMpU - 1) / kMpU, d.B);
-  if (d.V % 4 == 0)
-    hipLaunchKernelGGL(maxplus_kernel<true>, grid, dim3(kMpThreads), 0, s, E, P, inLen, labLen,
-                       best, arg, d);
+  const bool vec = d.V % 4 == 0 &&
+                   ((reinterpret_cast<uintptr_t>(E) | reinterpret_cast<uintptr_t>(P)) &
+                    (4 * sizeof(TIO) - 1)) == 0;
+  if (vec)
+    hipLaunchKernelGGL((maxplus_kernel<true, TIO>), grid, dim3(kMpThreads), 0, s, E, P, inLen,
+                       labLen, best, arg, d);
   else
-    hipLaunchKernelGGL(maxplus_kernel<false>, grid, dim3(kMpThreads), 0, s, E, P, inLen, labLen,
-                       best, arg, d);
+    hipLaunchKernelGGL((maxplus_kernel<false, TIO>), grid, dim3(kMpThreads), 0, s, E, P, inLen,
+                       labLen, best, arg, d);
   RNNT_LAUNCH_CHECK("maxplus_kernel");
   return kOk;
+}
+int launch_maxplus(const float* E, const float* P, const int* inLen, const int* labLen,
+                   float* best, int* arg, const Dims& d, hipStream_t s) {
+  return maxplus_any(E, P, inLen, labLen, best, arg, d, s);
+}
+int launch_maxplus(const bf16_t* E, const bf16_t* P, const int* inLen, const int* labLen,
+                   float* best, int* arg, const Dims& d, hipStream_t s) {
+  return maxplus_any(E, P, inLen, labLen, best, arg, d, s);
 }
 
 // 32-step words per column of the decision table (one spare)

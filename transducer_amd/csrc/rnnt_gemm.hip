@@ -74,7 +74,8 @@ __device__ inline float row_max(const float* __restrict__ x, int V, int vec4, in
   return wave_max(fmaxf(fmaxf(m0, m1), fmaxf(m2, m3)));
 }
 
-__global__ __launch_bounds__(256) void rowmax_kernel(const float* __restrict__ X,
+template <typename TIO>
+__global__ __launch_bounds__(256) void rowmax_kernel(const TIO* __restrict__ X,
                                                      float* __restrict__ out, long rows, int V,
                                                      int vec4, int rows_per_item,
                                                      const int* __restrict__ lengths, int extra) {
@@ -478,14 +479,23 @@ __global__ __launch_bounds__(256, 2) void egrads_kernel(
     if (_e != hipSuccess) return check_hip(_e, "launch " name, __FILE__, __LINE__); \
   } while (0)
 
-int launch_rowmax(const float* X, float* rowmax, long rows, int V, int rows_per_item,
-                  const int* lengths, int extra, hipStream_t s) {
+template <typename TIO>
+static int rowmax_any(const TIO* X, float* rowmax, long rows, int V, int rows_per_item,
+                      const int* lengths, int extra, hipStream_t s) {
   if (rows == 0) return kOk;
-  const int vec4 = (V % 4 == 0) && ((reinterpret_cast<uintptr_t>(X) & 15) == 0);
-  hipLaunchKernelGGL(rowmax_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, s, X, rowmax,
-                     rows, V, vec4, rows_per_item, lengths, extra);
+  const int vec4 = (V % RowAlign<TIO>::kElems == 0) && ((reinterpret_cast<uintptr_t>(X) & 15) == 0);
+  hipLaunchKernelGGL(rowmax_kernel<TIO>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, s, X,
+                     rowmax, rows, V, vec4, rows_per_item, lengths, extra);
   RNNT_LAUNCH_CHECK("rowmax_kernel");
   return kOk;
+}
+int launch_rowmax(const float* X, float* rowmax, long rows, int V, int rows_per_item,
+                  const int* lengths, int extra, hipStream_t s) {
+  return rowmax_any(X, rowmax, rows, V, rows_per_item, lengths, extra, s);
+}
+int launch_rowmax(const bf16_t* X, float* rowmax, long rows, int V, int rows_per_item,
+                  const int* lengths, int extra, hipStream_t s) {
+  return rowmax_any(X, rowmax, rows, V, rows_per_item, lengths, extra, s);
 }
 
 int launch_rowmax_pick(const float* E, const float* P, float* mE, float* mP, const int* labels,

@@ -101,6 +101,8 @@ int launch_unskew(const float* srcS, float* dst, const int* inLen, const int* la
                   const Dims& d, hipStream_t s);
 int launch_gather(const float* E, const float* P, const int* labels, const int* inLen,
                   const int* labLen, const Planes& p, const Dims& d, hipStream_t s);
+int launch_gather(const bf16_t* E, const bf16_t* P, const int* labels, const int* inLen,
+                  const int* labLen, const Planes& p, const Dims& d, hipStream_t s);
 int launch_alpha(const Planes& p, const int* inLen, const int* labLen, float* costs,
                  const Dims& d, hipStream_t s);
 int launch_weights(const Planes& p, const int* inLen, const int* labLen, const Dims& d,
@@ -118,6 +120,8 @@ int launch_blank_sums(const Planes& p, float* bsum, const int* labels, const int
                       const int* labLen, const Dims& d, hipStream_t s);
 int launch_maxplus(const float* E, const float* P, const int* inLen, const int* labLen,
                    float* best, int* arg, const Dims& d, hipStream_t s);
+int launch_maxplus(const bf16_t* E, const bf16_t* P, const int* inLen, const int* labLen,
+                   float* best, int* arg, const Dims& d, hipStream_t s);
 // bestS / argS: skewed planes of the max-plus table (argS carries int bits in float storage).
 int launch_viterbi(const Planes& p, const float* bestS, const float* argS,
                    unsigned long long* gbits, const int* inLen, const int* labLen,
@@ -130,6 +134,8 @@ int wplane_tw(int T);  // frame-axis pitch of the W planes (multiple of 64)
 // Row maxima of a [rows, V] array.  With `lengths`, rows at or past lengths[item] + extra inside
 // their item (rows_per_item rows each) are not read and report 0.
 int launch_rowmax(const float* X, float* rowmax, long rows, int V, int rows_per_item,
+                  const int* lengths, int extra, hipStream_t s);
+int launch_rowmax(const bf16_t* X, float* rowmax, long rows, int V, int rows_per_item,
                   const int* lengths, int extra, hipStream_t s);
 // Row maxima of E and P and, in the same pass, what launch_gather extracts (E[t,blank],
 // E[t,label_u], P[u,blank], P[u,label_u] into the planes); needs inLen and labLen.

@@ -25,6 +25,14 @@ __device__ inline float ldf(const bf16_t* p) { return bf16_to_float(p->bits); }
 __device__ inline void stf(float* p, float v) { *p = v; }
 __device__ inline void stf(bf16_t* p, float v) { p->bits = float_to_bf16(v); }
 
+// Four consecutive, naturally aligned elements (16 bytes of fp32, 8 of bf16).
+__device__ inline float4 load4(const float* p) { return *reinterpret_cast<const float4*>(p); }
+__device__ inline float4 load4(const bf16_t* p) {
+  const uint2 w = *reinterpret_cast<const uint2*>(p);
+  return make_float4(__uint_as_float(w.x << 16), __uint_as_float(w.x & 0xffff0000u),
+                     __uint_as_float(w.y << 16), __uint_as_float(w.y & 0xffff0000u));
+}
+
 // Eight consecutive elements of a row as they sit in registers after the load.
 template <typename T>
 struct Raw8;

@@ -141,12 +141,14 @@ class TransducerLoss(torch.nn.Module):
         B, T, V = emissions.shape
         U = predictions.shape[1]
         labels = torch.empty(size=(B, U - 1), device=device, dtype=torch.int32)
-        certify_inputs(emissions, predictions, labels, input_lengths, label_lengths)
+        bf16 = self.allow_bf16 and emissions.dtype is torch.bfloat16
+        certify_inputs(emissions, predictions, labels, input_lengths, label_lengths,
+                       score_dtype=torch.bfloat16 if bf16 else torch.float32)
         _require_device(emissions)
         emissions = emissions.contiguous()
         predictions = predictions.contiguous()
         with DeviceManager(device):
-            _transducer.viterbi_decode(
+            (_transducer.viterbi_decode_bf16 if bf16 else _transducer.viterbi_decode)(
                 emissions.data_ptr(), predictions.data_ptr(), input_lengths.data_ptr(),
                 label_lengths.data_ptr(), labels.data_ptr(), B, T, U, V, self.blank,
                 _stream(device))
