@@ -527,7 +527,27 @@ __global__ __launch_bounds__(256) void blank_sums_kernel(Planes p, float* __rest
   const float* __restrict__ wE = p.wE;
   const bool has_stay = t + 1 < Tb;
   float acc = (t == Tb - 1) ? -1.0f : 0.0f;
-  for (int u = Ub - 1; u >= 0; --u) {
+  // eight label positions per trip: their sixteen loads are requested together, the
+  // subtractions keep the reference's order
+  int u = Ub - 1;
+  for (; u >= 7; u -= 8) {
+    float ne[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const size_t o = plane_row(d, b, u - k) + t + (u - k);
+      ne[k] = dS[o + 1] * wB[o];
+    }
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      acc -= has_stay ? ne[k] : 0.0f;
+      const int uu = u - k;
+      if (uu + 1 < Ub && lab[uu] == d.blank) {
+        const size_t o = plane_row(d, b, uu) + t + uu;
+        acc -= dS[o + d.Dp + 1] * wE[o];
+      }
+    }
+  }
+  for (; u >= 0; --u) {
     const size_t o = plane_row(d, b, u) + t + u;
     const float ne = dS[o + 1] * wB[o];
     acc -= has_stay ? ne : 0.0f;
