@@ -14,21 +14,27 @@ from . import _transducer
 
 
 class DeviceManager(object):
-    """Makes the tensors' device current for the duration of a library call
-    (reference: torch_binding.py:7-20)."""
+    """``with DeviceManager(device):`` runs its body with `device` as torch's current HIP device
+    and puts the previous one back afterwards, as the reference brackets every library call
+    (torch_binding.py:7-20): the library works on the current device's pointers."""
 
     def __init__(self, device):
         self.device = device
         self.is_cuda = device.type == "cuda"
+        self._previous = None
 
     def __enter__(self):
-        if self.is_cuda:
-            self.old_device = torch.cuda.current_device()
-            torch.cuda.set_device(self.device)
+        if not self.is_cuda:
+            return self
+        self._previous = torch.cuda.current_device()
+        torch.cuda.set_device(self.device)
+        return self
 
-    def __exit__(self, exc_type, exc_value, traceback):
-        if self.is_cuda:
-            torch.cuda.set_device(self.old_device)
+    def __exit__(self, *exc_info):
+        if self._previous is not None:
+            torch.cuda.set_device(self._previous)
+            self._previous = None
+        return False
 
 
 def _require_device(tensor):
@@ -91,17 +97,18 @@ class Transducer(torch.autograd.Function):
 
 
 class TransducerLoss(torch.nn.Module):
-    """
-    The RNN-T loss function.
+    """RNN transducer loss: per-utterance negative log-likelihood of the label sequence, summed
+    over all alignments of the joint scores ``emissions[b,t,:] + predictions[b,u,:]``.
 
-    All input tensors must be on the same HIP device.
+    Same constructor and call signature as the reference's module (torch_binding.py:93-128);
+    every tensor has to sit on one HIP device.
 
-    Arguments:
-        blank (int, optional): Integer id of blank label (default is 0).
-        allow_bf16 (bool, optional): also accept ``torch.bfloat16`` emissions and predictions
-            (both), returning float32 costs and bfloat16 gradients.  Not in the reference, which
-            raises ``TypeError`` for anything but float32 -- and so does this module by default.
-            Needs a vocabulary that is a multiple of 8 and at most 112 label positions.
+    blank: id of the blank symbol (0 unless given).
+    allow_bf16: when True, ``torch.bfloat16`` emissions and predictions (both) are accepted as
+        well; costs are float32 and the gradients come back as bfloat16.  The reference raises
+        ``TypeError`` for anything but float32, and so does this module unless the flag is set.
+        Needs a vocabulary that is a multiple of 8 and, for the loss, at most 112 label
+        positions.
     """
 
     def __init__(self, blank=0, allow_bf16=False):
@@ -110,33 +117,25 @@ class TransducerLoss(torch.nn.Module):
         self.allow_bf16 = allow_bf16
 
     def forward(self, emissions, predictions, labels, input_lengths, label_lengths):
-        """
-        Arguments:
-          emissions (FloatTensor): unnormalized emission scores,
-            (minibatch, input length, vocab size).
-          predictions (FloatTensor): unnormalized prediction scores,
-            (minibatch, output length + 1, vocab size).
-          labels (IntTensor): (minibatch, output length), padded to the longest label.
-          input_lengths (IntTensor): (minibatch,) input length of each example.
-          label_lengths (IntTensor): (minibatch,) label length of each example.
+        """costs[B] (float32) for a padded batch.
 
-        Returns:
-          costs (FloatTensor): (minibatch,) negative log-likelihood of each example.
-        """
+        emissions:      float32 [B, T, V]     encoder-side scores, unnormalised
+        predictions:    float32 [B, U + 1, V] label-side scores, unnormalised (row u is used
+                                              after u labels have been emitted)
+        labels:         int32   [B, U]        targets, padded to the longest one
+        input_lengths:  int32   [B]           frames in use per utterance
+        label_lengths:  int32   [B]           labels in use per utterance
+
+        Differentiable with respect to emissions and predictions (once)."""
         return Transducer.apply(
             emissions, predictions, labels, input_lengths, label_lengths, self.blank,
             self.allow_bf16)
 
     @torch.no_grad()
     def viterbi(self, emissions, predictions, input_lengths, label_lengths):
-        """
-        Viterbi decoding of the RNN-T graph with teacher-forced predictions and given output
-        lengths (reference: torch_binding.py:130-177).
-
-        Returns:
-          labels (IntTensor): (minibatch, output length); entries past an example's label
-          length are arbitrary padding.
-        """
+        """Best alignment with the prediction rows forced and the number of labels per utterance
+        given; returns the labels on it as int32 [B, U] (reference: torch_binding.py:130-177).
+        Entries past an utterance's label length are unwritten padding."""
         device = emissions.device
         B, T, V = emissions.shape
         U = predictions.shape[1]
@@ -155,55 +154,41 @@ class TransducerLoss(torch.nn.Module):
         return labels
 
 
-def check_type(var, t, name):
-    if var.dtype is not t:
-        raise TypeError("{} must be {}".format(name, t))
-
-
-def check_contiguous(var, name):
-    if not var.is_contiguous():
-        raise ValueError("{} must be contiguous".format(name))
-
-
-def check_dim(var, dim, name):
-    if len(var.shape) != dim:
-        raise ValueError("{} must be {}D".format(name, dim))
-
-
 def certify_inputs(emissions, predictions, labels, input_lengths, label_lengths,
                    score_dtype=torch.float32):
-    """Same checks, order and messages as the reference (torch_binding.py:195-229)."""
-    check_type(emissions, score_dtype, "emissions")
-    check_type(predictions, score_dtype, "predictions")
-    check_type(labels, torch.int32, "labels")
-    check_type(input_lengths, torch.int32, "input_lengths")
-    check_type(label_lengths, torch.int32, "label_lengths")
-    check_contiguous(labels, "labels")
-    check_contiguous(label_lengths, "label_lengths")
-    check_contiguous(input_lengths, "lengths")
-
-    batchSize = emissions.shape[0]
-    if emissions.shape[2] != predictions.shape[2]:
-        raise ValueError("vocab size mismatch.")
-    if input_lengths.shape[0] != batchSize:
-        raise ValueError("must have a length per example.")
-    if label_lengths.shape[0] != batchSize:
-        raise ValueError("must have a label length per example.")
-    if labels.shape[0] != batchSize:
-        raise ValueError("must have a label per example.")
-    if labels.shape[1] != (predictions.shape[1] - 1):
-        raise ValueError("labels must be padded to maximum label length.")
-
-    check_dim(emissions, 3, "emissions")
-    check_dim(predictions, 3, "predictions")
-    check_dim(labels, 2, "labels")
-    check_dim(input_lengths, 1, "input_lengths")
-    check_dim(label_lengths, 1, "label_lengths")
-    max_T = torch.max(input_lengths)
-    max_U = torch.max(label_lengths)
-    T = emissions.shape[1]
-    U = predictions.shape[1]
-    if T < max_T:
+    """Argument validation with the reference's exception types, message texts and ORDER of
+    checks (torch_binding.py:180-229), so a caller sees the same error for the same mistake:
+    element types, then dense storage of the integer arrays, then sizes that must agree, then
+    ranks, then the padded extents against the longest utterance."""
+    named = (("emissions", emissions, score_dtype, 3), ("predictions", predictions, score_dtype, 3),
+             ("labels", labels, torch.int32, 2), ("input_lengths", input_lengths, torch.int32, 1),
+             ("label_lengths", label_lengths, torch.int32, 1))
+    for name, tensor, dtype, _ in named:
+        if tensor.dtype is not dtype:
+            raise TypeError("{} must be {}".format(name, dtype))
+    # (the reference reports input_lengths under the name "lengths" here)
+    for shown, tensor in (("labels", labels), ("label_lengths", label_lengths),
+                          ("lengths", input_lengths)):
+        if not tensor.is_contiguous():
+            raise ValueError("{} must be contiguous".format(shown))
+    # evaluated one after the other: an array of the wrong rank fails in the first relation that
+    # indexes a missing axis, before the rank checks below, exactly as it does upstream
+    batch = emissions.shape[0]
+    agreements = (
+        (lambda: emissions.shape[2] == predictions.shape[2], "vocab size mismatch."),
+        (lambda: input_lengths.shape[0] == batch, "must have a length per example."),
+        (lambda: label_lengths.shape[0] == batch, "must have a label length per example."),
+        (lambda: labels.shape[0] == batch, "must have a label per example."),
+        (lambda: labels.shape[1] == predictions.shape[1] - 1,
+         "labels must be padded to maximum label length."),
+    )
+    for holds, message in agreements:
+        if not holds():
+            raise ValueError(message)
+    for name, tensor, _, rank in named:
+        if tensor.dim() != rank:
+            raise ValueError("{} must be {}D".format(name, rank))
+    if emissions.shape[1] < int(input_lengths.max()):
         raise ValueError("Input length mismatch")
-    if U < max_U + 1:
+    if predictions.shape[1] < int(label_lengths.max()) + 1:
         raise ValueError("Output length mismatch")
