@@ -61,6 +61,8 @@ WORKLOADS = {
                      ragged_U=(75, 100), kind="viterbi", io="bf16"),
     "cfg4bf16": dict(B=32, T=2000, U=100, V=10000, sigma=1.0, ragged_T=(1500, 2000),
                      ragged_U=(75, 100), io="bf16"),
+    "cfg4f16": dict(B=32, T=2000, U=100, V=10000, sigma=1.0, ragged_T=(1500, 2000),
+                    ragged_U=(75, 100), io="f16"),
 }
 PEAK_VALU_TLANEOPS = 256 * 64 * 2.4e9 / 1e12  # 256 CUs x 64 fp32 lanes x 2.4 GHz, one op per lane
 
@@ -162,10 +164,12 @@ def viterbi_main(args, w, capi, E, P, d_il, d_ll, il, ll):
     out_labels = torch.empty((B, U1 - 1), dtype=torch.int32, device=E.device)
     stream = ctypes.c_void_p(torch.cuda.current_stream(E.device).cuda_stream)
     p = lambda t: ctypes.c_void_p(t.data_ptr())
-    bf16 = w.get("io") == "bf16"
+    io = w.get("io")
+    bf16 = io is not None
     if bf16:
-        E, P = E.to(torch.bfloat16), P.to(torch.bfloat16)
-    entry = "rnnt_hip_viterbi_decode" + ("_bf16" if bf16 else "")
+        dtype16 = {"bf16": torch.bfloat16, "f16": torch.float16}[io]
+        E, P = E.to(dtype16), P.to(dtype16)
+    entry = "rnnt_hip_viterbi_decode" + ("_" + io if bf16 else "")
 
     def step():
         capi.call(entry, p(E), p(P), p(d_il), p(d_ll), p(out_labels), B, T, U1, V, 0, stream)
@@ -193,7 +197,7 @@ def viterbi_main(args, w, capi, E, P, d_il, d_ll, il, ll):
         "value": round(ms_per_step, 4), "unit": "ms", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": False,
         "scaling": "weak", "vs_baseline": None,
-        "dtype": "f32 arithmetic on bf16 scores" if bf16 else "f32", "data": "synthetic",
+        "dtype": "f32 arithmetic on %s scores" % io if bf16 else "f32", "data": "synthetic",
         "config": {"workload": "%s: B=%d T=%d U=%d V=%d blank=0, N(0,1) scores%s, input_lengths "
                                "U[%d,%d], label_lengths U[%d,%d]"
                                % ((args.workload, B, T, w["U"], V,
@@ -238,10 +242,12 @@ def main():
     E, P, labels, d_il, d_ll, il, ll = make_device_inputs(w, args.seed, device)
     if w.get("kind") == "viterbi":
         return viterbi_main(args, w, capi, E, P, d_il, d_ll, il, ll)
-    bf16 = w.get("io") == "bf16"
+    io = w.get("io")  # None (fp32), "bf16" or "f16"
+    bf16 = io is not None
     if bf16:
-        E, P = E.to(torch.bfloat16), P.to(torch.bfloat16)
-    suffix, esize = ("_bf16", 2.0) if bf16 else ("", 4.0)
+        dtype16 = {"bf16": torch.bfloat16, "f16": torch.float16}[io]
+        E, P = E.to(dtype16), P.to(dtype16)
+    suffix, esize = ("_" + io, 2.0) if bf16 else ("", 4.0)
     costs = torch.empty(B, device=device)
     egrads = torch.empty_like(E)
     pgrads = torch.empty_like(P)
@@ -289,7 +295,7 @@ def main():
                  "pgrads": esize * B * U1 * V}
     hbm_gbs = (in_bytes + out_bytes[dom]) / (mfma_kernels[dom] * 1e-3) / 1e9
     out = {
-        "metric": METRIC + (" (bf16 scores and gradients)" if bf16 else ""),
+        "metric": METRIC + (" (%s scores and gradients)" % io if bf16 else ""),
         "value": round(ms_per_step, 4),
         "unit": "ms",
         "n_gpus": 1,
@@ -300,7 +306,7 @@ def main():
         "scaling": "weak",
         "vs_baseline": (round(ms_per_step / w["published_ms"], 5) if w.get("published_ms")
                         else None),
-        "dtype": "f32 arithmetic on bf16 scores, bf16 gradients" if bf16 else "f32",
+        "dtype": "f32 arithmetic on %s scores, %s gradients" % (io, io) if bf16 else "f32",
         "data": "synthetic",
         "config": {"workload": "%s: B=%d T=%d U=%d V=%d blank=0, %s scores, input_lengths "
                                "%s, label_lengths %s, deltas=1" %

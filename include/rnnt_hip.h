@@ -103,14 +103,16 @@ int rnnt_hip_loss_backward(const float* emissions, const float* predictions, con
                            size_t workspace_bytes, int B, int T, int U, int V, int blank,
                            rnnt_stream_t stream);
 
-/* The same two calls for bf16 scores (the 16 high bits of an fp32, as torch.bfloat16 stores
- * them) and bf16 gradients.  No counterpart in the reference, which refuses anything but
- * float32 (transducer/torch_binding.py:195-201): this is for a caller whose projection layers
- * emit bf16 logits, and it halves the traffic of the two [B,T,V] arrays.  A score converts to
- * fp32 exactly and all arithmetic is the fp32 path's; each gradient element is the fp32 result
- * (dense + blank/label terms, times deltas[b]) rounded once to nearest-even.  Shapes: V a
- * multiple of 8, at most 112 label positions (U <= 112), 16-byte aligned score arrays; anything
- * else is refused with an error.  Workspace as for the fp32 calls. */
+/* The same calls for 16-bit scores and gradients: bf16 (the 16 high bits of an fp32, as
+ * torch.bfloat16 stores them) and fp16 (IEEE binary16, torch.float16).  No counterpart in the
+ * reference, which refuses anything but float32 (transducer/torch_binding.py:195-201): these are
+ * for a caller whose projection layers emit 16-bit logits, and they halve the traffic of the two
+ * [B,T,V] arrays.  A score converts to fp32 exactly and all arithmetic is the fp32 path's; each
+ * gradient element is the fp32 result (dense + blank/label terms, times deltas[b]) rounded once
+ * to nearest-even (an fp16 gradient past 65504 becomes infinity).  Shapes: V a multiple of 8,
+ * 16-byte aligned score arrays, and for the loss at most 112 label positions (U <= 112);
+ * anything else is refused with an error.  Workspace as for the fp32 calls.  The best path of
+ * rnnt_hip_viterbi_decode_* is the one rnnt_hip_viterbi_decode finds on the same values. */
 int rnnt_hip_loss_forward_bf16(const uint16_t* emissions, const uint16_t* predictions,
                                const int* labels, const int* input_lengths,
                                const int* label_lengths, float* costs, void* workspace,
@@ -121,12 +123,22 @@ int rnnt_hip_loss_backward_bf16(const uint16_t* emissions, const uint16_t* predi
                                 const int* label_lengths, const float* deltas, uint16_t* egrads,
                                 uint16_t* pgrads, void* workspace, size_t workspace_bytes, int B,
                                 int T, int U, int V, int blank, rnnt_stream_t stream);
-
-/* rnnt_hip_viterbi_decode for bf16 scores (V a multiple of 8, 16-byte aligned arrays; any U up
- * to 1024).  The path is the one rnnt_hip_viterbi_decode finds on the same values in fp32. */
 int rnnt_hip_viterbi_decode_bf16(const uint16_t* emissions, const uint16_t* predictions,
                                  const int* input_lengths, const int* label_lengths, int* labels,
                                  int B, int T, int U, int V, int blank, rnnt_stream_t stream);
+int rnnt_hip_loss_forward_f16(const uint16_t* emissions, const uint16_t* predictions,
+                              const int* labels, const int* input_lengths,
+                              const int* label_lengths, float* costs, void* workspace,
+                              size_t workspace_bytes, int B, int T, int U, int V, int blank,
+                              rnnt_stream_t stream);
+int rnnt_hip_loss_backward_f16(const uint16_t* emissions, const uint16_t* predictions,
+                               const int* labels, const int* input_lengths,
+                               const int* label_lengths, const float* deltas, uint16_t* egrads,
+                               uint16_t* pgrads, void* workspace, size_t workspace_bytes, int B,
+                               int T, int U, int V, int blank, rnnt_stream_t stream);
+int rnnt_hip_viterbi_decode_f16(const uint16_t* emissions, const uint16_t* predictions,
+                                const int* input_lengths, const int* label_lengths, int* labels,
+                                int B, int T, int U, int V, int blank, rnnt_stream_t stream);
 
 /* Replaces TransducerLoss.viterbi (transducer/torch_binding.py:130-177): log-normaliser +
  * best path.  labels is int [B, U-1]. */

@@ -1,16 +1,18 @@
-"""bf16 scores and gradients through rnnt_hip_loss_forward_bf16 / rnnt_hip_loss_backward_bf16,
-and the best path through rnnt_hip_viterbi_decode_bf16.
+"""16-bit scores and gradients (bf16, fp16) through rnnt_hip_loss_forward_* /
+rnnt_hip_loss_backward_*, and the best path through rnnt_hip_viterbi_decode_*.
 
 The reference takes float32 only (transducer/torch_binding.py:195-201), so there is no reference
 output to match.  What pins these entry points:
 
-* a bf16 score converts to fp32 exactly, and the kernels are the fp32 ones with other loads and
-  stores, so the costs must EQUAL the fp32 entry points' costs on the upcast inputs, and each
-  gradient element must be the fp32 entry points' element rounded once to bf16 (allowing one bf16
-  unit where the two paths order an addition differently: the blank/label terms are always folded
-  into the dense kernels here, the fp32 path scatters them when the vocabulary is small);
+* a 16-bit score converts to fp32 exactly, and the kernels are the fp32 ones with other loads
+  and stores, so the costs must EQUAL the fp32 entry points' costs on the upcast inputs, and each
+  gradient element must be the fp32 entry points' element rounded once to the 16-bit type
+  (allowing one unit where the two paths order an addition differently: the blank/label terms
+  are always folded into the dense kernels here, the fp32 path scatters them when the
+  vocabulary is small);
 * against the CPU oracle on the upcast inputs the tolerance is the fp32 one plus half a unit of
-  bf16: |got - want| <= 1e-5 + (1e-4 + 2**-8) * |want|.
+  the type: |got - want| <= 1e-5 + (1e-4 + 2**-8) * |want| for bf16, 2**-11 for fp16 (plus
+  fp16's absolute floor of 2**-25 near zero, which the 1e-5 covers).
 """
 import numpy as np
 import pytest
@@ -24,14 +26,17 @@ import oracle  # noqa: E402
 from transducer_amd import capi  # noqa: E402
 from transducer_amd.synthetic import CONFIGS  # noqa: E402
 
-BF16_RTOL = RTOL + 2.0 ** -8
+# (torch type, entry-point suffix, relative half unit)
+KINDS = {"bf16": (torch.bfloat16, "_bf16", 2.0 ** -8), "f16": (torch.float16, "_f16", 2.0 ** -11)}
+KIND_NAMES = sorted(KINDS)
 
 
-def draw(B, T, U, V, seed, sigma=1.0, ragged=True):
+def draw(B, T, U, V, seed, sigma=1.0, ragged=True, kind="bf16"):
     g = torch.Generator(device="cuda:0")
     g.manual_seed(seed)
-    E = (torch.randn((B, T, V), generator=g, device="cuda:0") * sigma).to(torch.bfloat16)
-    P = (torch.randn((B, U, V), generator=g, device="cuda:0") * sigma).to(torch.bfloat16)
+    dtype = KINDS[kind][0]
+    E = (torch.randn((B, T, V), generator=g, device="cuda:0") * sigma).to(dtype)
+    P = (torch.randn((B, U, V), generator=g, device="cuda:0") * sigma).to(dtype)
     labels = torch.randint(1, V, (B, max(U - 1, 0)), generator=g, device="cuda:0",
                            dtype=torch.int32)
     rng = np.random.default_rng(seed)
@@ -43,7 +48,12 @@ def draw(B, T, U, V, seed, sigma=1.0, ragged=True):
     return E, P, labels, il, ll
 
 
-def loss_bf16(E, P, labels, il, ll, deltas=None, blank=0):
+def suffix_of(t):
+    return {torch.bfloat16: "_bf16", torch.float16: "_f16"}[t.dtype]
+
+
+def loss_16bit(E, P, labels, il, ll, deltas=None, blank=0):
+    """The 16-bit entry points that match the tensors' type."""
     B, T, V = E.shape
     U = P.shape[1]
     d_il, d_ll = dev(il), dev(ll)
@@ -52,10 +62,10 @@ def loss_bf16(E, P, labels, il, ll, deltas=None, blank=0):
     costs = torch.full((B,), float("nan"), device="cuda:0")
     eg = torch.full_like(E, float("nan"))
     pg = torch.full_like(P, float("nan"))
-    capi.call("rnnt_hip_loss_forward_bf16", ptr(E), ptr(P), ptr(labels), ptr(d_il), ptr(d_ll),
-              ptr(costs), ptr(ws), nbytes, B, T, U, V, blank, None)
-    capi.call("rnnt_hip_loss_backward_bf16", ptr(E), ptr(P), ptr(labels), ptr(d_il), ptr(d_ll),
-              ptr(deltas), ptr(eg), ptr(pg), ptr(ws), nbytes, B, T, U, V, blank, None)
+    capi.call("rnnt_hip_loss_forward" + suffix_of(E), ptr(E), ptr(P), ptr(labels), ptr(d_il),
+              ptr(d_ll), ptr(costs), ptr(ws), nbytes, B, T, U, V, blank, None)
+    capi.call("rnnt_hip_loss_backward" + suffix_of(E), ptr(E), ptr(P), ptr(labels), ptr(d_il),
+              ptr(d_ll), ptr(deltas), ptr(eg), ptr(pg), ptr(ws), nbytes, B, T, U, V, blank, None)
     torch.cuda.synchronize()
     return costs, eg, pg
 
@@ -79,9 +89,9 @@ def loss_fp32(E, P, labels, il, ll, deltas=None, blank=0):
     return costs, eg, pg
 
 
-def bf16_units_apart(got, want_fp32):
-    """|got - round_bf16(want)| in units of bf16 at want's magnitude, elementwise (device)."""
-    want = want_fp32.to(torch.bfloat16)
+def units_apart(got, want_fp32):
+    """|got - round(want)| in units of got's 16-bit type at want's magnitude, elementwise."""
+    want = want_fp32.to(got.dtype)
     gi = got.view(torch.int16).to(torch.int32)
     wi = want.view(torch.int16).to(torch.int32)
     # sign-magnitude -> monotone integers
@@ -91,11 +101,14 @@ def bf16_units_apart(got, want_fp32):
 
 
 def assert_rounds_the_fp32_result(got, want_fp32, what, exact_fraction):
-    assert got.dtype is torch.bfloat16
-    apart = bf16_units_apart(got, want_fp32)
+    assert got.dtype in (torch.bfloat16, torch.float16)
+    apart = units_apart(got, want_fp32)
     # around zero one unit of the integer view is a denormal step: judge those by value
-    small = want_fp32.abs() < 1e-30
-    assert bool((got.float()[small].abs() < 1e-30).all())
+    # (fp16 keeps nothing below 2**-25 = 3e-8)
+    floor = 1e-30 if got.dtype is torch.bfloat16 else 1e-7
+    small = want_fp32.abs() < floor
+    step = 1e-30 if got.dtype is torch.bfloat16 else 2.0 ** -24  # fp16's smallest step
+    assert bool(((got.float() - want_fp32)[small].abs() <= step).all())
     apart = apart[~small]
     worst = int(apart.max()) if apart.numel() else 0
     same = float((apart == 0).float().mean()) if apart.numel() else 1.0
@@ -116,11 +129,13 @@ SHAPES = [
 ]
 
 
+@pytest.mark.parametrize("kind", KIND_NAMES)
 @pytest.mark.parametrize("B,T,U,V", SHAPES)
-def test_bf16_against_the_fp32_entry_points_and_the_oracle(B, T, U, V):
-    E, P, labels, il, ll = draw(B, T, U, V, seed=B * 1000 + T + U + V)
+def test_16bit_against_the_fp32_entry_points_and_the_oracle(B, T, U, V, kind):
+    LOWP_RTOL = RTOL + KINDS[kind][2]
+    E, P, labels, il, ll = draw(B, T, U, V, seed=B * 1000 + T + U + V, kind=kind)
     deltas = torch.linspace(0.5, 2.0, B, device="cuda:0")
-    costs, eg, pg = loss_bf16(E, P, labels, il, ll, deltas)
+    costs, eg, pg = loss_16bit(E, P, labels, il, ll, deltas)
     c32, e32, p32 = loss_fp32(E, P, labels, il, ll, deltas)
     assert torch.equal(costs, c32)
     assert_rounds_the_fp32_result(eg, e32, "egrads", 0.999)
@@ -135,17 +150,19 @@ def test_bf16_against_the_fp32_entry_points_and_the_oracle(B, T, U, V):
     assert ve == 0.0
     for got, ref, what in ((eg, want["egrads"], "egrads"), (pg, want["pgrads"], "pgrads")):
         ref = ref * d[:, None, None]
-        frac, worst = violations(got.float().cpu().numpy(), ref, rtol=BF16_RTOL, atol=ATOL)
+        frac, worst = violations(got.float().cpu().numpy(), ref, rtol=LOWP_RTOL, atol=ATOL)
         assert frac == 0.0, "%s: %.4g%% outside rtol=%g atol=%g (max abs err %g)" % (
-            what, 100 * frac, BF16_RTOL, ATOL, worst)
+            what, 100 * frac, LOWP_RTOL, ATOL, worst)
 
 
-def test_bf16_blank_not_zero_and_repeated_labels():
+@pytest.mark.parametrize("kind", KIND_NAMES)
+def test_16bit_blank_not_zero_and_repeated_labels(kind):
+    LOWP_RTOL = RTOL + KINDS[kind][2]
     B, T, U, V = 2, 40, 7, 24
-    E, P, labels, il, ll = draw(B, T, U, V, seed=11, ragged=False)
+    E, P, labels, il, ll = draw(B, T, U, V, seed=11, ragged=False, kind=kind)
     labels[:] = torch.tensor([[3, 3, 5, 5, 5, 0], [1, 1, 1, 2, 0, 0]], dtype=torch.int32)
     blank = 4
-    costs, eg, pg = loss_bf16(E, P, labels, il, ll, blank=blank)
+    costs, eg, pg = loss_16bit(E, P, labels, il, ll, blank=blank)
     c32, e32, p32 = loss_fp32(E, P, labels, il, ll, blank=blank)
     assert torch.equal(costs, c32)
     assert_rounds_the_fp32_result(eg, e32, "egrads", 0.999)
@@ -153,90 +170,102 @@ def test_bf16_blank_not_zero_and_repeated_labels():
     want = oracle.loss_and_grads(E.float().cpu().numpy(), P.float().cpu().numpy(),
                                  labels.cpu().numpy(), il, ll, blank=blank)
     for got, ref in ((eg, want["egrads"]), (pg, want["pgrads"])):
-        frac, _ = violations(got.float().cpu().numpy(), ref, rtol=BF16_RTOL, atol=ATOL)
+        frac, _ = violations(got.float().cpu().numpy(), ref, rtol=LOWP_RTOL, atol=ATOL)
         assert frac == 0.0
 
 
-def test_bf16_empty_utterances_and_empty_batch():
+@pytest.mark.parametrize("kind", KIND_NAMES)
+def test_16bit_empty_utterances_and_empty_batch(kind):
     B, T, U, V = 3, 12, 4, 16
-    E, P, labels, il, ll = draw(B, T, U, V, seed=5)
+    E, P, labels, il, ll = draw(B, T, U, V, seed=5, kind=kind)
     il[1] = 0   # no frames: cost +inf, zero gradients (transducer_cpu.cpp:39-41)
     ll[2] = 0   # no labels
-    costs, eg, pg = loss_bf16(E, P, labels, il, ll)
+    costs, eg, pg = loss_16bit(E, P, labels, il, ll)
     c32, e32, p32 = loss_fp32(E, P, labels, il, ll)
     assert torch.equal(costs, c32) and bool(torch.isinf(costs[1]))
     assert not eg[1].any() and not pg[1].any()
     assert_rounds_the_fp32_result(eg, e32, "egrads", 0.999)
     assert_rounds_the_fp32_result(pg, p32, "pgrads", 0.999)
     # B == 0 and T == 0 are legal and touch nothing / clear the outputs
-    capi.call("rnnt_hip_loss_forward_bf16", None, None, None, None, None, None, None, 0,
+    sfx = KINDS[kind][1]
+    capi.call("rnnt_hip_loss_forward" + sfx, None, None, None, None, None, None, None, 0,
               0, T, U, V, 0, None)
-    eg0 = torch.full((2, 0, V), 1.0, device="cuda:0", dtype=torch.bfloat16)
-    pg0 = torch.full((2, U, V), 1.0, device="cuda:0", dtype=torch.bfloat16)
+    eg0 = torch.full((2, 0, V), 1.0, device="cuda:0", dtype=KINDS[kind][0])
+    pg0 = torch.full((2, U, V), 1.0, device="cuda:0", dtype=KINDS[kind][0])
     d_il, d_ll = dev(np.zeros(2, np.int32)), dev(np.zeros(2, np.int32))
-    capi.call("rnnt_hip_loss_backward_bf16", None, None, None, ptr(d_il), ptr(d_ll), None,
+    capi.call("rnnt_hip_loss_backward" + sfx, None, None, None, ptr(d_il), ptr(d_ll), None,
               ptr(eg0), ptr(pg0), None, 0, 2, 0, U, V, 0, None)
     torch.cuda.synchronize()
     assert not pg0.any()
 
 
+@pytest.mark.parametrize("kind", KIND_NAMES)
 @pytest.mark.parametrize("B,T,U,V,needle", [
     (1, 8, 3, 12, "multiple of 8"),
     (1, 8, 3, 4, "multiple of 8"),
     (1, 8, 113, 16, "112 label positions"),
 ])
-def test_bf16_shapes_outside_the_streaming_kernels_are_refused(B, T, U, V, needle):
-    E = torch.zeros((B, T, V), device="cuda:0", dtype=torch.bfloat16)
-    P = torch.zeros((B, U, V), device="cuda:0", dtype=torch.bfloat16)
+def test_16bit_shapes_outside_the_streaming_kernels_are_refused(B, T, U, V, needle, kind):
+    dtype, sfx, _ = KINDS[kind]
+    E = torch.zeros((B, T, V), device="cuda:0", dtype=dtype)
+    P = torch.zeros((B, U, V), device="cuda:0", dtype=dtype)
     labels = torch.ones((B, U - 1), device="cuda:0", dtype=torch.int32)
     il, ll = dev(np.full(B, T, np.int32)), dev(np.full(B, U - 1, np.int32))
     nbytes = capi.load().rnnt_hip_loss_workspace_bytes(B, T, U, V)
     ws = torch.empty(nbytes, dtype=torch.uint8, device="cuda:0")
     costs = torch.zeros((B,), device="cuda:0")
     with pytest.raises(capi.RnntHipError, match=needle):
-        capi.call("rnnt_hip_loss_forward_bf16", ptr(E), ptr(P), ptr(labels), ptr(il), ptr(ll),
+        capi.call("rnnt_hip_loss_forward" + sfx, ptr(E), ptr(P), ptr(labels), ptr(il), ptr(ll),
                   ptr(costs), ptr(ws), nbytes, B, T, U, V, 0, None)
     eg, pg = torch.zeros_like(E), torch.zeros_like(P)
     with pytest.raises(capi.RnntHipError, match=needle):
-        capi.call("rnnt_hip_loss_backward_bf16", ptr(E), ptr(P), ptr(labels), ptr(il), ptr(ll),
+        capi.call("rnnt_hip_loss_backward" + sfx, ptr(E), ptr(P), ptr(labels), ptr(il), ptr(ll),
                   None, ptr(eg), ptr(pg), ptr(ws), nbytes, B, T, U, V, 0, None)
 
 
-def test_bf16_through_the_torch_module():
+@pytest.mark.parametrize("kind", KIND_NAMES)
+def test_16bit_through_the_torch_module(kind):
     from transducer_amd import TransducerLoss
+    dtype = KINDS[kind][0]
     B, T, U, V = 3, 30, 6, 40
-    E, P, labels, il, ll = draw(B, T, U, V, seed=21)
+    E, P, labels, il, ll = draw(B, T, U, V, seed=21, kind=kind)
     d_il, d_ll = dev(il), dev(ll)
     with pytest.raises(TypeError, match="emissions must be torch.float32"):
         TransducerLoss()(E, P, labels, d_il, d_ll)  # the reference's behaviour stays the default
-    crit = TransducerLoss(allow_bf16=True)
-    with pytest.raises(TypeError, match="predictions must be torch.bfloat16"):
+    with pytest.raises(TypeError, match="emissions must be torch.float32"):
+        # the flag of the OTHER 16-bit type does not let this one in
+        TransducerLoss(allow_bf16=kind != "bf16", allow_fp16=kind != "f16")(
+            E, P, labels, d_il, d_ll)
+    crit = TransducerLoss(allow_bf16=kind == "bf16", allow_fp16=kind == "f16")
+    with pytest.raises(TypeError, match="predictions must be %s" % dtype):
         crit(E, P.float(), labels, d_il, d_ll)
     Et, Pt = E.clone().requires_grad_(True), P.clone().requires_grad_(True)
     costs = crit(Et, Pt, labels, d_il, d_ll)
     assert costs.dtype is torch.float32
     w = torch.linspace(1.0, 2.0, B, device="cuda:0")
     (costs * w).sum().backward()
-    c, eg, pg = loss_bf16(E, P, labels, il, ll, w)
+    c, eg, pg = loss_16bit(E, P, labels, il, ll, w)
     assert torch.equal(costs.detach(), c)
-    assert Et.grad.dtype is torch.bfloat16 and torch.equal(Et.grad, eg)
+    assert Et.grad.dtype is dtype and torch.equal(Et.grad, eg)
     assert torch.equal(Pt.grad, pg)
-    # float32 tensors still take the fp32 path under allow_bf16
+    # float32 tensors still take the fp32 path under the flag
     c32 = crit(E.float(), P.float(), labels, d_il, d_ll)
     assert torch.equal(c32, c)
 
 
-def test_bf16_headline_configuration_against_the_fp32_path():
+@pytest.mark.parametrize("kind", KIND_NAMES)
+def test_16bit_headline_configuration_against_the_fp32_path(kind):
+    dtype = KINDS[kind][0]
     cfg = CONFIGS["cfg4"]
     from transducer_amd.synthetic import lengths
     g = torch.Generator(device="cuda:0")
     g.manual_seed(17)
     B, T, U, V = cfg.B, cfg.T, cfg.U + 1, cfg.V
-    E = torch.randn((B, T, V), generator=g, device="cuda:0").to(torch.bfloat16)
-    P = torch.randn((B, U, V), generator=g, device="cuda:0").to(torch.bfloat16)
+    E = torch.randn((B, T, V), generator=g, device="cuda:0").to(dtype)
+    P = torch.randn((B, U, V), generator=g, device="cuda:0").to(dtype)
     labels = torch.randint(1, V, (B, U - 1), generator=g, device="cuda:0", dtype=torch.int32)
     il, ll = lengths(cfg, np.random.Generator(np.random.Philox(key=17)))
-    costs, eg, pg = loss_bf16(E, P, labels, il, ll)
+    costs, eg, pg = loss_16bit(E, P, labels, il, ll)
     assert torch.isfinite(costs).all() and torch.isfinite(eg.float()).all()
     d_il, d_ll = dev(il), dev(ll)
     tmask = torch.arange(T, device="cuda:0")[None, :] >= d_il[:, None]
@@ -245,18 +274,18 @@ def test_bf16_headline_configuration_against_the_fp32_path():
     c32, e32, p32 = loss_fp32(E, P, labels, il, ll)
     assert torch.equal(costs, c32)
     # both paths fold the sparse terms of egrads at this vocabulary: the same fp32 value, rounded
-    assert torch.equal(eg, e32.to(torch.bfloat16))
+    assert torch.equal(eg, e32.to(dtype))
     assert_rounds_the_fp32_result(pg, p32, "pgrads", 0.9999)
 
 
 # ------------------------------------------------------------------ best path
-def decode_bf16(E, P, il, ll, blank=0):
+def decode_16bit(E, P, il, ll, blank=0):
     B, T, V = E.shape
     U = P.shape[1]
     out = torch.full((B, U - 1), -1, dtype=torch.int32, device="cuda:0")
     d_il, d_ll = dev(il), dev(ll)
-    capi.call("rnnt_hip_viterbi_decode_bf16", ptr(E), ptr(P), ptr(d_il), ptr(d_ll), ptr(out),
-              B, T, U, V, blank, None)
+    capi.call("rnnt_hip_viterbi_decode" + suffix_of(E), ptr(E), ptr(P), ptr(d_il), ptr(d_ll),
+              ptr(out), B, T, U, V, blank, None)
     torch.cuda.synchronize()
     return out
 
@@ -273,15 +302,16 @@ def decode_fp32(E, P, il, ll, blank=0):
     return out
 
 
+@pytest.mark.parametrize("kind", KIND_NAMES)
 @pytest.mark.parametrize("B,T,U,V,blank", [(3, 37, 9, 64, 0), (2, 64, 33, 128, 5),
                                            (2, 300, 130, 40, 0), (4, 50, 11, 32, 31)])
-def test_bf16_best_path_is_the_fp32_path_and_the_oracles(B, T, U, V, blank):
-    """bf16 scores are exact in fp32 and the decode has no rounding step of its own, so the
+def test_16bit_best_path_is_the_fp32_path_and_the_oracles(B, T, U, V, blank, kind):
+    """16-bit scores are exact in fp32 and the decode has no rounding step of its own, so the
     path must be the fp32 decode's on the upcast scores, label for label; the oracle is fed the
     device's log-normaliser, as in the fp32 tests (the path is bit-exact GIVEN LN)."""
-    E, P, _, il, ll = draw(B, T, U, V, seed=7 * B + T + U + V)
+    E, P, _, il, ll = draw(B, T, U, V, seed=7 * B + T + U + V, kind=kind)
     ll = np.maximum(ll, 1).astype(np.int32)
-    got = decode_bf16(E, P, il, ll, blank)
+    got = decode_16bit(E, P, il, ll, blank)
     ref = decode_fp32(E, P, il, ll, blank)
     assert torch.equal(got, ref)
     E32, P32 = E.float().contiguous(), P.float().contiguous()
@@ -297,14 +327,16 @@ def test_bf16_best_path_is_the_fp32_path_and_the_oracles(B, T, U, V, blank):
         assert (g[b, ll[b]:] == -1).all()
 
 
-def test_bf16_best_path_through_the_torch_module():
+@pytest.mark.parametrize("kind", KIND_NAMES)
+def test_16bit_best_path_through_the_torch_module(kind):
     from transducer_amd import TransducerLoss
     B, T, U, V = 3, 40, 8, 48
-    E, P, _, il, ll = draw(B, T, U, V, seed=3)
+    E, P, _, il, ll = draw(B, T, U, V, seed=3, kind=kind)
     d_il, d_ll = dev(il), dev(ll)
     with pytest.raises(TypeError, match="emissions must be torch.float32"):
         TransducerLoss().viterbi(E, P, d_il, d_ll)
-    paths = TransducerLoss(allow_bf16=True).viterbi(E, P, d_il, d_ll)
-    ref = decode_bf16(E, P, il, ll)
+    paths = TransducerLoss(allow_bf16=kind == "bf16", allow_fp16=kind == "f16").viterbi(
+        E, P, d_il, d_ll)
+    ref = decode_16bit(E, P, il, ll)
     for b in range(B):
         assert torch.equal(paths[b, :ll[b]], ref[b, :ll[b]])

@@ -24,8 +24,11 @@ SIGNATURES = {
     "rnnt_hip_loss_backward": (_I, [_F] * 9 + [_Z] + [_I] * 5 + [_F]),
     "rnnt_hip_loss_forward_bf16": (_I, [_F] * 7 + [_Z] + [_I] * 5 + [_F]),
     "rnnt_hip_loss_backward_bf16": (_I, [_F] * 9 + [_Z] + [_I] * 5 + [_F]),
+    "rnnt_hip_loss_forward_f16": (_I, [_F] * 7 + [_Z] + [_I] * 5 + [_F]),
+    "rnnt_hip_loss_backward_f16": (_I, [_F] * 9 + [_Z] + [_I] * 5 + [_F]),
     "rnnt_hip_viterbi_decode": (_I, [_F] * 5 + [_I] * 5 + [_F]),
     "rnnt_hip_viterbi_decode_bf16": (_I, [_F] * 5 + [_I] * 5 + [_F]),
+    "rnnt_hip_viterbi_decode_f16": (_I, [_F] * 5 + [_I] * 5 + [_F]),
     "rnnt_hip_profile_enable": (_I, [_I]),
     "rnnt_hip_profile_stage_count": (_I, []),
     "rnnt_hip_profile_stage_name": (ctypes.c_char_p, [_I]),

@@ -139,7 +139,8 @@ PYBIND11_MODULE(_transducer, m) {
         "deltas"_a, "egrads"_a, "pgrads"_a, "workspace"_a, "workspace_bytes"_a, "batch_size"_a,
         "max_input_length"_a, "max_label_length"_a, "alphabet_size"_a, "blank"_a, "stream"_a = 0);
 
-  // bf16 scores and gradients (no counterpart in the reference, which takes float32 only)
+  // 16-bit scores and gradients, bf16 and fp16 (no counterpart in the reference, which takes
+  // float32 only)
   m.def("loss_forward_bf16",
         [](ptr_t emissions, ptr_t predictions, ptr_t labels, ptr_t input_lengths,
            ptr_t label_lengths, ptr_t costs, ptr_t workspace, std::size_t workspace_bytes,
@@ -155,12 +156,43 @@ PYBIND11_MODULE(_transducer, m) {
         "costs"_a, "workspace"_a, "workspace_bytes"_a, "batch_size"_a, "max_input_length"_a,
         "max_label_length"_a, "alphabet_size"_a, "blank"_a, "stream"_a = 0);
 
+  m.def("loss_forward_f16",
+        [](ptr_t emissions, ptr_t predictions, ptr_t labels, ptr_t input_lengths,
+           ptr_t label_lengths, ptr_t costs, ptr_t workspace, std::size_t workspace_bytes,
+           int batch_size, int max_input_length, int max_label_length, int alphabet_size,
+           int blank, ptr_t stream) {
+          raise_on(rnnt_hip_loss_forward_f16(
+              as<const uint16_t>(emissions), as<const uint16_t>(predictions),
+              as<const int>(labels), as<const int>(input_lengths), as<const int>(label_lengths),
+              as<float>(costs), as<void>(workspace), workspace_bytes, batch_size,
+              max_input_length, max_label_length, alphabet_size, blank, as<void>(stream)));
+        },
+        "emissions"_a, "predictions"_a, "labels"_a, "input_lengths"_a, "label_lengths"_a,
+        "costs"_a, "workspace"_a, "workspace_bytes"_a, "batch_size"_a, "max_input_length"_a,
+        "max_label_length"_a, "alphabet_size"_a, "blank"_a, "stream"_a = 0);
+
   m.def("loss_backward_bf16",
         [](ptr_t emissions, ptr_t predictions, ptr_t labels, ptr_t input_lengths,
            ptr_t label_lengths, ptr_t deltas, ptr_t egrads, ptr_t pgrads, ptr_t workspace,
            std::size_t workspace_bytes, int batch_size, int max_input_length,
            int max_label_length, int alphabet_size, int blank, ptr_t stream) {
           raise_on(rnnt_hip_loss_backward_bf16(
+              as<const uint16_t>(emissions), as<const uint16_t>(predictions),
+              as<const int>(labels), as<const int>(input_lengths), as<const int>(label_lengths),
+              as<const float>(deltas), as<uint16_t>(egrads), as<uint16_t>(pgrads),
+              as<void>(workspace), workspace_bytes, batch_size, max_input_length,
+              max_label_length, alphabet_size, blank, as<void>(stream)));
+        },
+        "emissions"_a, "predictions"_a, "labels"_a, "input_lengths"_a, "label_lengths"_a,
+        "deltas"_a, "egrads"_a, "pgrads"_a, "workspace"_a, "workspace_bytes"_a, "batch_size"_a,
+        "max_input_length"_a, "max_label_length"_a, "alphabet_size"_a, "blank"_a, "stream"_a = 0);
+
+  m.def("loss_backward_f16",
+        [](ptr_t emissions, ptr_t predictions, ptr_t labels, ptr_t input_lengths,
+           ptr_t label_lengths, ptr_t deltas, ptr_t egrads, ptr_t pgrads, ptr_t workspace,
+           std::size_t workspace_bytes, int batch_size, int max_input_length,
+           int max_label_length, int alphabet_size, int blank, ptr_t stream) {
+          raise_on(rnnt_hip_loss_backward_f16(
               as<const uint16_t>(emissions), as<const uint16_t>(predictions),
               as<const int>(labels), as<const int>(input_lengths), as<const int>(label_lengths),
               as<const float>(deltas), as<uint16_t>(egrads), as<uint16_t>(pgrads),
@@ -190,6 +222,20 @@ PYBIND11_MODULE(_transducer, m) {
            ptr_t labels, int batch_size, int max_input_length, int max_label_length,
            int alphabet_size, int blank, ptr_t stream) {
           raise_on(rnnt_hip_viterbi_decode_bf16(
+              as<const uint16_t>(emissions), as<const uint16_t>(predictions),
+              as<const int>(input_lengths), as<const int>(label_lengths), as<int>(labels),
+              batch_size, max_input_length, max_label_length, alphabet_size, blank,
+              as<void>(stream)));
+        },
+        "emissions"_a, "predictions"_a, "input_lengths"_a, "label_lengths"_a, "labels"_a,
+        "batch_size"_a, "max_input_length"_a, "max_label_length"_a, "alphabet_size"_a, "blank"_a,
+        "stream"_a = 0);
+
+  m.def("viterbi_decode_f16",
+        [](ptr_t emissions, ptr_t predictions, ptr_t input_lengths, ptr_t label_lengths,
+           ptr_t labels, int batch_size, int max_input_length, int max_label_length,
+           int alphabet_size, int blank, ptr_t stream) {
+          raise_on(rnnt_hip_viterbi_decode_f16(
               as<const uint16_t>(emissions), as<const uint16_t>(predictions),
               as<const int>(input_lengths), as<const int>(label_lengths), as<int>(labels),
               batch_size, max_input_length, max_label_length, alphabet_size, blank,

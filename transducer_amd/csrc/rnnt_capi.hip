@@ -217,6 +217,128 @@ int viterbi_impl(const TIO* E, const TIO* P, const float* LN, int* labels,
   return kOk;
 }
 
+
+// ---------------------------------------------------------------- 16-bit scores
+int check_lowp_shape(const void* E, const void* P, const Dims& d, bool loss, const char* who) {
+  if (d.V % 8 != 0)
+    return fail(kInvalid, "%s: 16-bit scores need a vocabulary that is a multiple of 8 (V=%d)",
+                who, d.V);
+  if ((reinterpret_cast<uintptr_t>(E) | reinterpret_cast<uintptr_t>(P)) & 15)
+    return fail(kInvalid, "%s: 16-bit scores must be 16-byte aligned", who);
+  if (loss && !egrads_stream_supported(d))
+    return fail(kInvalid, "%s: 16-bit scores take at most 112 label positions (U=%d)", who, d.U);
+  return kOk;
+}
+
+template <typename TIO>
+int lowp_loss_forward(const TIO* E, const TIO* P, const int* labels, const int* inLen,
+                      const int* labLen, float* costs, void* workspace, size_t workspace_bytes,
+                      int B, int T, int U, int V, int blank, rnnt_stream_t stream,
+                      const char* who) {
+  RNNT_TRY(check_dims(B, T, U, V));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (B == 0) return kOk;
+  if (!costs || !inLen || !labLen) return fail(kInvalid, "%s: null costs or lengths", who);
+  if (nothing_to_do(B, T, U)) return fill(costs, __builtin_huge_valf(), B, s);
+  if (V == 0) return fail(kInvalid, "%s: empty vocabulary", who);
+  if (!E || !P || (U > 1 && !labels)) return fail(kInvalid, "%s: null array argument", who);
+  if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & 255))
+    return fail(kInvalid, "%s: workspace must be a 256-byte aligned device pointer", who);
+  if (workspace_bytes < rnnt_hip_loss_workspace_bytes(B, T, U, V))
+    return fail(kWorkspace, "%s: workspace of %zu bytes, %zu needed", who, workspace_bytes,
+                rnnt_hip_loss_workspace_bytes(B, T, U, V));
+  const Dims d = make_dims(B, T, U, V, blank);
+  RNNT_TRY(check_lowp_shape(E, P, d, true, who));
+  if (!lse_stream_supported(E, d)) return fail(kInvalid, "%s: B*T*U too large", who);
+  LossWorkspace w;
+  loss_workspace_layout(d, workspace, &w);
+  RNNT_STAGE(kRowmax, launch_rowmax_pick_p(P, w.mP, labels, labLen, w.planes, d, s));
+  RNNT_STAGE(kYplanes, launch_yplanes(P, w.mP, w.lse_scratch, labLen, d, s));
+  RNNT_STAGE(kLse, launch_lse_stream(E, w.mE, w.mP, w.LN, w.lse_scratch, inLen, labLen, d, s,
+                                     labels, w.planes.elS, w.planes.eb));
+  RNNT_STAGE(kSkew, launch_skew(w.LN, w.planes.lnS, inLen, labLen, d, s));
+  RNNT_STAGE(kAlpha, launch_alpha(w.planes, inLen, labLen, costs, d, s));
+  return kOk;
+}
+
+template <typename TIO>
+int lowp_loss_backward(const TIO* E, const TIO* P, const int* labels, const int* inLen,
+                       const int* labLen, const float* deltas, TIO* egrads, TIO* pgrads,
+                       void* workspace, size_t workspace_bytes, int B, int T, int U, int V,
+                       int blank, rnnt_stream_t stream, const char* who) {
+  RNNT_TRY(check_dims(B, T, U, V));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (B == 0 || V == 0) return kOk;
+  if (nothing_to_do(B, T, U)) {
+    if (egrads && (size_t)T * V)
+      RNNT_HIP(hipMemsetAsync(egrads, 0, sizeof(TIO) * (size_t)B * T * V, s));
+    if (pgrads && (size_t)U * V)
+      RNNT_HIP(hipMemsetAsync(pgrads, 0, sizeof(TIO) * (size_t)B * U * V, s));
+    return kOk;
+  }
+  if (!E || !P || !egrads || !pgrads || !inLen || !labLen || (U > 1 && !labels))
+    return fail(kInvalid, "%s: null array argument", who);
+  if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & 255))
+    return fail(kInvalid, "%s: workspace must be a 256-byte aligned device pointer", who);
+  if (workspace_bytes < rnnt_hip_loss_workspace_bytes(B, T, U, V))
+    return fail(kWorkspace, "%s: workspace of %zu bytes, %zu needed", who, workspace_bytes,
+                rnnt_hip_loss_workspace_bytes(B, T, U, V));
+  const Dims d = make_dims(B, T, U, V, blank);
+  RNNT_TRY(check_lowp_shape(E, P, d, true, who));
+  if ((reinterpret_cast<uintptr_t>(egrads) | reinterpret_cast<uintptr_t>(pgrads)) & 1)
+    return fail(kInvalid, "%s: misaligned gradient arrays", who);
+  LossWorkspace w;
+  loss_workspace_layout(d, workspace, &w);
+  RNNT_STAGE(kWeights, launch_weights(w.planes, inLen, labLen, d, s));
+  RNNT_STAGE(kBeta, launch_beta(w.planes, labels, inLen, labLen, d, s));
+  RNNT_STAGE(kWplanes, launch_wplanes_skewed(w.planes.dS, w.planes.lnS, w.mE, w.mP, w.Wn, w.Wt,
+                                             inLen, labLen, d, s));
+  // Both gradients are rounded once, from the complete fp32 value: the blank / label terms are
+  // always folded into the dense kernels' write-outs here, whatever the vocabulary.  With
+  // U == 1 there are no labels; the kernels then never read the list, but its pointer is what
+  // switches the folding on, so any valid device pointer serves.
+  const int* lab = labels ? labels : inLen;
+  RNNT_STAGE(kSparse, launch_blank_sums(w.planes, w.bsum, lab, inLen, labLen, d, s));
+  SparseTerms sp;
+  sp.dS = w.planes.dS; sp.wE = w.planes.wE; sp.bsum = w.bsum; sp.labels = lab;
+  SparsePTerms spp;
+  spp.gB = w.planes.gB; spp.gL = w.planes.gL; spp.labels = lab;
+  RNNT_STAGE(kEgrads, launch_egrads_stream(E, P, w.mE, w.mP, w.Wn, deltas, egrads, inLen, labLen,
+                                           d, false, sp, s));
+  RNNT_STAGE(kPgrads, launch_pgrads_stream(E, P, w.mE, w.mP, w.Wt, deltas, pgrads, inLen, labLen,
+                                           d, false, spp, s));
+  return kOk;
+}
+
+template <typename TIO>
+int lowp_viterbi_decode(const TIO* E, const TIO* P, const int* inLen, const int* labLen,
+                        int* labels, int B, int T, int U, int V, int blank, rnnt_stream_t stream,
+                        const char* who) {
+  RNNT_TRY(check_dims(B, T, U, V));
+  if (nothing_to_do(B, T, U) || U == 1) return kOk;  // no label to emit
+  if (V == 0) return fail(kInvalid, "%s: empty vocabulary", who);
+  if (!E || !P || !labels || !inLen || !labLen)
+    return fail(kInvalid, "%s: null array argument", who);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const Dims d = make_dims(B, T, U, V, blank);
+  RNNT_TRY(check_lowp_shape(E, P, d, false, who));
+  if (!lse_stream_supported(E, d)) return fail(kInvalid, "%s: B*T*U too large", who);
+  Scratch scratch(s);
+  const size_t btu = sizeof(float) * (size_t)B * T * U;
+  const size_t yb = lse_scratch_bytes(d);
+  RNNT_TRY(scratch.reserve(align_up(sizeof(float) * (size_t)B * T) +
+                           align_up(sizeof(float) * (size_t)B * U) + align_up(btu) +
+                           align_up(yb)));
+  float* mE = static_cast<float*>(scratch.take(sizeof(float) * (size_t)B * T));
+  float* mP = static_cast<float*>(scratch.take(sizeof(float) * (size_t)B * U));
+  float* LN = static_cast<float*>(scratch.take(btu));
+  void* ys = scratch.take(yb);
+  RNNT_STAGE(kRowmax, launch_rowmax(P, mP, (long)B * U, V, U, labLen, 1, s));
+  RNNT_STAGE(kYplanes, launch_yplanes(P, mP, ys, labLen, d, s));
+  RNNT_STAGE(kLse, launch_lse_stream(E, mE, mP, LN, ys, inLen, labLen, d, s));
+  return viterbi_impl(E, P, LN, labels, inLen, labLen, d, s);
+}
+
 }  // namespace
 }  // namespace rnnt
 
@@ -443,141 +565,38 @@ int rnnt_hip_loss_backward(const float* E, const float* P, const int* labels, co
   return kOk;
 }
 
-// bf16 scores: the shapes the streaming kernels take (every launcher below exists for both
-// element types; the general-shape fallbacks are fp32 only).
-static int check_bf16_shape(const void* E, const void* P, const Dims& d, const char* who) {
-  if (d.V % 8 != 0)
-    return fail(kInvalid, "%s: bf16 scores need a vocabulary that is a multiple of 8 (V=%d)", who,
-                d.V);
-  if ((reinterpret_cast<uintptr_t>(E) | reinterpret_cast<uintptr_t>(P)) & 15)
-    return fail(kInvalid, "%s: bf16 scores must be 16-byte aligned", who);
-  if (!egrads_stream_supported(d) || d.U > 128)
-    return fail(kInvalid, "%s: bf16 scores take at most 112 label positions (U=%d)", who, d.U);
-  if (!lse_stream_supported(static_cast<const bf16_t*>(E), d))
-    return fail(kInvalid, "%s: B*T*U too large for the bf16 path", who);
-  return kOk;
-}
-
-int rnnt_hip_loss_forward_bf16(const uint16_t* E16, const uint16_t* P16, const int* labels,
-                               const int* inLen, const int* labLen, float* costs, void* workspace,
-                               size_t workspace_bytes, int B, int T, int U, int V, int blank,
-                               rnnt_stream_t stream) {
-  RNNT_TRY(check_dims(B, T, U, V));
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  if (B == 0) return kOk;
-  if (!costs || !inLen || !labLen)
-    return fail(kInvalid, "loss_forward_bf16: null costs or lengths");
-  if (nothing_to_do(B, T, U)) return fill(costs, __builtin_huge_valf(), B, s);
-  if (V == 0) return fail(kInvalid, "loss_forward_bf16: empty vocabulary");
-  if (!E16 || !P16 || (U > 1 && !labels))
-    return fail(kInvalid, "loss_forward_bf16: null array argument");
-  if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & 255))
-    return fail(kInvalid, "loss_forward_bf16: workspace must be a 256-byte aligned device pointer");
-  if (workspace_bytes < rnnt_hip_loss_workspace_bytes(B, T, U, V))
-    return fail(kWorkspace, "loss_forward_bf16: workspace of %zu bytes, %zu needed",
-                workspace_bytes, rnnt_hip_loss_workspace_bytes(B, T, U, V));
-  const Dims d = make_dims(B, T, U, V, blank);
-  RNNT_TRY(check_bf16_shape(E16, P16, d, "loss_forward_bf16"));
-  const bf16_t* E = reinterpret_cast<const bf16_t*>(E16);
-  const bf16_t* P = reinterpret_cast<const bf16_t*>(P16);
-  LossWorkspace w;
-  loss_workspace_layout(d, workspace, &w);
-  RNNT_STAGE(kRowmax, launch_rowmax_pick_p(P, w.mP, labels, labLen, w.planes, d, s));
-  RNNT_STAGE(kYplanes, launch_yplanes(P, w.mP, w.lse_scratch, labLen, d, s));
-  RNNT_STAGE(kLse, launch_lse_stream(E, w.mE, w.mP, w.LN, w.lse_scratch, inLen, labLen, d, s,
-                                     labels, w.planes.elS, w.planes.eb));
-  RNNT_STAGE(kSkew, launch_skew(w.LN, w.planes.lnS, inLen, labLen, d, s));
-  RNNT_STAGE(kAlpha, launch_alpha(w.planes, inLen, labLen, costs, d, s));
-  return kOk;
-}
-
-int rnnt_hip_loss_backward_bf16(const uint16_t* E16, const uint16_t* P16, const int* labels,
-                                const int* inLen, const int* labLen, const float* deltas,
-                                uint16_t* egrads16, uint16_t* pgrads16, void* workspace,
-                                size_t workspace_bytes, int B, int T, int U, int V, int blank,
-                                rnnt_stream_t stream) {
-  RNNT_TRY(check_dims(B, T, U, V));
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  if (B == 0 || V == 0) return kOk;
-  if (nothing_to_do(B, T, U)) {
-    if (egrads16 && (size_t)T * V)
-      RNNT_HIP(hipMemsetAsync(egrads16, 0, sizeof(uint16_t) * (size_t)B * T * V, s));
-    if (pgrads16 && (size_t)U * V)
-      RNNT_HIP(hipMemsetAsync(pgrads16, 0, sizeof(uint16_t) * (size_t)B * U * V, s));
-    return kOk;
+// 16-bit scores (bf16, fp16): the shapes the streaming kernels take (every launcher below exists
+// for all three element types; the general-shape fallbacks are fp32 only).  The three entry
+// points per type are thin wrappers around the templates above.
+#define RNNT_LOWP_ENTRY_POINTS(SUFFIX, TIO)                                                       \
+  int rnnt_hip_loss_forward_##SUFFIX(const uint16_t* E, const uint16_t* P, const int* labels,     \
+                                     const int* inLen, const int* labLen, float* costs,           \
+                                     void* workspace, size_t workspace_bytes, int B, int T,       \
+                                     int U, int V, int blank, rnnt_stream_t stream) {             \
+    return lowp_loss_forward(reinterpret_cast<const TIO*>(E), reinterpret_cast<const TIO*>(P),    \
+                             labels, inLen, labLen, costs, workspace, workspace_bytes, B, T, U,   \
+                             V, blank, stream, "loss_forward_" #SUFFIX);                          \
+  }                                                                                               \
+  int rnnt_hip_loss_backward_##SUFFIX(const uint16_t* E, const uint16_t* P, const int* labels,    \
+                                      const int* inLen, const int* labLen, const float* deltas,   \
+                                      uint16_t* egrads, uint16_t* pgrads, void* workspace,        \
+                                      size_t workspace_bytes, int B, int T, int U, int V,         \
+                                      int blank, rnnt_stream_t stream) {                          \
+    return lowp_loss_backward(reinterpret_cast<const TIO*>(E), reinterpret_cast<const TIO*>(P),   \
+                              labels, inLen, labLen, deltas, reinterpret_cast<TIO*>(egrads),      \
+                              reinterpret_cast<TIO*>(pgrads), workspace, workspace_bytes, B, T,   \
+                              U, V, blank, stream, "loss_backward_" #SUFFIX);                     \
+  }                                                                                               \
+  int rnnt_hip_viterbi_decode_##SUFFIX(const uint16_t* E, const uint16_t* P, const int* inLen,    \
+                                       const int* labLen, int* labels, int B, int T, int U,       \
+                                       int V, int blank, rnnt_stream_t stream) {                  \
+    return lowp_viterbi_decode(reinterpret_cast<const TIO*>(E), reinterpret_cast<const TIO*>(P),  \
+                               inLen, labLen, labels, B, T, U, V, blank, stream,                  \
+                               "viterbi_decode_" #SUFFIX);                                        \
   }
-  if (!E16 || !P16 || !egrads16 || !pgrads16 || !inLen || !labLen || (U > 1 && !labels))
-    return fail(kInvalid, "loss_backward_bf16: null array argument");
-  if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & 255))
-    return fail(kInvalid, "loss_backward_bf16: workspace must be a 256-byte aligned device pointer");
-  if (workspace_bytes < rnnt_hip_loss_workspace_bytes(B, T, U, V))
-    return fail(kWorkspace, "loss_backward_bf16: workspace of %zu bytes, %zu needed",
-                workspace_bytes, rnnt_hip_loss_workspace_bytes(B, T, U, V));
-  const Dims d = make_dims(B, T, U, V, blank);
-  RNNT_TRY(check_bf16_shape(E16, P16, d, "loss_backward_bf16"));
-  if ((reinterpret_cast<uintptr_t>(egrads16) | reinterpret_cast<uintptr_t>(pgrads16)) & 1)
-    return fail(kInvalid, "loss_backward_bf16: misaligned gradient arrays");
-  const bf16_t* E = reinterpret_cast<const bf16_t*>(E16);
-  const bf16_t* P = reinterpret_cast<const bf16_t*>(P16);
-  LossWorkspace w;
-  loss_workspace_layout(d, workspace, &w);
-  RNNT_STAGE(kWeights, launch_weights(w.planes, inLen, labLen, d, s));
-  RNNT_STAGE(kBeta, launch_beta(w.planes, labels, inLen, labLen, d, s));
-  RNNT_STAGE(kWplanes, launch_wplanes_skewed(w.planes.dS, w.planes.lnS, w.mE, w.mP, w.Wn, w.Wt,
-                                             inLen, labLen, d, s));
-  // Both gradients are rounded to bf16 once, from the complete fp32 value: the blank / label
-  // terms are always folded into the dense kernels' write-outs here, whatever the vocabulary.
-  // With U == 1 there are no labels; the kernels then never read the list, but its pointer is
-  // what switches the folding on, so any valid device pointer serves.
-  const int* lab = labels ? labels : inLen;
-  RNNT_STAGE(kSparse, launch_blank_sums(w.planes, w.bsum, lab, inLen, labLen, d, s));
-  SparseTerms sp;
-  sp.dS = w.planes.dS; sp.wE = w.planes.wE; sp.bsum = w.bsum; sp.labels = lab;
-  SparsePTerms spp;
-  spp.gB = w.planes.gB; spp.gL = w.planes.gL; spp.labels = lab;
-  RNNT_STAGE(kEgrads, launch_egrads_stream(E, P, w.mE, w.mP, w.Wn, deltas,
-                                           reinterpret_cast<bf16_t*>(egrads16), inLen, labLen, d,
-                                           false, sp, s));
-  RNNT_STAGE(kPgrads, launch_pgrads_stream(E, P, w.mE, w.mP, w.Wt, deltas,
-                                           reinterpret_cast<bf16_t*>(pgrads16), inLen, labLen, d,
-                                           false, spp, s));
-  return kOk;
-}
-
-int rnnt_hip_viterbi_decode_bf16(const uint16_t* E16, const uint16_t* P16, const int* inLen,
-                                 const int* labLen, int* labels, int B, int T, int U, int V,
-                                 int blank, rnnt_stream_t stream) {
-  RNNT_TRY(check_dims(B, T, U, V));
-  if (nothing_to_do(B, T, U) || U == 1) return kOk;  // no label to emit
-  if (V == 0) return fail(kInvalid, "viterbi_decode_bf16: empty vocabulary");
-  if (!E16 || !P16 || !labels || !inLen || !labLen)
-    return fail(kInvalid, "viterbi_decode_bf16: null array argument");
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  const Dims d = make_dims(B, T, U, V, blank);
-  if (d.V % 8 != 0)
-    return fail(kInvalid, "viterbi_decode_bf16: bf16 scores need a vocabulary that is a "
-                          "multiple of 8 (V=%d)", d.V);
-  if ((reinterpret_cast<uintptr_t>(E16) | reinterpret_cast<uintptr_t>(P16)) & 15)
-    return fail(kInvalid, "viterbi_decode_bf16: bf16 scores must be 16-byte aligned");
-  const bf16_t* E = reinterpret_cast<const bf16_t*>(E16);
-  const bf16_t* P = reinterpret_cast<const bf16_t*>(P16);
-  if (!lse_stream_supported(E, d))
-    return fail(kInvalid, "viterbi_decode_bf16: B*T*U too large for the bf16 path");
-  Scratch scratch(s);
-  const size_t btu = sizeof(float) * (size_t)B * T * U;
-  const size_t yb = lse_scratch_bytes(d);
-  RNNT_TRY(scratch.reserve(align_up(sizeof(float) * (size_t)B * T) +
-                           align_up(sizeof(float) * (size_t)B * U) + align_up(btu) +
-                           align_up(yb)));
-  float* mE = static_cast<float*>(scratch.take(sizeof(float) * (size_t)B * T));
-  float* mP = static_cast<float*>(scratch.take(sizeof(float) * (size_t)B * U));
-  float* LN = static_cast<float*>(scratch.take(btu));
-  void* ys = scratch.take(yb);
-  RNNT_STAGE(kRowmax, launch_rowmax(P, mP, (long)B * U, V, U, labLen, 1, s));
-  RNNT_STAGE(kYplanes, launch_yplanes(P, mP, ys, labLen, d, s));
-  RNNT_STAGE(kLse, launch_lse_stream(E, mE, mP, LN, ys, inLen, labLen, d, s));
-  return viterbi_impl(E, P, LN, labels, inLen, labLen, d, s);
-}
+RNNT_LOWP_ENTRY_POINTS(bf16, bf16_t)
+RNNT_LOWP_ENTRY_POINTS(f16, f16_t)
+#undef RNNT_LOWP_ENTRY_POINTS
 
 int rnnt_hip_viterbi_decode(const float* E, const float* P, const int* inLen, const int* labLen,
                             int* labels, int B, int T, int U, int V, int blank,

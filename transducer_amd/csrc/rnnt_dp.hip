@@ -1009,6 +1009,10 @@ int launch_gather(const bf16_t* E, const bf16_t* P, const int* labels, const int
                   const int* labLen, const Planes& p, const Dims& d, hipStream_t s) {
   return gather_any(E, P, labels, inLen, labLen, p, d, s);
 }
+int launch_gather(const f16_t* E, const f16_t* P, const int* labels, const int* inLen,
+                  const int* labLen, const Planes& p, const Dims& d, hipStream_t s) {
+  return gather_any(E, P, labels, inLen, labLen, p, d, s);
+}
 
 int launch_alpha(const Planes& p, const int* inLen, const int* labLen, float* costs,
                  const Dims& d, hipStream_t s) {
@@ -1107,6 +1111,10 @@ int launch_maxplus(const float* E, const float* P, const int* inLen, const int* 
   return maxplus_any(E, P, inLen, labLen, best, arg, d, s);
 }
 int launch_maxplus(const bf16_t* E, const bf16_t* P, const int* inLen, const int* labLen,
+                   float* best, int* arg, const Dims& d, hipStream_t s) {
+  return maxplus_any(E, P, inLen, labLen, best, arg, d, s);
+}
+int launch_maxplus(const f16_t* E, const f16_t* P, const int* inLen, const int* labLen,
                    float* best, int* arg, const Dims& d, hipStream_t s) {
   return maxplus_any(E, P, inLen, labLen, best, arg, d, s);
 }

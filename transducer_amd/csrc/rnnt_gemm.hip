@@ -14,6 +14,8 @@
 // Which element of the reduction sits in which k-slot is free as long as A and B agree, so a
 // lane takes four consecutive k of its row with one 16-byte LDS read and spends them on four
 // instructions.
+#include <type_traits>
+
 #include "rnnt_internal.h"
 
 namespace rnnt {
@@ -31,8 +33,9 @@ __device__ inline float wave_max(float m) {
 }
 
 // ------------------------------------------------------------------ row maxima
-// bf16 rows (V % 8 == 0 and 16-byte aligned when vec is set): eight elements per load.
-__device__ inline float row_max(const bf16_t* __restrict__ x, int V, int vec, int lane) {
+// 16-bit rows (V % 8 == 0 and 16-byte aligned when vec is set): eight elements per load.
+template <typename T16, typename = std::enable_if_t<sizeof(T16) == 2>>
+__device__ inline float row_max(const T16* __restrict__ x, int V, int vec, int lane) {
   float m0 = kNegInf, m1 = kNegInf;
   if (vec) {
     for (int i = lane; i < (V >> 3); i += 64) {
@@ -497,6 +500,10 @@ int launch_rowmax(const bf16_t* X, float* rowmax, long rows, int V, int rows_per
                   const int* lengths, int extra, hipStream_t s) {
   return rowmax_any(X, rowmax, rows, V, rows_per_item, lengths, extra, s);
 }
+int launch_rowmax(const f16_t* X, float* rowmax, long rows, int V, int rows_per_item,
+                  const int* lengths, int extra, hipStream_t s) {
+  return rowmax_any(X, rowmax, rows, V, rows_per_item, lengths, extra, s);
+}
 
 int launch_rowmax_pick(const float* E, const float* P, float* mE, float* mP, const int* labels,
                        const int* inLen, const int* labLen, const Planes& p, const Dims& d,
@@ -528,6 +535,10 @@ int launch_rowmax_pick_p(const float* P, float* mP, const int* labels, const int
   return rowmax_pick_p_any(P, mP, labels, labLen, p, d, s);
 }
 int launch_rowmax_pick_p(const bf16_t* P, float* mP, const int* labels, const int* labLen,
+                         const Planes& p, const Dims& d, hipStream_t s) {
+  return rowmax_pick_p_any(P, mP, labels, labLen, p, d, s);
+}
+int launch_rowmax_pick_p(const f16_t* P, float* mP, const int* labels, const int* labLen,
                          const Planes& p, const Dims& d, hipStream_t s) {
   return rowmax_pick_p_any(P, mP, labels, labLen, p, d, s);
 }

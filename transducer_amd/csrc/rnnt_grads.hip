@@ -640,6 +640,13 @@ int launch_egrads_stream(const bf16_t* E, const bf16_t* P, const float* mE, cons
   return egrads_stream_any(E, P, mE, mP, Wn, deltas, egrads, inLen, labLen, d, accumulate, sparse,
                            s);
 }
+int launch_egrads_stream(const f16_t* E, const f16_t* P, const float* mE, const float* mP,
+                         const float* Wn, const float* deltas, f16_t* egrads, const int* inLen,
+                         const int* labLen, const Dims& d, bool accumulate,
+                         const SparseTerms& sparse, hipStream_t s) {
+  return egrads_stream_any(E, P, mE, mP, Wn, deltas, egrads, inLen, labLen, d, accumulate, sparse,
+                           s);
+}
 
 template <typename TIO>
 static int pgrads_stream_any(const TIO* E, const TIO* P, const float* mE, const float* mP,
@@ -667,6 +674,12 @@ int launch_pgrads_stream(const float* E, const float* P, const float* mE, const 
 }
 int launch_pgrads_stream(const bf16_t* E, const bf16_t* P, const float* mE, const float* mP,
                          const float* Wt, const float* deltas, bf16_t* pgrads, const int* inLen,
+                         const int* labLen, const Dims& d, bool accumulate,
+                         const SparsePTerms& sp, hipStream_t s) {
+  return pgrads_stream_any(E, P, mE, mP, Wt, deltas, pgrads, inLen, labLen, d, accumulate, sp, s);
+}
+int launch_pgrads_stream(const f16_t* E, const f16_t* P, const float* mE, const float* mP,
+                         const float* Wt, const float* deltas, f16_t* pgrads, const int* inLen,
                          const int* labLen, const Dims& d, bool accumulate,
                          const SparsePTerms& sp, hipStream_t s) {
   return pgrads_stream_any(E, P, mE, mP, Wt, deltas, pgrads, inLen, labLen, d, accumulate, sp, s);

@@ -103,6 +103,8 @@ int launch_gather(const float* E, const float* P, const int* labels, const int* 
                   const int* labLen, const Planes& p, const Dims& d, hipStream_t s);
 int launch_gather(const bf16_t* E, const bf16_t* P, const int* labels, const int* inLen,
                   const int* labLen, const Planes& p, const Dims& d, hipStream_t s);
+int launch_gather(const f16_t* E, const f16_t* P, const int* labels, const int* inLen,
+                  const int* labLen, const Planes& p, const Dims& d, hipStream_t s);
 int launch_alpha(const Planes& p, const int* inLen, const int* labLen, float* costs,
                  const Dims& d, hipStream_t s);
 int launch_weights(const Planes& p, const int* inLen, const int* labLen, const Dims& d,
@@ -122,6 +124,8 @@ int launch_maxplus(const float* E, const float* P, const int* inLen, const int* 
                    float* best, int* arg, const Dims& d, hipStream_t s);
 int launch_maxplus(const bf16_t* E, const bf16_t* P, const int* inLen, const int* labLen,
                    float* best, int* arg, const Dims& d, hipStream_t s);
+int launch_maxplus(const f16_t* E, const f16_t* P, const int* inLen, const int* labLen,
+                   float* best, int* arg, const Dims& d, hipStream_t s);
 // bestS / argS: skewed planes of the max-plus table (argS carries int bits in float storage).
 int launch_viterbi(const Planes& p, const float* bestS, const float* argS,
                    unsigned long long* gbits, const int* inLen, const int* labLen,
@@ -136,6 +140,8 @@ int wplane_tw(int T);  // frame-axis pitch of the W planes (multiple of 64)
 int launch_rowmax(const float* X, float* rowmax, long rows, int V, int rows_per_item,
                   const int* lengths, int extra, hipStream_t s);
 int launch_rowmax(const bf16_t* X, float* rowmax, long rows, int V, int rows_per_item,
+                  const int* lengths, int extra, hipStream_t s);
+int launch_rowmax(const f16_t* X, float* rowmax, long rows, int V, int rows_per_item,
                   const int* lengths, int extra, hipStream_t s);
 // Row maxima of E and P and, in the same pass, what launch_gather extracts (E[t,blank],
 // E[t,label_u], P[u,blank], P[u,label_u] into the planes); needs inLen and labLen.
@@ -153,10 +159,13 @@ int launch_lse(const float* E, const float* P, const float* mE, const float* mP,
 // arrays (rnnt_io.h); the bf16 forms need V % 8 == 0.
 bool lse_stream_supported(const float* E, const Dims& d);
 bool lse_stream_supported(const bf16_t* E, const Dims& d);
+bool lse_stream_supported(const f16_t* E, const Dims& d);
 size_t lse_scratch_bytes(const Dims& d);
 int launch_yplanes(const float* P, const float* mP, void* scratch, const int* labLen,
                    const Dims& d, hipStream_t s);
 int launch_yplanes(const bf16_t* P, const float* mP, void* scratch, const int* labLen,
+                   const Dims& d, hipStream_t s);
+int launch_yplanes(const f16_t* P, const float* mP, void* scratch, const int* labLen,
                    const Dims& d, hipStream_t s);
 // With elS / eb (skewed label-score plane and blank-score vector) it also copies E[t, label_u]
 // and E[t, blank] out of the rows it streams (what launch_gather does for the emissions).
@@ -168,10 +177,16 @@ int launch_lse_stream(const bf16_t* E, float* mE, const float* mP, float* LN,
                       const void* scratch, const int* inLen, const int* labLen, const Dims& d,
                       hipStream_t s, const int* labels = nullptr, float* elS = nullptr,
                       float* eb = nullptr);
+int launch_lse_stream(const f16_t* E, float* mE, const float* mP, float* LN,
+                      const void* scratch, const int* inLen, const int* labLen, const Dims& d,
+                      hipStream_t s, const int* labels = nullptr, float* elS = nullptr,
+                      float* eb = nullptr);
 // P[u, blank] and P[u, label_u] into the planes, with the row maxima of P (one pass).
 int launch_rowmax_pick_p(const float* P, float* mP, const int* labels, const int* labLen,
                          const Planes& p, const Dims& d, hipStream_t s);
 int launch_rowmax_pick_p(const bf16_t* P, float* mP, const int* labels, const int* labLen,
+                         const Planes& p, const Dims& d, hipStream_t s);
+int launch_rowmax_pick_p(const f16_t* P, float* mP, const int* labels, const int* labLen,
                          const Planes& p, const Dims& d, hipStream_t s);
 int launch_wplanes(const float* lngrads, const float* LN, const float* mE, const float* mP,
                    float* Wn, float* Wt, const int* inLen, const int* labLen, const Dims& d,
@@ -219,12 +234,20 @@ int launch_egrads_stream(const bf16_t* E, const bf16_t* P, const float* mE, cons
                          const float* Wn, const float* deltas, bf16_t* egrads, const int* inLen,
                          const int* labLen, const Dims& d, bool accumulate,
                          const SparseTerms& sparse, hipStream_t s);
+int launch_egrads_stream(const f16_t* E, const f16_t* P, const float* mE, const float* mP,
+                         const float* Wn, const float* deltas, f16_t* egrads, const int* inLen,
+                         const int* labLen, const Dims& d, bool accumulate,
+                         const SparseTerms& sparse, hipStream_t s);
 int launch_pgrads_stream(const float* E, const float* P, const float* mE, const float* mP,
                          const float* Wt, const float* deltas, float* pgrads, const int* inLen,
                          const int* labLen, const Dims& d, bool accumulate,
                          const SparsePTerms& sparse, hipStream_t s);
 int launch_pgrads_stream(const bf16_t* E, const bf16_t* P, const float* mE, const float* mP,
                          const float* Wt, const float* deltas, bf16_t* pgrads, const int* inLen,
+                         const int* labLen, const Dims& d, bool accumulate,
+                         const SparsePTerms& sparse, hipStream_t s);
+int launch_pgrads_stream(const f16_t* E, const f16_t* P, const float* mE, const float* mP,
+                         const float* Wt, const float* deltas, f16_t* pgrads, const int* inLen,
                          const int* labLen, const Dims& d, bool accumulate,
                          const SparsePTerms& sparse, hipStream_t s);
 

@@ -1,7 +1,7 @@
 // Element types of the score arrays (emissions, predictions) and of their gradients at the
-// library's interface: fp32, as in the reference, or bf16 for a caller whose projection layers
-// produce bf16 logits.  The kernels are written once over these helpers; all arithmetic stays
-// fp32 (a bf16 score converts exactly), only the loads and the final stores differ.
+// library's interface: fp32, as in the reference, or bf16 / fp16 for a caller whose projection
+// layers produce 16-bit logits.  The kernels are written once over these helpers; all arithmetic
+// stays fp32 (a 16-bit score converts exactly), only the loads and the final stores differ.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -20,7 +20,20 @@ __device__ inline unsigned short float_to_bf16(float v) {
   return __builtin_bit_cast(unsigned short, (__bf16)v);
 }
 
+struct f16_t {
+  unsigned short bits;
+};
+__device__ inline float f16_to_float(unsigned short b) {
+  return (float)__builtin_bit_cast(_Float16, b);
+}
+// round to nearest even (v_cvt_f16_f32); values past 65504 become infinity
+__device__ inline unsigned short float_to_f16(float v) {
+  return __builtin_bit_cast(unsigned short, (_Float16)v);
+}
+
 __device__ inline float ldf(const float* p) { return *p; }
+__device__ inline float ldf(const f16_t* p) { return f16_to_float(p->bits); }
+__device__ inline void stf(f16_t* p, float v) { p->bits = float_to_f16(v); }
 __device__ inline float ldf(const bf16_t* p) { return bf16_to_float(p->bits); }
 __device__ inline void stf(float* p, float v) { *p = v; }
 __device__ inline void stf(bf16_t* p, float v) { p->bits = float_to_bf16(v); }
@@ -33,6 +46,14 @@ __device__ inline float4 load4(const bf16_t* p) {
                      __uint_as_float(w.y << 16), __uint_as_float(w.y & 0xffff0000u));
 }
 
+__device__ inline float4 load4(const f16_t* p) {
+  const uint2 w = *reinterpret_cast<const uint2*>(p);
+  return make_float4(f16_to_float((unsigned short)(w.x & 0xffffu)),
+                     f16_to_float((unsigned short)(w.x >> 16)),
+                     f16_to_float((unsigned short)(w.y & 0xffffu)),
+                     f16_to_float((unsigned short)(w.y >> 16)));
+}
+
 // Eight consecutive elements of a row as they sit in registers after the load.
 template <typename T>
 struct Raw8;
@@ -42,6 +63,10 @@ struct Raw8<float> {
 };
 template <>
 struct Raw8<bf16_t> {
+  uint4 w;
+};
+template <>
+struct Raw8<f16_t> {
   uint4 w;
 };
 
@@ -58,6 +83,20 @@ __device__ inline Raw8<bf16_t> load8(const bf16_t* row, int v, int V) {
   Raw8<bf16_t> r;
   r.w = *reinterpret_cast<const uint4*>(row + min(v, V - 8));
   return r;
+}
+
+__device__ inline Raw8<f16_t> load8(const f16_t* row, int v, int V) {
+  Raw8<f16_t> r;
+  r.w = *reinterpret_cast<const uint4*>(row + min(v, V - 8));
+  return r;
+}
+__device__ inline void expand(const Raw8<f16_t>& r, float (&e)[8]) {
+  const unsigned w[4] = {r.w.x, r.w.y, r.w.z, r.w.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    e[2 * i] = f16_to_float((unsigned short)(w[i] & 0xffffu));
+    e[2 * i + 1] = f16_to_float((unsigned short)(w[i] >> 16));
+  }
 }
 
 __device__ inline void expand(const Raw8<float>& r, float (&e)[8]) {
@@ -80,6 +119,10 @@ struct RowAlign<float> {
 };
 template <>
 struct RowAlign<bf16_t> {
+  static constexpr int kElems = 8;
+};
+template <>
+struct RowAlign<f16_t> {
   static constexpr int kElems = 8;
 };
 

@@ -433,6 +433,7 @@ static bool lse_stream_ok(const TIO* E, const Dims& d) {
 }
 bool lse_stream_supported(const float* E, const Dims& d) { return lse_stream_ok(E, d); }
 bool lse_stream_supported(const bf16_t* E, const Dims& d) { return lse_stream_ok(E, d); }
+bool lse_stream_supported(const f16_t* E, const Dims& d) { return lse_stream_ok(E, d); }
 
 size_t lse_scratch_bytes(const Dims& d) {
   if (d.B == 0 || d.T == 0 || d.U == 0 || d.V % 4 != 0) return 0;
@@ -454,6 +455,10 @@ int launch_yplanes(const float* P, const float* mP, void* scratch, const int* la
   return yplanes_any(P, mP, scratch, labLen, d, s);
 }
 int launch_yplanes(const bf16_t* P, const float* mP, void* scratch, const int* labLen,
+                   const Dims& d, hipStream_t s) {
+  return yplanes_any(P, mP, scratch, labLen, d, s);
+}
+int launch_yplanes(const f16_t* P, const float* mP, void* scratch, const int* labLen,
                    const Dims& d, hipStream_t s) {
   return yplanes_any(P, mP, scratch, labLen, d, s);
 }
@@ -480,6 +485,11 @@ int launch_lse_stream(const float* E, float* mE, const float* mP, float* LN,
   return lse_stream_any(E, mE, mP, LN, scratch, inLen, labLen, d, s, labels, elS, eb);
 }
 int launch_lse_stream(const bf16_t* E, float* mE, const float* mP, float* LN,
+                      const void* scratch, const int* inLen, const int* labLen, const Dims& d,
+                      hipStream_t s, const int* labels, float* elS, float* eb) {
+  return lse_stream_any(E, mE, mP, LN, scratch, inLen, labLen, d, s, labels, elS, eb);
+}
+int launch_lse_stream(const f16_t* E, float* mE, const float* mP, float* LN,
                       const void* scratch, const int* inLen, const int* labLen, const Dims& d,
                       hipStream_t s, const int* labels, float* elS, float* eb) {
   return lse_stream_any(E, mE, mP, LN, scratch, inLen, labLen, d, s, labels, elS, eb);

@@ -43,6 +43,10 @@ def _require_device(tensor):
         raise ValueError("Transducer not built with the CPU backend.")
 
 
+# entry-point suffix per 16-bit score type
+_SUFFIX = {torch.bfloat16: "_bf16", torch.float16: "_f16"}
+
+
 def _stream(device):
     return torch.cuda.current_stream(device).cuda_stream
 
@@ -52,10 +56,10 @@ class Transducer(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, emissions, predictions, labels, input_lengths, label_lengths, blank=0,
-                allow_bf16=False):
-        bf16 = allow_bf16 and emissions.dtype is torch.bfloat16
+                low_precision=()):
+        suffix = _SUFFIX[emissions.dtype] if emissions.dtype in low_precision else ""
         certify_inputs(emissions, predictions, labels, input_lengths, label_lengths,
-                       score_dtype=torch.bfloat16 if bf16 else torch.float32)
+                       score_dtype=emissions.dtype if suffix else torch.float32)
         _require_device(emissions)
         device = emissions.device
         # the library reads raw pointers: dense row-major storage is required
@@ -67,14 +71,14 @@ class Transducer(torch.autograd.Function):
         nbytes = _transducer.loss_workspace_bytes(B, T, U, V)
         workspace = torch.empty(size=(nbytes,), device=device, dtype=torch.uint8)
         with DeviceManager(device):
-            (_transducer.loss_forward_bf16 if bf16 else _transducer.loss_forward)(
+            getattr(_transducer, "loss_forward" + suffix)(
                 emissions.data_ptr(), predictions.data_ptr(), labels.data_ptr(),
                 input_lengths.data_ptr(), label_lengths.data_ptr(), costs.data_ptr(),
                 workspace.data_ptr(), nbytes, B, T, U, V, blank, _stream(device))
         ctx.save_for_backward(
             emissions, predictions, labels, input_lengths, label_lengths, workspace)
         ctx.blank = blank
-        ctx.bf16 = bf16
+        ctx.suffix = suffix
         return costs
 
     @staticmethod
@@ -88,7 +92,7 @@ class Transducer(torch.autograd.Function):
         egrads = torch.empty(size=(B, T, V), device=device, dtype=emissions.dtype)
         pgrads = torch.empty(size=(B, U, V), device=device, dtype=emissions.dtype)
         with DeviceManager(device):
-            (_transducer.loss_backward_bf16 if ctx.bf16 else _transducer.loss_backward)(
+            getattr(_transducer, "loss_backward" + ctx.suffix)(
                 emissions.data_ptr(), predictions.data_ptr(), labels.data_ptr(),
                 input_lengths.data_ptr(), label_lengths.data_ptr(), deltas.data_ptr(),
                 egrads.data_ptr(), pgrads.data_ptr(), workspace.data_ptr(), workspace.numel(),
@@ -104,17 +108,24 @@ class TransducerLoss(torch.nn.Module):
     every tensor has to sit on one HIP device.
 
     blank: id of the blank symbol (0 unless given).
-    allow_bf16: when True, ``torch.bfloat16`` emissions and predictions (both) are accepted as
-        well; costs are float32 and the gradients come back as bfloat16.  The reference raises
-        ``TypeError`` for anything but float32, and so does this module unless the flag is set.
-        Needs a vocabulary that is a multiple of 8 and, for the loss, at most 112 label
-        positions.
+    allow_bf16, allow_fp16: when True, ``torch.bfloat16`` / ``torch.float16`` emissions and
+        predictions (both of the same type) are accepted as well; costs are float32 and the
+        gradients come back in the scores' type.  The reference raises ``TypeError`` for
+        anything but float32, and so does this module unless a flag is set.  Needs a vocabulary
+        that is a multiple of 8 and, for the loss, at most 112 label positions.
     """
 
-    def __init__(self, blank=0, allow_bf16=False):
+    def __init__(self, blank=0, allow_bf16=False, allow_fp16=False):
         super(TransducerLoss, self).__init__()
         self.blank = blank
         self.allow_bf16 = allow_bf16
+        self.allow_fp16 = allow_fp16
+
+    @property
+    def low_precision(self):
+        """Score types accepted besides float32."""
+        return tuple(t for t, on in ((torch.bfloat16, self.allow_bf16),
+                                     (torch.float16, self.allow_fp16)) if on)
 
     def forward(self, emissions, predictions, labels, input_lengths, label_lengths):
         """costs[B] (float32) for a padded batch.
@@ -129,7 +140,7 @@ class TransducerLoss(torch.nn.Module):
         Differentiable with respect to emissions and predictions (once)."""
         return Transducer.apply(
             emissions, predictions, labels, input_lengths, label_lengths, self.blank,
-            self.allow_bf16)
+            self.low_precision)
 
     @torch.no_grad()
     def viterbi(self, emissions, predictions, input_lengths, label_lengths):
@@ -140,14 +151,14 @@ class TransducerLoss(torch.nn.Module):
         B, T, V = emissions.shape
         U = predictions.shape[1]
         labels = torch.empty(size=(B, U - 1), device=device, dtype=torch.int32)
-        bf16 = self.allow_bf16 and emissions.dtype is torch.bfloat16
+        suffix = _SUFFIX[emissions.dtype] if emissions.dtype in self.low_precision else ""
         certify_inputs(emissions, predictions, labels, input_lengths, label_lengths,
-                       score_dtype=torch.bfloat16 if bf16 else torch.float32)
+                       score_dtype=emissions.dtype if suffix else torch.float32)
         _require_device(emissions)
         emissions = emissions.contiguous()
         predictions = predictions.contiguous()
         with DeviceManager(device):
-            (_transducer.viterbi_decode_bf16 if bf16 else _transducer.viterbi_decode)(
+            getattr(_transducer, "viterbi_decode" + suffix)(
                 emissions.data_ptr(), predictions.data_ptr(), input_lengths.data_ptr(),
                 label_lengths.data_ptr(), labels.data_ptr(), B, T, U, V, self.blank,
                 _stream(device))
