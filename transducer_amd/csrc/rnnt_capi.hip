@@ -554,14 +554,14 @@ int rnnt_hip_loss_backward(const float* E, const float* P, const int* labels, co
   }
   RNNT_STAGE(kEgrads, launch_egrads(E, P, w.mE, w.mP, w.Wn, deltas, egrads, inLen, labLen, d, false,
                                     sp, s));
-  // pgrads takes its blank / label totals in its write-out too (the same two fp32 operations
-  // the scatter kernel would do afterwards, so the same bits)
+  // pgrads always takes its blank / label totals in its write-out (the same two fp32 operations
+  // the scatter kernel would do afterwards, so the same bits, and no extra launch)
   SparsePTerms spp;
-  if (fold) { spp.gB = w.planes.gB; spp.gL = w.planes.gL; spp.labels = labels; }
+  spp.gB = w.planes.gB; spp.gL = w.planes.gL; spp.labels = labels;
   RNNT_STAGE(kPgrads, launch_pgrads(E, P, w.mE, w.mP, w.Wt, deltas, pgrads, inLen, labLen, d, false,
                                     spp, s));
   if (!fold)
-    RNNT_STAGE(kSparse, launch_sparse(w.planes, egrads, pgrads, labels, inLen, labLen, deltas, true, d, s));
+    RNNT_STAGE(kSparse, launch_sparse(w.planes, egrads, nullptr, labels, inLen, labLen, deltas, true, d, s));
   return kOk;
 }
 

@@ -114,6 +114,7 @@ int launch_beta(const Planes& p, const int* labels, const int* inLen, const int*
 // Sparse blank/label terms.  add == false: written onto zero-filled egrads/pgrads exactly as
 // the reference's backward leaves them.  add == true: added, times scale[b] (1 when scale is
 // null), onto arrays that already hold the dense part.
+// pgrads == nullptr: only the egrads terms.
 int launch_sparse(const Planes& p, float* egrads, float* pgrads, const int* labels,
                   const int* inLen, const int* labLen, const float* scale, bool add,
                   const Dims& d, hipStream_t s);
