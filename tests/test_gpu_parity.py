@@ -392,3 +392,23 @@ def test_whole_loss_at_T2000_violation_fraction():
     err_dev = np.abs(eg - t["egrads"]).max()
     err_ref = np.abs(a["egrads"] - t["egrads"]).max()
     assert err_dev < 4 * err_ref + 1e-5
+
+
+def test_pgrads_split_over_frames_gives_the_bits_of_the_unsplit_walk():
+    """With a small vocabulary and a small batch several workgroups share a tile's frames
+    (chunks of 8 slabs, summed in chunk order); the additions are the ones the unsplit walk
+    performs, so one utterance alone (split) and the same utterance repeated 130 times (too
+    many tiles to split) must agree bit for bit, and so must a batch of 3."""
+    cfg = small_config(1, 600, 20, 100, ragged=False)
+    E, P, labels, il, ll = unpack(make_inputs(cfg, seed=4))
+    il = np.array([571], np.int32)   # not a multiple of a chunk, nor of a slab
+    ll = np.array([17], np.int32)
+    one = gpu_loss(DeviceCase(E, P, labels, il, ll))
+    for copies in (3, 130):
+        rep = lambda a: np.repeat(a, copies, axis=0)
+        many = gpu_loss(DeviceCase(rep(E), rep(P), rep(labels), rep(il), rep(ll)))
+        for got, want in zip(many, one):
+            assert np.array_equal(got[0], want[0]) and np.array_equal(got[-1], want[0])
+    want = oracle.loss_and_grads(E, P, labels, il, ll)
+    assert_close(one[0], want["costs"], what="costs")
+    assert_close(one[2], want["pgrads"], what="pgrads")

@@ -150,6 +150,7 @@ struct LossWorkspace {
   Planes planes;
   float *mE, *mP, *LN, *Wn, *Wt, *bsum;
   void* lse_scratch;
+  void* psplit;  // pgrads_split_bytes(d) bytes, or null
 };
 
 size_t loss_workspace_layout(const Dims& d, void* base, LossWorkspace* w) {
@@ -172,9 +173,11 @@ size_t loss_workspace_layout(const Dims& d, void* base, LossWorkspace* w) {
   float* Wt = take(wb);
   float* bsum = take(sizeof(float) * (size_t)d.B * d.T);
   void* ys = take(lse_scratch_bytes(d));  // forward only
+  void* ps = take(pgrads_split_bytes(d));  // backward only
   if (base) {
     w->mE = mE; w->mP = mP; w->LN = LN; w->Wn = Wn; w->Wt = Wt; w->bsum = bsum;
     w->lse_scratch = lse_scratch_bytes(d) ? ys : nullptr;
+    w->psplit = pgrads_split_bytes(d) ? ps : nullptr;
   }
   return off;
 }
@@ -306,7 +309,7 @@ int lowp_loss_backward(const TIO* E, const TIO* P, const int* labels, const int*
   RNNT_STAGE(kEgrads, launch_egrads_stream(E, P, w.mE, w.mP, w.Wn, deltas, egrads, inLen, labLen,
                                            d, false, sp, s));
   RNNT_STAGE(kPgrads, launch_pgrads_stream(E, P, w.mE, w.mP, w.Wt, deltas, pgrads, inLen, labLen,
-                                           d, false, spp, s));
+                                           d, false, spp, w.psplit, s));
   return kOk;
 }
 
@@ -468,18 +471,20 @@ int rnnt_hip_dense_grads(const float* E, const float* P, float* egrads, float* p
   const size_t wb = sizeof(float) * (size_t)B * wplane_tw(T) * wplane_up(U);
   Scratch scratch(s);
   RNNT_TRY(scratch.reserve(align_up(sizeof(float) * (size_t)B * T) +
-                           align_up(sizeof(float) * (size_t)B * U) + 2 * align_up(wb)));
+                           align_up(sizeof(float) * (size_t)B * U) + 2 * align_up(wb) +
+                           align_up(pgrads_split_bytes(d))));
   float* mE = static_cast<float*>(scratch.take(sizeof(float) * (size_t)B * T));
   float* mP = static_cast<float*>(scratch.take(sizeof(float) * (size_t)B * U));
   float* Wn = static_cast<float*>(scratch.take(wb));
   float* Wt = static_cast<float*>(scratch.take(wb));
+  void* psplit = pgrads_split_bytes(d) ? scratch.take(pgrads_split_bytes(d)) : nullptr;
   RNNT_STAGE(kRowmax, launch_rowmax(E, mE, (long)B * T, V, T, inLen, 0, s));
   RNNT_STAGE(kRowmax, launch_rowmax(P, mP, (long)B * U, V, U, labLen, 1, s));
   RNNT_STAGE(kWplanes, launch_wplanes(lngrads, LN, mE, mP, Wn, Wt, inLen, labLen, d, s));
   RNNT_STAGE(kEgrads, launch_egrads(E, P, mE, mP, Wn, deltas, egrads, inLen, labLen, d, true,
                                     SparseTerms(), s));
   RNNT_STAGE(kPgrads, launch_pgrads(E, P, mE, mP, Wt, deltas, pgrads, inLen, labLen, d, true,
-                                    SparsePTerms(), s));
+                                    SparsePTerms(), psplit, s));
   return kOk;
 }
 
@@ -559,7 +564,7 @@ int rnnt_hip_loss_backward(const float* E, const float* P, const int* labels, co
   SparsePTerms spp;
   spp.gB = w.planes.gB; spp.gL = w.planes.gL; spp.labels = labels;
   RNNT_STAGE(kPgrads, launch_pgrads(E, P, w.mE, w.mP, w.Wt, deltas, pgrads, inLen, labLen, d, false,
-                                    spp, s));
+                                    spp, w.psplit, s));
   if (!fold)
     RNNT_STAGE(kSparse, launch_sparse(w.planes, egrads, nullptr, labels, inLen, labLen, deltas, true, d, s));
   return kOk;

@@ -603,10 +603,10 @@ int launch_egrads(const float* E, const float* P, const float* mE, const float* 
 int launch_pgrads(const float* E, const float* P, const float* mE, const float* mP,
                   const float* Wt, const float* deltas, float* pgrads, const int* inLen,
                   const int* labLen, const Dims& d, bool accumulate, const SparsePTerms& sparse,
-                  hipStream_t s) {
+                  void* split_ws, hipStream_t s) {
   if (d.B == 0 || d.T == 0 || d.U == 0) return kOk;
   return launch_pgrads_stream(E, P, mE, mP, Wt, deltas, pgrads, inLen, labLen, d, accumulate,
-                              sparse, s);
+                              sparse, split_ws, s);
 }
 
 }  // namespace rnnt

@@ -387,15 +387,30 @@ struct PRowTerms {
   int label[128];
 };
 
+// Splitting a tile's frames over several workgroups (small grids: one utterance with a small
+// vocabulary is a single tile, whose workgroup would walk all frames alone).  Workgroup c of
+// `chunks` sums slabs [c*per, (c+1)*per) and leaves its sums in `partial`; the one that arrives
+// last at the tile's counter adds all of them up in chunk order (so the result does not depend
+// on who was last) and writes the tile.  Nobody waits for anybody.  per == kPsFlush, always:
+// see pgrads_split_plan.
+struct PSplit {
+  int chunks = 1, per = 0;
+  float* partial = nullptr;  // [tile][chunk][4 blocks][16 registers][256 threads]
+  int* counter = nullptr;    // [tile], zero before the launch
+};
+constexpr int kPsPartialFloats = 4 * 16 * 256;
+
 // One workgroup's 128 x 128 tile with NMB 32-row blocks of label positions in use (a template
 // parameter, so the matrix instructions of a slice form one straight-line block).  Products are
 // formed on the bf16 matrix cores from exact three-way splits of both operands (rnnt_split.h).
-template <int NMB, bool kAccumulate, typename TIO>
+template <int NMB, bool kAccumulate, bool kSplit, typename TIO>
 __device__ __forceinline__ void pgrads_tile(
     const TIO* __restrict__ E, const TIO* __restrict__ P, const float* __restrict__ mE,
     const float* __restrict__ mP, const float* __restrict__ Wt, const float* __restrict__ deltas,
     TIO* __restrict__ pgrads, unsigned short (*As)[3][kPsPlane], float (*Ms)[32], const Dims& d,
-    int Up, int Tw, int b, int u0, int Tb, int Ub, const PRowTerms* rt) {
+    int Up, int Tw, int b, int u0, int Tb, int Ub, const PRowTerms* rt, const PSplit& split,
+    int chunk, int tile, int* last_flag) {
+  if (kSplit && NMB == 0 && chunk > 0) return;  // nothing to sum: chunk 0 alone writes the zeros
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, h = lane >> 5;
   const int vcol = blockIdx.x * 128 + wave * 32 + l32;
   const bool vok = vcol < d.V;
@@ -459,12 +474,15 @@ __device__ __forceinline__ void pgrads_tile(
       if (tid < 32) Ms[buf][tid] = s.m;
     };
 
-    const int nk = (Tb + 31) >> 5;
-    store_slab(0, fetch_slab(0));
-    XRegs xr = fetch_x(0);
+    const int nk_all = (Tb + 31) >> 5;
+    const int k_lo = kSplit ? min(chunk * split.per, nk_all) : 0;
+    const int nk = kSplit ? min(k_lo + split.per, nk_all) : nk_all;  // one past the last slab
+    const int k_first = min(k_lo, nk_all - 1);  // (a chunk past the utterance loads, sums nothing)
+    store_slab(0, fetch_slab(k_first * 32));
+    XRegs xr = fetch_x(k_first * 32);
     __syncthreads();
     int cur = 0;
-    for (int kt = 0; kt < nk; ++kt) {
+    for (int kt = k_lo; kt < nk; ++kt) {
       // X = exp(E - mE) for this slab (finite everywhere; W^T is zero past the utterance and
       // columns past V are dropped on the way out), split into its three pieces in the
       // instruction's operand layout
@@ -510,7 +528,7 @@ __device__ __forceinline__ void pgrads_tile(
 #pragma unroll
         for (int mb = 0; mb < NMB; ++mb) acc[mb] = mfma_bf16(ah[mb], xb[s].h, acc[mb]);
       }
-      if ((kt + 1) % kPsFlush == 0) {
+      if ((kt - k_lo + 1) % kPsFlush == 0) {
 #pragma unroll
         for (int mb = 0; mb < NMB; ++mb)
 #pragma unroll
@@ -525,6 +543,37 @@ __device__ __forceinline__ void pgrads_tile(
   for (int mb = 0; mb < NMB; ++mb)
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[mb][r] += tot[mb][r];
+
+  if (kSplit && NMB > 0) {
+    float* mine = split.partial + ((size_t)tile * split.chunks + chunk) * kPsPartialFloats;
+#pragma unroll
+    for (int mb = 0; mb < NMB; ++mb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) mine[(mb * 16 + r) * 256 + tid] = acc[mb][r];
+    __threadfence();  // the sums are out before the arrival is counted
+    __syncthreads();
+    if (tid == 0) {
+      const int before = __hip_atomic_fetch_add(&split.counter[tile], 1, __ATOMIC_ACQ_REL,
+                                                __HIP_MEMORY_SCOPE_AGENT);
+      *last_flag = before == split.chunks - 1;
+    }
+    __syncthreads();
+    if (!*last_flag) return;
+    __threadfence();  // the others' sums are visible after their arrivals were seen
+    const float* all = split.partial + (size_t)tile * split.chunks * kPsPartialFloats;
+#pragma unroll
+    for (int mb = 0; mb < NMB; ++mb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[mb][r] = 0.0f;
+    for (int c = 0; c < split.chunks; ++c) {
+      const float* src = all + (size_t)c * kPsPartialFloats;
+#pragma unroll
+      for (int mb = 0; mb < NMB; ++mb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          acc[mb][r] += __builtin_nontemporal_load(&src[(mb * 16 + r) * 256 + tid]);
+    }
+  }
 
   const TIO* Pb = P + (size_t)b * d.U * d.V;
   const float* mPb = mP + (size_t)b * d.U;
@@ -551,16 +600,22 @@ __device__ __forceinline__ void pgrads_tile(
     }
 }
 
-template <bool kAccumulate, typename TIO>
+template <bool kAccumulate, bool kSplit, typename TIO>
 __global__ __launch_bounds__(256, 2) void pgrads_stream_kernel(
     const TIO* __restrict__ E, const TIO* __restrict__ P, const float* __restrict__ mE,
     const float* __restrict__ mP, const float* __restrict__ Wt, const float* __restrict__ deltas,
     TIO* __restrict__ pgrads, const int* __restrict__ inLen, const int* __restrict__ labLen,
-    Dims d, int Up, int Tw, SparsePTerms sp) {
+    Dims d, int Up, int Tw, SparsePTerms sp, PSplit split) {
   __shared__ __attribute__((aligned(16))) unsigned short As[2][3][kPsPlane];
   __shared__ __attribute__((aligned(16))) float Ms[2][32];
   __shared__ PRowTerms Rt;
-  const int b = blockIdx.z, u0 = blockIdx.y * 128;
+  __shared__ int last_flag;
+  const int b = blockIdx.z;
+  const int ut = kSplit ? blockIdx.y / split.chunks : blockIdx.y;
+  const int chunk = kSplit ? blockIdx.y - ut * split.chunks : 0;
+  const int utiles = kSplit ? gridDim.y / split.chunks : gridDim.y;
+  const int tile = (b * utiles + ut) * gridDim.x + blockIdx.x;
+  const int u0 = ut * 128;
   int Tb, Ub;
   utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
   const bool folding = !kAccumulate && sp.gB != nullptr;
@@ -577,9 +632,9 @@ __global__ __launch_bounds__(256, 2) void pgrads_stream_kernel(
   if (folding) __syncthreads();
   const PRowTerms* rt = folding ? &Rt : nullptr;
   const int nmb = (u0 < Ub && Tb > 0) ? min(4, (Ub - u0 + 31) >> 5) : 0;  // 32-row blocks in use
-#define RNNT_PG_TILE(NMB)                                                                    \
-  pgrads_tile<NMB, kAccumulate>(E, P, mE, mP, Wt, deltas, pgrads, As, Ms, d, Up, Tw, b, u0, \
-                                Tb, Ub, rt)
+#define RNNT_PG_TILE(NMB)                                                                   \
+  pgrads_tile<NMB, kAccumulate, kSplit>(E, P, mE, mP, Wt, deltas, pgrads, As, Ms, d, Up, Tw, \
+                                        b, u0, Tb, Ub, rt, split, chunk, tile, &last_flag)
   switch (nmb) {
     case 0: RNNT_PG_TILE(0); break;
     case 1: RNNT_PG_TILE(1); break;
@@ -648,41 +703,99 @@ int launch_egrads_stream(const f16_t* E, const f16_t* P, const float* mE, const 
                            s);
 }
 
+// Whether the workgroups of a tile share its frames.  A chunk is always kPsFlush slabs, the
+// period at which the unsplit walk moves its running sum into the second-level sum: the
+// chunks' sums, added in chunk order, then go through exactly the additions the unsplit walk
+// performs, so split and unsplit results are the same bits and an utterance's gradient does
+// not depend on the batch it is computed in.  Split only when the device would otherwise be
+// nearly empty (at most one workgroup per CU after the split): each chunk pays a start-up, a
+// device-scope fence and a share of the final addition.
+static void pgrads_split_plan(const Dims& d, int& chunks, int& per) {
+  const long tiles = (long)((d.V + 127) / 128) * ((d.U + 127) / 128) * d.B;
+  const int nk = (d.T + 31) / 32;
+  per = kPsFlush;
+  chunks = (nk + per - 1) / per;
+  if (chunks < 2 || tiles * chunks > 256) chunks = 1;
+}
+
+size_t pgrads_split_bytes(const Dims& d) {
+  if (d.B == 0 || d.T == 0 || d.U == 0 || d.V == 0) return 0;
+  int chunks, per;
+  pgrads_split_plan(d, chunks, per);
+  if (chunks <= 1) return 0;
+  const size_t tiles = (size_t)((d.V + 127) / 128) * ((d.U + 127) / 128) * d.B;
+  return tiles * chunks * kPsPartialFloats * sizeof(float) + ((tiles * sizeof(int) + 255) & ~(size_t)255);
+}
+
+__global__ void zero_ints_kernel(int* x, int n) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i < n) x[i] = 0;
+}
+
 template <typename TIO>
 static int pgrads_stream_any(const TIO* E, const TIO* P, const float* mE, const float* mP,
                              const float* Wt, const float* deltas, TIO* pgrads, const int* inLen,
                              const int* labLen, const Dims& d, bool accumulate,
-                             const SparsePTerms& sp, hipStream_t s) {
+                             const SparsePTerms& sp, void* split_ws, hipStream_t s) {
   if (sp.gB && accumulate)
     return fail(kInvalid, "sparse-term folding and accumulation are mutually exclusive");
   const int Up = wplane_up(d.U), Tw = wplane_tw(d.T);
-  const dim3 grid((d.V + 127) / 128, (d.U + 127) / 128, d.B);
+  const int vtiles = (d.V + 127) / 128, utiles = (d.U + 127) / 128;
+  PSplit split;
+  if (split_ws != nullptr) pgrads_split_plan(d, split.chunks, split.per);
+  if (split.chunks > 1) {
+    // counters first (256-byte multiple), partial sums behind them; cleared by a kernel, not a
+    // memset node, so that the call can be captured into a graph
+    const int tiles = vtiles * utiles * d.B;
+    split.counter = static_cast<int*>(split_ws);
+    split.partial = reinterpret_cast<float*>(static_cast<char*>(split_ws) +
+                                             ((tiles * sizeof(int) + 255) & ~(size_t)255));
+    hipLaunchKernelGGL(zero_ints_kernel, dim3((tiles + 255) / 256), dim3(256), 0, s,
+                       split.counter, tiles);
+    RNNT_LAUNCH_CHECK("zero_ints_kernel");
+    const dim3 grid(vtiles, utiles * split.chunks, d.B);
+    if (accumulate)
+      hipLaunchKernelGGL((pgrads_stream_kernel<true, true, TIO>), grid, dim3(256), 0, s, E, P, mE,
+                         mP, Wt, deltas, pgrads, inLen, labLen, d, Up, Tw, sp, split);
+    else
+      hipLaunchKernelGGL((pgrads_stream_kernel<false, true, TIO>), grid, dim3(256), 0, s, E, P, mE,
+                         mP, Wt, deltas, pgrads, inLen, labLen, d, Up, Tw, sp, split);
+    RNNT_LAUNCH_CHECK("pgrads_stream_kernel (split)");
+    return kOk;
+  }
+  const dim3 grid(vtiles, utiles, d.B);
   if (accumulate)
-    hipLaunchKernelGGL((pgrads_stream_kernel<true, TIO>), grid, dim3(256), 0, s, E, P, mE, mP, Wt,
-                       deltas, pgrads, inLen, labLen, d, Up, Tw, sp);
+    hipLaunchKernelGGL((pgrads_stream_kernel<true, false, TIO>), grid, dim3(256), 0, s, E, P, mE,
+                       mP, Wt, deltas, pgrads, inLen, labLen, d, Up, Tw, sp, split);
   else
-    hipLaunchKernelGGL((pgrads_stream_kernel<false, TIO>), grid, dim3(256), 0, s, E, P, mE, mP, Wt,
-                       deltas, pgrads, inLen, labLen, d, Up, Tw, sp);
+    hipLaunchKernelGGL((pgrads_stream_kernel<false, false, TIO>), grid, dim3(256), 0, s, E, P, mE,
+                       mP, Wt, deltas, pgrads, inLen, labLen, d, Up, Tw, sp, split);
   RNNT_LAUNCH_CHECK("pgrads_stream_kernel");
   return kOk;
 }
 int launch_pgrads_stream(const float* E, const float* P, const float* mE, const float* mP,
                          const float* Wt, const float* deltas, float* pgrads, const int* inLen,
                          const int* labLen, const Dims& d, bool accumulate,
-                         const SparsePTerms& sp, hipStream_t s) {
-  return pgrads_stream_any(E, P, mE, mP, Wt, deltas, pgrads, inLen, labLen, d, accumulate, sp, s);
+                         const SparsePTerms& sp, void* split_ws,
+                         hipStream_t s) {
+  return pgrads_stream_any(E, P, mE, mP, Wt, deltas, pgrads, inLen, labLen, d, accumulate, sp,
+                           split_ws, s);
 }
 int launch_pgrads_stream(const bf16_t* E, const bf16_t* P, const float* mE, const float* mP,
                          const float* Wt, const float* deltas, bf16_t* pgrads, const int* inLen,
                          const int* labLen, const Dims& d, bool accumulate,
-                         const SparsePTerms& sp, hipStream_t s) {
-  return pgrads_stream_any(E, P, mE, mP, Wt, deltas, pgrads, inLen, labLen, d, accumulate, sp, s);
+                         const SparsePTerms& sp, void* split_ws,
+                         hipStream_t s) {
+  return pgrads_stream_any(E, P, mE, mP, Wt, deltas, pgrads, inLen, labLen, d, accumulate, sp,
+                           split_ws, s);
 }
 int launch_pgrads_stream(const f16_t* E, const f16_t* P, const float* mE, const float* mP,
                          const float* Wt, const float* deltas, f16_t* pgrads, const int* inLen,
                          const int* labLen, const Dims& d, bool accumulate,
-                         const SparsePTerms& sp, hipStream_t s) {
-  return pgrads_stream_any(E, P, mE, mP, Wt, deltas, pgrads, inLen, labLen, d, accumulate, sp, s);
+                         const SparsePTerms& sp, void* split_ws,
+                         hipStream_t s) {
+  return pgrads_stream_any(E, P, mE, mP, Wt, deltas, pgrads, inLen, labLen, d, accumulate, sp,
+                           split_ws, s);
 }
 
 }  // namespace rnnt

@@ -219,10 +219,13 @@ int launch_egrads(const float* E, const float* P, const float* mE, const float* 
                   const float* Wn, const float* deltas, float* egrads, const int* inLen,
                   const int* labLen, const Dims& d, bool accumulate, const SparseTerms& sparse,
                   hipStream_t s);
+// split_ws: pgrads_split_bytes(d) bytes of scratch that let several workgroups share a tile's
+// frames when the grid is small (null: one workgroup per tile).
+size_t pgrads_split_bytes(const Dims& d);
 int launch_pgrads(const float* E, const float* P, const float* mE, const float* mP,
                   const float* Wt, const float* deltas, float* pgrads, const int* inLen,
                   const int* labLen, const Dims& d, bool accumulate, const SparsePTerms& sparse,
-                  hipStream_t s);
+                  void* split_ws, hipStream_t s);
 
 
 // ---------------------------------------------------------------- launchers (rnnt_grads.hip)
@@ -242,14 +245,17 @@ int launch_egrads_stream(const f16_t* E, const f16_t* P, const float* mE, const 
 int launch_pgrads_stream(const float* E, const float* P, const float* mE, const float* mP,
                          const float* Wt, const float* deltas, float* pgrads, const int* inLen,
                          const int* labLen, const Dims& d, bool accumulate,
-                         const SparsePTerms& sparse, hipStream_t s);
+                         const SparsePTerms& sparse, void* split_ws,
+                         hipStream_t s);
 int launch_pgrads_stream(const bf16_t* E, const bf16_t* P, const float* mE, const float* mP,
                          const float* Wt, const float* deltas, bf16_t* pgrads, const int* inLen,
                          const int* labLen, const Dims& d, bool accumulate,
-                         const SparsePTerms& sparse, hipStream_t s);
+                         const SparsePTerms& sparse, void* split_ws,
+                         hipStream_t s);
 int launch_pgrads_stream(const f16_t* E, const f16_t* P, const float* mE, const float* mP,
                          const float* Wt, const float* deltas, f16_t* pgrads, const int* inLen,
                          const int* labLen, const Dims& d, bool accumulate,
-                         const SparsePTerms& sparse, hipStream_t s);
+                         const SparsePTerms& sparse, void* split_ws,
+                         hipStream_t s);
 
 }  // namespace rnnt
