@@ -194,26 +194,28 @@ int fill(float* x, float v, int n, hipStream_t s) {
   return check_hip(hipGetLastError(), "launch fill_kernel", __FILE__, __LINE__);
 }
 
+// Scratch the best-path stages need (planes, the two max-plus planes, the decision table).
+size_t viterbi_scratch_bytes(const Dims& d) {
+  const size_t plane = sizeof(float) * (size_t)d.B * d.Ua * d.Dp + 64;
+  return align_up(planes_bytes(d)) + 2 * align_up(plane) + align_up(viterbi_bits_bytes(d));
+}
+
+// `scratch` has viterbi_scratch_bytes(d) left to take (one allocation per call, made by the caller
+// together with whatever else it needs: the allocator calls are a visible part of a small decode).
 template <typename TIO>
 int viterbi_impl(const TIO* E, const TIO* P, const float* LN, int* labels,
-                        const int* inLen, const int* labLen, const Dims& d, hipStream_t s) {
-  const size_t btu = sizeof(float) * (size_t)d.B * d.T * d.U;
+                        const int* inLen, const int* labLen, const Dims& d, Scratch& scratch,
+                        hipStream_t s) {
   const size_t plane = sizeof(float) * (size_t)d.B * d.Ua * d.Dp + 64;
-  Scratch scratch(s);
-  RNNT_TRY(scratch.reserve(align_up(planes_bytes(d)) + 2 * align_up(btu) + 2 * align_up(plane) +
-                           align_up(viterbi_bits_bytes(d))));
   Planes p;
   carve_planes(scratch.take(planes_bytes(d)), d, &p);
-  float* best = static_cast<float*>(scratch.take(btu));
-  int* arg = static_cast<int*>(scratch.take(btu));
   float* bestS = static_cast<float*>(scratch.take(plane));
   float* argS = static_cast<float*>(scratch.take(plane));
   unsigned long long* bits =
       static_cast<unsigned long long*>(scratch.take(viterbi_bits_bytes(d)));
-  RNNT_STAGE(kMaxplus, launch_maxplus(E, P, inLen, labLen, best, arg, d, s));
+  RNNT_STAGE(kMaxplus, launch_maxplus(E, P, inLen, labLen, bestS, reinterpret_cast<int*>(argS), d,
+                                      s));
   RNNT_STAGE(kSkew, launch_skew(LN, p.lnS, inLen, labLen, d, s));
-  RNNT_STAGE(kSkew, launch_skew(best, bestS, inLen, labLen, d, s));
-  RNNT_STAGE(kSkew, launch_skew(reinterpret_cast<const float*>(arg), argS, inLen, labLen, d, s));
   // blank scores only: the label planes of the gather are not needed here
   RNNT_STAGE(kGather, launch_gather(E, P, nullptr, inLen, labLen, p, d, s));
   RNNT_STAGE(kViterbi, launch_viterbi(p, bestS, argS, bits, inLen, labLen, labels, d, s));
@@ -331,7 +333,7 @@ int lowp_viterbi_decode(const TIO* E, const TIO* P, const int* inLen, const int*
   const size_t yb = lse_scratch_bytes(d);
   RNNT_TRY(scratch.reserve(align_up(sizeof(float) * (size_t)B * T) +
                            align_up(sizeof(float) * (size_t)B * U) + align_up(btu) +
-                           align_up(yb)));
+                           align_up(yb) + viterbi_scratch_bytes(d)));
   float* mE = static_cast<float*>(scratch.take(sizeof(float) * (size_t)B * T));
   float* mP = static_cast<float*>(scratch.take(sizeof(float) * (size_t)B * U));
   float* LN = static_cast<float*>(scratch.take(btu));
@@ -339,7 +341,7 @@ int lowp_viterbi_decode(const TIO* E, const TIO* P, const int* inLen, const int*
   RNNT_STAGE(kRowmax, launch_rowmax(P, mP, (long)B * U, V, U, labLen, 1, s));
   RNNT_STAGE(kYplanes, launch_yplanes(P, mP, ys, labLen, d, s));
   RNNT_STAGE(kLse, launch_lse_stream(E, mE, mP, LN, ys, inLen, labLen, d, s));
-  return viterbi_impl(E, P, LN, labels, inLen, labLen, d, s);
+  return viterbi_impl(E, P, LN, labels, inLen, labLen, d, scratch, s);
 }
 
 }  // namespace
@@ -436,8 +438,11 @@ int rnnt_hip_viterbi(const float* E, const float* P, const float* LN, int* label
   if (nothing_to_do(B, T, U) || U == 1) return kOk;  // no label to emit
   if (!E || !P || !LN || !labels || !inLen || !labLen)
     return fail(kInvalid, "viterbi: null array argument");
-  return viterbi_impl(E, P, LN, labels, inLen, labLen, make_dims(B, T, U, V, blank),
-                      static_cast<hipStream_t>(stream));
+  const Dims d = make_dims(B, T, U, V, blank);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  Scratch scratch(s);
+  RNNT_TRY(scratch.reserve(viterbi_scratch_bytes(d)));
+  return viterbi_impl(E, P, LN, labels, inLen, labLen, d, scratch, s);
 }
 
 int rnnt_hip_log_norms(const float* E, const float* P, float* LN, const int* inLen,
@@ -618,13 +623,13 @@ int rnnt_hip_viterbi_decode(const float* E, const float* P, const int* inLen, co
   const size_t yb = lse_stream_supported(E, d) ? lse_scratch_bytes(d) : 0;
   RNNT_TRY(scratch.reserve(align_up(sizeof(float) * (size_t)B * T) +
                            align_up(sizeof(float) * (size_t)B * U) + align_up(btu) +
-                           align_up(yb)));
+                           align_up(yb) + viterbi_scratch_bytes(d)));
   float* mE = static_cast<float*>(scratch.take(sizeof(float) * (size_t)B * T));
   float* mP = static_cast<float*>(scratch.take(sizeof(float) * (size_t)B * U));
   float* LN = static_cast<float*>(scratch.take(btu));
   void* ys = yb ? scratch.take(yb) : nullptr;
   RNNT_TRY(log_norms_stages(E, P, mE, mP, LN, ys, inLen, labLen, d, s));
-  return viterbi_impl(E, P, LN, labels, inLen, labLen, d, s);
+  return viterbi_impl(E, P, LN, labels, inLen, labLen, d, scratch, s);
 }
 
 }  // extern "C"

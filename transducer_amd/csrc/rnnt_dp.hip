@@ -827,7 +827,9 @@ __global__ __launch_bounds__(kMpThreads) void maxplus_kernel(const TIO* __restri
           if (ldf(e + v) + ldf(q + v) == top[i][r]) { at = v; break; }
         }
       }
-      const size_t o = ((size_t)b * d.T + t) * d.U + u;
+      // straight into the skewed planes the lattice walk reads (consecutive frames of one label
+      // position are neighbours there)
+      const size_t o = plane_row(d, b, u) + t + u;
       best[o] = top[i][r];
       arg[o] = at;
     }

@@ -121,6 +121,7 @@ int launch_sparse(const Planes& p, float* egrads, float* pgrads, const int* labe
 // bsum[b,t] = what the sparse terms leave in egrads[b,t,blank] (see blank_sums_kernel).
 int launch_blank_sums(const Planes& p, float* bsum, const int* labels, const int* inLen,
                       const int* labLen, const Dims& d, hipStream_t s);
+// best / arg: skewed planes ([B][Ua][Dp], see plane_row), written for valid cells only.
 int launch_maxplus(const float* E, const float* P, const int* inLen, const int* labLen,
                    float* best, int* arg, const Dims& d, hipStream_t s);
 int launch_maxplus(const bf16_t* E, const bf16_t* P, const int* inLen, const int* labLen,
