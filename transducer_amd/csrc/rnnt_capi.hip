@@ -119,15 +119,20 @@ bool nothing_to_do(int B, int T, int U) { return B == 0 || T == 0 || U == 0; }
 // recursions need (no separate gather).
 int log_norms_stages(const float* E, const float* P, float* mE, float* mP, float* LN,
                      void* scratch, const int* inLen, const int* labLen, const Dims& d,
-                     hipStream_t s, const Planes* planes = nullptr, const int* labels = nullptr) {
+                     hipStream_t s, const Planes* planes = nullptr, const int* labels = nullptr,
+                     bool* ln_in_plane = nullptr) {
+  if (ln_in_plane) *ln_in_plane = false;
   if (scratch && lse_stream_supported(E, d)) {
     // one pass over E: the streaming kernel finds its own per-frame reference and leaves it in mE
     // and, with `planes`, copies the blank / label scores out of the rows as they stream by
     if (planes && d.U - 1 <= 1024) {
       RNNT_STAGE(kRowmax, launch_rowmax_pick_p(P, mP, labels, labLen, *planes, d, s));
       RNNT_STAGE(kYplanes, launch_yplanes(P, mP, scratch, labLen, d, s));
+      // (with the flag the caller says it only needs LN in the lattice plane)
       RNNT_STAGE(kLse, launch_lse_stream(E, mE, mP, LN, scratch, inLen, labLen, d, s, labels,
-                                         planes->elS, planes->eb));
+                                         planes->elS, planes->eb,
+                                         ln_in_plane ? planes->lnS : nullptr));
+      if (ln_in_plane) *ln_in_plane = true;
       return kOk;
     }
     RNNT_STAGE(kRowmax, launch_rowmax(P, mP, (long)d.B * d.U, d.V, d.U, labLen, 1, s));
@@ -260,8 +265,7 @@ int lowp_loss_forward(const TIO* E, const TIO* P, const int* labels, const int* 
   RNNT_STAGE(kRowmax, launch_rowmax_pick_p(P, w.mP, labels, labLen, w.planes, d, s));
   RNNT_STAGE(kYplanes, launch_yplanes(P, w.mP, w.lse_scratch, labLen, d, s));
   RNNT_STAGE(kLse, launch_lse_stream(E, w.mE, w.mP, w.LN, w.lse_scratch, inLen, labLen, d, s,
-                                     labels, w.planes.elS, w.planes.eb));
-  RNNT_STAGE(kSkew, launch_skew(w.LN, w.planes.lnS, inLen, labLen, d, s));
+                                     labels, w.planes.elS, w.planes.eb, w.planes.lnS));
   RNNT_STAGE(kAlpha, launch_alpha(w.planes, inLen, labLen, costs, d, s));
   return kOk;
 }
@@ -517,9 +521,10 @@ int rnnt_hip_loss_forward(const float* E, const float* P, const int* labels, con
   const Dims d = make_dims(B, T, U, V, blank);
   LossWorkspace w;
   loss_workspace_layout(d, workspace, &w);
+  bool ln_in_plane = false;
   RNNT_TRY(log_norms_stages(E, P, w.mE, w.mP, w.LN, w.lse_scratch, inLen, labLen, d, s,
-                            &w.planes, labels));
-  RNNT_STAGE(kSkew, launch_skew(w.LN, w.planes.lnS, inLen, labLen, d, s));
+                            &w.planes, labels, &ln_in_plane));
+  if (!ln_in_plane) RNNT_STAGE(kSkew, launch_skew(w.LN, w.planes.lnS, inLen, labLen, d, s));
   RNNT_STAGE(kAlpha, launch_alpha(w.planes, inLen, labLen, costs, d, s));
   return kOk;
 }

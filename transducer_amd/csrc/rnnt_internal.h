@@ -171,18 +171,19 @@ int launch_yplanes(const f16_t* P, const float* mP, void* scratch, const int* la
                    const Dims& d, hipStream_t s);
 // With elS / eb (skewed label-score plane and blank-score vector) it also copies E[t, label_u]
 // and E[t, blank] out of the rows it streams (what launch_gather does for the emissions).
+// With lnS it writes LN into that skewed plane (valid cells) INSTEAD of the row-major LN.
 int launch_lse_stream(const float* E, float* mE, const float* mP, float* LN,
                       const void* scratch, const int* inLen, const int* labLen, const Dims& d,
                       hipStream_t s, const int* labels = nullptr, float* elS = nullptr,
-                      float* eb = nullptr);
+                      float* eb = nullptr, float* lnS = nullptr);
 int launch_lse_stream(const bf16_t* E, float* mE, const float* mP, float* LN,
                       const void* scratch, const int* inLen, const int* labLen, const Dims& d,
                       hipStream_t s, const int* labels = nullptr, float* elS = nullptr,
-                      float* eb = nullptr);
+                      float* eb = nullptr, float* lnS = nullptr);
 int launch_lse_stream(const f16_t* E, float* mE, const float* mP, float* LN,
                       const void* scratch, const int* inLen, const int* labLen, const Dims& d,
                       hipStream_t s, const int* labels = nullptr, float* elS = nullptr,
-                      float* eb = nullptr);
+                      float* eb = nullptr, float* lnS = nullptr);
 // P[u, blank] and P[u, label_u] into the planes, with the row maxima of P (one pass).
 int launch_rowmax_pick_p(const float* P, float* mP, const int* labels, const int* labLen,
                          const Planes& p, const Dims& d, hipStream_t s);

@@ -112,7 +112,8 @@ __global__ __launch_bounds__(64 * kWaves, kWaves / 2) void lse_stream_kernel(
     const TIO* __restrict__ E, float* __restrict__ mE, const float* __restrict__ mP,
     const uint4* __restrict__ Yp, float* __restrict__ LN, const int* __restrict__ inLen,
     const int* __restrict__ labLen, Dims d, int ttiles, int utiles, int total, int nub, int nks,
-    const int* __restrict__ labels, float* __restrict__ elS, float* __restrict__ ebv) {
+    const int* __restrict__ labels, float* __restrict__ elS, float* __restrict__ ebv,
+    float* __restrict__ lnS) {
   constexpr int kThreads = 64 * kWaves;
   constexpr int MB = 16 / kWaves;          // 32-frame blocks per wavefront
   constexpr int NR = 512 / kThreads;       // (row, eight v) items a thread stages per slab
@@ -134,11 +135,14 @@ __global__ __launch_bounds__(64 * kWaves, kWaves / 2) void lse_stream_kernel(
   float* LNb = LN + (size_t)b * d.T * d.U;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, h = lane >> 5;
 
+  // lnS given: LN goes straight into the lattice walk's skewed plane (valid cells only, as a
+  // transposing copy would leave it) and the row-major array is not written at all.
   if (t0 >= Tb || u0 >= Ub) {
-    for (int e = tid; e < kRows * 128; e += kThreads) {
-      const int t = t0 + e / 128, u = u0 + e % 128;
-      if (t < d.T && u < d.U) LNb[(size_t)t * d.U + u] = 0.0f;
-    }
+    if (lnS == nullptr)
+      for (int e = tid; e < kRows * 128; e += kThreads) {
+        const int t = t0 + e / 128, u = u0 + e % 128;
+        if (t < d.T && u < d.U) LNb[(size_t)t * d.U + u] = 0.0f;
+      }
     if (t0 >= Tb)  // frames past the utterance report a reference of 0
       for (int r = tid; r < kRows; r += kThreads)
         if (t0 + r < d.T) mE[(size_t)b * d.T + t0 + r] = 0.0f;
@@ -395,7 +399,7 @@ __global__ __launch_bounds__(64 * kWaves, kWaves / 2) void lse_stream_kernel(
   const int u = 32 * ublock + l32;
   if (!active) {
     // label positions past the utterance (but inside U) are written as zeros
-    if (u < d.U)
+    if (u < d.U && lnS == nullptr)
       for (int r = 0; r < 16 * MB; ++r) {
         const int t = t0 + 32 * (mb0 + (r >> 4)) + mfma_row(r & 15, h);
         if (t < d.T) LNb[(size_t)t * d.U + u] = 0.0f;
@@ -411,7 +415,8 @@ __global__ __launch_bounds__(64 * kWaves, kWaves / 2) void lse_stream_kernel(
       if (t < d.T && u < d.U) {
         float v = 0.0f;
         if (t < Tb && u < Ub) v = (logf(tot[m][r] + acc[m][r]) + mfin[row]) + mu;
-        LNb[(size_t)t * d.U + u] = v;
+        if (lnS == nullptr) LNb[(size_t)t * d.U + u] = v;
+        else if (t < Tb && u < Ub) lnS[plane_row(d, b, u) + t + u] = v;
       }
     }
 }
@@ -467,7 +472,7 @@ template <typename TIO>
 static int lse_stream_any(const TIO* E, float* mE, const float* mP, float* LN,
                           const void* scratch, const int* inLen, const int* labLen,
                           const Dims& d, hipStream_t s, const int* labels, float* elS,
-                          float* eb) {
+                          float* eb, float* lnS) {
   const int nub = y_ublocks(d), nks = y_steps(d);
   const int ttiles = (d.T + kRows - 1) / kRows, utiles = (d.U + 127) / 128;
   const long total = (long)ttiles * utiles * d.B;
@@ -475,24 +480,27 @@ static int lse_stream_any(const TIO* E, float* mE, const float* mP, float* LN,
   constexpr int kWaves = 4;
   hipLaunchKernelGGL((lse_stream_kernel<kWaves, TIO>), dim3(grid), dim3(64 * kWaves), 0, s, E, mE, mP,
                      static_cast<const uint4*>(scratch), LN, inLen, labLen, d, ttiles, utiles,
-                     (int)total, nub, nks, labels, elS, eb);
+                     (int)total, nub, nks, labels, elS, eb, lnS);
   RNNT_LAUNCH_CHECK("lse_stream_kernel");
   return kOk;
 }
 int launch_lse_stream(const float* E, float* mE, const float* mP, float* LN,
                       const void* scratch, const int* inLen, const int* labLen, const Dims& d,
-                      hipStream_t s, const int* labels, float* elS, float* eb) {
-  return lse_stream_any(E, mE, mP, LN, scratch, inLen, labLen, d, s, labels, elS, eb);
+                      hipStream_t s, const int* labels, float* elS, float* eb,
+                      float* lnS) {
+  return lse_stream_any(E, mE, mP, LN, scratch, inLen, labLen, d, s, labels, elS, eb, lnS);
 }
 int launch_lse_stream(const bf16_t* E, float* mE, const float* mP, float* LN,
                       const void* scratch, const int* inLen, const int* labLen, const Dims& d,
-                      hipStream_t s, const int* labels, float* elS, float* eb) {
-  return lse_stream_any(E, mE, mP, LN, scratch, inLen, labLen, d, s, labels, elS, eb);
+                      hipStream_t s, const int* labels, float* elS, float* eb,
+                      float* lnS) {
+  return lse_stream_any(E, mE, mP, LN, scratch, inLen, labLen, d, s, labels, elS, eb, lnS);
 }
 int launch_lse_stream(const f16_t* E, float* mE, const float* mP, float* LN,
                       const void* scratch, const int* inLen, const int* labLen, const Dims& d,
-                      hipStream_t s, const int* labels, float* elS, float* eb) {
-  return lse_stream_any(E, mE, mP, LN, scratch, inLen, labLen, d, s, labels, elS, eb);
+                      hipStream_t s, const int* labels, float* elS, float* eb,
+                      float* lnS) {
+  return lse_stream_any(E, mE, mP, LN, scratch, inLen, labLen, d, s, labels, elS, eb, lnS);
 }
 
 }  // namespace rnnt
