@@ -300,14 +300,13 @@ int lowp_loss_backward(const TIO* E, const TIO* P, const int* labels, const int*
   loss_workspace_layout(d, workspace, &w);
   RNNT_STAGE(kWeights, launch_weights(w.planes, inLen, labLen, d, s));
   RNNT_STAGE(kBeta, launch_beta(w.planes, labels, inLen, labLen, d, s));
-  RNNT_STAGE(kWplanes, launch_wplanes_skewed(w.planes.dS, w.planes.lnS, w.mE, w.mP, w.Wn, w.Wt,
-                                             inLen, labLen, d, s));
   // Both gradients are rounded once, from the complete fp32 value: the blank / label terms are
   // always folded into the dense kernels' write-outs here, whatever the vocabulary.  With
   // U == 1 there are no labels; the kernels then never read the list, but its pointer is what
   // switches the folding on, so any valid device pointer serves.
   const int* lab = labels ? labels : inLen;
-  RNNT_STAGE(kSparse, launch_blank_sums(w.planes, w.bsum, lab, inLen, labLen, d, s));
+  RNNT_STAGE(kWplanes, launch_post_beta(w.planes, w.mE, w.mP, w.Wn, w.Wt, w.bsum, lab, inLen,
+                                        labLen, d, s));
   SparseTerms sp;
   sp.dS = w.planes.dS; sp.wE = w.planes.wE; sp.bsum = w.bsum; sp.labels = lab;
   SparsePTerms spp;
@@ -553,8 +552,7 @@ int rnnt_hip_loss_backward(const float* E, const float* P, const int* labels, co
   loss_workspace_layout(d, workspace, &w);
   RNNT_STAGE(kWeights, launch_weights(w.planes, inLen, labLen, d, s));
   RNNT_STAGE(kBeta, launch_beta(w.planes, labels, inLen, labLen, d, s));
-  RNNT_STAGE(kWplanes, launch_wplanes_skewed(w.planes.dS, w.planes.lnS, w.mE, w.mP, w.Wn, w.Wt,
-                                             inLen, labLen, d, s));
+
   // The blank/label terms of egrads are folded into the dense kernel's write-out (a scatter
   // afterwards would touch one cache line of the 2.5 GB array per lattice cell); for label axes
   // too long for that kernel they are scattered as in rnnt_hip_backward.
@@ -562,11 +560,10 @@ int rnnt_hip_loss_backward(const float* E, const float* P, const int* labels, co
   // their terms queue up in the dense kernel -- B=8 V=100: 0.17 ms folded, 0.03 + 0.04 ms
   // scattered; from V=1000 on folding is level or ahead)
   const bool fold = egrads_fusion_supported(d) && labels != nullptr && d.V >= 512;
+  RNNT_STAGE(kWplanes, launch_post_beta(w.planes, w.mE, w.mP, w.Wn, w.Wt,
+                                        fold ? w.bsum : nullptr, labels, inLen, labLen, d, s));
   SparseTerms sp;
-  if (fold) {
-    RNNT_STAGE(kSparse, launch_blank_sums(w.planes, w.bsum, labels, inLen, labLen, d, s));
-    sp.dS = w.planes.dS; sp.wE = w.planes.wE; sp.bsum = w.bsum; sp.labels = labels;
-  }
+  if (fold) { sp.dS = w.planes.dS; sp.wE = w.planes.wE; sp.bsum = w.bsum; sp.labels = labels; }
   RNNT_STAGE(kEgrads, launch_egrads(E, P, w.mE, w.mP, w.Wn, deltas, egrads, inLen, labLen, d, false,
                                     sp, s));
   // pgrads always takes its blank / label totals in its write-out (the same two fp32 operations

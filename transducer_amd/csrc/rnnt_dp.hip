@@ -586,12 +586,12 @@ __global__ __launch_bounds__(64) void sparse_e_rows_kernel(Planes p, float* __re
 // (transducer/transducer_cpu.cpp:96,106,138 and the label moves whose label is the blank): the
 // value sparse_e_kernel would leave in that column.  Used when the label-column terms are folded
 // into the dense egrads kernel instead of being scattered afterwards.
-__global__ __launch_bounds__(256) void blank_sums_kernel(Planes p, float* __restrict__ bsum,
-                                                         const int* __restrict__ labels,
-                                                         const int* __restrict__ inLen,
-                                                         const int* __restrict__ labLen, Dims d) {
-  const int b = blockIdx.y;
-  const int t = blockIdx.x * 256 + threadIdx.x;
+__device__ __forceinline__ void blank_sums_block(const Planes& p, float* __restrict__ bsum,
+                                                 const int* __restrict__ labels,
+                                                 const int* __restrict__ inLen,
+                                                 const int* __restrict__ labLen, const Dims& d,
+                                                 int bx, int b) {
+  const int t = bx * 256 + threadIdx.x;
   int Tb, Ub;
   utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
   if (Ub == 0 || t >= Tb) return;
@@ -628,6 +628,63 @@ __global__ __launch_bounds__(256) void blank_sums_kernel(Planes p, float* __rest
     if (u + 1 < Ub && lab[u] == d.blank) acc -= dS[o + d.Dp + 1] * wE[o];
   }
   bsum[(size_t)b * d.T + t] = acc;
+}
+
+// The same from the skewed planes the lattice kernels leave behind (dalpha and LN stored
+// [u][t+u]): no un-skewed copy of dalpha is needed first.  Same arithmetic, same bits.
+__device__ __forceinline__ void wplanes_skewed_block(
+    const float* __restrict__ dS, const float* __restrict__ lnS, const float* __restrict__ mE,
+    const float* __restrict__ mP, float* __restrict__ Wn, float* __restrict__ Wt,
+    const int* __restrict__ inLen, const int* __restrict__ labLen, const Dims& d, int Up, int Tw,
+    float (*tile)[65], int bx, int by, int b) {
+  const int t0 = bx * 64, u0 = by * 64;
+  int Tb, Ub;
+  utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int u = u0 + ty + 4 * i, t = t0 + tx;
+    float w = 0.0f;
+    if (t < Tb && u < Ub) {
+      const size_t o = plane_row(d, b, u) + t + u;
+      w = dS[o] * expf((mE[(size_t)b * d.T + t] + mP[(size_t)b * d.U + u]) - lnS[o]);
+    }
+    tile[ty + 4 * i][tx] = w;
+    if (t < Tw && u < Up) Wt[((size_t)b * Up + u) * Tw + t] = w;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int t = t0 + ty + 4 * i, u = u0 + tx;
+    if (t < Tw && u < Up) Wn[((size_t)b * Tw + t) * Up + u] = tile[tx][ty + 4 * i];
+  }
+}
+
+
+// W planes and per-frame blank totals in one launch: both only need the finished dalpha plane and
+// neither needs the other, so the blocks of the second fill the device beside the first's
+// instead of waiting behind a kernel boundary.  Blocks [0, nw) form W (tile bx, by of utterance
+// b), the rest the blank totals (bsum == nullptr: none).
+__global__ __launch_bounds__(256) void post_beta_kernel(Planes p, const float* __restrict__ mE,
+                                                        const float* __restrict__ mP,
+                                                        float* __restrict__ Wn,
+                                                        float* __restrict__ Wt,
+                                                        float* __restrict__ bsum,
+                                                        const int* __restrict__ labels,
+                                                        const int* __restrict__ inLen,
+                                                        const int* __restrict__ labLen, Dims d,
+                                                        int Up, int Tw, int wx, int wy, int nw,
+                                                        int sx) {
+  __shared__ float tile[64][65];
+  const int n = blockIdx.x;
+  if (n < nw) {
+    const int b = n / (wx * wy), r = n - b * (wx * wy);
+    wplanes_skewed_block(p.dS, p.lnS, mE, mP, Wn, Wt, inLen, labLen, d, Up, Tw, tile, r % wx,
+                         r / wx, b);
+  } else {
+    const int m = n - nw;
+    blank_sums_block(p, bsum, labels, inLen, labLen, d, m % sx, m / sx);
+  }
 }
 
 __global__ __launch_bounds__(256) void sparse_p_kernel(Planes p, float* __restrict__ pgrads,
@@ -1164,12 +1221,16 @@ int launch_sparse(const Planes& p, float* egrads, float* pgrads, const int* labe
   return kOk;
 }
 
-int launch_blank_sums(const Planes& p, float* bsum, const int* labels, const int* inLen,
-                      const int* labLen, const Dims& d, hipStream_t s) {
+int launch_post_beta(const Planes& p, const float* mE, const float* mP, float* Wn, float* Wt,
+                     float* bsum, const int* labels, const int* inLen, const int* labLen,
+                     const Dims& d, hipStream_t s) {
   if (d.B == 0 || d.T == 0 || d.U == 0) return kOk;
-  hipLaunchKernelGGL(blank_sums_kernel, dim3((d.T + 255) / 256, d.B), dim3(256), 0, s, p, bsum,
-                     labels, inLen, labLen, d);
-  RNNT_LAUNCH_CHECK("blank_sums_kernel");
+  const int Up = wplane_up(d.U), Tw = wplane_tw(d.T);
+  const int wx = Tw / 64, wy = (Up + 63) / 64, nw = wx * wy * d.B;
+  const int sx = (d.T + 255) / 256, ns = bsum ? sx * d.B : 0;
+  hipLaunchKernelGGL(post_beta_kernel, dim3(nw + ns), dim3(256), 0, s, p, mE, mP, Wn, Wt, bsum,
+                     labels, inLen, labLen, d, Up, Tw, wx, wy, nw, sx);
+  RNNT_LAUNCH_CHECK("post_beta_kernel");
   return kOk;
 }
 

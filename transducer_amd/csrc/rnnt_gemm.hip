@@ -356,41 +356,6 @@ __global__ __launch_bounds__(256) void wplanes_kernel(const float* __restrict__ 
   }
 }
 
-// The same from the skewed planes the lattice kernels leave behind (dalpha and LN stored
-// [u][t+u]): no un-skewed copy of dalpha is needed first.  Same arithmetic, same bits.
-__global__ __launch_bounds__(256) void wplanes_skewed_kernel(const float* __restrict__ dS,
-                                                             const float* __restrict__ lnS,
-                                                             const float* __restrict__ mE,
-                                                             const float* __restrict__ mP,
-                                                             float* __restrict__ Wn,
-                                                             float* __restrict__ Wt,
-                                                             const int* __restrict__ inLen,
-                                                             const int* __restrict__ labLen,
-                                                             Dims d, int Up, int Tw) {
-  __shared__ float tile[64][65];
-  const int b = blockIdx.z, t0 = blockIdx.x * 64, u0 = blockIdx.y * 64;
-  int Tb, Ub;
-  utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
-  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
-#pragma unroll
-  for (int i = 0; i < 16; ++i) {
-    const int u = u0 + ty + 4 * i, t = t0 + tx;
-    float w = 0.0f;
-    if (t < Tb && u < Ub) {
-      const size_t o = plane_row(d, b, u) + t + u;
-      w = dS[o] * expf((mE[(size_t)b * d.T + t] + mP[(size_t)b * d.U + u]) - lnS[o]);
-    }
-    tile[ty + 4 * i][tx] = w;
-    if (t < Tw && u < Up) Wt[((size_t)b * Up + u) * Tw + t] = w;
-  }
-  __syncthreads();
-#pragma unroll
-  for (int i = 0; i < 16; ++i) {
-    const int t = t0 + ty + 4 * i, u = u0 + tx;
-    if (t < Tw && u < Up) Wn[((size_t)b * Tw + t) * Up + u] = tile[tx][ty + 4 * i];
-  }
-}
-
 // ------------------------------------------------------------------ shared tile code
 // "A rows k-contiguous, B rows n-contiguous": As[m][k] pitch KP (16-byte reads, four k per
 // lane), Bs[k][n] pitch NP (4-byte reads, 32 consecutive n per half-wave).
@@ -564,17 +529,6 @@ int launch_wplanes(const float* lngrads, const float* LN, const float* mE, const
   hipLaunchKernelGGL(wplanes_kernel, dim3(Tw / 64, (Up + 63) / 64, d.B), dim3(256), 0, s, lngrads,
                      LN, mE, mP, Wn, Wt, inLen, labLen, d, Up, Tw);
   RNNT_LAUNCH_CHECK("wplanes_kernel");
-  return kOk;
-}
-
-int launch_wplanes_skewed(const float* dS, const float* lnS, const float* mE, const float* mP,
-                          float* Wn, float* Wt, const int* inLen, const int* labLen,
-                          const Dims& d, hipStream_t s) {
-  if (d.B == 0 || d.T == 0 || d.U == 0) return kOk;
-  const int Up = wplane_up(d.U), Tw = wplane_tw(d.T);
-  hipLaunchKernelGGL(wplanes_skewed_kernel, dim3(Tw / 64, (Up + 63) / 64, d.B), dim3(256), 0, s,
-                     dS, lnS, mE, mP, Wn, Wt, inLen, labLen, d, Up, Tw);
-  RNNT_LAUNCH_CHECK("wplanes_skewed_kernel");
   return kOk;
 }
 

@@ -118,9 +118,12 @@ int launch_beta(const Planes& p, const int* labels, const int* inLen, const int*
 int launch_sparse(const Planes& p, float* egrads, float* pgrads, const int* labels,
                   const int* inLen, const int* labLen, const float* scale, bool add,
                   const Dims& d, hipStream_t s);
-// bsum[b,t] = what the sparse terms leave in egrads[b,t,blank] (see blank_sums_kernel).
-int launch_blank_sums(const Planes& p, float* bsum, const int* labels, const int* inLen,
-                      const int* labLen, const Dims& d, hipStream_t s);
+// After the dalpha walk, in one launch: the W planes (both orientations, from the skewed dalpha
+// and LN planes) and, with bsum != nullptr, bsum[b,t] = what the blank/label terms leave in
+// egrads[b,t,blank] (for folding into the dense kernel's write-out).
+int launch_post_beta(const Planes& p, const float* mE, const float* mP, float* Wn, float* Wt,
+                     float* bsum, const int* labels, const int* inLen, const int* labLen,
+                     const Dims& d, hipStream_t s);
 // best / arg: skewed planes ([B][Ua][Dp], see plane_row), written for valid cells only.
 int launch_maxplus(const float* E, const float* P, const int* inLen, const int* labLen,
                    float* best, int* arg, const Dims& d, hipStream_t s);
@@ -194,10 +197,6 @@ int launch_rowmax_pick_p(const f16_t* P, float* mP, const int* labels, const int
 int launch_wplanes(const float* lngrads, const float* LN, const float* mE, const float* mP,
                    float* Wn, float* Wt, const int* inLen, const int* labLen, const Dims& d,
                    hipStream_t s);
-// The same from the skewed dalpha and LN planes of the lattice kernels.
-int launch_wplanes_skewed(const float* dS, const float* lnS, const float* mE, const float* mP,
-                          float* Wn, float* Wt, const int* inLen, const int* labLen,
-                          const Dims& d, hipStream_t s);
 // Sparse blank/label terms of egrads for folding into the dense kernel's write-out: with
 // labels != nullptr, out = delta * (dense + sparse) (needs accumulate == false and a label axis
 // short enough for the streaming kernel, see egrads_fusion_supported).
