@@ -38,7 +38,7 @@ PEAK_HBM_GBS = 8000.0
 # HBM bytes per launch (fetched + written) from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this
 # file, scaled by what the counters read for a plain copy of known size
 # (profiles/cfg4_hbm_traffic_counters.md).  Recorded, not measured live: counters need rocprofv3.
-RECORDED_TRAFFIC_BYTES = {"cfg4": {"lse": 2.533e9, "egrads": 5.668e9, "pgrads": 3.125e9}}
+RECORDED_TRAFFIC_BYTES = {"cfg4": {"lse": 2.546e9, "egrads": 5.633e9, "pgrads": 3.129e9}}
 
 WORKLOADS = {
     # BASELINE configs[3]: the shape the metric is quoted on
