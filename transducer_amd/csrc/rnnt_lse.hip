@@ -75,6 +75,7 @@ __global__ __launch_bounds__(256) void yplanes_kernel(const TIO* __restrict__ P,
   const int lane = threadIdx.x & 63, l32 = lane & 31, h = lane >> 5;
   int Ub = d.U;
   if (labLen) Ub = min(max(labLen[b], 0) + 1, d.U);
+  if (32 * ub >= Ub) return;  // a block of rows past the utterance is never read
   const int u = 32 * ub + l32, v0 = 16 * ks + 8 * h;
   float y[8];
 #pragma unroll
