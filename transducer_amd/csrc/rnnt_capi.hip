@@ -193,6 +193,28 @@ __global__ void fill_kernel(float* x, float v, int n) {
   if (i < n) x[i] = v;
 }
 
+// Zero fill by a kernel (the whole-loss entry points enqueue kernels only, so that a caller
+// may capture them into a graph; this is their degenerate T == 0 / U == 0 case).
+__global__ void zero_bytes_kernel(unsigned char* x, size_t n) {
+  const size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 16;
+  if (i + 16 <= n) {
+    if ((reinterpret_cast<uintptr_t>(x) & 15) == 0) {
+      *reinterpret_cast<uint4*>(x + i) = make_uint4(0, 0, 0, 0);
+      return;
+    }
+  }
+  for (size_t k = i; k < n && k < i + 16; ++k) x[k] = 0;
+}
+
+int zero_fill(void* x, size_t bytes, hipStream_t s) {
+  if (x == nullptr || bytes == 0) return kOk;
+  const size_t blocks = (bytes + 4095) / 4096;
+  if (blocks > 0x7fffffffu) return fail(kInvalid, "array too large to clear");
+  hipLaunchKernelGGL(zero_bytes_kernel, dim3((unsigned)blocks), dim3(256), 0, s,
+                     static_cast<unsigned char*>(x), bytes);
+  return check_hip(hipGetLastError(), "launch zero_bytes_kernel", __FILE__, __LINE__);
+}
+
 int fill(float* x, float v, int n, hipStream_t s) {
   if (n == 0) return kOk;
   hipLaunchKernelGGL(fill_kernel, dim3((n + 255) / 256), dim3(256), 0, s, x, v, n);
@@ -279,10 +301,8 @@ int lowp_loss_backward(const TIO* E, const TIO* P, const int* labels, const int*
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (B == 0 || V == 0) return kOk;
   if (nothing_to_do(B, T, U)) {
-    if (egrads && (size_t)T * V)
-      RNNT_HIP(hipMemsetAsync(egrads, 0, sizeof(TIO) * (size_t)B * T * V, s));
-    if (pgrads && (size_t)U * V)
-      RNNT_HIP(hipMemsetAsync(pgrads, 0, sizeof(TIO) * (size_t)B * U * V, s));
+    RNNT_TRY(zero_fill(egrads, sizeof(TIO) * (size_t)B * T * V, s));
+    RNNT_TRY(zero_fill(pgrads, sizeof(TIO) * (size_t)B * U * V, s));
     return kOk;
   }
   if (!E || !P || !egrads || !pgrads || !inLen || !labLen || (U > 1 && !labels))
@@ -536,8 +556,8 @@ int rnnt_hip_loss_backward(const float* E, const float* P, const int* labels, co
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (B == 0 || V == 0) return kOk;
   if (nothing_to_do(B, T, U)) {
-    if (egrads && (size_t)T * V) RNNT_HIP(hipMemsetAsync(egrads, 0, sizeof(float) * (size_t)B * T * V, s));
-    if (pgrads && (size_t)U * V) RNNT_HIP(hipMemsetAsync(pgrads, 0, sizeof(float) * (size_t)B * U * V, s));
+    RNNT_TRY(zero_fill(egrads, sizeof(float) * (size_t)B * T * V, s));
+    RNNT_TRY(zero_fill(pgrads, sizeof(float) * (size_t)B * U * V, s));
     return kOk;
   }
   if (!E || !P || !egrads || !pgrads || !inLen || !labLen || (U > 1 && !labels))
