@@ -156,8 +156,8 @@ def test_backward_twice_on_one_forward_gives_the_same_gradients():
     assert torch.equal(E.grad, e1) and torch.equal(P.grad, p1)
 
 
-def _small_problem(seed=23):
-    d = make_inputs(small_config(3, 150, 20, 260, ragged=True), seed=seed)
+def _small_problem(seed=23, shape=(3, 150, 20, 260)):
+    d = make_inputs(small_config(*shape, ragged=True), seed=seed)
     dev = torch.device("cuda")
     return (torch.tensor(d["emissions"], device=dev), torch.tensor(d["predictions"], device=dev),
             torch.tensor(d["labels"], device=dev), torch.tensor(d["input_lengths"], device=dev),
@@ -186,13 +186,16 @@ def test_loss_on_a_side_stream_matches_the_default_stream():
     assert torch.equal(paths[written], again[written])
 
 
-def test_fused_entry_points_replay_from_a_captured_graph():
+# the second shape has 19 slabs of frames on few tiles: the prediction-gradient walk splits over
+# frames there, and its arrival counters must be cleared again inside every replay
+@pytest.mark.parametrize("shape", [(3, 150, 20, 260), (2, 600, 20, 1024)])
+def test_fused_entry_points_replay_from_a_captured_graph(shape):
     """rnnt_hip_loss_forward / rnnt_hip_loss_backward allocate nothing and use kernels only, so
     a caller may capture them; every replay (with eager work and synchronisation in between)
     must reproduce the eager result bit for bit."""
     import ctypes
     from transducer_amd import capi
-    E, P, labels, il, ll = _small_problem(seed=29)
+    E, P, labels, il, ll = _small_problem(seed=29, shape=shape)
     B, T, V = E.shape
     U = P.shape[1]
     p = lambda t: ctypes.c_void_p(t.data_ptr())
@@ -214,7 +217,7 @@ def test_fused_entry_points_replay_from_a_captured_graph():
         run(ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
     for _ in range(3):
         costs.fill_(float("nan")); eg.fill_(float("nan")); pg.fill_(float("nan"))
-        ws.zero_()
+        ws.fill_(0xff)  # the calls may assume nothing about the workspace's contents
         torch.cuda.synchronize()
         graph.replay()
         torch.cuda.synchronize()
