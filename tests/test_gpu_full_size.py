@@ -190,3 +190,40 @@ def test_configuration_whole_against_the_oracle(name):
     assert ve <= max(2 * floor_e, 0.02) and vp <= max(2 * floor_p, 0.02)
     for i in range(E.shape[0]):
         assert not eg[i, il[i]:].any() and not pg[i, ll[i] + 1:].any()
+
+
+# ------------------------------------------------------------------ more than 2^31 score elements
+def test_arrays_past_two_to_the_31_elements_index_like_small_ones():
+    """B*T*V = 2.3e9 elements (9.2 GB of emissions): element offsets no longer fit 32 bits.  The
+    last utterances lie wholly past that point, and an utterance's result does not depend on the
+    batch around it, so each must come out with the bits it has as a batch of one (whose offsets
+    are small); the size-free properties hold over the whole batch."""
+    from transducer_amd.synthetic import small_config
+    cfg = small_config(24, 2000, 30, 48000, ragged=True)
+    c = DeviceBatch(cfg, seed=11)
+    B, T, U, V = c.dims
+    assert B * T * V > 2 ** 31 and (B - 1) * T * V > 2 ** 31
+    costs, eg, pg = loss_on_device(c)
+    assert torch.isfinite(costs).all() and (costs > 0).all()
+    tmask = torch.arange(T, device="cuda:0")[None, :] >= c.il[:, None]
+    umask = torch.arange(U, device="cuda:0")[None, :] > c.ll[:, None]
+    assert not eg[tmask].any() and not pg[umask].any()
+    se = eg.sum(-1, dtype=torch.float64).abs()
+    ae = eg.abs().sum(-1, dtype=torch.float64)
+    assert torch.isfinite(se).all()
+    assert float(ae[~tmask].min()) > 1e-3
+    assert bool((se <= 1e-5 + 2e-5 * ae).all())
+    for b in (0, B - 2, B - 1):
+        one = c.cut(b)
+        c1, e1, p1 = loss_on_device(one)
+        assert torch.equal(c1[0], costs[b]), b
+        assert torch.equal(e1[0], eg[b]) and torch.equal(p1[0], pg[b]), b
+    del eg, pg
+
+    LN = log_norms_on_device(c)
+    paths = viterbi_on_device(c, LN)
+    for b in (0, B - 1):
+        one = c.cut(b)
+        alone = viterbi_on_device(one, LN[b:b + 1].contiguous())
+        n = int(c.ll_h[b])
+        assert torch.equal(alone[0, :n], paths[b, :n]), b
