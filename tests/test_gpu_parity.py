@@ -293,7 +293,11 @@ def test_log_norms_wide_dynamic_range():
 
 
 # ------------------------------------------------------------------ dense gradient kernels
-@pytest.mark.parametrize("B,T,U,V", [(2, 50, 11, 32), (2, 130, 101, 333), (1, 300, 140, 64)])
+# (U counts the rows of predictions; 113, 224, 225 sit on the edges of the 112-position slices
+# the egrads kernel contracts per launch)
+@pytest.mark.parametrize("B,T,U,V", [(2, 50, 11, 32), (2, 130, 101, 333), (1, 300, 140, 64),
+                                     (2, 40, 113, 128), (2, 36, 224, 516), (3, 36, 225, 64),
+                                     (2, 20, 470, 40)])
 def test_dense_grads_against_oracle(B, T, U, V):
     cfg = small_config(B, T, U - 1, V, ragged=True)
     E, P, labels, il, ll = unpack(make_inputs(cfg, seed=T))
@@ -328,16 +332,21 @@ def test_whole_loss_cfg1(cfg, seed):
         assert_close(pg, f["pgrads"], what="pgrads vs reference fixture")
 
 
-@pytest.mark.parametrize("T,U,V", [(60, 150, 36), (60, 150, 37), (40, 260, 16), (33, 113, 520)])
-def test_whole_loss_with_a_label_axis_past_the_streaming_kernels(T, U, V):
-    """More than 112 label positions: egrads falls back to the general kernel (slice by slice
-    over the label axis) and the blank/label terms are scattered; odd V also takes the general
-    log-normaliser.  Same entry points, same bar."""
+@pytest.mark.parametrize("T,U,V", [(60, 150, 36), (60, 150, 37), (40, 260, 16), (33, 113, 520),
+                                   (40, 111, 520), (40, 112, 520), (36, 223, 516), (36, 224, 1028),
+                                   (20, 500, 64)])
+def test_whole_loss_with_a_label_axis_longer_than_one_slice(T, U, V):
+    """egrads contracts 112 label positions per launch; a longer axis goes slice by slice, the
+    later slices adding to what is in egrads and only the last one applying the upstream factors
+    (so U + 1 = 112, 113, 224, 225 sit on the slice edges).  With V >= 512 the blank/label terms
+    ride in the first slice's write-out, below that they are scattered; odd V also takes the
+    general log-normaliser.  Same entry points, same bar."""
     cfg = small_config(2, T, U, V, ragged=True)
     E, P, labels, il, ll = unpack(make_inputs(cfg, seed=T + U + V))
-    want = oracle.loss_and_grads(E, P, labels, il, ll, lse="naive")
-    other = oracle.loss_and_grads(E, P, labels, il, ll, lse="sep")
-    costs, eg, pg = gpu_loss(DeviceCase(E, P, labels, il, ll))
+    deltas = np.array([0.5, 3.0], np.float32)
+    want = oracle.loss_and_grads(E, P, labels, il, ll, lse="naive", deltas=deltas)
+    other = oracle.loss_and_grads(E, P, labels, il, ll, lse="sep", deltas=deltas)
+    costs, eg, pg = gpu_loss(DeviceCase(E, P, labels, il, ll), deltas=deltas)
     assert_close(costs, want["costs"], what="costs")
     # a lattice this long along the label axis moves by more than the tolerance when LN moves in
     # its last bits: the bar is the oracle's own spread between its two summation orders of LN

@@ -257,7 +257,7 @@ int check_lowp_shape(const void* E, const void* P, const Dims& d, bool loss, con
                 who, d.V);
   if ((reinterpret_cast<uintptr_t>(E) | reinterpret_cast<uintptr_t>(P)) & 15)
     return fail(kInvalid, "%s: 16-bit scores must be 16-byte aligned", who);
-  if (loss && !egrads_stream_supported(d))
+  if (loss && !egrads_one_pass(d))
     return fail(kInvalid, "%s: 16-bit scores take at most 112 label positions (U=%d)", who, d.U);
   return kOk;
 }
@@ -574,12 +574,11 @@ int rnnt_hip_loss_backward(const float* E, const float* P, const int* labels, co
   RNNT_STAGE(kBeta, launch_beta(w.planes, labels, inLen, labLen, d, s));
 
   // The blank/label terms of egrads are folded into the dense kernel's write-out (a scatter
-  // afterwards would touch one cache line of the 2.5 GB array per lattice cell); for label axes
-  // too long for that kernel they are scattered as in rnnt_hip_backward.
+  // afterwards would touch one cache line of the 2.5 GB array per lattice cell).
   // (not with a small vocabulary: many labels then fall into one wavefront's 32 columns and
   // their terms queue up in the dense kernel -- B=8 V=100: 0.17 ms folded, 0.03 + 0.04 ms
   // scattered; from V=1000 on folding is level or ahead)
-  const bool fold = egrads_fusion_supported(d) && labels != nullptr && d.V >= 512;
+  const bool fold = labels != nullptr && d.V >= 512;
   RNNT_STAGE(kWplanes, launch_post_beta(w.planes, w.mE, w.mP, w.Wn, w.Wt,
                                         fold ? w.bsum : nullptr, labels, inLen, labLen, d, s));
   SparseTerms sp;

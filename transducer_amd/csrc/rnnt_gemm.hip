@@ -356,89 +356,6 @@ __global__ __launch_bounds__(256) void wplanes_kernel(const float* __restrict__ 
   }
 }
 
-// ------------------------------------------------------------------ shared tile code
-// "A rows k-contiguous, B rows n-contiguous": As[m][k] pitch KP (16-byte reads, four k per
-// lane), Bs[k][n] pitch NP (4-byte reads, 32 consecutive n per half-wave).
-template <int KP, int NP>
-__device__ inline void mma_group(const float* As, const float* Bs, int arow, int bcol, int kbase,
-                                 int h, floatx16& acc) {
-  const float4 a4 = *reinterpret_cast<const float4*>(&As[arow * KP + kbase + 4 * h]);
-  const float b0 = Bs[(kbase + 4 * h + 0) * NP + bcol];
-  const float b1 = Bs[(kbase + 4 * h + 1) * NP + bcol];
-  const float b2 = Bs[(kbase + 4 * h + 2) * NP + bcol];
-  const float b3 = Bs[(kbase + 4 * h + 3) * NP + bcol];
-  acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a4.x, b0, acc, 0, 0, 0);
-  acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a4.y, b1, acc, 0, 0, 0);
-  acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a4.z, b2, acc, 0, 0, 0);
-  acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a4.w, b3, acc, 0, 0, 0);
-}
-
-// ------------------------------------------------------------------ egrads, any label length
-// Fallback for label axes too long for the register-resident form in rnnt_grads.hip.
-// Block tile 64 (t) x 64 (v); a slice of the reduction over u (<= kEgMaxK) sits in LDS at once.
-constexpr int kEgMaxK = 112, kEgKP = kEgMaxK + 4, kEgNP = 64 + 4;
-
-__global__ __launch_bounds__(256, 2) void egrads_kernel(
-    const float* __restrict__ E, const float* __restrict__ P, const float* __restrict__ mE,
-    const float* __restrict__ mP, const float* __restrict__ Wn, const float* __restrict__ deltas,
-    float* __restrict__ egrads, const int* __restrict__ inLen, const int* __restrict__ labLen,
-    Dims d, int Up, int Tw, int kofs, int accumulate, int last) {
-  __shared__ __attribute__((aligned(16))) float As[64 * kEgKP];
-  __shared__ __attribute__((aligned(16))) float Bs[kEgMaxK * kEgNP];
-  const int b = blockIdx.z, v0 = blockIdx.x * 64, t0 = blockIdx.y * 64;
-  int Tb, Ub;
-  utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  float* out = egrads + (size_t)b * d.T * d.V;
-  if (t0 >= Tb) {  // padded frames: the dense part is exactly zero
-    const float dl = (deltas && last) ? deltas[b] : 1.0f;
-    for (int e = tid; e < 64 * 64; e += 256) {
-      const int t = t0 + e / 64, v = v0 + e % 64;
-      if (t < d.T && v < d.V) {
-        const size_t o = (size_t)t * d.V + v;
-        out[o] = accumulate ? dl * out[o] : 0.0f;
-      }
-    }
-    return;
-  }
-  const int K = min(Up - kofs, kEgMaxK);  // this launch's slice of the label axis
-  // A: W rows (t), k = u contiguous
-  for (int e = tid; e < 64 * K; e += 256) {
-    const int r = e / K, k = e % K;
-    As[r * kEgKP + k] = Wn[((size_t)b * Tw + t0 + r) * Up + kofs + k];
-  }
-  // B: exp(P[u,v] - mP[u]) rows (u), n = v contiguous
-  const float* Pb = P + (size_t)b * d.U * d.V;
-  for (int e = tid; e < K * 64; e += 256) {
-    const int k = e / 64, n = e % 64, u = kofs + k, v = v0 + n;
-    float y = 0.0f;
-    if (u < Ub && v < d.V) y = __expf(Pb[(size_t)u * d.V + v] - mP[(size_t)b * d.U + u]);
-    Bs[k * kEgNP + n] = y;
-  }
-  __syncthreads();
-  const int wm = wave >> 1, wn = wave & 1, l32 = lane & 31, h = lane >> 5;
-  floatx16 acc;
-#pragma unroll
-  for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
-  for (int k = 0; k < K; k += 8)
-    mma_group<kEgKP, kEgNP>(As, Bs, 32 * wm + l32, 32 * wn + l32, k, h, acc);
-
-  const float delta = (deltas && last) ? deltas[b] : 1.0f;
-  const float* Eb = E + (size_t)b * d.T * d.V;
-#pragma unroll
-  for (int r = 0; r < 16; ++r) {
-    const int t = t0 + 32 * wm + 8 * (r >> 2) + 4 * h + (r & 3);
-    const int v = v0 + 32 * wn + l32;
-    if (t < d.T && v < d.V) {
-      const size_t o = (size_t)t * d.V + v;
-      float g = 0.0f;
-      if (t < Tb) g = __expf(Eb[o] - mE[(size_t)b * d.T + t]) * acc[r];
-      if (accumulate) g = out[o] + g;
-      out[o] = delta * g;
-    }
-  }
-}
-
 }  // namespace
 
 #define RNNT_LAUNCH_CHECK(name)                                                    \
@@ -532,26 +449,13 @@ int launch_wplanes(const float* lngrads, const float* LN, const float* mE, const
   return kOk;
 }
 
-bool egrads_fusion_supported(const Dims& d) { return egrads_stream_supported(d); }
-
 int launch_egrads(const float* E, const float* P, const float* mE, const float* mP,
                   const float* Wn, const float* deltas, float* egrads, const int* inLen,
                   const int* labLen, const Dims& d, bool accumulate, const SparseTerms& sparse,
                   hipStream_t s) {
   if (d.B == 0 || d.T == 0 || d.U == 0) return kOk;
-  if (egrads_stream_supported(d))
-    return launch_egrads_stream(E, P, mE, mP, Wn, deltas, egrads, inLen, labLen, d, accumulate,
-                                sparse, s);
-  if (sparse.labels) return fail(kInvalid, "sparse-term folding needs the streaming egrads kernel");
-  const int Up = wplane_up(d.U), Tw = wplane_tw(d.T);
-  // label axes longer than one LDS slice are contracted slice by slice, accumulating
-  for (int kofs = 0; kofs < Up; kofs += kEgMaxK) {
-    hipLaunchKernelGGL(egrads_kernel, dim3((d.V + 63) / 64, (d.T + 63) / 64, d.B), dim3(256), 0, s,
-                       E, P, mE, mP, Wn, deltas, egrads, inLen, labLen, d, Up, Tw, kofs,
-                       (accumulate || kofs > 0) ? 1 : 0, kofs + kEgMaxK >= Up ? 1 : 0);
-    RNNT_LAUNCH_CHECK("egrads_kernel");
-  }
-  return kOk;
+  return launch_egrads_stream(E, P, mE, mP, Wn, deltas, egrads, inLen, labLen, d, accumulate,
+                              sparse, s);
 }
 
 int launch_pgrads(const float* E, const float* P, const float* mE, const float* mP,

@@ -39,6 +39,7 @@ constexpr int kEsPitch = 16 * kEsMaxS + 8;  // LDS row pitch of a W-slab plane i
                                             // 16-byte reads of 8 consecutive rows spread over all banks)
 constexpr int kEsPlane = 32 * kEsPitch;
 constexpr int kEsPrefetch = 2;          // labels per 32-column block whose sparse terms are prefetched
+constexpr int kMaxLabels = 1024;        // longest label axis the lattice kernels take
 
 // Row of the 32x32 output block that register r of lane-half h holds.
 __device__ inline int mfma_row(int r, int h) { return 8 * (r >> 2) + 4 * h + (r & 3); }
@@ -65,7 +66,7 @@ __device__ __forceinline__ void egrads_walk(
     const TIO* __restrict__ E, const TIO* __restrict__ P, const float* __restrict__ mE,
     const float* __restrict__ mP, const float* __restrict__ Wn, const float* __restrict__ deltas,
     TIO* __restrict__ egrads, unsigned short (*As)[3][kEsPlane], float (*Ms)[32], const Dims& d,
-    int Up, int Tw, int tiles_per_chunk, int b, int Tb, int Ub, const SparseTerms& sp,
+    int Up, int Tw, int tiles_per_chunk, int u_lo, int b, int Tb, int Ub, const SparseTerms& sp,
     const unsigned short* match, int nmatch, float (*Sp)[32]) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, h = lane >> 5;
   const int wave_col0 = blockIdx.x * 128 + wave * 32;  // this wavefront's 32 columns
@@ -86,7 +87,7 @@ __device__ __forceinline__ void egrads_walk(
   const float* mEb = mE + (size_t)b * d.T;
 
   // Y fragments for this wavefront's columns (branch-free: clamped address, masked value):
-  // step s holds label positions 16 s + 8 h + i, split into their three bf16 pieces
+  // step s holds label positions u_lo + 16 s + 8 h + i, split into their three bf16 pieces
   Frag3 Yf[NS];
   if (tile_lo < tile_valid) {
     const TIO* Pb = P + (size_t)b * d.U * d.V;
@@ -96,7 +97,7 @@ __device__ __forceinline__ void egrads_walk(
       float y[8];
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
-        const int u = 16 * s + 8 * h + i;
+        const int u = u_lo + 16 * s + 8 * h + i;
         const bool uok = u < Ub;
         const int uc = uok ? u : 0;
         const float e = __expf(ldf(Pb + (size_t)uc * d.V + vc) - mPb[uc]);
@@ -106,17 +107,20 @@ __device__ __forceinline__ void egrads_walk(
     }
   }
 
-  // W slab staging: the 32 x Up slab of frame tile ti is one contiguous run of 8*Up float4;
-  // each is split into its three pieces on the way into LDS
-  const int up4 = Up >> 2, nvec = 8 * Up;
+  // W slab staging: columns u_lo .. u_lo + 16 NS of the 32 x Up slab of frame tile ti (all of
+  // it when the label axis fits one launch), float4 by float4, each split into its three pieces
+  // on the way into LDS
+  const int up4 = Up >> 2, lo4 = u_lo >> 2, cw4 = min(Up - u_lo, 16 * kEsMaxS) >> 2;
+  const int nvec = 32 * cw4;
   int lds_off[4], src_idx[4];
   bool vec_ok[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int idx = tid + 256 * i;
     vec_ok[i] = idx < nvec;
-    src_idx[i] = vec_ok[i] ? idx : nvec - 1;  // loads stay unconditional, stores are masked
-    lds_off[i] = vec_ok[i] ? (idx / up4) * kEsPitch + 4 * (idx % up4) : 0;
+    const int ic = vec_ok[i] ? idx : nvec - 1;  // loads stay unconditional, stores are masked
+    src_idx[i] = (ic / cw4) * up4 + lo4 + ic % cw4;
+    lds_off[i] = vec_ok[i] ? (idx / cw4) * kEsPitch + 4 * (idx % cw4) : 0;
   }
   // per-lane part of the element offset inside a tile; the per-register part is r-dependent
   // only through compile-time multiples of V
@@ -334,15 +338,18 @@ __global__ __launch_bounds__(256, 2) void egrads_stream_kernel(
     const TIO* __restrict__ E, const TIO* __restrict__ P, const float* __restrict__ mE,
     const float* __restrict__ mP, const float* __restrict__ Wn, const float* __restrict__ deltas,
     TIO* __restrict__ egrads, const int* __restrict__ inLen, const int* __restrict__ labLen,
-    Dims d, int Up, int Tw, int tiles_per_chunk, SparseTerms sp) {
+    Dims d, int Up, int Tw, int tiles_per_chunk, int u_lo, SparseTerms sp) {
   __shared__ __attribute__((aligned(16))) unsigned short As[2][3][kEsPlane];
   __shared__ __attribute__((aligned(16))) float Ms[2][32];  // mE of the slab's frames
   __shared__ __attribute__((aligned(16))) float Strip[4][32];  // per wavefront: sparse terms
-  __shared__ unsigned short Match[4][kEsMaxS * 16];  // per wavefront: label positions whose label
-                                                    // is one of its 32 columns
+  __shared__ unsigned short Match[4][kMaxLabels];  // per wavefront: label positions whose label
+                                                   // is one of its 32 columns
   const int b = blockIdx.z;
   int Tb, Ub;
   utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
+  // a later slice of the label axis that lies past this utterance adds nothing; only the last
+  // slice (the one that is given the factors) still has to scale what is there
+  if (kAccumulate && u_lo > 0 && u_lo >= Ub && deltas == nullptr) return;
   int nmatch = 0;
   if (sp.labels) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -361,11 +368,11 @@ __global__ __launch_bounds__(256, 2) void egrads_stream_kernel(
   for (int e = threadIdx.x; e < 3 * kEsPlane; e += 256)
     reinterpret_cast<unsigned*>(&As[0][0][0])[e] = 0u;
   __syncthreads();
-  const int nsteps = (Ub + 15) >> 4;
+  const int nsteps = (min(max(Ub - u_lo, 0), 16 * kEsMaxS) + 15) >> 4;
 #define RNNT_EG_WALK(NS)                                                                      \
   egrads_walk<NS, kAccumulate>(E, P, mE, mP, Wn, deltas, egrads, As, Ms, d, Up, Tw,          \
-                               tiles_per_chunk, b, Tb, Ub, sp, Match[threadIdx.x >> 6], nmatch,             \
-                               &Strip[threadIdx.x >> 6])
+                               tiles_per_chunk, u_lo, b, Tb, Ub, sp, Match[threadIdx.x >> 6], \
+                               nmatch, &Strip[threadIdx.x >> 6])
   if (nsteps <= 2) RNNT_EG_WALK(2);
   else if (nsteps <= 4) RNNT_EG_WALK(4);
   else if (nsteps == 5) RNNT_EG_WALK(5);
@@ -653,7 +660,7 @@ __global__ __launch_bounds__(256, 2) void pgrads_stream_kernel(
     if (_e != hipSuccess) return check_hip(_e, "launch " name, __FILE__, __LINE__); \
   } while (0)
 
-bool egrads_stream_supported(const Dims& d) { return wplane_up(d.U) <= 16 * kEsMaxS; }
+bool egrads_one_pass(const Dims& d) { return wplane_up(d.U) <= 16 * kEsMaxS; }
 
 template <typename TIO>
 static int egrads_stream_any(const TIO* E, const TIO* P, const float* mE, const float* mP,
@@ -672,13 +679,24 @@ static int egrads_stream_any(const TIO* E, const TIO* P, const float* mE, const 
   if (chunks > max_chunks) chunks = max_chunks;
   const int per = (ntiles + chunks - 1) / chunks;
   chunks = (ntiles + per - 1) / per;
-  if (accumulate)
-    hipLaunchKernelGGL((egrads_stream_kernel<true, TIO>), dim3(vtiles, chunks, d.B), dim3(256), 0, s, E,
-                       P, mE, mP, Wn, deltas, egrads, inLen, labLen, d, Up, Tw, per, sparse);
-  else
-    hipLaunchKernelGGL((egrads_stream_kernel<false, TIO>), dim3(vtiles, chunks, d.B), dim3(256), 0, s, E,
-                       P, mE, mP, Wn, deltas, egrads, inLen, labLen, d, Up, Tw, per, sparse);
-  RNNT_LAUNCH_CHECK("egrads_stream_kernel");
+  if (d.U > kMaxLabels) return fail(kInvalid, "egrads: more than %d label positions", kMaxLabels);
+  // A launch contracts 16 * kEsMaxS label positions (what a wavefront keeps of Y in registers);
+  // a longer label axis goes slice by slice, each later slice adding to what the earlier ones
+  // left in egrads.  Only the last slice is given the factors, and scales the whole sum.
+  const SparseTerms none;
+  for (int u_lo = 0; u_lo < Up; u_lo += 16 * kEsMaxS) {
+    const bool last = u_lo + 16 * kEsMaxS >= Up;
+    const float* dl = last ? deltas : nullptr;
+    if (accumulate || u_lo > 0)
+      hipLaunchKernelGGL((egrads_stream_kernel<true, TIO>), dim3(vtiles, chunks, d.B), dim3(256),
+                         0, s, E, P, mE, mP, Wn, dl, egrads, inLen, labLen, d, Up, Tw, per, u_lo,
+                         none);
+    else
+      hipLaunchKernelGGL((egrads_stream_kernel<false, TIO>), dim3(vtiles, chunks, d.B), dim3(256),
+                         0, s, E, P, mE, mP, Wn, dl, egrads, inLen, labLen, d, Up, Tw, per, u_lo,
+                         sparse);
+    RNNT_LAUNCH_CHECK("egrads_stream_kernel");
+  }
   return kOk;
 }
 int launch_egrads_stream(const float* E, const float* P, const float* mE, const float* mP,

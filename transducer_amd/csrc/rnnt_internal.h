@@ -198,8 +198,7 @@ int launch_wplanes(const float* lngrads, const float* LN, const float* mE, const
                    float* Wn, float* Wt, const int* inLen, const int* labLen, const Dims& d,
                    hipStream_t s);
 // Sparse blank/label terms of egrads for folding into the dense kernel's write-out: with
-// labels != nullptr, out = delta * (dense + sparse) (needs accumulate == false and a label axis
-// short enough for the streaming kernel, see egrads_fusion_supported).
+// labels != nullptr, out = delta * (dense + sparse) (needs accumulate == false).
 struct SparseTerms {
   const float* dS = nullptr;    // skewed dalpha plane
   const float* wE = nullptr;    // skewed label-move weight plane
@@ -213,7 +212,6 @@ struct SparsePTerms {
   const float* gL = nullptr;
   const int* labels = nullptr;  // [B,U-1]; may be null when U == 1
 };
-bool egrads_fusion_supported(const Dims& d);
 // accumulate == false: out = delta * dense.   accumulate == true: out = delta * (out + dense),
 // the update of transducer/torch_binding.py:86-89.
 int launch_egrads(const float* E, const float* P, const float* mE, const float* mP,
@@ -230,7 +228,9 @@ int launch_pgrads(const float* E, const float* P, const float* mE, const float* 
 
 
 // ---------------------------------------------------------------- launchers (rnnt_grads.hip)
-bool egrads_stream_supported(const Dims& d);
+// Whether one launch covers the label axis (16-bit gradients are only formed that way: a
+// second slice would round the running sum to 16 bits in between).
+bool egrads_one_pass(const Dims& d);
 int launch_egrads_stream(const float* E, const float* P, const float* mE, const float* mP,
                          const float* Wn, const float* deltas, float* egrads, const int* inLen,
                          const int* labLen, const Dims& d, bool accumulate,
