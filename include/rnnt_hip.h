@@ -109,9 +109,11 @@ int rnnt_hip_loss_backward(const float* emissions, const float* predictions, con
  * for a caller whose projection layers emit 16-bit logits, and they halve the traffic of the two
  * [B,T,V] arrays.  A score converts to fp32 exactly and all arithmetic is the fp32 path's; each
  * gradient element is the fp32 result (dense + blank/label terms, times deltas[b]) rounded once
- * to nearest-even (an fp16 gradient past 65504 becomes infinity).  Shapes: V a multiple of 8,
- * 16-byte aligned score arrays, and for the loss at most 112 label positions (U <= 112);
- * anything else is refused with an error.  Workspace as for the fp32 calls.  The best path of
+ * to nearest-even (an fp16 gradient past 65504 becomes infinity).  The loss takes at most 112
+ * label positions (U <= 112) and refuses more with an error: a longer label axis is contracted
+ * in slices whose running sum would be rounded to 16 bits in between.  Any V; 16-byte loads are
+ * used when V is a multiple of 8 and the arrays are 16-byte aligned.  Workspace as for the fp32
+ * calls.  The best path of
  * rnnt_hip_viterbi_decode_* is the one rnnt_hip_viterbi_decode finds on the same values. */
 int rnnt_hip_loss_forward_bf16(const uint16_t* emissions, const uint16_t* predictions,
                                const int* labels, const int* input_lengths,

@@ -251,12 +251,7 @@ int viterbi_impl(const TIO* E, const TIO* P, const float* LN, int* labels,
 
 
 // ---------------------------------------------------------------- 16-bit scores
-int check_lowp_shape(const void* E, const void* P, const Dims& d, bool loss, const char* who) {
-  if (d.V % 8 != 0)
-    return fail(kInvalid, "%s: 16-bit scores need a vocabulary that is a multiple of 8 (V=%d)",
-                who, d.V);
-  if ((reinterpret_cast<uintptr_t>(E) | reinterpret_cast<uintptr_t>(P)) & 15)
-    return fail(kInvalid, "%s: 16-bit scores must be 16-byte aligned", who);
+int check_lowp_shape(const Dims& d, bool loss, const char* who) {
   if (loss && !egrads_one_pass(d))
     return fail(kInvalid, "%s: 16-bit scores take at most 112 label positions (U=%d)", who, d.U);
   return kOk;
@@ -280,7 +275,7 @@ int lowp_loss_forward(const TIO* E, const TIO* P, const int* labels, const int* 
     return fail(kWorkspace, "%s: workspace of %zu bytes, %zu needed", who, workspace_bytes,
                 rnnt_hip_loss_workspace_bytes(B, T, U, V));
   const Dims d = make_dims(B, T, U, V, blank);
-  RNNT_TRY(check_lowp_shape(E, P, d, true, who));
+  RNNT_TRY(check_lowp_shape(d, true, who));
   if (!lse_stream_supported(E, d)) return fail(kInvalid, "%s: B*T*U too large", who);
   LossWorkspace w;
   loss_workspace_layout(d, workspace, &w);
@@ -313,7 +308,7 @@ int lowp_loss_backward(const TIO* E, const TIO* P, const int* labels, const int*
     return fail(kWorkspace, "%s: workspace of %zu bytes, %zu needed", who, workspace_bytes,
                 rnnt_hip_loss_workspace_bytes(B, T, U, V));
   const Dims d = make_dims(B, T, U, V, blank);
-  RNNT_TRY(check_lowp_shape(E, P, d, true, who));
+  RNNT_TRY(check_lowp_shape(d, true, who));
   if ((reinterpret_cast<uintptr_t>(egrads) | reinterpret_cast<uintptr_t>(pgrads)) & 1)
     return fail(kInvalid, "%s: misaligned gradient arrays", who);
   LossWorkspace w;
@@ -349,7 +344,7 @@ int lowp_viterbi_decode(const TIO* E, const TIO* P, const int* inLen, const int*
     return fail(kInvalid, "%s: null array argument", who);
   hipStream_t s = static_cast<hipStream_t>(stream);
   const Dims d = make_dims(B, T, U, V, blank);
-  RNNT_TRY(check_lowp_shape(E, P, d, false, who));
+  RNNT_TRY(check_lowp_shape(d, false, who));
   if (!lse_stream_supported(E, d)) return fail(kInvalid, "%s: B*T*U too large", who);
   Scratch scratch(s);
   const size_t btu = sizeof(float) * (size_t)B * T * U;

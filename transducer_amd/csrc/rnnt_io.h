@@ -110,6 +110,37 @@ __device__ inline void expand(const Raw8<bf16_t>& r, float (&e)[8]) {
   e[6] = __uint_as_float(r.w.w << 16); e[7] = __uint_as_float(r.w.w & 0xffff0000u);
 }
 
+// The same eight elements fetched one by one, each index clamped to the row's last element: for
+// rows whose length or start does not allow 16-byte loads (a vocabulary that is not a multiple
+// of the vector width, an unaligned array).
+__device__ inline Raw8<float> load8_any(const float* row, int v, int V) {
+  Raw8<float> r;
+  r.lo = make_float4(row[min(v, V - 1)], row[min(v + 1, V - 1)], row[min(v + 2, V - 1)],
+                     row[min(v + 3, V - 1)]);
+  r.hi = make_float4(row[min(v + 4, V - 1)], row[min(v + 5, V - 1)], row[min(v + 6, V - 1)],
+                     row[min(v + 7, V - 1)]);
+  return r;
+}
+template <typename T16>
+__device__ inline uint4 load8_any_bits(const T16* row, int v, int V) {
+  unsigned w[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+    w[i] = (unsigned)row[min(v + 2 * i, V - 1)].bits |
+           ((unsigned)row[min(v + 2 * i + 1, V - 1)].bits << 16);
+  return make_uint4(w[0], w[1], w[2], w[3]);
+}
+__device__ inline Raw8<bf16_t> load8_any(const bf16_t* row, int v, int V) {
+  Raw8<bf16_t> r;
+  r.w = load8_any_bits(row, v, V);
+  return r;
+}
+__device__ inline Raw8<f16_t> load8_any(const f16_t* row, int v, int V) {
+  Raw8<f16_t> r;
+  r.w = load8_any_bits(row, v, V);
+  return r;
+}
+
 // Vector width (elements) that makes a row start 16-byte aligned.
 template <typename T>
 struct RowAlign;

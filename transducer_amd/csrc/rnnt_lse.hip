@@ -108,7 +108,9 @@ __global__ __launch_bounds__(256) void yplanes_kernel(const TIO* __restrict__ P,
 // kWaves = 4: a wavefront owns one block of 32 label positions and all 128 frames (four
 // accumulators).  kWaves = 8: two wavefronts share a block, 64 frames each (two accumulators,
 // half the registers, twice the wavefronts to hide each other's staging).
-template <int kWaves, typename TIO>
+// kVec: rows start 16-byte aligned and hold a multiple of the vector width, so a thread's eight
+// values are one or two 16-byte loads; otherwise they are fetched one by one.
+template <int kWaves, typename TIO, bool kVec>
 __global__ __launch_bounds__(64 * kWaves, kWaves / 2) void lse_stream_kernel(
     const TIO* __restrict__ E, float* __restrict__ mE, const float* __restrict__ mP,
     const uint4* __restrict__ Yp, float* __restrict__ LN, const int* __restrict__ inLen,
@@ -175,9 +177,9 @@ __global__ __launch_bounds__(64 * kWaves, kWaves / 2) void lse_stream_kernel(
   int next_slab = -1;  // slab of entry `cursor` (kept in a register: no LDS access on slabs without one)
 
   // staging: thread -> rows srow (+ 64 with four wavefronts) of the tile, v = slab start +
-  // 8*c8 .. +7.  Rows past the utterance repeat its last frame, groups of four past V repeat
-  // the row's last group (V % 4 == 0): finite values that meet zeros in Y or are dropped on
-  // the way out.
+  // 8*c8 .. +7.  Rows past the utterance repeat its last frame, columns past V repeat earlier
+  // ones of the row (its last group of four or eight, or its last element when the values are
+  // fetched one by one): finite values that meet zeros in Y or are dropped on the way out.
   const int srow = tid >> 2, c8 = tid & 3;
   const TIO* px[NR];
   float mx[NR];  // the row's reference; the four threads that share a row always agree on it
@@ -194,7 +196,8 @@ __global__ __launch_bounds__(64 * kWaves, kWaves / 2) void lse_stream_kernel(
   auto fetch = [&](int k0) -> XRegs {
     XRegs r;
 #pragma unroll
-    for (int i = 0; i < NR; ++i) r.x[i] = load8(px[i], k0 + 8 * c8, d.V);
+    for (int i = 0; i < NR; ++i)
+      r.x[i] = kVec ? load8(px[i], k0 + 8 * c8, d.V) : load8_any(px[i], k0 + 8 * c8, d.V);
     return r;
   };
   // copies column `col` (which lies in the slab held in r) of this thread's rows to dst[t]
@@ -432,17 +435,16 @@ __global__ __launch_bounds__(64 * kWaves, kWaves / 2) void lse_stream_kernel(
 
 template <typename TIO>
 static bool lse_stream_ok(const TIO* E, const Dims& d) {
-  constexpr int kA = RowAlign<TIO>::kElems;
+  (void)E;
   const long total = (long)((d.T + kRows - 1) / kRows) * ((d.U + 127) / 128) * d.B;
-  return d.V % kA == 0 && d.V >= kA && (reinterpret_cast<uintptr_t>(E) & 15) == 0 &&
-         total < (1l << 30);
+  return d.V >= 1 && total < (1l << 30);
 }
 bool lse_stream_supported(const float* E, const Dims& d) { return lse_stream_ok(E, d); }
 bool lse_stream_supported(const bf16_t* E, const Dims& d) { return lse_stream_ok(E, d); }
 bool lse_stream_supported(const f16_t* E, const Dims& d) { return lse_stream_ok(E, d); }
 
 size_t lse_scratch_bytes(const Dims& d) {
-  if (d.B == 0 || d.T == 0 || d.U == 0 || d.V % 4 != 0) return 0;
+  if (d.B == 0 || d.T == 0 || d.U == 0 || d.V == 0) return 0;
   return (size_t)d.B * y_ublocks(d) * y_steps(d) * 3 * 64 * sizeof(uint4);
 }
 
@@ -479,9 +481,16 @@ static int lse_stream_any(const TIO* E, float* mE, const float* mP, float* LN,
   const long total = (long)ttiles * utiles * d.B;
   const int grid = (int)((total + 7) / 8 * 8);
   constexpr int kWaves = 4;
-  hipLaunchKernelGGL((lse_stream_kernel<kWaves, TIO>), dim3(grid), dim3(64 * kWaves), 0, s, E, mE, mP,
-                     static_cast<const uint4*>(scratch), LN, inLen, labLen, d, ttiles, utiles,
-                     (int)total, nub, nks, labels, elS, eb, lnS);
+  constexpr int kA = RowAlign<TIO>::kElems;
+  const bool vec = d.V % kA == 0 && d.V >= kA && (reinterpret_cast<uintptr_t>(E) & 15) == 0;
+  if (vec)
+    hipLaunchKernelGGL((lse_stream_kernel<kWaves, TIO, true>), dim3(grid), dim3(64 * kWaves), 0,
+                       s, E, mE, mP, static_cast<const uint4*>(scratch), LN, inLen, labLen, d,
+                       ttiles, utiles, (int)total, nub, nks, labels, elS, eb, lnS);
+  else
+    hipLaunchKernelGGL((lse_stream_kernel<kWaves, TIO, false>), dim3(grid), dim3(64 * kWaves), 0,
+                       s, E, mE, mP, static_cast<const uint4*>(scratch), LN, inLen, labLen, d,
+                       ttiles, utiles, (int)total, nub, nks, labels, elS, eb, lnS);
   RNNT_LAUNCH_CHECK("lse_stream_kernel");
   return kOk;
 }

@@ -111,8 +111,8 @@ class TransducerLoss(torch.nn.Module):
     allow_bf16, allow_fp16: when True, ``torch.bfloat16`` / ``torch.float16`` emissions and
         predictions (both of the same type) are accepted as well; costs are float32 and the
         gradients come back in the scores' type.  The reference raises ``TypeError`` for
-        anything but float32, and so does this module unless a flag is set.  Needs a vocabulary
-        that is a multiple of 8 and, for the loss, at most 112 label positions.
+        anything but float32, and so does this module unless a flag is set.  The loss takes at
+        most 112 label positions in these types (any vocabulary size).
     """
 
     def __init__(self, blank=0, allow_bf16=False, allow_fp16=False):
