@@ -33,7 +33,7 @@ __device__ inline float wave_max(float m) {
 }
 
 // ------------------------------------------------------------------ row maxima
-// 16-bit rows (V % 8 == 0 and 16-byte aligned when vec is set): eight elements per load.
+// 16-bit rows (V % 8 == 0 and 16-byte aligned when vec is set): eight elements per aligned load.
 template <typename T16, typename = std::enable_if_t<sizeof(T16) == 2>>
 __device__ inline float row_max(const T16* __restrict__ x, int V, int vec, int lane) {
   float m0 = kNegInf, m1 = kNegInf;
@@ -45,7 +45,14 @@ __device__ inline float row_max(const T16* __restrict__ x, int V, int vec, int l
       m1 = fmaxf(m1, fmaxf(fmaxf(e[4], e[5]), fmaxf(e[6], e[7])));
     }
   } else {
-    for (int i = lane; i < V; i += 64) m0 = fmaxf(m0, ldf(x + i));
+    // whole eights at the element type's own alignment, then the row's last few one by one
+    for (int i = lane; i < (V >> 3); i += 64) {
+      float e[8];
+      expand(load8_any(x, 8 * i, V), e);
+      m0 = fmaxf(m0, fmaxf(fmaxf(e[0], e[1]), fmaxf(e[2], e[3])));
+      m1 = fmaxf(m1, fmaxf(fmaxf(e[4], e[5]), fmaxf(e[6], e[7])));
+    }
+    for (int i = (V & ~7) + lane; i < V; i += 64) m0 = fmaxf(m0, ldf(x + i));
   }
   return wave_max(fmaxf(m0, m1));
 }
@@ -72,7 +79,14 @@ __device__ inline float row_max(const float* __restrict__ x, int V, int vec4, in
       m0 = fmaxf(m0, fmaxf(fmaxf(a.x, a.y), fmaxf(a.z, a.w)));
     }
   } else {
-    for (int i = lane; i < V; i += 64) m0 = fmaxf(m0, x[i]);
+    // whole eights as 4-byte aligned wide loads, then the row's last few one by one
+    for (int i = lane; i < (V >> 3); i += 64) {
+      float e[8];
+      expand(load8_any(x, 8 * i, V), e);
+      m0 = fmaxf(m0, fmaxf(fmaxf(e[0], e[1]), fmaxf(e[2], e[3])));
+      m1 = fmaxf(m1, fmaxf(fmaxf(e[4], e[5]), fmaxf(e[6], e[7])));
+    }
+    for (int i = (V & ~7) + lane; i < V; i += 64) m0 = fmaxf(m0, x[i]);
   }
   return wave_max(fmaxf(fmaxf(m0, m1), fmaxf(m2, m3)));
 }

@@ -110,11 +110,22 @@ __device__ inline void expand(const Raw8<bf16_t>& r, float (&e)[8]) {
   e[6] = __uint_as_float(r.w.w << 16); e[7] = __uint_as_float(r.w.w & 0xffff0000u);
 }
 
-// The same eight elements fetched one by one, each index clamped to the row's last element: for
-// rows whose length or start does not allow 16-byte loads (a vocabulary that is not a multiple
-// of the vector width, an unaligned array).
+// The same eight elements of a row whose length or start does not allow aligned 16-byte loads
+// (a vocabulary that is not a multiple of the vector width, an unaligned array).  Eight that lie
+// inside the row come in as loads of the same width at the element type's own alignment, which
+// global memory serves; the row's last, partial eight are fetched one by one, each index clamped
+// to the row's last element.
+typedef float float4_align4 __attribute__((ext_vector_type(4), aligned(4)));
+typedef unsigned uint4_align2 __attribute__((ext_vector_type(4), aligned(2)));
 __device__ inline Raw8<float> load8_any(const float* row, int v, int V) {
   Raw8<float> r;
+  if (v + 8 <= V) {
+    const float4_align4 a = *reinterpret_cast<const float4_align4*>(row + v);
+    const float4_align4 b = *reinterpret_cast<const float4_align4*>(row + v + 4);
+    r.lo = make_float4(a.x, a.y, a.z, a.w);
+    r.hi = make_float4(b.x, b.y, b.z, b.w);
+    return r;
+  }
   r.lo = make_float4(row[min(v, V - 1)], row[min(v + 1, V - 1)], row[min(v + 2, V - 1)],
                      row[min(v + 3, V - 1)]);
   r.hi = make_float4(row[min(v + 4, V - 1)], row[min(v + 5, V - 1)], row[min(v + 6, V - 1)],
@@ -123,6 +134,10 @@ __device__ inline Raw8<float> load8_any(const float* row, int v, int V) {
 }
 template <typename T16>
 __device__ inline uint4 load8_any_bits(const T16* row, int v, int V) {
+  if (v + 8 <= V) {
+    const uint4_align2 a = *reinterpret_cast<const uint4_align2*>(row + v);
+    return make_uint4(a.x, a.y, a.z, a.w);
+  }
   unsigned w[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i)

@@ -83,18 +83,13 @@ __global__ __launch_bounds__(256) void yplanes_kernel(const TIO* __restrict__ P,
   if (u < Ub) {
     const TIO* row = P + ((size_t)b * d.U + u) * d.V;
     const float m = mP[(size_t)b * d.U + u];
-    if (vec4) {
-      if (v0 < d.V) {
-        float e[8];
-        expand(load8(row, v0, d.V), e);  // a clamped group repeats values; masked below
-#pragma unroll
-        for (int i = 0; i < 8; ++i)
-          if (v0 + i < d.V) y[i] = __expf(e[i] - m);
-      }
-    } else {
+    if (v0 < d.V) {
+      float e[8];  // clamped loads repeat values of the row; masked below
+      if (vec4) expand(load8(row, v0, d.V), e);
+      else expand(load8_any(row, v0, d.V), e);
 #pragma unroll
       for (int i = 0; i < 8; ++i)
-        if (v0 + i < d.V) y[i] = __expf(ldf(row + v0 + i) - m);
+        if (v0 + i < d.V) y[i] = __expf(e[i] - m);
     }
   }
   const Frag3 f = split8(y);
