@@ -340,7 +340,7 @@ def test_whole_loss_with_a_label_axis_longer_than_one_slice(T, U, V):
     later slices adding to what is in egrads and only the last one applying the upstream factors
     (so U + 1 = 112, 113, 224, 225 sit on the slice edges).  With V >= 512 the blank/label terms
     ride in the first slice's write-out, below that they are scattered; odd V also takes the
-    general log-normaliser.  Same entry points, same bar."""
+    log-normaliser's unaligned row loads.  Same entry points, same bar."""
     cfg = small_config(2, T, U, V, ragged=True)
     E, P, labels, il, ll = unpack(make_inputs(cfg, seed=T + U + V))
     deltas = np.array([0.5, 3.0], np.float32)

@@ -113,41 +113,34 @@ int check_dims(int B, int T, int U, int V) {
 
 bool nothing_to_do(int B, int T, int U) { return B == 0 || T == 0 || U == 0; }
 
-// Row maxima of both score arrays, then the log-normaliser: the streaming kernel when the
-// shape allows it and `scratch` (lse_scratch_bytes) is given, else the general one.
-// With `planes`, the row-maximum pass also extracts the blank / label scores the lattice
-// recursions need (no separate gather).
+// Row maxima of the predictions, the Y pieces, then the streaming log-normaliser (which finds
+// the emissions' per-frame reference itself); `scratch` holds lse_scratch_bytes(d).
+// With `planes`, the blank / label scores the lattice recursions need are extracted on the way
+// (no separate gather).
 int log_norms_stages(const float* E, const float* P, float* mE, float* mP, float* LN,
                      void* scratch, const int* inLen, const int* labLen, const Dims& d,
                      hipStream_t s, const Planes* planes = nullptr, const int* labels = nullptr,
                      bool* ln_in_plane = nullptr) {
   if (ln_in_plane) *ln_in_plane = false;
-  if (scratch && lse_stream_supported(E, d)) {
-    // one pass over E: the streaming kernel finds its own per-frame reference and leaves it in mE
-    // and, with `planes`, copies the blank / label scores out of the rows as they stream by
-    if (planes && d.U - 1 <= 1024) {
-      RNNT_STAGE(kRowmax, launch_rowmax_pick_p(P, mP, labels, labLen, *planes, d, s));
-      RNNT_STAGE(kYplanes, launch_yplanes(P, mP, scratch, labLen, d, s));
-      // (with the flag the caller says it only needs LN in the lattice plane)
-      RNNT_STAGE(kLse, launch_lse_stream(E, mE, mP, LN, scratch, inLen, labLen, d, s, labels,
-                                         planes->elS, planes->eb,
-                                         ln_in_plane ? planes->lnS : nullptr));
-      if (ln_in_plane) *ln_in_plane = true;
-      return kOk;
-    }
-    RNNT_STAGE(kRowmax, launch_rowmax(P, mP, (long)d.B * d.U, d.V, d.U, labLen, 1, s));
+  if (!scratch || !lse_stream_supported(E, d))
+    return fail(kInvalid, "log-normaliser: more than 2^30 tiles of 128 frames x 128 label "
+                          "positions (B=%d T=%d U=%d)", d.B, d.T, d.U);
+  // one pass over E: the streaming kernel finds its own per-frame reference and leaves it in mE
+  // and, with `planes`, copies the blank / label scores out of the rows as they stream by
+  if (planes && d.U - 1 <= 1024) {
+    RNNT_STAGE(kRowmax, launch_rowmax_pick_p(P, mP, labels, labLen, *planes, d, s));
     RNNT_STAGE(kYplanes, launch_yplanes(P, mP, scratch, labLen, d, s));
-    RNNT_STAGE(kLse, launch_lse_stream(E, mE, mP, LN, scratch, inLen, labLen, d, s));
-    if (planes) RNNT_STAGE(kGather, launch_gather(E, P, labels, inLen, labLen, *planes, d, s));
+    // (with the flag the caller says it only needs LN in the lattice plane)
+    RNNT_STAGE(kLse, launch_lse_stream(E, mE, mP, LN, scratch, inLen, labLen, d, s, labels,
+                                       planes->elS, planes->eb,
+                                       ln_in_plane ? planes->lnS : nullptr));
+    if (ln_in_plane) *ln_in_plane = true;
     return kOk;
   }
-  if (planes) {
-    RNNT_STAGE(kRowmax, launch_rowmax_pick(E, P, mE, mP, labels, inLen, labLen, *planes, d, s));
-  } else {
-    RNNT_STAGE(kRowmax, launch_rowmax(E, mE, (long)d.B * d.T, d.V, d.T, inLen, 0, s));
-    RNNT_STAGE(kRowmax, launch_rowmax(P, mP, (long)d.B * d.U, d.V, d.U, labLen, 1, s));
-  }
-  RNNT_STAGE(kLse, launch_lse(E, P, mE, mP, LN, inLen, labLen, d, s));
+  RNNT_STAGE(kRowmax, launch_rowmax(P, mP, (long)d.B * d.U, d.V, d.U, labLen, 1, s));
+  RNNT_STAGE(kYplanes, launch_yplanes(P, mP, scratch, labLen, d, s));
+  RNNT_STAGE(kLse, launch_lse_stream(E, mE, mP, LN, scratch, inLen, labLen, d, s));
+  if (planes) RNNT_STAGE(kGather, launch_gather(E, P, labels, inLen, labLen, *planes, d, s));
   return kOk;
 }
 
@@ -591,8 +584,8 @@ int rnnt_hip_loss_backward(const float* E, const float* P, const int* labels, co
   return kOk;
 }
 
-// 16-bit scores (bf16, fp16): the shapes the streaming kernels take (every launcher below exists
-// for all three element types; the general-shape fallbacks are fp32 only).  The three entry
+// 16-bit scores (bf16, fp16): every launcher below exists for all three element types; only the
+// sliced label axis of egrads (more than 112 label positions) is fp32 only.  The three entry
 // points per type are thin wrappers around the templates above.
 #define RNNT_LOWP_ENTRY_POINTS(SUFFIX, TIO)                                                       \
   int rnnt_hip_loss_forward_##SUFFIX(const uint16_t* E, const uint16_t* P, const int* labels,     \

@@ -1,19 +1,8 @@
-// The three vocabulary-sized contractions of the RNN-T loss on the gfx950 matrix cores, with
-// their exponentials and logarithms fused in so that nothing of size B*T*U*V -- and no copy of
-// the [B,T,V] emissions -- ever goes to memory:
-//
-//   log-normaliser (transducer/torch_binding.py:35-40)
-//       LN[t,u] = log( sum_v exp(E[t,v]-mE[t]) * exp(P[u,v]-mP[u]) ) + mE[t] + mP[u]
-//   dense gradient parts (transducer/torch_binding.py:85-89), W[t,u] = dalpha[t,u]/sum_v(...)
+// Row maxima of the score arrays, the W planes that feed the two gradient contractions, and
+// the launchers of those contractions (rnnt_grads.hip).  W[t,u] = dalpha[t,u] / sum_v(...) as in
+// the dense gradient parts of transducer/torch_binding.py:85-89:
 //       egrads[t,v] = delta * exp(E[t,v]-mE[t]) * sum_u W[t,u] * exp(P[u,v]-mP[u])
 //       pgrads[u,v] = delta * exp(P[u,v]-mP[u]) * sum_t W[t,u] * exp(E[t,v]-mE[t])
-//
-// All three use v_mfma_f32_32x32x2_f32 (fp32 in, fp32 accumulate).  A wavefront owns 32x32
-// output blocks; for one instruction lane l supplies A[row l%32][k-slot l/32] and
-// B[k-slot l/32][col l%32] and receives D[8*(r/4) + 4*(l/32) + r%4][l%32] in register r.
-// Which element of the reduction sits in which k-slot is free as long as A and B agree, so a
-// lane takes four consecutive k of its row with one 16-byte LDS read and spends them on four
-// instructions.
 #include <type_traits>
 
 #include "rnnt_internal.h"
@@ -21,8 +10,6 @@
 namespace rnnt {
 
 namespace {
-
-typedef float floatx16 __attribute__((ext_vector_type(16)));
 
 constexpr float kNegInf = -__builtin_huge_valf();
 
@@ -110,77 +97,8 @@ __global__ __launch_bounds__(256) void rowmax_kernel(const TIO* __restrict__ X,
   if (lane == 0) out[row] = m;
 }
 
-// Row maxima of the emissions plus the elements of each row that the lattice recursions need:
-// E[t, blank] and E[t, label_u] for every label position, written to the skewed planes (what
-// gather_kernel of rnnt_dp.hip does with one scattered HBM sector per element; here the sectors
-// are part of the row that is being streamed anyway).  A workgroup takes 16 consecutive frames of
-// one utterance, four per wavefront; the picked scores meet in LDS and leave as runs of 16
-// consecutive frames per label position.  Frames past the utterance are skipped.
-constexpr int kPickRows = 16, kPickU = 256;
-
-__global__ __launch_bounds__(256) void rowmax_pick_e_kernel(const float* __restrict__ E,
-                                                            float* __restrict__ mE,
-                                                            const int* __restrict__ labels,
-                                                            const int* __restrict__ inLen,
-                                                            const int* __restrict__ labLen,
-                                                            Planes p, Dims d, int vec4) {
-  __shared__ float tile[kPickRows][kPickU + 1];
-  __shared__ float blanks[kPickRows];
-  const int b = blockIdx.y, t0 = blockIdx.x * kPickRows;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  int Tb, Ub;
-  utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
-  const int nlab = labels ? max(Ub - 1, 0) : 0;
-  // label columns of this lane (first kPickU label positions)
-  int col[kPickU / 64];
-#pragma unroll
-  for (int i = 0; i < kPickU / 64; ++i) {
-    const int u = lane + 64 * i;
-    col[i] = u < nlab ? labels[(size_t)b * (d.U - 1) + u] : d.blank;
-  }
-  // The picks of a frame are requested right after its row has been streamed (they hit L2) and
-  // are put away after the NEXT row's stream, so their latency is never waited for.
-  float pick[kPickU / 64], xb = 0.0f;
-  int pending = -1;  // tile row the registers belong to
-  auto put_away = [&]() {
-    if (pending < 0) return;
-#pragma unroll
-    for (int k = 0; k < kPickU / 64; ++k) tile[pending][lane + 64 * k] = pick[k];
-    if (lane == 0) blanks[pending] = xb;
-    pending = -1;
-  };
-  for (int r = 0; r < 4; ++r) {
-    const int i = 4 * wave + r, t = t0 + i;
-    if (t >= d.T) break;
-    const size_t row = (size_t)b * d.T + t;
-    if (t >= Tb) {
-      if (lane == 0) mE[row] = 0.0f;
-      continue;
-    }
-    const float* x = E + row * d.V;
-    const float m = row_max(x, d.V, vec4, lane);
-    if (lane == 0) mE[row] = m;
-    put_away();
-#pragma unroll
-    for (int k = 0; k < kPickU / 64; ++k) pick[k] = x[col[k]];
-    xb = x[d.blank];
-    pending = i;
-    // label positions past the first kPickU: straight from the row
-    for (int u = kPickU + lane; u < nlab; u += 64)
-      p.elS[plane_row(d, b, u) + t + u] = x[labels[(size_t)b * (d.U - 1) + u]];
-  }
-  put_away();
-  __syncthreads();
-  const int nrows = min(kPickRows, Tb - t0);  // may be <= 0
-  if ((int)threadIdx.x < nrows) p.eb[(size_t)b * d.Tp + d.Eo + t0 + threadIdx.x] = blanks[threadIdx.x];
-  const int nu = min(nlab, kPickU);
-  for (int idx = threadIdx.x; idx < nu * kPickRows; idx += 256) {
-    const int u = idx >> 4, i = idx & 15;
-    if (i < nrows) p.elS[plane_row(d, b, u) + t0 + i + u] = tile[i][u];
-  }
-}
-
-// The same for the predictions: P[u, blank] and P[u, label_u].
+// Row maxima of the predictions plus the elements of each row that the lattice recursions need,
+// P[u, blank] and P[u, label_u], written to the small per-position vectors.
 template <typename TIO>
 __global__ __launch_bounds__(256) void rowmax_pick_p_kernel(const TIO* __restrict__ P,
                                                             float* __restrict__ mP,
@@ -204,133 +122,6 @@ __global__ __launch_bounds__(256) void rowmax_pick_p_kernel(const TIO* __restric
     p.pb[(size_t)b * d.Ua + u] = ldf(x + d.blank);
     p.pl[(size_t)b * d.Ua + u] = has_label ? ldf(x + labels[(size_t)b * (d.U - 1) + u]) : 0.0f;
   }
-}
-
-// ------------------------------------------------------------------ log-normaliser, any shape
-// Scalar-load form for vocabularies that are not a multiple of 4 or unaligned inputs.
-// Block tile 128 (t) x 128 (u), reduction over v in slices of 32; 4 wavefronts, each 64x64.
-// Both operands are v-contiguous in memory and are staged as S[row][v] with a 36-float pitch
-// (16-byte reads of consecutive rows then fall into distinct bank groups).
-constexpr int kLseBM = 128, kLseBN = 128, kLseBK = 32, kLsePitch = kLseBK + 4;
-
-__global__ __launch_bounds__(256, 2) void lse_kernel(const float* __restrict__ E,
-                                                     const float* __restrict__ P,
-                                                     const float* __restrict__ mE,
-                                                     const float* __restrict__ mP,
-                                                     float* __restrict__ LN,
-                                                     const int* __restrict__ inLen,
-                                                     const int* __restrict__ labLen, Dims d) {
-  __shared__ __attribute__((aligned(16))) float As[kLseBM * kLsePitch];
-  __shared__ __attribute__((aligned(16))) float Bs[kLseBN * kLsePitch];
-  const int b = blockIdx.z, t0 = blockIdx.x * kLseBM, u0 = blockIdx.y * kLseBN;
-  int Tb, Ub;
-  utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  float* LNb = LN + (size_t)b * d.T * d.U;
-
-  if (t0 >= Tb || u0 >= Ub) {
-    // nothing valid here: the array still gets defined contents (zeros, as in the torch-free
-    // reference helper transducer/test.h:58)
-    for (int e = tid; e < kLseBM * kLseBN; e += 256) {
-      const int t = t0 + e / kLseBN, u = u0 + e % kLseBN;
-      if (t < d.T && u < d.U) LNb[(size_t)t * d.U + u] = 0.0f;
-    }
-    return;
-  }
-
-  const float* Eb = E + (size_t)b * d.T * d.V;
-  const float* Pb = P + (size_t)b * d.U * d.V;
-  const float* mEb = mE + (size_t)b * d.T;
-  const float* mPb = mP + (size_t)b * d.U;
-
-  // staging assignment: element e = tid + 256*i -> row e/32, column e%32 (a wavefront reads two
-  // 128-byte row segments per load instruction)
-  const int lcol = tid & 31, lrow0 = tid >> 5;  // rows lrow0 + 8*i, i < 16
-  float ra[16], rb[16];
-  float ma[16], mb[16];
-  const float* pa[16];
-  const float* pb[16];
-#pragma unroll
-  for (int i = 0; i < 16; ++i) {
-    const int r = lrow0 + 8 * i;
-    const int t = min(t0 + r, d.T - 1), u = min(u0 + r, d.U - 1);
-    pa[i] = Eb + (size_t)t * d.V;
-    pb[i] = Pb + (size_t)u * d.V;
-    ma[i] = mEb[t];
-    mb[i] = mPb[u];
-  }
-  auto fetch = [&](int k0) {
-    const int v = k0 + lcol;
-    const bool ok = v < d.V;
-    const int vc = ok ? v : d.V - 1;
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const float x = pa[i][vc], y = pb[i][vc];
-      ra[i] = ok ? x : kNegInf;  // exp(-inf - m) = 0: past-the-end terms add nothing
-      rb[i] = ok ? y : kNegInf;
-    }
-  };
-
-  const int wm = wave >> 1, wn = wave & 1, l32 = lane & 31, h = lane >> 5;
-  floatx16 acc[2][2];
-#pragma unroll
-  for (int i = 0; i < 2; ++i)
-#pragma unroll
-    for (int j = 0; j < 2; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
-
-  const int nk = (d.V + kLseBK - 1) / kLseBK;
-  fetch(0);
-  for (int kt = 0; kt < nk; ++kt) {
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const int r = lrow0 + 8 * i;
-      As[r * kLsePitch + lcol] = __expf(ra[i] - ma[i]);
-      Bs[r * kLsePitch + lcol] = __expf(rb[i] - mb[i]);
-    }
-    __syncthreads();
-    if (kt + 1 < nk) fetch((kt + 1) * kLseBK);
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      float4 a4[2], b4[2];
-#pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        a4[i] = *reinterpret_cast<const float4*>(
-            &As[(64 * wm + 32 * i + l32) * kLsePitch + 8 * j + 4 * h]);
-        b4[i] = *reinterpret_cast<const float4*>(
-            &Bs[(64 * wn + 32 * i + l32) * kLsePitch + 8 * j + 4 * h]);
-      }
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-#pragma unroll
-        for (int i = 0; i < 2; ++i)
-#pragma unroll
-          for (int jj = 0; jj < 2; ++jj) {
-            const float av = q == 0 ? a4[i].x : (q == 1 ? a4[i].y : (q == 2 ? a4[i].z : a4[i].w));
-            const float bv =
-                q == 0 ? b4[jj].x : (q == 1 ? b4[jj].y : (q == 2 ? b4[jj].z : b4[jj].w));
-            acc[i][jj] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc[i][jj], 0, 0, 0);
-          }
-      }
-    }
-    __syncthreads();
-  }
-
-#pragma unroll
-  for (int i = 0; i < 2; ++i)
-#pragma unroll
-    for (int jj = 0; jj < 2; ++jj)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int t = t0 + 64 * wm + 32 * i + 8 * (r >> 2) + 4 * h + (r & 3);
-        const int u = u0 + 64 * wn + 32 * jj + l32;
-        if (t < d.T && u < d.U) {
-          float v = 0.0f;
-          if (t < Tb && u < Ub) v = (logf(acc[i][jj][r]) + mEb[t]) + mPb[u];
-          LNb[(size_t)t * d.U + u] = v;
-        }
-      }
 }
 
 // ------------------------------------------------------------------ W planes
@@ -401,21 +192,6 @@ int launch_rowmax(const f16_t* X, float* rowmax, long rows, int V, int rows_per_
   return rowmax_any(X, rowmax, rows, V, rows_per_item, lengths, extra, s);
 }
 
-int launch_rowmax_pick(const float* E, const float* P, float* mE, float* mP, const int* labels,
-                       const int* inLen, const int* labLen, const Planes& p, const Dims& d,
-                       hipStream_t s) {
-  if (d.B == 0 || d.T == 0 || d.U == 0) return kOk;
-  const int ve = (d.V % 4 == 0) && ((reinterpret_cast<uintptr_t>(E) & 15) == 0);
-  const int vp = (d.V % 4 == 0) && ((reinterpret_cast<uintptr_t>(P) & 15) == 0);
-  hipLaunchKernelGGL(rowmax_pick_e_kernel, dim3((d.T + kPickRows - 1) / kPickRows, d.B), dim3(256),
-                     0, s, E, mE, labels, inLen, labLen, p, d, ve);
-  RNNT_LAUNCH_CHECK("rowmax_pick_e_kernel");
-  hipLaunchKernelGGL(rowmax_pick_p_kernel<float>, dim3((unsigned)(((long)d.B * d.U + 3) / 4)),
-                     dim3(256), 0, s, P, mP, labels, labLen, p, d, vp);
-  RNNT_LAUNCH_CHECK("rowmax_pick_p_kernel");
-  return kOk;
-}
-
 template <typename TIO>
 static int rowmax_pick_p_any(const TIO* P, float* mP, const int* labels, const int* labLen,
                              const Planes& p, const Dims& d, hipStream_t s) {
@@ -437,16 +213,6 @@ int launch_rowmax_pick_p(const bf16_t* P, float* mP, const int* labels, const in
 int launch_rowmax_pick_p(const f16_t* P, float* mP, const int* labels, const int* labLen,
                          const Planes& p, const Dims& d, hipStream_t s) {
   return rowmax_pick_p_any(P, mP, labels, labLen, p, d, s);
-}
-
-int launch_lse(const float* E, const float* P, const float* mE, const float* mP, float* LN,
-               const int* inLen, const int* labLen, const Dims& d, hipStream_t s) {
-  if (d.B == 0 || d.T == 0 || d.U == 0) return kOk;
-  hipLaunchKernelGGL(lse_kernel,
-                     dim3((d.T + kLseBM - 1) / kLseBM, (d.U + kLseBN - 1) / kLseBN, d.B),
-                     dim3(256), 0, s, E, P, mE, mP, LN, inLen, labLen, d);
-  RNNT_LAUNCH_CHECK("lse_kernel");
-  return kOk;
 }
 
 int wplane_up(int U) { return (U + 7) & ~7; }

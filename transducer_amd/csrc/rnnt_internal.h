@@ -148,21 +148,13 @@ int launch_rowmax(const bf16_t* X, float* rowmax, long rows, int V, int rows_per
                   const int* lengths, int extra, hipStream_t s);
 int launch_rowmax(const f16_t* X, float* rowmax, long rows, int V, int rows_per_item,
                   const int* lengths, int extra, hipStream_t s);
-// Row maxima of E and P and, in the same pass, what launch_gather extracts (E[t,blank],
-// E[t,label_u], P[u,blank], P[u,label_u] into the planes); needs inLen and labLen.
-int launch_rowmax_pick(const float* E, const float* P, float* mE, float* mP, const int* labels,
-                       const int* inLen, const int* labLen, const Planes& p, const Dims& d,
-                       hipStream_t s);
-// Log-normaliser, general form (any V and alignment; fp32 matrix instructions).
-int launch_lse(const float* E, const float* P, const float* mE, const float* mP, float* LN,
-               const int* inLen, const int* labLen, const Dims& d, hipStream_t s);
-// Log-normaliser, streaming form (rnnt_lse.hip): any V; 16-byte row loads when V is a multiple of
+// Log-normaliser (rnnt_lse.hip): any V; 16-byte row loads when V is a multiple of
 // the vector width and E is 16-byte aligned, element loads otherwise.  The pieces of
 // exp(P - mP) are first written to `scratch` (lse_scratch_bytes) in matrix-operand order.
 // launch_lse_stream needs mP only and WRITES mE (one reference value per frame, >= the row
 // maximum minus a fixed slack; what the gradient kernels need as mE).
-// Each launcher that reads the scores or writes their gradients exists for fp32 and for bf16
-// arrays (rnnt_io.h).
+// Each launcher that reads the scores or writes their gradients exists for fp32, bf16 and
+// fp16 arrays (rnnt_io.h).
 bool lse_stream_supported(const float* E, const Dims& d);
 bool lse_stream_supported(const bf16_t* E, const Dims& d);
 bool lse_stream_supported(const f16_t* E, const Dims& d);
