@@ -344,3 +344,60 @@ def test_16bit_best_path_through_the_torch_module(kind):
     ref = decode_16bit(E, P, il, ll)
     for b in range(B):
         assert torch.equal(paths[b, :ll[b]], ref[b, :ll[b]])
+
+
+def _loss_any(E, P, eg, pg, labels, il, ll, deltas):
+    """Whole loss through the entry points of the tensors' type, on exactly these arrays."""
+    sfx = "" if E.dtype is torch.float32 else suffix_of(E)
+    B, T, V = E.shape
+    U = P.shape[1]
+    d_il, d_ll = dev(il), dev(ll)
+    nbytes = capi.load().rnnt_hip_loss_workspace_bytes(B, T, U, V)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device="cuda:0")
+    costs = torch.full((B,), float("nan"), device="cuda:0")
+    capi.call("rnnt_hip_loss_forward" + sfx, ptr(E), ptr(P), ptr(labels), ptr(d_il), ptr(d_ll),
+              ptr(costs), ptr(ws), nbytes, B, T, U, V, 0, None)
+    capi.call("rnnt_hip_loss_backward" + sfx, ptr(E), ptr(P), ptr(labels), ptr(d_il), ptr(d_ll),
+              ptr(deltas), ptr(eg), ptr(pg), ptr(ws), nbytes, B, T, U, V, 0, None)
+    torch.cuda.synchronize()
+    return costs
+
+
+@pytest.mark.parametrize("kind", ["f32"] + KIND_NAMES)
+@pytest.mark.parametrize("B,T,U,V", [(2, 40, 9, 24), (2, 70, 20, 1000), (3, 130, 33, 520)])
+def test_arrays_that_start_off_a_16_byte_boundary_give_the_same_bits(B, T, U, V, kind):
+    """The vocabulary allows 16-byte row loads but the arrays start one element past a 16-byte
+    boundary (4-byte aligned fp32, 2-byte aligned 16-bit), as a view into a larger buffer does:
+    rows then come in through the loads at the element's own alignment.  Only the loads differ,
+    so costs, gradients and the best path are the aligned call's, bit for bit."""
+    dtype = torch.float32 if kind == "f32" else KINDS[kind][0]
+    E, P, labels, il, ll = draw(B, T, U, V, seed=B + T + U + V, kind="bf16" if kind == "f32" else kind)
+    E, P = E.to(dtype), P.to(dtype)
+    deltas = torch.tensor([0.5, 2.0, 1.0][:B], device="cuda:0")
+
+    def shifted(x, fill):
+        buf = torch.full((x.numel() + 16,), fill, device="cuda:0", dtype=x.dtype)
+        view = buf[1:1 + x.numel()].view(x.shape)
+        view.copy_(x)
+        assert view.data_ptr() % 16 == x.element_size() and view.is_contiguous()
+        return view
+
+    eg, pg = torch.full_like(E, float("nan")), torch.full_like(P, float("nan"))
+    costs = _loss_any(E, P, eg, pg, labels, il, ll, deltas)
+    Es, Ps = shifted(E, float("nan")), shifted(P, float("nan"))
+    egs, pgs = shifted(eg, float("nan")), shifted(pg, float("nan"))
+    costs_s = _loss_any(Es, Ps, egs, pgs, labels, il, ll, deltas)
+    assert torch.equal(costs, costs_s)
+    assert torch.equal(eg.view(torch.uint8), egs.contiguous().view(torch.uint8))
+    assert torch.equal(pg.view(torch.uint8), pgs.contiguous().view(torch.uint8))
+
+    sfx = "" if kind == "f32" else KINDS[kind][1]
+    d_il, d_ll = dev(il), dev(ll)
+    paths = []
+    for e, p in ((E, P), (Es, Ps)):
+        out = torch.full((B, U - 1), -1, device="cuda:0", dtype=torch.int32)
+        capi.call("rnnt_hip_viterbi_decode" + sfx, ptr(e), ptr(p), ptr(d_il), ptr(d_ll),
+                  ptr(out), B, T, U, V, 0, None)
+        torch.cuda.synchronize()
+        paths.append(out)
+    assert torch.equal(paths[0], paths[1])

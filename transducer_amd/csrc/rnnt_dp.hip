@@ -779,11 +779,8 @@ __global__ __launch_bounds__(kMpThreads) void maxplus_kernel(const TIO* __restri
     if (kVec) {  // columns past V are re-read from the row's last four (E: masked below; P: any
                  // finite value will do there, E is -inf)
       x = load4(src + min(v, d.V - 4));
-    } else {
-      x.x = ldf(src + min(v, d.V - 1));
-      x.y = ldf(src + min(v + 1, d.V - 1));
-      x.z = ldf(src + min(v + 2, d.V - 1));
-      x.w = ldf(src + min(v + 3, d.V - 1));
+    } else {  // one wide load at the element's own alignment, one by one at the row's end
+      x = load4_any(src, min(v, d.V - 1), d.V);
     }
     return x;
   };

@@ -54,6 +54,45 @@ __device__ inline float4 load4(const f16_t* p) {
                      f16_to_float((unsigned short)(w.y >> 16)));
 }
 
+// Wide loads at the element type's own alignment (global memory serves them at any such
+// address): for rows whose length or start does not allow the naturally aligned ones.
+typedef float float4_align4 __attribute__((ext_vector_type(4), aligned(4)));
+typedef unsigned uint4_align2 __attribute__((ext_vector_type(4), aligned(2)));
+typedef unsigned uint2_align2 __attribute__((ext_vector_type(2), aligned(2)));
+
+// Elements v .. v+3 of a row of V elements at any alignment: one wide load when all four lie
+// inside the row, else one by one with the index clamped to the row's last element.
+__device__ inline float4 load4_any(const float* row, int v, int V) {
+  if (v + 4 <= V) {
+    const float4_align4 a = *reinterpret_cast<const float4_align4*>(row + v);
+    return make_float4(a.x, a.y, a.z, a.w);
+  }
+  return make_float4(row[min(v, V - 1)], row[min(v + 1, V - 1)], row[min(v + 2, V - 1)],
+                     row[min(v + 3, V - 1)]);
+}
+template <typename T16>
+__device__ inline uint2 load4_any_bits(const T16* row, int v, int V) {
+  if (v + 4 <= V) {
+    const uint2_align2 a = *reinterpret_cast<const uint2_align2*>(row + v);
+    return make_uint2(a.x, a.y);
+  }
+  return make_uint2(
+      (unsigned)row[min(v, V - 1)].bits | ((unsigned)row[min(v + 1, V - 1)].bits << 16),
+      (unsigned)row[min(v + 2, V - 1)].bits | ((unsigned)row[min(v + 3, V - 1)].bits << 16));
+}
+__device__ inline float4 load4_any(const bf16_t* row, int v, int V) {
+  const uint2 w = load4_any_bits(row, v, V);
+  return make_float4(__uint_as_float(w.x << 16), __uint_as_float(w.x & 0xffff0000u),
+                     __uint_as_float(w.y << 16), __uint_as_float(w.y & 0xffff0000u));
+}
+__device__ inline float4 load4_any(const f16_t* row, int v, int V) {
+  const uint2 w = load4_any_bits(row, v, V);
+  return make_float4(f16_to_float((unsigned short)(w.x & 0xffffu)),
+                     f16_to_float((unsigned short)(w.x >> 16)),
+                     f16_to_float((unsigned short)(w.y & 0xffffu)),
+                     f16_to_float((unsigned short)(w.y >> 16)));
+}
+
 // Eight consecutive elements of a row as they sit in registers after the load.
 template <typename T>
 struct Raw8;
@@ -115,8 +154,6 @@ __device__ inline void expand(const Raw8<bf16_t>& r, float (&e)[8]) {
 // inside the row come in as loads of the same width at the element type's own alignment, which
 // global memory serves; the row's last, partial eight are fetched one by one, each index clamped
 // to the row's last element.
-typedef float float4_align4 __attribute__((ext_vector_type(4), aligned(4)));
-typedef unsigned uint4_align2 __attribute__((ext_vector_type(4), aligned(2)));
 __device__ inline Raw8<float> load8_any(const float* row, int v, int V) {
   Raw8<float> r;
   if (v + 8 <= V) {
