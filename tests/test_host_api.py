@@ -153,3 +153,37 @@ def test_setup_script_names_the_package_and_builds_through_the_in_tree_build():
     assert out[0] == "transducer_amd" and out[1][0].isdigit()
     text = open(os.path.join(root, "setup.py")).read()
     assert "build_all()" in text and "check_call" not in text  # no cmake / network step of its own
+
+
+def test_a_cxx_caller_of_the_reference_header_compiles_links_and_sees_its_exceptions(tmp_path):
+    """A translation unit written against the reference's transducer.h (three free functions,
+    C++ linkage, transducer/transducer.h:3-49) builds against include/transducer.h and
+    libtransducer.so with a plain g++ line; the backend that is not built reports
+    std::invalid_argument as transducer/transducer.cpp:41,97,147 do (no device is touched)."""
+    src = tmp_path / "caller.cpp"
+    src.write_text(r'''
+#include <cstdio>
+#include <stdexcept>
+#include <string>
+#include "transducer.h"
+template <typename F> static int refused(F f) {
+  try { f(); } catch (const std::invalid_argument& e) {
+    return std::string(e.what()).find("not built") != std::string::npos ? 1 : 0;
+  }
+  return 0;
+}
+int main() {
+  float x[8] = {0}; int n[2] = {1, 0}; int lab[2] = {0, 0};
+  int ok = 0;
+  ok += refused([&] { forward(x, x, x, x, x, lab, n, n + 1, 1, 1, 1, 2, 0, false); });
+  ok += refused([&] { backward(x, x, x, x, x, x, x, lab, n, n + 1, 1, 1, 1, 2, 0, false); });
+  ok += refused([&] { viterbi(x, x, x, lab, n, n + 1, 1, 1, 1, 2, 0, false); });
+  std::printf("%d\n", ok);
+  return ok == 3 ? 0 : 1;
+}
+''')
+    exe = tmp_path / "caller"
+    subprocess.check_call(["g++", "-std=c++11", "-I", os.path.join(ROOT, "include"), str(src),
+                           "-o", str(exe), "-L", PKG, "-ltransducer", "-lrnnt_hip",
+                           "-Wl,-rpath," + PKG])
+    assert subprocess.check_output([str(exe)], text=True).strip() == "3"
