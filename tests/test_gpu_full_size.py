@@ -98,8 +98,11 @@ def viterbi_on_device(c, LN, blank=0):
 
 
 # ------------------------------------------------------------------ headline configuration
-def test_headline_configuration_properties_and_one_utterance_against_the_oracle():
-    c = DeviceBatch(CONFIGS["cfg4"], seed=3)
+@pytest.mark.parametrize("V", [10000, 10001])
+def test_headline_configuration_properties_and_one_utterance_against_the_oracle(V):
+    """V = 10001: the same at a vocabulary whose rows do not start on 16-byte boundaries (every
+    row of the [B,T,V] arrays then comes in through the loads at the element's own alignment)."""
+    c = DeviceBatch(CONFIGS["cfg4"]._replace(V=V), seed=3)
     B, T, U, V = c.dims
     costs, eg, pg = loss_on_device(c)
     assert torch.isfinite(costs).all() and (costs > 0).all()
@@ -153,9 +156,9 @@ def test_headline_configuration_properties_and_one_utterance_against_the_oracle(
     assert ve <= 0.02 and vp <= 0.02
 
 
-@pytest.mark.parametrize("near_ties", [False, True])
-def test_headline_viterbi_one_utterance_bit_exact_and_batch_independent(near_ties):
-    c = DeviceBatch(CONFIGS["cfg5"], seed=5, near_ties=near_ties)
+@pytest.mark.parametrize("near_ties,V", [(False, 10000), (True, 10000), (True, 10001)])
+def test_headline_viterbi_one_utterance_bit_exact_and_batch_independent(near_ties, V):
+    c = DeviceBatch(CONFIGS["cfg5"]._replace(V=V), seed=5, near_ties=near_ties)
     LN = log_norms_on_device(c)
     paths = viterbi_on_device(c, LN)
     U = c.U
