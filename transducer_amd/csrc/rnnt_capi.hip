@@ -222,22 +222,27 @@ size_t viterbi_scratch_bytes(const Dims& d) {
 
 // `scratch` has viterbi_scratch_bytes(d) left to take (one allocation per call, made by the caller
 // together with whatever else it needs: the allocator calls are a visible part of a small decode).
+// With `ready`, the lattice planes were carved by the caller and already hold LN and the blank
+// scores (the log-normaliser left them there): no transposing copy, no gather.
 template <typename TIO>
 int viterbi_impl(const TIO* E, const TIO* P, const float* LN, int* labels,
                         const int* inLen, const int* labLen, const Dims& d, Scratch& scratch,
-                        hipStream_t s) {
+                        hipStream_t s, const Planes* ready = nullptr) {
   const size_t plane = sizeof(float) * (size_t)d.B * d.Ua * d.Dp + 64;
   Planes p;
-  carve_planes(scratch.take(planes_bytes(d)), d, &p);
+  if (ready) p = *ready;
+  else carve_planes(scratch.take(planes_bytes(d)), d, &p);
   float* bestS = static_cast<float*>(scratch.take(plane));
   float* argS = static_cast<float*>(scratch.take(plane));
   unsigned long long* bits =
       static_cast<unsigned long long*>(scratch.take(viterbi_bits_bytes(d)));
   RNNT_STAGE(kMaxplus, launch_maxplus(E, P, inLen, labLen, bestS, reinterpret_cast<int*>(argS), d,
                                       s));
-  RNNT_STAGE(kSkew, launch_skew(LN, p.lnS, inLen, labLen, d, s));
-  // blank scores only: the label planes of the gather are not needed here
-  RNNT_STAGE(kGather, launch_gather(E, P, nullptr, inLen, labLen, p, d, s));
+  if (!ready) {
+    RNNT_STAGE(kSkew, launch_skew(LN, p.lnS, inLen, labLen, d, s));
+    // blank scores only: the label planes of the gather are not needed here
+    RNNT_STAGE(kGather, launch_gather(E, P, nullptr, inLen, labLen, p, d, s));
+  }
   RNNT_STAGE(kViterbi, launch_viterbi(p, bestS, argS, bits, inLen, labLen, labels, d, s));
   return kOk;
 }
@@ -339,20 +344,24 @@ int lowp_viterbi_decode(const TIO* E, const TIO* P, const int* inLen, const int*
   const Dims d = make_dims(B, T, U, V, blank);
   RNNT_TRY(check_lowp_shape(d, false, who));
   if (!lse_stream_supported(E, d)) return fail(kInvalid, "%s: B*T*U too large", who);
+  if (U > 1024)
+    return fail(kInvalid, "%s: prediction length %d exceeds the supported maximum of 1024", who, U);
   Scratch scratch(s);
-  const size_t btu = sizeof(float) * (size_t)B * T * U;
   const size_t yb = lse_scratch_bytes(d);
   RNNT_TRY(scratch.reserve(align_up(sizeof(float) * (size_t)B * T) +
-                           align_up(sizeof(float) * (size_t)B * U) + align_up(btu) +
-                           align_up(yb) + viterbi_scratch_bytes(d)));
+                           align_up(sizeof(float) * (size_t)B * U) + align_up(yb) +
+                           viterbi_scratch_bytes(d)));
   float* mE = static_cast<float*>(scratch.take(sizeof(float) * (size_t)B * T));
   float* mP = static_cast<float*>(scratch.take(sizeof(float) * (size_t)B * U));
-  float* LN = static_cast<float*>(scratch.take(btu));
   void* ys = scratch.take(yb);
-  RNNT_STAGE(kRowmax, launch_rowmax(P, mP, (long)B * U, V, U, labLen, 1, s));
+  // LN and the blank scores go straight into the lattice planes, as in the whole-loss path
+  Planes p;
+  carve_planes(scratch.take(planes_bytes(d)), d, &p);
+  RNNT_STAGE(kRowmax, launch_rowmax_pick_p(P, mP, nullptr, labLen, p, d, s));
   RNNT_STAGE(kYplanes, launch_yplanes(P, mP, ys, labLen, d, s));
-  RNNT_STAGE(kLse, launch_lse_stream(E, mE, mP, LN, ys, inLen, labLen, d, s));
-  return viterbi_impl(E, P, LN, labels, inLen, labLen, d, scratch, s);
+  RNNT_STAGE(kLse, launch_lse_stream(E, mE, mP, nullptr, ys, inLen, labLen, d, s, nullptr, p.elS,
+                                     p.eb, p.lnS));
+  return viterbi_impl(E, P, nullptr, labels, inLen, labLen, d, scratch, s, &p);
 }
 
 }  // namespace
@@ -627,18 +636,26 @@ int rnnt_hip_viterbi_decode(const float* E, const float* P, const int* inLen, co
     return fail(kInvalid, "viterbi_decode: null array argument");
   hipStream_t s = static_cast<hipStream_t>(stream);
   const Dims d = make_dims(B, T, U, V, blank);
+  if (U > 1024)
+    return fail(kInvalid, "viterbi_decode: prediction length %d exceeds the supported maximum of "
+                          "1024", U);
   Scratch scratch(s);
-  const size_t btu = sizeof(float) * (size_t)B * T * U;
   const size_t yb = lse_stream_supported(E, d) ? lse_scratch_bytes(d) : 0;
   RNNT_TRY(scratch.reserve(align_up(sizeof(float) * (size_t)B * T) +
-                           align_up(sizeof(float) * (size_t)B * U) + align_up(btu) +
-                           align_up(yb) + viterbi_scratch_bytes(d)));
+                           align_up(sizeof(float) * (size_t)B * U) + align_up(yb) +
+                           viterbi_scratch_bytes(d)));
   float* mE = static_cast<float*>(scratch.take(sizeof(float) * (size_t)B * T));
   float* mP = static_cast<float*>(scratch.take(sizeof(float) * (size_t)B * U));
-  float* LN = static_cast<float*>(scratch.take(btu));
   void* ys = yb ? scratch.take(yb) : nullptr;
-  RNNT_TRY(log_norms_stages(E, P, mE, mP, LN, ys, inLen, labLen, d, s));
-  return viterbi_impl(E, P, LN, labels, inLen, labLen, d, scratch, s);
+  // LN and the blank scores go straight into the lattice planes, as in the whole-loss path
+  // (no row-major LN, no transposing copy, no gather)
+  Planes p;
+  carve_planes(scratch.take(planes_bytes(d)), d, &p);
+  bool ln_in_plane = false;
+  RNNT_TRY(log_norms_stages(E, P, mE, mP, nullptr, ys, inLen, labLen, d, s, &p, nullptr,
+                            &ln_in_plane));
+  if (!ln_in_plane) return fail(kInvalid, "viterbi_decode: log-normaliser left no plane");
+  return viterbi_impl(E, P, nullptr, labels, inLen, labLen, d, scratch, s, &p);
 }
 
 }  // extern "C"
