@@ -160,6 +160,47 @@ const char* rnnt_hip_profile_stage_name(int stage);
  * the first n entries of the two HOST arrays, and clears the record. */
 int rnnt_hip_profile_read(double* total_ms, int* launches, int n);
 
+/* ---- diagnostics of the lattice walks (no counterpart in the reference) ------------------ */
+
+/* The alpha and best-path walks deal a long label axis to two wavefronts of a workgroup; the
+ * upper one waits, with a trip bound, for the lower one's progress counter.  Should the bound
+ * ever run out the kernel still finishes, with invalid results, and raises a flag on its
+ * device.  This call waits for `stream`, reads the current device's flag and clears it:
+ * RNNT_OK if no kernel gave up since the last check, else RNNT_HIP_FAILURE with a message.
+ * (The reference's kernels synchronise with __syncthreads and cannot hang this way,
+ * transducer/transducer_cuda.cu:65-90.) */
+int rnnt_hip_check_kernels(rnnt_stream_t stream);
+/* Sets the trip bound (negative: back to the default) and returns the previous one.  For
+ * tests of the give-up path: with 0 the upper wavefront gives up at its first unmet wait. */
+int rnnt_hip_set_spin_limit(int trips);
+
+/* The lattice kernels' expf and log1pf, which restate the C library's (glibc 2.35, the one the
+ * reference's std::exp / std::log1p resolve to, transducer/transducer_cpu.cpp:16-24,124-135) so
+ * that alphas and transition weights carry the reference's bits: expf_out[i] = expf(x[i]),
+ * log1pf_out[i] = log1pf(x[i]) for n device floats (log1pf for x >= 0 only).  For tests that
+ * hold them to the host's library. */
+int rnnt_hip_libm_probe(const float* x, float* expf_out, float* log1pf_out, long n,
+                        rnnt_stream_t stream);
+
+/* The alpha walk forms log(exp(a) + exp(b)) on the hardware exp/log units and keeps that
+ * sum only where it can show that the library's sum rounds to the same float (otherwise the
+ * lane takes the library's algorithm).  The proof rests on a bound of the fast value's distance
+ * from log1pf(expf(d)), d = -|a - b|.  This call checks that bound for EVERY float d whose bit
+ * pattern lies in [lo_bits, hi_bits] (0x80000000 = -0 ... 0xff800000 = -inf; the whole range
+ * takes a fraction of a second) on the current device, synchronously: *violations = patterns
+ * where the bound fails (must be 0), *worst_ratio = largest distance / bound seen. */
+int rnnt_hip_lse_bound_check(unsigned lo_bits, unsigned hi_bits, unsigned long long* violations,
+                             float* worst_ratio);
+
+/* Latency floor of one step of a lattice walk: runs `steps` steps of the bare dependent chain
+ * of one cell (kind 0: alpha -- hand-over, checked fast log-sum-exp with no lane falling back,
+ * the three additions of a move; kind 1: dalpha -- hand-over, two multiplies, an add; kind 2:
+ * kind 0 with every lane on the library's expf/log1pf) on a single wavefront with every operand in
+ * registers, times it with HIP events on the null stream (best of five) and writes nanoseconds
+ * per step to the HOST double.  The measured walks are reported against this floor
+ * (transducer/transducer_cuda.cu:65-90,141-175 are the loops it bounds). */
+int rnnt_hip_chain_floor(int kind, int steps, double* ns_per_step);
+
 #ifdef __cplusplus
 }
 #endif

@@ -104,6 +104,22 @@ def log_norms_truth(E, P, input_lengths=None, label_lengths=None):
     return LN
 
 
+def libm_expf(x):
+    """expf of the host's C library, elementwise (what std::exp(float) is in the reference)."""
+    x = _np(x, np.float32)
+    y = np.empty_like(x)
+    lib().orc_libm_expf(_p(x), _p(y), ctypes.c_long(x.size))
+    return y
+
+
+def libm_log1pf(x):
+    """log1pf of the host's C library, elementwise."""
+    x = _np(x, np.float32)
+    y = np.empty_like(x)
+    lib().orc_libm_log1pf(_p(x), _p(y), ctypes.c_long(x.size))
+    return y
+
+
 def forward(E, P, LN, labels, input_lengths, label_lengths, blank=0, precision="f32"):
     """-> costs[B], alphas[B,T,U] (cells outside the valid region hold NaN)."""
     dt, sfx = _real(precision)

@@ -96,3 +96,15 @@ void orc_best_labels_f32_table(const float* E, const float* P, float* best, int*
       }
   }
 }
+
+/* The C library's expf / log1pf elementwise: what the reference's std::exp / std::log1p resolve
+ * to on floats (transducer/transducer_cpu.cpp:16-24).  The device's restatements of the two are
+ * held to these bit for bit. */
+void orc_libm_expf(const float* x, float* y, long n) {
+#pragma omp parallel for
+  for (long i = 0; i < n; ++i) y[i] = expf(x[i]);
+}
+void orc_libm_log1pf(const float* x, float* y, long n) {
+#pragma omp parallel for
+  for (long i = 0; i < n; ++i) y[i] = log1pf(x[i]);
+}

@@ -9,7 +9,7 @@ import pytest
 
 import oracle
 from transducer_amd.synthetic import CONFIGS, make_inputs, small_config
-from util import (DeviceCase, assert_close, check_close_reference, gpu_backward, gpu_dense_grads,
+from util import (DeviceCase, assert_close, assert_same_bits, check_close_reference, gpu_backward, gpu_dense_grads,
                   gpu_forward, gpu_log_norms, gpu_loss, gpu_viterbi, ref_cases, reference_vectors,
                   vector_case, violations)
 
@@ -79,11 +79,15 @@ def test_boundary_against_reference_fixture(name):
     assert np.array_equal(np.isinf(costs), np.isinf(f["costs"]))
     assert_close(costs, f["costs"], what="costs")
     assert np.array_equal(np.isnan(alphas), np.isnan(f["alphas"])), "cells outside must be untouched"
-    assert_close(alphas, f["alphas"], what="alphas")
-    eg, pg, lng = gpu_backward(c, f["alphas"], LN)
-    assert_close(lng, f["lngrads"], what="lngrads")
-    assert_close(eg, f["egrads_sparse"], what="egrads (sparse)")
-    assert_close(pg, f["pgrads_sparse"], what="pgrads (sparse)")
+    # The lattice kernels use the C library's own expf / log1pf and the reference's order of
+    # operations: with the same log_norms every alpha, every dalpha and every blank / label
+    # term carries the bits the reference's compiled CPU sources produced.
+    assert_same_bits(costs, f["costs"], what="costs")
+    assert_same_bits(alphas, f["alphas"], what="alphas")
+    eg, pg, lng = gpu_backward(c, alphas, LN)
+    assert_same_bits(lng, f["lngrads"], what="lngrads")
+    assert_same_bits(eg, f["egrads_sparse"], what="egrads (sparse)")
+    assert_same_bits(pg, f["pgrads_sparse"], what="pgrads (sparse)")
     if "viterbi" in f:
         got = gpu_viterbi(c, LN)
         assert np.array_equal(got, f["viterbi"])
@@ -144,17 +148,15 @@ def test_boundary_at_T2000(V, sigma, ragged):
     costs_o, alphas_o = oracle.forward(E, P, LN, labels, il, ll)
     c = DeviceCase(E, P, labels, il, ll)
     costs, alphas = gpu_forward(c, LN)
-    m = ~np.isnan(alphas_o)
-    exact = float((alphas[m] == alphas_o[m]).mean())
-    assert exact > 0.95, "alphas bit-exact in only %.3f of cells" % exact
-    assert_close(costs, costs_o, what="costs")
-    assert_close(alphas[m], alphas_o[m], what="alphas")
+    # same expf / log1pf, same order of operations: the same bits in every cell
+    assert_same_bits(costs, costs_o, what="costs")
+    assert_same_bits(alphas, alphas_o, what="alphas")
     # backward from the device's own alphas, as a caller would chain the two calls
     eg, pg, lng = gpu_backward(c, alphas, LN)
     eg_o, pg_o, lng_o = oracle.backward(E, P, np.nan_to_num(alphas_o), LN, labels, il, ll)
-    assert_close(lng, lng_o, what="lngrads")
-    assert_close(eg, eg_o, what="egrads (sparse)")
-    assert_close(pg, pg_o, what="pgrads (sparse)")
+    assert_same_bits(lng, lng_o, what="lngrads")
+    assert_same_bits(eg, eg_o, what="egrads (sparse)")
+    assert_same_bits(pg, pg_o, what="pgrads (sparse)")
     # every path crosses each anti-diagonal exactly once
     for b in range(E.shape[0]):
         Tb, Ub = il[b], ll[b] + 1
@@ -376,6 +378,33 @@ def test_whole_loss_handles_empty_utterance_and_empty_label():
     assert_close(eg, want["egrads"], what="egrads")
     assert_close(pg, want["pgrads"], what="pgrads")
     assert not eg[1].any() and not pg[1].any()
+
+
+@pytest.mark.parametrize("V", [40, 600])
+def test_labels_outside_the_vocabulary_act_as_the_nearest_valid_index(V):
+    """The reference indexes its score rows with whatever the label array holds
+    (transducer_cpu.cpp:63-66), which reads and writes past the row for a value outside [0, V).
+    Every kernel here reads labels through one clamping function, so such a label means column
+    0 or V-1 everywhere: same bits as the clamped labels, in the whole loss (scattered terms
+    below 512 columns, folded ones from there on) and in the three boundary functions."""
+    cfg = small_config(3, 70, 20, V, ragged=True)
+    E, P, labels, il, ll = unpack(make_inputs(cfg, seed=V))
+    il[:] = 70
+    ll[:] = 20
+    bad = labels.copy()
+    bad[0, 3], bad[0, 7], bad[1, 0], bad[2, 19] = -5, V, V + 1000, -(1 << 30)
+    good = np.clip(bad, 0, V - 1)
+    for got, want in zip(gpu_loss(DeviceCase(E, P, bad, il, ll)),
+                         gpu_loss(DeviceCase(E, P, good, il, ll))):
+        assert np.array_equal(got, want)
+    LN = oracle.log_norms_naive(E, P, il, ll)
+    cb, cg = DeviceCase(E, P, bad, il, ll), DeviceCase(E, P, good, il, ll)
+    (costs_b, alphas_b), (costs_g, alphas_g) = gpu_forward(cb, LN), gpu_forward(cg, LN)
+    assert np.array_equal(costs_b, costs_g) and np.array_equal(alphas_b, alphas_g)
+    for got, want in zip(gpu_backward(cb, alphas_g, LN), gpu_backward(cg, alphas_g, LN)):
+        assert np.array_equal(got, want)
+    want = oracle.loss_and_grads(E, P, good, il, ll)
+    assert_close(costs_g, want["costs"], what="costs")
 
 
 def test_whole_loss_at_T2000_violation_fraction():

@@ -57,6 +57,40 @@ def test_bad_sizes_are_rejected_before_any_device_work():
     assert lib.rnnt_hip_loss_workspace_bytes(32, 2000, 101, 10000) < 600 * 2**20
 
 
+def test_blank_outside_the_vocabulary_is_refused_by_every_entry_point_that_takes_one():
+    """The reference indexes rows with `blank` unchecked (transducer_cpu.cpp:46,96); here a blank
+    outside [0, V) is an argument error, reported before any pointer is looked at."""
+    from transducer_amd import capi
+    lib = capi.load()
+    n = None
+    for blank in (-1, 7, 1 << 20):
+        calls = [
+            lib.rnnt_hip_forward(n, n, n, n, n, n, n, n, 2, 5, 3, 7, blank, n),
+            lib.rnnt_hip_backward(n, n, n, n, n, n, n, n, n, n, 2, 5, 3, 7, blank, n),
+            lib.rnnt_hip_viterbi(n, n, n, n, n, n, 2, 5, 3, 7, blank, n),
+            lib.rnnt_hip_loss_forward(n, n, n, n, n, n, n, 0, 2, 5, 3, 7, blank, n),
+            lib.rnnt_hip_loss_backward(n, n, n, n, n, n, n, n, n, 0, 2, 5, 3, 7, blank, n),
+            lib.rnnt_hip_viterbi_decode(n, n, n, n, n, 2, 5, 3, 7, blank, n),
+            lib.rnnt_hip_loss_forward_bf16(n, n, n, n, n, n, n, 0, 2, 5, 3, 7, blank, n),
+            lib.rnnt_hip_loss_backward_f16(n, n, n, n, n, n, n, n, n, 0, 2, 5, 3, 7, blank, n),
+            lib.rnnt_hip_viterbi_decode_bf16(n, n, n, n, n, 2, 5, 3, 7, blank, n),
+        ]
+        assert calls == [1] * len(calls), (blank, calls)
+        assert b"blank index" in lib.rnnt_hip_last_error()
+    # the last valid index passes this check (and then fails on the null pointers instead)
+    assert lib.rnnt_hip_forward(n, n, n, n, n, n, n, n, 2, 5, 3, 7, 6, n) == 1
+    assert b"blank index" not in lib.rnnt_hip_last_error()
+
+
+def test_front_end_refuses_a_blank_outside_the_vocabulary():
+    from transducer_amd import torch_binding
+    with pytest.raises(ValueError, match="blank must lie in"):
+        torch_binding._check_blank(5, 5)
+    with pytest.raises(ValueError, match="blank must lie in"):
+        torch_binding._check_blank(-1, 5)
+    torch_binding._check_blank(4, 5)
+
+
 def test_workspace_has_no_BTV_or_BTUV_term():
     """O(B*T*U) lattice planes plus one O(B*U*V) entry (the pieces of exp(P - mP), 6 bytes per
     element of predictions with U rounded up to 32): growing V by dV adds exactly that much, for

@@ -61,6 +61,17 @@ def assert_close(got, want, rtol=RTOL, atol=ATOL, what=""):
         what, 100 * frac, rtol, atol, worst)
 
 
+def assert_same_bits(got, want, what=""):
+    """Bit for bit, NaN patterns included (cells the library must leave untouched hold the NaN
+    they were filled with on both sides)."""
+    got = np.ascontiguousarray(got, np.float32).view(np.uint32)
+    want = np.ascontiguousarray(want, np.float32).view(np.uint32)
+    both_nan = np.isnan(got.view(np.float32)) & np.isnan(want.view(np.float32))
+    diff = (got != want) & ~both_nan
+    assert not diff.any(), "%s: %d of %d entries differ in their bits (%.4g%%)" % (
+        what, int(diff.sum()), diff.size, 100.0 * diff.mean())
+
+
 def check_close_reference(a, b, rtol=1e-6, atol=1e-5):
     """The reference's own comparison (transducer/test.h:19-29): threshold
     max(rtol*max(|a|,|b|), atol), infinities must match exactly."""

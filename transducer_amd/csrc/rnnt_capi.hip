@@ -2,6 +2,9 @@
 // stream-ordered scratch, and the kernel sequences.  No torch types, no exceptions.
 #include <stdarg.h>
 #include <stdio.h>
+#include <string.h>
+
+#include <mutex>
 
 #include "../../include/rnnt_hip.h"
 #include "rnnt_internal.h"
@@ -75,16 +78,28 @@ namespace {
 
 size_t align_up(size_t x) { return (x + 255) & ~(size_t)255; }
 
-// One stream-ordered allocation carved into pieces; released on the same stream.
+// Device scratch of one call, carved into pieces.  Either one stream-ordered allocation,
+// released on the same stream when the call returns, or a fixed region that the caller of the
+// constructor owns (the static array of the entry point that allocates nothing).
 class Scratch {
  public:
   explicit Scratch(hipStream_t s) : stream_(s) {}
+  Scratch(void* fixed, size_t capacity, const char* who)
+      : stream_(nullptr), fixed_(fixed), capacity_(capacity), who_(who) {}
   ~Scratch() {
-    if (base_) (void)hipFreeAsync(base_, stream_);
+    if (base_ && !fixed_) (void)hipFreeAsync(base_, stream_);
   }
   int reserve(size_t bytes) {
     if (bytes == 0) return kOk;
-    RNNT_HIP(hipMallocAsync(&base_, bytes, stream_));
+    if (fixed_) {
+      if (bytes > capacity_)
+        return fail(kWorkspace, "%s: this problem needs %zu bytes of scratch, the built-in "
+                                "array holds %zu; use the allocating entry point", who_, bytes,
+                    capacity_);
+      base_ = fixed_;
+    } else {
+      RNNT_HIP(hipMallocAsync(&base_, bytes, stream_));
+    }
     size_ = bytes;
     return kOk;
   }
@@ -98,6 +113,9 @@ class Scratch {
 
  private:
   hipStream_t stream_;
+  void* fixed_ = nullptr;
+  size_t capacity_ = 0;
+  const char* who_ = "";
   void* base_ = nullptr;
   size_t size_ = 0, used_ = 0;
 };
@@ -108,6 +126,14 @@ int check_dims(int B, int T, int U, int V) {
   if ((long long)T * V >= (1ll << 31) || (long long)U * V >= (1ll << 31) ||
       (long long)T * U >= (1ll << 31))
     return fail(kInvalid, "one utterance's T*V, U*V or T*U exceeds 2^31 elements");
+  return kOk;
+}
+
+// The reference indexes rows with `blank` unchecked (transducer/transducer_cpu.cpp:46,96); a
+// value outside the vocabulary would read and write past every row, so it is refused here.
+int check_blank(int V, int blank) {
+  if (V > 0 && (blank < 0 || blank >= V))
+    return fail(kInvalid, "blank index %d outside the vocabulary [0, %d)", blank, V);
   return kOk;
 }
 
@@ -261,6 +287,7 @@ int lowp_loss_forward(const TIO* E, const TIO* P, const int* labels, const int* 
                       int B, int T, int U, int V, int blank, rnnt_stream_t stream,
                       const char* who) {
   RNNT_TRY(check_dims(B, T, U, V));
+  RNNT_TRY(check_blank(V, blank));
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (B == 0) return kOk;
   if (!costs || !inLen || !labLen) return fail(kInvalid, "%s: null costs or lengths", who);
@@ -291,6 +318,7 @@ int lowp_loss_backward(const TIO* E, const TIO* P, const int* labels, const int*
                        void* workspace, size_t workspace_bytes, int B, int T, int U, int V,
                        int blank, rnnt_stream_t stream, const char* who) {
   RNNT_TRY(check_dims(B, T, U, V));
+  RNNT_TRY(check_blank(V, blank));
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (B == 0 || V == 0) return kOk;
   if (nothing_to_do(B, T, U)) {
@@ -336,6 +364,7 @@ int lowp_viterbi_decode(const TIO* E, const TIO* P, const int* inLen, const int*
                         int* labels, int B, int T, int U, int V, int blank, rnnt_stream_t stream,
                         const char* who) {
   RNNT_TRY(check_dims(B, T, U, V));
+  RNNT_TRY(check_blank(V, blank));
   if (nothing_to_do(B, T, U) || U == 1) return kOk;  // no label to emit
   if (V == 0) return fail(kInvalid, "%s: empty vocabulary", who);
   if (!E || !P || !labels || !inLen || !labLen)
@@ -361,6 +390,38 @@ int lowp_viterbi_decode(const TIO* E, const TIO* P, const int* inLen, const int*
   RNNT_STAGE(kYplanes, launch_yplanes(P, mP, ys, labLen, d, s));
   RNNT_STAGE(kLse, launch_lse_stream(E, mE, mP, nullptr, ys, inLen, labLen, d, s, nullptr, p.elS,
                                      p.eb, p.lnS));
+  return viterbi_impl(E, P, nullptr, labels, inLen, labLen, d, scratch, s, &p);
+}
+
+// The best-path decode on fp32 scores; `scratch` decides where its device scratch comes from.
+int decode_fp32(const float* E, const float* P, const int* inLen, const int* labLen, int* labels,
+                int B, int T, int U, int V, int blank, hipStream_t s, Scratch& scratch,
+                const char* who) {
+  RNNT_TRY(check_dims(B, T, U, V));
+  RNNT_TRY(check_blank(V, blank));
+  if (nothing_to_do(B, T, U) || U == 1) return kOk;
+  if (V == 0) return fail(kInvalid, "%s: empty vocabulary", who);
+  if (!E || !P || !labels || !inLen || !labLen)
+    return fail(kInvalid, "%s: null array argument", who);
+  const Dims d = make_dims(B, T, U, V, blank);
+  if (U > 1024)
+    return fail(kInvalid, "%s: prediction length %d exceeds the supported maximum of 1024", who, U);
+  if (!lse_stream_supported(E, d)) return fail(kInvalid, "%s: B*T*U too large", who);
+  const size_t yb = lse_scratch_bytes(d);
+  RNNT_TRY(scratch.reserve(align_up(sizeof(float) * (size_t)B * T) +
+                           align_up(sizeof(float) * (size_t)B * U) + align_up(yb) +
+                           viterbi_scratch_bytes(d)));
+  float* mE = static_cast<float*>(scratch.take(sizeof(float) * (size_t)B * T));
+  float* mP = static_cast<float*>(scratch.take(sizeof(float) * (size_t)B * U));
+  void* ys = scratch.take(yb);
+  // LN and the blank scores go straight into the lattice planes, as in the whole-loss path
+  // (no row-major LN, no transposing copy, no gather)
+  Planes p;
+  carve_planes(scratch.take(planes_bytes(d)), d, &p);
+  bool ln_in_plane = false;
+  RNNT_TRY(log_norms_stages(E, P, mE, mP, nullptr, ys, inLen, labLen, d, s, &p, nullptr,
+                            &ln_in_plane));
+  if (!ln_in_plane) return fail(kInvalid, "%s: log-normaliser left no plane", who);
   return viterbi_impl(E, P, nullptr, labels, inLen, labLen, d, scratch, s, &p);
 }
 
@@ -396,10 +457,83 @@ int rnnt_hip_profile_read(double* total_ms, int* launches, int n) {
   return kOk;
 }
 
+int rnnt_hip_check_kernels(rnnt_stream_t stream) {
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  int* flag = nullptr;
+  RNNT_TRY(trouble_flag(&flag));
+  RNNT_HIP(hipStreamSynchronize(s));
+  int raised = 0;
+  RNNT_HIP(hipMemcpy(&raised, flag, sizeof(int), hipMemcpyDeviceToHost));
+  if (raised == 0) return kOk;
+  raised = 0;
+  RNNT_HIP(hipMemcpy(flag, &raised, sizeof(int), hipMemcpyHostToDevice));
+  return fail(kHipError, "a lattice kernel gave up waiting for its neighbouring wavefront's "
+                         "progress (alpha or viterbi hand-over); results of the calls since the "
+                         "last check are not valid");
+}
+
+int rnnt_hip_set_spin_limit(int trips) {
+  const int before = g_spin_limit;
+  g_spin_limit = trips < 0 ? kDefaultSpinLimit : trips;
+  return before;
+}
+
+int rnnt_hip_libm_probe(const float* x, float* expf_out, float* log1pf_out, long n,
+                        rnnt_stream_t stream) {
+  if (n < 0 || (n > 0 && (!x || !expf_out || !log1pf_out)))
+    return fail(kInvalid, "libm_probe: null array argument");
+  return launch_libm_probe(x, expf_out, log1pf_out, n, static_cast<hipStream_t>(stream));
+}
+
+int rnnt_hip_lse_bound_check(unsigned lo_bits, unsigned hi_bits, unsigned long long* violations,
+                             float* worst_ratio) {
+  if (lo_bits > hi_bits || lo_bits < 0x80000000u || hi_bits > 0xff800000u || !violations ||
+      !worst_ratio)
+    return fail(kInvalid, "lse_bound_check: bit patterns must name floats in [-inf, -0]");
+  int* words = nullptr;
+  RNNT_TRY(trouble_flag(&words));
+  unsigned* out = reinterpret_cast<unsigned*>(words + 32);  // two spare words of the flag array
+  const unsigned zero[2] = {0u, 0u};
+  RNNT_HIP(hipMemcpy(out, zero, sizeof(zero), hipMemcpyHostToDevice));
+  RNNT_TRY(launch_lse_bound_check(lo_bits, hi_bits, out, nullptr));
+  unsigned got[2];
+  RNNT_HIP(hipMemcpy(got, out, sizeof(got), hipMemcpyDeviceToHost));
+  *violations = got[0];
+  float ratio;
+  memcpy(&ratio, &got[1], sizeof(ratio));
+  *worst_ratio = ratio;
+  return kOk;
+}
+
+int rnnt_hip_chain_floor(int kind, int steps, double* ns_per_step) {
+  if (kind < 0 || kind > 2 || steps < 1 || !ns_per_step)
+    return fail(kInvalid, "chain_floor: kind must be 0, 1 or 2, steps positive, result non-null");
+  hipEvent_t t0, t1;
+  RNNT_HIP(hipEventCreate(&t0));
+  RNNT_HIP(hipEventCreate(&t1));
+  int st = launch_chain_floor(kind, steps, nullptr);  // warm-up (code object, clocks)
+  float best = 0.0f;
+  for (int rep = 0; st == kOk && rep < 5; ++rep) {
+    (void)hipEventRecord(t0, nullptr);
+    st = launch_chain_floor(kind, steps, nullptr);
+    (void)hipEventRecord(t1, nullptr);
+    if (st == kOk) st = check_hip(hipEventSynchronize(t1), "hipEventSynchronize", __FILE__, __LINE__);
+    float ms = 0.0f;
+    if (st == kOk) st = check_hip(hipEventElapsedTime(&ms, t0, t1), "hipEventElapsedTime", __FILE__, __LINE__);
+    if (rep == 0 || ms < best) best = ms;
+  }
+  (void)hipEventDestroy(t0);
+  (void)hipEventDestroy(t1);
+  if (st != kOk) return st;
+  *ns_per_step = 1.0e6 * best / steps;
+  return kOk;
+}
+
 int rnnt_hip_forward(const float* E, const float* P, float* costs, float* alphas, const float* LN,
                      const int* labels, const int* inLen, const int* labLen, int B, int T, int U,
                      int V, int blank, rnnt_stream_t stream) {
   RNNT_TRY(check_dims(B, T, U, V));
+  RNNT_TRY(check_blank(V, blank));
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (B == 0) return kOk;
   if (!costs || !inLen || !labLen) return fail(kInvalid, "forward: null costs or lengths");
@@ -423,6 +557,7 @@ int rnnt_hip_backward(const float* E, const float* P, float* egrads, float* pgra
                       const int* labLen, int B, int T, int U, int V, int blank,
                       rnnt_stream_t stream) {
   RNNT_TRY(check_dims(B, T, U, V));
+  RNNT_TRY(check_blank(V, blank));
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (B == 0) return kOk;
   // transducer_cuda.cu:326-331: the library clears all three outputs itself
@@ -455,6 +590,7 @@ int rnnt_hip_viterbi(const float* E, const float* P, const float* LN, int* label
                      const int* inLen, const int* labLen, int B, int T, int U, int V, int blank,
                      rnnt_stream_t stream) {
   RNNT_TRY(check_dims(B, T, U, V));
+  RNNT_TRY(check_blank(V, blank));
   if (nothing_to_do(B, T, U) || U == 1) return kOk;  // no label to emit
   if (!E || !P || !LN || !labels || !inLen || !labLen)
     return fail(kInvalid, "viterbi: null array argument");
@@ -523,6 +659,7 @@ int rnnt_hip_loss_forward(const float* E, const float* P, const int* labels, con
                           const int* labLen, float* costs, void* workspace, size_t workspace_bytes,
                           int B, int T, int U, int V, int blank, rnnt_stream_t stream) {
   RNNT_TRY(check_dims(B, T, U, V));
+  RNNT_TRY(check_blank(V, blank));
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (B == 0) return kOk;
   if (!costs || !inLen || !labLen) return fail(kInvalid, "loss_forward: null costs or lengths");
@@ -550,6 +687,7 @@ int rnnt_hip_loss_backward(const float* E, const float* P, const int* labels, co
                            void* workspace, size_t workspace_bytes, int B, int T, int U, int V,
                            int blank, rnnt_stream_t stream) {
   RNNT_TRY(check_dims(B, T, U, V));
+  RNNT_TRY(check_blank(V, blank));
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (B == 0 || V == 0) return kOk;
   if (nothing_to_do(B, T, U)) {
@@ -629,33 +767,9 @@ RNNT_LOWP_ENTRY_POINTS(f16, f16_t)
 int rnnt_hip_viterbi_decode(const float* E, const float* P, const int* inLen, const int* labLen,
                             int* labels, int B, int T, int U, int V, int blank,
                             rnnt_stream_t stream) {
-  RNNT_TRY(check_dims(B, T, U, V));
-  if (nothing_to_do(B, T, U) || U == 1) return kOk;
-  if (V == 0) return fail(kInvalid, "viterbi_decode: empty vocabulary");
-  if (!E || !P || !labels || !inLen || !labLen)
-    return fail(kInvalid, "viterbi_decode: null array argument");
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const Dims d = make_dims(B, T, U, V, blank);
-  if (U > 1024)
-    return fail(kInvalid, "viterbi_decode: prediction length %d exceeds the supported maximum of "
-                          "1024", U);
   Scratch scratch(s);
-  const size_t yb = lse_stream_supported(E, d) ? lse_scratch_bytes(d) : 0;
-  RNNT_TRY(scratch.reserve(align_up(sizeof(float) * (size_t)B * T) +
-                           align_up(sizeof(float) * (size_t)B * U) + align_up(yb) +
-                           viterbi_scratch_bytes(d)));
-  float* mE = static_cast<float*>(scratch.take(sizeof(float) * (size_t)B * T));
-  float* mP = static_cast<float*>(scratch.take(sizeof(float) * (size_t)B * U));
-  void* ys = yb ? scratch.take(yb) : nullptr;
-  // LN and the blank scores go straight into the lattice planes, as in the whole-loss path
-  // (no row-major LN, no transposing copy, no gather)
-  Planes p;
-  carve_planes(scratch.take(planes_bytes(d)), d, &p);
-  bool ln_in_plane = false;
-  RNNT_TRY(log_norms_stages(E, P, mE, mP, nullptr, ys, inLen, labLen, d, s, &p, nullptr,
-                            &ln_in_plane));
-  if (!ln_in_plane) return fail(kInvalid, "viterbi_decode: log-normaliser left no plane");
-  return viterbi_impl(E, P, nullptr, labels, inLen, labLen, d, scratch, s, &p);
+  return decode_fp32(E, P, inLen, labLen, labels, B, T, U, V, blank, s, scratch, "viterbi_decode");
 }
 
 }  // extern "C"

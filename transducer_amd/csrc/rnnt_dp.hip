@@ -12,7 +12,10 @@
 // Operands are read from "skewed" planes [u][t+u] so that four steps are one 16-byte load per
 // lane, prefetched a group ahead.  This file is compiled with -ffp-contract=off: the rounding
 // sequence of every cell must equal the reference's.
+#include <mutex>
+
 #include "rnnt_internal.h"
+#include "rnnt_libm.h"
 
 namespace rnnt {
 
@@ -48,13 +51,91 @@ __device__ inline float log1p_unit(float y) {
   return log_1to2(w) + lost * __builtin_amdgcn_rcpf(w);
 }
 
-// transducer/transducer_cpu.cpp:16-24
+// log1p(exp(d)) for d <= 0 on the hardware transcendental units: within a few ulp of the C
+// library's value at a seventh of its instructions.
+__device__ inline float softplus_fast(float d) { return log1p_unit(exp_neg(d)); }
+
+// Bound on |softplus_fast(d) - log1pf(expf(d))| (the library's floats) as a function of the fast
+// value lf: lf * (kFastRelA + kFastRelB * |d|) + 2^-125.  The first term covers the rounding of both
+// evaluations (a few ulp of lf), the second the rounding of d * log2(e) ahead of v_exp_f32,
+// whose effect on the result grows with |d|.  The bound is not taken from data sheets: the
+// fast value is compared with the exact one for EVERY float d <= 0 (rnnt_hip_lse_bound_check,
+// run by the tests), where it holds with a factor of two to spare.
+constexpr float kFastRelA = 5.0f * 0x1p-23f;
+constexpr float kFastRelB = 1.25f * 0x1p-23f;
+// The bound for fast value lf at argument d.  The clamp keeps 0 * inf out of it at d = -inf;
+// the added 2^-125 covers d below -87.3, where the library's value is a subnormal number and
+// the hardware units return 0.
+__device__ inline float fast_bound(float lf, float d) {
+  return __builtin_fmaf(lf, __builtin_fmaf(-kFastRelB, fmaxf(d, -256.0f), kFastRelA), 0x1p-125f);
+}
+
+// transducer/transducer_cpu.cpp:16-24 with the C library's own expf and log1pf (rnnt_libm.h):
+// the same bits as the reference's CPU backend for every pair of operands.
+__device__ inline float lse2_libm(float a, float b, const unsigned long long* tab) {
+  // One operand -inf: |a - b| = inf, expf gives 0, log1pf(0) = 0 and the sum is the other
+  // operand exactly, as the reference's early returns have it; only both -inf needs a guard.
+  const float hi = a > b ? a : b;
+  const float r = hi + log1pf_glibc(expf_glibc_nonpositive(-fabsf(a - b), tab));
+  return (hi == kNegInf) ? kNegInf : r;
+}
+
+// The same bits, mostly without the library's ~100 instructions.  What the recursion keeps is
+// r = fl(hi + l) with l = log1pf(expf(d)) at most log 2, and from a few hundred steps into a
+// lattice |hi| is in the thousands: the sum's spacing is then thousands of times the
+// uncertainty of a fast l, so nearly every fast sum is provably the library's sum.  Per lane:
+//   r = fl(hi + lf), t = (hi + lf) - r exactly (Fast2Sum: |hi| >= 1 > lf);
+//   the library's sum rounds to the same r if |t| + bound(lf) stays below half the spacing of
+//   floats around r (and r is not a power of two, where the spacing below is half as wide).
+// Lanes that cannot show this take the library path; a wavefront skips it when none does
+// (Ziv's strategy).  Either way the result is the library's, bit for bit.
+__device__ inline float lse2_checked(float a, float b, const unsigned long long* tab) {
+  const float hi = a > b ? a : b;
+  const float d = -fabsf(a - b);
+  const float lf = softplus_fast(d);
+  float r = hi + lf;
+  const float t = lf - (r - hi);
+  const float bound = fast_bound(lf, d);
+  const int rb = __float_as_int(r);
+  const float half_spacing = __int_as_float((rb & 0x7f800000) - (24 << 23));
+  const bool safe = (fabsf(t) + bound < half_spacing) && (fabsf(hi) >= 1.0f) &&
+                    ((rb & 0x007fffff) != 0);
+  // Both operands -inf (a cell that has not started): the sum is -inf by the reference's early
+  // return, nothing to show.  NaN operands fail the comparisons and take the library path.
+  if (!safe && hi != kNegInf) r = lse2_libm(a, b, tab);
+  return (hi == kNegInf) ? kNegInf : r;
+}
+
+// The same on the hardware units alone (no check): for the chain-latency probe.
 __device__ inline float lse2(float a, float b) {
   // One operand -inf: |a - b| = inf, exp gives 0, log1p(0) = 0 and the sum is the other operand
   // exactly, as the reference's early returns have it; only both -inf (inf - inf) needs a guard.
   const float hi = fmaxf(a, b);
   const float r = hi + log1p_unit(exp_neg(-fabsf(a - b)));
   return (hi == kNegInf) ? kNegInf : r;
+}
+
+// The wait of an upper wavefront for the progress counter of the one below it (LDS, same
+// workgroup).  The lower wavefront never waits for an upper one, so the counter always gets
+// there; the trip bound only turns a logic slip of a future edit into an error report instead
+// of a hung device: when it runs out the wavefront raises the device's trouble flag, stops
+// waiting for good (returns a count no later `need` exceeds) and finishes its walk on whatever
+// the hand-over array holds.  The host reads the flag with rnnt_hip_check_kernels().
+__device__ inline int bounded_wait(const int* counter, int have, int need, int spin_limit,
+                                   int* __restrict__ trouble) {
+  int spins = 0;
+  while (have < need) {
+    have = __hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    asm volatile("" ::: "memory");
+    if (have < need) {
+      if (spins++ >= spin_limit) {
+        if ((threadIdx.x & 63) == 0) *reinterpret_cast<volatile int*>(trouble) = 1;
+        return 0x7fffffff;
+      }
+      __builtin_amdgcn_s_sleep(1);
+    }
+  }
+  return have;
 }
 
 __device__ inline float f4get(const float4& v, int j) {
@@ -132,7 +213,7 @@ __global__ __launch_bounds__(256) void gather_kernel(const TIO* __restrict__ E,
   utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
   if (u >= Ub) return;
   const bool has_label = labels != nullptr && (u + 1 < Ub);
-  const int l = has_label ? labels[(size_t)b * (d.U - 1) + u] : d.blank;
+  const int l = has_label ? label_at(labels, d, b, u) : d.blank;
   const TIO* Eb = E + (size_t)b * d.T * d.V;
   if (t < Tb) {
     if (has_label) p.elS[plane_row(d, b, u) + t + u] = ldf(Eb + (size_t)t * d.V + l);
@@ -147,10 +228,10 @@ __global__ __launch_bounds__(256) void gather_kernel(const TIO* __restrict__ E,
 
 // ------------------------------------------------------------------ alpha
 // transducer/transducer_cpu.cpp:30-79 (one utterance per wavefront).
-// A cell that has not started yet (t < 0) keeps its -inf hand-over scores, which makes lse2
-// return the other operand untouched -- exactly the reference's first-row / first-column
-// special cases.  Cells past the utterance (t >= T_b, u >= U_b) are computed on whatever the
-// planes hold there and are never read by a valid cell.
+// A cell that has not started yet (t < 0) keeps its -inf hand-over scores, which makes the
+// log-sum-exp return the other operand untouched -- exactly the reference's first-row /
+// first-column special cases.  Cells past the utterance (t >= T_b, u >= U_b) hand -inf on as
+// well and are never read by a valid cell.
 // W > 1: the label positions are dealt to W wavefronts of one workgroup (wavefront w owns
 // positions [64 C w, 64 C (w+1))), because the walk is bound by how fast ONE wavefront issues
 // the ~22 instructions of a cell: a step costs about 30 + 65 C ns.  The only value that crosses
@@ -163,10 +244,12 @@ template <int C, int W>
 __global__ __launch_bounds__(64 * W) void alpha_kernel(Planes p, const int* __restrict__ inLen,
                                                        const int* __restrict__ labLen,
                                                        float* __restrict__ costs, Dims d,
-                                                       int hand_stride) {
+                                                       int hand_stride, int spin_limit,
+                                                       int* __restrict__ trouble) {
   extern __shared__ __attribute__((aligned(16))) float hand[];  // [W-1][hand_stride]: entry s =
                                                                 // score handed to step s
   __shared__ int done[W];          // steps a wavefront has published
+  __shared__ unsigned long long etab[32];  // expf's table (rnnt_libm.h)
   const int b = blockIdx.x, lane = threadIdx.x & 63;
   const int wave = W > 1 ? __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) : 0;
   int Tb, Ub;
@@ -178,11 +261,12 @@ __global__ __launch_bounds__(64 * W) void alpha_kernel(Planes p, const int* __re
   const int nsteps = Tb + Ub - 1;
   const int ngroups = (nsteps + 3) >> 2;
   const int u0 = (wave * 64 + lane) * C;
+  exp2_table_to_lds(etab);
   if (W > 1) {
     if (threadIdx.x < W) done[threadIdx.x] = 0;
     if (threadIdx.x < W - 1) hand[threadIdx.x * hand_stride] = kNegInf;  // nothing enters step 0
-    __syncthreads();
   }
+  __syncthreads();
   float* hand_out = hand + wave * hand_stride;                     // wave < W-1
   const float* hand_in = hand + (wave > 0 ? wave - 1 : 0) * hand_stride;  // wave > 0
   // E[t,blank] for the cells of step s sits at ebp[s - u]; column c at step s = 4g+j reads
@@ -190,11 +274,13 @@ __global__ __launch_bounds__(64 * W) void alpha_kernel(Planes p, const int* __re
   const float* ebl = p.eb + (size_t)b * d.Tp + d.Eo - u0;
 
   float stay[C], emit[C], pbv[C], plv[C];
+  unsigned tlim[C];  // frames of this column: T_b, or 0 for a label position past the utterance
   const float* lnp[C];
   const float* elp[C];
   float* ap[C];
 #pragma unroll
   for (int c = 0; c < C; ++c) {
+    tlim[c] = (u0 + c < Ub) ? (unsigned)Tb : 0u;
     const size_t row = plane_row(d, b, u0 + c);  // u0 + c < Ua always
     lnp[c] = p.lnS + row;
     elp[c] = p.elS + row;
@@ -226,11 +312,7 @@ __global__ __launch_bounds__(64 * W) void alpha_kernel(Planes p, const int* __re
     // LDS serves a wavefront's requests in order, so no hardware fence is needed on either
     // side (a release/acquire pair would also wait for the global prefetches in flight);
     // the empty asm statements only keep the compiler from moving LDS accesses across
-    while (avail < need) {
-      avail = __hip_atomic_load(&done[wave - 1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-      asm volatile("" ::: "memory");
-      if (avail < need) __builtin_amdgcn_s_sleep(1);
-    }
+    avail = bounded_wait(&done[wave - 1], avail, need, spin_limit, trouble);
   };
   auto run_group = [&](int g, const Group& cur) {
     float4 aout[C];
@@ -249,7 +331,7 @@ __global__ __launch_bounds__(64 * W) void alpha_kernel(Planes p, const int* __re
 #pragma unroll
         for (int c = C - 1; c >= 0; --c) {
           const float left = (c == 0) ? from_left : emit[c - 1];
-          float a = lse2(left, stay[c]);
+          float a = lse2_checked(left, stay[c], etab);
           if (j == 0 && g == 0) a = (u0 + c == 0) ? 0.0f : a;  // :43
           const float ln = f4get(cur.ln[c], j);
           float sb = a + cur.eb[j - c + (C - 1)];
@@ -258,9 +340,13 @@ __global__ __launch_bounds__(64 * W) void alpha_kernel(Planes p, const int* __re
           float se = a + f4get(cur.el[c], j);
           se = se + plv[c];
           se = se - ln;
-          const bool started = s >= u0 + c;
-          stay[c] = started ? sb : kNegInf;
-          emit[c] = started ? se : kNegInf;
+          // a cell of the lattice: 0 <= t = s - u < T_b (one unsigned comparison).  Cells before
+          // the first frame or past the last one hand -inf on, so whatever the planes hold
+          // outside the utterance never enters a log-sum-exp (where it would cost the whole
+          // wavefront the library path).
+          const bool inside = (unsigned)(s - (u0 + c)) < tlim[c];
+          stay[c] = inside ? sb : kNegInf;
+          emit[c] = inside ? se : kNegInf;
           f4set(aout[c], j, a);
         }
       }
@@ -306,6 +392,9 @@ __global__ __launch_bounds__(64 * W) void alpha_kernel(Planes p, const int* __re
 // recursion below needs no bounds of its own.
 __global__ __launch_bounds__(256) void weights_kernel(Planes p, const int* __restrict__ inLen,
                                                       const int* __restrict__ labLen, Dims d) {
+  __shared__ unsigned long long etab[32];  // expf's table (rnnt_libm.h)
+  exp2_table_to_lds(etab);
+  __syncthreads();
   const int b = blockIdx.z, u = blockIdx.y;
   const int dg = blockIdx.x * 256 + threadIdx.x;
   if (dg >= d.Dp) return;
@@ -321,14 +410,14 @@ __global__ __launch_bounds__(256) void weights_kernel(Planes p, const int* __res
       x = x + p.pb[(size_t)b * d.Ua + u];
       x = x - ln;
       x = x - p.aS[o + 1];
-      wb = expf(x);
+      wb = expf_glibc(x, etab);
     }
     if (u + 1 < Ub) {
       float x = a + p.elS[o];
       x = x + p.pl[(size_t)b * d.Ua + u];
       x = x - ln;
       x = x - p.aS[o + d.Dp + 1];
-      we = expf(x);
+      we = expf_glibc(x, etab);
     }
   }
   p.wB[o] = wb;
@@ -369,7 +458,7 @@ __global__ __launch_bounds__(64) void beta_kernel(Planes p, const int* __restric
     dcol[c] = (u == Ub - 1) ? 1.0f : 0.0f;   // :95
     accB[c] = (u == Ub - 1) ? -1.0f : 0.0f;  // :97
     accL[c] = 0.0f;
-    fold[c] = (u + 1 < Ub) && labels[(size_t)b * (d.U - 1) + u] == d.blank;
+    fold[c] = (u + 1 < Ub) && label_at(labels, d, b, u) == d.blank;
   }
 
   struct Group {
@@ -493,7 +582,7 @@ __global__ __launch_bounds__(256) void sparse_e_kernel(Planes p, float* __restri
       if (u >= 0) {
         blank_acc -= cur.ne[k];
         if (u + 1 < Ub) {
-          const int l = lab[u];
+          const int l = clampi(lab[u], 0, d.V - 1);
           // Label columns are updated with no-return hardware adds: nothing waits on them,
           // and since this thread alone touches row t and its requests to one address stay
           // in order, repeated labels still accumulate in the reference's order.
@@ -553,8 +642,7 @@ __global__ __launch_bounds__(64) void sparse_e_rows_kernel(Planes p, float* __re
       if (u >= 0) {  // uniform
         blank_acc -= has_stay ? ne[k] : 0.0f;
         if (u + 1 < Ub) {
-          const int l = clampi(lab[u], 0, d.V - 1);  // a label outside the vocabulary must not
-                                                     // index past the row
+          const int l = clampi(lab[u], 0, d.V - 1);
           if (l == d.blank) blank_acc -= em[k];
           else mine[l] -= em[k];
         }
@@ -615,7 +703,7 @@ __device__ __forceinline__ void blank_sums_block(const Planes& p, float* __restr
     for (int k = 0; k < 8; ++k) {
       acc -= has_stay ? ne[k] : 0.0f;
       const int uu = u - k;
-      if (uu + 1 < Ub && lab[uu] == d.blank) {
+      if (uu + 1 < Ub && clampi(lab[uu], 0, d.V - 1) == d.blank) {
         const size_t o = plane_row(d, b, uu) + t + uu;
         acc -= dS[o + d.Dp + 1] * wE[o];
       }
@@ -625,7 +713,7 @@ __device__ __forceinline__ void blank_sums_block(const Planes& p, float* __restr
     const size_t o = plane_row(d, b, u) + t + u;
     const float ne = dS[o + 1] * wB[o];
     acc -= has_stay ? ne : 0.0f;
-    if (u + 1 < Ub && lab[u] == d.blank) acc -= dS[o + d.Dp + 1] * wE[o];
+    if (u + 1 < Ub && clampi(lab[u], 0, d.V - 1) == d.blank) acc -= dS[o + d.Dp + 1] * wE[o];
   }
   bsum[(size_t)b * d.T + t] = acc;
 }
@@ -701,7 +789,7 @@ __global__ __launch_bounds__(256) void sparse_p_kernel(Planes p, float* __restri
   float* row = pgrads + ((size_t)b * d.U + u) * d.V;
   const float gb = p.gB[(size_t)b * d.Ua + u], gl = p.gL[(size_t)b * d.Ua + u];
   const bool has_label = u + 1 < Ub;
-  const int l = has_label ? labels[(size_t)b * (d.U - 1) + u] : d.blank;
+  const int l = has_label ? label_at(labels, d, b, u) : d.blank;
   if (add) {
     const float sc = scale ? scale[b] : 1.0f;
     row[d.blank] += sc * gb;
@@ -914,7 +1002,8 @@ __global__ __launch_bounds__(64 * W) void viterbi_kernel(Planes p, const float* 
                                                          const int* __restrict__ labLen,
                                                          unsigned* __restrict__ gcols,
                                                          int* __restrict__ labels_out, Dims d,
-                                                         int hand_stride, int nw) {
+                                                         int hand_stride, int nw, int spin_limit,
+                                                         int* __restrict__ trouble) {
   extern __shared__ __attribute__((aligned(16))) int dyn[];
   __shared__ int done[W];  // steps a wavefront has published
   const int b = blockIdx.x, lane = threadIdx.x & 63, tidx = threadIdx.x;
@@ -974,11 +1063,7 @@ __global__ __launch_bounds__(64 * W) void viterbi_kernel(Planes p, const float* 
   };
   int avail = 0;  // steps the wavefront below is known to have published (see alpha_kernel)
   auto wait_for = [&](int need) {
-    while (avail < need) {
-      avail = __hip_atomic_load(&done[wave - 1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-      asm volatile("" ::: "memory");
-      if (avail < need) __builtin_amdgcn_s_sleep(1);
-    }
+    avail = bounded_wait(&done[wave - 1], avail, need, spin_limit, trouble);
   };
   // A cell that has not started (t < 0) keeps -inf scores and never takes a label; cells past
   // the utterance run on whatever the planes hold and are never consulted by the backtrace.
@@ -1069,11 +1154,162 @@ __global__ __launch_bounds__(64 * W) void viterbi_kernel(Planes p, const float* 
   const int* argI = reinterpret_cast<const int*>(argS);
   for (int u1 = tidx; u1 < Ub - 1; u1 += 64 * W) {
     const int st = taken[u1];
-    if (st >= 0) out[u1] = argI[plane_row(d, b, u1) + st - 1];
+    // (a label is never taken at step 0 on a lattice that was walked; the clamp keeps the read
+    // inside the plane whatever the decision bits hold)
+    if (st >= 0) out[u1] = argI[plane_row(d, b, u1) + max(st - 1, 0)];
   }
 }
 
+// ------------------------------------------------------------------ chain-latency floor
+// What ONE step of a lattice walk costs when nothing but its dependent chain is left: operands
+// in registers, no loads, no stores, no bookkeeping, one wavefront alone on its SIMD.
+//   kind 0: a cell of alpha_kernel -- DPP hand-over, log-sum-exp on the hardware units with
+//           the check that its sum is the C library's (lse2_checked; the operands are large, so
+//           no lane falls back), then the three additions of a move;
+//   kind 1: a cell of beta_kernel -- DPP hand-over, two multiplies and an add;
+//   kind 2: kind 0 with every lane on the library path (rnnt_libm.h: ~100 instructions, two of
+//           them divisions): what a step costs while any lane of the wavefront falls back.
+// The walks cannot run faster than steps x this; the ratio is what the prefetch, the stores and
+// the second wavefront's hand-over cost on top.
+template <int kKind>
+__global__ __launch_bounds__(64) void chain_floor_kernel(float* __restrict__ sink, int steps,
+                                                         float e, float p, float ln, float w) {
+  __shared__ unsigned long long etab[32];
+  exp2_table_to_lds(etab);
+  __syncthreads();
+  const int lane = threadIdx.x;
+  float stay = -5000.0f - 0.37f * lane, emit = -5000.0f - 0.61f * lane, dcol = 1.0f / (1 + lane);
+#pragma unroll 4
+  for (int s = 0; s < steps; ++s) {
+    if (kKind != 1) {
+      const float left = wave_shr1(emit, kNegInf);
+      const float a = kKind == 0 ? lse2_checked(left, stay, etab) : lse2_libm(left, stay, etab);
+      float sb = a + e;
+      sb = sb + p;
+      sb = sb - ln;
+      float se = a + p;
+      se = se + e;
+      se = se - ln;
+      stay = sb;
+      emit = se;
+    } else {
+      const float right = wave_shl1(dcol, 0.0f);
+      const float ne = dcol * w;
+      const float em = right * w;
+      dcol = ne + em;
+    }
+  }
+  sink[lane] = kKind != 1 ? stay + emit : dcol;
+}
+
 }  // namespace
+
+namespace {
+// The two library functions applied elementwise, for the tests that hold them to the host's C
+// library bit for bit.
+__global__ __launch_bounds__(256) void libm_probe_kernel(const float* __restrict__ x,
+                                                         float* __restrict__ e,
+                                                         float* __restrict__ l, long n) {
+  __shared__ unsigned long long etab[32];
+  exp2_table_to_lds(etab);
+  __syncthreads();
+  const long i = (long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  e[i] = expf_glibc(x[i], etab);
+  l[i] = log1pf_glibc(x[i]);
+}
+}  // namespace
+
+namespace {
+// For every float d with bit pattern in [lo, hi] (d <= 0): does the bound of lse2_checked cover
+// the distance between the fast and the library value of log1p(exp(d))?  out[0] counts the
+// patterns where it does not, out[1] keeps the largest ratio distance / bound (as float bits;
+// ratios are non-negative, so their bit patterns order like integers).
+__global__ __launch_bounds__(256) void lse_bound_kernel(unsigned lo, unsigned hi,
+                                                        unsigned* __restrict__ out) {
+  __shared__ unsigned long long etab[32];
+  exp2_table_to_lds(etab);
+  __syncthreads();
+  unsigned bad = 0;
+  float worst = 0.0f;
+  const unsigned long long n = (unsigned long long)hi - lo + 1;
+  for (unsigned long long i = (unsigned long long)blockIdx.x * 256 + threadIdx.x; i < n;
+       i += (unsigned long long)gridDim.x * 256) {
+    const float d = __uint_as_float(lo + (unsigned)i);
+    const float exact = log1pf_glibc(expf_glibc_nonpositive(d, etab));
+    const float lf = softplus_fast(d);
+    const float bound = fast_bound(lf, d);
+    const float dist = fabsf(lf - exact);
+    if (!(dist <= bound)) {
+      ++bad;
+    } else if (bound > 0.0f) {
+      worst = fmaxf(worst, dist / bound);
+    }
+  }
+  if (bad) atomicAdd(&out[0], bad);
+  atomicMax(&out[1], __float_as_uint(worst));
+}
+}  // namespace
+
+int launch_lse_bound_check(unsigned lo, unsigned hi, unsigned* out, hipStream_t s) {
+  hipLaunchKernelGGL(lse_bound_kernel, dim3(4096), dim3(256), 0, s, lo, hi, out);
+  hipError_t err = hipGetLastError();
+  if (err != hipSuccess) return check_hip(err, "launch lse_bound_kernel", __FILE__, __LINE__);
+  return kOk;
+}
+
+int launch_libm_probe(const float* x, float* e, float* l, long n, hipStream_t s) {
+  if (n == 0) return kOk;
+  const long blocks = (n + 255) / 256;
+  if (blocks > 0x7fffffffl) return fail(kInvalid, "libm_probe: too many elements");
+  hipLaunchKernelGGL(libm_probe_kernel, dim3((unsigned)blocks), dim3(256), 0, s, x, e, l, n);
+  hipError_t err = hipGetLastError();
+  if (err != hipSuccess) return check_hip(err, "launch libm_probe_kernel", __FILE__, __LINE__);
+  return kOk;
+}
+
+int launch_chain_floor(int kind, int steps, hipStream_t s) {
+  int* words = nullptr;
+  RNNT_TRY(trouble_flag(&words));
+  float* sink = reinterpret_cast<float*>(words + 64);
+  // scores that keep the recursion near zero: a step adds log 2 and takes it off again
+  if (kind == 0)
+    hipLaunchKernelGGL(chain_floor_kernel<0>, dim3(1), dim3(64), 0, s, sink, steps, 0.3f, 0.2f,
+                       0.5f + 0.693147f, 0.5f);
+  else if (kind == 2)
+    hipLaunchKernelGGL(chain_floor_kernel<2>, dim3(1), dim3(64), 0, s, sink, steps, 0.3f, 0.2f,
+                       0.5f + 0.693147f, 0.5f);
+  else
+    hipLaunchKernelGGL(chain_floor_kernel<1>, dim3(1), dim3(64), 0, s, sink, steps, 0.3f, 0.2f,
+                       0.5f, 0.5f);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return check_hip(e, "launch chain_floor_kernel", __FILE__, __LINE__);
+  return kOk;
+}
+
+// ------------------------------------------------------------------ trouble flag
+// One int per device, raised by a lattice kernel whose bounded wait ran out (bounded_wait).  The
+// array's name is a host-side handle, not a device address: the address is looked up once per
+// device, with that device current, and kernels are given that pointer.
+static __device__ int g_trouble_word[128];  // [0]: the flag; [64..127]: sink of the floor probe
+constexpr int kMaxDevices = 64;
+static int* g_trouble_ptr[kMaxDevices];
+static std::mutex g_trouble_mutex;
+int g_spin_limit = kDefaultSpinLimit;
+
+int trouble_flag(int** out) {
+  int dev = 0;
+  RNNT_HIP(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices) return fail(kInvalid, "device index %d not supported", dev);
+  std::lock_guard<std::mutex> lock(g_trouble_mutex);
+  if (g_trouble_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    RNNT_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(g_trouble_word)));
+    g_trouble_ptr[dev] = static_cast<int*>(p);
+  }
+  *out = g_trouble_ptr[dev];
+  return kOk;
+}
 
 // ------------------------------------------------------------------ workspace layout
 static size_t align_up(size_t x) { return (x + 255) & ~(size_t)255; }
@@ -1155,11 +1391,13 @@ int launch_alpha(const Planes& p, const int* inLen, const int* labLen, float* co
   // instruction, and with four wavefronts the CU's vector memory pipeline becomes the limit)
   const int W = (cpl >= 2 && stride * sizeof(float) <= 48 * 1024) ? 2 : 1;
   const size_t lds = W > 1 ? sizeof(float) * (size_t)(W - 1) * stride : 0;
+  int* trouble = nullptr;
+  RNNT_TRY(trouble_flag(&trouble));
   switch (cpl / W * 100 + W) {
 #define CASE(C, W)                                                                          \
   case C * 100 + W:                                                                         \
     hipLaunchKernelGGL((alpha_kernel<C, W>), dim3(d.B), dim3(64 * W), lds, s, p, inLen,    \
-                       labLen, costs, d, stride);                                           \
+                       labLen, costs, d, stride, g_spin_limit, trouble);                    \
     break;
     CASE(1, 1) CASE(2, 1) CASE(4, 1) CASE(8, 1) CASE(16, 1)
     CASE(1, 2) CASE(2, 2) CASE(4, 2) CASE(8, 2)
@@ -1280,15 +1518,19 @@ int launch_viterbi(const Planes& p, const float* bestS, const float* argS,
   const size_t cols_lds = sizeof(unsigned) * (size_t)64 * cpl * nw;
   const bool use_lds = base_lds + cols_lds <= 60 * 1024;
   const size_t lds = base_lds + (use_lds ? cols_lds : 0);
+  int* trouble = nullptr;
+  RNNT_TRY(trouble_flag(&trouble));
   switch (cpl / W * 100 + W) {
 #define CASE(C, W)                                                                             \
   case C * 100 + W:                                                                            \
     if (use_lds)                                                                               \
       hipLaunchKernelGGL((viterbi_kernel<C, W, true>), dim3(d.B), dim3(64 * W), lds, s, p,    \
-                         bestS, argS, inLen, labLen, gcols, labels_out, d, stride, nw);        \
+                         bestS, argS, inLen, labLen, gcols, labels_out, d, stride, nw,         \
+                         g_spin_limit, trouble);                                               \
     else                                                                                       \
       hipLaunchKernelGGL((viterbi_kernel<C, W, false>), dim3(d.B), dim3(64 * W), lds, s, p,   \
-                         bestS, argS, inLen, labLen, gcols, labels_out, d, stride, nw);        \
+                         bestS, argS, inLen, labLen, gcols, labels_out, d, stride, nw,         \
+                         g_spin_limit, trouble);                                               \
     break;
     CASE(1, 1) CASE(2, 1) CASE(4, 1) CASE(8, 1) CASE(16, 1)
     CASE(1, 2) CASE(2, 2) CASE(4, 2) CASE(8, 2)

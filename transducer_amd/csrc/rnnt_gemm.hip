@@ -120,7 +120,7 @@ __global__ __launch_bounds__(256) void rowmax_pick_p_kernel(const TIO* __restric
     mP[row] = m;
     const bool has_label = labels != nullptr && (u + 1 < Ub);
     p.pb[(size_t)b * d.Ua + u] = ldf(x + d.blank);
-    p.pl[(size_t)b * d.Ua + u] = has_label ? ldf(x + labels[(size_t)b * (d.U - 1) + u]) : 0.0f;
+    p.pl[(size_t)b * d.Ua + u] = has_label ? ldf(x + label_at(labels, d, b, u)) : 0.0f;
   }
 }
 

@@ -161,7 +161,7 @@ __device__ __forceinline__ void egrads_walk(
 #pragma unroll
   for (int i = 0; i < kEsPrefetch; ++i) {
     mu[i] = (sp.labels && i < nmatch) ? match[i] : 0;
-    mc[i] = (sp.labels && i < nmatch) ? sp.labels[(size_t)b * (d.U - 1) + mu[i]] - wave_col0 : -1;
+    mc[i] = (sp.labels && i < nmatch) ? label_at(sp.labels, d, b, mu[i]) - wave_col0 : -1;
   }
 
   // bf16 only: with half the bytes the kernel is held by how long a request takes, not by how
@@ -283,7 +283,7 @@ __device__ __forceinline__ void egrads_walk(
         const int u = match[i];
         const size_t o = plane_row(d, b, u) + min(t0 + l32, Tb - 1) + u;
         apply(row_ok ? sp.dS[o + d.Dp + 1] * sp.wE[o] : 0.0f,
-              sp.labels[(size_t)b * (d.U - 1) + u] - wave_col0, -1.0f);
+              label_at(sp.labels, d, b, u) - wave_col0, -1.0f);
       }
       if (blank_lane >= 0) apply(row_ok ? sbl : 0.0f, blank_lane, 1.0f);
     }
@@ -356,7 +356,7 @@ __global__ __launch_bounds__(256, 2) void egrads_stream_kernel(
     const int col0 = blockIdx.x * 128 + wave * 32;
     for (int u0 = 0; u0 < Ub - 1; u0 += 64) {
       const int u = u0 + lane;
-      const int l = (u < Ub - 1) ? sp.labels[(size_t)b * (d.U - 1) + u] : -1;
+      const int l = (u < Ub - 1) ? label_at(sp.labels, d, b, u) : -1;
       const bool hit = l >= col0 && l < col0 + 32 && l != d.blank;
       const unsigned long long m = __ballot(hit);
       if (hit) Match[wave][nmatch + __popcll(m & ((1ull << lane) - 1))] = (unsigned short)u;
@@ -631,7 +631,7 @@ __global__ __launch_bounds__(256, 2) void pgrads_stream_kernel(
     // matches no column.  Visible to all after the barriers of the walk (or the one below).
     const int k = threadIdx.x, u = u0 + k;
     const bool valid = Tb > 0 && u < Ub, has_label = valid && u + 1 < Ub;
-    const int l = has_label ? sp.labels[(size_t)b * (d.U - 1) + u] : d.blank;
+    const int l = has_label ? label_at(sp.labels, d, b, u) : d.blank;
     Rt.gB[k] = valid ? sp.gB[(size_t)b * d.Ua + u] : 0.0f;
     Rt.gL[k] = has_label ? sp.gL[(size_t)b * d.Ua + u] : 0.0f;
     Rt.label[k] = (has_label && l != d.blank) ? l : -1;

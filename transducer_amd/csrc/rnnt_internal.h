@@ -76,6 +76,14 @@ __device__ inline void utt_extent(const int* inLen, const int* labLen, int b, in
   Ub = labLen ? clampi(labLen[b] + 1, 0, U) : U;
 }
 
+// Label of position u of utterance b, forced into the vocabulary.  The reference indexes its
+// score rows with whatever the caller wrote (transducer/transducer_cpu.cpp:63-66); here every
+// kernel reads labels through this one function, so a value outside [0, V) can neither read nor
+// write past a row and all kernels agree on which column it means.
+__device__ inline int label_at(const int* __restrict__ labels, const Dims& d, int b, int u) {
+  return clampi(labels[(size_t)b * (d.U - 1) + u], 0, d.V - 1);
+}
+
 // Buffers of the lattice recursions, all in the skewed layout except the three small vectors.
 struct Planes {
   float* lnS;   // log-normaliser LN[t,u]
@@ -90,6 +98,24 @@ struct Planes {
   float* gB;    // per-(b,u) blank-column sum of the sparse pgrads term   [B, Ua]
   float* gL;    // per-(b,u) label-column sum of the sparse pgrads term   [B, Ua]
 };
+
+// Trips a wavefront of the lattice kernels may spend waiting for its neighbour's progress
+// counter before it gives up and raises the trouble flag (each trip is an LDS read and a short
+// sleep, roughly 50 ns; the longest legitimate wait is a few dozen trips).
+constexpr int kDefaultSpinLimit = 1 << 20;
+extern int g_spin_limit;
+// Device address of the current device's trouble flag (a static device int, looked up once per
+// device).
+int trouble_flag(int** out);
+
+// One wavefront running `steps` steps of the bare dependent chain of an alpha (kind 0) or dalpha
+// (kind 1) cell; see chain_floor_kernel.
+int launch_chain_floor(int kind, int steps, hipStream_t s);
+// expf_glibc / log1pf_glibc (rnnt_libm.h) of n floats, for the tests.
+int launch_libm_probe(const float* x, float* e, float* l, long n, hipStream_t s);
+// out[0] += number of floats d <= 0 with bit pattern in [lo, hi] for which the error bound of the
+// fast log-sum-exp fails, out[1] = max(out[1], bits of the largest distance / bound).
+int launch_lse_bound_check(unsigned lo, unsigned hi, unsigned* out, hipStream_t s);
 
 size_t planes_bytes(const Dims& d);
 void carve_planes(void* base, const Dims& d, Planes* p);

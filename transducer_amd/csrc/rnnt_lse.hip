@@ -55,6 +55,18 @@ __device__ inline float quad_xor2(float x) {
   return __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(x), 0x4E, 0xf, 0xf, true));
 }
 
+// a + b + c rounded once: the two partial sums are carried with their rounding errors (two
+// error-free additions; this file is compiled without contraction or reassociation), so the
+// log-normaliser's epilogue log(sum) + mE + mP adds half an ulp to the error of the logarithm
+// instead of three half ulps.
+__device__ inline float add3(float a, float b, float c) {
+  const float s = b + c, bv = s - b;
+  const float s_err = (b - (s - bv)) + (c - bv);
+  const float r = a + s, av = r - a;
+  const float r_err = (a - (r - av)) + (s - av);
+  return r + (r_err + s_err);
+}
+
 // 16-byte slot of (row, c8 = which eight of the slab's 32 v) inside a piece plane
 __device__ inline int xslot(int row, int c8) { return row * 4 + (c8 ^ ((row >> 2) & 3)); }
 
@@ -155,7 +167,7 @@ __global__ __launch_bounds__(64 * kWaves, kWaves / 2) void lse_stream_kernel(
   const int nlab = (picking && labels != nullptr) ? min(Ub - 1, 1024) : 0;
   const int npick = picking ? nlab + 1 : 0;  // entry nlab is the blank column
   for (int u = tid; u < npick; u += kThreads)
-    labs[u] = u < nlab ? labels[(size_t)b * (d.U - 1) + u] : d.blank;
+    labs[u] = u < nlab ? label_at(labels, d, b, u) : d.blank;
   __syncthreads();
   // rank every entry by (column, index): the slabs come by in column order, so one cursor into
   // the sorted list tells each slab which columns to copy, at one LDS read per slab
@@ -413,7 +425,7 @@ __global__ __launch_bounds__(64 * kWaves, kWaves / 2) void lse_stream_kernel(
       const int row = 32 * (mb0 + m) + mfma_row(r, h), t = t0 + row;
       if (t < d.T && u < d.U) {
         float v = 0.0f;
-        if (t < Tb && u < Ub) v = (logf(tot[m][r] + acc[m][r]) + mfin[row]) + mu;
+        if (t < Tb && u < Ub) v = add3(logf(tot[m][r] + acc[m][r]), mfin[row], mu);
         if (lnS == nullptr) LNb[(size_t)t * d.U + u] = v;
         else if (t < Tb && u < Ub) lnS[plane_row(d, b, u) + t + u] = v;
       }

@@ -47,6 +47,13 @@ def _require_device(tensor):
 _SUFFIX = {torch.bfloat16: "_bf16", torch.float16: "_f16"}
 
 
+def _check_blank(blank, vocabulary):
+    """The reference indexes score rows with `blank` unchecked; an index outside the vocabulary
+    would read and write past every row, so it is refused (the library refuses it as well)."""
+    if not 0 <= blank < vocabulary:
+        raise ValueError("blank must lie in [0, {}), got {}".format(vocabulary, blank))
+
+
 def _stream(device):
     return torch.cuda.current_stream(device).cuda_stream
 
@@ -61,6 +68,7 @@ class Transducer(torch.autograd.Function):
         certify_inputs(emissions, predictions, labels, input_lengths, label_lengths,
                        score_dtype=emissions.dtype if suffix else torch.float32)
         _require_device(emissions)
+        _check_blank(blank, emissions.shape[2])
         device = emissions.device
         # the library reads raw pointers: dense row-major storage is required
         emissions = emissions.contiguous()
@@ -155,6 +163,7 @@ class TransducerLoss(torch.nn.Module):
         certify_inputs(emissions, predictions, labels, input_lengths, label_lengths,
                        score_dtype=emissions.dtype if suffix else torch.float32)
         _require_device(emissions)
+        _check_blank(self.blank, V)
         emissions = emissions.contiguous()
         predictions = predictions.contiguous()
         with DeviceManager(device):
