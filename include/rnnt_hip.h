@@ -148,6 +148,23 @@ int rnnt_hip_viterbi_decode(const float* emissions, const float* predictions,
                             const int* input_lengths, const int* label_lengths, int* labels,
                             int B, int T, int U, int V, int blank, rnnt_stream_t stream);
 
+/* rnnt_hip_viterbi_decode for callers that cannot allocate (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference, whose
+ * viterbi allocates and frees its scratch on every call (transducer/transducer_cuda.cu:364-369,
+ * 386-387).  Same arguments, same result; all scratch lives in an array built into the library
+ * (rnnt_hip_static_scratch_bytes() bytes, held on every GPU the library runs on until the
+ * process ends), and the call makes no hipMalloc / hipFree / hipMemset of any kind.  A problem
+ * whose scratch does not fit is refused with RNNT_WORKSPACE_TOO_SMALL (one utterance of the
+ * headline shape, T=2000 U=101 V=10000, needs 17 MB of the 64).  Every call on a GPU uses that
+ * GPU's one array: calls that overlap on one GPU (two streams, two threads) race; calls queued
+ * on one stream do not.  The array's address is looked up on the first call on each device, so
+ * make that first call outside any graph capture. */
+int rnnt_hip_viterbi_decode_static(const float* emissions, const float* predictions,
+                                   const int* input_lengths, const int* label_lengths,
+                                   int* labels, int B, int T, int U, int V, int blank,
+                                   rnnt_stream_t stream);
+size_t rnnt_hip_static_scratch_bytes(void);
+
 /* ---- stage timing (diagnostic; no counterpart in the reference, whose only instrumentation
  * is wall-clock loops in transducer/benchmark.cpp:21-34) ---------------------------------- */
 

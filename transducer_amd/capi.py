@@ -27,6 +27,8 @@ SIGNATURES = {
     "rnnt_hip_loss_forward_f16": (_I, [_F] * 7 + [_Z] + [_I] * 5 + [_F]),
     "rnnt_hip_loss_backward_f16": (_I, [_F] * 9 + [_Z] + [_I] * 5 + [_F]),
     "rnnt_hip_viterbi_decode": (_I, [_F] * 5 + [_I] * 5 + [_F]),
+    "rnnt_hip_viterbi_decode_static": (_I, [_F] * 5 + [_I] * 5 + [_F]),
+    "rnnt_hip_static_scratch_bytes": (_Z, []),
     "rnnt_hip_viterbi_decode_bf16": (_I, [_F] * 5 + [_I] * 5 + [_F]),
     "rnnt_hip_viterbi_decode_f16": (_I, [_F] * 5 + [_I] * 5 + [_F]),
     "rnnt_hip_check_kernels": (_I, [_F]),

@@ -425,6 +425,32 @@ int decode_fp32(const float* E, const float* P, const int* inLen, const int* lab
   return viterbi_impl(E, P, nullptr, labels, inLen, labLen, d, scratch, s, &p);
 }
 
+// ---------------------------------------------------------------- built-in scratch
+// Scratch of rnnt_hip_viterbi_decode_static: a device array that exists from the moment the
+// library's code is loaded on a GPU until the process ends, so that entry point never calls an
+// allocator.  `g_static_scratch` is a host-side handle, not a device address: the address is
+// looked up once per device, with that device current, and only that pointer is ever used.
+constexpr size_t kStaticScratchBytes = (size_t)64 << 20;
+static __device__ __align__(256) unsigned char g_static_scratch[kStaticScratchBytes];
+constexpr int kMaxScratchDevices = 64;
+static void* g_static_scratch_ptr[kMaxScratchDevices];
+static std::mutex g_static_scratch_mutex;
+
+int static_scratch(void** out) {
+  int dev = 0;
+  RNNT_HIP(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxScratchDevices)
+    return fail(kInvalid, "device index %d not supported", dev);
+  std::lock_guard<std::mutex> lock(g_static_scratch_mutex);
+  if (g_static_scratch_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    RNNT_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(g_static_scratch)));
+    g_static_scratch_ptr[dev] = p;
+  }
+  *out = g_static_scratch_ptr[dev];
+  return kOk;
+}
+
 }  // namespace
 }  // namespace rnnt
 
@@ -771,5 +797,18 @@ int rnnt_hip_viterbi_decode(const float* E, const float* P, const int* inLen, co
   Scratch scratch(s);
   return decode_fp32(E, P, inLen, labLen, labels, B, T, U, V, blank, s, scratch, "viterbi_decode");
 }
+
+int rnnt_hip_viterbi_decode_static(const float* E, const float* P, const int* inLen,
+                                   const int* labLen, int* labels, int B, int T, int U, int V,
+                                   int blank, rnnt_stream_t stream) {
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  void* base = nullptr;
+  RNNT_TRY(static_scratch(&base));
+  Scratch scratch(base, kStaticScratchBytes, "viterbi_decode_static");
+  return decode_fp32(E, P, inLen, labLen, labels, B, T, U, V, blank, s, scratch,
+                     "viterbi_decode_static");
+}
+
+size_t rnnt_hip_static_scratch_bytes(void) { return kStaticScratchBytes; }
 
 }  // extern "C"
