@@ -83,13 +83,16 @@ def log_norms_naive(E, P, input_lengths=None, label_lengths=None, precision="f32
     return LN
 
 
-def log_norms_sep(E, P, precision="f32", return_sum=False):
+def log_norms_sep(E, P, precision="f32", return_sum=False, lanes=1):
+    """Separable-max form (torch_binding.py:35-40).  lanes: partial sums of the inner sum (1 =
+    index order; 8 = the order of a vectorised dot product; the reference leaves it to BLAS)."""
     dt, sfx = _real(precision)
     E, P = _np(E, dt), _np(P, dt)
     B, T, U, V = _dims(E, P)
     LN = np.empty((B, T, U), dt)
     S = np.empty((B, T, U), dt) if return_sum else None
-    getattr(lib(), "orc_log_norms_sep" + sfx)(_p(E), _p(P), _p(LN), _p(S), B, T, U, V)
+    getattr(lib(), "orc_log_norms_sep_lanes" + sfx)(_p(E), _p(P), _p(LN), _p(S), B, T, U, V,
+                                                    int(lanes))
     return (LN, S) if return_sum else LN
 
 
@@ -198,11 +201,14 @@ def loss_and_grads(E, P, labels, input_lengths, label_lengths, blank=0, deltas=N
                    precision="f32", lse="naive"):
     """The torch-free end-to-end path of the reference's C++ tests (transducer/test.cpp:7-90):
     log-normaliser -> forward -> backward -> dense gradient accumulation.
-    ``lse``: "naive" (test.h:51-80) or "sep" (torch_binding.py:35-40,85-89, with deltas)."""
+    ``lse``: "naive" (test.h:51-80), "sep" (torch_binding.py:35-40,85-89, with deltas; inner
+    sums in index order) or "sep8" (the same with eight partial sums per inner sum)."""
     dt, _ = _real(precision)
     B = E.shape[0]
     if lse == "naive":
         LN = log_norms_naive(E, P, input_lengths, label_lengths, precision)
+    elif lse == "sep8":
+        LN = log_norms_sep(E, P, precision, lanes=8)
     else:
         LN = log_norms_sep(E, P, precision)
     costs, alphas = forward(E, P, LN, labels, input_lengths, label_lengths, blank, precision)

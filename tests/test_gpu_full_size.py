@@ -139,7 +139,8 @@ LN_ULP_BAR = 2.5
 # ------------------------------------------------------------------ headline configuration
 # fraction of gradient entries of the cut-out utterance outside rel 1e-4 / abs 1e-5 end to end
 # (each side with its own log-normaliser): (egrads, pgrads)
-CUT_OUT_BAR = (0.02, 0.02)
+# measured: 0.0001 % / 0 at V=10000, 0 / 0 at V=10001
+CUT_OUT_BAR = (2e-4, 2e-4)
 
 
 @pytest.mark.parametrize("V", [10000, 10001])
@@ -241,24 +242,33 @@ def test_headline_viterbi_one_utterance_bit_exact_and_batch_independent(near_tie
 
 
 # ------------------------------------------------------------------ the smaller configurations, whole
-# fraction of gradient entries outside rel 1e-4 / abs 1e-5 end to end, each side with its own
-# log-normaliser: about three times what was measured, per configuration (egrads, pgrads)
-END_TO_END_BAR = {"cfg2": (0.02, 0.02), "cfg3a": (0.02, 0.02), "cfg3b": (0.02, 0.02)}
+# Fraction of gradient entries outside rel 1e-4 / abs 1e-5 end to end, each side with its own
+# log-normaliser: about three times what was measured, per configuration (egrads, pgrads).
+# Measured: cfg2 0.0005 % / 0 (the reference's own spread between two orders of its LN sum: 0 / 0),
+# cfg3a 0.038 % / 0.197 % (spread 0.035 % / 0.181 %), cfg3b 0 / 0 (spread 0.030 % / 0.156 %).
+# The test takes the larger of this and twice the spread measured on the same inputs.
+END_TO_END_BAR = {"cfg2": (2e-5, 2e-5), "cfg3a": (1.2e-3, 6e-3), "cfg3b": (1e-4, 1e-4)}
 
 
 @pytest.mark.parametrize("name", ["cfg2", "cfg3a", "cfg3b"])
 def test_configuration_whole_against_the_oracle(name):
     E, P, labels, il, ll = unpack(make_inputs(CONFIGS[name], seed=0))
     a = oracle.loss_and_grads(E, P, labels, il, ll, lse="naive")
+    # How far the reference's own fp32 result moves when only the summation order of ITS
+    # normaliser changes: the separable form of torch_binding.py:35-40 with the inner sum in
+    # index order against the same with eight partial sums (the reference leaves that order to
+    # torch.bmm).  Index order against test.h's sequential sum says little: the two accumulate
+    # in the same order and round alike.
     b = oracle.loss_and_grads(E, P, labels, il, ll, lse="sep")
-    floor_e, _ = violations(b["egrads"], a["egrads"])
-    floor_p, _ = violations(b["pgrads"], a["pgrads"])
+    b8 = oracle.loss_and_grads(E, P, labels, il, ll, lse="sep8")
+    floor_e = max(violations(b["egrads"], a["egrads"])[0], violations(b8["egrads"], b["egrads"])[0])
+    floor_p = max(violations(b["pgrads"], a["pgrads"])[0], violations(b8["pgrads"], b["pgrads"])[0])
     costs, eg, pg = gpu_loss(DeviceCase(E, P, labels, il, ll))
     assert_close(costs, a["costs"], rtol=RTOL, atol=max(ATOL, 1e-3), what="costs")
     ve, worst_e = violations(eg, a["egrads"])
     vp, worst_p = violations(pg, a["pgrads"])
-    print("%s: violations egrads %.4f%% (oracle floor between two LN orders %.4f%%), pgrads "
-          "%.4f%% (floor %.4f%%); max abs err %.3g / %.3g"
+    print("%s: violations egrads %.4f%% (the reference's own spread between LN orders %.4f%%), "
+          "pgrads %.4f%% (spread %.4f%%); max abs err %.3g / %.3g"
           % (name, 100 * ve, 100 * floor_e, 100 * vp, 100 * floor_p, worst_e, worst_p))
     bar_e, bar_p = END_TO_END_BAR[name]
     assert ve <= max(2 * floor_e, bar_e) and vp <= max(2 * floor_p, bar_p)

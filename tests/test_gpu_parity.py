@@ -424,7 +424,8 @@ def test_whole_loss_at_T2000_violation_fraction():
     print("violations egrads %.4f%% (oracle floor %.4f%%), pgrads %.4f%% (floor %.4f%%); "
           "max abs err %.3g / %.3g" % (100 * ve, 100 * floor_e, 100 * vp, 100 * floor_p,
                                        worst_e, worst_p))
-    assert ve <= max(2 * floor_e, 0.02) and vp <= max(2 * floor_p, 0.02)
+    # (measured: 0.0003 % / 0.416 % with floors of 0.505 % / 1.267 % on these inputs)
+    assert ve <= max(2 * floor_e, 1e-3) and vp <= max(2 * floor_p, 1e-3)
     # fp64 truth: the device result must not be further from it than the reference's fp32 is
     t = oracle.loss_and_grads(E, P, labels, il, ll, precision="f64")
     err_dev = np.abs(eg - t["egrads"]).max()

@@ -10,13 +10,18 @@ answer is defined there."""
 import numpy as np
 import pytest
 
-from util import (DeviceCase, gpu_backward, gpu_forward, gpu_log_norms, gpu_loss, gpu_viterbi,
-                  violations)
+from util import (DeviceCase, assert_close, assert_same_bits, gpu_backward, gpu_forward,
+                  gpu_log_norms, gpu_loss, gpu_viterbi, violations)
 
 pytestmark = pytest.mark.gpu
 
 torch = pytest.importorskip("torch")
 import oracle  # noqa: E402
+
+# fraction of gradient entries that may sit outside rel 1e-4 / abs 1e-5 end to end, each side
+# with its own log-normaliser (largest measured over these seeds: 0.112 % of egrads, 0.082 % of
+# pgrads, both on one lattice of 131 x 129 cells; 34 of the 40 cases have none)
+END_TO_END_BAR = 0.004
 
 EDGES = [1, 2, 3, 31, 32, 33, 63, 64, 65, 96, 97, 127, 128, 129]
 VOCABS = [1, 2, 3, 4, 5, 7, 8, 9, 31, 32, 33, 100, 127, 128, 129, 255, 256, 260, 511, 512, 513,
@@ -62,33 +67,41 @@ def test_random_shape_against_the_oracle(seed):
           % (B, T, U, V, blank, il.tolist(), ll.tolist()), flush=True)
     c = DeviceCase(E, P, labels, il, ll)
 
-    # whole loss: costs to the tolerance (they are O(T) sums: absolute 1e-3 as for the long
-    # configurations), gradients with at most 1 % of entries moved by the last bits of LN
+    # whole loss end to end, each side with its own log-normaliser: costs to the tolerance (they
+    # are O(T) sums: absolute 1e-3 as for the long configurations); gradients move with the last
+    # bit of LN where the lattice is long, so a small fraction of entries may sit outside
     want = oracle.loss_and_grads(E, P, labels, il, ll, blank=blank)
     costs, eg, pg = gpu_loss(c, blank=blank)
     assert np.allclose(costs, want["costs"], rtol=1e-4, atol=1e-3, equal_nan=True)
     assert np.isfinite(eg).all() and np.isfinite(pg).all()
     live = np.isfinite(want["costs"])
     if live.any():
-        assert violations(eg[live], want["egrads"][live])[0] <= 0.01
-        assert violations(pg[live], want["pgrads"][live])[0] <= 0.01
+        fe = violations(eg[live], want["egrads"][live])[0]
+        fp = violations(pg[live], want["pgrads"][live])[0]
+        print("end to end: %.4f%% of egrads, %.4f%% of pgrads outside" % (100 * fe, 100 * fp))
+        assert fe <= END_TO_END_BAR and fp <= END_TO_END_BAR
     for b in range(B):
         assert not eg[b, il[b]:].any() and not pg[b, ll[b] + 1:].any()
 
-    # the C++ interface's three functions on one shared LN: no entry outside the tolerance
+    # the same with ONE log-normaliser (the device's) on both sides: no entry outside
     LN = gpu_log_norms(c)
     oc, oa = oracle.forward(E, P, LN, labels, il, ll, blank=blank)
+    oeg, opg, olng = oracle.backward(E, P, np.nan_to_num(oa), LN, labels, il, ll, blank=blank)
+    deg, dpg = oracle.accumulate_grads(E, P, oeg, opg, olng, LN, il, ll)
+    if live.any():
+        assert_close(costs[live], oc[live], what="costs, shared LN")
+        assert_close(eg[live], deg[live], what="egrads, shared LN")
+        assert_close(pg[live], dpg[live], what="pgrads, shared LN")
+
+    # the C++ interface's three functions on that LN: the reference's bits in every alpha, every
+    # dalpha and every blank / label term (same expf / log1pf, same order of operations)
     gc, ga = gpu_forward(c, LN, blank=blank)
-    assert np.allclose(gc, oc, rtol=1e-4, atol=1e-4, equal_nan=True)
-    oeg, opg, olng = oracle.backward(E, P, oa, LN, labels, il, ll, blank=blank)
-    geg, gpg, glng = gpu_backward(c, oa, LN, blank=blank)
-    for b in range(B):
-        if il[b] == 0:
-            continue
-        n, m = il[b], ll[b] + 1
-        assert violations(ga[b, :n, :m], oa[b, :n, :m], atol=1e-4)[0] == 0
-        assert violations(glng[b], olng[b])[0] == 0
-        assert violations(geg[b], oeg[b])[0] == 0 and violations(gpg[b], opg[b])[0] == 0
+    assert_same_bits(gc, oc, what="costs")
+    assert_same_bits(ga, oa, what="alphas")
+    geg, gpg, glng = gpu_backward(c, ga, LN, blank=blank)
+    assert_same_bits(glng, olng, what="lngrads")
+    assert_same_bits(geg, oeg, what="egrads (sparse)")
+    assert_same_bits(gpg, opg, what="pgrads (sparse)")
 
     # best path: exact
     if U > 1:

@@ -258,3 +258,21 @@ def test_empty_utterance_costs_infinity_and_zero_grads():
     r = oracle.loss_and_grads(E, P, labels, il, ll)
     assert np.isposinf(r["costs"][1]) and np.isfinite(r["costs"][[0, 2]]).all()
     assert not r["egrads"][1].any() and not r["pgrads"][1].any() and not r["lngrads"][1].any()
+
+
+def test_separable_log_norms_with_partial_sums_is_the_same_mathematics():
+    """log_norms_sep(lanes=8) only re-orders the inner sum (eight partial sums, as a vectorised
+    dot product forms them): the fp64 instance agrees with index order to fp64 rounding, the fp32
+    instance to a few fp32 spacings, and the two are not bit-identical (else it would measure
+    nothing)."""
+    rng = np.random.default_rng(3)
+    E = rng.standard_normal((2, 9, 301)).astype(np.float32)
+    P = rng.standard_normal((2, 5, 301)).astype(np.float32)
+    a64 = oracle.log_norms_sep(E, P, precision="f64")
+    b64 = oracle.log_norms_sep(E, P, precision="f64", lanes=8)
+    assert np.abs(a64 - b64).max() < 1e-13
+    a32 = oracle.log_norms_sep(E, P)
+    b32 = oracle.log_norms_sep(E, P, lanes=8)
+    assert np.abs(a32 - a64).max() < 4e-6 and np.abs(b32 - a64).max() < 4e-6
+    assert not np.array_equal(a32, b32)
+    assert np.array_equal(oracle.log_norms_sep(E, P, lanes=1), a32)
