@@ -3,22 +3,37 @@
 
 A "step" is one forward+backward of the loss (log-normaliser, alpha recursion, dalpha recursion,
 dense + sparse gradients) on one synthetic batch that is already resident in HBM, called through
-the C interface of librnnt_hip.so.  Prints ONE JSON line:
+the C interface of librnnt_hip.so.  Inputs come from the seeded host generator the tests use
+(transducer_amd/synthetic.py), so a (workload, seed) pair names the same bits everywhere.
+Prints ONE JSON line:
 
-  value / ms_per_step   milliseconds per fwd+bwd at the headline shape (lower is better)
-  roofline              the slowest matrix-core kernel: algorithmic fp32 flops of one launch
-                        (2 * V * sum_b T_b*(U_b+1), valid lattice cells only) over its mean
-                        duration, measured with HIP events on the launch stream during the
-                        timed steps, against the 157.3 TFLOP/s fp32 matrix peak (the kernels
-                        form each fp32 product from six bf16 matrix products, so this fraction
-                        may pass 1); "hbm" inside it prices the same launch against 8 TB/s with
-                        the bytes the algorithm must move (valid rows of E and P read once,
-                        the kernel's output written once)
+  value / ms_per_step   milliseconds per fwd+bwd at the headline shape (lower is better), from a
+                        timed loop with stage timing switched off; the per-stage breakdown comes
+                        from a second loop of the same length
+  roofline              the bound that holds the workload, chosen from the measured stages:
+                        "mfma"  -- the slowest matrix-core kernel: algorithmic fp32 flops of one
+                                   launch (2 * V * sum_b T_b*(U_b+1), valid lattice cells only)
+                                   over its mean duration (HIP events on the launch stream),
+                                   against the 157.3 TFLOP/s fp32 matrix peak; "hbm" inside it
+                                   prices the same launch against 8 TB/s with the bytes the
+                                   algorithm must move; "traffic" is the fetched + written bytes
+                                   of that kernel from the counter run recorded in
+                                   profiles/hbm_traffic.json (null when that file has no entry
+                                   for the workload)
+                        "chain-latency" -- when the two lattice walks take longer than any
+                                   contraction (small vocabularies): nanoseconds per anti-diagonal
+                                   step of the alpha walk against the floor that
+                                   rnnt_hip_chain_floor measures in the same run (one wavefront,
+                                   the bare dependent chain of one cell)
+  checks                what the timed calls wrote: costs finite and positive, rows of egrads and
+                        pgrads summing to zero, padding exactly zero, and -- when the CPU baseline
+                        ran on the whole batch -- the device result against it
   cpu_baseline          the CPU path (the OpenMP restatement in oracle/, which is checked bit for
-                        bit against the reference's compiled sources) timed on the host cores
-                        over a bounded sample of the same workload and scaled by lattice-cell
-                        count; the lattice recursions are also timed through the reference's
-                        own transducer_cpu.cpp build (oracle/_ref) when it is present
+                        bit against the reference's compiled sources) timed on the host cores on
+                        the bench's own inputs: the whole batch when that fits about a minute,
+                        else a bounded sample scaled by lattice-cell count ("scaled": true); the
+                        lattice recursions are also timed through the reference's own
+                        transducer_cpu.cpp build (oracle/_ref) when it is present
 """
 import argparse
 import ctypes
@@ -32,95 +47,96 @@ import numpy as np
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
+from transducer_amd.synthetic import CONFIGS, Config, make_inputs  # noqa: E402
+
 METRIC = "ms per fwd+bwd RNN-T loss, B=32 T=2000 U=100 V=10000; % of roofline"
 PEAK_FP32_MATRIX_TFLOPS = 157.3
 PEAK_HBM_GBS = 8000.0
-# HBM bytes per launch (fetched + written) from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this
-# file, scaled by what the counters read for a plain copy of known size
-# (profiles/cfg4_hbm_traffic_counters.md).  Recorded, not measured live: counters need rocprofv3.
-RECORDED_TRAFFIC_BYTES = {"cfg4": {"lse": 2.546e9, "egrads": 5.633e9, "pgrads": 3.129e9}}
+PEAK_VALU_TLANEOPS = 256 * 64 * 2.4e9 / 1e12  # 256 CUs x 64 fp32 lanes x 2.4 GHz, one op per lane
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+KERNEL_OF_STAGE = {"lse": "lse_stream_kernel", "egrads": "egrads_stream_kernel",
+                   "pgrads": "pgrads_stream_kernel"}
 
+# name -> (configuration of the seeded generator, options).  cfg2..cfg5 are BASELINE's
+# configurations; the rest are variants of the headline shape.
+_HEAD = CONFIGS["cfg4"]
 WORKLOADS = {
-    # BASELINE configs[3]: the shape the metric is quoted on
-    "cfg4": dict(B=32, T=2000, U=100, V=10000, sigma=1.0, ragged_T=(1500, 2000), ragged_U=(75, 100)),
-    "cfg2": dict(B=8, T=2000, U=100, V=100, sigma=1.0, ragged_T=None, ragged_U=None),
-    "cfg3a": dict(B=8, T=2000, U=100, V=1000, sigma=2.0, ragged_T=(1000, 2000), ragged_U=(50, 100)),
-    "cfg3b": dict(B=8, T=2000, U=100, V=2000, sigma=2.0, ragged_T=(1000, 2000), ragged_U=(50, 100)),
-    # BASELINE configs[4]: teacher-forced best path (log-normaliser + max-plus + lattice + backtrace)
-    "cfg5": dict(B=32, T=2000, U=100, V=10000, sigma=1.0, ragged_T=(1500, 2000), ragged_U=(75, 100),
-                 kind="viterbi"),
-    "cfg5ties": dict(B=32, T=2000, U=100, V=10000, sigma=1.0, ragged_T=(1500, 2000),
-                     ragged_U=(75, 100), kind="viterbi", near_ties=True),
+    "cfg4": (CONFIGS["cfg4"], {}),
+    "cfg2": (CONFIGS["cfg2"], {}),
+    "cfg3a": (CONFIGS["cfg3a"], {}),
+    "cfg3b": (CONFIGS["cfg3b"], {}),
+    # teacher-forced best path (log-normaliser + max-plus + lattice + backtrace)
+    "cfg5": (CONFIGS["cfg5"], dict(kind="viterbi")),
+    "cfg5ties": (CONFIGS["cfg5"], dict(kind="viterbi", near_ties=True)),
     # the inputs of the reference's own benchmark script at the shape its README quotes 223.33 ms
     # for on an A100 (benchmarks/torch_benchmarks.py:26-35: uniform [0,1) scores, full lengths)
-    "readme": dict(B=32, T=2000, U=100, V=10000, sigma=1.0, ragged_T=None, ragged_U=None,
-                   uniform=True, published_ms=223.33),
-    # the headline shape with bf16 scores and gradients (rnnt_hip_loss_*_bf16; not a reference
-    # configuration: the reference takes float32 only)
-    "cfg5bf16": dict(B=32, T=2000, U=100, V=10000, sigma=1.0, ragged_T=(1500, 2000),
-                     ragged_U=(75, 100), kind="viterbi", io="bf16"),
-    "cfg4bf16": dict(B=32, T=2000, U=100, V=10000, sigma=1.0, ragged_T=(1500, 2000),
-                     ragged_U=(75, 100), io="bf16"),
-    "cfg4f16": dict(B=32, T=2000, U=100, V=10000, sigma=1.0, ragged_T=(1500, 2000),
-                    ragged_U=(75, 100), io="f16"),
+    "readme": (Config("readme", 32, 2000, 100, 10000, 1.0, None, None),
+               dict(uniform=True, published_ms=223.33)),
+    # the headline shape with 16-bit scores and gradients (not a reference configuration: the
+    # reference takes float32 only)
+    "cfg4bf16": (_HEAD, dict(io="bf16")),
+    "cfg4f16": (_HEAD, dict(io="f16")),
+    "cfg5bf16": (CONFIGS["cfg5"], dict(kind="viterbi", io="bf16")),
 }
-PEAK_VALU_TLANEOPS = 256 * 64 * 2.4e9 / 1e12  # 256 CUs x 64 fp32 lanes x 2.4 GHz, one op per lane
 
 
-def make_device_inputs(w, seed, device):
-    import torch
-    g = torch.Generator(device=device)
-    g.manual_seed(seed)
-    B, T, U, V = w["B"], w["T"], w["U"], w["V"]
-    draw = torch.rand if w.get("uniform") else torch.randn
-    E = draw((B, T, V), generator=g, device=device, dtype=torch.float32) * w["sigma"]
-    P = draw((B, U + 1, V), generator=g, device=device, dtype=torch.float32) * w["sigma"]
-    if w.get("near_ties"):  # a tenth of every frame's entries repeat another column's value
-        for b in range(B):
-            dst = torch.randint(1, V, (T, V // 10), generator=g, device=device)
-            src = torch.randint(1, V, (T, V // 10), generator=g, device=device)
-            E[b].scatter_(1, dst, E[b].gather(1, src))
-    labels = torch.randint(1, V, (B, U), generator=g, device=device, dtype=torch.int32)
-    rng = np.random.Generator(np.random.Philox(key=seed))
-    il = np.full(B, T, np.int32)
-    ll = np.full(B, U, np.int32)
-    if w["ragged_T"]:
-        il = rng.integers(w["ragged_T"][0], w["ragged_T"][1] + 1, B).astype(np.int32)
-        il[0] = T
-    if w["ragged_U"]:
-        ll = rng.integers(w["ragged_U"][0], w["ragged_U"][1] + 1, B).astype(np.int32)
-        ll[B - 1] = U
-    return E, P, labels, torch.from_numpy(il).to(device), torch.from_numpy(ll).to(device), il, ll
+def host_inputs(cfg, opt, seed):
+    """Seeded host arrays of the workload (numpy's counter-based generator)."""
+    d = make_inputs(cfg, seed=seed, near_ties=bool(opt.get("near_ties")))
+    if opt.get("uniform"):  # the reference's benchmark draws uniform [0, 1) scores
+        rng = np.random.Generator(np.random.Philox(key=seed + 1000))
+        d["emissions"] = rng.random(d["emissions"].shape, dtype=np.float32)
+        d["predictions"] = rng.random(d["predictions"].shape, dtype=np.float32)
+    return d
 
 
-def cpu_baseline(w, il, ll, seconds_budget=15.0):
-    """Times the CPU path on a bounded sample of the workload and scales to the full batch.
+def describe(name, cfg, opt):
+    return ("%s: B=%d T=%d U=%d V=%d blank=0, %s scores%s, input_lengths %s, label_lengths %s, "
+            "deltas=1" % (name, cfg.B, cfg.T, cfg.U, cfg.V,
+                          "uniform [0,1)" if opt.get("uniform") else "N(0,%g)" % cfg.sigma,
+                          ", a tenth of the emission entries duplicated" if opt.get("near_ties")
+                          else "",
+                          "U[%d,%d]" % cfg.ragged_T if cfg.ragged_T else "=T",
+                          "U[%d,%d]" % cfg.ragged_U if cfg.ragged_U else "=U"))
+
+
+def recorded_traffic(workload, kernel):
+    """fetched + written bytes per launch of `kernel` from the tracked counter summary, or None."""
+    try:
+        with open(TRAFFIC_FILE) as f:
+            rec = json.load(f)
+        k = rec["workloads"][workload][kernel]
+        return {"bytes": k["fetched_bytes"] + k["written_bytes"], "fetched_bytes": k["fetched_bytes"],
+                "written_bytes": k["written_bytes"], "recorded": rec.get("recorded"),
+                "source": rec.get("source")}
+    except (OSError, KeyError, ValueError):
+        return None
+
+
+def cpu_baseline(d, seconds_budget=60.0):
+    """The CPU path on the bench's own inputs.
 
     Full path = log-normaliser + alpha + dalpha + dense gradient accumulation, i.e. the
     torch-free end-to-end sequence of the reference's C++ tests (transducer/test.cpp:7-90), run
     by the OpenMP restatement in oracle/ (the reference's own LSE / dense-gradient helpers in
     test.h are single-threaded test code).  The lattice recursions alone are also timed through
-    the reference's own transducer_cpu.cpp when oracle/_ref was built."""
+    the reference's own transducer_cpu.cpp when oracle/_ref was built.  Returns the record and,
+    when the whole batch was run, its results (for the parity check)."""
     import oracle  # checker code, used here only as the timed CPU baseline
     threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
-    B, T, U, V = w["B"], w["T"], w["U"], w["V"]
-    Bs = max(1, min(B, threads))
-    rng = np.random.Generator(np.random.Philox(key=1234))
-    P = rng.standard_normal((Bs, U + 1, V), dtype=np.float32) * np.float32(w["sigma"])
-    labels = rng.integers(1, V, (Bs, U)).astype(np.int32)
-    sll = ll[:Bs].astype(np.int32)
+    E, P, labels = d["emissions"], d["predictions"], d["labels"]
+    il, ll = d["input_lengths"], d["label_lengths"]
+    B, T, V = E.shape
+    U = P.shape[1] - 1
 
-    def run(Ts):
-        E = rng.standard_normal((Bs, Ts, V), dtype=np.float32) * np.float32(w["sigma"])
-        sil = np.minimum(il[:Bs], Ts).astype(np.int32)
-        sil[0] = Ts
+    def run(E, P, labels, sil, sll, keep):
         t0 = time.perf_counter()
         LN = oracle.log_norms_naive(E, P, sil, sll)
         t1 = time.perf_counter()
         costs, alphas = oracle.forward(E, P, LN, labels, sil, sll)
         eg, pg, lng = oracle.backward(E, P, np.nan_to_num(alphas), LN, labels, sil, sll)
         t2 = time.perf_counter()
-        oracle.accumulate_grads(E, P, eg, pg, lng, LN, sil, sll)
+        eg, pg = oracle.accumulate_grads(E, P, eg, pg, lng, LN, sil, sll)
         t3 = time.perf_counter()
         dp_ref = None
         if oracle.have_ref():
@@ -129,88 +145,171 @@ def cpu_baseline(w, il, ll, seconds_budget=15.0):
             oracle.ref_backward(E, P, np.nan_to_num(ra), LN, labels, sil, sll)
             dp_ref = time.perf_counter() - r0
         cells = float(np.sum(sil.astype(np.int64) * (sll.astype(np.int64) + 1)))
-        return (t1 - t0, t2 - t1, t3 - t2, dp_ref, cells)
+        res = dict(costs=costs, egrads=eg, pgrads=pg) if keep else None
+        return (t1 - t0, t2 - t1, t3 - t2, dp_ref, cells, res)
 
-    probe = run(min(T, 16))  # calibrates the sample size to the time budget
-    per_frame = max(sum(probe[:3]) / min(T, 16), 1e-6)
-    Ts = int(max(16, min(T, seconds_budget / per_frame)))
-    lse_s, dp_s, acc_s, dp_ref_s, cells_sample = run(Ts)
+    # calibrate on the first 16 frames of every utterance
+    Tp = min(T, 16)
+    probe = run(np.ascontiguousarray(E[:, :Tp]), P, labels, np.minimum(il, Tp).astype(np.int32),
+                ll, False)
     cells_full = float(np.sum(il.astype(np.int64) * (ll.astype(np.int64) + 1)))
-    scale = cells_full / cells_sample
+    estimate = sum(probe[:3]) * cells_full / max(probe[4], 1.0)
+    if estimate <= seconds_budget:
+        lse_s, dp_s, acc_s, dp_ref_s, cells, res = run(E, P, labels, il, ll, True)
+        scale, scaled = 1.0, False
+        sample = "the whole batch (%d utterances, the bench's own inputs)" % B
+    else:  # a prefix of the frames of the first `threads` utterances, scaled by cell count
+        Bs = max(1, min(B, threads))
+        per_frame = sum(probe[:3]) / Tp * Bs / B
+        Ts = int(max(16, min(T, 20.0 / max(per_frame, 1e-9))))
+        lse_s, dp_s, acc_s, dp_ref_s, cells, res = run(
+            np.ascontiguousarray(E[:Bs, :Ts]), np.ascontiguousarray(P[:Bs]),
+            np.ascontiguousarray(labels[:Bs]), np.minimum(il[:Bs], Ts).astype(np.int32),
+            np.ascontiguousarray(ll[:Bs]), False)
+        scale, scaled = cells_full / cells, True
+        sample = "%d of %d utterances x first %d of %d frames of the bench's inputs" % (Bs, B, Ts, T)
     out = {
         "value": round((lse_s + dp_s + acc_s) * 1e3 * scale, 1),
-        "unit": "ms per fwd+bwd, scaled from the sample by lattice-cell count",
+        "unit": "ms per fwd+bwd",
         "cores": threads,
         "kind": "port",
-        "sample": "%d of %d utterances x first %d of %d frames, U=%d V=%d; naive LSE + alpha + "
-                  "dalpha + dense gradient accumulation (OpenMP over utterances); measured %.2f s"
-                  % (Bs, B, Ts, T, U, V, lse_s + dp_s + acc_s),
+        "scaled": scaled,
+        "sample": "%s, U=%d V=%d; naive LSE + alpha + dalpha + dense gradient accumulation "
+                  "(OpenMP over utterances); measured %.2f s" % (sample, U, V, lse_s + dp_s + acc_s),
         "lse_ms": round(lse_s * 1e3 * scale, 1),
         "lattice_ms": round(dp_s * 1e3 * scale, 2),
         "dense_grads_ms": round(acc_s * 1e3 * scale, 1),
     }
     if dp_ref_s is not None:
         out["lattice_ms_reference_build"] = round(dp_ref_s * 1e3 * scale, 2)
+    return out, res
+
+
+def outside(got, want, rtol=1e-4, atol=1e-5):
+    """fraction of entries with |got - want| > atol + rtol |want| (one utterance at a time: the
+    arrays are gigabytes)"""
+    bad = 0
+    for g, w in zip(got, want):
+        g = np.asarray(g, np.float64)
+        bad += int(np.count_nonzero(np.abs(g - w) > atol + rtol * np.abs(w)))
+    return bad / float(max(got.size, 1))
+
+
+def output_checks(costs, egrads, pgrads, il, ll):
+    """What the timed calls left in their outputs, on the device: finite positive costs, gradient
+    rows that sum to zero (sum_v softmax = 1 and a node's occupancy equals its two outgoing
+    moves), exact zeros in the padding."""
+    import torch
+    B, T, V = egrads.shape
+    U1 = pgrads.shape[1]
+    dev = egrads.device
+    d_il = torch.as_tensor(il, device=dev)
+    d_ll = torch.as_tensor(ll, device=dev)
+    tmask = torch.arange(T, device=dev)[None, :] >= d_il[:, None]
+    umask = torch.arange(U1, device=dev)[None, :] > d_ll[:, None]
+    eg = egrads.float() if egrads.dtype != torch.float32 else egrads
+    pg = pgrads.float() if pgrads.dtype != torch.float32 else pgrads
+    se = eg.sum(-1, dtype=torch.float64).abs()
+    ae = eg.abs().sum(-1, dtype=torch.float64)
+    sp = pg.sum(-1, dtype=torch.float64).abs()
+    ap_ = pg.abs().sum(-1, dtype=torch.float64)
+    out = {
+        "costs_finite_positive": bool(torch.isfinite(costs).all() and (costs > 0).all()),
+        "gradients_finite": bool(torch.isfinite(eg).all() and torch.isfinite(pg).all()),
+        "padding_exactly_zero": bool(not eg[tmask].any() and not pg[umask].any()),
+        "largest_row_sum_over_row_size": {
+            "egrads": float((se / (ae + 1e-30)).max()), "pgrads": float((sp / (ap_ + 1e-30)).max())},
+    }
+    tol = 2e-5 if egrads.dtype == torch.float32 else 2e-2
+    out["rows_sum_to_zero"] = bool((se <= 1e-5 + tol * ae).all() and (sp <= 1e-5 + tol * ap_).all())
+    out["ok"] = all(out[k] for k in ("costs_finite_positive", "gradients_finite",
+                                     "padding_exactly_zero", "rows_sum_to_zero"))
     return out
 
 
-def viterbi_main(args, w, capi, E, P, d_il, d_ll, il, ll):
-    """--workload cfg5: one step = rnnt_hip_viterbi_decode (log-normaliser, best label per cell,
-    best-path lattice, backtrace).  The dominant kernel is the max-plus scan, which has no
-    matrix form: it is priced in vector lane-operations (one add and one compare/select per
-    (t, u, v) of the valid lattice) against 256 CUs x 64 lanes x 2.4 GHz."""
+def time_steps(step, steps):
     import torch
-    B, T, U1, V = w["B"], w["T"], w["U"] + 1, w["V"]
-    out_labels = torch.empty((B, U1 - 1), dtype=torch.int32, device=E.device)
-    stream = ctypes.c_void_p(torch.cuda.current_stream(E.device).cuda_stream)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+        torch.cuda.synchronize()  # a device sync per call, as in benchmarks/torch_benchmarks.py:8-20
+    return (time.perf_counter() - t0) * 1e3 / steps
+
+
+def stage_times(capi, step, steps):
+    """Per-stage milliseconds from a loop of its own (HIP events around every kernel stage)."""
+    import torch
+    capi.profile_enable(True)
+    torch.cuda.synchronize()
+    for _ in range(steps):
+        step()
+        torch.cuda.synchronize()
+    stages = capi.profile_read()
+    capi.profile_enable(False)
+    per_launch = {k: (ms / n) for k, (ms, n) in stages.items() if n}
+    per_step = {k: round(ms / steps, 4) for k, (ms, n) in stages.items() if n}
+    return per_launch, per_step
+
+
+def chain_floor(capi, kind, steps=20000):
+    out = ctypes.c_double(0.0)
+    capi.call("rnnt_hip_chain_floor", kind, steps, ctypes.byref(out))
+    return out.value
+
+
+def viterbi_main(args, name, cfg, opt, capi, d, device):
+    """one step = rnnt_hip_viterbi_decode (log-normaliser, best label per cell, best-path
+    lattice, backtrace).  The dominant kernel is the max-plus scan, which has no matrix form: it
+    is priced in vector lane-operations (one add and one compare/select per (t, u, v) of the
+    valid lattice) against 256 CUs x 64 lanes x 2.4 GHz."""
+    import torch
+    B, T, U1, V = cfg.B, cfg.T, cfg.U + 1, cfg.V
+    il, ll = d["input_lengths"], d["label_lengths"]
+    E = torch.from_numpy(d["emissions"]).to(device)
+    P = torch.from_numpy(d["predictions"]).to(device)
+    d_il, d_ll = torch.from_numpy(il).to(device), torch.from_numpy(ll).to(device)
+    out_labels = torch.full((B, U1 - 1), -1, dtype=torch.int32, device=device)
+    stream = ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
     p = lambda t: ctypes.c_void_p(t.data_ptr())
-    io = w.get("io")
-    bf16 = io is not None
-    if bf16:
+    io = opt.get("io")
+    if io:
         dtype16 = {"bf16": torch.bfloat16, "f16": torch.float16}[io]
         E, P = E.to(dtype16), P.to(dtype16)
-    entry = "rnnt_hip_viterbi_decode" + ("_" + io if bf16 else "")
+    entry = "rnnt_hip_viterbi_decode" + ("_" + io if io else "")
 
     def step():
         capi.call(entry, p(E), p(P), p(d_il), p(d_ll), p(out_labels), B, T, U1, V, 0, stream)
 
     for _ in range(args.warmup):
         step()
-        torch.cuda.synchronize()
-    capi.profile_enable(True)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-        torch.cuda.synchronize()
-    t1 = time.perf_counter()
-    stages = capi.profile_read()
-    capi.profile_enable(False)
-    ms_per_step = (t1 - t0) * 1e3 / args.steps
-    per_launch = {k: (ms / n) for k, (ms, n) in stages.items() if n}
-    per_step = {k: round(ms / args.steps, 4) for k, (ms, n) in stages.items() if n}
+    ms_per_step = time_steps(step, args.steps)
+    per_launch, per_step = stage_times(capi, step, args.steps)
+    paths = out_labels.cpu().numpy()
+    written = np.arange(U1 - 1)[None, :] < ll[:, None]
+    checks = {"labels_inside_vocabulary": bool(((paths >= 1) & (paths < V))[written].all()),
+              "padding_untouched": bool((paths[~written] == -1).all())}
+    checks["ok"] = all(checks.values())
     cells = float(np.sum(il.astype(np.int64) * (ll.astype(np.int64) + 1)))
     lane_ops = 2.0 * (V - 1) * cells
     achieved = lane_ops / (per_launch["maxplus"] * 1e-3) / 1e12
     out = {
-        "metric": "ms per teacher-forced viterbi decode, B=%d T=%d U=%d V=%d" % (B, T, w["U"], V),
+        "metric": "ms per teacher-forced viterbi decode, B=%d T=%d U=%d V=%d" % (B, T, cfg.U, V),
         "value": round(ms_per_step, 4), "unit": "ms", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": False,
         "scaling": "weak", "vs_baseline": None,
-        "dtype": "f32 arithmetic on %s scores" % io if bf16 else "f32", "data": "synthetic",
-        "config": {"workload": "%s: B=%d T=%d U=%d V=%d blank=0, N(0,1) scores%s, input_lengths "
-                               "U[%d,%d], label_lengths U[%d,%d]"
-                               % ((args.workload, B, T, w["U"], V,
-                                   ", a tenth of each frame's entries duplicated"
-                                   if w.get("near_ties") else "") + w["ragged_T"] + w["ragged_U"]),
-                   "seed": args.seed, "valid_lattice_cells": int(cells)},
+        "dtype": "f32 arithmetic on %s scores" % io if io else "f32", "data": "synthetic",
+        "config": {"workload": describe(name, cfg, opt), "seed": args.seed,
+                   "valid_lattice_cells": int(cells)},
         "roofline": {"bound": "valu", "kernel": "maxplus_kernel", "achieved": round(achieved, 2),
                      "peak": round(PEAK_VALU_TLANEOPS, 2), "unit": "Tlane-op/s",
                      "frac": round(achieved / PEAK_VALU_TLANEOPS, 4), "traffic": None,
                      "kernel_ms": round(per_launch["maxplus"], 4), "lane_ops_per_launch": lane_ops},
         "stage_ms_per_step": per_step,
+        "checks": checks,
     }
     print(json.dumps(out))
+    return 0 if checks["ok"] else 1
 
 
 def main():
@@ -237,20 +336,25 @@ def main():
         sys.exit("bench.py needs a HIP device")
     capi.load()  # raises if librnnt_hip.so is not built: there is no fallback path
     device = torch.device("cuda:0")
-    w = WORKLOADS[args.workload]
-    B, T, U1, V = w["B"], w["T"], w["U"] + 1, w["V"]
-    E, P, labels, d_il, d_ll, il, ll = make_device_inputs(w, args.seed, device)
-    if w.get("kind") == "viterbi":
-        return viterbi_main(args, w, capi, E, P, d_il, d_ll, il, ll)
-    io = w.get("io")  # None (fp32), "bf16" or "f16"
-    bf16 = io is not None
-    if bf16:
+    cfg, opt = WORKLOADS[args.workload]
+    d = host_inputs(cfg, opt, args.seed)
+    if opt.get("kind") == "viterbi":
+        return viterbi_main(args, args.workload, cfg, opt, capi, d, device)
+
+    B, T, U1, V = cfg.B, cfg.T, cfg.U + 1, cfg.V
+    il, ll = d["input_lengths"], d["label_lengths"]
+    E = torch.from_numpy(d["emissions"]).to(device)
+    P = torch.from_numpy(d["predictions"]).to(device)
+    labels = torch.from_numpy(d["labels"]).to(device)
+    d_il, d_ll = torch.from_numpy(il).to(device), torch.from_numpy(ll).to(device)
+    io = opt.get("io")  # None (fp32), "bf16" or "f16"
+    if io:
         dtype16 = {"bf16": torch.bfloat16, "f16": torch.float16}[io]
         E, P = E.to(dtype16), P.to(dtype16)
-    suffix, esize = ("_" + io, 2.0) if bf16 else ("", 4.0)
-    costs = torch.empty(B, device=device)
-    egrads = torch.empty_like(E)
-    pgrads = torch.empty_like(P)
+    suffix, esize = ("_" + io, 2.0) if io else ("", 4.0)
+    costs = torch.full((B,), float("nan"), device=device)
+    egrads = torch.full_like(E, float("nan"))
+    pgrads = torch.full_like(P, float("nan"))
     deltas = torch.ones(B, device=device)
     nbytes = capi.load().rnnt_hip_loss_workspace_bytes(B, T, U1, V)
     ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
@@ -269,20 +373,11 @@ def main():
     if args.copy_calibration:
         torch.mul(E, 1.0, out=egrads)  # vectorized_elementwise_kernel: reads E, writes egrads
         torch.cuda.synchronize()
-    capi.profile_enable(True)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-        torch.cuda.synchronize()  # a device sync per call, as in benchmarks/torch_benchmarks.py:8-20
-    torch.cuda.synchronize()
-    t1 = time.perf_counter()
-    stages = capi.profile_read()
-    capi.profile_enable(False)
-    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    ms_per_step = time_steps(step, args.steps)          # the figure: stage timing off
+    per_launch, per_step = stage_times(capi, step, args.steps)
+    capi.call("rnnt_hip_check_kernels", stream)          # no lattice kernel gave up a wait
+    checks = output_checks(costs, egrads, pgrads, il, ll)
 
-    per_launch = {k: (ms / n) for k, (ms, n) in stages.items() if n}
-    per_step = {k: round(ms / args.steps, 4) for k, (ms, n) in stages.items() if n}
     cells = float(np.sum(il.astype(np.int64) * (ll.astype(np.int64) + 1)))
     flops_one = 2.0 * V * cells  # one contraction over the valid lattice
     mfma_kernels = {k: per_launch[k] for k in ("lse", "egrads", "pgrads") if k in per_launch}
@@ -294,8 +389,47 @@ def main():
     out_bytes = {"lse": 4.0 * B * T * U1, "egrads": esize * B * T * V,
                  "pgrads": esize * B * U1 * V}
     hbm_gbs = (in_bytes + out_bytes[dom]) / (mfma_kernels[dom] * 1e-3) / 1e9
+    traffic = recorded_traffic(args.workload, KERNEL_OF_STAGE[dom])
+    mfma_roofline = {
+        "bound": "mfma", "kernel": KERNEL_OF_STAGE[dom],
+        "achieved": round(achieved, 2), "peak": PEAK_FP32_MATRIX_TFLOPS,
+        "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP32_MATRIX_TFLOPS, 4),
+        "traffic": traffic["bytes"] if traffic else None,
+        "traffic_record": traffic,
+        "kernel_ms": round(mfma_kernels[dom], 4),
+        "flops_per_launch": flops_one,
+        "hbm": {"achieved": round(hbm_gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                "frac": round(hbm_gbs / PEAK_HBM_GBS, 4),
+                "bytes_per_launch": in_bytes + out_bytes[dom]},
+        "all_kernels_frac_of_fp32_matrix_peak": {
+            k: round(flops_one / (v * 1e-3) / 1e12 / PEAK_FP32_MATRIX_TFLOPS, 4)
+            for k, v in mfma_kernels.items()}}
+    # the two lattice walks: nanoseconds per anti-diagonal step against the measured floor of one
+    # step's dependent chain (all utterances walk at once, so the longest one sets the time)
+    walk_steps = int(np.max(il.astype(np.int64) + ll.astype(np.int64)))  # T_b + (U_b + 1) - 1
+    floors = {"alpha": chain_floor(capi, 0), "beta": chain_floor(capi, 1),
+              "alpha_when_a_lane_takes_the_library_path": chain_floor(capi, 2)}
+    chain = {k: {"ns_per_step": round(per_launch[k] * 1e6 / walk_steps, 1),
+                 "floor_ns_per_step": round(floors[k], 1),
+                 "frac": round(floors[k] / (per_launch[k] * 1e6 / walk_steps), 4)}
+             for k in ("alpha", "beta") if k in per_launch}
+    chain["steps"] = walk_steps
+    chain["floor_alpha_library_path_ns_per_step"] = round(
+        floors["alpha_when_a_lane_takes_the_library_path"], 1)
+    walks_ms = per_launch.get("alpha", 0.0) + per_launch.get("beta", 0.0)
+    if walks_ms > mfma_kernels[dom]:
+        a = chain["alpha"]
+        roofline = {"bound": "chain-latency", "kernel": "alpha_kernel",
+                    "achieved": a["ns_per_step"], "peak": a["floor_ns_per_step"],
+                    "unit": "ns/step (lower is better; frac = peak / achieved)",
+                    "frac": a["frac"], "traffic": None,
+                    "kernel_ms": round(per_launch["alpha"], 4), "steps_per_launch": walk_steps,
+                    "walks": chain, "contractions": mfma_roofline}
+    else:
+        roofline = dict(mfma_roofline, walks=chain)
+
     out = {
-        "metric": METRIC + (" (%s scores and gradients)" % io if bf16 else ""),
+        "metric": METRIC + (" (%s scores and gradients)" % io if io else ""),
         "value": round(ms_per_step, 4),
         "unit": "ms",
         "n_gpus": 1,
@@ -304,39 +438,32 @@ def main():
         "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": False,
         "scaling": "weak",
-        "vs_baseline": (round(ms_per_step / w["published_ms"], 5) if w.get("published_ms")
+        "vs_baseline": (round(ms_per_step / opt["published_ms"], 5) if opt.get("published_ms")
                         else None),
-        "dtype": "f32 arithmetic on %s scores, %s gradients" % (io, io) if bf16 else "f32",
+        "dtype": "f32 arithmetic on %s scores, %s gradients" % (io, io) if io else "f32",
         "data": "synthetic",
-        "config": {"workload": "%s: B=%d T=%d U=%d V=%d blank=0, %s scores, input_lengths "
-                               "%s, label_lengths %s, deltas=1" %
-                               (args.workload, B, T, w["U"], V,
-                                "uniform [0,1)" if w.get("uniform") else "N(0,%g)" % w["sigma"],
-                                "U[%d,%d]" % w["ragged_T"] if w["ragged_T"] else "=T",
-                                "U[%d,%d]" % w["ragged_U"] if w["ragged_U"] else "=U"),
-                   "seed": args.seed, "valid_lattice_cells": int(cells)},
-        "roofline": {"bound": "mfma", "kernel": {"lse": "lse_stream_kernel",
-                                                 "egrads": "egrads_stream_kernel",
-                                                 "pgrads": "pgrads_stream_kernel"}[dom],
-                     "achieved": round(achieved, 2), "peak": PEAK_FP32_MATRIX_TFLOPS,
-                     "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP32_MATRIX_TFLOPS, 4),
-                     "traffic": RECORDED_TRAFFIC_BYTES.get(args.workload, {}).get(dom),
-                     "kernel_ms": round(mfma_kernels[dom], 4),
-                     "flops_per_launch": flops_one,
-                     "hbm": {"achieved": round(hbm_gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                             "frac": round(hbm_gbs / PEAK_HBM_GBS, 4),
-                             "bytes_per_launch": in_bytes + out_bytes[dom]},
-                     "all_kernels_frac_of_fp32_matrix_peak": {
-                         k: round(flops_one / (v * 1e-3) / 1e12 / PEAK_FP32_MATRIX_TFLOPS, 4)
-                         for k, v in mfma_kernels.items()}},
+        "config": {"workload": describe(args.workload, cfg, opt), "seed": args.seed,
+                   "valid_lattice_cells": int(cells)},
+        "roofline": roofline,
         "whole_step_frac_of_mfma_roofline": round(
             (flops_all / (PEAK_FP32_MATRIX_TFLOPS * 1e12)) / (ms_per_step * 1e-3), 4),
         "stage_ms_per_step": per_step,
+        "checks": checks,
     }
-    if not args.no_cpu_baseline and not bf16:  # the CPU path has no bf16 form
-        out["cpu_baseline"] = cpu_baseline(w, il, ll)
+    if not args.no_cpu_baseline and not io:  # the CPU path has no 16-bit form
+        out["cpu_baseline"], cpu = cpu_baseline(d)
+        if cpu is not None:  # the whole batch ran on the CPU: hold the device result to it
+            checks["against_cpu_baseline"] = {
+                "costs_outside_rel1e-4_abs1e-3": outside(costs.cpu().numpy(), cpu["costs"],
+                                                         atol=1e-3),
+                "egrads_outside_rel1e-4_abs1e-5": outside(egrads.cpu().numpy(), cpu["egrads"]),
+                "pgrads_outside_rel1e-4_abs1e-5": outside(pgrads.cpu().numpy(), cpu["pgrads"]),
+            }
+            checks["ok"] = checks["ok"] and \
+                checks["against_cpu_baseline"]["costs_outside_rel1e-4_abs1e-3"] == 0.0
     print(json.dumps(out))
+    return 0 if checks["ok"] else 1
 
 
 if __name__ == "__main__":
-    main()
+    sys.exit(main())

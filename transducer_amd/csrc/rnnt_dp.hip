@@ -13,6 +13,7 @@
 // lane, prefetched a group ahead.  This file is compiled with -ffp-contract=off: the rounding
 // sequence of every cell must equal the reference's.
 #include <mutex>
+#include <type_traits>
 
 #include "rnnt_internal.h"
 #include "rnnt_libm.h"
@@ -22,6 +23,11 @@ namespace rnnt {
 namespace {
 
 constexpr float kNegInf = -__builtin_huge_valf();
+// Score of a cell outside the lattice in the alpha walk: far below any alpha, so a log-sum-exp
+// returns the other operand untouched -- as -inf would -- but FINITE, so that two of them do
+// not meet as inf - inf (which only the library path can sort out, and an idle lane would then
+// send its whole wavefront there at every step).
+constexpr float kOutside = -1.0e30f;
 constexpr float kPosInf = __builtin_huge_valf();
 
 // lane L receives the value of lane L-1; lane 0 receives `fill`.
@@ -84,11 +90,15 @@ __device__ inline float lse2_libm(float a, float b, const unsigned long long* ta
 // r = fl(hi + l) with l = log1pf(expf(d)) at most log 2, and from a few hundred steps into a
 // lattice |hi| is in the thousands: the sum's spacing is then thousands of times the
 // uncertainty of a fast l, so nearly every fast sum is provably the library's sum.  Per lane:
-//   r = fl(hi + lf), t = (hi + lf) - r exactly (Fast2Sum: |hi| >= 1 > lf);
+//   r = fl(hi + lf), t = lf - (r - hi): the exact remainder (hi + lf) - r whenever |hi| >= lf;
 //   the library's sum rounds to the same r if |t| + bound(lf) stays below half the spacing of
-//   floats around r (and r is not a power of two, where the spacing below is half as wide).
-// Lanes that cannot show this take the library path; a wavefront skips it when none does
-// (Ziv's strategy).  Either way the result is the library's, bit for bit.
+//   floats on the narrower side of r (the spacing at the float just below |r|: halves when r is
+//   a power of two).
+// Where |hi| < lf the remainder is not exact, but then |r| < 2 lf, the half spacing is below
+// 2^-23 lf and bound(lf) >= 5 * 2^-23 lf alone exceeds it: the test fails by itself.  r = 0, NaN
+// operands and two operands of -inf (inf - inf) fail it too.  Lanes that fail take the library
+// path; a wavefront skips it when none does (Ziv's strategy).  Either way the result is the
+// library's, bit for bit.
 __device__ inline float lse2_checked(float a, float b, const unsigned long long* tab) {
   const float hi = a > b ? a : b;
   const float d = -fabsf(a - b);
@@ -96,14 +106,10 @@ __device__ inline float lse2_checked(float a, float b, const unsigned long long*
   float r = hi + lf;
   const float t = lf - (r - hi);
   const float bound = fast_bound(lf, d);
-  const int rb = __float_as_int(r);
-  const float half_spacing = __int_as_float((rb & 0x7f800000) - (24 << 23));
-  const bool safe = (fabsf(t) + bound < half_spacing) && (fabsf(hi) >= 1.0f) &&
-                    ((rb & 0x007fffff) != 0);
-  // Both operands -inf (a cell that has not started): the sum is -inf by the reference's early
-  // return, nothing to show.  NaN operands fail the comparisons and take the library path.
-  if (!safe && hi != kNegInf) r = lse2_libm(a, b, tab);
-  return (hi == kNegInf) ? kNegInf : r;
+  const int below = (__float_as_int(r) - 1) & 0x7f800000;  // exponent of the float below |r|
+  const float half_spacing = __int_as_float(below - (24 << 23));
+  if (!(fabsf(t) + bound < half_spacing)) r = lse2_libm(a, b, tab);
+  return r;
 }
 
 // The same on the hardware units alone (no check): for the chain-latency probe.
@@ -264,7 +270,7 @@ __global__ __launch_bounds__(64 * W) void alpha_kernel(Planes p, const int* __re
   exp2_table_to_lds(etab);
   if (W > 1) {
     if (threadIdx.x < W) done[threadIdx.x] = 0;
-    if (threadIdx.x < W - 1) hand[threadIdx.x * hand_stride] = kNegInf;  // nothing enters step 0
+    if (threadIdx.x < W - 1) hand[threadIdx.x * hand_stride] = kOutside;  // nothing enters step 0
   }
   __syncthreads();
   float* hand_out = hand + wave * hand_stride;                     // wave < W-1
@@ -287,8 +293,9 @@ __global__ __launch_bounds__(64 * W) void alpha_kernel(Planes p, const int* __re
     ap[c] = p.aS + row;
     pbv[c] = p.pb[(size_t)b * d.Ua + u0 + c];
     plv[c] = p.pl[(size_t)b * d.Ua + u0 + c];
-    stay[c] = kNegInf;
-    emit[c] = kNegInf;
+    // :43 alpha[0,0] = 0: cell (0,0) finds 0 coming up from below and nothing from the left
+    stay[c] = (u0 + c == 0) ? 0.0f : kOutside;
+    emit[c] = kOutside;
   }
 
   struct Group {
@@ -314,9 +321,11 @@ __global__ __launch_bounds__(64 * W) void alpha_kernel(Planes p, const int* __re
     // the empty asm statements only keep the compiler from moving LDS accesses across
     avail = bounded_wait(&done[wave - 1], avail, need, spin_limit, trouble);
   };
-  auto run_group = [&](int g, const Group& cur) {
+  // kWhole: all four steps of the group exist (every group but the last; no test per step)
+  auto run_group = [&](int g, const Group& cur, auto whole) {
+    constexpr bool kWhole = decltype(whole)::value;
     float4 aout[C];
-    float4 hin = {kNegInf, kNegInf, kNegInf, kNegInf};
+    float4 hin = {kOutside, kOutside, kOutside, kOutside};
     if (W > 1 && wave > 0) {
       wait_for(4 * g + 3);  // the scores entering steps 4g .. 4g+3 left steps 4g-1 .. 4g+2
       hin = *reinterpret_cast<const float4*>(hand_in + 4 * g);
@@ -325,14 +334,13 @@ __global__ __launch_bounds__(64 * W) void alpha_kernel(Planes p, const int* __re
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int s = 4 * g + j;
-      if (s < nsteps) {  // uniform; only the last group can be partial
-        float from_left = wave_shr1(emit[C - 1], kNegInf);
+      if (kWhole || s < nsteps) {  // uniform; a step past the last must not touch the scores
+        float from_left = wave_shr1(emit[C - 1], kOutside);
         if (W > 1) from_left = (lane == 0) ? f4get(hin, j) : from_left;
 #pragma unroll
         for (int c = C - 1; c >= 0; --c) {
           const float left = (c == 0) ? from_left : emit[c - 1];
-          float a = lse2_checked(left, stay[c], etab);
-          if (j == 0 && g == 0) a = (u0 + c == 0) ? 0.0f : a;  // :43
+          const float a = lse2_checked(left, stay[c], etab);
           const float ln = f4get(cur.ln[c], j);
           float sb = a + cur.eb[j - c + (C - 1)];
           sb = sb + pbv[c];
@@ -341,12 +349,12 @@ __global__ __launch_bounds__(64 * W) void alpha_kernel(Planes p, const int* __re
           se = se + plv[c];
           se = se - ln;
           // a cell of the lattice: 0 <= t = s - u < T_b (one unsigned comparison).  Cells before
-          // the first frame or past the last one hand -inf on, so whatever the planes hold
+          // the first frame or past the last one hand kOutside on, so whatever the planes hold
           // outside the utterance never enters a log-sum-exp (where it would cost the whole
           // wavefront the library path).
           const bool inside = (unsigned)(s - (u0 + c)) < tlim[c];
-          stay[c] = inside ? sb : kNegInf;
-          emit[c] = inside ? se : kNegInf;
+          stay[c] = inside ? sb : kOutside;
+          emit[c] = inside ? se : kOutside;
           f4set(aout[c], j, a);
         }
       }
@@ -368,16 +376,25 @@ __global__ __launch_bounds__(64 * W) void alpha_kernel(Planes p, const int* __re
   Group q0 = load_group(0), q1 = load_group(clamp_g(1)), q2 = load_group(clamp_g(2)),
         q3 = load_group(clamp_g(3));
   if (W > 1 && wave > 0) wait_for(min(4 * ngroups, 4 * 8 * wave));  // fall a few groups behind
-  for (int g = 0; g < ngroups; g += 4) {
-    run_group(g, q0);
+  const std::true_type whole;
+  const std::false_type partial;
+  const int nwhole = nsteps >> 2;  // groups with all four steps
+  int g = 0;
+  for (; g + 4 <= nwhole; g += 4) {
+    run_group(g, q0, whole);
     q0 = load_group(clamp_g(g + 4));
-    if (g + 1 < ngroups) run_group(g + 1, q1);
+    run_group(g + 1, q1, whole);
     q1 = load_group(clamp_g(g + 5));
-    if (g + 2 < ngroups) run_group(g + 2, q2);
+    run_group(g + 2, q2, whole);
     q2 = load_group(clamp_g(g + 6));
-    if (g + 3 < ngroups) run_group(g + 3, q3);
+    run_group(g + 3, q3, whole);
     q3 = load_group(clamp_g(g + 7));
   }
+  // the last one to four groups, the very last of which may be partial
+  if (g < ngroups) run_group(g, q0, partial);
+  if (g + 1 < ngroups) run_group(g + 1, q1, partial);
+  if (g + 2 < ngroups) run_group(g + 2, q2, partial);
+  if (g + 3 < ngroups) run_group(g + 3, q3, partial);
   // :73-78 the blank move out of the last cell, negated; that cell was the last one its
   // column processed
 #pragma unroll
@@ -1182,7 +1199,7 @@ __global__ __launch_bounds__(64) void chain_floor_kernel(float* __restrict__ sin
 #pragma unroll 4
   for (int s = 0; s < steps; ++s) {
     if (kKind != 1) {
-      const float left = wave_shr1(emit, kNegInf);
+      const float left = wave_shr1(emit, kOutside);
       const float a = kKind == 0 ? lse2_checked(left, stay, etab) : lse2_libm(left, stay, etab);
       float sb = a + e;
       sb = sb + p;
