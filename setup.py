@@ -27,18 +27,17 @@ def _load_build_module():
 
 
 class HipBuild(build_ext):
-    """Builds librnnt_hip.so, libtransducer.so and the _transducer module next to the sources;
-    a non-inplace build then copies them into build_lib."""
+    """Builds librnnt_hip.so, libtransducer.so and the _transducer module: next to the sources
+    with --inplace, else straight into build_lib (objects into build_temp), leaving the source
+    tree untouched."""
 
     def run(self):
-        _load_build_module().build_all()
-        if not self.inplace:
-            import glob
-            import shutil
-            dst = os.path.join(self.build_lib, "transducer_amd")
-            os.makedirs(dst, exist_ok=True)
-            for so in glob.glob(os.path.join(HERE, "transducer_amd", "*.so")):
-                shutil.copy2(so, dst)
+        build = _load_build_module()
+        if self.inplace:
+            build.build_all()
+        else:
+            build.build_all(out_dir=os.path.join(self.build_lib, "transducer_amd"),
+                            obj_dir=os.path.join(self.build_temp, "transducer_amd"))
 
     def get_outputs(self):
         return []

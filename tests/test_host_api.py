@@ -221,3 +221,27 @@ int main() {
                            "-o", str(exe), "-L", PKG, "-ltransducer", "-lrnnt_hip",
                            "-Wl,-rpath," + PKG])
     assert subprocess.check_output([str(exe)], text=True).strip() == "3"
+
+
+def test_setup_py_builds_an_importable_package_outside_the_source_tree(tmp_path):
+    """The counterpart of the reference's setup.py:23-73 (build_ext through CMake and a pybind11
+    fetched from the network): here build_ext drives hipcc and g++ directly.  A non-inplace
+    build must leave a package that imports and exports the C interface from its own copy of
+    the libraries, without touching the ones in the source tree."""
+    lib, tmp = str(tmp_path / "lib"), str(tmp_path / "tmp")
+    before = os.path.getmtime(os.path.join(PKG, "librnnt_hip.so"))
+    subprocess.check_call(
+        ["python", os.path.join(ROOT, "setup.py"), "-q", "build_py", "--build-lib", lib,
+         "build_ext", "--build-lib", lib, "--build-temp", tmp], cwd=ROOT,
+        stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
+    assert os.path.getmtime(os.path.join(PKG, "librnnt_hip.so")) == before
+    built = os.listdir(os.path.join(lib, "transducer_amd"))
+    assert "librnnt_hip.so" in built and "libtransducer.so" in built
+    assert any(f.startswith("_transducer") and f.endswith(".so") for f in built)
+    code = ("import os, transducer_amd; from transducer_amd import capi, _transducer; "
+            "assert os.path.dirname(capi.LIB_PATH) == os.path.dirname(transducer_amd.__file__); "
+            "print(capi.load().rnnt_hip_abi_version(), _transducer.__version__, "
+            "transducer_amd.__file__)")
+    env = dict(os.environ, PYTHONPATH=lib)
+    out = subprocess.check_output(["python", "-c", code], cwd=str(tmp_path), env=env, text=True)
+    assert out.split()[0] == "1" and lib in out.split()[2]

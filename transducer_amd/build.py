@@ -33,40 +33,50 @@ def _run(cmd):
     subprocess.check_call(cmd)
 
 
-def hip_library_path():
-    return os.path.join(HERE, "librnnt_hip.so")
+def hip_library_path(out_dir=HERE):
+    return os.path.join(out_dir, "librnnt_hip.so")
 
 
-def build_hip(verbose=True):
-    objs = []
+def build_hip(out_dir=HERE, obj_dir=CSRC):
+    """The translation units are compiled side by side (a handful of hipcc processes), then
+    linked."""
+    from concurrent.futures import ThreadPoolExecutor
+    os.makedirs(obj_dir, exist_ok=True)
+    jobs = []
     for src in HIP_SOURCES:
-        obj = os.path.join(CSRC, src.replace(".hip", ".o"))
-        _run(["hipcc"] + HIPCC_FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj])
-        objs.append(obj)
-    _run(["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", hip_library_path()] + objs)
+        obj = os.path.join(obj_dir, src.replace(".hip", ".o"))
+        jobs.append((["hipcc"] + HIPCC_FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj], obj))
+    workers = max(1, min(len(jobs), (os.cpu_count() or 2) // 2))
+    with ThreadPoolExecutor(workers) as pool:
+        list(pool.map(lambda job: _run(job[0]), jobs))
+    _run(["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", hip_library_path(out_dir)] +
+         [obj for _, obj in jobs])
 
 
-def build_cxx():
-    lib = os.path.join(HERE, "libtransducer.so")
+def build_cxx(out_dir=HERE):
+    lib = os.path.join(out_dir, "libtransducer.so")
     _run(["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-I", INCLUDE,
           os.path.join(CSRC, "transducer.cpp"), "-o", lib,
-          "-L", HERE, "-lrnnt_hip", "-Wl,-rpath,$ORIGIN"])
+          "-L", out_dir, "-lrnnt_hip", "-Wl,-rpath,$ORIGIN"])
 
 
-def build_pybind():
+def build_pybind(out_dir=HERE):
     import pybind11
     ext = sysconfig.get_config_var("EXT_SUFFIX")
-    out = os.path.join(HERE, "_transducer" + ext)
+    out = os.path.join(out_dir, "_transducer" + ext)
     _run(["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden",
           "-I", INCLUDE, "-I", pybind11.get_include(), "-I", sysconfig.get_paths()["include"],
           os.path.join(CSRC, "_transducer.cpp"), "-o", out,
-          "-L", HERE, "-ltransducer", "-lrnnt_hip", "-Wl,-rpath,$ORIGIN"])
+          "-L", out_dir, "-ltransducer", "-lrnnt_hip", "-Wl,-rpath,$ORIGIN"])
 
 
-def build_all():
-    build_hip()
-    build_cxx()
-    build_pybind()
+def build_all(out_dir=HERE, obj_dir=CSRC):
+    """out_dir: where the three libraries go (default: next to the sources, where the package
+    loads them from); obj_dir: where the object files go."""
+    os.makedirs(out_dir, exist_ok=True)
+    build_hip(out_dir, obj_dir)
+    build_cxx(out_dir)
+    build_pybind(out_dir)
 
 
 if __name__ == "__main__":

@@ -243,7 +243,8 @@ int fill(float* x, float v, int n, hipStream_t s) {
 // Scratch the best-path stages need (planes, the two max-plus planes, the decision table).
 size_t viterbi_scratch_bytes(const Dims& d) {
   const size_t plane = sizeof(float) * (size_t)d.B * d.Ua * d.Dp + 64;
-  return align_up(planes_bytes(d)) + 2 * align_up(plane) + align_up(viterbi_bits_bytes(d));
+  return align_up(planes_bytes(d, true)) + 2 * align_up(plane) +
+         align_up(viterbi_bits_bytes(d));
 }
 
 // `scratch` has viterbi_scratch_bytes(d) left to take (one allocation per call, made by the caller
@@ -257,7 +258,7 @@ int viterbi_impl(const TIO* E, const TIO* P, const float* LN, int* labels,
   const size_t plane = sizeof(float) * (size_t)d.B * d.Ua * d.Dp + 64;
   Planes p;
   if (ready) p = *ready;
-  else carve_planes(scratch.take(planes_bytes(d)), d, &p);
+  else carve_planes(scratch.take(planes_bytes(d, true)), d, &p, true);
   float* bestS = static_cast<float*>(scratch.take(plane));
   float* argS = static_cast<float*>(scratch.take(plane));
   unsigned long long* bits =
@@ -385,7 +386,7 @@ int lowp_viterbi_decode(const TIO* E, const TIO* P, const int* inLen, const int*
   void* ys = scratch.take(yb);
   // LN and the blank scores go straight into the lattice planes, as in the whole-loss path
   Planes p;
-  carve_planes(scratch.take(planes_bytes(d)), d, &p);
+  carve_planes(scratch.take(planes_bytes(d, true)), d, &p, true);
   RNNT_STAGE(kRowmax, launch_rowmax_pick_p(P, mP, nullptr, labLen, p, d, s));
   RNNT_STAGE(kYplanes, launch_yplanes(P, mP, ys, labLen, d, s));
   RNNT_STAGE(kLse, launch_lse_stream(E, mE, mP, nullptr, ys, inLen, labLen, d, s, nullptr, p.elS,
@@ -417,7 +418,7 @@ int decode_fp32(const float* E, const float* P, const int* inLen, const int* lab
   // LN and the blank scores go straight into the lattice planes, as in the whole-loss path
   // (no row-major LN, no transposing copy, no gather)
   Planes p;
-  carve_planes(scratch.take(planes_bytes(d)), d, &p);
+  carve_planes(scratch.take(planes_bytes(d, true)), d, &p, true);
   bool ln_in_plane = false;
   RNNT_TRY(log_norms_stages(E, P, mE, mP, nullptr, ys, inLen, labLen, d, s, &p, nullptr,
                             &ln_in_plane));

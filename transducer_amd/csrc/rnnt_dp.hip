@@ -1331,18 +1331,22 @@ int trouble_flag(int** out) {
 // ------------------------------------------------------------------ workspace layout
 static size_t align_up(size_t x) { return (x + 255) & ~(size_t)255; }
 
-size_t planes_bytes(const Dims& d) {
+size_t planes_bytes(const Dims& d, bool decode_only) {
   const size_t plane = align_up(sizeof(float) * (size_t)d.B * d.Ua * d.Dp + 64);
-  return 6 * plane + align_up(sizeof(float) * (size_t)d.B * d.Tp) +
+  return (decode_only ? 1 : 6) * plane + align_up(sizeof(float) * (size_t)d.B * d.Tp) +
          4 * align_up(sizeof(float) * (size_t)d.B * d.Ua);
 }
 
-void carve_planes(void* base, const Dims& d, Planes* p) {
+void carve_planes(void* base, const Dims& d, Planes* p, bool decode_only) {
   char* c = static_cast<char*>(base);
   const size_t plane = align_up(sizeof(float) * (size_t)d.B * d.Ua * d.Dp + 64);
   auto take = [&](size_t n) { float* r = reinterpret_cast<float*>(c); c += n; return r; };
-  p->lnS = take(plane); p->elS = take(plane); p->aS = take(plane);
-  p->wB = take(plane); p->wE = take(plane); p->dS = take(plane);
+  p->lnS = take(plane);
+  p->elS = p->aS = p->wB = p->wE = p->dS = nullptr;
+  if (!decode_only) {
+    p->elS = take(plane); p->aS = take(plane);
+    p->wB = take(plane); p->wE = take(plane); p->dS = take(plane);
+  }
   p->eb = take(align_up(sizeof(float) * (size_t)d.B * d.Tp));
   const size_t bu = align_up(sizeof(float) * (size_t)d.B * d.Ua);
   p->pb = take(bu); p->pl = take(bu); p->gB = take(bu); p->gL = take(bu);

@@ -117,8 +117,10 @@ int launch_libm_probe(const float* x, float* e, float* l, long n, hipStream_t s)
 // fast log-sum-exp fails, out[1] = max(out[1], bits of the largest distance / bound).
 int launch_lse_bound_check(unsigned lo, unsigned hi, unsigned* out, hipStream_t s);
 
-size_t planes_bytes(const Dims& d);
-void carve_planes(void* base, const Dims& d, Planes* p);
+// decode_only: just what the best-path walk reads (the LN plane and the small vectors); the
+// five other lattice planes are left out and their pointers null.
+size_t planes_bytes(const Dims& d, bool decode_only = false);
+void carve_planes(void* base, const Dims& d, Planes* p, bool decode_only = false);
 
 // ---------------------------------------------------------------- launchers (rnnt_dp.hip)
 int launch_skew(const float* src, float* dstS, const int* inLen, const int* labLen, const Dims& d,

@@ -162,8 +162,9 @@ __global__ __launch_bounds__(64 * kWaves, kWaves / 2) void lse_stream_kernel(
   if (tid == 0) moved = 0;
   // Picks: the lattice recursions need E[t, blank] and E[t, label_u] in the skewed planes.  Every
   // element of the tile's rows passes through the staging registers exactly once, so the thread
-  // that holds a wanted column copies it out then (first label tile only; elS == nullptr: off).
-  const bool picking = elS != nullptr && u0 == 0;
+  // that holds a wanted column copies it out then (first label tile only; ebv == nullptr: off;
+  // without labels only the blank column is wanted and elS is not touched).
+  const bool picking = ebv != nullptr && u0 == 0;
   const int nlab = (picking && labels != nullptr) ? min(Ub - 1, 1024) : 0;
   const int npick = picking ? nlab + 1 : 0;  // entry nlab is the blank column
   for (int u = tid; u < npick; u += kThreads)
