@@ -234,6 +234,75 @@ def test_long_label_axis_uses_more_cells_per_lane():
     assert np.array_equal(gpu_viterbi(c, LN), oracle.viterbi(E, P, LN, il, ll))
 
 
+@pytest.mark.parametrize("T,U,V", [(40, 1024, 9), (30, 1025, 9), (50, 1500, 7), (24, 2100, 520),
+                                   (300, 1300, 5)])
+def test_label_axis_longer_than_one_block_of_1024_positions(T, U, V):
+    """The lattice walks give a lane at most 16 label positions: 1024 per launch.  A longer axis
+    is walked block by block (alpha and the best path upwards, dalpha downwards), the scores of
+    the boundary column handed on through memory; the reference strides its loop instead
+    (transducer_cuda.cu:74,150,220).  U counts the rows of predictions: 1024 is the last single
+    block, 1025 the first double one, 2100 takes three; V = 520 also takes the whole loss
+    through the scattered blank / label terms (the folded ones stop at 1024 labels).  Same bars
+    as everywhere: the reference's bits at the boundary, the oracle's tolerance for the loss,
+    the exact path."""
+    cfg = small_config(2, T, U - 1, V, ragged=True)
+    E, P, labels, il, ll = unpack(make_inputs(cfg, seed=U))
+    il[0], ll[0] = T, U - 1          # one utterance uses every block, the other is ragged
+    ll[1] = min(ll[1], U - 1)
+    c = DeviceCase(E, P, labels, il, ll)
+    LN = oracle.log_norms_naive(E, P, il, ll)
+    costs_o, alphas_o = oracle.forward(E, P, LN, labels, il, ll)
+    costs, alphas = gpu_forward(c, LN)
+    assert_same_bits(costs, costs_o, what="costs")
+    assert_same_bits(alphas, alphas_o, what="alphas")
+    eg, pg, lng = gpu_backward(c, alphas, LN)
+    eg_o, pg_o, lng_o = oracle.backward(E, P, np.nan_to_num(alphas_o), LN, labels, il, ll)
+    assert_same_bits(lng, lng_o, what="lngrads")
+    assert_same_bits(eg, eg_o, what="egrads (sparse)")
+    assert_same_bits(pg, pg_o, what="pgrads (sparse)")
+    assert np.array_equal(gpu_viterbi(c, LN), oracle.viterbi(E, P, LN, il, ll))
+    # the whole loss on the device's own log-normaliser: fed that LN the oracle agrees in every
+    # entry; against the oracle's own LN a lattice this long along the label axis moves with the
+    # last bit of LN, and the bar is the spread of the reference's result between two summation
+    # orders of its own LN
+    costs, eg, pg = gpu_loss(c)
+    LNd = gpu_log_norms(c)
+    oc, oa = oracle.forward(E, P, LNd, labels, il, ll)
+    oeg, opg, olng = oracle.backward(E, P, np.nan_to_num(oa), LNd, labels, il, ll)
+    deg, dpg = oracle.accumulate_grads(E, P, oeg, opg, olng, LNd, il, ll)
+    assert_close(costs, oc, what="costs, shared LN")
+    # (the dense sums run over a thousand and more label positions here, in a dozen slices on
+    # the device and one sequential fp32 sum in the oracle: a few entries in ten thousand that
+    # are small differences of large terms land just outside; none is far off)
+    for got, ref, name in ((eg, deg, "egrads"), (pg, dpg, "pgrads")):
+        frac, worst = violations(got, ref)
+        print("%s, shared LN: %.4f%% outside, max abs err %.3g" % (name, 100 * frac, worst))
+        assert frac <= 1e-3 and violations(got, ref, rtol=1e-3, atol=1e-4)[0] == 0.0
+    # Against the oracle's OWN log-normaliser such a lattice (a thousand and more label
+    # positions, a handful of symbols) moves with the last bit of LN far more than the benchmark
+    # shapes do -- the reference's result does too when only the order of its LN sum changes --
+    # so end to end only the costs and a cap on the fraction are held here; the entry-wise bar
+    # is the shared-LN comparison above.
+    want = oracle.loss_and_grads(E, P, labels, il, ll)
+    assert_close(costs, want["costs"], rtol=1e-4, atol=1e-3, what="costs")
+    sep, sep8 = (oracle.loss_and_grads(E, P, labels, il, ll, lse=k) for k in ("sep", "sep8"))
+    for got, name in ((eg, "egrads"), (pg, "pgrads")):
+        spread = max(violations(sep[name], want[name])[0], violations(sep8[name], sep[name])[0])
+        frac, worst = violations(got, want[name])
+        print("%s: %.4f%% outside end to end (the reference's own spread between orders of its "
+              "LN sum: %.4f%%), max abs err %.3g" % (name, 100 * frac, 100 * spread, worst))
+        if V >= 64:  # (below that the eight partial sums of the second order hold one term each)
+            assert frac <= max(3 * spread, 4e-3)
+    import torch
+    from transducer_amd import capi
+    from util import ptr
+    out = torch.full((2, U - 1), -1, dtype=torch.int32, device="cuda:0")
+    capi.call("rnnt_hip_viterbi_decode", ptr(c.E), ptr(c.P), ptr(c.il), ptr(c.ll), ptr(out),
+              2, T, U, V, 0, None)
+    torch.cuda.synchronize()
+    assert np.array_equal(out.cpu().numpy(), oracle.viterbi(E, P, LNd, il, ll))
+
+
 # ------------------------------------------------------------------ log-normaliser
 @pytest.mark.parametrize("B,T,U,V,sigma", [(2, 70, 9, 31, 1.0), (1, 200, 101, 1000, 2.0),
                                            (3, 129, 130, 257, 1.0), (1, 64, 17, 4099, 3.0),

@@ -153,7 +153,8 @@ int log_norms_stages(const float* E, const float* P, float* mE, float* mP, float
                           "positions (B=%d T=%d U=%d)", d.B, d.T, d.U);
   // one pass over E: the streaming kernel finds its own per-frame reference and leaves it in mE
   // and, with `planes`, copies the blank / label scores out of the rows as they stream by
-  if (planes && d.U - 1 <= 1024) {
+  // (its pick list holds 1024 labels; without labels only the blank column is picked)
+  if (planes && (labels == nullptr || d.U - 1 <= 1024)) {
     RNNT_STAGE(kRowmax, launch_rowmax_pick_p(P, mP, labels, labLen, *planes, d, s));
     RNNT_STAGE(kYplanes, launch_yplanes(P, mP, scratch, labLen, d, s));
     // (with the flag the caller says it only needs LN in the lattice plane)
@@ -374,8 +375,6 @@ int lowp_viterbi_decode(const TIO* E, const TIO* P, const int* inLen, const int*
   const Dims d = make_dims(B, T, U, V, blank);
   RNNT_TRY(check_lowp_shape(d, false, who));
   if (!lse_stream_supported(E, d)) return fail(kInvalid, "%s: B*T*U too large", who);
-  if (U > 1024)
-    return fail(kInvalid, "%s: prediction length %d exceeds the supported maximum of 1024", who, U);
   Scratch scratch(s);
   const size_t yb = lse_scratch_bytes(d);
   RNNT_TRY(scratch.reserve(align_up(sizeof(float) * (size_t)B * T) +
@@ -405,18 +404,16 @@ int decode_fp32(const float* E, const float* P, const int* inLen, const int* lab
   if (!E || !P || !labels || !inLen || !labLen)
     return fail(kInvalid, "%s: null array argument", who);
   const Dims d = make_dims(B, T, U, V, blank);
-  if (U > 1024)
-    return fail(kInvalid, "%s: prediction length %d exceeds the supported maximum of 1024", who, U);
   if (!lse_stream_supported(E, d)) return fail(kInvalid, "%s: B*T*U too large", who);
   const size_t yb = lse_scratch_bytes(d);
+  // LN and the blank scores go straight into the lattice planes, as in the whole-loss path
+  // (no row-major LN, no transposing copy, no gather)
   RNNT_TRY(scratch.reserve(align_up(sizeof(float) * (size_t)B * T) +
                            align_up(sizeof(float) * (size_t)B * U) + align_up(yb) +
                            viterbi_scratch_bytes(d)));
   float* mE = static_cast<float*>(scratch.take(sizeof(float) * (size_t)B * T));
   float* mP = static_cast<float*>(scratch.take(sizeof(float) * (size_t)B * U));
   void* ys = scratch.take(yb);
-  // LN and the blank scores go straight into the lattice planes, as in the whole-loss path
-  // (no row-major LN, no transposing copy, no gather)
   Planes p;
   carve_planes(scratch.take(planes_bytes(d, true)), d, &p, true);
   bool ln_in_plane = false;
@@ -740,7 +737,9 @@ int rnnt_hip_loss_backward(const float* E, const float* P, const int* labels, co
   // (not with a small vocabulary: many labels then fall into one wavefront's 32 columns and
   // their terms queue up in the dense kernel -- B=8 V=100: 0.17 ms folded, 0.03 + 0.04 ms
   // scattered; from V=1000 on folding is level or ahead)
-  const bool fold = labels != nullptr && d.V >= 512;
+  // (and not with more than 1024 labels: the dense kernel's per-wavefront match list holds
+  // that many)
+  const bool fold = labels != nullptr && d.V >= 512 && d.U - 1 <= 1024;
   RNNT_STAGE(kWplanes, launch_post_beta(w.planes, w.mE, w.mP, w.Wn, w.Wt,
                                         fold ? w.bsum : nullptr, labels, inLen, labLen, d, s));
   SparseTerms sp;

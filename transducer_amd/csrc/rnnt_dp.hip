@@ -246,12 +246,19 @@ __global__ __launch_bounds__(256) void gather_kernel(const TIO* __restrict__ E,
 // got; the upper one runs a few groups behind, so it finds its inputs there without waiting and
 // re-reads the progress counter only once every few groups.  The lowest
 // wavefront waits for nobody and every wavefront runs all groups, so the waits are bounded.
+// A label axis longer than one workgroup's 64 C W positions is walked block by block, one launch
+// per block of 64 C W positions (u_base = its first one), lowest block first.  The only values
+// that cross a block boundary are the label-move scores of the block's last column, one per
+// step: a launch leaves them in `ghout` ([B][hand_stride], entry s = score entering step s;
+// null for the last block) and the next one reads them from `ghin` (null for the first block).
 template <int C, int W>
 __global__ __launch_bounds__(64 * W) void alpha_kernel(Planes p, const int* __restrict__ inLen,
                                                        const int* __restrict__ labLen,
                                                        float* __restrict__ costs, Dims d,
                                                        int hand_stride, int spin_limit,
-                                                       int* __restrict__ trouble) {
+                                                       int* __restrict__ trouble, int u_base,
+                                                       const float* __restrict__ ghin,
+                                                       float* __restrict__ ghout) {
   extern __shared__ __attribute__((aligned(16))) float hand[];  // [W-1][hand_stride]: entry s =
                                                                 // score handed to step s
   __shared__ int done[W];          // steps a wavefront has published
@@ -261,12 +268,16 @@ __global__ __launch_bounds__(64 * W) void alpha_kernel(Planes p, const int* __re
   int Tb, Ub;
   utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
   if (Tb == 0 || Ub == 0) {  // :39-41
-    if (threadIdx.x == 0) costs[b] = kPosInf;
+    if (threadIdx.x == 0 && u_base == 0) costs[b] = kPosInf;
     return;
   }
+  if (u_base >= Ub) return;  // a block past this utterance's labels: nobody reads what it would leave
   const int nsteps = Tb + Ub - 1;
   const int ngroups = (nsteps + 3) >> 2;
-  const int u0 = (wave * 64 + lane) * C;
+  const int u0 = u_base + (wave * 64 + lane) * C;
+  const float* gin = ghin ? ghin + (size_t)b * hand_stride : nullptr;
+  float* gout = ghout ? ghout + (size_t)b * hand_stride : nullptr;
+  if (gout && threadIdx.x == 0) gout[0] = kOutside;  // nothing enters step 0
   exp2_table_to_lds(etab);
   if (W > 1) {
     if (threadIdx.x < W) done[threadIdx.x] = 0;
@@ -301,6 +312,7 @@ __global__ __launch_bounds__(64 * W) void alpha_kernel(Planes p, const int* __re
   struct Group {
     float4 ln[C], el[C];
     float eb[C + 3];
+    float4 gh;  // scores entering the block's first column from the block below
   };
   auto load_group = [&](int g) -> Group {
     Group r;
@@ -311,6 +323,8 @@ __global__ __launch_bounds__(64 * W) void alpha_kernel(Planes p, const int* __re
     }
 #pragma unroll
     for (int k = 0; k < C + 3; ++k) r.eb[k] = ebl[4 * g + k - (C - 1)];
+    r.gh = make_float4(kOutside, kOutside, kOutside, kOutside);
+    if (gin) r.gh = *reinterpret_cast<const float4*>(gin + 4 * g);  // uniform
     return r;
   };
 
@@ -325,18 +339,20 @@ __global__ __launch_bounds__(64 * W) void alpha_kernel(Planes p, const int* __re
   auto run_group = [&](int g, const Group& cur, auto whole) {
     constexpr bool kWhole = decltype(whole)::value;
     float4 aout[C];
-    float4 hin = {kOutside, kOutside, kOutside, kOutside};
+    float4 hin = cur.gh;  // wavefront 0: from the block below (or nothing)
     if (W > 1 && wave > 0) {
       wait_for(4 * g + 3);  // the scores entering steps 4g .. 4g+3 left steps 4g-1 .. 4g+2
       hin = *reinterpret_cast<const float4*>(hand_in + 4 * g);
     }
     float hout[4];
+    float gsend[4];  // what this lane's last column hands to the right after each step
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int s = 4 * g + j;
+      gsend[j] = kOutside;
       if (kWhole || s < nsteps) {  // uniform; a step past the last must not touch the scores
         float from_left = wave_shr1(emit[C - 1], kOutside);
-        if (W > 1) from_left = (lane == 0) ? f4get(hin, j) : from_left;
+        if (W > 1 || gin) from_left = (lane == 0) ? f4get(hin, j) : from_left;
 #pragma unroll
         for (int c = C - 1; c >= 0; --c) {
           const float left = (c == 0) ? from_left : emit[c - 1];
@@ -357,12 +373,17 @@ __global__ __launch_bounds__(64 * W) void alpha_kernel(Planes p, const int* __re
           emit[c] = inside ? se : kOutside;
           f4set(aout[c], j, a);
         }
+        gsend[j] = emit[C - 1];
       }
       if (W > 1)
         hout[j] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(emit[C - 1]), 63));
     }
 #pragma unroll
     for (int c = 0; c < C; ++c) *reinterpret_cast<float4*>(ap[c] + 4 * g) = aout[c];
+    if (gout && wave == W - 1 && lane == 63) {  // entries 4g+1 .. 4g+4 for the block above
+#pragma unroll
+      for (int j = 0; j < 4; ++j) gout[4 * g + 1 + j] = gsend[j];
+    }
     if (W > 1 && wave < W - 1 && lane == 0) {  // entries 4g+1 .. 4g+4, then the progress
 #pragma unroll
       for (int j = 0; j < 4; ++j) hand_out[4 * g + 1 + j] = hout[j];
@@ -401,6 +422,7 @@ __global__ __launch_bounds__(64 * W) void alpha_kernel(Planes p, const int* __re
   for (int c = 0; c < C; ++c)
     if (u0 + c == Ub - 1) costs[b] = -stay[c];
 }
+
 
 // ------------------------------------------------------------------ transition weights
 // Everything of the dalpha recursion that does not depend on dalpha itself
@@ -448,17 +470,29 @@ __global__ __launch_bounds__(256) void weights_kernel(Planes p, const int* __res
 // keeps the running sums that the reference subtracts from pgrads[u,blank] and pgrads[u,l_u],
 // in the reference's own order (t descending).  Operands are prefetched two groups of four
 // steps ahead through three rotating register sets.
+// A label axis longer than 64 C positions is walked block by block (u_base = first position of
+// the block), HIGHEST block first: what crosses a boundary here is dalpha of the upper block's
+// first column, one value per diagonal, left in `ghout` ([B][hand_stride], entry s = its dalpha
+// on diagonal s; null for the lowest block) and read by the block below from `ghin` (null for
+// the highest block).
 template <int C>
 __global__ __launch_bounds__(64) void beta_kernel(Planes p, const int* __restrict__ labels,
                                                   const int* __restrict__ inLen,
-                                                  const int* __restrict__ labLen, Dims d) {
+                                                  const int* __restrict__ labLen, Dims d,
+                                                  int hand_stride, int u_base,
+                                                  const float* __restrict__ ghin,
+                                                  float* __restrict__ ghout) {
   const int b = blockIdx.x, lane = threadIdx.x;
   int Tb, Ub;
   utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
   if (Tb == 0 || Ub == 0) return;  // :92-94
+  if (u_base >= Ub) return;        // a block past this utterance's labels
   const int nsteps = Tb + Ub - 1;
   const int last = nsteps - 1;  // diagonal of the last cell
-  const int u0 = lane * C;
+  const int u0 = u_base + lane * C;
+  // the block above exists for this utterance only if its first column does
+  const float* gin = (ghin && u_base + 64 * C < Ub) ? ghin + (size_t)b * hand_stride : nullptr;
+  float* gout = ghout ? ghout + (size_t)b * hand_stride : nullptr;
 
   float dcol[C], accB[C], accL[C];
   bool fold[C];  // label of this position equals blank: both sums share one accumulator
@@ -480,6 +514,7 @@ __global__ __launch_bounds__(64) void beta_kernel(Planes p, const int* __restric
 
   struct Group {
     float4 wb[C], we[C];
+    float gh[4];  // dalpha of the block above's first column on diagonals 4g+1 .. 4g+4
   };
   auto load_group = [&](int g) -> Group {
     Group r;
@@ -489,20 +524,27 @@ __global__ __launch_bounds__(64) void beta_kernel(Planes p, const int* __restric
       r.wb[c] = *reinterpret_cast<const float4*>(wbp[c] + 4 * gc);
       r.we[c] = *reinterpret_cast<const float4*>(wep[c] + 4 * gc);
     }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) r.gh[j] = gin ? gin[4 * gc + 1 + j] : 0.0f;  // uniform
     return r;
   };
   // steps last-1 .. 0 are computed; the slot of step `last` receives the seed and the slots
   // after it (same group of four) zeros
   auto run_group = [&](int g, const Group& w) {
     float4 dout[C];
+    float gsend[4];  // dalpha of this lane's first column after each step
 #pragma unroll
     for (int j = 3; j >= 0; --j) {
       const int s = 4 * g + j;
       if (s >= last) {  // uniform; only in the first group run
 #pragma unroll
         for (int c = 0; c < C; ++c) f4set(dout[c], j, s == last ? dcol[c] : 0.0f);
+        gsend[j] = s == last ? dcol[0] : 0.0f;
       } else {
-        const float from_right = wave_shl1(dcol[0], 0.0f);
+        float from_right = wave_shl1(dcol[0], 0.0f);
+        // the column right of lane 63's last one belongs to the block above: its dalpha on the
+        // diagonal just done, s + 1
+        if (gin) from_right = (lane == 63) ? w.gh[j] : from_right;
 #pragma unroll
         for (int c = 0; c < C; ++c) {
           const float right = (c == C - 1) ? from_right : dcol[c + 1];
@@ -515,10 +557,15 @@ __global__ __launch_bounds__(64) void beta_kernel(Planes p, const int* __restric
           dcol[c] = dn;
           f4set(dout[c], j, dn);
         }
+        gsend[j] = dcol[0];
       }
     }
 #pragma unroll
     for (int c = 0; c < C; ++c) *reinterpret_cast<float4*>(dp[c] + 4 * g) = dout[c];
+    if (gout && lane == 0) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) gout[4 * g + j] = gsend[j];
+    }
   };
 
   int g = last >> 2;  // the group that holds the seed
@@ -1020,7 +1067,10 @@ __global__ __launch_bounds__(64 * W) void viterbi_kernel(Planes p, const float* 
                                                          unsigned* __restrict__ gcols,
                                                          int* __restrict__ labels_out, Dims d,
                                                          int hand_stride, int nw, int spin_limit,
-                                                         int* __restrict__ trouble) {
+                                                         int* __restrict__ trouble, int u_base,
+                                                         const float* __restrict__ ghin,
+                                                         float* __restrict__ ghout,
+                                                         int traces) {
   extern __shared__ __attribute__((aligned(16))) int dyn[];
   __shared__ int done[W];  // steps a wavefront has published
   const int b = blockIdx.x, lane = threadIdx.x & 63, tidx = threadIdx.x;
@@ -1028,13 +1078,21 @@ __global__ __launch_bounds__(64 * W) void viterbi_kernel(Planes p, const float* 
   int Tb, Ub;
   utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
   if (Tb == 0 || Ub == 0) return;  // :152-154
+  // A label axis longer than 64 C W positions is walked block by block, lowest first, as in
+  // alpha_kernel (u_base, ghin, ghout); the decision columns then live in global memory and the
+  // launch of the highest block (traces != 0) follows the path back through all of them.
+  const bool walks = u_base < Ub;
+  if (!walks && !traces) return;
   const int nsteps = Tb + Ub - 1;
   const int ngroups = (nsteps + 3) >> 2;
   int* taken = dyn;                                                   // [U rounded up to 4]
   float* hand = reinterpret_cast<float*>(dyn + ((d.U + 3) & ~3));     // [W-1][hand_stride]
   unsigned* cols = kLdsBits
       ? reinterpret_cast<unsigned*>(hand + (W - 1) * hand_stride)     // [64 C W][nw]
-      : gcols + (size_t)b * (64 * C * W) * nw;
+      : gcols + (size_t)b * d.Ua * nw;                                // [Ua][nw]
+  const float* gin = ghin ? ghin + (size_t)b * hand_stride : nullptr;
+  float* gout = (ghout && walks) ? ghout + (size_t)b * hand_stride : nullptr;
+  if (gout && tidx == 0) gout[0] = kNegInf;  // nothing enters step 0
   if (W > 1) {
     if (tidx < W) done[tidx] = 0;
     if (tidx < W - 1) hand[tidx * hand_stride] = kNegInf;  // nothing enters step 0
@@ -1043,7 +1101,7 @@ __global__ __launch_bounds__(64 * W) void viterbi_kernel(Planes p, const float* 
   __syncthreads();
   float* hand_out = hand + wave * hand_stride;                            // wave < W-1
   const float* hand_in = hand + (wave > 0 ? wave - 1 : 0) * hand_stride;  // wave > 0
-  const int u0 = (wave * 64 + lane) * C;
+  const int u0 = u_base + (wave * 64 + lane) * C;
   // E[t,blank] for the cells of step s sits at ebl[s - u]; column c at step 4g+j reads
   // ebl[4g + j - c], so one run of C+3 values serves all columns of a group
   const float* ebl = p.eb + (size_t)b * d.Tp + d.Eo - u0;
@@ -1066,6 +1124,7 @@ __global__ __launch_bounds__(64 * W) void viterbi_kernel(Planes p, const float* 
   struct Group {
     float4 ln[C], bs[C];
     float eb[C + 3];
+    float4 gh;  // scores entering the block's first column from the block below
   };
   auto load_group = [&](int g) -> Group {
     Group r;
@@ -1076,6 +1135,8 @@ __global__ __launch_bounds__(64 * W) void viterbi_kernel(Planes p, const float* 
     }
 #pragma unroll
     for (int k = 0; k < C + 3; ++k) r.eb[k] = ebl[4 * g + k - (C - 1)];
+    r.gh = make_float4(kNegInf, kNegInf, kNegInf, kNegInf);
+    if (gin) r.gh = *reinterpret_cast<const float4*>(gin + 4 * g);  // uniform
     return r;
   };
   int avail = 0;  // steps the wavefront below is known to have published (see alpha_kernel)
@@ -1085,18 +1146,19 @@ __global__ __launch_bounds__(64 * W) void viterbi_kernel(Planes p, const float* 
   // A cell that has not started (t < 0) keeps -inf scores and never takes a label; cells past
   // the utterance run on whatever the planes hold and are never consulted by the backtrace.
   auto run_group = [&](int g, const Group& cur) {
-    float4 hin = {kNegInf, kNegInf, kNegInf, kNegInf};
+    float4 hin = cur.gh;  // wavefront 0: from the block below (or nothing)
     if (W > 1 && wave > 0) {
       wait_for(4 * g + 3);
       hin = *reinterpret_cast<const float4*>(hand_in + 4 * g);
     }
     float hout[4];
+    float gsend[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int s = 4 * g + j;
       const unsigned sbit = 1u << (s & 31);  // uniform
       float from_left = wave_shr1(emit[C - 1], kNegInf);
-      if (W > 1) from_left = (lane == 0) ? f4get(hin, j) : from_left;
+      if (W > 1 || gin) from_left = (lane == 0) ? f4get(hin, j) : from_left;
 #pragma unroll
       for (int c = C - 1; c >= 0; --c) {
         const float left = (c == 0) ? from_left : emit[c - 1];
@@ -1114,8 +1176,13 @@ __global__ __launch_bounds__(64 * W) void viterbi_kernel(Planes p, const float* 
         stay[c] = started ? sb : kNegInf;
         emit[c] = started ? se : kNegInf;
       }
+      gsend[j] = emit[C - 1];
       if (W > 1)
         hout[j] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(emit[C - 1]), 63));
+    }
+    if (gout && wave == W - 1 && lane == 63) {  // entries 4g+1 .. 4g+4 for the block above
+#pragma unroll
+      for (int j = 0; j < 4; ++j) gout[4 * g + 1 + j] = gsend[j];
     }
     if ((g & 7) == 7 || g == ngroups - 1) {  // uniform: a word of 32 steps is complete
 #pragma unroll
@@ -1135,8 +1202,9 @@ __global__ __launch_bounds__(64 * W) void viterbi_kernel(Planes p, const float* 
   auto clamp_g = [&](int g) { return g < ngroups ? g : ngroups - 1; };
   Group q0 = load_group(0), q1 = load_group(clamp_g(1)), q2 = load_group(clamp_g(2)),
         q3 = load_group(clamp_g(3));
-  if (W > 1 && wave > 0) wait_for(min(4 * ngroups, 4 * 8 * wave));  // fall a few groups behind
-  for (int g = 0; g < ngroups; g += 4) {
+  const int nwalk = walks ? ngroups : 0;  // a block past the utterance's labels only traces
+  if (W > 1 && wave > 0 && walks) wait_for(min(4 * ngroups, 4 * 8 * wave));  // fall a few groups behind
+  for (int g = 0; g < nwalk; g += 4) {
     run_group(g, q0);
     q0 = load_group(clamp_g(g + 4));
     if (g + 1 < ngroups) run_group(g + 1, q1);
@@ -1148,6 +1216,7 @@ __global__ __launch_bounds__(64 * W) void viterbi_kernel(Planes p, const float* 
   }
   if (!kLdsBits) __threadfence();  // the columns in global memory, before another lane reads them
   __syncthreads();
+  if (!traces) return;
   // Backtrace (:208-219): from (T_b - 1, U_b - 1); a set bit at (step, u) means "entered from
   // u - 1 with a label", a clear one "entered from t - 1 with a blank".
   if (tidx == 0) {
@@ -1334,7 +1403,8 @@ static size_t align_up(size_t x) { return (x + 255) & ~(size_t)255; }
 size_t planes_bytes(const Dims& d, bool decode_only) {
   const size_t plane = align_up(sizeof(float) * (size_t)d.B * d.Ua * d.Dp + 64);
   return (decode_only ? 1 : 6) * plane + align_up(sizeof(float) * (size_t)d.B * d.Tp) +
-         4 * align_up(sizeof(float) * (size_t)d.B * d.Ua);
+         4 * align_up(sizeof(float) * (size_t)d.B * d.Ua) +
+         2 * align_up(sizeof(float) * (size_t)d.B * d.Dp);
 }
 
 void carve_planes(void* base, const Dims& d, Planes* p, bool decode_only) {
@@ -1350,6 +1420,8 @@ void carve_planes(void* base, const Dims& d, Planes* p, bool decode_only) {
   p->eb = take(align_up(sizeof(float) * (size_t)d.B * d.Tp));
   const size_t bu = align_up(sizeof(float) * (size_t)d.B * d.Ua);
   p->pb = take(bu); p->pl = take(bu); p->gB = take(bu); p->gL = take(bu);
+  const size_t bh = align_up(sizeof(float) * (size_t)d.B * d.Dp);
+  p->hand[0] = take(bh); p->hand[1] = take(bh);
 }
 
 // ------------------------------------------------------------------ launchers
@@ -1401,32 +1473,46 @@ int launch_gather(const f16_t* E, const f16_t* P, const int* labels, const int* 
   return gather_any(E, P, labels, inLen, labLen, p, d, s);
 }
 
+// Label positions one launch of a lattice walk covers: the whole axis up to 1024, else blocks of
+// 1024 (64 lanes x 16 positions), one launch per block.
+static int block_cells_per_lane(const Dims& d) { return min(cells_per_lane(d.U), 16); }
+static int label_blocks(const Dims& d) {
+  const int width = 64 * block_cells_per_lane(d);
+  return (d.U + width - 1) / width;
+}
+
 int launch_alpha(const Planes& p, const int* inLen, const int* labLen, float* costs,
                  const Dims& d, hipStream_t s) {
   if (d.B == 0) return kOk;
   // cells per lane of a single wavefront; split over two wavefronts when the hand-over
   // array (one float per step and boundary) fits LDS
-  const int cpl = cells_per_lane(d.U);
-  const int stride = ((d.T + d.U + 3) & ~3) + 8;
+  const int cpl = block_cells_per_lane(d), nblocks = label_blocks(d);
+  const int stride = d.Dp;
   // (two wavefronts, not four: every lane reads its own plane row, 64 cache lines per load
   // instruction, and with four wavefronts the CU's vector memory pipeline becomes the limit)
   const int W = (cpl >= 2 && stride * sizeof(float) <= 48 * 1024) ? 2 : 1;
   const size_t lds = W > 1 ? sizeof(float) * (size_t)(W - 1) * stride : 0;
   int* trouble = nullptr;
   RNNT_TRY(trouble_flag(&trouble));
-  switch (cpl / W * 100 + W) {
+  for (int k = 0; k < nblocks; ++k) {  // lowest block first
+    const float* ghin = k == 0 ? nullptr : p.hand[(k - 1) & 1];
+    float* ghout = k == nblocks - 1 ? nullptr : p.hand[k & 1];
+    const int u_base = k * 64 * cpl;
+    switch (cpl / W * 100 + W) {
 #define CASE(C, W)                                                                          \
   case C * 100 + W:                                                                         \
     hipLaunchKernelGGL((alpha_kernel<C, W>), dim3(d.B), dim3(64 * W), lds, s, p, inLen,    \
-                       labLen, costs, d, stride, g_spin_limit, trouble);                    \
+                       labLen, costs, d, stride, g_spin_limit, trouble, u_base, ghin,       \
+                       ghout);                                                              \
     break;
-    CASE(1, 1) CASE(2, 1) CASE(4, 1) CASE(8, 1) CASE(16, 1)
-    CASE(1, 2) CASE(2, 2) CASE(4, 2) CASE(8, 2)
+      CASE(1, 1) CASE(2, 1) CASE(4, 1) CASE(8, 1) CASE(16, 1)
+      CASE(1, 2) CASE(2, 2) CASE(4, 2) CASE(8, 2)
 #undef CASE
-    default:
-      return fail(kInvalid, "prediction length %d exceeds the supported maximum of 1024", d.U);
+      default:
+        return fail(kInvalid, "alpha: no kernel for %d label positions per lane", cpl);
+    }
+    RNNT_LAUNCH_CHECK("alpha_kernel");
   }
-  RNNT_LAUNCH_CHECK("alpha_kernel");
   return kOk;
 }
 
@@ -1442,17 +1528,24 @@ int launch_weights(const Planes& p, const int* inLen, const int* labLen, const D
 int launch_beta(const Planes& p, const int* labels, const int* inLen, const int* labLen,
                 const Dims& d, hipStream_t s) {
   if (d.B == 0 || d.T == 0 || d.U == 0) return kOk;
-  switch (cells_per_lane(d.U)) {
-#define CASE(C)                                                                              \
-  case C:                                                                                    \
-    hipLaunchKernelGGL(beta_kernel<C>, dim3(d.B), dim3(64), 0, s, p, labels, inLen, labLen, d); \
+  const int cpl = block_cells_per_lane(d), nblocks = label_blocks(d);
+  for (int k = nblocks - 1; k >= 0; --k) {  // highest block first
+    const float* ghin = k == nblocks - 1 ? nullptr : p.hand[(k + 1) & 1];
+    float* ghout = k == 0 ? nullptr : p.hand[k & 1];
+    const int u_base = k * 64 * cpl;
+    switch (cpl) {
+#define CASE(C)                                                                                \
+  case C:                                                                                      \
+    hipLaunchKernelGGL(beta_kernel<C>, dim3(d.B), dim3(64), 0, s, p, labels, inLen, labLen, d, \
+                       d.Dp, u_base, ghin, ghout);                                             \
     break;
-    CASE(1) CASE(2) CASE(4) CASE(8) CASE(16)
+      CASE(1) CASE(2) CASE(4) CASE(8) CASE(16)
 #undef CASE
-    default:
-      return fail(kInvalid, "prediction length %d exceeds the supported maximum of 1024", d.U);
+      default:
+        return fail(kInvalid, "dalpha: no kernel for %d label positions per lane", cpl);
+    }
+    RNNT_LAUNCH_CHECK("beta_kernel");
   }
-  RNNT_LAUNCH_CHECK("beta_kernel");
   return kOk;
 }
 
@@ -1528,38 +1621,47 @@ int launch_viterbi(const Planes& p, const float* bestS, const float* argS,
                    int* labels_out, const Dims& d, hipStream_t s) {
   if (d.B == 0 || d.T == 0 || d.U <= 1) return kOk;
   unsigned* gcols = reinterpret_cast<unsigned*>(gbits);
-  const int cpl = cells_per_lane(d.U);
-  const int stride = ((d.T + d.U + 3) & ~3) + 8;
+  const int cpl = block_cells_per_lane(d), nblocks = label_blocks(d);
+  const int stride = d.Dp;
   const int nw = viterbi_words(d);
   const int W = (cpl >= 2 && stride * sizeof(float) <= 16 * 1024) ? 2 : 1;
   // dynamic LDS: one int per label position, the hand-over array between the two wavefronts,
-  // and the decision columns when they fit
+  // and the decision columns when they fit (one block only: with several, every block's columns
+  // must be there for the backtrace of the last launch)
   const size_t base_lds = sizeof(int) * (size_t)((d.U + 3) & ~3) +
                           (W > 1 ? sizeof(float) * (size_t)(W - 1) * stride : 0);
   const size_t cols_lds = sizeof(unsigned) * (size_t)64 * cpl * nw;
-  const bool use_lds = base_lds + cols_lds <= 60 * 1024;
+  const bool use_lds = nblocks == 1 && base_lds + cols_lds <= 60 * 1024;
   const size_t lds = base_lds + (use_lds ? cols_lds : 0);
+  if (lds > 64 * 1024)
+    return fail(kInvalid, "viterbi: %d label positions and %d steps need %zu bytes of LDS", d.U,
+                stride, lds);
   int* trouble = nullptr;
   RNNT_TRY(trouble_flag(&trouble));
-  switch (cpl / W * 100 + W) {
+  for (int k = 0; k < nblocks; ++k) {  // lowest block first; the last launch traces the path
+    const float* ghin = k == 0 ? nullptr : p.hand[(k - 1) & 1];
+    float* ghout = k == nblocks - 1 ? nullptr : p.hand[k & 1];
+    const int u_base = k * 64 * cpl, traces = k == nblocks - 1 ? 1 : 0;
+    switch (cpl / W * 100 + W) {
 #define CASE(C, W)                                                                             \
   case C * 100 + W:                                                                            \
     if (use_lds)                                                                               \
       hipLaunchKernelGGL((viterbi_kernel<C, W, true>), dim3(d.B), dim3(64 * W), lds, s, p,    \
                          bestS, argS, inLen, labLen, gcols, labels_out, d, stride, nw,         \
-                         g_spin_limit, trouble);                                               \
+                         g_spin_limit, trouble, u_base, ghin, ghout, traces);                  \
     else                                                                                       \
       hipLaunchKernelGGL((viterbi_kernel<C, W, false>), dim3(d.B), dim3(64 * W), lds, s, p,   \
                          bestS, argS, inLen, labLen, gcols, labels_out, d, stride, nw,         \
-                         g_spin_limit, trouble);                                               \
+                         g_spin_limit, trouble, u_base, ghin, ghout, traces);                  \
     break;
-    CASE(1, 1) CASE(2, 1) CASE(4, 1) CASE(8, 1) CASE(16, 1)
-    CASE(1, 2) CASE(2, 2) CASE(4, 2) CASE(8, 2)
+      CASE(1, 1) CASE(2, 1) CASE(4, 1) CASE(8, 1) CASE(16, 1)
+      CASE(1, 2) CASE(2, 2) CASE(4, 2) CASE(8, 2)
 #undef CASE
-    default:
-      return fail(kInvalid, "prediction length %d exceeds the supported maximum of 1024", d.U);
+      default:
+        return fail(kInvalid, "viterbi: no kernel for %d label positions per lane", cpl);
+    }
+    RNNT_LAUNCH_CHECK("viterbi_kernel");
   }
-  RNNT_LAUNCH_CHECK("viterbi_kernel");
   return kOk;
 }
 

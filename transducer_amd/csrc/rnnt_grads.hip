@@ -39,7 +39,7 @@ constexpr int kEsPitch = 16 * kEsMaxS + 8;  // LDS row pitch of a W-slab plane i
                                             // 16-byte reads of 8 consecutive rows spread over all banks)
 constexpr int kEsPlane = 32 * kEsPitch;
 constexpr int kEsPrefetch = 2;          // labels per 32-column block whose sparse terms are prefetched
-constexpr int kMaxLabels = 1024;        // longest label axis the lattice kernels take
+constexpr int kMaxLabels = 1024;        // labels whose terms the egrads write-out can fold in
 
 // Row of the 32x32 output block that register r of lane-half h holds.
 __device__ inline int mfma_row(int r, int h) { return 8 * (r >> 2) + 4 * h + (r & 3); }
@@ -679,7 +679,9 @@ static int egrads_stream_any(const TIO* E, const TIO* P, const float* mE, const 
   if (chunks > max_chunks) chunks = max_chunks;
   const int per = (ntiles + chunks - 1) / chunks;
   chunks = (ntiles + per - 1) / per;
-  if (d.U > kMaxLabels) return fail(kInvalid, "egrads: more than %d label positions", kMaxLabels);
+  if (sparse.labels && d.U - 1 > kMaxLabels)  // the per-wavefront match list of the folded terms
+    return fail(kInvalid, "egrads: blank/label terms can be folded in for at most %d labels",
+                kMaxLabels);
   // A launch contracts 16 * kEsMaxS label positions (what a wavefront keeps of Y in registers);
   // a longer label axis goes slice by slice, each later slice adding to what the earlier ones
   // left in egrads.  Only the last slice is given the factors, and scales the whole sum.

@@ -45,7 +45,9 @@ struct Dims {
 // 16-byte load per lane.  The pitch leaves room for the last partial group of four.
 __host__ __device__ inline int plane_pitch(int T, int U) { return ((T + U + 3) & ~3) + 8; }
 
-// Label positions one lane of the lattice wavefront owns: 1, 2, 4, 8 or 16 (U <= 1024).
+// Label positions one lane would own if one wavefront took the whole label axis: a power of two.
+// It sets the row count of the skewed planes (Ua = 64 x this); the walks themselves give a lane at
+// most 16 positions and take a longer axis in blocks of 1024.
 inline int cells_per_lane(int U) {
   int c = 1;
   while (c * 64 < U) c *= 2;
@@ -97,6 +99,8 @@ struct Planes {
   float* pl;    // P[u, label_u]         [B, Ua]
   float* gB;    // per-(b,u) blank-column sum of the sparse pgrads term   [B, Ua]
   float* gL;    // per-(b,u) label-column sum of the sparse pgrads term   [B, Ua]
+  float* hand[2];  // [B, Dp] each: what crosses from one block of 1024 label positions to the
+                   // next when a lattice walk takes the label axis block by block
 };
 
 // Trips a wavefront of the lattice kernels may spend waiting for its neighbour's progress
