@@ -169,7 +169,7 @@ int launch_viterbi(const Planes& p, const float* bestS, const float* argS,
                    int* labels_out, const Dims& d, hipStream_t s);
 size_t viterbi_bits_bytes(const Dims& d);
 
-// ---------------------------------------------------------------- launchers (rnnt_gemm.hip)
+// ---------------------------------------------------------------- launchers (rnnt_prep.hip)
 int wplane_up(int U);  // label-axis pitch of the W planes (multiple of 8)
 int wplane_tw(int T);  // frame-axis pitch of the W planes (multiple of 64)
 // Row maxima of a [rows, V] array.  With `lengths`, rows at or past lengths[item] + extra inside
