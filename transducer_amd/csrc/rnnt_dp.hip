@@ -251,7 +251,9 @@ __global__ __launch_bounds__(256) void gather_kernel(const TIO* __restrict__ E,
 // that cross a block boundary are the label-move scores of the block's last column, one per
 // step: a launch leaves them in `ghout` ([B][hand_stride], entry s = score entering step s;
 // null for the last block) and the next one reads them from `ghin` (null for the first block).
-template <int C, int W>
+// kMulti: this launch is one of several blocks (the hand-over code is compiled in only then: in
+// the single-block kernel even an unused hand-over load costs the walk its prefetch distance).
+template <int C, int W, bool kMulti>
 __global__ __launch_bounds__(64 * W) void alpha_kernel(Planes p, const int* __restrict__ inLen,
                                                        const int* __restrict__ labLen,
                                                        float* __restrict__ costs, Dims d,
@@ -275,9 +277,9 @@ __global__ __launch_bounds__(64 * W) void alpha_kernel(Planes p, const int* __re
   const int nsteps = Tb + Ub - 1;
   const int ngroups = (nsteps + 3) >> 2;
   const int u0 = u_base + (wave * 64 + lane) * C;
-  const float* gin = ghin ? ghin + (size_t)b * hand_stride : nullptr;
-  float* gout = ghout ? ghout + (size_t)b * hand_stride : nullptr;
-  if (gout && threadIdx.x == 0) gout[0] = kOutside;  // nothing enters step 0
+  const float* gin = (kMulti && ghin) ? ghin + (size_t)b * hand_stride : nullptr;
+  float* gout = (kMulti && ghout) ? ghout + (size_t)b * hand_stride : nullptr;
+  if (kMulti && gout && threadIdx.x == 0) gout[0] = kOutside;  // nothing enters step 0
   exp2_table_to_lds(etab);
   if (W > 1) {
     if (threadIdx.x < W) done[threadIdx.x] = 0;
@@ -323,8 +325,10 @@ __global__ __launch_bounds__(64 * W) void alpha_kernel(Planes p, const int* __re
     }
 #pragma unroll
     for (int k = 0; k < C + 3; ++k) r.eb[k] = ebl[4 * g + k - (C - 1)];
-    r.gh = make_float4(kOutside, kOutside, kOutside, kOutside);
-    if (gin) r.gh = *reinterpret_cast<const float4*>(gin + 4 * g);  // uniform
+    if constexpr (kMulti) {
+      r.gh = make_float4(kOutside, kOutside, kOutside, kOutside);
+      if (gin) r.gh = *reinterpret_cast<const float4*>(gin + 4 * g);  // uniform
+    }
     return r;
   };
 
@@ -339,7 +343,8 @@ __global__ __launch_bounds__(64 * W) void alpha_kernel(Planes p, const int* __re
   auto run_group = [&](int g, const Group& cur, auto whole) {
     constexpr bool kWhole = decltype(whole)::value;
     float4 aout[C];
-    float4 hin = cur.gh;  // wavefront 0: from the block below (or nothing)
+    float4 hin = {kOutside, kOutside, kOutside, kOutside};
+    if constexpr (kMulti) hin = cur.gh;  // wavefront 0: from the block below (or nothing)
     if (W > 1 && wave > 0) {
       wait_for(4 * g + 3);  // the scores entering steps 4g .. 4g+3 left steps 4g-1 .. 4g+2
       hin = *reinterpret_cast<const float4*>(hand_in + 4 * g);
@@ -349,10 +354,10 @@ __global__ __launch_bounds__(64 * W) void alpha_kernel(Planes p, const int* __re
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int s = 4 * g + j;
-      gsend[j] = kOutside;
+      if constexpr (kMulti) gsend[j] = kOutside;
       if (kWhole || s < nsteps) {  // uniform; a step past the last must not touch the scores
         float from_left = wave_shr1(emit[C - 1], kOutside);
-        if (W > 1 || gin) from_left = (lane == 0) ? f4get(hin, j) : from_left;
+        if (W > 1 || kMulti) from_left = (lane == 0) ? f4get(hin, j) : from_left;
 #pragma unroll
         for (int c = C - 1; c >= 0; --c) {
           const float left = (c == 0) ? from_left : emit[c - 1];
@@ -373,16 +378,18 @@ __global__ __launch_bounds__(64 * W) void alpha_kernel(Planes p, const int* __re
           emit[c] = inside ? se : kOutside;
           f4set(aout[c], j, a);
         }
-        gsend[j] = emit[C - 1];
+        if constexpr (kMulti) gsend[j] = emit[C - 1];
       }
       if (W > 1)
         hout[j] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(emit[C - 1]), 63));
     }
 #pragma unroll
     for (int c = 0; c < C; ++c) *reinterpret_cast<float4*>(ap[c] + 4 * g) = aout[c];
-    if (gout && wave == W - 1 && lane == 63) {  // entries 4g+1 .. 4g+4 for the block above
+    if constexpr (kMulti) {
+      if (gout && wave == W - 1 && lane == 63) {  // entries 4g+1 .. 4g+4 for the block above
 #pragma unroll
-      for (int j = 0; j < 4; ++j) gout[4 * g + 1 + j] = gsend[j];
+        for (int j = 0; j < 4; ++j) gout[4 * g + 1 + j] = gsend[j];
+      }
     }
     if (W > 1 && wave < W - 1 && lane == 0) {  // entries 4g+1 .. 4g+4, then the progress
 #pragma unroll
@@ -475,7 +482,7 @@ __global__ __launch_bounds__(256) void weights_kernel(Planes p, const int* __res
 // first column, one value per diagonal, left in `ghout` ([B][hand_stride], entry s = its dalpha
 // on diagonal s; null for the lowest block) and read by the block below from `ghin` (null for
 // the highest block).
-template <int C>
+template <int C, bool kMulti>
 __global__ __launch_bounds__(64) void beta_kernel(Planes p, const int* __restrict__ labels,
                                                   const int* __restrict__ inLen,
                                                   const int* __restrict__ labLen, Dims d,
@@ -491,8 +498,9 @@ __global__ __launch_bounds__(64) void beta_kernel(Planes p, const int* __restric
   const int last = nsteps - 1;  // diagonal of the last cell
   const int u0 = u_base + lane * C;
   // the block above exists for this utterance only if its first column does
-  const float* gin = (ghin && u_base + 64 * C < Ub) ? ghin + (size_t)b * hand_stride : nullptr;
-  float* gout = ghout ? ghout + (size_t)b * hand_stride : nullptr;
+  const float* gin =
+      (kMulti && ghin && u_base + 64 * C < Ub) ? ghin + (size_t)b * hand_stride : nullptr;
+  float* gout = (kMulti && ghout) ? ghout + (size_t)b * hand_stride : nullptr;
 
   float dcol[C], accB[C], accL[C];
   bool fold[C];  // label of this position equals blank: both sums share one accumulator
@@ -524,8 +532,10 @@ __global__ __launch_bounds__(64) void beta_kernel(Planes p, const int* __restric
       r.wb[c] = *reinterpret_cast<const float4*>(wbp[c] + 4 * gc);
       r.we[c] = *reinterpret_cast<const float4*>(wep[c] + 4 * gc);
     }
+    if constexpr (kMulti) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) r.gh[j] = gin ? gin[4 * gc + 1 + j] : 0.0f;  // uniform
+      for (int j = 0; j < 4; ++j) r.gh[j] = gin ? gin[4 * gc + 1 + j] : 0.0f;  // uniform
+    }
     return r;
   };
   // steps last-1 .. 0 are computed; the slot of step `last` receives the seed and the slots
@@ -539,12 +549,12 @@ __global__ __launch_bounds__(64) void beta_kernel(Planes p, const int* __restric
       if (s >= last) {  // uniform; only in the first group run
 #pragma unroll
         for (int c = 0; c < C; ++c) f4set(dout[c], j, s == last ? dcol[c] : 0.0f);
-        gsend[j] = s == last ? dcol[0] : 0.0f;
+        if constexpr (kMulti) gsend[j] = s == last ? dcol[0] : 0.0f;
       } else {
         float from_right = wave_shl1(dcol[0], 0.0f);
         // the column right of lane 63's last one belongs to the block above: its dalpha on the
         // diagonal just done, s + 1
-        if (gin) from_right = (lane == 63) ? w.gh[j] : from_right;
+        if constexpr (kMulti) from_right = (gin && lane == 63) ? w.gh[j] : from_right;
 #pragma unroll
         for (int c = 0; c < C; ++c) {
           const float right = (c == C - 1) ? from_right : dcol[c + 1];
@@ -557,14 +567,16 @@ __global__ __launch_bounds__(64) void beta_kernel(Planes p, const int* __restric
           dcol[c] = dn;
           f4set(dout[c], j, dn);
         }
-        gsend[j] = dcol[0];
+        if constexpr (kMulti) gsend[j] = dcol[0];
       }
     }
 #pragma unroll
     for (int c = 0; c < C; ++c) *reinterpret_cast<float4*>(dp[c] + 4 * g) = dout[c];
-    if (gout && lane == 0) {
+    if constexpr (kMulti) {
+      if (gout && lane == 0) {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) gout[4 * g + j] = gsend[j];
+        for (int j = 0; j < 4; ++j) gout[4 * g + j] = gsend[j];
+      }
     }
   };
 
@@ -1059,7 +1071,7 @@ __global__ __launch_bounds__(kMpThreads) void maxplus_kernel(const TIO* __restri
 // afterwards.
 // Dynamic LDS: one int per label position (steps at which labels were taken), the hand-over
 // array (W > 1), the columns (kLdsBits; else they live in global memory).
-template <int C, int W, bool kLdsBits>
+template <int C, int W, bool kLdsBits, bool kMulti>
 __global__ __launch_bounds__(64 * W) void viterbi_kernel(Planes p, const float* __restrict__ bestS,
                                                          const float* __restrict__ argS,
                                                          const int* __restrict__ inLen,
@@ -1090,9 +1102,9 @@ __global__ __launch_bounds__(64 * W) void viterbi_kernel(Planes p, const float* 
   unsigned* cols = kLdsBits
       ? reinterpret_cast<unsigned*>(hand + (W - 1) * hand_stride)     // [64 C W][nw]
       : gcols + (size_t)b * d.Ua * nw;                                // [Ua][nw]
-  const float* gin = ghin ? ghin + (size_t)b * hand_stride : nullptr;
-  float* gout = (ghout && walks) ? ghout + (size_t)b * hand_stride : nullptr;
-  if (gout && tidx == 0) gout[0] = kNegInf;  // nothing enters step 0
+  const float* gin = (kMulti && ghin) ? ghin + (size_t)b * hand_stride : nullptr;
+  float* gout = (kMulti && ghout && walks) ? ghout + (size_t)b * hand_stride : nullptr;
+  if (kMulti && gout && tidx == 0) gout[0] = kNegInf;  // nothing enters step 0
   if (W > 1) {
     if (tidx < W) done[tidx] = 0;
     if (tidx < W - 1) hand[tidx * hand_stride] = kNegInf;  // nothing enters step 0
@@ -1135,8 +1147,10 @@ __global__ __launch_bounds__(64 * W) void viterbi_kernel(Planes p, const float* 
     }
 #pragma unroll
     for (int k = 0; k < C + 3; ++k) r.eb[k] = ebl[4 * g + k - (C - 1)];
-    r.gh = make_float4(kNegInf, kNegInf, kNegInf, kNegInf);
-    if (gin) r.gh = *reinterpret_cast<const float4*>(gin + 4 * g);  // uniform
+    if constexpr (kMulti) {
+      r.gh = make_float4(kNegInf, kNegInf, kNegInf, kNegInf);
+      if (gin) r.gh = *reinterpret_cast<const float4*>(gin + 4 * g);  // uniform
+    }
     return r;
   };
   int avail = 0;  // steps the wavefront below is known to have published (see alpha_kernel)
@@ -1146,7 +1160,8 @@ __global__ __launch_bounds__(64 * W) void viterbi_kernel(Planes p, const float* 
   // A cell that has not started (t < 0) keeps -inf scores and never takes a label; cells past
   // the utterance run on whatever the planes hold and are never consulted by the backtrace.
   auto run_group = [&](int g, const Group& cur) {
-    float4 hin = cur.gh;  // wavefront 0: from the block below (or nothing)
+    float4 hin = {kNegInf, kNegInf, kNegInf, kNegInf};
+    if constexpr (kMulti) hin = cur.gh;  // wavefront 0: from the block below (or nothing)
     if (W > 1 && wave > 0) {
       wait_for(4 * g + 3);
       hin = *reinterpret_cast<const float4*>(hand_in + 4 * g);
@@ -1158,7 +1173,7 @@ __global__ __launch_bounds__(64 * W) void viterbi_kernel(Planes p, const float* 
       const int s = 4 * g + j;
       const unsigned sbit = 1u << (s & 31);  // uniform
       float from_left = wave_shr1(emit[C - 1], kNegInf);
-      if (W > 1 || gin) from_left = (lane == 0) ? f4get(hin, j) : from_left;
+      if (W > 1 || kMulti) from_left = (lane == 0) ? f4get(hin, j) : from_left;
 #pragma unroll
       for (int c = C - 1; c >= 0; --c) {
         const float left = (c == 0) ? from_left : emit[c - 1];
@@ -1176,13 +1191,15 @@ __global__ __launch_bounds__(64 * W) void viterbi_kernel(Planes p, const float* 
         stay[c] = started ? sb : kNegInf;
         emit[c] = started ? se : kNegInf;
       }
-      gsend[j] = emit[C - 1];
+      if constexpr (kMulti) gsend[j] = emit[C - 1];
       if (W > 1)
         hout[j] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(emit[C - 1]), 63));
     }
-    if (gout && wave == W - 1 && lane == 63) {  // entries 4g+1 .. 4g+4 for the block above
+    if constexpr (kMulti) {
+      if (gout && wave == W - 1 && lane == 63) {  // entries 4g+1 .. 4g+4 for the block above
 #pragma unroll
-      for (int j = 0; j < 4; ++j) gout[4 * g + 1 + j] = gsend[j];
+        for (int j = 0; j < 4; ++j) gout[4 * g + 1 + j] = gsend[j];
+      }
     }
     if ((g & 7) == 7 || g == ngroups - 1) {  // uniform: a word of 32 steps is complete
 #pragma unroll
@@ -1498,15 +1515,16 @@ int launch_alpha(const Planes& p, const int* inLen, const int* labLen, float* co
     const float* ghin = k == 0 ? nullptr : p.hand[(k - 1) & 1];
     float* ghout = k == nblocks - 1 ? nullptr : p.hand[k & 1];
     const int u_base = k * 64 * cpl;
-    switch (cpl / W * 100 + W) {
-#define CASE(C, W)                                                                          \
-  case C * 100 + W:                                                                         \
-    hipLaunchKernelGGL((alpha_kernel<C, W>), dim3(d.B), dim3(64 * W), lds, s, p, inLen,    \
-                       labLen, costs, d, stride, g_spin_limit, trouble, u_base, ghin,       \
-                       ghout);                                                              \
+    switch ((nblocks > 1 ? 10000 : 0) + cpl / W * 100 + W) {
+#define CASE(C, W, M)                                                                        \
+  case (M ? 10000 : 0) + C * 100 + W:                                                        \
+    hipLaunchKernelGGL((alpha_kernel<C, W, M>), dim3(d.B), dim3(64 * W), lds, s, p, inLen,  \
+                       labLen, costs, d, stride, g_spin_limit, trouble, u_base, ghin,        \
+                       ghout);                                                               \
     break;
-      CASE(1, 1) CASE(2, 1) CASE(4, 1) CASE(8, 1) CASE(16, 1)
-      CASE(1, 2) CASE(2, 2) CASE(4, 2) CASE(8, 2)
+      CASE(1, 1, false) CASE(2, 1, false) CASE(4, 1, false) CASE(8, 1, false) CASE(16, 1, false)
+      CASE(1, 2, false) CASE(2, 2, false) CASE(4, 2, false) CASE(8, 2, false)
+      CASE(16, 1, true) CASE(8, 2, true)  // several blocks: always 1024 positions each
 #undef CASE
       default:
         return fail(kInvalid, "alpha: no kernel for %d label positions per lane", cpl);
@@ -1533,13 +1551,14 @@ int launch_beta(const Planes& p, const int* labels, const int* inLen, const int*
     const float* ghin = k == nblocks - 1 ? nullptr : p.hand[(k + 1) & 1];
     float* ghout = k == 0 ? nullptr : p.hand[k & 1];
     const int u_base = k * 64 * cpl;
-    switch (cpl) {
-#define CASE(C)                                                                                \
-  case C:                                                                                      \
-    hipLaunchKernelGGL(beta_kernel<C>, dim3(d.B), dim3(64), 0, s, p, labels, inLen, labLen, d, \
-                       d.Dp, u_base, ghin, ghout);                                             \
+    switch ((nblocks > 1 ? 100 : 0) + cpl) {
+#define CASE(C, M)                                                                           \
+  case (M ? 100 : 0) + C:                                                                    \
+    hipLaunchKernelGGL((beta_kernel<C, M>), dim3(d.B), dim3(64), 0, s, p, labels, inLen,    \
+                       labLen, d, d.Dp, u_base, ghin, ghout);                                \
     break;
-      CASE(1) CASE(2) CASE(4) CASE(8) CASE(16)
+      CASE(1, false) CASE(2, false) CASE(4, false) CASE(8, false) CASE(16, false)
+      CASE(16, true)
 #undef CASE
       default:
         return fail(kInvalid, "dalpha: no kernel for %d label positions per lane", cpl);
@@ -1642,21 +1661,29 @@ int launch_viterbi(const Planes& p, const float* bestS, const float* argS,
     const float* ghin = k == 0 ? nullptr : p.hand[(k - 1) & 1];
     float* ghout = k == nblocks - 1 ? nullptr : p.hand[k & 1];
     const int u_base = k * 64 * cpl, traces = k == nblocks - 1 ? 1 : 0;
-    switch (cpl / W * 100 + W) {
+    switch ((nblocks > 1 ? 10000 : 0) + cpl / W * 100 + W) {
 #define CASE(C, W)                                                                             \
   case C * 100 + W:                                                                            \
     if (use_lds)                                                                               \
-      hipLaunchKernelGGL((viterbi_kernel<C, W, true>), dim3(d.B), dim3(64 * W), lds, s, p,    \
-                         bestS, argS, inLen, labLen, gcols, labels_out, d, stride, nw,         \
+      hipLaunchKernelGGL((viterbi_kernel<C, W, true, false>), dim3(d.B), dim3(64 * W), lds,   \
+                         s, p, bestS, argS, inLen, labLen, gcols, labels_out, d, stride, nw,   \
                          g_spin_limit, trouble, u_base, ghin, ghout, traces);                  \
     else                                                                                       \
-      hipLaunchKernelGGL((viterbi_kernel<C, W, false>), dim3(d.B), dim3(64 * W), lds, s, p,   \
-                         bestS, argS, inLen, labLen, gcols, labels_out, d, stride, nw,         \
+      hipLaunchKernelGGL((viterbi_kernel<C, W, false, false>), dim3(d.B), dim3(64 * W), lds,  \
+                         s, p, bestS, argS, inLen, labLen, gcols, labels_out, d, stride, nw,   \
                          g_spin_limit, trouble, u_base, ghin, ghout, traces);                  \
+    break;
+#define CASE_MULTI(C, W)                                                                       \
+  case 10000 + C * 100 + W:                                                                    \
+    hipLaunchKernelGGL((viterbi_kernel<C, W, false, true>), dim3(d.B), dim3(64 * W), lds, s,  \
+                       p, bestS, argS, inLen, labLen, gcols, labels_out, d, stride, nw,        \
+                       g_spin_limit, trouble, u_base, ghin, ghout, traces);                    \
     break;
       CASE(1, 1) CASE(2, 1) CASE(4, 1) CASE(8, 1) CASE(16, 1)
       CASE(1, 2) CASE(2, 2) CASE(4, 2) CASE(8, 2)
+      CASE_MULTI(16, 1) CASE_MULTI(8, 2)  // several blocks: always 1024 positions each
 #undef CASE
+#undef CASE_MULTI
       default:
         return fail(kInvalid, "viterbi: no kernel for %d label positions per lane", cpl);
     }
