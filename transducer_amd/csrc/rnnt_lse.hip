@@ -30,6 +30,8 @@
 //    as mE[t] for the gradient kernels, which only need it to be consistent with LN.
 //  * Workgroups are renumbered so that all frame tiles of one utterance run on the same XCD
 //    (workgroup ids are dealt round-robin to the 8 XCDs) and share its L2 copy of Y[b].
+#include <type_traits>
+
 #include "rnnt_internal.h"
 #include "rnnt_io.h"
 #include "rnnt_split.h"
@@ -53,6 +55,20 @@ __device__ inline float quad_xor1(float x) {
 }
 __device__ inline float quad_xor2(float x) {
   return __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(x), 0x4E, 0xf, 0xf, true));
+}
+
+// Maxima as single instructions.  fmaxf on values that come straight from memory makes the
+// compiler quiet possible signalling NaNs first (one extra instruction per operand); the
+// instructions themselves already return the other operand for a NaN.
+__device__ inline float vmax3(float a, float b, float c) {
+  float r;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
+__device__ inline float vmax2(float a, float b) {
+  float r;
+  asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
 }
 
 // a + b + c rounded once: the two partial sums are carried with their rounding errors (two
@@ -133,6 +149,7 @@ __global__ __launch_bounds__(64 * kWaves, kWaves / 2) void lse_stream_kernel(
   __shared__ int moved;           // some row's reference moved while the last slab was staged
   __shared__ int labs[1025];      // columns to pick: the utterance's labels, then the blank
   __shared__ short order[1025];   // their indices sorted by column
+  __shared__ int scol[1025];      // and the columns in that order
   // XCD-aware renumbering: physical id n runs on XCD n % 8
   const int n = blockIdx.x, per_xcd = gridDim.x >> 3;
   const int logical = (n & 7) * per_xcd + (n >> 3);
@@ -180,9 +197,17 @@ __global__ __launch_bounds__(64 * kWaves, kWaves / 2) void lse_stream_kernel(
       rank += (cw < c || (cw == c && w < u)) ? 1 : 0;
     }
     order[rank] = (short)u;
+    scol[rank] = c;
   }
-  int cursor = 0;      // uniform: entries before it have been copied
-  int next_slab = -1;  // slab of entry `cursor` (kept in a register: no LDS access on slabs without one)
+  int cursor = 0;   // uniform: entries before it have been copied
+  int ncol = -1;    // column and index of entry `cursor`, -1 past the last: read one entry ahead, so
+  int nu = 0;       // that a slab without a pick costs one scalar comparison
+  auto next_pick = [&]() {
+    const bool more = cursor < npick;
+    const int c = more ? scol[cursor] : -1, u = more ? order[cursor] : 0;
+    ncol = __builtin_amdgcn_readfirstlane(c);
+    nu = __builtin_amdgcn_readfirstlane(u);
+  };
 
   // staging: thread -> rows srow (+ 64 with four wavefronts) of the tile, v = slab start +
   // 8*c8 .. +7.  Rows past the utterance repeat its last frame, columns past V repeat earlier
@@ -231,34 +256,37 @@ __global__ __launch_bounds__(64 * kWaves, kWaves / 2) void lse_stream_kernel(
     }
   };
   auto picks = [&](const XRegs& r, int kslab) {
-    while (next_slab == kslab) {  // uniform
-      const int u = order[cursor], col = labs[u];
-      if (u == nlab) pick(r, col, ebv + (size_t)b * d.Tp + d.Eo);
-      else pick(r, col, elS + plane_row(d, b, u) + u);
+    while ((ncol >> 5) == kslab) {  // uniform
+      if (nu == nlab) pick(r, ncol, ebv + (size_t)b * d.Tp + d.Eo);
+      else pick(r, ncol, elS + plane_row(d, b, nu) + nu);
       ++cursor;
-      next_slab = cursor < npick ? (labs[order[cursor]] >> 5) : -1;
+      next_pick();
     }
   };
   auto stash = [&](int buf, const XRegs& r, bool first, int kslab) {
-    if (picking) picks(r, kslab);
+    // maximum of each row's 32 values of this slab (values past V repeat earlier ones); taken
+    // before the picks so that the loads are waited for here and not inside the pick loop
+    float lm[NR];
 #pragma unroll
     for (int i = 0; i < NR; ++i) {
-      // maximum of the row's 32 values of this slab (values past V repeat earlier ones)
       float e[8];
       expand(r.x[i], e);
-      float lm = fmaxf(fmaxf(fmaxf(e[0], e[1]), fmaxf(e[2], e[3])),
-                       fmaxf(fmaxf(e[4], e[5]), fmaxf(e[6], e[7])));
-      lm = fmaxf(lm, quad_xor1(lm));  // the four threads of a row are one quad of lanes
-      lm = fmaxf(lm, quad_xor2(lm));
-      lm = fmaxf(lm, kLowest);
-      if (first) {
-        mx[i] = lm;
-      } else if (lm > mx[i] + kSlack) {
-        // everything summed for this row so far shrinks by exp(old - new) (0 if old was -inf)
-        if (c8 == 0) scale[srow + (kThreads / 4) * i] = __expf(mx[i] - lm);
-        moved = 1;
-        mx[i] = lm;
-      }
+      float m = vmax3(e[0], e[1], e[2]);
+      m = vmax3(m, e[3], e[4]);
+      m = vmax2(m, vmax3(e[5], e[6], e[7]));
+      m = vmax2(m, quad_xor1(m));  // the four threads of a row are one quad of lanes
+      lm[i] = vmax3(m, quad_xor2(m), kLowest);
+    }
+    if (picking) picks(r, kslab);
+    float was[NR];
+    bool need[NR];
+#pragma unroll
+    for (int i = 0; i < NR; ++i) {
+      was[i] = mx[i];
+      need[i] = !first && lm[i] > mx[i] + kSlack;
+      mx[i] = (first || need[i]) ? lm[i] : mx[i];
+      float e[8];
+      expand(r.x[i], e);
       const float m = mx[i];
       const float x[8] = {__expf(e[0] - m), __expf(e[1] - m), __expf(e[2] - m), __expf(e[3] - m),
                           __expf(e[4] - m), __expf(e[5] - m), __expf(e[6] - m), __expf(e[7] - m)};
@@ -266,6 +294,19 @@ __global__ __launch_bounds__(64 * kWaves, kWaves / 2) void lse_stream_kernel(
       Xs[buf][0][slot[i]] = f.h;
       Xs[buf][1][slot[i]] = f.m;
       Xs[buf][2][slot[i]] = f.l;
+    }
+    // rare: a row's reference moved; everything summed for it so far shrinks by exp(old - new)
+    // (0 if old stood for -inf).  One uniform branch for the wavefront, after the staging.
+    bool any = false;
+#pragma unroll
+    for (int i = 0; i < NR; ++i) any = any || need[i];
+    if (__builtin_amdgcn_ballot_w64(any) != 0) {
+#pragma unroll
+      for (int i = 0; i < NR; ++i)
+        if (need[i]) {
+          if (c8 == 0) scale[srow + (kThreads / 4) * i] = __expf(was[i] - mx[i]);
+          moved = 1;
+        }
     }
   };
 
@@ -306,10 +347,14 @@ __global__ __launch_bounds__(64 * kWaves, kWaves / 2) void lse_stream_kernel(
   // again).  Left to itself the compiler reads every fragment just before its first use and the
   // matrix instructions wait for LDS one by one.
   struct YRegs { Frag3 s0, s1; };
-  auto slab = [&](int kt, YRegs& y) {
+  auto slab = [&](int kt, YRegs& y, auto act) {
+    constexpr bool kAct = decltype(act)::value;
     const int ktn = min(kt + 1, nk - 1);
+    // did a row's reference move while this slab was staged?  Read together with the fragments
+    // (LDS answers in order), so the flag costs no round trip of its own.
+    const int mv = moved;
     const XRegs xs = fetch(ktn * kSlice);
-    if (active) {
+    if (kAct) {
       uint4 ah[MB], am[MB], al[MB];
 #pragma unroll
       for (int m = 0; m < MB; ++m) al[m] = Xs[cur][2][aslot[0][m]];
@@ -318,6 +363,16 @@ __global__ __launch_bounds__(64 * kWaves, kWaves / 2) void lse_stream_kernel(
 #pragma unroll
       for (int m = 0; m < MB; ++m) am[m] = Xs[cur][1][aslot[0][m]];
       __builtin_amdgcn_sched_barrier(0);
+      if (mv) {  // uniform; rare: apply the factors before the re-referenced slab is multiplied
+#pragma unroll
+        for (int m = 0; m < MB; ++m)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const float f = scale[32 * (mb0 + m) + mfma_row(r, h)];
+            acc[m][r] *= f;
+            tot[m][r] *= f;
+          }
+      }
       // six piece products per block, smallest first; blocks interleaved so that consecutive
       // instructions do not wait on each other's accumulator
 #pragma unroll
@@ -359,28 +414,18 @@ __global__ __launch_bounds__(64 * kWaves, kWaves / 2) void lse_stream_kernel(
       y.s1 = fetch_y(2 * ktn + 1);
     }
     __builtin_amdgcn_sched_barrier(0);
-    stash(cur ^ 1, xs, false, min(kt + 1, nk - 1));
-    __syncthreads();
-    cur ^= 1;
-    if (moved) {  // uniform; rare: apply the factors before the re-referenced slab is multiplied
-      if (active) {
-#pragma unroll
-        for (int m = 0; m < MB; ++m)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const float f = scale[32 * (mb0 + m) + mfma_row(r, h)];
-            acc[m][r] *= f;
-            tot[m][r] *= f;
-          }
-      }
+    if (mv) {  // every wavefront has used the factors: back to 1 before the staging sets new ones
       __syncthreads();
       for (int r = tid; r < kRows; r += kThreads) scale[r] = 1.0f;
       if (tid == 0) moved = 0;
       __syncthreads();
     }
+    stash(cur ^ 1, xs, false, min(kt + 1, nk - 1));
+    __syncthreads();
+    cur ^= 1;
   };
   __syncthreads();  // order
-  if (npick > 0) next_slab = labs[order[0]] >> 5;
+  next_pick();
   stash(0, fetch(0), true, 0);
   YRegs y0;
   if (active) {
@@ -388,14 +433,21 @@ __global__ __launch_bounds__(64 * kWaves, kWaves / 2) void lse_stream_kernel(
     y0.s1 = fetch_y(1);
   }
   __syncthreads();
-  for (int kt = 0; kt < nk; ++kt) {
-    slab(kt, y0);
-    if (active && (kt + 1) % kFlush == 0) {
+  // Two copies of the loop, so that a wavefront with nothing to multiply is a path of its own:
+  // inside one loop the counted waits for the emission loads would have to hold on both paths,
+  // and the one without Y requests in flight makes the multiplying wavefronts wait for theirs.
+  if (active) {
+    for (int kt = 0; kt < nk; ++kt) {
+      slab(kt, y0, std::true_type{});
+      if ((kt + 1) % kFlush == 0) {
 #pragma unroll
-      for (int m = 0; m < MB; ++m)
+        for (int m = 0; m < MB; ++m)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) { tot[m][r] += acc[m][r]; acc[m][r] = 0.0f; }
+          for (int r = 0; r < 16; ++r) { tot[m][r] += acc[m][r]; acc[m][r] = 0.0f; }
+      }
     }
+  } else {
+    for (int kt = 0; kt < nk; ++kt) slab(kt, y0, std::false_type{});
   }
 
   // final references: to LDS for the write-out below, to mE for the kernels that come later
