@@ -112,9 +112,10 @@ int rnnt_hip_loss_backward(const float* emissions, const float* predictions, con
  * for a caller whose projection layers emit 16-bit logits, and they halve the traffic of the two
  * [B,T,V] arrays.  A score converts to fp32 exactly and all arithmetic is the fp32 path's; each
  * gradient element is the fp32 result (dense + blank/label terms, times deltas[b]) rounded once
- * to nearest-even (an fp16 gradient past 65504 becomes infinity).  The loss takes at most 112
- * label positions (U <= 112) and refuses more with an error: a longer label axis is contracted
- * in slices whose running sum would be rounded to 16 bits in between.  Any V; 16-byte loads are
+ * to nearest-even (an fp16 gradient past 65504 becomes infinity).  A label axis of more than
+ * 112 positions is contracted in slices that add up in fp32 (in the workspace, a window of frames
+ * at a time) before the one rounding; the loss takes at most 1025 label positions (U <= 1025) in
+ * these types and refuses more with an error.  Any V; 16-byte loads are
  * used when V is a multiple of 8 and the arrays are 16-byte aligned.  Workspace as for the fp32
  * calls.  The best path of
  * rnnt_hip_viterbi_decode_* is the one rnnt_hip_viterbi_decode finds on the same values. */

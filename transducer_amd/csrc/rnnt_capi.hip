@@ -278,8 +278,10 @@ int viterbi_impl(const TIO* E, const TIO* P, const float* LN, int* labels,
 
 // ---------------------------------------------------------------- 16-bit scores
 int check_lowp_shape(const Dims& d, bool loss, const char* who) {
-  if (loss && !egrads_one_pass(d))
-    return fail(kInvalid, "%s: 16-bit scores take at most 112 label positions (U=%d)", who, d.U);
+  // the blank / label terms are folded into the dense kernels' write-outs (one rounding per
+  // gradient entry), which keep a list of at most 1024 labels per wavefront
+  if (loss && d.U - 1 > 1024)
+    return fail(kInvalid, "%s: 16-bit scores take at most 1025 label positions (U=%d)", who, d.U);
   return kOk;
 }
 
@@ -354,8 +356,11 @@ int lowp_loss_backward(const TIO* E, const TIO* P, const int* labels, const int*
   sp.dS = w.planes.dS; sp.wE = w.planes.wE; sp.bsum = w.bsum; sp.labels = lab;
   SparsePTerms spp;
   spp.gB = w.planes.gB; spp.gL = w.planes.gL; spp.labels = lab;
+  // a label axis of more than one slice: the slices add up in fp32, in the part of the workspace
+  // that held the log-normaliser's Y pieces during the forward pass (free by now)
   RNNT_STAGE(kEgrads, launch_egrads_stream(E, P, w.mE, w.mP, w.Wn, deltas, egrads, inLen, labLen,
-                                           d, false, sp, s));
+                                           d, false, sp, s, static_cast<float*>(w.lse_scratch),
+                                           lse_scratch_bytes(d)));
   RNNT_STAGE(kPgrads, launch_pgrads_stream(E, P, w.mE, w.mP, w.Wt, deltas, pgrads, inLen, labLen,
                                            d, false, spp, w.psplit, s));
   return kOk;
@@ -757,8 +762,7 @@ int rnnt_hip_loss_backward(const float* E, const float* P, const int* labels, co
   return kOk;
 }
 
-// 16-bit scores (bf16, fp16): every launcher below exists for all three element types; only the
-// sliced label axis of egrads (more than 112 label positions) is fp32 only.  The three entry
+// 16-bit scores (bf16, fp16): every launcher below exists for all three element types.  The three entry
 // points per type are thin wrappers around the templates above.
 #define RNNT_LOWP_ENTRY_POINTS(SUFFIX, TIO)                                                       \
   int rnnt_hip_loss_forward_##SUFFIX(const uint16_t* E, const uint16_t* P, const int* labels,     \

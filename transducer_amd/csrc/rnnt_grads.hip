@@ -16,6 +16,7 @@
 //
 // v_mfma_f32_32x32x16_bf16 takes, per lane, eight consecutive k of its row (A) or column (B):
 // k = 8*(lane/32) + i.  A lane reads them with one 16-byte LDS load per piece.
+#include <algorithm>
 #include <type_traits>
 
 #include "rnnt_internal.h"
@@ -57,17 +58,24 @@ struct SlabRegs {
   float m;
 };
 
+// The frames one egrads launch covers and where they go: tiles [tile_begin, tile_end) of 32
+// frames; frame t of utterance b lands in row b * out_T + (t - t_base) of the output array.  The
+// whole frame axis into the caller's array: {0, tiles of T, T, 0}.
+struct EgradsWindow {
+  int tile_begin, tile_end, out_T, t_base;
+};
+
 // The walk of one workgroup over its frame tiles with NS steps of sixteen label positions
 // (a template parameter, so the matrix instructions of a tile form one straight-line block).
 // Label positions past the utterance contribute exact zeros: their Y rows are masked and the
 // W slab is zero there.
-template <int NS, bool kAccumulate, typename TIO>
+template <int NS, bool kAccumulate, typename TIO, typename TOUT>
 __device__ __forceinline__ void egrads_walk(
     const TIO* __restrict__ E, const TIO* __restrict__ P, const float* __restrict__ mE,
     const float* __restrict__ mP, const float* __restrict__ Wn, const float* __restrict__ deltas,
-    TIO* __restrict__ egrads, unsigned short (*As)[3][kEsPlane], float (*Ms)[32], const Dims& d,
+    TOUT* __restrict__ egrads, unsigned short (*As)[3][kEsPlane], float (*Ms)[32], const Dims& d,
     int Up, int Tw, int tiles_per_chunk, int u_lo, int b, int Tb, int Ub, const SparseTerms& sp,
-    const unsigned short* match, int nmatch, float (*Sp)[32]) {
+    const unsigned short* match, int nmatch, float (*Sp)[32], const EgradsWindow& win) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, h = lane >> 5;
   const int wave_col0 = blockIdx.x * 128 + wave * 32;  // this wavefront's 32 columns
   const int vcol = wave_col0 + l32;
@@ -77,13 +85,13 @@ __device__ __forceinline__ void egrads_walk(
   // lane that owns the blank column, if it is one of this wavefront's and terms are folded in
   const int blank_lane = (sp.labels && d.blank >= wave_col0 && d.blank < wave_col0 + 32)
                              ? d.blank - wave_col0 : -1;
-  const int ntiles = (d.T + 31) >> 5;
-  const int tile_lo = blockIdx.y * tiles_per_chunk;
-  const int tile_hi = min(tile_lo + tiles_per_chunk, ntiles);
+  const int tile_lo = win.tile_begin + blockIdx.y * tiles_per_chunk;
+  const int tile_hi = min(tile_lo + tiles_per_chunk, win.tile_end);
   const int tile_valid = min(tile_hi, (Tb + 31) >> 5);  // tiles that hold frames of the utterance
   const float delta = deltas ? deltas[b] : 1.0f;
   const TIO* Eb = E + (size_t)b * d.T * d.V;
-  TIO* out = egrads + (size_t)b * d.T * d.V;
+  // frame t of the utterance is row t - win.t_base of its block of win.out_T rows in `egrads`
+  TOUT* out = egrads + (size_t)b * win.out_T * d.V;
   const float* mEb = mE + (size_t)b * d.T;
 
   // Y fragments for this wavefront's columns (branch-free: clamped address, masked value):
@@ -191,7 +199,7 @@ __device__ __forceinline__ void egrads_walk(
     const SlabRegs nxt = fetch_slab(min(ti + 1, tile_valid - 1));
     const bool interior = cols_full && (t0 + 32 <= Tb);  // no row or column needs a guard
     const TIO* Etile = Eb + (size_t)t0 * d.V;
-    TIO* Otile = out + (size_t)t0 * d.V;
+    TOUT* Otile = out + (size_t)(t0 - win.t_base) * d.V;
     float evl[16];
     float (&ev)[16] = pick_set(ahead, evc, evl);
     if constexpr (decltype(ahead)::value) {
@@ -290,7 +298,7 @@ __device__ __forceinline__ void egrads_walk(
     if (interior) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        TIO* o = Otile + (lane_off + (unsigned)(8 * (r >> 2) + (r & 3)) * (unsigned)d.V);
+        TOUT* o = Otile + (lane_off + (unsigned)(8 * (r >> 2) + (r & 3)) * (unsigned)d.V);
         stf(o, delta * (kAccumulate ? ldf(o) + v[r] : v[r]));
       }
     } else {
@@ -298,7 +306,7 @@ __device__ __forceinline__ void egrads_walk(
       for (int r = 0; r < 16; ++r) {
         const int t = t0 + mfma_row(r, h);
         if (t < d.T && vok) {
-          TIO* o = out + (size_t)t * d.V + vcol;
+          TOUT* o = out + (size_t)(t - win.t_base) * d.V + vcol;
           stf(o, delta * (kAccumulate ? ldf(o) + v[r] : v[r]));
         }
       }
@@ -326,19 +334,19 @@ __device__ __forceinline__ void egrads_walk(
     for (int r = 0; r < 16; ++r) {
       const int t = ti * 32 + mfma_row(r, h);
       if (t < d.T && vok) {
-        TIO* o = out + (size_t)t * d.V + vcol;
+        TOUT* o = out + (size_t)(t - win.t_base) * d.V + vcol;
         stf(o, kAccumulate ? delta * ldf(o) : 0.0f);
       }
     }
   }
 }
 
-template <bool kAccumulate, typename TIO>
+template <bool kAccumulate, typename TIO, typename TOUT>
 __global__ __launch_bounds__(256, 2) void egrads_stream_kernel(
     const TIO* __restrict__ E, const TIO* __restrict__ P, const float* __restrict__ mE,
     const float* __restrict__ mP, const float* __restrict__ Wn, const float* __restrict__ deltas,
-    TIO* __restrict__ egrads, const int* __restrict__ inLen, const int* __restrict__ labLen,
-    Dims d, int Up, int Tw, int tiles_per_chunk, int u_lo, SparseTerms sp) {
+    TOUT* __restrict__ egrads, const int* __restrict__ inLen, const int* __restrict__ labLen,
+    Dims d, int Up, int Tw, int tiles_per_chunk, int u_lo, SparseTerms sp, EgradsWindow win) {
   __shared__ __attribute__((aligned(16))) unsigned short As[2][3][kEsPlane];
   __shared__ __attribute__((aligned(16))) float Ms[2][32];  // mE of the slab's frames
   __shared__ __attribute__((aligned(16))) float Strip[4][32];  // per wavefront: sparse terms
@@ -372,7 +380,7 @@ __global__ __launch_bounds__(256, 2) void egrads_stream_kernel(
 #define RNNT_EG_WALK(NS)                                                                      \
   egrads_walk<NS, kAccumulate>(E, P, mE, mP, Wn, deltas, egrads, As, Ms, d, Up, Tw,          \
                                tiles_per_chunk, u_lo, b, Tb, Ub, sp, Match[threadIdx.x >> 6], \
-                               nmatch, &Strip[threadIdx.x >> 6])
+                               nmatch, &Strip[threadIdx.x >> 6], win)
   if (nsteps <= 2) RNNT_EG_WALK(2);
   else if (nsteps <= 4) RNNT_EG_WALK(4);
   else if (nsteps == 5) RNNT_EG_WALK(5);
@@ -662,15 +670,15 @@ __global__ __launch_bounds__(256, 2) void pgrads_stream_kernel(
 
 bool egrads_one_pass(const Dims& d) { return wplane_up(d.U) <= 16 * kEsMaxS; }
 
-template <typename TIO>
-static int egrads_stream_any(const TIO* E, const TIO* P, const float* mE, const float* mP,
-                             const float* Wn, const float* deltas, TIO* egrads, const int* inLen,
-                             const int* labLen, const Dims& d, bool accumulate,
-                             const SparseTerms& sparse, hipStream_t s) {
-  if (sparse.labels && accumulate)
-    return fail(kInvalid, "sparse-term folding and accumulation are mutually exclusive");
+// One pass of the egrads kernels over the frames of `win` (all slices of the label axis), into
+// `out` (the caller's array, or a wide copy of a window of it).
+template <typename TIO, typename TOUT>
+static int egrads_window(const TIO* E, const TIO* P, const float* mE, const float* mP,
+                         const float* Wn, const float* deltas, TOUT* out, const int* inLen,
+                         const int* labLen, const Dims& d, bool accumulate,
+                         const SparseTerms& sparse, const EgradsWindow& win, hipStream_t s) {
   const int Up = wplane_up(d.U), Tw = wplane_tw(d.T);
-  const int vtiles = (d.V + 127) / 128, ntiles = (d.T + 31) / 32;
+  const int vtiles = (d.V + 127) / 128, ntiles = win.tile_end - win.tile_begin;
   // enough workgroups to fill 256 CUs two deep several times over, but long enough runs of
   // frames per workgroup to amortise loading the Y fragments
   int chunks = (2048 + vtiles * d.B - 1) / (vtiles * d.B);
@@ -679,25 +687,71 @@ static int egrads_stream_any(const TIO* E, const TIO* P, const float* mE, const 
   if (chunks > max_chunks) chunks = max_chunks;
   const int per = (ntiles + chunks - 1) / chunks;
   chunks = (ntiles + per - 1) / per;
-  if (sparse.labels && d.U - 1 > kMaxLabels)  // the per-wavefront match list of the folded terms
-    return fail(kInvalid, "egrads: blank/label terms can be folded in for at most %d labels",
-                kMaxLabels);
   // A launch contracts 16 * kEsMaxS label positions (what a wavefront keeps of Y in registers);
   // a longer label axis goes slice by slice, each later slice adding to what the earlier ones
-  // left in egrads.  Only the last slice is given the factors, and scales the whole sum.
+  // left in the output.  Only the last slice is given the factors, and scales the whole sum.
   const SparseTerms none;
   for (int u_lo = 0; u_lo < Up; u_lo += 16 * kEsMaxS) {
     const bool last = u_lo + 16 * kEsMaxS >= Up;
     const float* dl = last ? deltas : nullptr;
     if (accumulate || u_lo > 0)
-      hipLaunchKernelGGL((egrads_stream_kernel<true, TIO>), dim3(vtiles, chunks, d.B), dim3(256),
-                         0, s, E, P, mE, mP, Wn, dl, egrads, inLen, labLen, d, Up, Tw, per, u_lo,
-                         none);
+      hipLaunchKernelGGL((egrads_stream_kernel<true, TIO, TOUT>), dim3(vtiles, chunks, d.B),
+                         dim3(256), 0, s, E, P, mE, mP, Wn, dl, out, inLen, labLen, d, Up, Tw,
+                         per, u_lo, none, win);
     else
-      hipLaunchKernelGGL((egrads_stream_kernel<false, TIO>), dim3(vtiles, chunks, d.B), dim3(256),
-                         0, s, E, P, mE, mP, Wn, dl, egrads, inLen, labLen, d, Up, Tw, per, u_lo,
-                         sparse);
+      hipLaunchKernelGGL((egrads_stream_kernel<false, TIO, TOUT>), dim3(vtiles, chunks, d.B),
+                         dim3(256), 0, s, E, P, mE, mP, Wn, dl, out, inLen, labLen, d, Up, Tw,
+                         per, u_lo, sparse, win);
     RNNT_LAUNCH_CHECK("egrads_stream_kernel");
+  }
+  return kOk;
+}
+
+// rows [t_lo, t_lo + n) of every utterance of dst[B][T][V] = the rows [0, n) of src[B][Tc][V],
+// each value rounded once
+template <typename TIO>
+__global__ void narrow_rows_kernel(const float* __restrict__ src, TIO* __restrict__ dst, int T,
+                                   int Tc, int V, int t_lo, int per_row) {
+  const int b = blockIdx.y, t = blockIdx.x / per_row;
+  const int v = (blockIdx.x - t * per_row) * 256 + threadIdx.x;
+  if (v < V) stf(dst + ((size_t)b * T + t_lo + t) * V + v, src[((size_t)b * Tc + t) * V + v]);
+}
+
+// `wide`, `wide_bytes`: fp32 scratch for 16-bit gradients whose label axis needs more than one
+// slice.  Slices add up in the output array, which for a 16-bit array would round every partial
+// sum; so the frames are taken a window at a time, the slices add up in an fp32 copy of the
+// window, and the finished window is rounded once on its way into the caller's array.
+template <typename TIO>
+static int egrads_stream_any(const TIO* E, const TIO* P, const float* mE, const float* mP,
+                             const float* Wn, const float* deltas, TIO* egrads, const int* inLen,
+                             const int* labLen, const Dims& d, bool accumulate,
+                             const SparseTerms& sparse, hipStream_t s, float* wide = nullptr,
+                             size_t wide_bytes = 0) {
+  if (sparse.labels && accumulate)
+    return fail(kInvalid, "sparse-term folding and accumulation are mutually exclusive");
+  if (sparse.labels && d.U - 1 > kMaxLabels)  // the per-wavefront match list of the folded terms
+    return fail(kInvalid, "egrads: blank/label terms can be folded in for at most %d labels",
+                kMaxLabels);
+  const int ntiles = (d.T + 31) / 32;
+  if (sizeof(TIO) == sizeof(float) || egrads_one_pass(d)) {
+    const EgradsWindow all{0, ntiles, d.T, 0};
+    return egrads_window(E, P, mE, mP, Wn, deltas, egrads, inLen, labLen, d, accumulate, sparse,
+                         all, s);
+  }
+  if (accumulate) return fail(kInvalid, "egrads: 16-bit gradients cannot be added to");
+  const size_t row_bytes = sizeof(float) * (size_t)d.B * d.V;
+  const int Tc = (int)std::min<size_t>(wide ? wide_bytes / row_bytes / 32 * 32 : 0, (size_t)ntiles * 32);
+  if (Tc < 32)
+    return fail(kWorkspace, "egrads: no room for a window of 32 frames of fp32 gradients");
+  for (int t_lo = 0; t_lo < d.T; t_lo += Tc) {
+    const EgradsWindow win{t_lo / 32, std::min(ntiles, (t_lo + Tc) / 32), Tc, t_lo};
+    RNNT_TRY(egrads_window(E, P, mE, mP, Wn, deltas, wide, inLen, labLen, d, false, sparse, win,
+                           s));
+    const int n = std::min(Tc, d.T - t_lo);
+    const unsigned per_row = (unsigned)((d.V + 255) / 256);
+    hipLaunchKernelGGL((narrow_rows_kernel<TIO>), dim3(per_row * (unsigned)n, d.B), dim3(256), 0,
+                       s, wide, egrads, d.T, Tc, d.V, t_lo, (int)per_row);
+    RNNT_LAUNCH_CHECK("narrow_rows_kernel");
   }
   return kOk;
 }
@@ -711,16 +765,18 @@ int launch_egrads_stream(const float* E, const float* P, const float* mE, const 
 int launch_egrads_stream(const bf16_t* E, const bf16_t* P, const float* mE, const float* mP,
                          const float* Wn, const float* deltas, bf16_t* egrads, const int* inLen,
                          const int* labLen, const Dims& d, bool accumulate,
-                         const SparseTerms& sparse, hipStream_t s) {
+                         const SparseTerms& sparse, hipStream_t s, float* wide,
+                         size_t wide_bytes) {
   return egrads_stream_any(E, P, mE, mP, Wn, deltas, egrads, inLen, labLen, d, accumulate, sparse,
-                           s);
+                           s, wide, wide_bytes);
 }
 int launch_egrads_stream(const f16_t* E, const f16_t* P, const float* mE, const float* mP,
                          const float* Wn, const float* deltas, f16_t* egrads, const int* inLen,
                          const int* labLen, const Dims& d, bool accumulate,
-                         const SparseTerms& sparse, hipStream_t s) {
+                         const SparseTerms& sparse, hipStream_t s, float* wide,
+                         size_t wide_bytes) {
   return egrads_stream_any(E, P, mE, mP, Wn, deltas, egrads, inLen, labLen, d, accumulate, sparse,
-                           s);
+                           s, wide, wide_bytes);
 }
 
 // Whether the workgroups of a tile share its frames.  A chunk is always kPsFlush slabs, the

@@ -253,8 +253,10 @@ int launch_pgrads(const float* E, const float* P, const float* mE, const float* 
 
 
 // ---------------------------------------------------------------- launchers (rnnt_grads.hip)
-// Whether one launch covers the label axis (16-bit gradients are only formed that way: a
-// second slice would round the running sum to 16 bits in between).
+// Whether one launch covers the label axis.  A longer axis goes slice by slice, the slices adding
+// up in the output array; 16-bit gradients then go through `wide` (fp32 scratch of wide_bytes,
+// at least 32 frames of B * V values), a window of frames at a time, so that each value is still
+// rounded once.
 bool egrads_one_pass(const Dims& d);
 int launch_egrads_stream(const float* E, const float* P, const float* mE, const float* mP,
                          const float* Wn, const float* deltas, float* egrads, const int* inLen,
@@ -263,11 +265,13 @@ int launch_egrads_stream(const float* E, const float* P, const float* mE, const 
 int launch_egrads_stream(const bf16_t* E, const bf16_t* P, const float* mE, const float* mP,
                          const float* Wn, const float* deltas, bf16_t* egrads, const int* inLen,
                          const int* labLen, const Dims& d, bool accumulate,
-                         const SparseTerms& sparse, hipStream_t s);
+                         const SparseTerms& sparse, hipStream_t s, float* wide = nullptr,
+                         size_t wide_bytes = 0);
 int launch_egrads_stream(const f16_t* E, const f16_t* P, const float* mE, const float* mP,
                          const float* Wn, const float* deltas, f16_t* egrads, const int* inLen,
                          const int* labLen, const Dims& d, bool accumulate,
-                         const SparseTerms& sparse, hipStream_t s);
+                         const SparseTerms& sparse, hipStream_t s, float* wide = nullptr,
+                         size_t wide_bytes = 0);
 int launch_pgrads_stream(const float* E, const float* P, const float* mE, const float* mP,
                          const float* Wt, const float* deltas, float* pgrads, const int* inLen,
                          const int* labLen, const Dims& d, bool accumulate,

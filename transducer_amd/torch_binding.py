@@ -120,7 +120,7 @@ class TransducerLoss(torch.nn.Module):
         predictions (both of the same type) are accepted as well; costs are float32 and the
         gradients come back in the scores' type.  The reference raises ``TypeError`` for
         anything but float32, and so does this module unless a flag is set.  The loss takes at
-        most 112 label positions in these types (any vocabulary size).
+        most 1025 label positions in these types (any vocabulary size).
     """
 
     def __init__(self, blank=0, allow_bf16=False, allow_fp16=False):
