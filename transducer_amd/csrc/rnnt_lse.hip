@@ -75,12 +75,26 @@ __device__ inline float vmax2(float a, float b) {
 // error-free additions; this file is compiled without contraction or reassociation), so the
 // log-normaliser's epilogue log(sum) + mE + mP adds half an ulp to the error of the logarithm
 // instead of three half ulps.
-__device__ inline float add3(float a, float b, float c) {
+// `tiny`: a fourth term far below the others' last bits, added to the carried errors.
+__device__ inline float add3(float a, float b, float c, float tiny = 0.0f) {
   const float s = b + c, bv = s - b;
   const float s_err = (b - (s - bv)) + (c - bv);
   const float r = a + s, av = r - a;
   const float r_err = (a - (r - av)) + (s - av);
-  return r + (r_err + s_err);
+  return r + ((r_err + s_err) + tiny);
+}
+
+// X = exp(e - m) for the 32 values of a slab that share the row's reference m.  With m log2(e)
+// formed once per row and slab, an exponential is one fused multiply-add and one v_exp_f32
+// instead of a subtraction, a multiplication and the v_exp_f32.  The rounding of that product
+// moves the reference actually used to m' = fl(m log2 e) / log2 e: the same for every value of
+// the row, so it does not touch the sum's accuracy, and the write-out adds m' - m back
+// (reference_shift) so that the log-normaliser does not carry it either.
+constexpr float kLog2e = 1.44269504088896340736f;
+__device__ inline float reference_shift(float m) {
+  const float ml = m * kLog2e;
+  const float lost = __builtin_fmaf(m, kLog2e, -ml);  // m log2 e - fl(m log2 e), exactly
+  return -lost * (1.0f / kLog2e);
 }
 
 // 16-byte slot of (row, c8 = which eight of the slab's 32 v) inside a piece plane
@@ -287,9 +301,11 @@ __global__ __launch_bounds__(64 * kWaves, kWaves / 2) void lse_stream_kernel(
       mx[i] = (first || need[i]) ? lm[i] : mx[i];
       float e[8];
       expand(r.x[i], e);
-      const float m = mx[i];
-      const float x[8] = {__expf(e[0] - m), __expf(e[1] - m), __expf(e[2] - m), __expf(e[3] - m),
-                          __expf(e[4] - m), __expf(e[5] - m), __expf(e[6] - m), __expf(e[7] - m)};
+      const float ml = mx[i] * kLog2e;
+      float x[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        x[j] = __builtin_amdgcn_exp2f(__builtin_fmaf(e[j], kLog2e, -ml));
       const Frag3 f = split8(x);
       Xs[buf][0][slot[i]] = f.h;
       Xs[buf][1][slot[i]] = f.m;
@@ -478,7 +494,8 @@ __global__ __launch_bounds__(64 * kWaves, kWaves / 2) void lse_stream_kernel(
       const int row = 32 * (mb0 + m) + mfma_row(r, h), t = t0 + row;
       if (t < d.T && u < d.U) {
         float v = 0.0f;
-        if (t < Tb && u < Ub) v = add3(logf(tot[m][r] + acc[m][r]), mfin[row], mu);
+        if (t < Tb && u < Ub)
+          v = add3(logf(tot[m][r] + acc[m][r]), mfin[row], mu, reference_shift(mfin[row]));
         if (lnS == nullptr) LNb[(size_t)t * d.U + u] = v;
         else if (t < Tb && u < Ub) lnS[plane_row(d, b, u) + t + u] = v;
       }
