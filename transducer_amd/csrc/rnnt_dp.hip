@@ -540,7 +540,11 @@ __global__ __launch_bounds__(64) void beta_kernel(Planes p, const int* __restric
   };
   // steps last-1 .. 0 are computed; the slot of step `last` receives the seed and the slots
   // after it (same group of four) zeros
-  auto run_group = [&](int g, const Group& w) {
+  // with_fold: some position of this wavefront has the blank as its label, whose two sums then
+  // share one accumulator.  Real transcripts have none, and the walk without the two selects per
+  // cell is a fifth shorter (x - 0 is x, so the sums come out the same bits either way).
+  auto run_group = [&](int g, const Group& w, auto with_fold) {
+    constexpr bool kFold = decltype(with_fold)::value;
     float4 dout[C];
     float gsend[4];  // dalpha of this lane's first column after each step
 #pragma unroll
@@ -561,9 +565,14 @@ __global__ __launch_bounds__(64) void beta_kernel(Planes p, const int* __restric
           const float ne = dcol[c] * f4get(w.wb[c], j);
           const float em = right * f4get(w.we[c], j);
           const float dn = ne + em;
-          const float em_b = fold[c] ? em : 0.0f, em_l = fold[c] ? 0.0f : em;
-          accB[c] = (accB[c] - ne) - em_b;
-          accL[c] = accL[c] - em_l;
+          if constexpr (kFold) {
+            const float em_b = fold[c] ? em : 0.0f, em_l = fold[c] ? 0.0f : em;
+            accB[c] = (accB[c] - ne) - em_b;
+            accL[c] = accL[c] - em_l;
+          } else {
+            accB[c] = accB[c] - ne;
+            accL[c] = accL[c] - em;
+          }
           dcol[c] = dn;
           f4set(dout[c], j, dn);
         }
@@ -580,18 +589,25 @@ __global__ __launch_bounds__(64) void beta_kernel(Planes p, const int* __restric
     }
   };
 
-  int g = last >> 2;  // the group that holds the seed
-  Group x = load_group(g), y = load_group(g - 1), z = load_group(g - 2);
-  for (; g >= 2; g -= 3) {
-    run_group(g, x);
-    x = load_group(g - 3);
-    run_group(g - 1, y);
-    y = load_group(g - 4);
-    run_group(g - 2, z);
-    z = load_group(g - 5);
-  }
-  if (g >= 0) run_group(g, x);
-  if (g >= 1) run_group(g - 1, y);
+  auto walk = [&](auto with_fold) __attribute__((always_inline)) {
+    int g = last >> 2;  // the group that holds the seed
+    Group x = load_group(g), y = load_group(g - 1), z = load_group(g - 2);
+    for (; g >= 2; g -= 3) {
+      run_group(g, x, with_fold);
+      x = load_group(g - 3);
+      run_group(g - 1, y, with_fold);
+      y = load_group(g - 4);
+      run_group(g - 2, z, with_fold);
+      z = load_group(g - 5);
+    }
+    if (g >= 0) run_group(g, x, with_fold);
+    if (g >= 1) run_group(g - 1, y, with_fold);
+  };
+  bool any_fold = false;
+#pragma unroll
+  for (int c = 0; c < C; ++c) any_fold = any_fold || fold[c];
+  if (__ballot(any_fold) != 0) walk(std::true_type{});
+  else walk(std::false_type{});
 
 #pragma unroll
   for (int c = 0; c < C; ++c) {
