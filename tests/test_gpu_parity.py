@@ -368,9 +368,13 @@ def test_log_norms_wide_dynamic_range():
 # ------------------------------------------------------------------ dense gradient kernels
 # (U counts the rows of predictions; 113, 224, 225 sit on the edges of the 112-position slices
 # the egrads kernel contracts per launch)
+# (V = 16 mod 32, where every other row starts half a cache line in: one frame, an odd and an even
+# number of frames, rows past a tile)
 @pytest.mark.parametrize("B,T,U,V", [(2, 50, 11, 32), (2, 130, 101, 333), (1, 300, 140, 64),
                                      (2, 40, 113, 128), (2, 36, 224, 516), (3, 36, 225, 64),
-                                     (2, 20, 470, 40)])
+                                     (2, 20, 470, 40), (3, 1, 5, 16), (2, 2, 3, 48),
+                                     (2, 65, 20, 528), (1, 127, 101, 1040), (2, 64, 9, 16),
+                                     (2, 130, 120, 80)])
 def test_dense_grads_against_oracle(B, T, U, V):
     cfg = small_config(B, T, U - 1, V, ragged=True)
     E, P, labels, il, ll = unpack(make_inputs(cfg, seed=T))
@@ -407,7 +411,7 @@ def test_whole_loss_cfg1(cfg, seed):
 
 @pytest.mark.parametrize("T,U,V", [(60, 150, 36), (60, 150, 37), (40, 260, 16), (33, 113, 520),
                                    (40, 111, 520), (40, 112, 520), (36, 223, 516), (36, 224, 1028),
-                                   (20, 500, 64)])
+                                   (20, 500, 64), (33, 113, 528), (70, 100, 528)])
 def test_whole_loss_with_a_label_axis_longer_than_one_slice(T, U, V):
     """egrads contracts 112 label positions per launch; a longer axis goes slice by slice, the
     later slices adding to what is in egrads and only the last one applying the upstream factors
