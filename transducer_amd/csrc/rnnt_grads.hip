@@ -110,16 +110,27 @@ __device__ __forceinline__ void egrads_walk(
   if (tile_lo < tile_valid) {
     const TIO* Pb = P + (size_t)b * d.U * d.V;
     const float* mPb = mP + (size_t)b * d.U;
+    // (all scores and row maxima are requested before the first is used: step by step, each
+    // step's loads are waited for before the next step's are issued)
+    float praw[NS][8], mraw[NS][8];
+#pragma unroll
+    for (int s = 0; s < NS; ++s)
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int u = u_lo + 16 * s + 8 * h + i;
+        const int uc = u < Ub ? u : 0;
+        praw[s][i] = ldf(Pb + (size_t)uc * d.V + vc);
+        mraw[s][i] = mPb[uc];
+      }
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int s = 0; s < NS; ++s) {
       float y[8];
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
         const int u = u_lo + 16 * s + 8 * h + i;
-        const bool uok = u < Ub;
-        const int uc = uok ? u : 0;
-        const float e = __expf(ldf(Pb + (size_t)uc * d.V + vc) - mPb[uc]);
-        y[i] = (uok && vok) ? e : 0.0f;
+        const float e = __expf(praw[s][i] - mraw[s][i]);
+        y[i] = (u < Ub && vok) ? e : 0.0f;
       }
       Yf[s] = split8(y);
     }
