@@ -1044,28 +1044,52 @@ __global__ __launch_bounds__(kMpThreads) void maxplus_kernel(const TIO* __restri
     cur ^= 1;
   }
   if (!active) return;
-  // recover the lowest index inside the winning chunk
+  // Recover the lowest index inside the winning chunk: the chunk's 32 columns of the cell's two
+  // rows come in as sixteen 16-byte loads, all requested before the first is looked at, and the
+  // sums are compared in registers.  (Looked up column by column, the way the reference scans,
+  // this was two dependent loads and a wait per column and cell: five hundred memory round
+  // trips in a row at the end of every wavefront.)  Every lane goes through the loads with
+  // clamped rows; only cells of the utterance are written.
 #pragma unroll
   for (int i = 0; i < 2; ++i)
 #pragma unroll
     for (int r = 0; r < kMpRows; ++r) {
       const int t = t0 + lane + 64 * i, u = ur0 + r;
-      if (t >= Tb || u >= Ub) continue;
+      const bool cell = t < Tb && u < Ub;
+      const int v0 = max(chunk[i][r], 0) * kMpK;
+      const TIO* e = Eb + (size_t)min(t, Tb - 1) * d.V;
+      const TIO* q = Pb + (size_t)min(u, Ub - 1) * d.V;
+      float4 ev[kMpK / 4], pv[kMpK / 4];
+#pragma unroll
+      for (int g = 0; g < kMpK / 4; ++g) {
+        const int v = v0 + 4 * g;
+        // (kVec: a group of four is inside the row or past it as a whole, and one past it is
+        // never looked at, so the clamped start only keeps the load inside the array)
+        ev[g] = kVec ? load4(e + min(v, d.V - 4)) : load4_any(e, min(v, d.V - 1), d.V);
+        pv[g] = kVec ? load4(q + min(v, d.V - 4)) : load4_any(q, min(v, d.V - 1), d.V);
+      }
       int at = 0;  // :160 the scan starts from index 0 and keeps it if nothing beats -inf
       if (chunk[i][r] >= 0) {
-        const int v0 = chunk[i][r] * kMpK;
-        const TIO* e = Eb + (size_t)t * d.V;
-        const TIO* q = Pb + (size_t)u * d.V;
-        for (int v = v0; v < v0 + kMpK && v < d.V; ++v) {
-          if (v == d.blank) continue;
-          if (ldf(e + v) + ldf(q + v) == top[i][r]) { at = v; break; }
+        const float want = top[i][r];
+        // from the last column down, so that the lowest match is what remains
+#pragma unroll
+        for (int g = kMpK / 4 - 1; g >= 0; --g) {
+          const float sum[4] = {ev[g].x + pv[g].x, ev[g].y + pv[g].y, ev[g].z + pv[g].z,
+                                ev[g].w + pv[g].w};
+#pragma unroll
+          for (int j = 3; j >= 0; --j) {
+            const int v = v0 + 4 * g + j;
+            if (v < d.V && v != d.blank && sum[j] == want) at = v;
+          }
         }
       }
-      // straight into the skewed planes the lattice walk reads (consecutive frames of one label
-      // position are neighbours there)
-      const size_t o = plane_row(d, b, u) + t + u;
-      best[o] = top[i][r];
-      arg[o] = at;
+      if (cell) {
+        // straight into the skewed planes the lattice walk reads (consecutive frames of one
+        // label position are neighbours there)
+        const size_t o = plane_row(d, b, u) + t + u;
+        best[o] = top[i][r];
+        arg[o] = at;
+      }
     }
 }
 
