@@ -195,6 +195,21 @@ int rnnt_hip_check_kernels(rnnt_stream_t stream);
  * tests of the give-up path: with 0 the upper wavefront gives up at its first unmet wait. */
 int rnnt_hip_set_spin_limit(int trips);
 
+/* How the best-path calls find best[t,u] = max over v != blank of E[t,v] + P[u,v] and its
+ * lowest index (transducer/transducer_cpu.cpp:158-171; the reference's device kernel scans every
+ * column per cell, transducer/transducer_cuda.cu:178-207).  0 (default): from short candidate
+ * lists with an exactness test per cell where the vocabulary is long enough to pay for them
+ * (cells that fail the test are evaluated over every column), over every column otherwise;
+ * 1: over every column always; 2: from lists wherever the shape allows.  The labels returned are
+ * the same in every mode; the setting is process-wide.  No counterpart in the reference. */
+int rnnt_hip_set_maxplus_mode(int mode);
+/* The table itself, for tests of the two ways of building it: best[b][t][u] and arg[b][t][u]
+ * ([B][T][U]; -inf and -1 outside an utterance's T_b x U_b cells).  fp32 scores; scratch from
+ * the stream-ordered allocator. */
+int rnnt_hip_maxplus_table(const float* emissions, const float* predictions,
+                           const int* input_lengths, const int* label_lengths, float* best,
+                           int* arg, int B, int T, int U, int V, int blank, rnnt_stream_t stream);
+
 /* The lattice kernels' expf and log1pf, which restate the C library's (glibc 2.35, the one the
  * reference's std::exp / std::log1p resolve to, transducer/transducer_cpu.cpp:16-24,124-135) so
  * that alphas and transition weights carry the reference's bits: expf_out[i] = expf(x[i]),

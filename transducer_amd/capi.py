@@ -33,6 +33,8 @@ SIGNATURES = {
     "rnnt_hip_viterbi_decode_f16": (_I, [_F] * 5 + [_I] * 5 + [_F]),
     "rnnt_hip_check_kernels": (_I, [_F]),
     "rnnt_hip_set_spin_limit": (_I, [_I]),
+    "rnnt_hip_set_maxplus_mode": (_I, [_I]),
+    "rnnt_hip_maxplus_table": (_I, [_F] * 6 + [_I] * 5 + [_F]),
     "rnnt_hip_chain_floor": (_I, [_I, _I, _F]),
     "rnnt_hip_lse_bound_check": (_I, [ctypes.c_uint, ctypes.c_uint, _F, _F]),
     "rnnt_hip_libm_probe": (_I, [_F, _F, _F, ctypes.c_long, _F]),

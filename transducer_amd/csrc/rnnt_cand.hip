@@ -1,0 +1,716 @@
+// The max-plus table from short candidate lists.
+//
+// best[t,u] = max over v != blank of E[t,v] + P[u,v], arg = lowest such v
+// (transducer/transducer_cpu.cpp:158-171) costs one add and one compare per (t, u, v) when every
+// column is looked at.  Nearly all of them cannot win: with a threshold tE[t] for the frame's
+// row of E and tP[u] for the label position's row of P,
+//   A_t = { v : E[t,v] > tE[t] },   C_u = { v : P[u,v] > tP[u] },
+// every column outside both sets has E[t,v] + P[u,v] <= tE[t] + tP[u] (rounding is monotone, so
+// this holds for the rounded sums too).  If the best sum over A_t and C_u is strictly above
+// that bound, it is the row's maximum and every column that reaches it is in one of the two
+// sets: maximum and lowest index are exact.  A cell that fails the test is flagged and
+// evaluated over all columns afterwards.  The thresholds only decide how long the lists are
+// and how many cells fail, never what is returned.
+//
+//   * cand_lists_p_kernel: threshold and sorted list for every row of P, plus P transposed
+//     (cand_transpose_p_kernel) so that one candidate column's 64 label positions are one
+//     256-byte read;
+//   * cand_rows_kernel: per frame, the row of E goes into LDS, gets its threshold and list, and
+//     the two wavefronts of the workgroup (64 label positions each) evaluate A_t against the
+//     transposed P and C_u against the LDS row;
+//   * tiles of 128 frames x 64 label positions with more than kCdTileLimit flagged cells are
+//     redone by the all-columns kernel (maxplus_kernel), the others' flagged cells one by one
+//     (cand_cells_kernel): the cost of a failed test is bounded either way.
+//
+// A threshold is the value with about kCdTarget of the 256 sub-maxima of a row above it (each
+// thread keeps the maxima of two interleaved subsets of its elements): for values drawn
+// independently that puts about 1.4 % of a 10000-column row on the list, whatever their scale,
+// and a constant or heavily tied row gets an empty list instead of a full one.
+#include <hip/hip_runtime.h>
+
+#include <type_traits>
+
+#include "rnnt_internal.h"
+
+namespace rnnt {
+namespace {
+
+constexpr float kNegInf = -__builtin_huge_valf();
+constexpr int kCdThreads = 256;  // four wavefronts
+constexpr int kCdWaves = kCdThreads / 64;
+constexpr int kCdCap = 192;      // entries per wavefront's quarter of a row's list
+constexpr int kCdSeg = kCdCap + 8;  // a quarter's slots: one batch of padding can follow a full one
+constexpr int kCdDepth = 384;    // entries of a stored list of P
+constexpr int kCdStored = kCdDepth + 8;  // with one batch of padding behind a full list
+constexpr int kCdRank = 30;      // sub-maxima of a wavefront (of 64) above its threshold
+constexpr int kCdBisect = 16;    // halvings of the key interval
+constexpr int kCdFrames = 16;    // frames per workgroup of cand_rows_kernel
+constexpr int kCdPre = 12;       // 16-byte pieces of a row a thread has in flight while staging
+constexpr int kCdBatch = 8;      // candidates per batch (two batches in flight)
+constexpr int kCdTileT = 128, kCdTileU = 64;  // the all-columns kernel's tile
+constexpr int kCdTileLimit = 64;  // flagged cells a tile may hold and still be redone cell by cell
+constexpr int kCdCellShare = 16;  // workgroups that share a tile's flagged cells
+constexpr int kNone = 0x7fffffff;
+static_assert(kCdCap % (2 * kCdBatch) == 0 && kCdDepth % (2 * kCdBatch) == 0 && kCdBatch % 4 == 0 &&
+                  kCdSeg % 4 == 0,
+              "whole pairs of batches, read four entries at a time");
+
+#define RNNT_LAUNCH_CHECK(name)                                                    \
+  do {                                                                             \
+    hipError_t _e = hipGetLastError();                                             \
+    if (_e != hipSuccess) return check_hip(_e, "launch " name, __FILE__, __LINE__); \
+  } while (0)
+
+// order-preserving map of the floats onto the unsigned integers, and back
+__device__ inline unsigned float_key(float x) {
+  const unsigned b = __float_as_uint(x);
+  return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+}
+__device__ inline float key_float(unsigned k) {
+  return __uint_as_float((k & 0x80000000u) ? (k & 0x7fffffffu) : ~k);
+}
+
+__device__ inline int lanes_below(unsigned long long mask) {
+  return __builtin_amdgcn_mbcnt_hi((unsigned)(mask >> 32),
+                                   __builtin_amdgcn_mbcnt_lo((unsigned)mask, 0));
+}
+template <int kLane>
+__device__ inline float lane_value(float x) {
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), kLane));
+}
+
+// LDS of one workgroup: the row (Vp floats, Vp = V rounded up to 256), then this
+struct RowLists {
+  int idx[kCdWaves * kCdSeg];     // columns above the threshold, ascending: wavefront w's quarter
+  float val[kCdWaves * kCdSeg];   // of the row in [w kCdSeg, w kCdSeg + n[w]), then {0, -inf}
+                                  // up to the next multiple of 2 kCdBatch and one batch more
+  unsigned off[kCdWaves * kCdSeg];  // byte offset of the column's row in the transposed P
+  int n[kCdWaves];                // entries of each quarter (without the padding)
+  float tau[kCdWaves];            // each wavefront's threshold for its own sub-maxima
+  int bad;                        // a quarter did not fit: the list is not the whole set
+  float mtop[2][2][64];           // what the second wavefront of a block of label positions
+  int marg[2][2][64];             // found, for the first one to merge ([parity][block][lane])
+};
+
+__host__ __device__ inline int padded_row(int V) { return (V + 255) & ~255; }
+__host__ inline size_t cand_lds_bytes(int V) {
+  return sizeof(float) * (size_t)padded_row(V) + sizeof(RowLists);
+}
+
+// kVec: a piece lies inside the row or past it as a whole
+template <bool kVec>
+__device__ inline float store_piece(float* row, int v, float4 y, int V) {
+  if (kVec) {
+    if (v >= V) y = make_float4(kNegInf, kNegInf, kNegInf, kNegInf);
+  } else {
+    y.x = v < V ? y.x : kNegInf;
+    y.y = v + 1 < V ? y.y : kNegInf;
+    y.z = v + 2 < V ? y.z : kNegInf;
+    y.w = v + 3 < V ? y.w : kNegInf;
+  }
+  *reinterpret_cast<float4*>(row + v) = y;
+  return fmaxf(fmaxf(y.x, y.y), fmaxf(y.z, y.w));
+}
+
+// One row of V scores -> LDS copy (blank and padding at -inf), threshold, list.  All threads
+// call it; on return (after a barrier) row and L->idx/val/off/n/bad are complete and every
+// thread holds the threshold.  `pitch`: bytes between two columns' rows of the transposed P
+// (what L->off is counted in).
+// The threshold: every thread keeps the maximum of its own share of the row (about V/256
+// interleaved elements); each wavefront finds, by halving the interval of float keys, a value
+// with at most kCdRank of its 64 maxima above it, and the row's threshold is the largest of the
+// four.  For values drawn independently that puts about 1.4 % of a 10000-column row on the
+// list, whatever their scale; a constant or heavily tied row gets an empty list, not a full one.
+template <bool kVec, typename TIO>
+__device__ inline float stage_row(const TIO* __restrict__ src, int V, int blank, unsigned pitch,
+                                  float* row, RowLists* L) {
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int Vp = padded_row(V);
+  float m = kNegInf;
+  for (int v0 = 0; v0 < Vp; v0 += 4 * kCdThreads * kCdPre) {
+    float4 x[kCdPre];
+#pragma unroll
+    for (int j = 0; j < kCdPre; ++j) {
+      const int v = v0 + 4 * (tid + kCdThreads * j);
+      if (v < Vp) {
+        if (kVec) x[j] = load4(src + min(v, V - 4));
+        else x[j] = load4_any(src, min(v, V - 1), V);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < kCdPre; ++j) {
+      const int v = v0 + 4 * (tid + kCdThreads * j);
+      if (v < Vp) m = fmaxf(m, store_piece<kVec>(row, v, x[j], V));
+    }
+  }
+  // the blank never wins: the thread that wrote its piece takes it out (its own maximum may
+  // still count it, which only moves the threshold)
+  if (tid == ((blank >> 2) & (kCdThreads - 1))) row[blank] = kNegInf;
+
+  const unsigned key = float_key(m);
+  unsigned lo = 0u, hi = 0xffffffffu;  // at most kCdRank keys of the wavefront lie above hi
+  for (int it = 0; it < kCdBisect; ++it) {
+    const unsigned mid = lo + ((hi - lo) >> 1);
+    if (__builtin_popcountll(__ballot(key > mid)) > kCdRank) lo = mid; else hi = mid;
+  }
+  if (lane == 0) L->tau[wave] = key_float(hi);
+  if (tid == 0) L->bad = 0;
+  __syncthreads();
+  const float tau = fmaxf(fmaxf(L->tau[0], L->tau[1]), fmaxf(L->tau[2], L->tau[3]));
+
+  // this wavefront's quarter of the row, 64 columns at a time in column order
+  const int quarter = Vp >> 2, c0 = wave * quarter;
+  int* idx = L->idx + wave * kCdSeg;
+  float* val = L->val + wave * kCdSeg;
+  unsigned* off = L->off + wave * kCdSeg;
+  int count = 0;
+  for (int c = 0; c < quarter; c += 64 * 4) {
+    float x[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) x[j] = row[c0 + min(c + 64 * j, quarter - 64) + lane];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const bool hit = (c + 64 * j < quarter) && x[j] > tau;
+      const unsigned long long mask = __ballot(hit);
+      if (mask) {
+        const int pos = count + lanes_below(mask);
+        if (hit && pos < kCdCap) {
+          const int col = c0 + c + 64 * j + lane;
+          idx[pos] = col;
+          val[pos] = x[j];
+          off[pos] = (unsigned)col * pitch;
+        }
+        count += __builtin_popcountll(mask);
+      }
+    }
+  }
+  const int kept = min(count, kCdCap);
+  // fill up to a whole pair of batches, and the batch a walk requests beyond its last pair
+  if (lane < ((-kept) & (2 * kCdBatch - 1)) + kCdBatch) {
+    idx[kept + lane] = 0;
+    val[kept + lane] = kNegInf;
+    off[kept + lane] = 0u;
+  }
+  if (lane == 0) {
+    L->n[wave] = kept;
+    if (count > kCdCap) L->bad = 1;
+  }
+  __syncthreads();
+  return tau;
+}
+
+// ------------------------------------------------------------------ lists of P
+// Scratch of the list path (Uq = U rounded up to 4, Ub64 = U rounded up to 64)
+struct CandScratch {
+  float* PT;      // [B][V][Uq]   P transposed
+  int2* plist;    // [B][Ub64 / 64][kCdDepth][64]   {4 x column, score bits} of label position
+                  // 64 block + lane, ascending columns, padded with {0, -inf}
+  int* pcount;    // [B][U]   entries of each list
+  float* ptau;    // [B][U]   thresholds (+inf where the list did not fit)
+  int* tile_fail; // [B][tiles of 128 frames][tiles of 64 label positions]   flagged cells
+  int* tile_cells;  // [tiles][kCdTileLimit]   the first flagged cells of a tile (cell index in the tile)
+};
+
+template <bool kVec, typename TIO>
+__global__ __launch_bounds__(kCdThreads) void cand_lists_p_kernel(const TIO* __restrict__ P,
+                                                                  CandScratch w, Dims d) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  float* row = reinterpret_cast<float*>(lds_raw);
+  RowLists* L = reinterpret_cast<RowLists*>(row + padded_row(d.V));
+  const int b = blockIdx.y, u = blockIdx.x, tid = threadIdx.x;
+  const int blocks = (d.U + 63) >> 6;
+  int2* out = w.plist + (((size_t)b * blocks + (u >> 6)) * kCdStored) * 64 + (u & 63);
+  const int2 nothing = make_int2(0, __float_as_int(kNegInf));
+  if (u >= d.U) {  // a lane of the last block that no label position stands behind
+    for (int k = tid; k < kCdStored; k += kCdThreads) out[(size_t)k * 64] = nothing;
+    return;
+  }
+  const TIO* src = P + ((size_t)b * d.U + u) * d.V;
+  const float tau = stage_row<kVec>(src, d.V, d.blank, 0u, row, L);
+  const int c1 = L->n[0], c2 = c1 + L->n[1], c3 = c2 + L->n[2], total = c3 + L->n[3];
+  const bool bad = L->bad != 0 || total > kCdDepth;
+  for (int k = tid; k < kCdStored; k += kCdThreads) {
+    int2 e = nothing;
+    if (!bad && k < total) {
+      const int slot = k < c1 ? k : (k < c2 ? kCdSeg + k - c1
+                                            : (k < c3 ? 2 * kCdSeg + k - c2 : 3 * kCdSeg + k - c3));
+      e = make_int2(4 * L->idx[slot], __float_as_int(L->val[slot]));
+    }
+    out[(size_t)k * 64] = e;
+  }
+  if (tid == 0) {
+    w.pcount[(size_t)b * d.U + u] = bad ? 0 : total;
+    w.ptau[(size_t)b * d.U + u] = bad ? __builtin_huge_valf() : tau;
+  }
+}
+
+// PT[b][v][u] = P[b][u][v]
+template <typename TIO>
+__global__ __launch_bounds__(256) void cand_transpose_p_kernel(const TIO* __restrict__ P,
+                                                               float* __restrict__ PT, Dims d,
+                                                               int Uq) {
+  __shared__ float tile[32][33];
+  const int b = blockIdx.z, v0 = blockIdx.x * 32, u0 = blockIdx.y * 32;
+  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+  for (int i = ty; i < 32; i += 8) {
+    const int u = u0 + i, v = v0 + tx;
+    tile[i][tx] = (u < d.U && v < d.V) ? ldf(P + ((size_t)b * d.U + u) * d.V + v) : 0.0f;
+  }
+  __syncthreads();
+  for (int i = ty; i < 32; i += 8) {
+    const int v = v0 + i, u = u0 + tx;
+    if (v < d.V && u < Uq) PT[((size_t)b * d.V + v) * Uq + u] = tile[tx][i];
+  }
+}
+
+// ------------------------------------------------------------------ rows of E
+// A workgroup takes kCdFrames frames of one utterance, one at a time.  Wavefronts 0 and 1 own
+// label positions [0, 64) and [64, 128) of a block of 128 and take the first half of either
+// list (quarters 0 and 1 of the frame's list, the lower positions of the label positions'
+// lists); wavefronts 2 and 3 own the same label positions and take the second half, and hand
+// what they found to the first two through LDS.
+// A list is walked in batches of kCdBatch candidates: the batch's largest sum is one add and
+// half a three-way maximum per candidate, and a lane only notes the first batch that reached
+// its maximum.  Afterwards it walks that one batch again, from its last candidate down, and
+// keeps the lowest column whose sum equals the maximum.  Lists are in column order, so that
+// is the lowest column of the whole half; halves and lists are then merged by (larger sum,
+// lower column).
+// While a frame is evaluated, one load per cache line of the next frame's row brings that row
+// into L2, so that staging it waits for L2 and not for HBM.
+template <bool kVec, typename TIO>
+__global__ __launch_bounds__(kCdThreads) void cand_rows_kernel(const TIO* __restrict__ E,
+                                                               const int* __restrict__ inLen,
+                                                               const int* __restrict__ labLen,
+                                                               float* __restrict__ best,
+                                                               int* __restrict__ arg,
+                                                               CandScratch w, Dims d, int Uq) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  float* row = reinterpret_cast<float*>(lds_raw);
+  RowLists* L = reinterpret_cast<RowLists*>(row + padded_row(d.V));
+  const int b = blockIdx.y, t_lo = blockIdx.x * kCdFrames;
+  int Tb, Ub;
+  utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
+  if (t_lo >= Tb || Ub == 0) return;
+  const int t_hi = min(t_lo + kCdFrames, Tb);
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int blk = wave & 1, part = wave >> 1;
+  const TIO* Eb = E + (size_t)b * d.T * d.V;
+  const char* ptb = reinterpret_cast<const char*>(w.PT + (size_t)b * d.V * Uq);
+  const char* rowb = reinterpret_cast<const char*>(row);
+  const unsigned pitch = 4u * (unsigned)Uq;
+  const int blocks = (d.U + 63) >> 6;
+  const int tiles_t = (d.T + kCdTileT - 1) / kCdTileT, tiles_u = (d.U + kCdTileU - 1) / kCdTileU;
+  const int row_lines = (int)(((size_t)d.V * sizeof(TIO) + 63) >> 6);
+  unsigned touched = 0u;
+
+  // what the first block of 128 label positions needs of P's lists is the same for every frame
+  const int u_first = 64 * blk + lane;
+  const bool first_valid = u_first < Ub;
+  const float ptau_first = first_valid ? w.ptau[(size_t)b * d.U + u_first] : 0.0f;
+  int nmax_first = first_valid ? w.pcount[(size_t)b * d.U + u_first] : 0;
+#pragma unroll
+  for (int s = 1; s < 64; s <<= 1) nmax_first = max(nmax_first, __shfl_xor(nmax_first, s, 64));
+  nmax_first = __builtin_amdgcn_readfirstlane(nmax_first);
+
+  int parity = 0;
+  for (int t = t_lo; t < t_hi; ++t) {
+    const float tau = stage_row<kVec>(Eb + (size_t)t * d.V, d.V, d.blank, pitch, row, L);
+    unsigned warm[4] = {0u, 0u, 0u, 0u};
+    if (t + 1 < t_hi) {
+      const char* next = reinterpret_cast<const char*>(Eb + (size_t)(t + 1) * d.V);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int line = tid + kCdThreads * i;
+        if (line < row_lines)
+          warm[i] = *reinterpret_cast<const unsigned short*>(next + ((size_t)line << 6));
+      }
+    }
+    const bool bad = L->bad != 0;
+    for (int ub = 0; ub < Ub; ub += 2 * 64, parity ^= 1) {
+      const int u = ub + 64 * blk + lane;
+      const bool live = ub + 64 * blk < Ub;  // uniform: some of this wavefront's positions exist
+      const bool valid = u < Ub;
+      const int uc = valid ? u : Ub - 1;
+      float top = kNegInf;
+      int at = kNone;
+      if (live) {
+        // ---- A_t against the transposed P
+        const unsigned ubyte = 4u * (unsigned)uc;
+        float topa = kNegInf;
+        int wina = 0;  // first slot of the batch that reached topa
+        struct ABatch {
+          float p[kCdBatch], x[kCdBatch];
+        };
+        auto arequest = [&](int slot, ABatch& r) {
+          unsigned o[kCdBatch];
+#pragma unroll
+          for (int j = 0; j < kCdBatch; j += 4) {
+            const uint4 ov = *reinterpret_cast<const uint4*>(&L->off[slot + j]);
+            const float4 xv = *reinterpret_cast<const float4*>(&L->val[slot + j]);
+            o[j] = ov.x; o[j + 1] = ov.y; o[j + 2] = ov.z; o[j + 3] = ov.w;
+            r.x[j] = xv.x; r.x[j + 1] = xv.y; r.x[j + 2] = xv.z; r.x[j + 3] = xv.w;
+          }
+#pragma unroll
+          for (int j = 0; j < kCdBatch; ++j)
+            r.p[j] = *reinterpret_cast<const float*>(ptb + (o[j] + ubyte));
+        };
+        auto avisit = [&](int slot, const ABatch& r) {
+          float bm = kNegInf;
+#pragma unroll
+          for (int j = 0; j < kCdBatch; j += 2)
+            bm = fmaxf(fmaxf(bm, r.x[j] + r.p[j]), r.x[j + 1] + r.p[j + 1]);
+          if (bm > topa) { topa = bm; wina = slot; }
+        };
+#pragma unroll 1
+        for (int q = 2 * part; q < 2 * part + 2; ++q) {
+          const int n = __builtin_amdgcn_readfirstlane(L->n[q]);
+          const int s_lo = q * kCdSeg, s_hi = s_lo + ((n + 2 * kCdBatch - 1) & ~(2 * kCdBatch - 1));
+          if (s_lo < s_hi) {  // two batches in flight; the last request of a walk reads padding
+            ABatch a0, a1;
+            arequest(s_lo, a0);
+#pragma unroll 1
+            for (int sl = s_lo; sl < s_hi; sl += 2 * kCdBatch) {
+              arequest(sl + kCdBatch, a1);
+              avisit(sl, a0);
+              arequest(sl + 2 * kCdBatch, a0);
+              avisit(sl + kCdBatch, a1);
+            }
+          }
+        }
+        int ata = kNone;
+        if (topa > kNegInf) {  // the batch again, last candidate first
+          float p[kCdBatch], x[kCdBatch];
+          int c[kCdBatch];
+#pragma unroll
+          for (int j = 0; j < kCdBatch; ++j) {
+            c[j] = L->idx[wina + j];
+            x[j] = L->val[wina + j];
+            p[j] = *reinterpret_cast<const float*>(ptb + (L->off[wina + j] + ubyte));
+          }
+#pragma unroll
+          for (int j = kCdBatch - 1; j >= 0; --j)
+            if (x[j] + p[j] == topa) ata = c[j];
+        }
+
+        // ---- C_u against the row in LDS
+        float topc = kNegInf;
+        int winc = 0;  // first list position of the batch that reached topc
+        int nmax = nmax_first;
+        if (ub > 0) {
+          nmax = valid ? w.pcount[(size_t)b * d.U + u] : 0;
+#pragma unroll
+          for (int s = 1; s < 64; s <<= 1) nmax = max(nmax, __shfl_xor(nmax, s, 64));
+          nmax = __builtin_amdgcn_readfirstlane(nmax);
+        }
+        const int chalf = (((nmax + 1) >> 1) + 2 * kCdBatch - 1) & ~(2 * kCdBatch - 1);
+        const int c_lo = part * chalf, c_hi = min(kCdDepth, c_lo + chalf);
+        // {4 x column, score} of list position k for this lane: plk + 512 k
+        const char* plblock = reinterpret_cast<const char*>(
+            w.plist + (((size_t)b * blocks + ((ub >> 6) + blk)) * kCdStored) * 64);
+        const unsigned lane8 = 8u * (unsigned)lane;
+        struct CBatch {
+          int2 e[kCdBatch];
+        };
+        auto crequest = [&](int k0, CBatch& r) {
+          const char* kb = plblock + (size_t)k0 * 512;
+#pragma unroll
+          for (int j = 0; j < kCdBatch; ++j)
+            r.e[j] = *reinterpret_cast<const int2*>((kb + j * 512) + lane8);
+        };
+        auto cvisit = [&](int k0, const CBatch& r) {
+          float bm = kNegInf;
+#pragma unroll
+          for (int j = 0; j < kCdBatch; j += 2) {
+            const float s0 =
+                *reinterpret_cast<const float*>(rowb + r.e[j].x) + __int_as_float(r.e[j].y);
+            const float s1 = *reinterpret_cast<const float*>(rowb + r.e[j + 1].x) +
+                             __int_as_float(r.e[j + 1].y);
+            bm = fmaxf(fmaxf(bm, s0), s1);
+          }
+          if (bm > topc) { topc = bm; winc = k0; }
+        };
+        if (c_lo < c_hi && c_lo < nmax) {
+          CBatch e0, e1;
+          crequest(c_lo, e0);
+#pragma unroll 1
+          for (int k0 = c_lo; k0 < c_hi; k0 += 2 * kCdBatch) {
+            crequest(k0 + kCdBatch, e1);
+            cvisit(k0, e0);
+            crequest(k0 + 2 * kCdBatch, e0);
+            cvisit(k0 + kCdBatch, e1);
+          }
+        }
+        int atc = kNone;
+        if (topc > kNegInf) {
+          const char* kb = plblock + (size_t)winc * 512 + lane8;  // per lane
+          int2 e[kCdBatch];
+#pragma unroll
+          for (int j = 0; j < kCdBatch; ++j) e[j] = *reinterpret_cast<const int2*>(kb + j * 512);
+#pragma unroll
+          for (int j = kCdBatch - 1; j >= 0; --j)
+            if (*reinterpret_cast<const float*>(rowb + e[j].x) + __int_as_float(e[j].y) == topc)
+              atc = e[j].x >> 2;
+        }
+        top = topa;
+        at = ata;
+        if (topc > top || (topc == top && atc < at)) { top = topc; at = atc; }
+        if (part == 1) {
+          L->mtop[parity][blk][lane] = top;
+          L->marg[parity][blk][lane] = at;
+        }
+      }
+      __syncthreads();
+      if (live && part == 0) {
+        const float ot = L->mtop[parity][blk][lane];
+        const int oa = L->marg[parity][blk][lane];
+        if (ot > top || (ot == top && oa < at)) { top = ot; at = oa; }
+        const float bound =
+            tau + (ub == 0 ? ptau_first : (valid ? w.ptau[(size_t)b * d.U + u] : 0.0f));
+        const bool ok = !bad && top > bound;
+        if (valid) {
+          const size_t o = plane_row(d, b, u) + t + u;
+          best[o] = top;
+          arg[o] = ok ? at : -1;
+        }
+        const unsigned long long failed = __ballot(valid && !ok);
+        if (failed) {  // count them per tile and leave the first few where they can be found
+          const size_t tile = ((size_t)b * tiles_t + t / kCdTileT) * tiles_u + (ub >> 6) + blk;
+          int base = 0;
+          if (lane == 0) base = atomicAdd(&w.tile_fail[tile], __builtin_popcountll(failed));
+          base = __builtin_amdgcn_readfirstlane(base);
+          const int slot = base + lanes_below(failed);
+          if (valid && !ok && slot < kCdTileLimit)
+            w.tile_cells[tile * kCdTileLimit + slot] = (t & (kCdTileT - 1)) + kCdTileT * lane;
+        }
+      }
+    }
+    touched ^= warm[0] ^ warm[1] ^ warm[2] ^ warm[3];
+    // (no barrier here: after the hand-over barrier nobody reads the row or the lists again,
+    // and the hand-over arrays are next written two barriers further on)
+  }
+  // keeps the warming loads alive: 16-bit values never add up to this
+  if (touched == 0xffffffffu) best[0] = 0.0f;
+}
+
+// ------------------------------------------------------------------ flagged cells, one by one
+// Workgroup (x, y, z) of the grid (tiles of frames x kCdCellShare, tiles of label positions,
+// B) takes every kCdCellShare-th flagged cell of its tile: all columns, 256 threads, each keeping
+// the lowest column of its own maximum; (larger sum, lower column) merges them.
+template <typename TIO>
+__global__ __launch_bounds__(256) void cand_cells_kernel(const TIO* __restrict__ E,
+                                                         const TIO* __restrict__ P,
+                                                         float* __restrict__ best,
+                                                         int* __restrict__ arg,
+                                                         const int* __restrict__ tile_fail,
+                                                         const int* __restrict__ tile_cells,
+                                                         Dims d) {
+  __shared__ float rtop[4];
+  __shared__ int rarg[4];
+  const int tile_x = blockIdx.x / kCdCellShare, share = blockIdx.x % kCdCellShare;
+  const int b = blockIdx.z, t0 = tile_x * kCdTileT, u0 = blockIdx.y * kCdTileU;
+  const size_t tile = ((size_t)b * (gridDim.x / kCdCellShare) + tile_x) * gridDim.y + blockIdx.y;
+  const int failed = tile_fail[tile];
+  if (failed == 0 || failed > kCdTileLimit) return;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  for (int i = share; i < failed; i += kCdCellShare) {
+    const int c = tile_cells[tile * kCdTileLimit + i];
+    const int t = t0 + (c & (kCdTileT - 1)), u = u0 + c / kCdTileT;
+    const TIO* e = E + ((size_t)b * d.T + t) * d.V;
+    const TIO* p = P + ((size_t)b * d.U + u) * d.V;
+    float top = kNegInf;
+    int at = kNone;
+    for (int v = 4 * tid; v < d.V; v += 4 * 256) {  // four columns at a time, ascending
+      const float4 x = load4_any(e, v, d.V), y = load4_any(p, v, d.V);
+      const float s[4] = {x.x + y.x, x.y + y.y, x.z + y.z, x.w + y.w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if (v + j < d.V && v + j != d.blank && s[j] > top) { top = s[j]; at = v + j; }
+    }
+#pragma unroll
+    for (int s = 1; s < 64; s <<= 1) {
+      const float ot = __shfl_xor(top, s, 64);
+      const int oa = __shfl_xor(at, s, 64);
+      if (ot > top || (ot == top && oa < at)) { top = ot; at = oa; }
+    }
+    if (lane == 0) { rtop[wave] = top; rarg[wave] = at; }
+    __syncthreads();
+    if (tid == 0) {
+#pragma unroll
+      for (int k = 1; k < 4; ++k)
+        if (rtop[k] > top || (rtop[k] == top && rarg[k] < at)) { top = rtop[k]; at = rarg[k]; }
+      const size_t o = plane_row(d, b, u) + t + u;
+      best[o] = top;
+      arg[o] = at == kNone ? 0 : at;  // :160 nothing beat -inf: index 0 stays
+    }
+    __syncthreads();
+  }
+}
+
+__global__ void cand_zero_kernel(int* x, int n) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i < n) x[i] = 0;
+}
+
+// the skewed planes as plain [B][T][U] arrays (cells outside an utterance: -inf / -1)
+__global__ __launch_bounds__(256) void table_out_kernel(const float* __restrict__ bestS,
+                                                        const int* __restrict__ argS,
+                                                        const int* __restrict__ inLen,
+                                                        const int* __restrict__ labLen,
+                                                        float* __restrict__ best,
+                                                        int* __restrict__ arg, Dims d) {
+  const int b = blockIdx.z, t = blockIdx.y, u = blockIdx.x * 256 + threadIdx.x;
+  if (u >= d.U) return;
+  int Tb, Ub;
+  utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
+  const bool cell = t < Tb && u < Ub;
+  const size_t o = plane_row(d, b, u) + t + u, q = ((size_t)b * d.T + t) * d.U + u;
+  best[q] = cell ? bestS[o] : kNegInf;
+  arg[q] = cell ? argS[o] : -1;
+}
+
+size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
+int cand_uq(const Dims& d) { return (d.U + 3) & ~3; }
+size_t cand_tiles(const Dims& d) {
+  return (size_t)d.B * ((d.T + kCdTileT - 1) / kCdTileT) * ((d.U + kCdTileU - 1) / kCdTileU);
+}
+
+void carve(void* base, const Dims& d, CandScratch* w) {
+  char* p = static_cast<char*>(base);
+  const int Uq = cand_uq(d);
+  w->PT = reinterpret_cast<float*>(p);
+  p += align256(sizeof(float) * (size_t)d.B * d.V * Uq);
+  w->plist = reinterpret_cast<int2*>(p);
+  p += align256(sizeof(int2) * (size_t)d.B * ((d.U + 63) / 64) * kCdStored * 64);
+  w->pcount = reinterpret_cast<int*>(p);
+  p += align256(sizeof(int) * (size_t)d.B * d.U);
+  w->ptau = reinterpret_cast<float*>(p);
+  p += align256(sizeof(float) * (size_t)d.B * d.U);
+  w->tile_fail = reinterpret_cast<int*>(p);
+  p += align256(sizeof(int) * cand_tiles(d));
+  w->tile_cells = reinterpret_cast<int*>(p);
+}
+
+template <typename K>
+int allow_lds(K kernel, size_t bytes) {
+  if (bytes <= 64 * 1024) return kOk;
+  RNNT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes));
+  return kOk;
+}
+
+template <typename TIO>
+int cand_any(const TIO* E, const TIO* P, const int* inLen, const int* labLen, float* best,
+             int* arg, const Dims& d, void* scratch, hipStream_t s) {
+  CandScratch w;
+  carve(scratch, d, &w);
+  const int Uq = cand_uq(d);
+  const bool vec = d.V % 4 == 0 &&
+                   ((reinterpret_cast<uintptr_t>(E) | reinterpret_cast<uintptr_t>(P)) &
+                    (4 * sizeof(TIO) - 1)) == 0;
+  const size_t lds = cand_lds_bytes(d.V);
+  const int tiles = (int)cand_tiles(d);
+  hipLaunchKernelGGL(cand_zero_kernel, dim3((tiles + 255) / 256), dim3(256), 0, s, w.tile_fail,
+                     tiles);
+  RNNT_LAUNCH_CHECK("cand_zero_kernel");
+  hipLaunchKernelGGL((cand_transpose_p_kernel<TIO>),
+                     dim3((d.V + 31) / 32, (Uq + 31) / 32, d.B), dim3(256), 0, s, P, w.PT, d, Uq);
+  RNNT_LAUNCH_CHECK("cand_transpose_p_kernel");
+  const dim3 pgrid(((d.U + 63) / 64) * 64, d.B), rgrid((d.T + kCdFrames - 1) / kCdFrames, d.B);
+  if (vec) {
+    RNNT_TRY(allow_lds(cand_lists_p_kernel<true, TIO>, lds));
+    RNNT_TRY(allow_lds(cand_rows_kernel<true, TIO>, lds));
+    hipLaunchKernelGGL((cand_lists_p_kernel<true, TIO>), pgrid, dim3(kCdThreads), lds, s, P, w, d);
+    RNNT_LAUNCH_CHECK("cand_lists_p_kernel");
+    hipLaunchKernelGGL((cand_rows_kernel<true, TIO>), rgrid, dim3(kCdThreads), lds, s, E, inLen,
+                       labLen, best, arg, w, d, Uq);
+  } else {
+    RNNT_TRY(allow_lds(cand_lists_p_kernel<false, TIO>, lds));
+    RNNT_TRY(allow_lds(cand_rows_kernel<false, TIO>, lds));
+    hipLaunchKernelGGL((cand_lists_p_kernel<false, TIO>), pgrid, dim3(kCdThreads), lds, s, P, w,
+                       d);
+    RNNT_LAUNCH_CHECK("cand_lists_p_kernel");
+    hipLaunchKernelGGL((cand_rows_kernel<false, TIO>), rgrid, dim3(kCdThreads), lds, s, E, inLen,
+                       labLen, best, arg, w, d, Uq);
+  }
+  RNNT_LAUNCH_CHECK("cand_rows_kernel");
+  return kOk;
+}
+
+template <typename TIO>
+int cells_any(const TIO* E, const TIO* P, const int* inLen, const int* labLen, float* best,
+              int* arg, const Dims& d, void* scratch, hipStream_t s) {
+  CandScratch w;
+  carve(scratch, d, &w);
+  const dim3 grid(((d.T + kCdTileT - 1) / kCdTileT) * kCdCellShare,
+                  (d.U + kCdTileU - 1) / kCdTileU, d.B);
+  hipLaunchKernelGGL((cand_cells_kernel<TIO>), grid, dim3(256), 0, s, E, P, best, arg,
+                     w.tile_fail, w.tile_cells, d);
+  RNNT_LAUNCH_CHECK("cand_cells_kernel");
+  return kOk;
+}
+
+}  // namespace
+
+int maxplus_tile_limit() { return kCdTileLimit; }
+
+// Whether the list path can take this shape at all: the row and its lists fit the LDS of a
+// compute unit, and an offset into one utterance's transposed P fits 31 bits.
+bool maxplus_lists_possible(const Dims& d) {
+  if (d.B == 0 || d.T == 0 || d.U == 0 || d.V < 4) return false;
+  if (cand_lds_bytes(d.V) > 160 * 1024 - 1024) return false;
+  if ((size_t)d.V * cand_uq(d) >= ((size_t)1 << 29)) return false;
+  return true;
+}
+
+size_t maxplus_lists_bytes(const Dims& d) {
+  if (!maxplus_lists_possible(d)) return 0;
+  const int Uq = cand_uq(d);
+  return align256(sizeof(float) * (size_t)d.B * d.V * Uq) +
+         align256(sizeof(int2) * (size_t)d.B * ((d.U + 63) / 64) * kCdStored * 64) +
+         2 * align256(sizeof(int) * (size_t)d.B * d.U) + align256(sizeof(int) * cand_tiles(d)) +
+         align256(sizeof(int) * cand_tiles(d) * kCdTileLimit);
+}
+
+const int* maxplus_lists_tile_fail(void* scratch, const Dims& d) {
+  CandScratch w;
+  carve(scratch, d, &w);
+  return w.tile_fail;
+}
+
+int launch_table_out(const float* bestS, const int* argS, const int* inLen, const int* labLen,
+                     float* best, int* arg, const Dims& d, hipStream_t s) {
+  if (d.B == 0 || d.T == 0 || d.U == 0) return kOk;
+  hipLaunchKernelGGL(table_out_kernel, dim3((d.U + 255) / 256, d.T, d.B), dim3(256), 0, s, bestS,
+                     argS, inLen, labLen, best, arg, d);
+  RNNT_LAUNCH_CHECK("table_out_kernel");
+  return kOk;
+}
+
+int launch_maxplus_lists(const float* E, const float* P, const int* inLen, const int* labLen,
+                         float* best, int* arg, const Dims& d, void* scratch, hipStream_t s) {
+  return cand_any(E, P, inLen, labLen, best, arg, d, scratch, s);
+}
+int launch_maxplus_lists(const bf16_t* E, const bf16_t* P, const int* inLen, const int* labLen,
+                         float* best, int* arg, const Dims& d, void* scratch, hipStream_t s) {
+  return cand_any(E, P, inLen, labLen, best, arg, d, scratch, s);
+}
+int launch_maxplus_lists(const f16_t* E, const f16_t* P, const int* inLen, const int* labLen,
+                         float* best, int* arg, const Dims& d, void* scratch, hipStream_t s) {
+  return cand_any(E, P, inLen, labLen, best, arg, d, scratch, s);
+}
+int launch_maxplus_cells(const float* E, const float* P, const int* inLen, const int* labLen,
+                         float* best, int* arg, const Dims& d, void* scratch, hipStream_t s) {
+  return cells_any(E, P, inLen, labLen, best, arg, d, scratch, s);
+}
+int launch_maxplus_cells(const bf16_t* E, const bf16_t* P, const int* inLen, const int* labLen,
+                         float* best, int* arg, const Dims& d, void* scratch, hipStream_t s) {
+  return cells_any(E, P, inLen, labLen, best, arg, d, scratch, s);
+}
+int launch_maxplus_cells(const f16_t* E, const f16_t* P, const int* inLen, const int* labLen,
+                         float* best, int* arg, const Dims& d, void* scratch, hipStream_t s) {
+  return cells_any(E, P, inLen, labLen, best, arg, d, scratch, s);
+}
+
+}  // namespace rnnt

@@ -245,7 +245,8 @@ int fill(float* x, float v, int n, hipStream_t s) {
 size_t viterbi_scratch_bytes(const Dims& d) {
   const size_t plane = sizeof(float) * (size_t)d.B * d.Ua * d.Dp + 64;
   return align_up(planes_bytes(d, true)) + 2 * align_up(plane) +
-         align_up(viterbi_bits_bytes(d));
+         align_up(viterbi_bits_bytes(d)) +
+         (maxplus_uses_lists(d) ? align_up(maxplus_lists_bytes(d)) : 0);
 }
 
 // `scratch` has viterbi_scratch_bytes(d) left to take (one allocation per call, made by the caller
@@ -264,8 +265,9 @@ int viterbi_impl(const TIO* E, const TIO* P, const float* LN, int* labels,
   float* argS = static_cast<float*>(scratch.take(plane));
   unsigned long long* bits =
       static_cast<unsigned long long*>(scratch.take(viterbi_bits_bytes(d)));
+  void* lists = maxplus_uses_lists(d) ? scratch.take(maxplus_lists_bytes(d)) : nullptr;
   RNNT_STAGE(kMaxplus, launch_maxplus(E, P, inLen, labLen, bestS, reinterpret_cast<int*>(argS), d,
-                                      s));
+                                      s, lists));
   if (!ready) {
     RNNT_STAGE(kSkew, launch_skew(LN, p.lnS, inLen, labLen, d, s));
     // blank scores only: the label planes of the gather are not needed here
@@ -505,6 +507,34 @@ int rnnt_hip_set_spin_limit(int trips) {
   const int before = g_spin_limit;
   g_spin_limit = trips < 0 ? kDefaultSpinLimit : trips;
   return before;
+}
+
+int rnnt_hip_maxplus_table(const float* E, const float* P, const int* inLen, const int* labLen,
+                           float* best, int* arg, int B, int T, int U, int V, int blank,
+                           rnnt_stream_t stream) {
+  RNNT_TRY(check_dims(B, T, U, V));
+  RNNT_TRY(check_blank(V, blank));
+  if (nothing_to_do(B, T, U)) return kOk;
+  if (V == 0) return fail(kInvalid, "maxplus_table: empty vocabulary");
+  if (!E || !P || !best || !arg) return fail(kInvalid, "maxplus_table: null array argument");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const Dims d = make_dims(B, T, U, V, blank);
+  const size_t plane = sizeof(float) * (size_t)d.B * d.Ua * d.Dp + 64;
+  const bool with_lists = maxplus_uses_lists(d);
+  Scratch scratch(s);
+  RNNT_TRY(scratch.reserve(2 * align_up(plane) +
+                           (with_lists ? align_up(maxplus_lists_bytes(d)) : 0)));
+  float* bestS = static_cast<float*>(scratch.take(plane));
+  int* argS = static_cast<int*>(scratch.take(plane));
+  void* lists = with_lists ? scratch.take(maxplus_lists_bytes(d)) : nullptr;
+  RNNT_STAGE(kMaxplus, launch_maxplus(E, P, inLen, labLen, bestS, argS, d, s, lists));
+  return launch_table_out(bestS, argS, inLen, labLen, best, arg, d, s);
+}
+
+int rnnt_hip_set_maxplus_mode(int mode) {
+  if (mode < 0 || mode > 2) return fail(kInvalid, "set_maxplus_mode: mode %d (0, 1 or 2)", mode);
+  set_maxplus_mode(mode);
+  return kOk;
 }
 
 int rnnt_hip_libm_probe(const float* x, float* expf_out, float* log1pf_out, long n,

@@ -12,6 +12,7 @@
 // Operands are read from "skewed" planes [u][t+u] so that four steps are one 16-byte load per
 // lane, prefetched a group ahead.  This file is compiled with -ffp-contract=off: the rounding
 // sequence of every cell must equal the reference's.
+#include <atomic>
 #include <mutex>
 #include <type_traits>
 
@@ -924,10 +925,16 @@ __global__ __launch_bounds__(kMpThreads) void maxplus_kernel(const TIO* __restri
                                                        const int* __restrict__ inLen,
                                                        const int* __restrict__ labLen,
                                                        float* __restrict__ best,
-                                                       int* __restrict__ arg, Dims d) {
+                                                       int* __restrict__ arg, Dims d,
+                                                       const int* __restrict__ tile_fail,
+                                                       int fail_limit) {
   __shared__ __attribute__((aligned(16))) float Es[2][kMpT * kMpPitch];
   __shared__ __attribute__((aligned(16))) float Ps[2][kMpU * kMpK];
   const int b = blockIdx.z, t0 = blockIdx.x * kMpT, u0 = blockIdx.y * kMpU;
+  // after the list pass: only the tiles in which too many cells failed its test are redone
+  if (tile_fail &&
+      tile_fail[((size_t)b * gridDim.x + blockIdx.x) * gridDim.y + blockIdx.y] <= fail_limit)
+    return;
   int Tb, Ub;
   utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
   if (t0 >= Tb || u0 >= Ub) return;
@@ -1642,34 +1649,53 @@ int launch_post_beta(const Planes& p, const float* mE, const float* mP, float* W
   return kOk;
 }
 
+// 0: lists where the shape allows and the vocabulary is long enough to pay for them; 1: every
+// column for every cell; 2: lists wherever the shape allows (tests run small shapes through them)
+static std::atomic<int> g_maxplus_mode{0};
+void set_maxplus_mode(int mode) { g_maxplus_mode.store(mode); }
+constexpr int kListsFromV = 2048;
+
+bool maxplus_uses_lists(const Dims& d) {
+  const int mode = g_maxplus_mode.load();
+  if (mode == 1 || !maxplus_lists_possible(d)) return false;
+  return mode == 2 || d.V >= kListsFromV;
+}
+
 template <typename TIO>
 static int maxplus_any(const TIO* E, const TIO* P, const int* inLen, const int* labLen,
-                       float* best, int* arg, const Dims& d, hipStream_t s) {
+                       float* best, int* arg, const Dims& d, hipStream_t s, void* lists) {
   if (d.B == 0 || d.T == 0 || d.U == 0) return kOk;
+  static_assert(kMpT == 128 && kMpU == 64, "the list pass counts failures per tile of this kernel");
+  const int* tile_fail = nullptr;
+  if (lists && maxplus_uses_lists(d)) {
+    RNNT_TRY(launch_maxplus_lists(E, P, inLen, labLen, best, arg, d, lists, s));
+    tile_fail = maxplus_lists_tile_fail(lists, d);
+  }
   const dim3 grid((d.T + kMpT - 1) / kMpT, (d.U + kMpU - 1) / kMpU, d.B);
   const bool vec = d.V % 4 == 0 &&
                    ((reinterpret_cast<uintptr_t>(E) | reinterpret_cast<uintptr_t>(P)) &
                     (4 * sizeof(TIO) - 1)) == 0;
   if (vec)
     hipLaunchKernelGGL((maxplus_kernel<true, TIO>), grid, dim3(kMpThreads), 0, s, E, P, inLen,
-                       labLen, best, arg, d);
+                       labLen, best, arg, d, tile_fail, maxplus_tile_limit());
   else
     hipLaunchKernelGGL((maxplus_kernel<false, TIO>), grid, dim3(kMpThreads), 0, s, E, P, inLen,
-                       labLen, best, arg, d);
+                       labLen, best, arg, d, tile_fail, maxplus_tile_limit());
   RNNT_LAUNCH_CHECK("maxplus_kernel");
+  if (tile_fail) RNNT_TRY(launch_maxplus_cells(E, P, inLen, labLen, best, arg, d, lists, s));
   return kOk;
 }
 int launch_maxplus(const float* E, const float* P, const int* inLen, const int* labLen,
-                   float* best, int* arg, const Dims& d, hipStream_t s) {
-  return maxplus_any(E, P, inLen, labLen, best, arg, d, s);
+                   float* best, int* arg, const Dims& d, hipStream_t s, void* lists) {
+  return maxplus_any(E, P, inLen, labLen, best, arg, d, s, lists);
 }
 int launch_maxplus(const bf16_t* E, const bf16_t* P, const int* inLen, const int* labLen,
-                   float* best, int* arg, const Dims& d, hipStream_t s) {
-  return maxplus_any(E, P, inLen, labLen, best, arg, d, s);
+                   float* best, int* arg, const Dims& d, hipStream_t s, void* lists) {
+  return maxplus_any(E, P, inLen, labLen, best, arg, d, s, lists);
 }
 int launch_maxplus(const f16_t* E, const f16_t* P, const int* inLen, const int* labLen,
-                   float* best, int* arg, const Dims& d, hipStream_t s) {
-  return maxplus_any(E, P, inLen, labLen, best, arg, d, s);
+                   float* best, int* arg, const Dims& d, hipStream_t s, void* lists) {
+  return maxplus_any(E, P, inLen, labLen, best, arg, d, s, lists);
 }
 
 // 32-step words per column of the decision table (one spare)

@@ -158,11 +158,31 @@ int launch_post_beta(const Planes& p, const float* mE, const float* mP, float* W
                      const Dims& d, hipStream_t s);
 // best / arg: skewed planes ([B][Ua][Dp], see plane_row), written for valid cells only.
 int launch_maxplus(const float* E, const float* P, const int* inLen, const int* labLen,
-                   float* best, int* arg, const Dims& d, hipStream_t s);
+                   float* best, int* arg, const Dims& d, hipStream_t s, void* lists = nullptr);
 int launch_maxplus(const bf16_t* E, const bf16_t* P, const int* inLen, const int* labLen,
-                   float* best, int* arg, const Dims& d, hipStream_t s);
+                   float* best, int* arg, const Dims& d, hipStream_t s, void* lists = nullptr);
 int launch_maxplus(const f16_t* E, const f16_t* P, const int* inLen, const int* labLen,
-                   float* best, int* arg, const Dims& d, hipStream_t s);
+                   float* best, int* arg, const Dims& d, hipStream_t s, void* lists = nullptr);
+// `lists`: maxplus_lists_bytes(d) bytes of scratch, or null.  With it, and where
+// maxplus_uses_lists(d) says so, most cells are settled from short candidate lists
+// (rnnt_cand.hip) and only the cells whose bound test fails are evaluated over every column.
+bool maxplus_lists_possible(const Dims& d);
+bool maxplus_uses_lists(const Dims& d);
+size_t maxplus_lists_bytes(const Dims& d);
+void set_maxplus_mode(int mode);
+int maxplus_tile_limit();
+const int* maxplus_lists_tile_fail(void* scratch, const Dims& d);
+#define RNNT_DECLARE_LISTS(T)                                                                   \
+  int launch_maxplus_lists(const T* E, const T* P, const int* inLen, const int* labLen,        \
+                           float* best, int* arg, const Dims& d, void* scratch, hipStream_t s); \
+  int launch_maxplus_cells(const T* E, const T* P, const int* inLen, const int* labLen,        \
+                           float* best, int* arg, const Dims& d, void* scratch, hipStream_t s);
+RNNT_DECLARE_LISTS(float)
+RNNT_DECLARE_LISTS(bf16_t)
+RNNT_DECLARE_LISTS(f16_t)
+#undef RNNT_DECLARE_LISTS
+int launch_table_out(const float* bestS, const int* argS, const int* inLen, const int* labLen,
+                     float* best, int* arg, const Dims& d, hipStream_t s);
 // bestS / argS: skewed planes of the max-plus table (argS carries int bits in float storage).
 int launch_viterbi(const Planes& p, const float* bestS, const float* argS,
                    unsigned long long* gbits, const int* inLen, const int* labLen,
