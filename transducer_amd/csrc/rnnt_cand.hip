@@ -39,10 +39,11 @@ constexpr float kNegInf = -__builtin_huge_valf();
 constexpr int kCdThreads = 256;  // four wavefronts
 constexpr int kCdWaves = kCdThreads / 64;
 constexpr int kCdCap = 192;      // entries per wavefront's quarter of a row's list
-constexpr int kCdSeg = kCdCap + 8;  // a quarter's slots: one batch of padding can follow a full one
+constexpr int kCdSeg = kCdCap + 16;  // a quarter's slots: two batches of padding can follow a full one
 constexpr int kCdDepth = 384;    // entries of a stored list of P
-constexpr int kCdStored = kCdDepth + 8;  // with one batch of padding behind a full list
-constexpr int kCdRank = 30;      // sub-maxima of a wavefront (of 64) above its threshold
+constexpr int kCdStored = kCdDepth + 16;  // with two batches of padding behind a full list
+constexpr int kCdRankE = 38;     // sub-maxima of a wavefront (of 64) above its threshold: rows of E
+constexpr int kCdRankP = 22;     // ... rows of P (an entry of P's lists costs twice the bytes)
 constexpr int kCdBisect = 16;    // halvings of the key interval
 constexpr int kCdFrames = 16;    // frames per workgroup of cand_rows_kernel
 constexpr int kCdPre = 12;       // 16-byte pieces of a row a thread has in flight while staging
@@ -51,9 +52,9 @@ constexpr int kCdTileT = 128, kCdTileU = 64;  // the all-columns kernel's tile
 constexpr int kCdTileLimit = 64;  // flagged cells a tile may hold and still be redone cell by cell
 constexpr int kCdCellShare = 16;  // workgroups that share a tile's flagged cells
 constexpr int kNone = 0x7fffffff;
-static_assert(kCdCap % (2 * kCdBatch) == 0 && kCdDepth % (2 * kCdBatch) == 0 && kCdBatch % 4 == 0 &&
+static_assert(kCdCap % kCdBatch == 0 && kCdDepth % kCdBatch == 0 && kCdBatch % 4 == 0 &&
                   kCdSeg % 4 == 0,
-              "whole pairs of batches, read four entries at a time");
+              "whole batches, read four entries at a time");
 
 #define RNNT_LAUNCH_CHECK(name)                                                    \
   do {                                                                             \
@@ -118,12 +119,12 @@ __device__ inline float store_piece(float* row, int v, float4 y, int V) {
 // (what L->off is counted in).
 // The threshold: every thread keeps the maximum of its own share of the row (about V/256
 // interleaved elements); each wavefront finds, by halving the interval of float keys, a value
-// with at most kCdRank of its 64 maxima above it, and the row's threshold is the largest of the
+// with at most `rank` of its 64 maxima above it, and the row's threshold is the largest of the
 // four.  For values drawn independently that puts about 1.4 % of a 10000-column row on the
 // list, whatever their scale; a constant or heavily tied row gets an empty list, not a full one.
 template <bool kVec, typename TIO>
 __device__ inline float stage_row(const TIO* __restrict__ src, int V, int blank, unsigned pitch,
-                                  float* row, RowLists* L) {
+                                  int rank, float* row, RowLists* L) {
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int Vp = padded_row(V);
@@ -149,10 +150,10 @@ __device__ inline float stage_row(const TIO* __restrict__ src, int V, int blank,
   if (tid == ((blank >> 2) & (kCdThreads - 1))) row[blank] = kNegInf;
 
   const unsigned key = float_key(m);
-  unsigned lo = 0u, hi = 0xffffffffu;  // at most kCdRank keys of the wavefront lie above hi
+  unsigned lo = 0u, hi = 0xffffffffu;  // at most `rank` keys of the wavefront lie above hi
   for (int it = 0; it < kCdBisect; ++it) {
     const unsigned mid = lo + ((hi - lo) >> 1);
-    if (__builtin_popcountll(__ballot(key > mid)) > kCdRank) lo = mid; else hi = mid;
+    if (__builtin_popcountll(__ballot(key > mid)) > rank) lo = mid; else hi = mid;
   }
   if (lane == 0) L->tau[wave] = key_float(hi);
   if (tid == 0) L->bad = 0;
@@ -186,8 +187,8 @@ __device__ inline float stage_row(const TIO* __restrict__ src, int V, int blank,
     }
   }
   const int kept = min(count, kCdCap);
-  // fill up to a whole pair of batches, and the batch a walk requests beyond its last pair
-  if (lane < ((-kept) & (2 * kCdBatch - 1)) + kCdBatch) {
+  // fill the last batch, and the two batches a walk may touch beyond it
+  if (lane < ((-kept) & (kCdBatch - 1)) + 2 * kCdBatch) {
     idx[kept + lane] = 0;
     val[kept + lane] = kNegInf;
     off[kept + lane] = 0u;
@@ -227,7 +228,7 @@ __global__ __launch_bounds__(kCdThreads) void cand_lists_p_kernel(const TIO* __r
     return;
   }
   const TIO* src = P + ((size_t)b * d.U + u) * d.V;
-  const float tau = stage_row<kVec>(src, d.V, d.blank, 0u, row, L);
+  const float tau = stage_row<kVec>(src, d.V, d.blank, 0u, kCdRankP, row, L);
   const int c1 = L->n[0], c2 = c1 + L->n[1], c3 = c2 + L->n[2], total = c3 + L->n[3];
   const bool bad = L->bad != 0 || total > kCdDepth;
   for (int k = tid; k < kCdStored; k += kCdThreads) {
@@ -316,7 +317,7 @@ __global__ __launch_bounds__(kCdThreads) void cand_rows_kernel(const TIO* __rest
 
   int parity = 0;
   for (int t = t_lo; t < t_hi; ++t) {
-    const float tau = stage_row<kVec>(Eb + (size_t)t * d.V, d.V, d.blank, pitch, row, L);
+    const float tau = stage_row<kVec>(Eb + (size_t)t * d.V, d.V, d.blank, pitch, kCdRankE, row, L);
     unsigned warm[4] = {0u, 0u, 0u, 0u};
     if (t + 1 < t_hi) {
       const char* next = reinterpret_cast<const char*>(Eb + (size_t)(t + 1) * d.V);
@@ -363,19 +364,23 @@ __global__ __launch_bounds__(kCdThreads) void cand_rows_kernel(const TIO* __rest
             bm = fmaxf(fmaxf(bm, r.x[j] + r.p[j]), r.x[j + 1] + r.p[j + 1]);
           if (bm > topa) { topa = bm; wina = slot; }
         };
-#pragma unroll 1
-        for (int q = 2 * part; q < 2 * part + 2; ++q) {
-          const int n = __builtin_amdgcn_readfirstlane(L->n[q]);
-          const int s_lo = q * kCdSeg, s_hi = s_lo + ((n + 2 * kCdBatch - 1) & ~(2 * kCdBatch - 1));
-          if (s_lo < s_hi) {  // two batches in flight; the last request of a walk reads padding
+        {
+          // this wavefront's two quarters as one run of batches; two are in flight, and past the
+          // last one the walk requests (and with an odd count also visits) padding
+          const int n0 = __builtin_amdgcn_readfirstlane(L->n[2 * part]);
+          const int n1 = __builtin_amdgcn_readfirstlane(L->n[2 * part + 1]);
+          const int nb0 = (n0 + kCdBatch - 1) / kCdBatch, nb = nb0 + (n1 + kCdBatch - 1) / kCdBatch;
+          const int base0 = 2 * part * kCdSeg, base1 = base0 + kCdSeg - nb0 * kCdBatch;
+          auto slot_of = [&](int i) { return (i < nb0 ? base0 : base1) + i * kCdBatch; };
+          if (nb > 0) {
             ABatch a0, a1;
-            arequest(s_lo, a0);
+            arequest(slot_of(0), a0);
 #pragma unroll 1
-            for (int sl = s_lo; sl < s_hi; sl += 2 * kCdBatch) {
-              arequest(sl + kCdBatch, a1);
-              avisit(sl, a0);
-              arequest(sl + 2 * kCdBatch, a0);
-              avisit(sl + kCdBatch, a1);
+            for (int i = 0; i < nb; i += 2) {
+              arequest(slot_of(i + 1), a1);
+              avisit(slot_of(i), a0);
+              arequest(slot_of(i + 2), a0);
+              avisit(slot_of(i + 1), a1);
             }
           }
         }
@@ -404,8 +409,8 @@ __global__ __launch_bounds__(kCdThreads) void cand_rows_kernel(const TIO* __rest
           for (int s = 1; s < 64; s <<= 1) nmax = max(nmax, __shfl_xor(nmax, s, 64));
           nmax = __builtin_amdgcn_readfirstlane(nmax);
         }
-        const int chalf = (((nmax + 1) >> 1) + 2 * kCdBatch - 1) & ~(2 * kCdBatch - 1);
-        const int c_lo = part * chalf, c_hi = min(kCdDepth, c_lo + chalf);
+        const int cbatches = (nmax + kCdBatch - 1) / kCdBatch, chalf = (cbatches + 1) >> 1;
+        const int c_lo = part * chalf * kCdBatch, c_hi = min(cbatches, (part + 1) * chalf) * kCdBatch;
         // {4 x column, score} of list position k for this lane: plk + 512 k
         const char* plblock = reinterpret_cast<const char*>(
             w.plist + (((size_t)b * blocks + ((ub >> 6) + blk)) * kCdStored) * 64);
@@ -431,7 +436,7 @@ __global__ __launch_bounds__(kCdThreads) void cand_rows_kernel(const TIO* __rest
           }
           if (bm > topc) { topc = bm; winc = k0; }
         };
-        if (c_lo < c_hi && c_lo < nmax) {
+        if (c_lo < c_hi) {  // (an odd count of batches: one more, the other half's or padding)
           CBatch e0, e1;
           crequest(c_lo, e0);
 #pragma unroll 1
