@@ -197,12 +197,21 @@ int rnnt_hip_set_spin_limit(int trips);
 
 /* How the best-path calls find best[t,u] = max over v != blank of E[t,v] + P[u,v] and its
  * lowest index (transducer/transducer_cpu.cpp:158-171; the reference's device kernel scans every
- * column per cell, transducer/transducer_cuda.cu:178-207).  0 (default): from short candidate
- * lists with an exactness test per cell where the vocabulary is long enough to pay for them
- * (cells that fail the test are evaluated over every column), over every column otherwise;
- * 1: over every column always; 2: from lists wherever the shape allows.  The labels returned are
- * the same in every mode; the setting is process-wide.  No counterpart in the reference. */
+ * column per cell, transducer/transducer_cuda.cu:178-207).
+ *   0 (default): over every column, except for vocabularies of 8000 to about 17000 entries:
+ *      there each frame and each label position first gets a short list of its largest scores,
+ *      a cell is settled from the two lists where a bound proves that no other column can win,
+ *      and the remaining cells are evaluated over every column; the call looks at a sample of
+ *      the cells first and goes back to every column if too many of them fail the bound
+ *      (scores with a hard upper edge, such as uniform ones, do);
+ *   1: over every column always;
+ *   2: lists wherever a row fits a compute unit's LDS, without the sample (for tests).
+ * The labels returned are the same in every mode; the setting is process-wide.  No counterpart
+ * in the reference. */
 int rnnt_hip_set_maxplus_mode(int mode);
+/* 1 if a best-path call of this shape starts on the list path under the current mode (it may
+ * still turn back after looking at a sample of the cells), else 0. */
+int rnnt_hip_maxplus_tries_lists(int B, int T, int U, int V);
 /* The table itself, for tests of the two ways of building it: best[b][t][u] and arg[b][t][u]
  * ([B][T][U]; -inf and -1 outside an utterance's T_b x U_b cells).  fp32 scores; scratch from
  * the stream-ordered allocator. */

@@ -184,6 +184,25 @@ def test_many_failing_cells_in_a_tile_and_few():
     check(E, P, il, ll, 0)
 
 
+@pytest.mark.parametrize("dist", ["normal", "uniform", "quantised"])
+def test_default_mode_in_the_range_where_lists_are_tried(dist):
+    # V = 8192 is inside the range where the default mode starts on lists and lets a sample of
+    # the cells (two utterances, one frame in sixteen) decide whether to go on.  Uniform scores
+    # fail the bound too often and send the call back to every column, normal ones do not; a
+    # third utterance is outside the sample either way.
+    rng = np.random.default_rng(21)
+    B, T, U, V = 3, 37, 9, 8192
+    assert capi.load().rnnt_hip_maxplus_tries_lists(B, T, U, V) == 1
+    if dist == "normal":
+        E, P = rng.standard_normal((B, T, V)), rng.standard_normal((B, U, V))
+    elif dist == "uniform":
+        E, P = rng.random((B, T, V)), rng.random((B, U, V))
+    else:
+        E, P = rng.integers(0, 5, (B, T, V)) * 0.5, rng.integers(0, 5, (B, U, V)) * 0.25
+    il, ll = np.array([T, T - 5, T - 1], np.int32), np.array([U - 1, U - 3, U - 2], np.int32)
+    check(E, P, il, ll, 0, modes=(0,))
+
+
 @pytest.mark.parametrize("mode", [0, 1, 2])
 def test_decode_labels_against_oracle(mode):
     import torch

@@ -51,6 +51,7 @@ constexpr int kCdBatch = 8;      // candidates per batch (two batches in flight)
 constexpr int kCdTileT = 128, kCdTileU = 64;  // the all-columns kernel's tile
 constexpr int kCdTileLimit = 64;  // flagged cells a tile may hold and still be redone cell by cell
 constexpr int kCdCellShare = 16;  // workgroups that share a tile's flagged cells
+constexpr int kCdSampleOdds = 400; // lists go on if at most one sampled cell in this many was flagged
 constexpr int kNone = 0x7fffffff;
 static_assert(kCdCap % kCdBatch == 0 && kCdDepth % kCdBatch == 0 && kCdBatch % 4 == 0 &&
                   kCdSeg % 4 == 0,
@@ -211,15 +212,29 @@ struct CandScratch {
   float* ptau;    // [B][U]   thresholds (+inf where the list did not fit)
   int* tile_fail; // [B][tiles of 128 frames][tiles of 64 label positions]   flagged cells
   int* tile_cells;  // [tiles][kCdTileLimit]   the first flagged cells of a tile (cell index in the tile)
+  int* stats;       // [0] flagged cells of the sample, [1] cells of the sample, [2] lists go on (0 / 1)
 };
+
+// Which utterances a launch takes.  Phase 0 (the sample): utterance `first` (grid index 0) and
+// `second` (index 1, if any).  Phase 1 (the rest): every utterance but those two, and nothing at
+// all unless the sample said that lists pay for these scores (stats[2]).
+struct Pass {
+  int phase, first, second;
+};
+__device__ inline int pass_utterance(const Pass& ps, int index, const int* stats) {
+  if (ps.phase == 0) return index == 0 ? ps.first : ps.second;
+  if (stats[2] == 0 || index == ps.first || index == ps.second) return -1;
+  return index;
+}
 
 template <bool kVec, typename TIO>
 __global__ __launch_bounds__(kCdThreads) void cand_lists_p_kernel(const TIO* __restrict__ P,
-                                                                  CandScratch w, Dims d) {
+                                                                  CandScratch w, Dims d, Pass ps) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   float* row = reinterpret_cast<float*>(lds_raw);
   RowLists* L = reinterpret_cast<RowLists*>(row + padded_row(d.V));
-  const int b = blockIdx.y, u = blockIdx.x, tid = threadIdx.x;
+  const int b = pass_utterance(ps, blockIdx.y, w.stats), u = blockIdx.x, tid = threadIdx.x;
+  if (b < 0) return;
   const int blocks = (d.U + 63) >> 6;
   int2* out = w.plist + (((size_t)b * blocks + (u >> 6)) * kCdStored) * 64 + (u & 63);
   const int2 nothing = make_int2(0, __float_as_int(kNegInf));
@@ -250,9 +265,11 @@ __global__ __launch_bounds__(kCdThreads) void cand_lists_p_kernel(const TIO* __r
 template <typename TIO>
 __global__ __launch_bounds__(256) void cand_transpose_p_kernel(const TIO* __restrict__ P,
                                                                float* __restrict__ PT, Dims d,
-                                                               int Uq) {
+                                                               int Uq, Pass ps,
+                                                               const int* __restrict__ stats) {
   __shared__ float tile[32][33];
-  const int b = blockIdx.z, v0 = blockIdx.x * 32, u0 = blockIdx.y * 32;
+  const int b = pass_utterance(ps, blockIdx.z, stats), v0 = blockIdx.x * 32, u0 = blockIdx.y * 32;
+  if (b < 0) return;
   const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
   for (int i = ty; i < 32; i += 8) {
     const int u = u0 + i, v = v0 + tx;
@@ -285,15 +302,25 @@ __global__ __launch_bounds__(kCdThreads) void cand_rows_kernel(const TIO* __rest
                                                                const int* __restrict__ labLen,
                                                                float* __restrict__ best,
                                                                int* __restrict__ arg,
-                                                               CandScratch w, Dims d, int Uq) {
+                                                               CandScratch w, Dims d, int Uq, Pass ps) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   float* row = reinterpret_cast<float*>(lds_raw);
   RowLists* L = reinterpret_cast<RowLists*>(row + padded_row(d.V));
-  const int b = blockIdx.y, t_lo = blockIdx.x * kCdFrames;
+  // The sample: the first frame of every workgroup's run of frames, in the sample's utterances.
+  // The rest: every other frame of those, and all frames of the others.
+  int b = blockIdx.y;
+  if (ps.phase == 0) b = b == 0 ? ps.first : ps.second;
+  else if (w.stats[2] == 0) return;
+  const bool sampled = b == ps.first || b == ps.second;
+  int t_lo = blockIdx.x * kCdFrames;
   int Tb, Ub;
   utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
   if (t_lo >= Tb || Ub == 0) return;
-  const int t_hi = min(t_lo + kCdFrames, Tb);
+  int t_hi = min(t_lo + kCdFrames, Tb);
+  if (ps.phase == 0) t_hi = t_lo + 1;
+  else if (sampled) ++t_lo;
+  if (t_lo >= t_hi) return;
+  const int phase = ps.phase;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int blk = wave & 1, part = wave >> 1;
@@ -480,6 +507,11 @@ __global__ __launch_bounds__(kCdThreads) void cand_rows_kernel(const TIO* __rest
           arg[o] = ok ? at : -1;
         }
         const unsigned long long failed = __ballot(valid && !ok);
+        const unsigned long long cells = __ballot(valid);
+        if (phase == 0 && lane == 0) {
+          atomicAdd(&w.stats[0], __builtin_popcountll(failed));
+          atomicAdd(&w.stats[1], __builtin_popcountll(cells));
+        }
         if (failed) {  // count them per tile and leave the first few where they can be found
           const size_t tile = ((size_t)b * tiles_t + t / kCdTileT) * tiles_u + (ub >> 6) + blk;
           int base = 0;
@@ -510,14 +542,14 @@ __global__ __launch_bounds__(256) void cand_cells_kernel(const TIO* __restrict__
                                                          int* __restrict__ arg,
                                                          const int* __restrict__ tile_fail,
                                                          const int* __restrict__ tile_cells,
-                                                         Dims d) {
+                                                         const int* __restrict__ stats, Dims d) {
   __shared__ float rtop[4];
   __shared__ int rarg[4];
   const int tile_x = blockIdx.x / kCdCellShare, share = blockIdx.x % kCdCellShare;
   const int b = blockIdx.z, t0 = tile_x * kCdTileT, u0 = blockIdx.y * kCdTileU;
   const size_t tile = ((size_t)b * (gridDim.x / kCdCellShare) + tile_x) * gridDim.y + blockIdx.y;
   const int failed = tile_fail[tile];
-  if (failed == 0 || failed > kCdTileLimit) return;
+  if (stats[2] == 0 || failed == 0 || failed > kCdTileLimit) return;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   for (int i = share; i < failed; i += kCdCellShare) {
     const int c = tile_cells[tile * kCdTileLimit + i];
@@ -551,6 +583,11 @@ __global__ __launch_bounds__(256) void cand_cells_kernel(const TIO* __restrict__
     }
     __syncthreads();
   }
+}
+
+// after the sample: lists go on if few enough of its cells were flagged (one thread)
+__global__ void cand_decide_kernel(int* stats, int force) {
+  stats[2] = (force || (long long)stats[0] * kCdSampleOdds <= (long long)stats[1]) ? 1 : 0;
 }
 
 __global__ void cand_zero_kernel(int* x, int n) {
@@ -593,7 +630,8 @@ void carve(void* base, const Dims& d, CandScratch* w) {
   w->ptau = reinterpret_cast<float*>(p);
   p += align256(sizeof(float) * (size_t)d.B * d.U);
   w->tile_fail = reinterpret_cast<int*>(p);
-  p += align256(sizeof(int) * cand_tiles(d));
+  w->stats = w->tile_fail + cand_tiles(d);  // cleared together
+  p += align256(sizeof(int) * (cand_tiles(d) + 4));
   w->tile_cells = reinterpret_cast<int*>(p);
 }
 
@@ -607,7 +645,7 @@ int allow_lds(K kernel, size_t bytes) {
 
 template <typename TIO>
 int cand_any(const TIO* E, const TIO* P, const int* inLen, const int* labLen, float* best,
-             int* arg, const Dims& d, void* scratch, hipStream_t s) {
+             int* arg, const Dims& d, void* scratch, bool force, hipStream_t s) {
   CandScratch w;
   carve(scratch, d, &w);
   const int Uq = cand_uq(d);
@@ -616,30 +654,40 @@ int cand_any(const TIO* E, const TIO* P, const int* inLen, const int* labLen, fl
                     (4 * sizeof(TIO) - 1)) == 0;
   const size_t lds = cand_lds_bytes(d.V);
   const int tiles = (int)cand_tiles(d);
-  hipLaunchKernelGGL(cand_zero_kernel, dim3((tiles + 255) / 256), dim3(256), 0, s, w.tile_fail,
-                     tiles);
+  hipLaunchKernelGGL(cand_zero_kernel, dim3((tiles + 4 + 255) / 256), dim3(256), 0, s,
+                     w.tile_fail, tiles + 4);
   RNNT_LAUNCH_CHECK("cand_zero_kernel");
-  hipLaunchKernelGGL((cand_transpose_p_kernel<TIO>),
-                     dim3((d.V + 31) / 32, (Uq + 31) / 32, d.B), dim3(256), 0, s, P, w.PT, d, Uq);
-  RNNT_LAUNCH_CHECK("cand_transpose_p_kernel");
-  const dim3 pgrid(((d.U + 63) / 64) * 64, d.B), rgrid((d.T + kCdFrames - 1) / kCdFrames, d.B);
-  if (vec) {
-    RNNT_TRY(allow_lds(cand_lists_p_kernel<true, TIO>, lds));
-    RNNT_TRY(allow_lds(cand_rows_kernel<true, TIO>, lds));
-    hipLaunchKernelGGL((cand_lists_p_kernel<true, TIO>), pgrid, dim3(kCdThreads), lds, s, P, w, d);
-    RNNT_LAUNCH_CHECK("cand_lists_p_kernel");
-    hipLaunchKernelGGL((cand_rows_kernel<true, TIO>), rgrid, dim3(kCdThreads), lds, s, E, inLen,
-                       labLen, best, arg, w, d, Uq);
-  } else {
-    RNNT_TRY(allow_lds(cand_lists_p_kernel<false, TIO>, lds));
-    RNNT_TRY(allow_lds(cand_rows_kernel<false, TIO>, lds));
-    hipLaunchKernelGGL((cand_lists_p_kernel<false, TIO>), pgrid, dim3(kCdThreads), lds, s, P, w,
-                       d);
-    RNNT_LAUNCH_CHECK("cand_lists_p_kernel");
-    hipLaunchKernelGGL((cand_rows_kernel<false, TIO>), rgrid, dim3(kCdThreads), lds, s, E, inLen,
-                       labLen, best, arg, w, d, Uq);
-  }
-  RNNT_LAUNCH_CHECK("cand_rows_kernel");
+  // The sample's utterances first (their lists, their transposed P, one frame in kCdFrames),
+  // then the verdict, then everything else -- whose launches return at once if the verdict is no.
+  const Pass sample{0, 0, d.B > 1 ? d.B / 2 : -1}, rest{1, sample.first, sample.second};
+  const int nsample = d.B > 1 ? 2 : 1;
+  const int chunks = (d.T + kCdFrames - 1) / kCdFrames, ublocks64 = ((d.U + 63) / 64) * 64;
+#define RNNT_CAND_PASS(VEC, PS, NB)                                                              \
+  do {                                                                                           \
+    hipLaunchKernelGGL((cand_transpose_p_kernel<TIO>),                                           \
+                       dim3((d.V + 31) / 32, (Uq + 31) / 32, NB), dim3(256), 0, s, P, w.PT, d,   \
+                       Uq, PS, w.stats);                                                         \
+    RNNT_LAUNCH_CHECK("cand_transpose_p_kernel");                                                \
+    hipLaunchKernelGGL((cand_lists_p_kernel<VEC, TIO>), dim3(ublocks64, NB), dim3(kCdThreads),  \
+                       lds, s, P, w, d, PS);                                                     \
+    RNNT_LAUNCH_CHECK("cand_lists_p_kernel");                                                    \
+    hipLaunchKernelGGL((cand_rows_kernel<VEC, TIO>), dim3(chunks, NB), dim3(kCdThreads), lds,   \
+                       s, E, inLen, labLen, best, arg, w, d, Uq, PS);                            \
+    RNNT_LAUNCH_CHECK("cand_rows_kernel");                                                       \
+  } while (0)
+#define RNNT_CAND_PASSES(VEC)                                                                    \
+  do {                                                                                           \
+    RNNT_TRY(allow_lds(cand_lists_p_kernel<VEC, TIO>, lds));                                     \
+    RNNT_TRY(allow_lds(cand_rows_kernel<VEC, TIO>, lds));                                        \
+    RNNT_CAND_PASS(VEC, sample, nsample);                                                        \
+    hipLaunchKernelGGL(cand_decide_kernel, dim3(1), dim3(1), 0, s, w.stats, force ? 1 : 0);      \
+    RNNT_LAUNCH_CHECK("cand_decide_kernel");                                                     \
+    RNNT_CAND_PASS(VEC, rest, d.B);                                                              \
+  } while (0)
+  if (vec) RNNT_CAND_PASSES(true);
+  else RNNT_CAND_PASSES(false);
+#undef RNNT_CAND_PASS
+#undef RNNT_CAND_PASSES
   return kOk;
 }
 
@@ -651,7 +699,7 @@ int cells_any(const TIO* E, const TIO* P, const int* inLen, const int* labLen, f
   const dim3 grid(((d.T + kCdTileT - 1) / kCdTileT) * kCdCellShare,
                   (d.U + kCdTileU - 1) / kCdTileU, d.B);
   hipLaunchKernelGGL((cand_cells_kernel<TIO>), grid, dim3(256), 0, s, E, P, best, arg,
-                     w.tile_fail, w.tile_cells, d);
+                     w.tile_fail, w.tile_cells, w.stats, d);
   RNNT_LAUNCH_CHECK("cand_cells_kernel");
   return kOk;
 }
@@ -669,19 +717,30 @@ bool maxplus_lists_possible(const Dims& d) {
   return true;
 }
 
+// Where the list path is tried without being asked for: a row long enough that walking two
+// lists of a few hundred columns can beat looking at all of them (measured on normally
+// distributed scores: from about 6000 columns), and short enough that two workgroups' rows and
+// lists fit a compute unit's LDS (with one, nothing covers the staging of a row).  Whether it
+// goes through with it is decided on the scores themselves (cand_decide_kernel).
+bool maxplus_lists_pay(const Dims& d) {
+  return maxplus_lists_possible(d) && d.V >= 8000 && 2 * cand_lds_bytes(d.V) <= 160 * 1024;
+}
+
 size_t maxplus_lists_bytes(const Dims& d) {
   if (!maxplus_lists_possible(d)) return 0;
   const int Uq = cand_uq(d);
   return align256(sizeof(float) * (size_t)d.B * d.V * Uq) +
          align256(sizeof(int2) * (size_t)d.B * ((d.U + 63) / 64) * kCdStored * 64) +
-         2 * align256(sizeof(int) * (size_t)d.B * d.U) + align256(sizeof(int) * cand_tiles(d)) +
+         2 * align256(sizeof(int) * (size_t)d.B * d.U) + align256(sizeof(int) * (cand_tiles(d) + 4)) +
          align256(sizeof(int) * cand_tiles(d) * kCdTileLimit);
 }
 
-const int* maxplus_lists_tile_fail(void* scratch, const Dims& d) {
+void maxplus_lists_counters(void* scratch, const Dims& d, const int** tile_fail,
+                            const int** lists_on) {
   CandScratch w;
   carve(scratch, d, &w);
-  return w.tile_fail;
+  *tile_fail = w.tile_fail;
+  *lists_on = w.stats + 2;
 }
 
 int launch_table_out(const float* bestS, const int* argS, const int* inLen, const int* labLen,
@@ -694,16 +753,19 @@ int launch_table_out(const float* bestS, const int* argS, const int* inLen, cons
 }
 
 int launch_maxplus_lists(const float* E, const float* P, const int* inLen, const int* labLen,
-                         float* best, int* arg, const Dims& d, void* scratch, hipStream_t s) {
-  return cand_any(E, P, inLen, labLen, best, arg, d, scratch, s);
+                         float* best, int* arg, const Dims& d, void* scratch, bool force,
+                         hipStream_t s) {
+  return cand_any(E, P, inLen, labLen, best, arg, d, scratch, force, s);
 }
 int launch_maxplus_lists(const bf16_t* E, const bf16_t* P, const int* inLen, const int* labLen,
-                         float* best, int* arg, const Dims& d, void* scratch, hipStream_t s) {
-  return cand_any(E, P, inLen, labLen, best, arg, d, scratch, s);
+                         float* best, int* arg, const Dims& d, void* scratch, bool force,
+                         hipStream_t s) {
+  return cand_any(E, P, inLen, labLen, best, arg, d, scratch, force, s);
 }
 int launch_maxplus_lists(const f16_t* E, const f16_t* P, const int* inLen, const int* labLen,
-                         float* best, int* arg, const Dims& d, void* scratch, hipStream_t s) {
-  return cand_any(E, P, inLen, labLen, best, arg, d, scratch, s);
+                         float* best, int* arg, const Dims& d, void* scratch, bool force,
+                         hipStream_t s) {
+  return cand_any(E, P, inLen, labLen, best, arg, d, scratch, force, s);
 }
 int launch_maxplus_cells(const float* E, const float* P, const int* inLen, const int* labLen,
                          float* best, int* arg, const Dims& d, void* scratch, hipStream_t s) {

@@ -531,6 +531,11 @@ int rnnt_hip_maxplus_table(const float* E, const float* P, const int* inLen, con
   return launch_table_out(bestS, argS, inLen, labLen, best, arg, d, s);
 }
 
+int rnnt_hip_maxplus_tries_lists(int B, int T, int U, int V) {
+  if (B <= 0 || T <= 0 || U <= 0 || V <= 0) return 0;
+  return maxplus_uses_lists(make_dims(B, T, U, V, 0)) ? 1 : 0;
+}
+
 int rnnt_hip_set_maxplus_mode(int mode) {
   if (mode < 0 || mode > 2) return fail(kInvalid, "set_maxplus_mode: mode %d (0, 1 or 2)", mode);
   set_maxplus_mode(mode);

@@ -927,12 +927,14 @@ __global__ __launch_bounds__(kMpThreads) void maxplus_kernel(const TIO* __restri
                                                        float* __restrict__ best,
                                                        int* __restrict__ arg, Dims d,
                                                        const int* __restrict__ tile_fail,
+                                                       const int* __restrict__ lists_on,
                                                        int fail_limit) {
   __shared__ __attribute__((aligned(16))) float Es[2][kMpT * kMpPitch];
   __shared__ __attribute__((aligned(16))) float Ps[2][kMpU * kMpK];
   const int b = blockIdx.z, t0 = blockIdx.x * kMpT, u0 = blockIdx.y * kMpU;
-  // after the list pass: only the tiles in which too many cells failed its test are redone
-  if (tile_fail &&
+  // after the list pass (if it went past its sample): only the tiles in which too many cells
+  // failed its test are redone
+  if (tile_fail && lists_on[0] != 0 &&
       tile_fail[((size_t)b * gridDim.x + blockIdx.x) * gridDim.y + blockIdx.y] <= fail_limit)
     return;
   int Tb, Ub;
@@ -1649,16 +1651,14 @@ int launch_post_beta(const Planes& p, const float* mE, const float* mP, float* W
   return kOk;
 }
 
-// 0: lists where the shape allows and the vocabulary is long enough to pay for them; 1: every
+// 0: lists where they can pay (maxplus_lists_pay) and a sample of the cells says they do; 1: every
 // column for every cell; 2: lists wherever the shape allows (tests run small shapes through them)
 static std::atomic<int> g_maxplus_mode{0};
 void set_maxplus_mode(int mode) { g_maxplus_mode.store(mode); }
-constexpr int kListsFromV = 2048;
-
 bool maxplus_uses_lists(const Dims& d) {
   const int mode = g_maxplus_mode.load();
   if (mode == 1 || !maxplus_lists_possible(d)) return false;
-  return mode == 2 || d.V >= kListsFromV;
+  return mode == 2 || maxplus_lists_pay(d);
 }
 
 template <typename TIO>
@@ -1666,10 +1666,11 @@ static int maxplus_any(const TIO* E, const TIO* P, const int* inLen, const int* 
                        float* best, int* arg, const Dims& d, hipStream_t s, void* lists) {
   if (d.B == 0 || d.T == 0 || d.U == 0) return kOk;
   static_assert(kMpT == 128 && kMpU == 64, "the list pass counts failures per tile of this kernel");
-  const int* tile_fail = nullptr;
+  const int *tile_fail = nullptr, *lists_on = nullptr;
   if (lists && maxplus_uses_lists(d)) {
-    RNNT_TRY(launch_maxplus_lists(E, P, inLen, labLen, best, arg, d, lists, s));
-    tile_fail = maxplus_lists_tile_fail(lists, d);
+    RNNT_TRY(launch_maxplus_lists(E, P, inLen, labLen, best, arg, d, lists,
+                                  g_maxplus_mode.load() == 2, s));
+    maxplus_lists_counters(lists, d, &tile_fail, &lists_on);
   }
   const dim3 grid((d.T + kMpT - 1) / kMpT, (d.U + kMpU - 1) / kMpU, d.B);
   const bool vec = d.V % 4 == 0 &&
@@ -1677,10 +1678,10 @@ static int maxplus_any(const TIO* E, const TIO* P, const int* inLen, const int* 
                     (4 * sizeof(TIO) - 1)) == 0;
   if (vec)
     hipLaunchKernelGGL((maxplus_kernel<true, TIO>), grid, dim3(kMpThreads), 0, s, E, P, inLen,
-                       labLen, best, arg, d, tile_fail, maxplus_tile_limit());
+                       labLen, best, arg, d, tile_fail, lists_on, maxplus_tile_limit());
   else
     hipLaunchKernelGGL((maxplus_kernel<false, TIO>), grid, dim3(kMpThreads), 0, s, E, P, inLen,
-                       labLen, best, arg, d, tile_fail, maxplus_tile_limit());
+                       labLen, best, arg, d, tile_fail, lists_on, maxplus_tile_limit());
   RNNT_LAUNCH_CHECK("maxplus_kernel");
   if (tile_fail) RNNT_TRY(launch_maxplus_cells(E, P, inLen, labLen, best, arg, d, lists, s));
   return kOk;

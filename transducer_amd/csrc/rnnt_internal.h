@@ -167,14 +167,17 @@ int launch_maxplus(const f16_t* E, const f16_t* P, const int* inLen, const int* 
 // maxplus_uses_lists(d) says so, most cells are settled from short candidate lists
 // (rnnt_cand.hip) and only the cells whose bound test fails are evaluated over every column.
 bool maxplus_lists_possible(const Dims& d);
+bool maxplus_lists_pay(const Dims& d);
 bool maxplus_uses_lists(const Dims& d);
 size_t maxplus_lists_bytes(const Dims& d);
 void set_maxplus_mode(int mode);
 int maxplus_tile_limit();
-const int* maxplus_lists_tile_fail(void* scratch, const Dims& d);
+void maxplus_lists_counters(void* scratch, const Dims& d, const int** tile_fail,
+                            const int** lists_on);
 #define RNNT_DECLARE_LISTS(T)                                                                   \
   int launch_maxplus_lists(const T* E, const T* P, const int* inLen, const int* labLen,        \
-                           float* best, int* arg, const Dims& d, void* scratch, hipStream_t s); \
+                           float* best, int* arg, const Dims& d, void* scratch, bool force,       \
+                           hipStream_t s);                                                      \
   int launch_maxplus_cells(const T* E, const T* P, const int* inLen, const int* labLen,        \
                            float* best, int* arg, const Dims& d, void* scratch, hipStream_t s);
 RNNT_DECLARE_LISTS(float)
