@@ -277,6 +277,7 @@ def viterbi_main(args, name, cfg, opt, capi, d, device):
         dtype16 = {"bf16": torch.bfloat16, "f16": torch.float16}[io]
         E, P = E.to(dtype16), P.to(dtype16)
     entry = "rnnt_hip_viterbi_decode" + ("_" + io if io else "")
+    capi.call("rnnt_hip_set_maxplus_mode", args.maxplus_mode)
 
     def step():
         capi.call(entry, p(E), p(P), p(d_il), p(d_ll), p(out_labels), B, T, U1, V, 0, stream)
@@ -317,7 +318,7 @@ def viterbi_main(args, name, cfg, opt, capi, d, device):
         "scaling": "weak", "vs_baseline": None,
         "dtype": "f32 arithmetic on %s scores" % io if io else "f32", "data": "synthetic",
         "config": {"workload": describe(name, cfg, opt), "seed": args.seed,
-                   "valid_lattice_cells": int(cells)},
+                   "valid_lattice_cells": int(cells), "maxplus_mode": args.maxplus_mode},
         "roofline": roofline,
         "stage_ms_per_step": per_step,
         "checks": checks,
@@ -334,6 +335,9 @@ def main():
     ap.add_argument("--workload", default="cfg4", choices=sorted(WORKLOADS))
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--maxplus-mode", type=int, default=0, choices=(0, 1, 2),
+                    help="best-path workloads: how the table of best labels is built "
+                         "(rnnt_hip_set_maxplus_mode: 0 default, 1 every column, 2 lists)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one plain elementwise copy of the emissions array (B*T*V*4 "
                          "bytes read, as many written) so that a counter run can scale "
