@@ -87,6 +87,41 @@ def test_gaussian_scores(shape):
     check(rng.standard_normal((B, T, V)), rng.standard_normal((B, U, V)), il, ll, blank)
 
 
+@pytest.mark.parametrize("seed", range(24))
+def test_random_shapes_lengths_and_distributions(seed):
+    rng = np.random.default_rng(9000 + seed)
+    B = int(rng.integers(1, 5))
+    T = int(rng.choice([1, 2, 15, 16, 17, 33, 129])) if rng.random() < 0.5 else int(rng.integers(1, 200))
+    U = int(rng.choice([1, 2, 63, 64, 65, 128, 129])) if rng.random() < 0.5 else int(rng.integers(1, 140))
+    V = int(rng.choice([4, 5, 255, 256, 257, 1024, 1027, 4096, 8192, 12001])) if rng.random() < 0.6 \
+        else int(rng.integers(4, 3000))
+    while B * T * U * V > 2e7:
+        if T > 4: T //= 2
+        elif U > 4: U //= 2
+        else: V //= 2
+    blank = int(rng.integers(0, V))
+    kind = int(rng.integers(0, 4))
+    if kind == 0:
+        E, P = rng.standard_normal((B, T, V)) * 3, rng.standard_normal((B, U, V))
+    elif kind == 1:
+        E, P = rng.random((B, T, V)), rng.random((B, U, V))
+    elif kind == 2:  # few distinct values
+        E, P = rng.integers(-2, 3, (B, T, V)) * 0.5, rng.integers(-2, 3, (B, U, V)) * 0.25
+    else:  # values rounded to bfloat16 (many equal sums), some -inf
+        E = rng.standard_normal((B, T, V)).astype(np.float32)
+        P = rng.standard_normal((B, U, V)).astype(np.float32)
+        E = (E.view(np.uint32) & 0xffff0000).view(np.float32).copy()
+        P = (P.view(np.uint32) & 0xffff0000).view(np.float32).copy()
+        E[rng.random(E.shape) < 0.01] = -np.inf
+    il = rng.integers(0, T + 1, B).astype(np.int32)
+    ll = rng.integers(0, U, B).astype(np.int32)
+    if rng.random() < 0.5:
+        il[0], ll[0] = T, U - 1
+    print("B=%d T=%d U=%d V=%d blank=%d kind=%d il=%s ll=%s" % (B, T, U, V, blank, kind, il.tolist(),
+                                                           ll.tolist()), flush=True)
+    check(E, P, il, ll, blank, modes=(0, 1, 2))
+
+
 @pytest.mark.parametrize("shape", [(2, 12, 6, 40, 0), (1, 30, 20, 2048, 5), (1, 16, 101, 10000, 0)],
                          ids=lambda s: "B%d_T%d_U%d_V%d_blank%d" % s)
 def test_quantised_scores_tie_everywhere(shape):

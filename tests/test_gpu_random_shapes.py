@@ -110,3 +110,11 @@ def test_random_shape_against_the_oracle(seed):
         for b in range(B):
             if il[b] > 0:
                 assert np.array_equal(paths[b, :ll[b]], wantp[b, :ll[b]])
+        # and with the table of best labels built from candidate lists instead of every column
+        from transducer_amd import capi
+        capi.call("rnnt_hip_set_maxplus_mode", 2)
+        try:
+            paths_lists = gpu_viterbi(c, LN, blank=blank)
+        finally:
+            capi.call("rnnt_hip_set_maxplus_mode", 0)
+        assert np.array_equal(paths_lists, paths)
