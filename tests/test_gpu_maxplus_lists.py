@@ -76,7 +76,9 @@ def lengths(rng, B, T, U):
 SHAPES = [(2, 9, 5, 12, 0), (1, 3, 2, 5, 4), (2, 17, 7, 100, 3), (1, 40, 70, 130, 0),
           (2, 33, 101, 1000, 999), (1, 20, 130, 515, 7), (2, 21, 9, 4096, 0),
           (1, 35, 66, 10000, 0), (1, 19, 4, 10001, 10000), (1, 5, 3, 4, 1),
-          (1, 6, 3, 20000, 0)]  # the last one: a row past 64 KB of LDS
+          (1, 6, 3, 20000, 0),   # a row past 64 KB of LDS
+          (1, 3, 2, 36000, 5),   # the longest row the list path takes (156 KB of LDS)
+          (2, 9, 300, 700, 3)]   # three blocks of 128 label positions
 
 
 @pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "B%d_T%d_U%d_V%d_blank%d" % s)

@@ -441,7 +441,9 @@ __global__ __launch_bounds__(kCdThreads) void cand_rows_kernel(const TIO* __rest
         // {4 x column, score} of list position k for this lane: plk + 512 k
         const char* plblock = reinterpret_cast<const char*>(
             w.plist + (((size_t)b * blocks + ((ub >> 6) + blk)) * kCdStored) * 64);
-        const unsigned lane8 = 8u * (unsigned)lane;
+        // (lanes past the utterance's last label position read the last one's entries: the same
+        // cache lines, where their own would be lines nobody needs)
+        const unsigned lane8 = 8u * (unsigned)(uc - ub - 64 * blk);
         struct CBatch {
           int2 e[kCdBatch];
         };
