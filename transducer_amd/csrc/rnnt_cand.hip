@@ -47,6 +47,7 @@ constexpr int kCdRankP = 22;     // ... rows of P (an entry of P's lists costs t
 constexpr int kCdBisect = 16;    // halvings of the key interval
 constexpr int kCdFrames = 16;    // frames per workgroup of cand_rows_kernel
 constexpr int kCdPre = 12;       // 16-byte pieces of a row a thread has in flight while staging
+constexpr int kCdAhead = 10;     // 16-byte pieces of the next row a thread holds while a row is evaluated
 constexpr int kCdBatch = 8;      // candidates per batch (two batches in flight)
 constexpr int kCdTileT = 128, kCdTileU = 64;  // the all-columns kernel's tile
 constexpr int kCdTileLimit = 64;  // flagged cells a tile may hold and still be redone cell by cell
@@ -89,7 +90,7 @@ struct RowLists {
   unsigned off[kCdWaves * kCdSeg];  // byte offset of the column's row in the transposed P
   int n[kCdWaves];                // entries of each quarter (without the padding)
   float tau[kCdWaves];            // each wavefront's threshold for its own sub-maxima
-  int bad;                        // a quarter did not fit: the list is not the whole set
+  int bad[2];                     // a quarter did not fit: the list is not the whole set (by frame parity)
   float mtop[2][2][64];           // what the second wavefront of a block of label positions
   int marg[2][2][64];             // found, for the first one to merge ([parity][block][lane])
 };
@@ -157,7 +158,7 @@ __device__ inline float stage_row(const TIO* __restrict__ src, int V, int blank,
     if (__builtin_popcountll(__ballot(key > mid)) > rank) lo = mid; else hi = mid;
   }
   if (lane == 0) L->tau[wave] = key_float(hi);
-  if (tid == 0) L->bad = 0;
+  if (tid == 0) L->bad[0] = 0;
   __syncthreads();
   const float tau = fmaxf(fmaxf(L->tau[0], L->tau[1]), fmaxf(L->tau[2], L->tau[3]));
 
@@ -196,10 +197,120 @@ __device__ inline float stage_row(const TIO* __restrict__ src, int V, int blank,
   }
   if (lane == 0) {
     L->n[wave] = kept;
-    if (count > kCdCap) L->bad = 1;
+    if (count > kCdCap) L->bad[0] = 1;
   }
   __syncthreads();
   return tau;
+}
+
+// The same for a row that is requested one frame ahead (cand_rows_kernel, rows of at most
+// 256 kCdAhead columns per wavefront): each wavefront owns one quarter of the row from the load
+// on, keeps it in registers while the previous frame is evaluated, and builds its part of the
+// list from those registers with its own threshold (any threshold is valid per column; the
+// row's bound is the largest of the four).  No wavefront waits for another before the one
+// barrier that ends the staging.
+struct QuarterRegs {
+  float4 x[kCdAhead];
+};
+template <bool kVec, typename TIO>
+__device__ inline void fetch_quarter(const TIO* __restrict__ src, int V, QuarterRegs& r) {
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int quarter = padded_row(V) >> 2, c0 = wave * quarter;
+#pragma unroll
+  for (int i = 0; i < kCdAhead; ++i) {
+    const int c = 256 * i + 4 * lane, v = c0 + c;
+    if (c < quarter) {
+      if (kVec) r.x[i] = load4(src + min(v, V - 4));
+      else r.x[i] = load4_any(src, min(v, V - 1), V);
+    }
+  }
+}
+
+template <bool kVec>
+__device__ inline void commit_quarter(QuarterRegs& r, int V, int blank, unsigned pitch, int rank,
+                                      int parity, float* row, RowLists* L) {
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int quarter = padded_row(V) >> 2, c0 = wave * quarter;
+  const float4 none = make_float4(kNegInf, kNegInf, kNegInf, kNegInf);
+  float m = kNegInf;
+#pragma unroll
+  for (int i = 0; i < kCdAhead; ++i) {
+    const int c = 256 * i + 4 * lane, v = c0 + c;
+    float4 y = none;
+    if (c < quarter) {
+      y = r.x[i];
+      if (kVec) {
+        if (v >= V) y = none;
+      } else {
+        y.x = v < V ? y.x : kNegInf;
+        y.y = v + 1 < V ? y.y : kNegInf;
+        y.z = v + 2 < V ? y.z : kNegInf;
+        y.w = v + 3 < V ? y.w : kNegInf;
+      }
+      *reinterpret_cast<float4*>(row + v) = y;
+      m = fmaxf(m, fmaxf(fmaxf(y.x, y.y), fmaxf(y.z, y.w)));
+    }
+    r.x[i] = y;
+  }
+  const int blank_wave = blank / quarter;  // uniform
+  if (wave == blank_wave && lane == (((blank - c0) & 255) >> 2)) row[blank] = kNegInf;
+
+  const unsigned key = float_key(m);
+  unsigned lo = 0u, hi = 0xffffffffu;
+  for (int it = 0; it < kCdBisect; ++it) {
+    const unsigned mid = lo + ((hi - lo) >> 1);
+    if (__builtin_popcountll(__ballot(key > mid)) > rank) lo = mid; else hi = mid;
+  }
+  const float tau = key_float(hi);
+
+  int* idx = L->idx + wave * kCdSeg;
+  float* val = L->val + wave * kCdSeg;
+  unsigned* off = L->off + wave * kCdSeg;
+  int count = 0;
+#pragma unroll
+  for (int i = 0; i < kCdAhead; ++i) {
+    const float4 y = r.x[i];
+    const bool h0 = y.x > tau, h1 = y.y > tau, h2 = y.z > tau, h3 = y.w > tau;
+    const unsigned long long m0 = __ballot(h0), m1 = __ballot(h1), m2 = __ballot(h2),
+                             m3 = __ballot(h3);
+    if (m0 | m1 | m2 | m3) {  // column order: lane after lane, a lane's four columns in turn
+      int pos = count + lanes_below(m0) + lanes_below(m1) + lanes_below(m2) + lanes_below(m3);
+      const int col = c0 + 256 * i + 4 * lane;
+      const float e[4] = {y.x, y.y, y.z, y.w};
+      const bool h[4] = {h0, h1, h2, h3};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        if (h[j]) {
+          if (pos < kCdCap) {
+            idx[pos] = col + j;
+            val[pos] = e[j];
+            off[pos] = (unsigned)(col + j) * pitch;
+          }
+          ++pos;
+        }
+      }
+      count += __builtin_popcountll(m0) + __builtin_popcountll(m1) + __builtin_popcountll(m2) +
+               __builtin_popcountll(m3);
+    }
+  }
+  const int kept = min(count, kCdCap);
+  if (wave == blank_wave) {  // the registers still hold the blank's score: out of the list with it
+#pragma unroll 1
+    for (int k = lane; k < kept; k += 64)
+      if (idx[k] == blank) val[k] = kNegInf;
+  }
+  if (lane < ((-kept) & (kCdBatch - 1)) + 2 * kCdBatch) {
+    idx[kept + lane] = 0;
+    val[kept + lane] = kNegInf;
+    off[kept + lane] = 0u;
+  }
+  if (lane == 0) {
+    L->n[wave] = kept;
+    L->tau[wave] = tau;
+    if (count > kCdCap) L->bad[parity] = 1;
+  }
 }
 
 // ------------------------------------------------------------------ lists of P
@@ -245,7 +356,7 @@ __global__ __launch_bounds__(kCdThreads) void cand_lists_p_kernel(const TIO* __r
   const TIO* src = P + ((size_t)b * d.U + u) * d.V;
   const float tau = stage_row<kVec>(src, d.V, d.blank, 0u, kCdRankP, row, L);
   const int c1 = L->n[0], c2 = c1 + L->n[1], c3 = c2 + L->n[2], total = c3 + L->n[3];
-  const bool bad = L->bad != 0 || total > kCdDepth;
+  const bool bad = L->bad[0] != 0 || total > kCdDepth;
   for (int k = tid; k < kCdStored; k += kCdThreads) {
     int2 e = nothing;
     if (!bad && k < total) {
@@ -296,7 +407,7 @@ __global__ __launch_bounds__(256) void cand_transpose_p_kernel(const TIO* __rest
 // lower column).
 // While a frame is evaluated, one load per cache line of the next frame's row brings that row
 // into L2, so that staging it waits for L2 and not for HBM.
-template <bool kVec, typename TIO>
+template <bool kVec, bool kAhead, typename TIO>
 __global__ __launch_bounds__(kCdThreads) void cand_rows_kernel(const TIO* __restrict__ E,
                                                                const int* __restrict__ inLen,
                                                                const int* __restrict__ labLen,
@@ -342,20 +453,39 @@ __global__ __launch_bounds__(kCdThreads) void cand_rows_kernel(const TIO* __rest
   for (int s = 1; s < 64; s <<= 1) nmax_first = max(nmax_first, __shfl_xor(nmax_first, s, 64));
   nmax_first = __builtin_amdgcn_readfirstlane(nmax_first);
 
+  QuarterRegs ahead;
+  if (kAhead) {
+    if (tid == 0) L->bad[0] = L->bad[1] = 0;
+    fetch_quarter<kVec>(Eb + (size_t)t_lo * d.V, d.V, ahead);
+    __syncthreads();
+  }
   int parity = 0;
   for (int t = t_lo; t < t_hi; ++t) {
-    const float tau = stage_row<kVec>(Eb + (size_t)t * d.V, d.V, d.blank, pitch, kCdRankE, row, L);
+    float tau;
+    bool bad;
     unsigned warm[4] = {0u, 0u, 0u, 0u};
-    if (t + 1 < t_hi) {
-      const char* next = reinterpret_cast<const char*>(Eb + (size_t)(t + 1) * d.V);
+    if (kAhead) {
+      // this frame's row is in registers; the next one's is requested before the evaluation
+      const int fp = (t - t_lo) & 1;
+      commit_quarter<kVec>(ahead, d.V, d.blank, pitch, kCdRankE, fp, row, L);
+      if (t + 1 < t_hi) fetch_quarter<kVec>(Eb + (size_t)(t + 1) * d.V, d.V, ahead);
+      __syncthreads();
+      if (tid == 0) L->bad[fp ^ 1] = 0;  // the next frame's flag: nobody sets it before the hand-over barrier
+      tau = fmaxf(fmaxf(L->tau[0], L->tau[1]), fmaxf(L->tau[2], L->tau[3]));
+      bad = L->bad[fp] != 0;
+    } else {
+      tau = stage_row<kVec>(Eb + (size_t)t * d.V, d.V, d.blank, pitch, kCdRankE, row, L);
+      if (t + 1 < t_hi) {
+        const char* next = reinterpret_cast<const char*>(Eb + (size_t)(t + 1) * d.V);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int line = tid + kCdThreads * i;
-        if (line < row_lines)
-          warm[i] = *reinterpret_cast<const unsigned short*>(next + ((size_t)line << 6));
+        for (int i = 0; i < 4; ++i) {
+          const int line = tid + kCdThreads * i;
+          if (line < row_lines)
+            warm[i] = *reinterpret_cast<const unsigned short*>(next + ((size_t)line << 6));
+        }
       }
+      bad = L->bad[0] != 0;
     }
-    const bool bad = L->bad != 0;
     for (int ub = 0; ub < Ub; ub += 2 * 64, parity ^= 1) {
       const int u = ub + 64 * blk + lane;
       const bool live = ub + 64 * blk < Ub;  // uniform: some of this wavefront's positions exist
@@ -663,6 +793,7 @@ int cand_any(const TIO* E, const TIO* P, const int* inLen, const int* labLen, fl
   // then the verdict, then everything else -- whose launches return at once if the verdict is no.
   const Pass sample{0, 0, d.B > 1 ? d.B / 2 : -1}, rest{1, sample.first, sample.second};
   const int nsample = d.B > 1 ? 2 : 1;
+  const bool ahead = padded_row(d.V) <= 4 * 256 * kCdAhead;  // a quarter fits the registers kept for it
   const int chunks = (d.T + kCdFrames - 1) / kCdFrames, ublocks64 = ((d.U + 63) / 64) * 64;
 #define RNNT_CAND_PASS(VEC, PS, NB)                                                              \
   do {                                                                                           \
@@ -673,14 +804,19 @@ int cand_any(const TIO* E, const TIO* P, const int* inLen, const int* labLen, fl
     hipLaunchKernelGGL((cand_lists_p_kernel<VEC, TIO>), dim3(ublocks64, NB), dim3(kCdThreads),  \
                        lds, s, P, w, d, PS);                                                     \
     RNNT_LAUNCH_CHECK("cand_lists_p_kernel");                                                    \
-    hipLaunchKernelGGL((cand_rows_kernel<VEC, TIO>), dim3(chunks, NB), dim3(kCdThreads), lds,   \
-                       s, E, inLen, labLen, best, arg, w, d, Uq, PS);                            \
+    if (ahead)                                                                                   \
+      hipLaunchKernelGGL((cand_rows_kernel<VEC, true, TIO>), dim3(chunks, NB), dim3(kCdThreads), \
+                         lds, s, E, inLen, labLen, best, arg, w, d, Uq, PS);                     \
+    else                                                                                         \
+      hipLaunchKernelGGL((cand_rows_kernel<VEC, false, TIO>), dim3(chunks, NB),                  \
+                         dim3(kCdThreads), lds, s, E, inLen, labLen, best, arg, w, d, Uq, PS);   \
     RNNT_LAUNCH_CHECK("cand_rows_kernel");                                                       \
   } while (0)
 #define RNNT_CAND_PASSES(VEC)                                                                    \
   do {                                                                                           \
     RNNT_TRY(allow_lds(cand_lists_p_kernel<VEC, TIO>, lds));                                     \
-    RNNT_TRY(allow_lds(cand_rows_kernel<VEC, TIO>, lds));                                        \
+    RNNT_TRY(allow_lds(cand_rows_kernel<VEC, true, TIO>, lds));                                  \
+    RNNT_TRY(allow_lds(cand_rows_kernel<VEC, false, TIO>, lds));                                        \
     RNNT_CAND_PASS(VEC, sample, nsample);                                                        \
     hipLaunchKernelGGL(cand_decide_kernel, dim3(1), dim3(1), 0, s, w.stats, force ? 1 : 0);      \
     RNNT_LAUNCH_CHECK("cand_decide_kernel");                                                     \
