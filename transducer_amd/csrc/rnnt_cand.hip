@@ -12,20 +12,23 @@
 // evaluated over all columns afterwards.  The thresholds only decide how long the lists are
 // and how many cells fail, never what is returned.
 //
-//   * cand_lists_p_kernel: threshold and sorted list for every row of P, plus P transposed
+//   * cand_lists_p_kernel: threshold and ascending list for every row of P, plus P transposed
 //     (cand_transpose_p_kernel) so that one candidate column's 64 label positions are one
 //     256-byte read;
-//   * cand_rows_kernel: per frame, the row of E goes into LDS, gets its threshold and list, and
-//     the two wavefronts of the workgroup (64 label positions each) evaluate A_t against the
-//     transposed P and C_u against the LDS row;
-//   * tiles of 128 frames x 64 label positions with more than kCdTileLimit flagged cells are
-//     redone by the all-columns kernel (maxplus_kernel), the others' flagged cells one by one
+//   * cand_rows_kernel: per frame, the row of E goes into LDS and gets its threshold and list,
+//     and the four wavefronts of the workgroup (64 label positions each, half of either list)
+//     evaluate A_t against the transposed P and C_u against the LDS row;
+//   * a sample of the cells goes first (two utterances, one frame in kCdFrames): if too many of
+//     them fail the test -- scores with a hard upper edge do -- everything else returns at once
+//     and the all-columns kernel (maxplus_kernel) builds the whole table;
+//   * otherwise tiles of 128 frames x 64 label positions with more than kCdTileLimit flagged
+//     cells are redone by that kernel, the others' flagged cells one by one
 //     (cand_cells_kernel): the cost of a failed test is bounded either way.
 //
-// A threshold is the value with about kCdTarget of the 256 sub-maxima of a row above it (each
-// thread keeps the maxima of two interleaved subsets of its elements): for values drawn
-// independently that puts about 1.4 % of a 10000-column row on the list, whatever their scale,
-// and a constant or heavily tied row gets an empty list instead of a full one.
+// A threshold is a value with at most kCdRankE (kCdRankP) of a wavefront's 64 per-thread maxima
+// above it, the largest of the four wavefronts' values: about 190 (90) of 10000 independently
+// drawn scores end up on a list, whatever their scale, and a constant or heavily tied row gets
+// an empty list instead of a full one.
 #include <hip/hip_runtime.h>
 
 #include <type_traits>
