@@ -242,21 +242,23 @@ int fill(float* x, float v, int n, hipStream_t s) {
 }
 
 // Scratch the best-path stages need (planes, the two max-plus planes, the decision table).
-size_t viterbi_scratch_bytes(const Dims& d) {
+// `lists`: whether this call builds its table of best labels from candidate lists (asked once
+// per call, so that what is reserved and what is taken agree whatever another thread sets).
+size_t viterbi_scratch_bytes(const Dims& d, bool lists) {
   const size_t plane = sizeof(float) * (size_t)d.B * d.Ua * d.Dp + 64;
   return align_up(planes_bytes(d, true)) + 2 * align_up(plane) +
          align_up(viterbi_bits_bytes(d)) +
-         (maxplus_uses_lists(d) ? align_up(maxplus_lists_bytes(d)) : 0);
+         (lists ? align_up(maxplus_lists_bytes(d)) : 0);
 }
 
-// `scratch` has viterbi_scratch_bytes(d) left to take (one allocation per call, made by the caller
+// `scratch` has viterbi_scratch_bytes(d, with_lists) left to take (one allocation per call, made by the caller
 // together with whatever else it needs: the allocator calls are a visible part of a small decode).
 // With `ready`, the lattice planes were carved by the caller and already hold LN and the blank
 // scores (the log-normaliser left them there): no transposing copy, no gather.
 template <typename TIO>
 int viterbi_impl(const TIO* E, const TIO* P, const float* LN, int* labels,
                         const int* inLen, const int* labLen, const Dims& d, Scratch& scratch,
-                        hipStream_t s, const Planes* ready = nullptr) {
+                        hipStream_t s, bool with_lists, const Planes* ready = nullptr) {
   const size_t plane = sizeof(float) * (size_t)d.B * d.Ua * d.Dp + 64;
   Planes p;
   if (ready) p = *ready;
@@ -265,7 +267,7 @@ int viterbi_impl(const TIO* E, const TIO* P, const float* LN, int* labels,
   float* argS = static_cast<float*>(scratch.take(plane));
   unsigned long long* bits =
       static_cast<unsigned long long*>(scratch.take(viterbi_bits_bytes(d)));
-  void* lists = maxplus_uses_lists(d) ? scratch.take(maxplus_lists_bytes(d)) : nullptr;
+  void* lists = with_lists ? scratch.take(maxplus_lists_bytes(d)) : nullptr;
   RNNT_STAGE(kMaxplus, launch_maxplus(E, P, inLen, labLen, bestS, reinterpret_cast<int*>(argS), d,
                                       s, lists));
   if (!ready) {
@@ -384,9 +386,10 @@ int lowp_viterbi_decode(const TIO* E, const TIO* P, const int* inLen, const int*
   if (!lse_stream_supported(E, d)) return fail(kInvalid, "%s: B*T*U too large", who);
   Scratch scratch(s);
   const size_t yb = lse_scratch_bytes(d);
+  const bool with_lists = maxplus_uses_lists(d);
   RNNT_TRY(scratch.reserve(align_up(sizeof(float) * (size_t)B * T) +
                            align_up(sizeof(float) * (size_t)B * U) + align_up(yb) +
-                           viterbi_scratch_bytes(d)));
+                           viterbi_scratch_bytes(d, with_lists)));
   float* mE = static_cast<float*>(scratch.take(sizeof(float) * (size_t)B * T));
   float* mP = static_cast<float*>(scratch.take(sizeof(float) * (size_t)B * U));
   void* ys = scratch.take(yb);
@@ -397,7 +400,7 @@ int lowp_viterbi_decode(const TIO* E, const TIO* P, const int* inLen, const int*
   RNNT_STAGE(kYplanes, launch_yplanes(P, mP, ys, labLen, d, s));
   RNNT_STAGE(kLse, launch_lse_stream(E, mE, mP, nullptr, ys, inLen, labLen, d, s, nullptr, p.elS,
                                      p.eb, p.lnS));
-  return viterbi_impl(E, P, nullptr, labels, inLen, labLen, d, scratch, s, &p);
+  return viterbi_impl(E, P, nullptr, labels, inLen, labLen, d, scratch, s, with_lists, &p);
 }
 
 // The best-path decode on fp32 scores; `scratch` decides where its device scratch comes from.
@@ -413,11 +416,12 @@ int decode_fp32(const float* E, const float* P, const int* inLen, const int* lab
   const Dims d = make_dims(B, T, U, V, blank);
   if (!lse_stream_supported(E, d)) return fail(kInvalid, "%s: B*T*U too large", who);
   const size_t yb = lse_scratch_bytes(d);
+  const bool with_lists = maxplus_uses_lists(d);
   // LN and the blank scores go straight into the lattice planes, as in the whole-loss path
   // (no row-major LN, no transposing copy, no gather)
   RNNT_TRY(scratch.reserve(align_up(sizeof(float) * (size_t)B * T) +
                            align_up(sizeof(float) * (size_t)B * U) + align_up(yb) +
-                           viterbi_scratch_bytes(d)));
+                           viterbi_scratch_bytes(d, with_lists)));
   float* mE = static_cast<float*>(scratch.take(sizeof(float) * (size_t)B * T));
   float* mP = static_cast<float*>(scratch.take(sizeof(float) * (size_t)B * U));
   void* ys = scratch.take(yb);
@@ -427,7 +431,7 @@ int decode_fp32(const float* E, const float* P, const int* inLen, const int* lab
   RNNT_TRY(log_norms_stages(E, P, mE, mP, nullptr, ys, inLen, labLen, d, s, &p, nullptr,
                             &ln_in_plane));
   if (!ln_in_plane) return fail(kInvalid, "%s: log-normaliser left no plane", who);
-  return viterbi_impl(E, P, nullptr, labels, inLen, labLen, d, scratch, s, &p);
+  return viterbi_impl(E, P, nullptr, labels, inLen, labLen, d, scratch, s, with_lists, &p);
 }
 
 // ---------------------------------------------------------------- built-in scratch
@@ -661,8 +665,9 @@ int rnnt_hip_viterbi(const float* E, const float* P, const float* LN, int* label
   const Dims d = make_dims(B, T, U, V, blank);
   hipStream_t s = static_cast<hipStream_t>(stream);
   Scratch scratch(s);
-  RNNT_TRY(scratch.reserve(viterbi_scratch_bytes(d)));
-  return viterbi_impl(E, P, LN, labels, inLen, labLen, d, scratch, s);
+  const bool with_lists = maxplus_uses_lists(d);
+  RNNT_TRY(scratch.reserve(viterbi_scratch_bytes(d, with_lists)));
+  return viterbi_impl(E, P, LN, labels, inLen, labLen, d, scratch, s, with_lists);
 }
 
 int rnnt_hip_log_norms(const float* E, const float* P, float* LN, const int* inLen,
