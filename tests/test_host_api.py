@@ -245,3 +245,37 @@ def test_setup_py_builds_an_importable_package_outside_the_source_tree(tmp_path)
     env = dict(os.environ, PYTHONPATH=lib)
     out = subprocess.check_output(["python", "-c", code], cwd=str(tmp_path), env=env, text=True)
     assert out.split()[0] == "1" and lib in out.split()[2]
+
+
+def test_the_build_module_imports_without_the_built_libraries():
+    # `python -m transducer_amd.build` must work in a tree that holds no .so yet (or a stale
+    # one): importing the package or its build module loads no native library; asking for
+    # TransducerLoss does.
+    import subprocess
+    import sys
+    code = ("import sys, transducer_amd, transducer_amd.build; "
+            "assert 'transducer_amd._transducer' not in sys.modules; "
+            "assert 'transducer_amd.torch_binding' not in sys.modules; "
+            "from transducer_amd import TransducerLoss; "
+            "assert 'transducer_amd._transducer' in sys.modules")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    subprocess.check_call([sys.executable, "-c", code], cwd=root)
+
+
+def test_maxplus_mode_setter_and_query():
+    from transducer_amd import capi
+    lib = capi.load()
+    try:
+        capi.call("rnnt_hip_set_maxplus_mode", 1)
+        assert lib.rnnt_hip_maxplus_tries_lists(32, 2000, 101, 10000) == 0
+        capi.call("rnnt_hip_set_maxplus_mode", 2)
+        assert lib.rnnt_hip_maxplus_tries_lists(2, 10, 5, 64) == 1
+        assert lib.rnnt_hip_maxplus_tries_lists(2, 10, 5, 50000) == 0  # a row past a CU's LDS
+        capi.call("rnnt_hip_set_maxplus_mode", 0)
+        assert lib.rnnt_hip_maxplus_tries_lists(32, 2000, 101, 10000) == 1
+        assert lib.rnnt_hip_maxplus_tries_lists(32, 2000, 101, 2000) == 0
+        assert lib.rnnt_hip_maxplus_tries_lists(32, 2000, 101, 32000) == 0
+        with pytest.raises(capi.RnntHipError):
+            capi.call("rnnt_hip_set_maxplus_mode", 7)
+    finally:
+        capi.call("rnnt_hip_set_maxplus_mode", 0)
