@@ -32,7 +32,8 @@ def case(B, T, U, V, seed):
 
 
 def test_static_decode_equals_the_allocating_decode_twice_in_a_row_second_call_smaller():
-    # one utterance of the headline shape (11 MB of the array), then a small ragged batch with a
+    # one utterance of the headline shape (16 MB of the array; its table of best labels comes from
+    # candidate lists at this vocabulary), then a small ragged batch with a
     # different vocabulary, label axis and blank index, then the first again
     first = case(1, 2000, 100, 10000, seed=1)
     second = case(3, 130, 37, 515, seed=2)
