@@ -241,6 +241,46 @@ def test_headline_viterbi_one_utterance_bit_exact_and_batch_independent(near_tie
     assert torch.equal(decode_on_device(c.cut(longest))[0], fused[longest])
 
 
+@pytest.mark.parametrize("near_ties,V,dist", [(False, 10000, "normal"), (True, 10000, "normal"),
+                                              (False, 10001, "normal"), (False, 10000, "uniform"),
+                                              (False, 12000, "bf16")])
+def test_headline_table_of_best_labels_is_the_same_however_it_is_built(near_ties, V, dist):
+    # every cell of the whole batch: over every column (mode 1), from candidate lists with the
+    # sampled go/no-go (default) and from lists unconditionally (mode 2) -- same maxima, same
+    # lowest indices.  Uniform scores make the default turn back after its sample; scores
+    # rounded to bfloat16 tie in many cells.
+    c = DeviceBatch(CONFIGS["cfg5"]._replace(V=V), seed=6, near_ties=near_ties)
+    if dist == "uniform":
+        c.E.uniform_(0.0, 1.0)
+        c.P.uniform_(0.0, 1.0)
+    elif dist == "bf16":
+        c.E = c.E.to(torch.bfloat16).float()
+        c.P = c.P.to(torch.bfloat16).float()
+    B, T, U, V = c.dims
+    tables = []
+    for mode in (1, 0, 2):
+        best = torch.full((B, T, U), float("nan"), device="cuda:0")
+        arg = torch.full((B, T, U), -7, dtype=torch.int32, device="cuda:0")
+        capi.call("rnnt_hip_set_maxplus_mode", mode)
+        try:
+            capi.call("rnnt_hip_maxplus_table", ptr(c.E), ptr(c.P), ptr(c.il), ptr(c.ll), ptr(best),
+                      ptr(arg), B, T, U, V, 0, None)
+            torch.cuda.synchronize()
+        finally:
+            capi.call("rnnt_hip_set_maxplus_mode", 0)
+        tables.append((best, arg))
+    for best, arg in tables[1:]:
+        assert torch.equal(arg, tables[0][1])
+        assert torch.equal(best.view(torch.int32), tables[0][0].view(torch.int32))
+    # and the all-columns table itself on one frame of one utterance, against numpy
+    b, t = 3, 777
+    s = (c.E[b, t][None, :] + c.P[b]).cpu().numpy()
+    s[:, 0] = -np.inf
+    ub = int(c.ll_h[b]) + 1
+    assert np.array_equal(tables[0][1][b, t, :ub].cpu().numpy(), s.argmax(axis=1)[:ub])
+    assert np.array_equal(tables[0][0][b, t, :ub].cpu().numpy(), s.max(axis=1)[:ub])
+
+
 # ------------------------------------------------------------------ the smaller configurations, whole
 # Fraction of gradient entries outside rel 1e-4 / abs 1e-5 end to end, each side with its own
 # log-normaliser: about three times what was measured, per configuration (egrads, pgrads).
