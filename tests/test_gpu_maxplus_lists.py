@@ -223,12 +223,12 @@ def test_many_failing_cells_in_a_tile_and_few():
 
 @pytest.mark.parametrize("dist", ["normal", "uniform", "quantised"])
 def test_default_mode_in_the_range_where_lists_are_tried(dist):
-    # V = 8192 is inside the range where the default mode starts on lists and lets a sample of
+    # V = 8192 with more than 64 label positions is inside the range where the default mode starts on lists and lets a sample of
     # the cells (two utterances, one frame in sixteen) decide whether to go on.  Uniform scores
     # fail the bound too often and send the call back to every column, normal ones do not; a
     # third utterance is outside the sample either way.
     rng = np.random.default_rng(21)
-    B, T, U, V = 3, 37, 9, 8192
+    B, T, U, V = 3, 37, 70, 8192
     assert capi.load().rnnt_hip_maxplus_tries_lists(B, T, U, V) == 1
     if dist == "normal":
         E, P = rng.standard_normal((B, T, V)), rng.standard_normal((B, U, V))

@@ -25,12 +25,16 @@
 //     cells are redone by that kernel, the others' flagged cells one by one
 //     (cand_cells_kernel): the cost of a failed test is bounded either way.
 //
-// A threshold is a value with at most kCdRankE (kCdRankP) of a wavefront's 64 per-thread maxima
-// above it, the largest of the four wavefronts' values: about 190 (90) of 10000 independently
-// drawn scores end up on a list, whatever their scale, and a constant or heavily tied row gets
-// an empty list instead of a full one.
+// A threshold is a value with at most `rank` of a wavefront's 64 per-thread maxima above it.
+// The rank is chosen (list_rank) so that about 2.3 sqrt(V) columns of a row of E and 0.75 sqrt(V)
+// of a row of P end up on a list if the scores are drawn independently, whatever their scale
+// (230 and 75 of 10000; the square root keeps the share of cells that fail the test level as
+// the vocabulary grows; an entry of P's lists costs twice the bytes of one of E's, hence the
+// shorter lists there; about one cell in 800 then fails the test at V = 10000, and each of
+// those costs the 80 KB of its two rows once more).  A constant or heavily tied row gets an empty list instead of a full one.
 #include <hip/hip_runtime.h>
 
+#include <cmath>
 #include <type_traits>
 
 #include "rnnt_internal.h"
@@ -45,16 +49,18 @@ constexpr int kCdCap = 192;      // entries per wavefront's quarter of a row's l
 constexpr int kCdSeg = kCdCap + 16;  // a quarter's slots: two batches of padding can follow a full one
 constexpr int kCdDepth = 384;    // entries of a stored list of P
 constexpr int kCdStored = kCdDepth + 16;  // with two batches of padding behind a full list
-constexpr int kCdRankE = 38;     // sub-maxima of a wavefront (of 64) above its threshold: rows of E
-constexpr int kCdRankP = 22;     // ... rows of P (an entry of P's lists costs twice the bytes)
+constexpr float kCdListE = 2.31f;  // list lengths the ranks are derived from, in units of sqrt(V): rows of E
+constexpr float kCdListP = 0.88f;  // ... rows of P (their threshold is the largest of four wavefronts' values,
+                                   // so their lists come out a fifth shorter than that)
 constexpr int kCdBisect = 16;    // halvings of the key interval
 constexpr int kCdFrames = 16;    // frames per workgroup of cand_rows_kernel
 constexpr int kCdPre = 12;       // 16-byte pieces of a row a thread has in flight while staging
-constexpr int kCdAhead = 10;     // 16-byte pieces of the next row a thread holds while a row is evaluated
+constexpr int kCdAheadShort = 10;  // 16-byte pieces of the next row a thread holds while a row is
+constexpr int kCdAheadLong = 17;   // evaluated: rows of up to 10240 / 17408 columns
 constexpr int kCdBatch = 8;      // candidates per batch (two batches in flight)
 constexpr int kCdTileT = 128, kCdTileU = 64;  // the all-columns kernel's tile
 constexpr int kCdTileLimit = 64;  // flagged cells a tile may hold and still be redone cell by cell
-constexpr int kCdCellShare = 16;  // workgroups that share a tile's flagged cells
+constexpr int kCdCellShare = 16;  // wavefronts (of four workgroups) that share a tile's flagged cells
 constexpr int kCdSampleOdds = 400; // lists go on if at most one sampled cell in this many was flagged
 constexpr int kNone = 0x7fffffff;
 static_assert(kCdCap % kCdBatch == 0 && kCdDepth % kCdBatch == 0 && kCdBatch % 4 == 0 &&
@@ -207,21 +213,22 @@ __device__ inline float stage_row(const TIO* __restrict__ src, int V, int blank,
 }
 
 // The same for a row that is requested one frame ahead (cand_rows_kernel, rows of at most
-// 256 kCdAhead columns per wavefront): each wavefront owns one quarter of the row from the load
+// 256 kPieces columns per wavefront): each wavefront owns one quarter of the row from the load
 // on, keeps it in registers while the previous frame is evaluated, and builds its part of the
 // list from those registers with its own threshold (any threshold is valid per column; the
 // row's bound is the largest of the four).  No wavefront waits for another before the one
 // barrier that ends the staging.
+template <int kPieces>
 struct QuarterRegs {
-  float4 x[kCdAhead];
+  float4 x[kPieces > 0 ? kPieces : 1];
 };
-template <bool kVec, typename TIO>
-__device__ inline void fetch_quarter(const TIO* __restrict__ src, int V, QuarterRegs& r) {
+template <bool kVec, int kPieces, typename TIO>
+__device__ inline void fetch_quarter(const TIO* __restrict__ src, int V, QuarterRegs<kPieces>& r) {
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int quarter = padded_row(V) >> 2, c0 = wave * quarter;
 #pragma unroll
-  for (int i = 0; i < kCdAhead; ++i) {
+  for (int i = 0; i < kPieces; ++i) {
     const int c = 256 * i + 4 * lane, v = c0 + c;
     if (c < quarter) {
       if (kVec) r.x[i] = load4(src + min(v, V - 4));
@@ -230,8 +237,8 @@ __device__ inline void fetch_quarter(const TIO* __restrict__ src, int V, Quarter
   }
 }
 
-template <bool kVec>
-__device__ inline void commit_quarter(QuarterRegs& r, int V, int blank, unsigned pitch, int rank,
+template <bool kVec, int kPieces>
+__device__ inline void commit_quarter(QuarterRegs<kPieces>& r, int V, int blank, unsigned pitch, int rank,
                                       int parity, float* row, RowLists* L) {
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -239,7 +246,7 @@ __device__ inline void commit_quarter(QuarterRegs& r, int V, int blank, unsigned
   const float4 none = make_float4(kNegInf, kNegInf, kNegInf, kNegInf);
   float m = kNegInf;
 #pragma unroll
-  for (int i = 0; i < kCdAhead; ++i) {
+  for (int i = 0; i < kPieces; ++i) {
     const int c = 256 * i + 4 * lane, v = c0 + c;
     float4 y = none;
     if (c < quarter) {
@@ -273,7 +280,7 @@ __device__ inline void commit_quarter(QuarterRegs& r, int V, int blank, unsigned
   unsigned* off = L->off + wave * kCdSeg;
   int count = 0;
 #pragma unroll
-  for (int i = 0; i < kCdAhead; ++i) {
+  for (int i = 0; i < kPieces; ++i) {
     const float4 y = r.x[i];
     const bool h0 = y.x > tau, h1 = y.y > tau, h2 = y.z > tau, h3 = y.w > tau;
     const unsigned long long m0 = __ballot(h0), m1 = __ballot(h1), m2 = __ballot(h2),
@@ -343,7 +350,8 @@ __device__ inline int pass_utterance(const Pass& ps, int index, const int* stats
 
 template <bool kVec, typename TIO>
 __global__ __launch_bounds__(kCdThreads) void cand_lists_p_kernel(const TIO* __restrict__ P,
-                                                                  CandScratch w, Dims d, Pass ps) {
+                                                                  CandScratch w, Dims d, Pass ps,
+                                                                  int2 ranks) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   float* row = reinterpret_cast<float*>(lds_raw);
   RowLists* L = reinterpret_cast<RowLists*>(row + padded_row(d.V));
@@ -357,7 +365,7 @@ __global__ __launch_bounds__(kCdThreads) void cand_lists_p_kernel(const TIO* __r
     return;
   }
   const TIO* src = P + ((size_t)b * d.U + u) * d.V;
-  const float tau = stage_row<kVec>(src, d.V, d.blank, 0u, kCdRankP, row, L);
+  const float tau = stage_row<kVec>(src, d.V, d.blank, 0u, ranks.y, row, L);
   const int c1 = L->n[0], c2 = c1 + L->n[1], c3 = c2 + L->n[2], total = c3 + L->n[3];
   const bool bad = L->bad[0] != 0 || total > kCdDepth;
   for (int k = tid; k < kCdStored; k += kCdThreads) {
@@ -410,13 +418,16 @@ __global__ __launch_bounds__(256) void cand_transpose_p_kernel(const TIO* __rest
 // lower column).
 // While a frame is evaluated, one load per cache line of the next frame's row brings that row
 // into L2, so that staging it waits for L2 and not for HBM.
-template <bool kVec, bool kAhead, typename TIO>
+// kPieces: 16-byte pieces per thread of the row requested ahead (0: rows too long for that are
+// staged when their turn comes).
+template <bool kVec, int kPieces, typename TIO>
 __global__ __launch_bounds__(kCdThreads) void cand_rows_kernel(const TIO* __restrict__ E,
                                                                const int* __restrict__ inLen,
                                                                const int* __restrict__ labLen,
                                                                float* __restrict__ best,
                                                                int* __restrict__ arg,
-                                                               CandScratch w, Dims d, int Uq, Pass ps) {
+                                                               CandScratch w, Dims d, int Uq, Pass ps,
+                                                               int2 ranks) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   float* row = reinterpret_cast<float*>(lds_raw);
   RowLists* L = reinterpret_cast<RowLists*>(row + padded_row(d.V));
@@ -456,10 +467,11 @@ __global__ __launch_bounds__(kCdThreads) void cand_rows_kernel(const TIO* __rest
   for (int s = 1; s < 64; s <<= 1) nmax_first = max(nmax_first, __shfl_xor(nmax_first, s, 64));
   nmax_first = __builtin_amdgcn_readfirstlane(nmax_first);
 
-  QuarterRegs ahead;
+  constexpr bool kAhead = kPieces > 0;
+  QuarterRegs<kPieces> ahead;
   if (kAhead) {
     if (tid == 0) L->bad[0] = L->bad[1] = 0;
-    fetch_quarter<kVec>(Eb + (size_t)t_lo * d.V, d.V, ahead);
+    fetch_quarter<kVec, kPieces>(Eb + (size_t)t_lo * d.V, d.V, ahead);
     __syncthreads();
   }
   int parity = 0;
@@ -470,14 +482,14 @@ __global__ __launch_bounds__(kCdThreads) void cand_rows_kernel(const TIO* __rest
     if (kAhead) {
       // this frame's row is in registers; the next one's is requested before the evaluation
       const int fp = (t - t_lo) & 1;
-      commit_quarter<kVec>(ahead, d.V, d.blank, pitch, kCdRankE, fp, row, L);
-      if (t + 1 < t_hi) fetch_quarter<kVec>(Eb + (size_t)(t + 1) * d.V, d.V, ahead);
+      commit_quarter<kVec, kPieces>(ahead, d.V, d.blank, pitch, ranks.x, fp, row, L);
+      if (t + 1 < t_hi) fetch_quarter<kVec, kPieces>(Eb + (size_t)(t + 1) * d.V, d.V, ahead);
       __syncthreads();
       if (tid == 0) L->bad[fp ^ 1] = 0;  // the next frame's flag: nobody sets it before the hand-over barrier
       tau = fmaxf(fmaxf(L->tau[0], L->tau[1]), fmaxf(L->tau[2], L->tau[3]));
       bad = L->bad[fp] != 0;
     } else {
-      tau = stage_row<kVec>(Eb + (size_t)t * d.V, d.V, d.blank, pitch, kCdRankE, row, L);
+      tau = stage_row<kVec>(Eb + (size_t)t * d.V, d.V, d.blank, pitch, ranks.x, row, L);
       if (t + 1 < t_hi) {
         const char* next = reinterpret_cast<const char*>(Eb + (size_t)(t + 1) * d.V);
 #pragma unroll
@@ -667,9 +679,9 @@ __global__ __launch_bounds__(kCdThreads) void cand_rows_kernel(const TIO* __rest
 }
 
 // ------------------------------------------------------------------ flagged cells, one by one
-// Workgroup (x, y, z) of the grid (tiles of frames x kCdCellShare, tiles of label positions,
-// B) takes every kCdCellShare-th flagged cell of its tile: all columns, 256 threads, each keeping
-// the lowest column of its own maximum; (larger sum, lower column) merges them.
+// Every wavefront of workgroup (x, y, z) of the grid (tiles of frames x kCdCellShare / 4, tiles of
+// label positions, B) takes every kCdCellShare-th flagged cell of its tile: all columns, each
+// lane keeping the lowest column of its own maximum; (larger sum, lower column) merges the lanes.
 template <typename TIO>
 __global__ __launch_bounds__(256) void cand_cells_kernel(const TIO* __restrict__ E,
                                                          const TIO* __restrict__ P,
@@ -678,27 +690,38 @@ __global__ __launch_bounds__(256) void cand_cells_kernel(const TIO* __restrict__
                                                          const int* __restrict__ tile_fail,
                                                          const int* __restrict__ tile_cells,
                                                          const int* __restrict__ stats, Dims d) {
-  __shared__ float rtop[4];
-  __shared__ int rarg[4];
-  const int tile_x = blockIdx.x / kCdCellShare, share = blockIdx.x % kCdCellShare;
+  constexpr int kGroups = kCdCellShare / 4;
+  const int tile_x = blockIdx.x / kGroups, group = blockIdx.x % kGroups;
   const int b = blockIdx.z, t0 = tile_x * kCdTileT, u0 = blockIdx.y * kCdTileU;
-  const size_t tile = ((size_t)b * (gridDim.x / kCdCellShare) + tile_x) * gridDim.y + blockIdx.y;
+  const size_t tile = ((size_t)b * (gridDim.x / kGroups) + tile_x) * gridDim.y + blockIdx.y;
   const int failed = tile_fail[tile];
   if (stats[2] == 0 || failed == 0 || failed > kCdTileLimit) return;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  for (int i = share; i < failed; i += kCdCellShare) {
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  for (int i = 4 * group + wave; i < failed; i += kCdCellShare) {
     const int c = tile_cells[tile * kCdTileLimit + i];
     const int t = t0 + (c & (kCdTileT - 1)), u = u0 + c / kCdTileT;
     const TIO* e = E + ((size_t)b * d.T + t) * d.V;
     const TIO* p = P + ((size_t)b * d.U + u) * d.V;
     float top = kNegInf;
     int at = kNone;
-    for (int v = 4 * tid; v < d.V; v += 4 * 256) {  // four columns at a time, ascending
-      const float4 x = load4_any(e, v, d.V), y = load4_any(p, v, d.V);
-      const float s[4] = {x.x + y.x, x.y + y.y, x.z + y.z, x.w + y.w};
+    // four columns at a time, ascending; eight such pieces of either row requested together
+    for (int v0 = 4 * lane; v0 < d.V; v0 += 4 * 64 * 8) {
+      float4 x[8], y[8];
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
-        if (v + j < d.V && v + j != d.blank && s[j] > top) { top = s[j]; at = v + j; }
+      for (int k = 0; k < 8; ++k) {
+        const int v = min(v0 + 4 * 64 * k, d.V - 1);
+        x[k] = load4_any(e, v, d.V);
+        y[k] = load4_any(p, v, d.V);
+      }
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        const int v = v0 + 4 * 64 * k;
+        const float s[4] = {x[k].x + y[k].x, x[k].y + y[k].y, x[k].z + y[k].z, x[k].w + y[k].w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          if (v + j < d.V && v + j != d.blank && s[j] > top) { top = s[j]; at = v + j; }
+      }
     }
 #pragma unroll
     for (int s = 1; s < 64; s <<= 1) {
@@ -706,17 +729,11 @@ __global__ __launch_bounds__(256) void cand_cells_kernel(const TIO* __restrict__
       const int oa = __shfl_xor(at, s, 64);
       if (ot > top || (ot == top && oa < at)) { top = ot; at = oa; }
     }
-    if (lane == 0) { rtop[wave] = top; rarg[wave] = at; }
-    __syncthreads();
-    if (tid == 0) {
-#pragma unroll
-      for (int k = 1; k < 4; ++k)
-        if (rtop[k] > top || (rtop[k] == top && rarg[k] < at)) { top = rtop[k]; at = rarg[k]; }
+    if (lane == 0) {
       const size_t o = plane_row(d, b, u) + t + u;
       best[o] = top;
       arg[o] = at == kNone ? 0 : at;  // :160 nothing beat -inf: index 0 stays
     }
-    __syncthreads();
   }
 }
 
@@ -770,6 +787,15 @@ void carve(void* base, const Dims& d, CandScratch* w) {
   w->tile_cells = reinterpret_cast<int*>(p);
 }
 
+// The rank (of 64 per-thread maxima of a wavefront) whose threshold leaves about
+// length_in_sqrt_v * sqrt(V) of V independently drawn scores above it: a thread's maximum lies
+// above a threshold that a share p of the scores exceeds with probability 1 - (1-p)^(V/256).
+int list_rank(float length_in_sqrt_v, int V) {
+  const double n = length_in_sqrt_v * std::sqrt((double)V);
+  const double r = 64.0 * (1.0 - std::exp(-n / 256.0));
+  return r < 8.0 ? 8 : (r > 56.0 ? 56 : (int)(r + 0.5));
+}
+
 template <typename K>
 int allow_lds(K kernel, size_t bytes) {
   if (bytes <= 64 * 1024) return kOk;
@@ -796,7 +822,8 @@ int cand_any(const TIO* E, const TIO* P, const int* inLen, const int* labLen, fl
   // then the verdict, then everything else -- whose launches return at once if the verdict is no.
   const Pass sample{0, 0, d.B > 1 ? d.B / 2 : -1}, rest{1, sample.first, sample.second};
   const int nsample = d.B > 1 ? 2 : 1;
-  const bool ahead = padded_row(d.V) <= 4 * 256 * kCdAhead;  // a quarter fits the registers kept for it
+  const int2 ranks = make_int2(list_rank(kCdListE, d.V), list_rank(kCdListP, d.V));
+  const int pieces = (padded_row(d.V) / 4 + 255) / 256;  // 16-byte pieces per thread of a quarter of a row
   const int chunks = (d.T + kCdFrames - 1) / kCdFrames, ublocks64 = ((d.U + 63) / 64) * 64;
 #define RNNT_CAND_PASS(VEC, PS, NB)                                                              \
   do {                                                                                           \
@@ -805,21 +832,27 @@ int cand_any(const TIO* E, const TIO* P, const int* inLen, const int* labLen, fl
                        Uq, PS, w.stats);                                                         \
     RNNT_LAUNCH_CHECK("cand_transpose_p_kernel");                                                \
     hipLaunchKernelGGL((cand_lists_p_kernel<VEC, TIO>), dim3(ublocks64, NB), dim3(kCdThreads),  \
-                       lds, s, P, w, d, PS);                                                     \
+                       lds, s, P, w, d, PS, ranks);                                              \
     RNNT_LAUNCH_CHECK("cand_lists_p_kernel");                                                    \
-    if (ahead)                                                                                   \
-      hipLaunchKernelGGL((cand_rows_kernel<VEC, true, TIO>), dim3(chunks, NB), dim3(kCdThreads), \
-                         lds, s, E, inLen, labLen, best, arg, w, d, Uq, PS);                     \
+    if (pieces <= kCdAheadShort)                                                                 \
+      hipLaunchKernelGGL((cand_rows_kernel<VEC, kCdAheadShort, TIO>), dim3(chunks, NB),          \
+                         dim3(kCdThreads), lds, s, E, inLen, labLen, best, arg, w, d, Uq, PS,    \
+                         ranks);                                                                 \
+    else if (pieces <= kCdAheadLong)                                                             \
+      hipLaunchKernelGGL((cand_rows_kernel<VEC, kCdAheadLong, TIO>), dim3(chunks, NB),           \
+                         dim3(kCdThreads), lds, s, E, inLen, labLen, best, arg, w, d, Uq, PS,    \
+                         ranks);                                                                 \
     else                                                                                         \
-      hipLaunchKernelGGL((cand_rows_kernel<VEC, false, TIO>), dim3(chunks, NB),                  \
-                         dim3(kCdThreads), lds, s, E, inLen, labLen, best, arg, w, d, Uq, PS);   \
+      hipLaunchKernelGGL((cand_rows_kernel<VEC, 0, TIO>), dim3(chunks, NB), dim3(kCdThreads),    \
+                         lds, s, E, inLen, labLen, best, arg, w, d, Uq, PS, ranks);              \
     RNNT_LAUNCH_CHECK("cand_rows_kernel");                                                       \
   } while (0)
 #define RNNT_CAND_PASSES(VEC)                                                                    \
   do {                                                                                           \
     RNNT_TRY(allow_lds(cand_lists_p_kernel<VEC, TIO>, lds));                                     \
-    RNNT_TRY(allow_lds(cand_rows_kernel<VEC, true, TIO>, lds));                                  \
-    RNNT_TRY(allow_lds(cand_rows_kernel<VEC, false, TIO>, lds));                                        \
+    RNNT_TRY(allow_lds(cand_rows_kernel<VEC, kCdAheadShort, TIO>, lds));                         \
+    RNNT_TRY(allow_lds(cand_rows_kernel<VEC, kCdAheadLong, TIO>, lds));                          \
+    RNNT_TRY(allow_lds(cand_rows_kernel<VEC, 0, TIO>, lds));                                        \
     RNNT_CAND_PASS(VEC, sample, nsample);                                                        \
     hipLaunchKernelGGL(cand_decide_kernel, dim3(1), dim3(1), 0, s, w.stats, force ? 1 : 0);      \
     RNNT_LAUNCH_CHECK("cand_decide_kernel");                                                     \
@@ -837,7 +870,7 @@ int cells_any(const TIO* E, const TIO* P, const int* inLen, const int* labLen, f
               int* arg, const Dims& d, void* scratch, hipStream_t s) {
   CandScratch w;
   carve(scratch, d, &w);
-  const dim3 grid(((d.T + kCdTileT - 1) / kCdTileT) * kCdCellShare,
+  const dim3 grid(((d.T + kCdTileT - 1) / kCdTileT) * (kCdCellShare / 4),
                   (d.U + kCdTileU - 1) / kCdTileU, d.B);
   hipLaunchKernelGGL((cand_cells_kernel<TIO>), grid, dim3(256), 0, s, E, P, best, arg,
                      w.tile_fail, w.tile_cells, w.stats, d);
@@ -858,13 +891,16 @@ bool maxplus_lists_possible(const Dims& d) {
   return true;
 }
 
-// Where the list path is tried without being asked for: a row long enough that walking two
-// lists of a few hundred columns can beat looking at all of them (measured on normally
-// distributed scores: from about 6000 columns), and short enough that two workgroups' rows and
-// lists fit a compute unit's LDS (with one, nothing covers the staging of a row).  Whether it
-// goes through with it is decided on the scores themselves (cand_decide_kernel).
+// Where the list path is tried without being asked for (measured on normally distributed
+// scores, B = 8 and 32, T = 2000): from about 5000 columns on, walking two lists of a few
+// hundred columns beats looking at all of them, by 20 to 35 %, as long as two workgroups' rows
+// and lists fit a compute unit's LDS (about 17400 columns; with one workgroup nothing covers
+// the staging of a row) and the label axis fills more than one wavefront (at 51 label positions
+// the all-columns kernel has half the work and the two are level).  Whether a call goes through
+// with it is decided on its own scores (cand_decide_kernel).
 bool maxplus_lists_pay(const Dims& d) {
-  return maxplus_lists_possible(d) && d.V >= 8000 && 2 * cand_lds_bytes(d.V) <= 160 * 1024;
+  return maxplus_lists_possible(d) && d.V >= 5000 && d.U > 64 &&
+         2 * cand_lds_bytes(d.V) <= 160 * 1024;
 }
 
 size_t maxplus_lists_bytes(const Dims& d) {
