@@ -819,7 +819,7 @@ int cand_any(const TIO* E, const TIO* P, const int* inLen, const int* labLen, fl
                      w.tile_fail, tiles + 4);
   RNNT_LAUNCH_CHECK("cand_zero_kernel");
   // The sample's utterances first (their lists, their transposed P, one frame in kCdFrames),
-  // then the verdict, then everything else -- whose launches return at once if the verdict is no.
+  // then the decision, then everything else -- whose launches return at once if it is a no.
   const Pass sample{0, 0, d.B > 1 ? d.B / 2 : -1}, rest{1, sample.first, sample.second};
   const int nsample = d.B > 1 ? 2 : 1;
   const int2 ranks = make_int2(list_rank(kCdListE, d.V), list_rank(kCdListP, d.V));
