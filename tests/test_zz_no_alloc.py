@@ -69,3 +69,35 @@ def test_static_decode_refuses_what_does_not_fit_and_runs_nothing():
     assert b"built-in array" in lib.rnnt_hip_last_error()
     torch.cuda.synchronize()
     assert (out == -1).all()
+
+
+def test_static_decode_replays_from_a_captured_graph_also_where_it_builds_its_table_from_lists():
+    # the callers this entry point is for capture it into a HIP graph: every replay (with eager
+    # work and synchronisation in between, and the outputs overwritten) must give the eager
+    # labels.  5120 columns and 70 label positions are inside the range where the table of best
+    # labels comes from candidate lists, whose counters must be cleared inside every replay.
+    import ctypes
+    assert capi.load().rnnt_hip_maxplus_tries_lists(2, 80, 70, 5120) == 1
+    E, P, labels, il, ll = case(2, 80, 69, 5120, seed=4)
+    c = DeviceCase(E, P, labels, il, ll)
+    B, T, U, V = c.dims
+    out = torch.full((B, U - 1), -1, dtype=torch.int32, device="cuda:0")
+
+    def run(stream):
+        capi.call("rnnt_hip_viterbi_decode_static", ptr(c.E), ptr(c.P), ptr(c.il), ptr(c.ll),
+                  ptr(out), B, T, U, V, 0, stream)
+
+    run(None)
+    torch.cuda.synchronize()
+    want = out.clone()
+    assert np.array_equal(want.cpu().numpy(), decode(c, "rnnt_hip_viterbi_decode", 0))
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        run(ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    for _ in range(3):
+        out.fill_(-1)
+        (c.E * 2.0).sum().item()  # eager work of the program's own between replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want)
