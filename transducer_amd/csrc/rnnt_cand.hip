@@ -67,12 +67,6 @@ static_assert(kCdCap % kCdBatch == 0 && kCdDepth % kCdBatch == 0 && kCdBatch % 4
                   kCdSeg % 4 == 0,
               "whole batches, read four entries at a time");
 
-#define RNNT_LAUNCH_CHECK(name)                                                    \
-  do {                                                                             \
-    hipError_t _e = hipGetLastError();                                             \
-    if (_e != hipSuccess) return check_hip(_e, "launch " name, __FILE__, __LINE__); \
-  } while (0)
-
 // order-preserving map of the floats onto the unsigned integers, and back
 __device__ inline unsigned float_key(float x) {
   const unsigned b = __float_as_uint(x);

@@ -1491,12 +1491,6 @@ void carve_planes(void* base, const Dims& d, Planes* p, bool decode_only) {
 }
 
 // ------------------------------------------------------------------ launchers
-#define RNNT_LAUNCH_CHECK(name)                                                    \
-  do {                                                                             \
-    hipError_t _e = hipGetLastError();                                             \
-    if (_e != hipSuccess) return check_hip(_e, "launch " name, __FILE__, __LINE__); \
-  } while (0)
-
 static dim3 tile_grid(const Dims& d) {
   return dim3((d.T + 63) / 64, (d.U + 63) / 64, d.B);
 }

@@ -699,12 +699,6 @@ __global__ __launch_bounds__(256, 2) void pgrads_stream_kernel(
 
 }  // namespace
 
-#define RNNT_LAUNCH_CHECK(name)                                                    \
-  do {                                                                             \
-    hipError_t _e = hipGetLastError();                                             \
-    if (_e != hipSuccess) return check_hip(_e, "launch " name, __FILE__, __LINE__); \
-  } while (0)
-
 bool egrads_one_pass(const Dims& d) { return wplane_up(d.U) <= 16 * kEsMaxS; }
 
 // One pass of the egrads kernels over the frames of `win` (all slices of the label axis), into

@@ -29,6 +29,13 @@ int check_hip(hipError_t e, const char* what, const char* file, int line);
     if (_st != ::rnnt::kOk) return _st; \
   } while (0)
 
+// After a kernel launch inside a function that returns a status: the launch error, if any.
+#define RNNT_LAUNCH_CHECK(name)                                                             \
+  do {                                                                                      \
+    hipError_t _e = hipGetLastError();                                                      \
+    if (_e != hipSuccess) return ::rnnt::check_hip(_e, "launch " name, __FILE__, __LINE__); \
+  } while (0)
+
 // ---------------------------------------------------------------- geometry
 // Problem sizes in the reference's vocabulary: U is the prediction length (longest label + 1).
 struct Dims {

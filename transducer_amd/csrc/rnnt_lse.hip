@@ -504,12 +504,6 @@ __global__ __launch_bounds__(64 * kWaves, kWaves / 2) void lse_stream_kernel(
 
 }  // namespace
 
-#define RNNT_LAUNCH_CHECK(name)                                                    \
-  do {                                                                             \
-    hipError_t _e = hipGetLastError();                                             \
-    if (_e != hipSuccess) return check_hip(_e, "launch " name, __FILE__, __LINE__); \
-  } while (0)
-
 template <typename TIO>
 static bool lse_stream_ok(const TIO* E, const Dims& d) {
   (void)E;

@@ -163,12 +163,6 @@ __global__ __launch_bounds__(256) void wplanes_kernel(const float* __restrict__ 
 
 }  // namespace
 
-#define RNNT_LAUNCH_CHECK(name)                                                    \
-  do {                                                                             \
-    hipError_t _e = hipGetLastError();                                             \
-    if (_e != hipSuccess) return check_hip(_e, "launch " name, __FILE__, __LINE__); \
-  } while (0)
-
 template <typename TIO>
 static int rowmax_any(const TIO* X, float* rowmax, long rows, int V, int rows_per_item,
                       const int* lengths, int extra, hipStream_t s) {
