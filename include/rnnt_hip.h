@@ -205,7 +205,7 @@ int rnnt_hip_set_spin_limit(int trips);
  *      the cells first and goes back to every column if too many of them fail the bound
  *      (scores with a hard upper edge, such as uniform ones, do);
  *   1: over every column always;
- *   2: lists wherever a row fits a compute unit's LDS, without the sample (for tests).
+ *   2: lists for every vocabulary of up to 17408 entries, without the sample (for tests).
  * The labels returned are the same in every mode; the setting is process-wide.  No counterpart
  * in the reference. */
 int rnnt_hip_set_maxplus_mode(int mode);

@@ -76,8 +76,9 @@ def lengths(rng, B, T, U):
 SHAPES = [(2, 9, 5, 12, 0), (1, 3, 2, 5, 4), (2, 17, 7, 100, 3), (1, 40, 70, 130, 0),
           (2, 33, 101, 1000, 999), (1, 20, 130, 515, 7), (2, 21, 9, 4096, 0),
           (1, 35, 66, 10000, 0), (1, 19, 4, 10001, 10000), (1, 5, 3, 4, 1),
-          (1, 6, 3, 20000, 0),   # a row past 64 KB of LDS
-          (1, 3, 2, 36000, 5),   # the longest row the list path takes (156 KB of LDS)
+          (1, 6, 3, 16000, 0),   # a row past 64 KB of LDS
+          (1, 3, 2, 17408, 5),   # the longest row the list path takes
+          (1, 3, 2, 17409, 5),   # one column more: every column (the mode setting cannot force lists)
           (2, 9, 300, 700, 3)]   # three blocks of 128 label positions
 
 

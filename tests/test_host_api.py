@@ -270,7 +270,8 @@ def test_maxplus_mode_setter_and_query():
         assert lib.rnnt_hip_maxplus_tries_lists(32, 2000, 101, 10000) == 0
         capi.call("rnnt_hip_set_maxplus_mode", 2)
         assert lib.rnnt_hip_maxplus_tries_lists(2, 10, 5, 64) == 1
-        assert lib.rnnt_hip_maxplus_tries_lists(2, 10, 5, 50000) == 0  # a row past a CU's LDS
+        assert lib.rnnt_hip_maxplus_tries_lists(2, 10, 5, 17408) == 1
+        assert lib.rnnt_hip_maxplus_tries_lists(2, 10, 5, 17409) == 0  # a row longer than a wavefront keeps
         capi.call("rnnt_hip_set_maxplus_mode", 0)
         assert lib.rnnt_hip_maxplus_tries_lists(32, 2000, 101, 10000) == 1
         assert lib.rnnt_hip_maxplus_tries_lists(32, 2000, 101, 2000) == 0

@@ -31,7 +31,8 @@
 // (230 and 75 of 10000; the square root keeps the share of cells that fail the test level as
 // the vocabulary grows; an entry of P's lists costs twice the bytes of one of E's, hence the
 // shorter lists there; about one cell in 800 then fails the test at V = 10000, and each of
-// those costs the 80 KB of its two rows once more).  A constant or heavily tied row gets an empty list instead of a full one.
+// those costs the 80 KB of its two rows once more).  A constant or heavily tied row gets an
+// empty list instead of a full one.
 #include <hip/hip_runtime.h>
 
 #include <cmath>
@@ -50,11 +51,10 @@ constexpr int kCdSeg = kCdCap + 16;  // a quarter's slots: two batches of paddin
 constexpr int kCdDepth = 384;    // entries of a stored list of P
 constexpr int kCdStored = kCdDepth + 16;  // with two batches of padding behind a full list
 constexpr float kCdListE = 2.31f;  // list lengths the ranks are derived from, in units of sqrt(V): rows of E
-constexpr float kCdListP = 0.88f;  // ... rows of P (their threshold is the largest of four wavefronts' values,
-                                   // so their lists come out a fifth shorter than that)
+constexpr float kCdListP = 0.88f;  // ... rows of P (their one threshold per row is the largest of four
+                                   // wavefronts' values: the lists come out a fifth shorter than that)
 constexpr int kCdBisect = 16;    // halvings of the key interval
 constexpr int kCdFrames = 16;    // frames per workgroup of cand_rows_kernel
-constexpr int kCdPre = 12;       // 16-byte pieces of a row a thread has in flight while staging
 constexpr int kCdAheadShort = 10;  // 16-byte pieces of the next row a thread holds while a row is
 constexpr int kCdAheadLong = 17;   // evaluated: rows of up to 10240 / 17408 columns
 constexpr int kCdBatch = 8;      // candidates per batch (two batches in flight)
@@ -103,118 +103,19 @@ __host__ inline size_t cand_lds_bytes(int V) {
   return sizeof(float) * (size_t)padded_row(V) + sizeof(RowLists);
 }
 
-// kVec: a piece lies inside the row or past it as a whole
-template <bool kVec>
-__device__ inline float store_piece(float* row, int v, float4 y, int V) {
-  if (kVec) {
-    if (v >= V) y = make_float4(kNegInf, kNegInf, kNegInf, kNegInf);
-  } else {
-    y.x = v < V ? y.x : kNegInf;
-    y.y = v + 1 < V ? y.y : kNegInf;
-    y.z = v + 2 < V ? y.z : kNegInf;
-    y.w = v + 3 < V ? y.w : kNegInf;
-  }
-  *reinterpret_cast<float4*>(row + v) = y;
-  return fmaxf(fmaxf(y.x, y.y), fmaxf(y.z, y.w));
-}
-
-// One row of V scores -> LDS copy (blank and padding at -inf), threshold, list.  All threads
-// call it; on return (after a barrier) row and L->idx/val/off/n/bad are complete and every
-// thread holds the threshold.  `pitch`: bytes between two columns' rows of the transposed P
-// (what L->off is counted in).
-// The threshold: every thread keeps the maximum of its own share of the row (about V/256
-// interleaved elements); each wavefront finds, by halving the interval of float keys, a value
-// with at most `rank` of its 64 maxima above it, and the row's threshold is the largest of the
-// four.  For values drawn independently that puts about 1.4 % of a 10000-column row on the
-// list, whatever their scale; a constant or heavily tied row gets an empty list, not a full one.
-template <bool kVec, typename TIO>
-__device__ inline float stage_row(const TIO* __restrict__ src, int V, int blank, unsigned pitch,
-                                  int rank, float* row, RowLists* L) {
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int Vp = padded_row(V);
-  float m = kNegInf;
-  for (int v0 = 0; v0 < Vp; v0 += 4 * kCdThreads * kCdPre) {
-    float4 x[kCdPre];
-#pragma unroll
-    for (int j = 0; j < kCdPre; ++j) {
-      const int v = v0 + 4 * (tid + kCdThreads * j);
-      if (v < Vp) {
-        if (kVec) x[j] = load4(src + min(v, V - 4));
-        else x[j] = load4_any(src, min(v, V - 1), V);
-      }
-    }
-#pragma unroll
-    for (int j = 0; j < kCdPre; ++j) {
-      const int v = v0 + 4 * (tid + kCdThreads * j);
-      if (v < Vp) m = fmaxf(m, store_piece<kVec>(row, v, x[j], V));
-    }
-  }
-  // the blank never wins: the thread that wrote its piece takes it out (its own maximum may
-  // still count it, which only moves the threshold)
-  if (tid == ((blank >> 2) & (kCdThreads - 1))) row[blank] = kNegInf;
-
-  const unsigned key = float_key(m);
-  unsigned lo = 0u, hi = 0xffffffffu;  // at most `rank` keys of the wavefront lie above hi
-  for (int it = 0; it < kCdBisect; ++it) {
-    const unsigned mid = lo + ((hi - lo) >> 1);
-    if (__builtin_popcountll(__ballot(key > mid)) > rank) lo = mid; else hi = mid;
-  }
-  if (lane == 0) L->tau[wave] = key_float(hi);
-  if (tid == 0) L->bad[0] = 0;
-  __syncthreads();
-  const float tau = fmaxf(fmaxf(L->tau[0], L->tau[1]), fmaxf(L->tau[2], L->tau[3]));
-
-  // this wavefront's quarter of the row, 64 columns at a time in column order
-  const int quarter = Vp >> 2, c0 = wave * quarter;
-  int* idx = L->idx + wave * kCdSeg;
-  float* val = L->val + wave * kCdSeg;
-  unsigned* off = L->off + wave * kCdSeg;
-  int count = 0;
-  for (int c = 0; c < quarter; c += 64 * 4) {
-    float x[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) x[j] = row[c0 + min(c + 64 * j, quarter - 64) + lane];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const bool hit = (c + 64 * j < quarter) && x[j] > tau;
-      const unsigned long long mask = __ballot(hit);
-      if (mask) {
-        const int pos = count + lanes_below(mask);
-        if (hit && pos < kCdCap) {
-          const int col = c0 + c + 64 * j + lane;
-          idx[pos] = col;
-          val[pos] = x[j];
-          off[pos] = (unsigned)col * pitch;
-        }
-        count += __builtin_popcountll(mask);
-      }
-    }
-  }
-  const int kept = min(count, kCdCap);
-  // fill the last batch, and the two batches a walk may touch beyond it
-  if (lane < ((-kept) & (kCdBatch - 1)) + 2 * kCdBatch) {
-    idx[kept + lane] = 0;
-    val[kept + lane] = kNegInf;
-    off[kept + lane] = 0u;
-  }
-  if (lane == 0) {
-    L->n[wave] = kept;
-    if (count > kCdCap) L->bad[0] = 1;
-  }
-  __syncthreads();
-  return tau;
-}
-
-// The same for a row that is requested one frame ahead (cand_rows_kernel, rows of at most
-// 256 kPieces columns per wavefront): each wavefront owns one quarter of the row from the load
-// on, keeps it in registers while the previous frame is evaluated, and builds its part of the
-// list from those registers with its own threshold (any threshold is valid per column; the
-// row's bound is the largest of the four).  No wavefront waits for another before the one
-// barrier that ends the staging.
+// One row of V scores -> LDS copy (blank and padding at -inf), thresholds, list.  Each wavefront
+// owns one quarter of the row (at most 256 kPieces columns) from the load on: fetch_quarter
+// requests it into registers -- in cand_rows_kernel one frame ahead, while the previous frame is
+// evaluated -- and commit_quarter writes it to LDS and lists the wavefront's columns from those
+// registers with the wavefront's own threshold.  Any threshold is valid per column; the row's
+// bound is the largest of the four (L->tau).  No wavefront waits for another before the one
+// barrier the caller places behind commit_quarter.
+// The threshold: every lane keeps the maximum of its own share of the quarter (interleaved
+// pieces of four columns); the wavefront finds, by halving the interval of float keys, a value
+// with at most `rank` of its 64 maxima above it.
 template <int kPieces>
 struct QuarterRegs {
-  float4 x[kPieces > 0 ? kPieces : 1];
+  float4 x[kPieces];
 };
 template <bool kVec, int kPieces, typename TIO>
 __device__ inline void fetch_quarter(const TIO* __restrict__ src, int V, QuarterRegs<kPieces>& r) {
@@ -231,9 +132,11 @@ __device__ inline void fetch_quarter(const TIO* __restrict__ src, int V, Quarter
   }
 }
 
+// Writes the quarter to LDS (blank and padding at -inf; the registers keep the padded values) and
+// returns the wavefront's threshold.
 template <bool kVec, int kPieces>
-__device__ inline void commit_quarter(QuarterRegs<kPieces>& r, int V, int blank, unsigned pitch, int rank,
-                                      int parity, float* row, RowLists* L) {
+__device__ inline float quarter_threshold(QuarterRegs<kPieces>& r, int V, int blank, int rank,
+                                         float* row) {
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int quarter = padded_row(V) >> 2, c0 = wave * quarter;
@@ -267,8 +170,18 @@ __device__ inline void commit_quarter(QuarterRegs<kPieces>& r, int V, int blank,
     const unsigned mid = lo + ((hi - lo) >> 1);
     if (__builtin_popcountll(__ballot(key > mid)) > rank) lo = mid; else hi = mid;
   }
-  const float tau = key_float(hi);
+  return key_float(hi);
+}
 
+// Lists the wavefront's columns above `tau`, in column order, from the registers; leaves the
+// count and `tau` (for the row's bound) in L.
+template <int kPieces>
+__device__ inline void quarter_list(const QuarterRegs<kPieces>& r, float tau, int V, int blank,
+                                    unsigned pitch, int parity, RowLists* L) {
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int quarter = padded_row(V) >> 2, c0 = wave * quarter;
+  const int blank_wave = blank / quarter;  // uniform
   int* idx = L->idx + wave * kCdSeg;
   float* val = L->val + wave * kCdSeg;
   unsigned* off = L->off + wave * kCdSeg;
@@ -317,6 +230,14 @@ __device__ inline void commit_quarter(QuarterRegs<kPieces>& r, int V, int blank,
   }
 }
 
+// Both at once, with the wavefront's own threshold (rows of E).
+template <bool kVec, int kPieces>
+__device__ inline void commit_quarter(QuarterRegs<kPieces>& r, int V, int blank, unsigned pitch,
+                                      int rank, int parity, float* row, RowLists* L) {
+  const float tau = quarter_threshold<kVec, kPieces>(r, V, blank, rank, row);
+  quarter_list<kPieces>(r, tau, V, blank, pitch, parity, L);
+}
+
 // ------------------------------------------------------------------ lists of P
 // Scratch of the list path (Uq = U rounded up to 4, Ub64 = U rounded up to 64)
 struct CandScratch {
@@ -359,7 +280,20 @@ __global__ __launch_bounds__(kCdThreads) void cand_lists_p_kernel(const TIO* __r
     return;
   }
   const TIO* src = P + ((size_t)b * d.U + u) * d.V;
-  const float tau = stage_row<kVec>(src, d.V, d.blank, 0u, ranks.y, row, L);
+  QuarterRegs<kCdAheadLong> regs;
+  fetch_quarter<kVec, kCdAheadLong>(src, d.V, regs);
+  if (tid == 0) L->bad[0] = 0;
+  __syncthreads();
+  // one threshold for the whole row, the largest of the four wavefronts' (their own would put a
+  // fifth more columns on the list for the same bound; for a row of E that is the price of not
+  // waiting for the other wavefronts, here the list is built once and walked for every frame)
+  const float tau_own = quarter_threshold<kVec, kCdAheadLong>(regs, d.V, d.blank, ranks.y, row);
+  if ((tid & 63) == 0) L->tau[tid >> 6] = tau_own;
+  __syncthreads();
+  const float tau = fmaxf(fmaxf(L->tau[0], L->tau[1]), fmaxf(L->tau[2], L->tau[3]));
+  __syncthreads();  // (quarter_list writes L->tau again)
+  quarter_list<kCdAheadLong>(regs, tau, d.V, d.blank, 0u, 0, L);
+  __syncthreads();
   const int c1 = L->n[0], c2 = c1 + L->n[1], c3 = c2 + L->n[2], total = c3 + L->n[3];
   const bool bad = L->bad[0] != 0 || total > kCdDepth;
   for (int k = tid; k < kCdStored; k += kCdThreads) {
@@ -412,8 +346,7 @@ __global__ __launch_bounds__(256) void cand_transpose_p_kernel(const TIO* __rest
 // lower column).
 // While a frame is evaluated, one load per cache line of the next frame's row brings that row
 // into L2, so that staging it waits for L2 and not for HBM.
-// kPieces: 16-byte pieces per thread of the row requested ahead (0: rows too long for that are
-// staged when their turn comes).
+// kPieces: 16-byte pieces per lane of a wavefront's quarter of a row.
 template <bool kVec, int kPieces, typename TIO>
 __global__ __launch_bounds__(kCdThreads) void cand_rows_kernel(const TIO* __restrict__ E,
                                                                const int* __restrict__ inLen,
@@ -449,9 +382,6 @@ __global__ __launch_bounds__(kCdThreads) void cand_rows_kernel(const TIO* __rest
   const unsigned pitch = 4u * (unsigned)Uq;
   const int blocks = (d.U + 63) >> 6;
   const int tiles_t = (d.T + kCdTileT - 1) / kCdTileT, tiles_u = (d.U + kCdTileU - 1) / kCdTileU;
-  const int row_lines = (int)(((size_t)d.V * sizeof(TIO) + 63) >> 6);
-  unsigned touched = 0u;
-
   // what the first block of 128 label positions needs of P's lists is the same for every frame
   const int u_first = 64 * blk + lane;
   const bool first_valid = u_first < Ub;
@@ -461,40 +391,20 @@ __global__ __launch_bounds__(kCdThreads) void cand_rows_kernel(const TIO* __rest
   for (int s = 1; s < 64; s <<= 1) nmax_first = max(nmax_first, __shfl_xor(nmax_first, s, 64));
   nmax_first = __builtin_amdgcn_readfirstlane(nmax_first);
 
-  constexpr bool kAhead = kPieces > 0;
   QuarterRegs<kPieces> ahead;
-  if (kAhead) {
-    if (tid == 0) L->bad[0] = L->bad[1] = 0;
-    fetch_quarter<kVec, kPieces>(Eb + (size_t)t_lo * d.V, d.V, ahead);
-    __syncthreads();
-  }
+  if (tid == 0) L->bad[0] = L->bad[1] = 0;
+  fetch_quarter<kVec, kPieces>(Eb + (size_t)t_lo * d.V, d.V, ahead);
+  __syncthreads();
   int parity = 0;
   for (int t = t_lo; t < t_hi; ++t) {
-    float tau;
-    bool bad;
-    unsigned warm[4] = {0u, 0u, 0u, 0u};
-    if (kAhead) {
-      // this frame's row is in registers; the next one's is requested before the evaluation
-      const int fp = (t - t_lo) & 1;
-      commit_quarter<kVec, kPieces>(ahead, d.V, d.blank, pitch, ranks.x, fp, row, L);
-      if (t + 1 < t_hi) fetch_quarter<kVec, kPieces>(Eb + (size_t)(t + 1) * d.V, d.V, ahead);
-      __syncthreads();
-      if (tid == 0) L->bad[fp ^ 1] = 0;  // the next frame's flag: nobody sets it before the hand-over barrier
-      tau = fmaxf(fmaxf(L->tau[0], L->tau[1]), fmaxf(L->tau[2], L->tau[3]));
-      bad = L->bad[fp] != 0;
-    } else {
-      tau = stage_row<kVec>(Eb + (size_t)t * d.V, d.V, d.blank, pitch, ranks.x, row, L);
-      if (t + 1 < t_hi) {
-        const char* next = reinterpret_cast<const char*>(Eb + (size_t)(t + 1) * d.V);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int line = tid + kCdThreads * i;
-          if (line < row_lines)
-            warm[i] = *reinterpret_cast<const unsigned short*>(next + ((size_t)line << 6));
-        }
-      }
-      bad = L->bad[0] != 0;
-    }
+    // this frame's row is in registers; the next one's is requested before the evaluation
+    const int fp = (t - t_lo) & 1;
+    commit_quarter<kVec, kPieces>(ahead, d.V, d.blank, pitch, ranks.x, fp, row, L);
+    if (t + 1 < t_hi) fetch_quarter<kVec, kPieces>(Eb + (size_t)(t + 1) * d.V, d.V, ahead);
+    __syncthreads();
+    if (tid == 0) L->bad[fp ^ 1] = 0;  // the next frame's flag: nobody sets it before the hand-over barrier
+    const float tau = fmaxf(fmaxf(L->tau[0], L->tau[1]), fmaxf(L->tau[2], L->tau[3]));
+    const bool bad = L->bad[fp] != 0;
     for (int ub = 0; ub < Ub; ub += 2 * 64, parity ^= 1) {
       const int u = ub + 64 * blk + lane;
       const bool live = ub + 64 * blk < Ub;  // uniform: some of this wavefront's positions exist
@@ -664,12 +574,9 @@ __global__ __launch_bounds__(kCdThreads) void cand_rows_kernel(const TIO* __rest
         }
       }
     }
-    touched ^= warm[0] ^ warm[1] ^ warm[2] ^ warm[3];
     // (no barrier here: after the hand-over barrier nobody reads the row or the lists again,
     // and the hand-over arrays are next written two barriers further on)
   }
-  // keeps the warming loads alive: 16-bit values never add up to this
-  if (touched == 0xffffffffu) best[0] = 0.0f;
 }
 
 // ------------------------------------------------------------------ flagged cells, one by one
@@ -832,13 +739,10 @@ int cand_any(const TIO* E, const TIO* P, const int* inLen, const int* labLen, fl
       hipLaunchKernelGGL((cand_rows_kernel<VEC, kCdAheadShort, TIO>), dim3(chunks, NB),          \
                          dim3(kCdThreads), lds, s, E, inLen, labLen, best, arg, w, d, Uq, PS,    \
                          ranks);                                                                 \
-    else if (pieces <= kCdAheadLong)                                                             \
+    else                                                                                         \
       hipLaunchKernelGGL((cand_rows_kernel<VEC, kCdAheadLong, TIO>), dim3(chunks, NB),           \
                          dim3(kCdThreads), lds, s, E, inLen, labLen, best, arg, w, d, Uq, PS,    \
                          ranks);                                                                 \
-    else                                                                                         \
-      hipLaunchKernelGGL((cand_rows_kernel<VEC, 0, TIO>), dim3(chunks, NB), dim3(kCdThreads),    \
-                         lds, s, E, inLen, labLen, best, arg, w, d, Uq, PS, ranks);              \
     RNNT_LAUNCH_CHECK("cand_rows_kernel");                                                       \
   } while (0)
 #define RNNT_CAND_PASSES(VEC)                                                                    \
@@ -846,7 +750,6 @@ int cand_any(const TIO* E, const TIO* P, const int* inLen, const int* labLen, fl
     RNNT_TRY(allow_lds(cand_lists_p_kernel<VEC, TIO>, lds));                                     \
     RNNT_TRY(allow_lds(cand_rows_kernel<VEC, kCdAheadShort, TIO>, lds));                         \
     RNNT_TRY(allow_lds(cand_rows_kernel<VEC, kCdAheadLong, TIO>, lds));                          \
-    RNNT_TRY(allow_lds(cand_rows_kernel<VEC, 0, TIO>, lds));                                        \
     RNNT_CAND_PASS(VEC, sample, nsample);                                                        \
     hipLaunchKernelGGL(cand_decide_kernel, dim3(1), dim3(1), 0, s, w.stats, force ? 1 : 0);      \
     RNNT_LAUNCH_CHECK("cand_decide_kernel");                                                     \
@@ -876,11 +779,12 @@ int cells_any(const TIO* E, const TIO* P, const int* inLen, const int* labLen, f
 
 int maxplus_tile_limit() { return kCdTileLimit; }
 
-// Whether the list path can take this shape at all: the row and its lists fit the LDS of a
-// compute unit, and an offset into one utterance's transposed P fits 31 bits.
+// Whether the list path can take this shape at all: a quarter of a row fits the registers a
+// wavefront keeps for it (which also keeps a row and its lists inside a compute unit's LDS), and
+// an offset into one utterance's transposed P fits 31 bits.
 bool maxplus_lists_possible(const Dims& d) {
   if (d.B == 0 || d.T == 0 || d.U == 0 || d.V < 4) return false;
-  if (cand_lds_bytes(d.V) > 160 * 1024 - 1024) return false;
+  if (padded_row(d.V) > 4 * 256 * kCdAheadLong) return false;
   if ((size_t)d.V * cand_uq(d) >= ((size_t)1 << 29)) return false;
   return true;
 }
