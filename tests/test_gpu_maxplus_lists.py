@@ -79,7 +79,9 @@ SHAPES = [(2, 9, 5, 12, 0), (1, 3, 2, 5, 4), (2, 17, 7, 100, 3), (1, 40, 70, 130
           (1, 6, 3, 16000, 0),   # a row past 64 KB of LDS
           (1, 3, 2, 17408, 5),   # the longest row the list path takes
           (1, 3, 2, 17409, 5),   # one column more: every column (the mode setting cannot force lists)
-          (2, 9, 300, 700, 3)]   # three blocks of 128 label positions
+          (2, 9, 300, 700, 3),   # three blocks of 128 label positions
+          (8, 40, 9, 300, 2),    # utterance counts that are multiples of eight: workgroups are dealt
+          (16, 35, 70, 260, 0)]  # out so that each of the eight dies works through utterances of its own
 
 
 @pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "B%d_T%d_U%d_V%d_blank%d" % s)

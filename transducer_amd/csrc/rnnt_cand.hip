@@ -117,6 +117,15 @@ template <int kPieces>
 struct QuarterRegs {
   float4 x[kPieces];
 };
+// A row of E is read once: the load says so, and L2 keeps its lines for the transposed P.
+__device__ inline float4 load4_once(const float* p) {
+  typedef float vec4 __attribute__((ext_vector_type(4)));
+  const vec4 x = __builtin_nontemporal_load(reinterpret_cast<const vec4*>(p));
+  return make_float4(x.x, x.y, x.z, x.w);
+}
+template <typename T16>
+__device__ inline float4 load4_once(const T16* p) { return load4(p); }
+
 template <bool kVec, int kPieces, typename TIO>
 __device__ inline void fetch_quarter(const TIO* __restrict__ src, int V, QuarterRegs<kPieces>& r) {
   const int lane = threadIdx.x & 63;
@@ -126,7 +135,7 @@ __device__ inline void fetch_quarter(const TIO* __restrict__ src, int V, Quarter
   for (int i = 0; i < kPieces; ++i) {
     const int c = 256 * i + 4 * lane, v = c0 + c;
     if (c < quarter) {
-      if (kVec) r.x[i] = load4(src + min(v, V - 4));
+      if (kVec) r.x[i] = load4_once(src + min(v, V - 4));
       else r.x[i] = load4_any(src, min(v, V - 1), V);
     }
   }
@@ -360,11 +369,16 @@ __global__ __launch_bounds__(kCdThreads) void cand_rows_kernel(const TIO* __rest
   RowLists* L = reinterpret_cast<RowLists*>(row + padded_row(d.V));
   // The sample: the first frame of every workgroup's run of frames, in the sample's utterances.
   // The rest: every other frame of those, and all frames of the others.
-  int b = blockIdx.y;
+  int b = blockIdx.y, group = blockIdx.x;
   if (ps.phase == 0) b = b == 0 ? ps.first : ps.second;
   else if (w.stats[2] == 0) return;
+  else if ((gridDim.y & 7) == 0) {
+    const unsigned lin = blockIdx.x + gridDim.x * blockIdx.y, slot = lin >> 3;
+    b = (int)((lin & 7) + 8 * (slot / gridDim.x));
+    group = (int)(slot % gridDim.x);
+  }
   const bool sampled = b == ps.first || b == ps.second;
-  int t_lo = blockIdx.x * kCdFrames;
+  int t_lo = group * kCdFrames;
   int Tb, Ub;
   utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
   if (t_lo >= Tb || Ub == 0) return;
