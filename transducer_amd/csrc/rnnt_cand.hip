@@ -117,15 +117,6 @@ template <int kPieces>
 struct QuarterRegs {
   float4 x[kPieces];
 };
-// A row of E is read once: the load says so, and L2 keeps its lines for the transposed P.
-__device__ inline float4 load4_once(const float* p) {
-  typedef float vec4 __attribute__((ext_vector_type(4)));
-  const vec4 x = __builtin_nontemporal_load(reinterpret_cast<const vec4*>(p));
-  return make_float4(x.x, x.y, x.z, x.w);
-}
-template <typename T16>
-__device__ inline float4 load4_once(const T16* p) { return load4(p); }
-
 template <bool kVec, int kPieces, typename TIO>
 __device__ inline void fetch_quarter(const TIO* __restrict__ src, int V, QuarterRegs<kPieces>& r) {
   const int lane = threadIdx.x & 63;
@@ -135,7 +126,7 @@ __device__ inline void fetch_quarter(const TIO* __restrict__ src, int V, Quarter
   for (int i = 0; i < kPieces; ++i) {
     const int c = 256 * i + 4 * lane, v = c0 + c;
     if (c < quarter) {
-      if (kVec) r.x[i] = load4_once(src + min(v, V - 4));
+      if (kVec) r.x[i] = load4_once(src + min(v, V - 4));  // a row of E: read once
       else r.x[i] = load4_any(src, min(v, V - 1), V);
     }
   }
@@ -372,10 +363,15 @@ __global__ __launch_bounds__(kCdThreads) void cand_rows_kernel(const TIO* __rest
   int b = blockIdx.y, group = blockIdx.x;
   if (ps.phase == 0) b = b == 0 ? ps.first : ps.second;
   else if (w.stats[2] == 0) return;
-  else if ((gridDim.y & 7) == 0) {
-    const unsigned lin = blockIdx.x + gridDim.x * blockIdx.y, slot = lin >> 3;
-    b = (int)((lin & 7) + 8 * (slot / gridDim.x));
-    group = (int)(slot % gridDim.x);
+  else {
+    // Workgroups are dealt to the eight dies in launch order, one each in turn; die k takes the
+    // k-th eighth of the (utterance, run of frames) pairs, so that at any time its L2 holds the
+    // transposed P of one or two utterances instead of everybody's.
+    const unsigned n = gridDim.x * gridDim.y, lin = blockIdx.x + gridDim.x * blockIdx.y;
+    const unsigned k = lin & 7, slot = lin >> 3, share = n >> 3, extra = n & 7;
+    const unsigned pair = k * share + min(k, extra) + slot;
+    b = (int)(pair / gridDim.x);
+    group = (int)(pair % gridDim.x);
   }
   const bool sampled = b == ps.first || b == ps.second;
   int t_lo = group * kCdFrames;

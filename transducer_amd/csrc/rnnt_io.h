@@ -40,18 +40,34 @@ __device__ inline void stf(bf16_t* p, float v) { p->bits = float_to_bf16(v); }
 
 // Four consecutive, naturally aligned elements (16 bytes of fp32, 8 of bf16).
 __device__ inline float4 load4(const float* p) { return *reinterpret_cast<const float4*>(p); }
-__device__ inline float4 load4(const bf16_t* p) {
-  const uint2 w = *reinterpret_cast<const uint2*>(p);
+__device__ inline float4 widen4(uint2 w, const bf16_t*) {
   return make_float4(__uint_as_float(w.x << 16), __uint_as_float(w.x & 0xffff0000u),
                      __uint_as_float(w.y << 16), __uint_as_float(w.y & 0xffff0000u));
 }
-
-__device__ inline float4 load4(const f16_t* p) {
-  const uint2 w = *reinterpret_cast<const uint2*>(p);
+__device__ inline float4 widen4(uint2 w, const f16_t*) {
   return make_float4(f16_to_float((unsigned short)(w.x & 0xffffu)),
                      f16_to_float((unsigned short)(w.x >> 16)),
                      f16_to_float((unsigned short)(w.y & 0xffffu)),
                      f16_to_float((unsigned short)(w.y >> 16)));
+}
+__device__ inline float4 load4(const bf16_t* p) {
+  return widen4(*reinterpret_cast<const uint2*>(p), p);
+}
+__device__ inline float4 load4(const f16_t* p) {
+  return widen4(*reinterpret_cast<const uint2*>(p), p);
+}
+// The same for data that a kernel reads once: the load says so, and L2 keeps its lines for
+// what the kernel's workgroups share.
+__device__ inline float4 load4_once(const float* p) {
+  typedef float vec4 __attribute__((ext_vector_type(4)));
+  const vec4 x = __builtin_nontemporal_load(reinterpret_cast<const vec4*>(p));
+  return make_float4(x.x, x.y, x.z, x.w);
+}
+template <typename T16>
+__device__ inline float4 load4_once(const T16* p) {
+  typedef unsigned vec2 __attribute__((ext_vector_type(2)));
+  const vec2 w = __builtin_nontemporal_load(reinterpret_cast<const vec2*>(p));
+  return widen4(make_uint2(w.x, w.y), p);
 }
 
 // Wide loads at the element type's own alignment (global memory serves them at any such
