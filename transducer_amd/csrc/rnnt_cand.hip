@@ -117,8 +117,15 @@ template <int kPieces>
 struct QuarterRegs {
   float4 x[kPieces];
 };
+// A quarter as its loads return it (16-bit scores stay 16-bit until the row is committed: a
+// conversion next to the load would wait for it there and then).
+template <int kPieces, typename TIO>
+struct QuarterBits {
+  decltype(load4_bits_once(static_cast<const TIO*>(nullptr))) x[kPieces];
+};
 template <bool kVec, int kPieces, typename TIO>
-__device__ inline void fetch_quarter(const TIO* __restrict__ src, int V, QuarterRegs<kPieces>& r) {
+__device__ inline void fetch_quarter(const TIO* __restrict__ src, int V,
+                                     QuarterBits<kPieces, TIO>& r) {
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int quarter = padded_row(V) >> 2, c0 = wave * quarter;
@@ -126,16 +133,17 @@ __device__ inline void fetch_quarter(const TIO* __restrict__ src, int V, Quarter
   for (int i = 0; i < kPieces; ++i) {
     const int c = 256 * i + 4 * lane, v = c0 + c;
     if (c < quarter) {
-      if (kVec) r.x[i] = load4_once(src + min(v, V - 4));  // a row of E: read once
-      else r.x[i] = load4_any(src, min(v, V - 1), V);
+      if (kVec) r.x[i] = load4_bits_once(src + min(v, V - 4));
+      else r.x[i] = load4_any_bits(src, min(v, V - 1), V);
     }
   }
 }
 
-// Writes the quarter to LDS (blank and padding at -inf; the registers keep the padded values) and
-// returns the wavefront's threshold.
-template <bool kVec, int kPieces>
-__device__ inline float quarter_threshold(QuarterRegs<kPieces>& r, int V, int blank, int rank,
+// Writes the quarter to LDS (blank and padding at -inf; `r` keeps the padded values) and returns
+// the wavefront's threshold.
+template <bool kVec, int kPieces, typename TIO>
+__device__ inline float quarter_threshold(const QuarterBits<kPieces, TIO>& in,
+                                         QuarterRegs<kPieces>& r, int V, int blank, int rank,
                                          float* row) {
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -147,7 +155,7 @@ __device__ inline float quarter_threshold(QuarterRegs<kPieces>& r, int V, int bl
     const int c = 256 * i + 4 * lane, v = c0 + c;
     float4 y = none;
     if (c < quarter) {
-      y = r.x[i];
+      y = widen4(in.x[i], static_cast<const TIO*>(nullptr));
       if (kVec) {
         if (v >= V) y = none;
       } else {
@@ -231,10 +239,12 @@ __device__ inline void quarter_list(const QuarterRegs<kPieces>& r, float tau, in
 }
 
 // Both at once, with the wavefront's own threshold (rows of E).
-template <bool kVec, int kPieces>
-__device__ inline void commit_quarter(QuarterRegs<kPieces>& r, int V, int blank, unsigned pitch,
-                                      int rank, int parity, float* row, RowLists* L) {
-  const float tau = quarter_threshold<kVec, kPieces>(r, V, blank, rank, row);
+template <bool kVec, int kPieces, typename TIO>
+__device__ inline void commit_quarter(const QuarterBits<kPieces, TIO>& in, int V, int blank,
+                                      unsigned pitch, int rank, int parity, float* row,
+                                      RowLists* L) {
+  QuarterRegs<kPieces> r;
+  const float tau = quarter_threshold<kVec, kPieces>(in, r, V, blank, rank, row);
   quarter_list<kPieces>(r, tau, V, blank, pitch, parity, L);
 }
 
@@ -280,14 +290,15 @@ __global__ __launch_bounds__(kCdThreads) void cand_lists_p_kernel(const TIO* __r
     return;
   }
   const TIO* src = P + ((size_t)b * d.U + u) * d.V;
+  QuarterBits<kCdAheadLong, TIO> bits;
   QuarterRegs<kCdAheadLong> regs;
-  fetch_quarter<kVec, kCdAheadLong>(src, d.V, regs);
+  fetch_quarter<kVec, kCdAheadLong>(src, d.V, bits);
   if (tid == 0) L->bad[0] = 0;
   __syncthreads();
   // one threshold for the whole row, the largest of the four wavefronts' (their own would put a
   // fifth more columns on the list for the same bound; for a row of E that is the price of not
   // waiting for the other wavefronts, here the list is built once and walked for every frame)
-  const float tau_own = quarter_threshold<kVec, kCdAheadLong>(regs, d.V, d.blank, ranks.y, row);
+  const float tau_own = quarter_threshold<kVec, kCdAheadLong>(bits, regs, d.V, d.blank, ranks.y, row);
   if ((tid & 63) == 0) L->tau[tid >> 6] = tau_own;
   __syncthreads();
   const float tau = fmaxf(fmaxf(L->tau[0], L->tau[1]), fmaxf(L->tau[2], L->tau[3]));
@@ -401,7 +412,7 @@ __global__ __launch_bounds__(kCdThreads) void cand_rows_kernel(const TIO* __rest
   for (int s = 1; s < 64; s <<= 1) nmax_first = max(nmax_first, __shfl_xor(nmax_first, s, 64));
   nmax_first = __builtin_amdgcn_readfirstlane(nmax_first);
 
-  QuarterRegs<kPieces> ahead;
+  QuarterBits<kPieces, TIO> ahead;
   if (tid == 0) L->bad[0] = L->bad[1] = 0;
   fetch_quarter<kVec, kPieces>(Eb + (size_t)t_lo * d.V, d.V, ahead);
   __syncthreads();

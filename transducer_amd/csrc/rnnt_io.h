@@ -56,18 +56,20 @@ __device__ inline float4 load4(const bf16_t* p) {
 __device__ inline float4 load4(const f16_t* p) {
   return widen4(*reinterpret_cast<const uint2*>(p), p);
 }
-// The same for data that a kernel reads once: the load says so, and L2 keeps its lines for
-// what the kernel's workgroups share.
-__device__ inline float4 load4_once(const float* p) {
+__device__ inline float4 widen4(float4 x, const float*) { return x; }
+// The same four elements as the load returns them (widen4 makes floats of them), for data that
+// a kernel reads once: the load says so, and L2 keeps its lines for what the kernel's
+// workgroups share.  Keeping the bits as they are leaves the load's wait to their first use.
+__device__ inline float4 load4_bits_once(const float* p) {
   typedef float vec4 __attribute__((ext_vector_type(4)));
   const vec4 x = __builtin_nontemporal_load(reinterpret_cast<const vec4*>(p));
   return make_float4(x.x, x.y, x.z, x.w);
 }
 template <typename T16>
-__device__ inline float4 load4_once(const T16* p) {
+__device__ inline uint2 load4_bits_once(const T16* p) {
   typedef unsigned vec2 __attribute__((ext_vector_type(2)));
   const vec2 w = __builtin_nontemporal_load(reinterpret_cast<const vec2*>(p));
-  return widen4(make_uint2(w.x, w.y), p);
+  return make_uint2(w.x, w.y);
 }
 
 // Wide loads at the element type's own alignment (global memory serves them at any such
@@ -96,17 +98,14 @@ __device__ inline uint2 load4_any_bits(const T16* row, int v, int V) {
       (unsigned)row[min(v, V - 1)].bits | ((unsigned)row[min(v + 1, V - 1)].bits << 16),
       (unsigned)row[min(v + 2, V - 1)].bits | ((unsigned)row[min(v + 3, V - 1)].bits << 16));
 }
+__device__ inline float4 load4_any_bits(const float* row, int v, int V) {
+  return load4_any(row, v, V);
+}
 __device__ inline float4 load4_any(const bf16_t* row, int v, int V) {
-  const uint2 w = load4_any_bits(row, v, V);
-  return make_float4(__uint_as_float(w.x << 16), __uint_as_float(w.x & 0xffff0000u),
-                     __uint_as_float(w.y << 16), __uint_as_float(w.y & 0xffff0000u));
+  return widen4(load4_any_bits(row, v, V), row);
 }
 __device__ inline float4 load4_any(const f16_t* row, int v, int V) {
-  const uint2 w = load4_any_bits(row, v, V);
-  return make_float4(f16_to_float((unsigned short)(w.x & 0xffffu)),
-                     f16_to_float((unsigned short)(w.x >> 16)),
-                     f16_to_float((unsigned short)(w.y & 0xffffu)),
-                     f16_to_float((unsigned short)(w.y >> 16)));
+  return widen4(load4_any_bits(row, v, V), row);
 }
 
 // Eight consecutive elements of a row as they sit in registers after the load.
