@@ -198,8 +198,9 @@ int rnnt_hip_set_spin_limit(int trips);
 /* How the best-path calls find best[t,u] = max over v != blank of E[t,v] + P[u,v] and its
  * lowest index (transducer/transducer_cpu.cpp:158-171; the reference's device kernel scans every
  * column per cell, transducer/transducer_cuda.cu:178-207).
- *   0 (default): over every column, except for vocabularies of 5000 to about 17400 entries with
- *      more than 64 label positions: there each frame and each label position first gets a short list of its largest scores,
+ *   0 (default): over every column, except for vocabularies of 3000 to about 17400 entries with
+ *      U x V of 250000 or more (say 33 label positions at 10000 entries, 101 at 3000): there
+ *      each frame and each label position first gets a short list of its largest scores,
  *      a cell is settled from the two lists where a bound proves that no other column can win,
  *      and the remaining cells are evaluated over every column; the call looks at a sample of
  *      the cells first and goes back to every column if too many of them fail the bound

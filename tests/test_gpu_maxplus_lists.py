@@ -210,28 +210,30 @@ def test_overflowing_lists_fall_back():
 
 def test_many_failing_cells_in_a_tile_and_few():
     # utterance 0, quantised scores: the test fails for most cells and the all-columns kernel
-    # redoes whole tiles.  Utterance 1: one quantised row of P, so one label position fails in
-    # every frame: 128 cells in the first tile of frames (redone as a tile), 3 in the second
-    # (redone cell by cell)
+    # redoes whole tiles.  Utterance 1: two quantised rows of P, so two label positions fail in
+    # every frame: 256 cells in the first tile of frames (more than a tile's list of flagged
+    # cells holds: redone as a tile), 6 in the second (redone cell by cell)
     rng = np.random.default_rng(9)
     B, T, U, V = 2, 140, 70, 2304
     E = rng.standard_normal((B, T, V)).astype(np.float32)
     P = rng.standard_normal((B, U, V)).astype(np.float32)
     E[0] = np.round(E[0] * 2) * 0.5
     P[0] = np.round(P[0] * 2) * 0.5
-    P[1, 5] = np.round(P[1, 5] * 2) * 0.5
+    P[1, 5:7] = np.round(P[1, 5:7] * 2) * 0.5
     il, ll = np.array([T, 131], np.int32), np.array([U - 1, U - 5], np.int32)
     check(E, P, il, ll, 0)
 
 
+@pytest.mark.parametrize("U,V", [(70, 8192), (33, 8192), (101, 3000)])
 @pytest.mark.parametrize("dist", ["normal", "uniform", "quantised"])
-def test_default_mode_in_the_range_where_lists_are_tried(dist):
-    # V = 8192 with more than 64 label positions is inside the range where the default mode starts on lists and lets a sample of
-    # the cells (two utterances, one frame in sixteen) decide whether to go on.  Uniform scores
-    # fail the bound too often and send the call back to every column, normal ones do not; a
-    # third utterance is outside the sample either way.
+def test_default_mode_in_the_range_where_lists_are_tried(dist, U, V):
+    # Shapes inside the range where the default mode starts on lists (3000 columns or more,
+    # U x V of 250000 or more) and lets a sample of the cells (two utterances, one frame in
+    # sixteen) decide whether to go on.  Uniform scores fail the bound too often and send the
+    # call back to every column, normal ones do not; a third utterance is outside the sample
+    # either way.
     rng = np.random.default_rng(21)
-    B, T, U, V = 3, 37, 70, 8192
+    B, T = 3, 37
     assert capi.load().rnnt_hip_maxplus_tries_lists(B, T, U, V) == 1
     if dist == "normal":
         E, P = rng.standard_normal((B, T, V)), rng.standard_normal((B, U, V))

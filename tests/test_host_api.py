@@ -275,7 +275,10 @@ def test_maxplus_mode_setter_and_query():
         capi.call("rnnt_hip_set_maxplus_mode", 0)
         assert lib.rnnt_hip_maxplus_tries_lists(32, 2000, 101, 10000) == 1
         assert lib.rnnt_hip_maxplus_tries_lists(32, 2000, 101, 2000) == 0
-        assert lib.rnnt_hip_maxplus_tries_lists(32, 2000, 51, 10000) == 0
+        assert lib.rnnt_hip_maxplus_tries_lists(32, 2000, 101, 3000) == 1
+        assert lib.rnnt_hip_maxplus_tries_lists(32, 2000, 51, 10000) == 1
+        assert lib.rnnt_hip_maxplus_tries_lists(32, 2000, 17, 10000) == 0   # U x V too small to pay
+        assert lib.rnnt_hip_maxplus_tries_lists(32, 2000, 33, 4000) == 0
         assert lib.rnnt_hip_maxplus_tries_lists(32, 2000, 101, 32000) == 0
         with pytest.raises(capi.RnntHipError):
             capi.call("rnnt_hip_set_maxplus_mode", 7)

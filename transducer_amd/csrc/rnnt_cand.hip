@@ -30,8 +30,11 @@
 // of a row of P end up on a list if the scores are drawn independently, whatever their scale
 // (230 and 75 of 10000; the square root keeps the share of cells that fail the test level as
 // the vocabulary grows; an entry of P's lists costs twice the bytes of one of E's, hence the
-// shorter lists there; about one cell in 800 then fails the test at V = 10000, and each of
-// those costs the 80 KB of its two rows once more).  A constant or heavily tied row gets an
+// shorter lists there; one cell in 300 to 800 then fails the test for 5000 to 17000 normally
+// distributed columns, and each of those costs the 80 KB of its two rows once more; heavier
+// tails fail far less often, scores with a hard upper edge -- uniform, or the sum of two
+// uniform ones -- one cell in 50 or more, which is where the sample's limit of one in
+// kCdSampleOdds sends a call back to every column).  A constant or heavily tied row gets an
 // empty list instead of a full one.
 #include <hip/hip_runtime.h>
 
@@ -59,9 +62,9 @@ constexpr int kCdAheadShort = 10;  // 16-byte pieces of the next row a thread ho
 constexpr int kCdAheadLong = 17;   // evaluated: rows of up to 10240 / 17408 columns
 constexpr int kCdBatch = 8;      // candidates per batch (two batches in flight)
 constexpr int kCdTileT = 128, kCdTileU = 64;  // the all-columns kernel's tile
-constexpr int kCdTileLimit = 64;  // flagged cells a tile may hold and still be redone cell by cell
+constexpr int kCdTileLimit = 128;  // flagged cells a tile may hold and still be redone cell by cell
 constexpr int kCdCellShare = 16;  // wavefronts (of four workgroups) that share a tile's flagged cells
-constexpr int kCdSampleOdds = 400; // lists go on if at most one sampled cell in this many was flagged
+constexpr int kCdSampleOdds = 150; // lists go on if at most one sampled cell in this many was flagged
 constexpr int kNone = 0x7fffffff;
 static_assert(kCdCap % kCdBatch == 0 && kCdDepth % kCdBatch == 0 && kCdBatch % 4 == 0 &&
                   kCdSeg % 4 == 0,
@@ -811,14 +814,17 @@ bool maxplus_lists_possible(const Dims& d) {
 }
 
 // Where the list path is tried without being asked for (measured on normally distributed
-// scores, B = 8 and 32, T = 2000): from about 5000 columns on, walking two lists of a few
-// hundred columns beats looking at all of them, by 20 to 35 %, as long as two workgroups' rows
-// and lists fit a compute unit's LDS (about 17400 columns; with one workgroup nothing covers
-// the staging of a row) and the label axis fills more than one wavefront (at 51 label positions
-// the all-columns kernel has half the work and the two are level).  Whether a call goes through
-// with it is decided on its own scores (cand_decide_kernel).
+// scores, B = 32, T = 2000).  Looking at every column costs time in proportion to U x V; the
+// list path's time is mostly the staging of the rows of E, in proportion to V, and grows slowly
+// with U.  The two are level at U = 101 with 2000 columns, at U = 33 with 4000-10000 and at
+// U = 64 with 4000; lists are 10 % ahead at (U, V) = (33, 10000) and (64, 4000), 15 % at
+// (101, 3000-4000), 22 % at (51-64, 10000), 30-47 % at U = 101 from 5000 columns up, and
+// further ahead on small grids (B x T of a few thousand frames, where the all-columns kernel's
+// tiles leave most of the device idle).  Two workgroups' rows and lists must fit a compute
+// unit's LDS (about 17400 columns; with one workgroup nothing covers the staging of a row).
+// Whether a call goes through with it is decided on its own scores (cand_decide_kernel).
 bool maxplus_lists_pay(const Dims& d) {
-  return maxplus_lists_possible(d) && d.V >= 5000 && d.U > 64 &&
+  return maxplus_lists_possible(d) && d.V >= 3000 && (size_t)d.U * d.V >= 250000 &&
          2 * cand_lds_bytes(d.V) <= 160 * 1024;
 }
 
