@@ -108,7 +108,7 @@ def recorded_traffic(workload, kernel):
         k = rec["workloads"][workload][kernel]
         return {"bytes": k["fetched_bytes"] + k["written_bytes"], "fetched_bytes": k["fetched_bytes"],
                 "written_bytes": k["written_bytes"], "recorded": rec.get("recorded"),
-                "source": rec.get("source")}
+                "source": k.get("source", rec.get("source"))}
     except (OSError, KeyError, ValueError):
         return None
 
@@ -306,9 +306,11 @@ def viterbi_main(args, name, cfg, opt, capi, d, device):
         esize = E.element_size()
         nbytes = float(np.sum(il.astype(np.int64))) * V * esize + float(B) * U1 * V * esize + 8.0 * cells
         gbs = nbytes / (per_launch["maxplus"] * 1e-3) / 1e9
+        traffic = recorded_traffic(args.workload, "cand_table_stage")
         roofline = {"bound": "hbm", "kernel": "cand_rows_kernel (+ lists of P, fallbacks)",
                     "achieved": round(gbs, 1), "peak": 8000.0, "unit": "GB/s",
-                    "frac": round(gbs / 8000.0, 4), "traffic": None,
+                    "frac": round(gbs / 8000.0, 4),
+                    "traffic": traffic["bytes"] if traffic else None, "traffic_record": traffic,
                     "kernel_ms": round(per_launch["maxplus"], 4), "bytes_per_launch": nbytes,
                     "all_columns_equivalent_tlaneops": round(achieved, 2)}
     out = {
