@@ -358,8 +358,11 @@ __global__ __launch_bounds__(256) void cand_transpose_p_kernel(const TIO* __rest
 // keeps the lowest column whose sum equals the maximum.  Lists are in column order, so that
 // is the lowest column of the whole half; halves and lists are then merged by (larger sum,
 // lower column).
-// While a frame is evaluated, one load per cache line of the next frame's row brings that row
-// into L2, so that staging it waits for L2 and not for HBM.
+// While a frame is evaluated, every wavefront already holds its quarter of the next frame's row
+// in registers (requested right after this frame's row was committed, as the loads return it),
+// so the wait for HBM lies behind the evaluation.  The rows are loaded as read-once, and the
+// workgroups are dealt to the dies by utterance, so that a die's L2 keeps the transposed P of
+// the one or two utterances it is working on.
 // kPieces: 16-byte pieces per lane of a wavefront's quarter of a row.
 template <bool kVec, int kPieces, typename TIO>
 __global__ __launch_bounds__(kCdThreads) void cand_rows_kernel(const TIO* __restrict__ E,
