@@ -58,6 +58,7 @@ constexpr float kCdListP = 0.88f;  // ... rows of P (their one threshold per row
                                    // wavefronts' values: the lists come out a fifth shorter than that)
 constexpr int kCdBisect = 16;    // halvings of the key interval
 constexpr int kCdFrames = 16;    // frames per workgroup of cand_rows_kernel
+constexpr int kCdGather = 4;     // frames whose results a lane stores together
 constexpr int kCdAheadShort = 10;  // 16-byte pieces of the next row a thread holds while a row is
 constexpr int kCdAheadLong = 17;   // evaluated: rows of up to 10240 / 17408 columns
 constexpr int kCdBatch = 8;      // candidates per batch (two batches in flight)
@@ -67,7 +68,7 @@ constexpr int kCdCellShare = 16;  // wavefronts (of four workgroups) that share 
 constexpr int kCdSampleOdds = 150; // lists go on if at most one sampled cell in this many was flagged
 constexpr int kNone = 0x7fffffff;
 static_assert(kCdCap % kCdBatch == 0 && kCdDepth % kCdBatch == 0 && kCdBatch % 4 == 0 &&
-                  kCdSeg % 4 == 0,
+                  kCdSeg % 4 == 0 && kCdGather % 4 == 0 && (kCdGather & (kCdGather - 1)) == 0,
               "whole batches, read four entries at a time");
 
 // order-preserving map of the floats onto the unsigned integers, and back
@@ -418,6 +419,16 @@ __global__ __launch_bounds__(kCdThreads) void cand_rows_kernel(const TIO* __rest
   for (int s = 1; s < 64; s <<= 1) nmax_first = max(nmax_first, __shfl_xor(nmax_first, s, 64));
   nmax_first = __builtin_amdgcn_readfirstlane(nmax_first);
 
+  // The results of kCdGather consecutive frames leave together, 16 bytes at a time (with at most
+  // 128 label positions, where a lane meets one cell per frame): a cell's neighbours in memory
+  // are the same label position's cells of the next frames, and a 4-byte store per frame would
+  // reach L2 as a sector of its own each time (measured: eight times the planes' bytes written
+  // back; gathering all of a workgroup's frames instead of four changes nothing further).
+  const bool gathered = Ub <= 2 * 64;
+  float qtop[kCdGather];
+  int qarg[kCdGather];
+#pragma unroll
+  for (int k = 0; k < kCdGather; ++k) { qtop[k] = 0.0f; qarg[k] = 0; }
   QuarterBits<kPieces, TIO> ahead;
   if (tid == 0) L->bad[0] = L->bad[1] = 0;
   fetch_quarter<kVec, kPieces>(Eb + (size_t)t_lo * d.V, d.V, ahead);
@@ -579,7 +590,33 @@ __global__ __launch_bounds__(kCdThreads) void cand_rows_kernel(const TIO* __rest
         const float bound =
             tau + (ub == 0 ? ptau_first : (valid ? w.ptau[(size_t)b * d.U + u] : 0.0f));
         const bool ok = !bad && top > bound;
-        if (valid) {
+        if (gathered) {
+          const int slot = (t - t_lo) & (kCdGather - 1);  // uniform
+#pragma unroll
+          for (int k = 0; k < kCdGather; ++k) {
+            qtop[k] = slot == k ? top : qtop[k];
+            qarg[k] = slot == k ? (ok ? at : -1) : qarg[k];
+          }
+          if (valid && (slot == kCdGather - 1 || t == t_hi - 1)) {
+            typedef int int4_align4 __attribute__((ext_vector_type(4), aligned(4)));
+            const size_t o = plane_row(d, b, u) + (t - slot) + u;
+#pragma unroll
+            for (int g = 0; g < kCdGather; g += 4) {
+              if (g + 3 <= slot) {
+                float4_align4 qt;
+                int4_align4 qa;
+                qt.x = qtop[g]; qt.y = qtop[g + 1]; qt.z = qtop[g + 2]; qt.w = qtop[g + 3];
+                qa.x = qarg[g]; qa.y = qarg[g + 1]; qa.z = qarg[g + 2]; qa.w = qarg[g + 3];
+                *reinterpret_cast<float4_align4*>(best + o + g) = qt;
+                *reinterpret_cast<int4_align4*>(arg + o + g) = qa;
+              } else {
+#pragma unroll
+                for (int k = g; k < g + 3; ++k)
+                  if (k <= slot) { best[o + k] = qtop[k]; arg[o + k] = qarg[k]; }
+              }
+            }
+          }
+        } else if (valid) {
           const size_t o = plane_row(d, b, u) + t + u;
           best[o] = top;
           arg[o] = ok ? at : -1;
