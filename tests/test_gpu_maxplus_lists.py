@@ -245,11 +245,14 @@ def test_default_mode_in_the_range_where_lists_are_tried(dist, U, V):
     check(E, P, il, ll, 0, modes=(0,))
 
 
+@pytest.mark.parametrize("shape", [(2, 60, 14, 2100), (2, 40, 80, 3200)],
+                         ids=lambda s: "B%d_T%d_U%d_V%d" % s)
 @pytest.mark.parametrize("mode", [0, 1, 2])
-def test_decode_labels_against_oracle(mode):
+def test_decode_labels_against_oracle(mode, shape):
+    # (the second shape is inside the range where the default mode starts on lists)
     import torch
     rng = np.random.default_rng(11)
-    B, T, U, V = 2, 60, 14, 2100
+    B, T, U, V = shape
     E = rng.standard_normal((B, T, V)).astype(np.float32)
     P = rng.standard_normal((B, U, V)).astype(np.float32)
     il, ll = np.array([T, T - 7], np.int32), np.array([U - 1, U - 4], np.int32)
