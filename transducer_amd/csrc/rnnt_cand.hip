@@ -18,7 +18,7 @@
 //   * cand_rows_kernel: per frame, the row of E goes into LDS and gets its threshold and list,
 //     and the four wavefronts of the workgroup (64 label positions each, half of either list)
 //     evaluate A_t against the transposed P and C_u against the LDS row;
-//   * a sample of the cells goes first (two utterances, one frame in kCdFrames): if too many of
+//   * a sample of the cells goes first (two utterances, one frame in kCdSampleEvery): if too many of
 //     them fail the test -- scores with a hard upper edge do -- everything else returns at once
 //     and the all-columns kernel (maxplus_kernel) builds the whole table;
 //   * otherwise tiles of 128 frames x 64 label positions with more than kCdTileLimit flagged
@@ -57,7 +57,9 @@ constexpr float kCdListE = 2.31f;  // list lengths the ranks are derived from, i
 constexpr float kCdListP = 0.88f;  // ... rows of P (their one threshold per row is the largest of four
                                    // wavefronts' values: the lists come out a fifth shorter than that)
 constexpr int kCdBisect = 16;    // halvings of the key interval
-constexpr int kCdFrames = 16;    // frames per workgroup of cand_rows_kernel
+constexpr int kCdFrames = 8;     // frames per workgroup of cand_rows_kernel (16: 5 % slower, more utterances'
+                                 // transposed P in flight per die; 4: level; 2: 3 % slower)
+constexpr int kCdSampleEvery = 16;  // the sample takes one frame in this many (a multiple of kCdFrames)
 constexpr int kCdGather = 4;     // frames whose results a lane stores together
 constexpr int kCdAheadShort = 10;  // 16-byte pieces of the next row a thread holds while a row is
 constexpr int kCdAheadLong = 17;   // evaluated: rows of up to 10240 / 17408 columns
@@ -68,7 +70,8 @@ constexpr int kCdCellShare = 16;  // wavefronts (of four workgroups) that share 
 constexpr int kCdSampleOdds = 150; // lists go on if at most one sampled cell in this many was flagged
 constexpr int kNone = 0x7fffffff;
 static_assert(kCdCap % kCdBatch == 0 && kCdDepth % kCdBatch == 0 && kCdBatch % 4 == 0 &&
-                  kCdSeg % 4 == 0 && kCdGather % 4 == 0 && (kCdGather & (kCdGather - 1)) == 0,
+                  kCdSeg % 4 == 0 && kCdGather % 4 == 0 && (kCdGather & (kCdGather - 1)) == 0 &&
+                  kCdSampleEvery % kCdFrames == 0,
               "whole batches, read four entries at a time");
 
 // order-preserving map of the floats onto the unsigned integers, and back
@@ -376,8 +379,8 @@ __global__ __launch_bounds__(kCdThreads) void cand_rows_kernel(const TIO* __rest
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   float* row = reinterpret_cast<float*>(lds_raw);
   RowLists* L = reinterpret_cast<RowLists*>(row + padded_row(d.V));
-  // The sample: the first frame of every workgroup's run of frames, in the sample's utterances.
-  // The rest: every other frame of those, and all frames of the others.
+  // The sample: every kCdSampleEvery-th frame of the sample's utterances, one per workgroup.
+  // The rest: every other frame of those, and all frames of the others, kCdFrames per workgroup.
   int b = blockIdx.y, group = blockIdx.x;
   if (ps.phase == 0) b = b == 0 ? ps.first : ps.second;
   else if (w.stats[2] == 0) return;
@@ -392,13 +395,13 @@ __global__ __launch_bounds__(kCdThreads) void cand_rows_kernel(const TIO* __rest
     group = (int)(pair % gridDim.x);
   }
   const bool sampled = b == ps.first || b == ps.second;
-  int t_lo = group * kCdFrames;
+  int t_lo = group * (ps.phase == 0 ? kCdSampleEvery : kCdFrames);
   int Tb, Ub;
   utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
   if (t_lo >= Tb || Ub == 0) return;
   int t_hi = min(t_lo + kCdFrames, Tb);
   if (ps.phase == 0) t_hi = t_lo + 1;
-  else if (sampled) ++t_lo;
+  else if (sampled && t_lo % kCdSampleEvery == 0) ++t_lo;
   if (t_lo >= t_hi) return;
   const int phase = ps.phase;
   const int tid = threadIdx.x, lane = tid & 63;
@@ -783,14 +786,15 @@ int cand_any(const TIO* E, const TIO* P, const int* inLen, const int* labLen, fl
   hipLaunchKernelGGL(cand_zero_kernel, dim3((tiles + 4 + 255) / 256), dim3(256), 0, s,
                      w.tile_fail, tiles + 4);
   RNNT_LAUNCH_CHECK("cand_zero_kernel");
-  // The sample's utterances first (their lists, their transposed P, one frame in kCdFrames),
+  // The sample's utterances first (their lists, their transposed P, one frame in kCdSampleEvery),
   // then the decision, then everything else -- whose launches return at once if it is a no.
   const Pass sample{0, 0, d.B > 1 ? d.B / 2 : -1}, rest{1, sample.first, sample.second};
   const int nsample = d.B > 1 ? 2 : 1;
   const int2 ranks = make_int2(list_rank(kCdListE, d.V), list_rank(kCdListP, d.V));
   const int pieces = (padded_row(d.V) / 4 + 255) / 256;  // 16-byte pieces per thread of a quarter of a row
   const int chunks = (d.T + kCdFrames - 1) / kCdFrames, ublocks64 = ((d.U + 63) / 64) * 64;
-#define RNNT_CAND_PASS(VEC, PS, NB)                                                              \
+  const int sample_chunks = (d.T + kCdSampleEvery - 1) / kCdSampleEvery;
+#define RNNT_CAND_PASS(VEC, PS, NB, CH)                                                            \
   do {                                                                                           \
     hipLaunchKernelGGL((cand_transpose_p_kernel<TIO>),                                           \
                        dim3((d.V + 31) / 32, (Uq + 31) / 32, NB), dim3(256), 0, s, P, w.PT, d,   \
@@ -800,11 +804,11 @@ int cand_any(const TIO* E, const TIO* P, const int* inLen, const int* labLen, fl
                        lds, s, P, w, d, PS, ranks);                                              \
     RNNT_LAUNCH_CHECK("cand_lists_p_kernel");                                                    \
     if (pieces <= kCdAheadShort)                                                                 \
-      hipLaunchKernelGGL((cand_rows_kernel<VEC, kCdAheadShort, TIO>), dim3(chunks, NB),          \
+      hipLaunchKernelGGL((cand_rows_kernel<VEC, kCdAheadShort, TIO>), dim3(CH, NB),              \
                          dim3(kCdThreads), lds, s, E, inLen, labLen, best, arg, w, d, Uq, PS,    \
                          ranks);                                                                 \
     else                                                                                         \
-      hipLaunchKernelGGL((cand_rows_kernel<VEC, kCdAheadLong, TIO>), dim3(chunks, NB),           \
+      hipLaunchKernelGGL((cand_rows_kernel<VEC, kCdAheadLong, TIO>), dim3(CH, NB),               \
                          dim3(kCdThreads), lds, s, E, inLen, labLen, best, arg, w, d, Uq, PS,    \
                          ranks);                                                                 \
     RNNT_LAUNCH_CHECK("cand_rows_kernel");                                                       \
@@ -814,10 +818,10 @@ int cand_any(const TIO* E, const TIO* P, const int* inLen, const int* labLen, fl
     RNNT_TRY(allow_lds(cand_lists_p_kernel<VEC, TIO>, lds));                                     \
     RNNT_TRY(allow_lds(cand_rows_kernel<VEC, kCdAheadShort, TIO>, lds));                         \
     RNNT_TRY(allow_lds(cand_rows_kernel<VEC, kCdAheadLong, TIO>, lds));                          \
-    RNNT_CAND_PASS(VEC, sample, nsample);                                                        \
+    RNNT_CAND_PASS(VEC, sample, nsample, sample_chunks);                                                   \
     hipLaunchKernelGGL(cand_decide_kernel, dim3(1), dim3(1), 0, s, w.stats, force ? 1 : 0);      \
     RNNT_LAUNCH_CHECK("cand_decide_kernel");                                                     \
-    RNNT_CAND_PASS(VEC, rest, d.B);                                                              \
+    RNNT_CAND_PASS(VEC, rest, d.B, chunks);                                                         \
   } while (0)
   if (vec) RNNT_CAND_PASSES(true);
   else RNNT_CAND_PASSES(false);
