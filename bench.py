@@ -34,6 +34,8 @@ Prints ONE JSON line:
                         else a bounded sample scaled by lattice-cell count ("scaled": true); the
                         lattice recursions are also timed through the reference's own
                         transducer_cpu.cpp build (oracle/_ref) when it is present
+                        (decode workloads: the CPU log-normaliser + best path, and the
+                        number of utterances whose labels equal the device's)
 """
 import argparse
 import ctypes
@@ -185,6 +187,65 @@ def cpu_baseline(d, seconds_budget=60.0):
     return out, res
 
 
+def viterbi_cpu_baseline(d, seconds_budget=60.0):
+    """The CPU decode on the bench's own inputs: log-normaliser (the torch-free form of the
+    reference's tests, transducer/test.h:51-80) + best path (transducer/transducer_cpu.cpp:145-222)
+    by the OpenMP restatement in oracle/; the best path alone also through the reference's own
+    transducer_cpu.cpp when oracle/_ref was built.  Returns the record and, when the whole batch
+    was run, the labels."""
+    import oracle  # checker code, used here only as the timed CPU baseline
+    threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    E, P = d["emissions"], d["predictions"]
+    il, ll = d["input_lengths"], d["label_lengths"]
+    B, T, V = E.shape
+    U = P.shape[1] - 1
+
+    def run(E, P, sil, sll):
+        t0 = time.perf_counter()
+        LN = oracle.log_norms_naive(E, P, sil, sll)
+        t1 = time.perf_counter()
+        labels = oracle.viterbi(E, P, LN, sil, sll)
+        t2 = time.perf_counter()
+        ref_s = None
+        if oracle.have_ref():
+            oracle.ref_viterbi(E, P, LN, sil, sll)
+            ref_s = time.perf_counter() - t2
+        cells = float(np.sum(sil.astype(np.int64) * (sll.astype(np.int64) + 1)))
+        return t1 - t0, t2 - t1, ref_s, cells, labels
+
+    Tp = min(T, 8)
+    probe = run(np.ascontiguousarray(E[:, :Tp]), P, np.minimum(il, Tp).astype(np.int32), ll)
+    cells_full = float(np.sum(il.astype(np.int64) * (ll.astype(np.int64) + 1)))
+    estimate = (probe[0] + probe[1] + (probe[2] or 0.0)) * cells_full / max(probe[3], 1.0)
+    if estimate <= seconds_budget:
+        lse_s, vit_s, ref_s, cells, labels = run(E, P, il, ll)
+        scale, scaled = 1.0, False
+        sample = "the whole batch (%d utterances, the bench's own inputs)" % B
+    else:
+        Bs = max(1, min(B, threads))
+        per_frame = (probe[0] + probe[1] + (probe[2] or 0.0)) / Tp * Bs / B
+        Ts = int(max(8, min(T, 20.0 / max(per_frame, 1e-9))))
+        lse_s, vit_s, ref_s, cells, labels = run(
+            np.ascontiguousarray(E[:Bs, :Ts]), np.ascontiguousarray(P[:Bs]),
+            np.minimum(il[:Bs], Ts).astype(np.int32), np.ascontiguousarray(ll[:Bs]))
+        scale, scaled, labels = cells_full / cells, True, None
+        sample = "%d of %d utterances x first %d of %d frames of the bench's inputs" % (Bs, B, Ts, T)
+    out = {
+        "value": round((lse_s + vit_s) * 1e3 * scale, 1),
+        "unit": "ms per decode",
+        "cores": threads,
+        "kind": "port",
+        "scaled": scaled,
+        "sample": "%s, U=%d V=%d; naive LSE + best path (OpenMP over utterances); measured %.2f s"
+                  % (sample, U, V, lse_s + vit_s),
+        "lse_ms": round(lse_s * 1e3 * scale, 1),
+        "best_path_ms": round(vit_s * 1e3 * scale, 1),
+    }
+    if ref_s is not None:
+        out["best_path_ms_reference_build"] = round(ref_s * 1e3 * scale, 1)
+    return out, labels
+
+
 def outside(got, want, rtol=1e-4, atol=1e-5):
     """fraction of entries with |got - want| > atol + rtol |want| (one utterance at a time: the
     arrays are gigabytes)"""
@@ -325,6 +386,15 @@ def viterbi_main(args, name, cfg, opt, capi, d, device):
         "stage_ms_per_step": per_step,
         "checks": checks,
     }
+    if not args.no_cpu_baseline and not io:  # the CPU path has no 16-bit form
+        out["cpu_baseline"], cpu_labels = viterbi_cpu_baseline(d)
+        if cpu_labels is not None:
+            # (reported, not part of "ok": the CPU path's own log-normaliser differs from the
+            # device's in its last bits, which may move a decision between two paths of nearly
+            # the same score)
+            same = [bool(np.array_equal(paths[b, :ll[b]], cpu_labels[b, :ll[b]])) for b in range(B)]
+            checks["against_cpu_baseline"] = {"utterances_with_the_same_labels": int(sum(same)),
+                                              "of": B}
     print(json.dumps(out))
     return 0 if checks["ok"] else 1
 
