@@ -203,8 +203,9 @@ int rnnt_hip_set_spin_limit(int trips);
  *      each frame and each label position first gets a short list of its largest scores,
  *      a cell is settled from the two lists where a bound proves that no other column can win,
  *      and the remaining cells are evaluated over every column; the call looks at a sample of
- *      the cells first and goes back to every column if too many of them fail the bound
- *      (scores with a hard upper edge, such as uniform ones, do);
+ *      the cells first, takes lists half as long again if too many of them fail the bound
+ *      (scores with a hard upper edge, such as uniform ones, do), and goes back to every column
+ *      if too many fail with those as well;
  *   1: over every column always;
  *   2: lists for every vocabulary of up to 17408 entries, without the sample (for tests).
  * The labels returned are the same in every mode; the setting is process-wide.  No counterpart

@@ -230,7 +230,8 @@ def test_default_mode_in_the_range_where_lists_are_tried(dist, U, V):
     # Shapes inside the range where the default mode starts on lists (3000 columns or more,
     # U x V of 250000 or more) and lets a sample of the cells (two utterances, one frame in
     # sixteen) decide whether to go on.  Uniform scores fail the bound too often and send the
-    # call back to every column, normal ones do not; a third utterance is outside the sample
+    # call on to a second pair of longer lists, quantised ones fail with those too and send it
+    # back to every column, normal ones pass at once; a third utterance is outside the sample
     # either way.
     rng = np.random.default_rng(21)
     B, T = 3, 37

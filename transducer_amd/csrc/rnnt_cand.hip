@@ -19,8 +19,9 @@
 //     and the four wavefronts of the workgroup (64 label positions each, half of either list)
 //     evaluate A_t against the transposed P and C_u against the LDS row;
 //   * a sample of the cells goes first (two utterances, one frame in kCdSampleEvery): if too many of
-//     them fail the test -- scores with a hard upper edge do -- everything else returns at once
-//     and the all-columns kernel (maxplus_kernel) builds the whole table;
+//     them fail the test -- scores with a hard upper edge do -- the sample is taken again with
+//     lists half as long again (kCdLongE, kCdLongP), and if that fails too everything else
+//     returns at once and the all-columns kernel (maxplus_kernel) builds the whole table;
 //   * otherwise tiles of 128 frames x 64 label positions with more than kCdTileLimit flagged
 //     cells are redone by that kernel, the others' flagged cells one by one
 //     (cand_cells_kernel): the cost of a failed test is bounded either way.
@@ -34,7 +35,7 @@
 // distributed columns, and each of those costs the 80 KB of its two rows once more; heavier
 // tails fail far less often, scores with a hard upper edge -- uniform, or the sum of two
 // uniform ones -- one cell in 50 or more, which is where the sample's limit of one in
-// kCdSampleOdds sends a call back to every column).  A constant or heavily tied row gets an
+// kCdSampleOdds sends a call on to the longer lists, and from there back to every column).  A constant or heavily tied row gets an
 // empty list instead of a full one.
 #include <hip/hip_runtime.h>
 
@@ -56,6 +57,10 @@ constexpr int kCdStored = kCdDepth + 16;  // with two batches of padding behind 
 constexpr float kCdListE = 2.31f;  // list lengths the ranks are derived from, in units of sqrt(V): rows of E
 constexpr float kCdListP = 0.88f;  // ... rows of P (their one threshold per row is the largest of four
                                    // wavefronts' values: the lists come out a fifth shorter than that)
+constexpr float kCdLongE = 3.5f, kCdLongP = 1.3f;  // the same for the longer lists that a call falls back
+                                   // to when too many cells of its sample fail with the usual ones
+                                   // (scores with a hard upper edge: uniform ones fail 1 cell in 12
+                                   // with the usual lists and 1 in 500 with these)
 constexpr int kCdBisect = 16;    // halvings of the key interval
 constexpr int kCdFrames = 8;     // frames per workgroup of cand_rows_kernel (16: 5 % slower, more utterances'
                                  // transposed P in flight per die; 4: level; 2: 3 % slower)
@@ -265,25 +270,34 @@ struct CandScratch {
   float* ptau;    // [B][U]   thresholds (+inf where the list did not fit)
   int* tile_fail; // [B][tiles of 128 frames][tiles of 64 label positions]   flagged cells
   int* tile_cells;  // [tiles][kCdTileLimit]   the first flagged cells of a tile (cell index in the tile)
-  int* stats;       // [0] flagged cells of the sample, [1] cells of the sample, [2] lists go on (0 / 1)
+  int* stats;       // [0] flagged cells of the sample, [1] cells of the sample, [2] the tier the call
+                    // goes on with (0: every column, 1: lists, 2: the longer lists), [3] the first
+                    // sample failed and the second is to run
 };
 
-// Which utterances a launch takes.  Phase 0 (the sample): utterance `first` (grid index 0) and
-// `second` (index 1, if any).  Phase 1 (the rest): every utterance but those two, and nothing at
-// all unless the sample said that lists pay for these scores (stats[2]).
+// Which utterances a launch takes, and with which lists.  Phase 0 (a sample): utterance `first`
+// (grid index 0) and `second` (index 1, if any), with the lists of `tier` (1: the usual
+// lengths, 2: the longer ones; the second sample runs only if the first one failed, stats[3]).
+// Phase 1 (the rest): every utterance but those two, with the lists of the tier the samples
+// settled on, and nothing at all if that is none (stats[2]).
 struct Pass {
-  int phase, first, second;
+  int phase, first, second, tier;
 };
+__device__ inline int pass_tier(const Pass& ps, const int* stats) {
+  if (ps.phase == 0) return (ps.tier == 1 || stats[3] != 0) ? ps.tier : 0;
+  return stats[2];
+}
 __device__ inline int pass_utterance(const Pass& ps, int index, const int* stats) {
+  if (pass_tier(ps, stats) == 0) return -1;
   if (ps.phase == 0) return index == 0 ? ps.first : ps.second;
-  if (stats[2] == 0 || index == ps.first || index == ps.second) return -1;
+  if (index == ps.first || index == ps.second) return -1;
   return index;
 }
 
 template <bool kVec, typename TIO>
 __global__ __launch_bounds__(kCdThreads) void cand_lists_p_kernel(const TIO* __restrict__ P,
                                                                   CandScratch w, Dims d, Pass ps,
-                                                                  int2 ranks) {
+                                                                  int4 ranks) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   float* row = reinterpret_cast<float*>(lds_raw);
   RowLists* L = reinterpret_cast<RowLists*>(row + padded_row(d.V));
@@ -305,7 +319,8 @@ __global__ __launch_bounds__(kCdThreads) void cand_lists_p_kernel(const TIO* __r
   // one threshold for the whole row, the largest of the four wavefronts' (their own would put a
   // fifth more columns on the list for the same bound; for a row of E that is the price of not
   // waiting for the other wavefronts, here the list is built once and walked for every frame)
-  const float tau_own = quarter_threshold<kVec, kCdAheadLong>(bits, regs, d.V, d.blank, ranks.y, row);
+  const int rank = pass_tier(ps, w.stats) == 2 ? ranks.w : ranks.y;
+  const float tau_own = quarter_threshold<kVec, kCdAheadLong>(bits, regs, d.V, d.blank, rank, row);
   if ((tid & 63) == 0) L->tau[tid >> 6] = tau_own;
   __syncthreads();
   const float tau = fmaxf(fmaxf(L->tau[0], L->tau[1]), fmaxf(L->tau[2], L->tau[3]));
@@ -375,15 +390,17 @@ __global__ __launch_bounds__(kCdThreads) void cand_rows_kernel(const TIO* __rest
                                                                float* __restrict__ best,
                                                                int* __restrict__ arg,
                                                                CandScratch w, Dims d, int Uq, Pass ps,
-                                                               int2 ranks) {
+                                                               int4 ranks) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   float* row = reinterpret_cast<float*>(lds_raw);
   RowLists* L = reinterpret_cast<RowLists*>(row + padded_row(d.V));
   // The sample: every kCdSampleEvery-th frame of the sample's utterances, one per workgroup.
   // The rest: every other frame of those, and all frames of the others, kCdFrames per workgroup.
   int b = blockIdx.y, group = blockIdx.x;
+  const int tier = pass_tier(ps, w.stats);
+  if (tier == 0) return;
+  const int rank = tier == 2 ? ranks.z : ranks.x;
   if (ps.phase == 0) b = b == 0 ? ps.first : ps.second;
-  else if (w.stats[2] == 0) return;
   else {
     // Workgroups are dealt to the eight dies in launch order, one each in turn; die k takes the
     // k-th eighth of the (utterance, run of frames) pairs, so that at any time its L2 holds the
@@ -440,7 +457,7 @@ __global__ __launch_bounds__(kCdThreads) void cand_rows_kernel(const TIO* __rest
   for (int t = t_lo; t < t_hi; ++t) {
     // this frame's row is in registers; the next one's is requested before the evaluation
     const int fp = (t - t_lo) & 1;
-    commit_quarter<kVec, kPieces>(ahead, d.V, d.blank, pitch, ranks.x, fp, row, L);
+    commit_quarter<kVec, kPieces>(ahead, d.V, d.blank, pitch, rank, fp, row, L);
     if (t + 1 < t_hi) fetch_quarter<kVec, kPieces>(Eb + (size_t)(t + 1) * d.V, d.V, ahead);
     __syncthreads();
     if (tid == 0) L->bad[fp ^ 1] = 0;  // the next frame's flag: nobody sets it before the hand-over barrier
@@ -705,9 +722,27 @@ __global__ __launch_bounds__(256) void cand_cells_kernel(const TIO* __restrict__
   }
 }
 
-// after the sample: lists go on if few enough of its cells were flagged (one thread)
-__global__ void cand_decide_kernel(int* stats, int force) {
-  stats[2] = (force || (long long)stats[0] * kCdSampleOdds <= (long long)stats[1]) ? 1 : 0;
+// After a sample: lists go on if few enough of its cells were flagged (one thread).  After the
+// first sample a failure asks for the second, with the longer lists; after the second it sends
+// the call to every column.
+__global__ void cand_decide_kernel(int* stats, int force, int stage, int* tile_fail,
+                                   int tiles_per_utterance, int first, int second) {
+  const bool few = (long long)stats[0] * kCdSampleOdds <= (long long)stats[1];
+  if (stage == 1) {
+    const bool ok = force || few;
+    stats[2] = ok ? 1 : 0;
+    stats[3] = ok ? 0 : 1;
+    if (!ok) {  // the second sample starts from nothing: it redoes and flags the same cells
+      stats[0] = stats[1] = 0;
+      for (int i = 0; i < tiles_per_utterance; ++i) {
+        tile_fail[(size_t)first * tiles_per_utterance + i] = 0;
+        if (second >= 0) tile_fail[(size_t)second * tiles_per_utterance + i] = 0;
+      }
+    }
+  } else if (stats[3] != 0) {
+    stats[2] = few ? 2 : 0;
+    stats[3] = 0;
+  }
 }
 
 __global__ void cand_zero_kernel(int* x, int n) {
@@ -787,19 +822,25 @@ int cand_any(const TIO* E, const TIO* P, const int* inLen, const int* labLen, fl
                      w.tile_fail, tiles + 4);
   RNNT_LAUNCH_CHECK("cand_zero_kernel");
   // The sample's utterances first (their lists, their transposed P, one frame in kCdSampleEvery),
-  // then the decision, then everything else -- whose launches return at once if it is a no.
-  const Pass sample{0, 0, d.B > 1 ? d.B / 2 : -1}, rest{1, sample.first, sample.second};
+  // then the decision; if it is a no, the same sample again with the longer lists, and the
+  // decision between those and every column; then everything else -- whose launches return at
+  // once if it is every column (as the second sample's do when the first one passed).
+  const int first = 0, second = d.B > 1 ? d.B / 2 : -1;
+  const Pass sample{0, first, second, 1}, again{0, first, second, 2}, rest{1, first, second, 0};
   const int nsample = d.B > 1 ? 2 : 1;
-  const int2 ranks = make_int2(list_rank(kCdListE, d.V), list_rank(kCdListP, d.V));
+  const int4 ranks = make_int4(list_rank(kCdListE, d.V), list_rank(kCdListP, d.V),
+                               list_rank(kCdLongE, d.V), list_rank(kCdLongP, d.V));
   const int pieces = (padded_row(d.V) / 4 + 255) / 256;  // 16-byte pieces per thread of a quarter of a row
   const int chunks = (d.T + kCdFrames - 1) / kCdFrames, ublocks64 = ((d.U + 63) / 64) * 64;
   const int sample_chunks = (d.T + kCdSampleEvery - 1) / kCdSampleEvery;
-#define RNNT_CAND_PASS(VEC, PS, NB, CH)                                                            \
+#define RNNT_CAND_PASS(VEC, PS, NB, CH, TRANSPOSE)                                               \
   do {                                                                                           \
-    hipLaunchKernelGGL((cand_transpose_p_kernel<TIO>),                                           \
-                       dim3((d.V + 31) / 32, (Uq + 31) / 32, NB), dim3(256), 0, s, P, w.PT, d,   \
-                       Uq, PS, w.stats);                                                         \
-    RNNT_LAUNCH_CHECK("cand_transpose_p_kernel");                                                \
+    if (TRANSPOSE) {                                                                             \
+      hipLaunchKernelGGL((cand_transpose_p_kernel<TIO>),                                         \
+                         dim3((d.V + 31) / 32, (Uq + 31) / 32, NB), dim3(256), 0, s, P, w.PT, d, \
+                         Uq, PS, w.stats);                                                       \
+      RNNT_LAUNCH_CHECK("cand_transpose_p_kernel");                                              \
+    }                                                                                            \
     hipLaunchKernelGGL((cand_lists_p_kernel<VEC, TIO>), dim3(ublocks64, NB), dim3(kCdThreads),  \
                        lds, s, P, w, d, PS, ranks);                                              \
     RNNT_LAUNCH_CHECK("cand_lists_p_kernel");                                                    \
@@ -813,19 +854,27 @@ int cand_any(const TIO* E, const TIO* P, const int* inLen, const int* labLen, fl
                          ranks);                                                                 \
     RNNT_LAUNCH_CHECK("cand_rows_kernel");                                                       \
   } while (0)
+#define RNNT_CAND_DECIDE(STAGE)                                                                  \
+  do {                                                                                           \
+    hipLaunchKernelGGL(cand_decide_kernel, dim3(1), dim3(1), 0, s, w.stats, force ? 1 : 0,       \
+                       STAGE, w.tile_fail, tiles / d.B, first, second);                          \
+    RNNT_LAUNCH_CHECK("cand_decide_kernel");                                                     \
+  } while (0)
 #define RNNT_CAND_PASSES(VEC)                                                                    \
   do {                                                                                           \
     RNNT_TRY(allow_lds(cand_lists_p_kernel<VEC, TIO>, lds));                                     \
     RNNT_TRY(allow_lds(cand_rows_kernel<VEC, kCdAheadShort, TIO>, lds));                         \
     RNNT_TRY(allow_lds(cand_rows_kernel<VEC, kCdAheadLong, TIO>, lds));                          \
-    RNNT_CAND_PASS(VEC, sample, nsample, sample_chunks);                                                   \
-    hipLaunchKernelGGL(cand_decide_kernel, dim3(1), dim3(1), 0, s, w.stats, force ? 1 : 0);      \
-    RNNT_LAUNCH_CHECK("cand_decide_kernel");                                                     \
-    RNNT_CAND_PASS(VEC, rest, d.B, chunks);                                                         \
+    RNNT_CAND_PASS(VEC, sample, nsample, sample_chunks, true);                                   \
+    RNNT_CAND_DECIDE(1);                                                                         \
+    RNNT_CAND_PASS(VEC, again, nsample, sample_chunks, false);                                   \
+    RNNT_CAND_DECIDE(2);                                                                         \
+    RNNT_CAND_PASS(VEC, rest, d.B, chunks, true);                                                \
   } while (0)
   if (vec) RNNT_CAND_PASSES(true);
   else RNNT_CAND_PASSES(false);
 #undef RNNT_CAND_PASS
+#undef RNNT_CAND_DECIDE
 #undef RNNT_CAND_PASSES
   return kOk;
 }
