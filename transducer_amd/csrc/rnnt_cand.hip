@@ -23,8 +23,9 @@
 //     lists half as long again (kCdLongE, kCdLongP), and if that fails too everything else
 //     returns at once and the all-columns kernel (maxplus_kernel) builds the whole table;
 //   * otherwise tiles of 128 frames x 64 label positions with more than kCdTileLimit flagged
-//     cells are redone by that kernel, the others' flagged cells one by one
-//     (cand_cells_kernel): the cost of a failed test is bounded either way.
+//     cells are redone by that kernel, the others' flagged cells one by one, from one list for
+//     the whole call that all wavefronts of cand_cells_kernel share: the cost of a failed test
+//     is bounded either way.
 //
 // A threshold is a value with at most `rank` of a wavefront's 64 per-thread maxima above it.
 // The rank is chosen (list_rank) so that about 2.3 sqrt(V) columns of a row of E and 0.75 sqrt(V)
@@ -71,7 +72,8 @@ constexpr int kCdAheadLong = 17;   // evaluated: rows of up to 10240 / 17408 col
 constexpr int kCdBatch = 8;      // candidates per batch (two batches in flight)
 constexpr int kCdTileT = 128, kCdTileU = 64;  // the all-columns kernel's tile
 constexpr int kCdTileLimit = 128;  // flagged cells a tile may hold and still be redone cell by cell
-constexpr int kCdCellShare = 16;  // wavefronts (of four workgroups) that share a tile's flagged cells
+constexpr int kCdCellGroups = 2048;  // workgroups (of four wavefronts) that share the flagged cells
+constexpr int kCdStats = 8;       // ints of CandScratch::stats
 constexpr int kCdSampleOdds = 150; // lists go on if at most one sampled cell in this many was flagged
 constexpr int kNone = 0x7fffffff;
 static_assert(kCdCap % kCdBatch == 0 && kCdDepth % kCdBatch == 0 && kCdBatch % 4 == 0 &&
@@ -269,10 +271,12 @@ struct CandScratch {
   int* pcount;    // [B][U]   entries of each list
   float* ptau;    // [B][U]   thresholds (+inf where the list did not fit)
   int* tile_fail; // [B][tiles of 128 frames][tiles of 64 label positions]   flagged cells
-  int* tile_cells;  // [tiles][kCdTileLimit]   the first flagged cells of a tile (cell index in the tile)
+  int2* cells;      // [cell_cap]   the flagged cells of the whole call, in the order they were
+                    // found: {b T + t, u}
+  int cell_cap;     // tiles x kCdTileLimit: room for every cell of every tile that is not redone whole
   int* stats;       // [0] flagged cells of the sample, [1] cells of the sample, [2] the tier the call
                     // goes on with (0: every column, 1: lists, 2: the longer lists), [3] the first
-                    // sample failed and the second is to run
+                    // sample failed and the second is to run, [4] entries of `cells`
 };
 
 // Which utterances a launch takes, and with which lists.  Phase 0 (a sample): utterance `first`
@@ -647,14 +651,20 @@ __global__ __launch_bounds__(kCdThreads) void cand_rows_kernel(const TIO* __rest
           atomicAdd(&w.stats[0], __builtin_popcountll(failed));
           atomicAdd(&w.stats[1], __builtin_popcountll(cells));
         }
-        if (failed) {  // count them per tile and leave the first few where they can be found
+        if (failed) {  // count them per tile and put them on the call's list
           const size_t tile = ((size_t)b * tiles_t + t / kCdTileT) * tiles_u + (ub >> 6) + blk;
+          const int n = __builtin_popcountll(failed);
           int base = 0;
-          if (lane == 0) base = atomicAdd(&w.tile_fail[tile], __builtin_popcountll(failed));
+          if (lane == 0) {
+            atomicAdd(&w.tile_fail[tile], n);
+            base = atomicAdd(&w.stats[4], n);
+          }
           base = __builtin_amdgcn_readfirstlane(base);
           const int slot = base + lanes_below(failed);
-          if (valid && !ok && slot < kCdTileLimit)
-            w.tile_cells[tile * kCdTileLimit + slot] = (t & (kCdTileT - 1)) + kCdTileT * lane;
+          if (valid && !ok) {
+            if ((unsigned)slot < (unsigned)w.cell_cap) w.cells[slot] = make_int2(b * d.T + t, u);
+            else atomicMax(&w.tile_fail[tile], kCdTileLimit + 1);  // no room: the tile is redone whole
+          }
         }
       }
     }
@@ -664,28 +674,27 @@ __global__ __launch_bounds__(kCdThreads) void cand_rows_kernel(const TIO* __rest
 }
 
 // ------------------------------------------------------------------ flagged cells, one by one
-// Every wavefront of workgroup (x, y, z) of the grid (tiles of frames x kCdCellShare / 4, tiles of
-// label positions, B) takes every kCdCellShare-th flagged cell of its tile: all columns, each
-// lane keeping the lowest column of its own maximum; (larger sum, lower column) merges the lanes.
+// The wavefronts of the grid share the call's list of flagged cells, one cell at a time each
+// (cells of tiles that maxplus_kernel redoes whole are passed over): all columns, each lane
+// keeping the lowest column of its own maximum; (larger sum, lower column) merges the lanes.
+// Neighbours on the list were flagged together -- the same frame, mostly -- so the four
+// wavefronts of a workgroup read the same row of E.
 template <typename TIO>
 __global__ __launch_bounds__(256) void cand_cells_kernel(const TIO* __restrict__ E,
                                                          const TIO* __restrict__ P,
                                                          float* __restrict__ best,
-                                                         int* __restrict__ arg,
-                                                         const int* __restrict__ tile_fail,
-                                                         const int* __restrict__ tile_cells,
-                                                         const int* __restrict__ stats, Dims d) {
-  constexpr int kGroups = kCdCellShare / 4;
-  const int tile_x = blockIdx.x / kGroups, group = blockIdx.x % kGroups;
-  const int b = blockIdx.z, t0 = tile_x * kCdTileT, u0 = blockIdx.y * kCdTileU;
-  const size_t tile = ((size_t)b * (gridDim.x / kGroups) + tile_x) * gridDim.y + blockIdx.y;
-  const int failed = tile_fail[tile];
-  if (stats[2] == 0 || failed == 0 || failed > kCdTileLimit) return;
+                                                         int* __restrict__ arg, CandScratch w,
+                                                         Dims d) {
+  if (w.stats[2] == 0) return;
+  const int count = min(w.stats[4], w.cell_cap);
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  for (int i = 4 * group + wave; i < failed; i += kCdCellShare) {
-    const int c = tile_cells[tile * kCdTileLimit + i];
-    const int t = t0 + (c & (kCdTileT - 1)), u = u0 + c / kCdTileT;
+  const int tiles_t = (d.T + kCdTileT - 1) / kCdTileT, tiles_u = (d.U + kCdTileU - 1) / kCdTileU;
+  for (int i = 4 * blockIdx.x + wave; i < count; i += 4 * gridDim.x) {
+    const int2 c = w.cells[i];
+    const int b = c.x / d.T, t = c.x - b * d.T, u = c.y;
+    if (w.tile_fail[((size_t)b * tiles_t + t / kCdTileT) * tiles_u + u / kCdTileU] > kCdTileLimit)
+      continue;
     const TIO* e = E + ((size_t)b * d.T + t) * d.V;
     const TIO* p = P + ((size_t)b * d.U + u) * d.V;
     float top = kNegInf;
@@ -768,6 +777,7 @@ __global__ __launch_bounds__(256) void table_out_kernel(const float* __restrict_
 }
 
 size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
+size_t min_size(size_t a, size_t b) { return a < b ? a : b; }
 int cand_uq(const Dims& d) { return (d.U + 3) & ~3; }
 size_t cand_tiles(const Dims& d) {
   return (size_t)d.B * ((d.T + kCdTileT - 1) / kCdTileT) * ((d.U + kCdTileU - 1) / kCdTileU);
@@ -786,8 +796,9 @@ void carve(void* base, const Dims& d, CandScratch* w) {
   p += align256(sizeof(float) * (size_t)d.B * d.U);
   w->tile_fail = reinterpret_cast<int*>(p);
   w->stats = w->tile_fail + cand_tiles(d);  // cleared together
-  p += align256(sizeof(int) * (cand_tiles(d) + 4));
-  w->tile_cells = reinterpret_cast<int*>(p);
+  p += align256(sizeof(int) * (cand_tiles(d) + kCdStats));
+  w->cells = reinterpret_cast<int2*>(p);
+  w->cell_cap = (int)min_size(cand_tiles(d) * kCdTileLimit, (size_t)1 << 30);
 }
 
 // The rank (of 64 per-thread maxima of a wavefront) whose threshold leaves about
@@ -818,8 +829,8 @@ int cand_any(const TIO* E, const TIO* P, const int* inLen, const int* labLen, fl
                     (4 * sizeof(TIO) - 1)) == 0;
   const size_t lds = cand_lds_bytes(d.V);
   const int tiles = (int)cand_tiles(d);
-  hipLaunchKernelGGL(cand_zero_kernel, dim3((tiles + 4 + 255) / 256), dim3(256), 0, s,
-                     w.tile_fail, tiles + 4);
+  hipLaunchKernelGGL(cand_zero_kernel, dim3((tiles + kCdStats + 255) / 256), dim3(256), 0, s,
+                     w.tile_fail, tiles + kCdStats);
   RNNT_LAUNCH_CHECK("cand_zero_kernel");
   // The sample's utterances first (their lists, their transposed P, one frame in kCdSampleEvery),
   // then the decision; if it is a no, the same sample again with the longer lists, and the
@@ -884,10 +895,9 @@ int cells_any(const TIO* E, const TIO* P, const int* inLen, const int* labLen, f
               int* arg, const Dims& d, void* scratch, hipStream_t s) {
   CandScratch w;
   carve(scratch, d, &w);
-  const dim3 grid(((d.T + kCdTileT - 1) / kCdTileT) * (kCdCellShare / 4),
-                  (d.U + kCdTileU - 1) / kCdTileU, d.B);
-  hipLaunchKernelGGL((cand_cells_kernel<TIO>), grid, dim3(256), 0, s, E, P, best, arg,
-                     w.tile_fail, w.tile_cells, w.stats, d);
+  const int groups = (int)min_size(kCdCellGroups, ((size_t)w.cell_cap + 3) / 4);
+  hipLaunchKernelGGL((cand_cells_kernel<TIO>), dim3(groups), dim3(256), 0, s, E, P, best, arg, w,
+                     d);
   RNNT_LAUNCH_CHECK("cand_cells_kernel");
   return kOk;
 }
@@ -897,12 +907,13 @@ int cells_any(const TIO* E, const TIO* P, const int* inLen, const int* labLen, f
 int maxplus_tile_limit() { return kCdTileLimit; }
 
 // Whether the list path can take this shape at all: a quarter of a row fits the registers a
-// wavefront keeps for it (which also keeps a row and its lists inside a compute unit's LDS), and
-// an offset into one utterance's transposed P fits 31 bits.
+// wavefront keeps for it (which also keeps a row and its lists inside a compute unit's LDS), an
+// offset into one utterance's transposed P fits 31 bits, and so does a count of the cells.
 bool maxplus_lists_possible(const Dims& d) {
   if (d.B == 0 || d.T == 0 || d.U == 0 || d.V < 4) return false;
   if (padded_row(d.V) > 4 * 256 * kCdAheadLong) return false;
   if ((size_t)d.V * cand_uq(d) >= ((size_t)1 << 29)) return false;
+  if ((size_t)d.B * d.T * d.U >= ((size_t)1 << 31)) return false;  // cells are counted in an int
   return true;
 }
 
@@ -926,8 +937,9 @@ size_t maxplus_lists_bytes(const Dims& d) {
   const int Uq = cand_uq(d);
   return align256(sizeof(float) * (size_t)d.B * d.V * Uq) +
          align256(sizeof(int2) * (size_t)d.B * ((d.U + 63) / 64) * kCdStored * 64) +
-         2 * align256(sizeof(int) * (size_t)d.B * d.U) + align256(sizeof(int) * (cand_tiles(d) + 4)) +
-         align256(sizeof(int) * cand_tiles(d) * kCdTileLimit);
+         2 * align256(sizeof(int) * (size_t)d.B * d.U) +
+         align256(sizeof(int) * (cand_tiles(d) + kCdStats)) +
+         align256(sizeof(int2) * min_size(cand_tiles(d) * kCdTileLimit, (size_t)1 << 30));
 }
 
 void maxplus_lists_counters(void* scratch, const Dims& d, const int** tile_fail,
