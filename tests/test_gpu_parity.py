@@ -165,6 +165,79 @@ def test_boundary_at_T2000(V, sigma, ragged):
         assert np.abs(diag - 1.0).max() < 2e-2
 
 
+def minus_inf_case(shape, kind, seed=5):
+    """Scores of -inf as a caller masks them: the blank from the middle of every utterance on
+    (no path reaches the end: cost +inf), one blank score of the predictions, one label score
+    of one frame, one label score of the predictions (no path again)."""
+    B, T, U, V = shape
+    E, P, labels, il, ll = (a.copy() for a in unpack(
+        make_inputs(small_config(B, T, U - 1, V, ragged=True), seed=seed)))
+    il[0], ll[0] = T, U - 1
+    for b in range(B):
+        Tb, Ub = il[b], ll[b] + 1
+        if kind == "blank_tail":
+            E[b, Tb // 2:, 0] = -np.inf
+        elif kind == "blank_p":
+            P[b, Ub // 2, 0] = -np.inf
+        elif kind == "label_cell" and Ub > 1:
+            E[b, Tb // 3, labels[b, (Ub - 1) // 2]] = -np.inf
+        elif kind == "label_row" and Ub > 1:
+            P[b, (Ub - 1) // 2, labels[b, (Ub - 1) // 2]] = -np.inf
+    return E, P, labels, il, ll
+
+
+# U = 1 (first column only), one wavefront, two wavefronts, two blocks of 1024 positions
+@pytest.mark.parametrize("shape", [(2, 12, 1, 8), (3, 40, 9, 16), (2, 150, 101, 24),
+                                   (2, 20, 1100, 6)])
+@pytest.mark.parametrize("kind", ["blank_tail", "blank_p", "label_cell", "label_row"])
+def test_minus_inf_scores_follow_the_reference(shape, kind):
+    """transducer/transducer_cpu.cpp:16-24,43-60: a score of -inf gives alphas of -inf (not a
+    large finite number), an unreachable last cell a cost of +inf, and the backward pass the
+    NaN (inf - inf) and 0 (exp(-inf)) entries the reference produces.  Same bits as the
+    oracle at the transducer.h boundary, infinities and NaN positions included."""
+    E, P, labels, il, ll = minus_inf_case(shape, kind)
+    LN = oracle.log_norms_naive(E, P, il, ll)
+    assert np.isfinite(LN[~np.isnan(LN)]).all()
+    costs_o, alphas_o = oracle.forward(E, P, LN, labels, il, ll)
+    c = DeviceCase(E, P, labels, il, ll)
+    costs, alphas = gpu_forward(c, LN)
+    assert np.array_equal(np.isposinf(costs), np.isposinf(costs_o))
+    assert_same_bits(costs, costs_o, what="costs")
+    assert np.array_equal(np.isneginf(alphas), np.isneginf(alphas_o)), "-inf alphas"
+    assert np.array_equal(np.isnan(alphas), np.isnan(alphas_o)), "cells outside must be untouched"
+    assert_same_bits(alphas, alphas_o, what="alphas")
+    # backward from these alphas (cells outside the lattice cleared, -inf kept)
+    import torch
+    from transducer_amd import capi
+    from util import dev, ptr
+    B, T, U, V = c.dims
+    a_in = np.where(np.isnan(alphas_o), np.float32(0), alphas_o)
+    eg_o, pg_o, lng_o = oracle.backward(E, P, a_in, LN, labels, il, ll)
+    eg = torch.full_like(c.E, float("nan"))
+    pg = torch.full_like(c.P, float("nan"))
+    lng = torch.full((B, T, U), float("nan"), device=c.E.device)
+    d_alphas, d_LN = dev(a_in), dev(LN)
+    capi.call("rnnt_hip_backward", ptr(c.E), ptr(c.P), ptr(eg), ptr(pg), ptr(lng), ptr(d_alphas),
+              ptr(d_LN), ptr(c.labels), ptr(c.il), ptr(c.ll), B, T, U, V, 0, None)
+    torch.cuda.synchronize()
+    for got, want, name in ((lng, lng_o, "lngrads"), (eg, eg_o, "egrads (sparse)"),
+                            (pg, pg_o, "pgrads (sparse)")):
+        got = got.cpu().numpy()
+        assert np.array_equal(np.isnan(got), np.isnan(want)), name + ": NaN positions"
+        assert_same_bits(got, want, what=name)
+    # the whole loss: +inf costs where the oracle has them, finite ones and every finite
+    # gradient entry within the tolerance, NaN where the oracle has NaN
+    if U > 128:  # (a label axis this long is compared end to end in its own test)
+        return
+    want = oracle.loss_and_grads(E, P, labels, il, ll)
+    costs_f, eg_f, pg_f = gpu_loss(c)
+    assert np.array_equal(np.isposinf(costs_f), np.isposinf(want["costs"]))
+    fin = np.isfinite(want["costs"])
+    assert_close(costs_f[fin], want["costs"][fin], what="costs (whole loss)")
+    assert_close(eg_f, want["egrads"], what="egrads (whole loss)")  # (NaN positions included)
+    assert_close(pg_f, want["pgrads"], what="pgrads (whole loss)")
+
+
 @pytest.mark.parametrize("near_ties", [False, True])
 def test_viterbi_at_T2000_is_bit_exact(near_ties):
     cfg = small_config(3, 2000, 100, 64, ragged=True)

@@ -34,6 +34,7 @@ SIGNATURES = {
     "rnnt_hip_check_kernels": (_I, [_F]),
     "rnnt_hip_set_spin_limit": (_I, [_I]),
     "rnnt_hip_set_maxplus_mode": (_I, [_I]),
+    "rnnt_hip_set_fused_grads": (_I, [_I]),
     "rnnt_hip_maxplus_tries_lists": (_I, [_I] * 4),
     "rnnt_hip_maxplus_table": (_I, [_F] * 6 + [_I] * 5 + [_F]),
     "rnnt_hip_chain_floor": (_I, [_I, _I, _F]),

@@ -4,6 +4,7 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <atomic>
 #include <mutex>
 
 #include "../../include/rnnt_hip.h"
@@ -12,6 +13,9 @@
 namespace rnnt {
 
 static thread_local char g_error[512] = "";
+
+// whether the whole-loss backward pass may form both dense gradients in one kernel
+static std::atomic<int> g_fused_grads{0};
 
 int fail(int code, const char* fmt, ...) {
   va_list ap;
@@ -34,11 +38,12 @@ namespace prof {
 
 enum Stage {
   kRowmax, kLse, kSkew, kGather, kAlpha, kUnskew, kWeights, kBeta, kWplanes, kEgrads, kPgrads,
-  kSparse, kMaxplus, kViterbi, kClear, kYplanes, kNumStages
+  kSparse, kMaxplus, kViterbi, kClear, kYplanes, kGrads, kNumStages
 };
 const char* const kNames[kNumStages] = {"rowmax", "lse", "skew", "gather", "alpha", "unskew",
                                         "weights", "beta", "wplanes", "egrads", "pgrads",
-                                        "sparse", "maxplus", "viterbi", "clear", "yplanes"};
+                                        "sparse", "maxplus", "viterbi", "clear", "yplanes",
+                                        "grads"};
 constexpr int kMaxRecords = 8192;
 struct Record { int stage; hipEvent_t begin, end; };
 
@@ -540,6 +545,10 @@ int rnnt_hip_maxplus_tries_lists(int B, int T, int U, int V) {
   return maxplus_uses_lists(make_dims(B, T, U, V, 0)) ? 1 : 0;
 }
 
+int rnnt_hip_set_fused_grads(int mode) {
+  return g_fused_grads.exchange(mode < 0 ? 0 : (mode > 2 ? 2 : mode));
+}
+
 int rnnt_hip_set_maxplus_mode(int mode) {
   if (mode < 0 || mode > 2) return fail(kInvalid, "set_maxplus_mode: mode %d (0, 1 or 2)", mode);
   set_maxplus_mode(mode);
@@ -784,17 +793,26 @@ int rnnt_hip_loss_backward(const float* E, const float* P, const int* labels, co
   // scattered; from V=1000 on folding is level or ahead)
   // (and not with more than 1024 labels: the dense kernel's per-wavefront match list holds
   // that many)
-  const bool fold = labels != nullptr && d.V >= 512 && d.U - 1 <= 1024;
+  const int fused_mode = g_fused_grads.load();
+  const bool use_fused = labels != nullptr && grads_fused_possible(d) &&
+                         (fused_mode == 2 || (fused_mode == 1 && grads_fused_pays(d)));
+  const bool fold = labels != nullptr && (d.V >= 512 || use_fused) && d.U - 1 <= 1024;
   RNNT_STAGE(kWplanes, launch_post_beta(w.planes, w.mE, w.mP, w.Wn, w.Wt,
                                         fold ? w.bsum : nullptr, labels, inLen, labLen, d, s));
   SparseTerms sp;
   if (fold) { sp.dS = w.planes.dS; sp.wE = w.planes.wE; sp.bsum = w.bsum; sp.labels = labels; }
-  RNNT_STAGE(kEgrads, launch_egrads(E, P, w.mE, w.mP, w.Wn, deltas, egrads, inLen, labLen, d, false,
-                                    sp, s));
   // pgrads always takes its blank / label totals in its write-out (the same two fp32 operations
   // the scatter kernel would do afterwards, so the same bits, and no extra launch)
   SparsePTerms spp;
   spp.gB = w.planes.gB; spp.gL = w.planes.gL; spp.labels = labels;
+  if (use_fused) {
+    // one walk over the frames for both gradients: each row of E is read once
+    RNNT_STAGE(kGrads, launch_grads_fused(E, P, w.mE, w.mP, w.Wn, w.Wt, deltas, egrads, pgrads,
+                                          inLen, labLen, d, sp, spp, s));
+    return kOk;
+  }
+  RNNT_STAGE(kEgrads, launch_egrads(E, P, w.mE, w.mP, w.Wn, deltas, egrads, inLen, labLen, d, false,
+                                    sp, s));
   RNNT_STAGE(kPgrads, launch_pgrads(E, P, w.mE, w.mP, w.Wt, deltas, pgrads, inLen, labLen, d, false,
                                     spp, w.psplit, s));
   if (!fold)

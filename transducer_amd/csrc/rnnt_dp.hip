@@ -24,10 +24,14 @@ namespace rnnt {
 namespace {
 
 constexpr float kNegInf = -__builtin_huge_valf();
-// Score of a cell outside the lattice in the alpha walk: far below any alpha, so a log-sum-exp
-// returns the other operand untouched -- as -inf would -- but FINITE, so that two of them do
-// not meet as inf - inf (which only the library path can sort out, and an idle lane would then
-// send its whole wavefront there at every step).
+// Label-move score handed on by a cell outside the lattice in the alpha walk: far below any
+// alpha, so a log-sum-exp returns the other operand untouched -- as -inf would -- but FINITE.
+// The blank-move score of such a cell is -inf; an idle lane therefore forms
+// lse(kOutside, -inf) = kOutside on the fast path, never inf - inf (which only the library path
+// can sort out, and an idle lane would then send its whole wavefront there at every step).
+// A cell INSIDE the lattice never sees this value: its left neighbour is inside too, and the
+// first column is handed -inf (below), so -inf scores of the caller propagate exactly as in
+// the reference (transducer/transducer_cpu.cpp:16-24,43-60).
 constexpr float kOutside = -1.0e30f;
 constexpr float kPosInf = __builtin_huge_valf();
 
@@ -235,10 +239,12 @@ __global__ __launch_bounds__(256) void gather_kernel(const TIO* __restrict__ E,
 
 // ------------------------------------------------------------------ alpha
 // transducer/transducer_cpu.cpp:30-79 (one utterance per wavefront).
-// A cell that has not started yet (t < 0) keeps its -inf hand-over scores, which makes the
-// log-sum-exp return the other operand untouched -- exactly the reference's first-row /
-// first-column special cases.  Cells past the utterance (t >= T_b, u >= U_b) hand -inf on as
-// well and are never read by a valid cell.
+// A cell that has not started yet (t < 0) hands on "nothing" -- -inf upwards (blank move),
+// kOutside to the right (label move) -- which makes the log-sum-exp of a first-row or
+// first-column cell return its one real operand untouched: exactly the reference's special
+// cases (:49-60), also when that operand is -inf (both operands are then -inf and the library
+// path returns -inf).  Cells past the utterance (t >= T_b, u >= U_b) hand on the same and are
+// never read by a valid cell.
 // W > 1: the label positions are dealt to W wavefronts of one workgroup (wavefront w owns
 // positions [64 C w, 64 C (w+1))), because the walk is bound by how fast ONE wavefront issues
 // the ~22 instructions of a cell: a step costs about 30 + 65 C ns.  The only value that crosses
@@ -278,6 +284,7 @@ __global__ __launch_bounds__(64 * W) void alpha_kernel(Planes p, const int* __re
   const int nsteps = Tb + Ub - 1;
   const int ngroups = (nsteps + 3) >> 2;
   const int u0 = u_base + (wave * 64 + lane) * C;
+  const bool first_column = u_base == 0 && wave == 0;  // lane 0 owns the lattice's column u = 0
   const float* gin = (kMulti && ghin) ? ghin + (size_t)b * hand_stride : nullptr;
   float* gout = (kMulti && ghout) ? ghout + (size_t)b * hand_stride : nullptr;
   if (kMulti && gout && threadIdx.x == 0) gout[0] = kOutside;  // nothing enters step 0
@@ -308,7 +315,7 @@ __global__ __launch_bounds__(64 * W) void alpha_kernel(Planes p, const int* __re
     pbv[c] = p.pb[(size_t)b * d.Ua + u0 + c];
     plv[c] = p.pl[(size_t)b * d.Ua + u0 + c];
     // :43 alpha[0,0] = 0: cell (0,0) finds 0 coming up from below and nothing from the left
-    stay[c] = (u0 + c == 0) ? 0.0f : kOutside;
+    stay[c] = (u0 + c == 0) ? 0.0f : kNegInf;
     emit[c] = kOutside;
   }
 
@@ -344,8 +351,16 @@ __global__ __launch_bounds__(64 * W) void alpha_kernel(Planes p, const int* __re
   auto run_group = [&](int g, const Group& cur, auto whole) {
     constexpr bool kWhole = decltype(whole)::value;
     float4 aout[C];
-    float4 hin = {kOutside, kOutside, kOutside, kOutside};
-    if constexpr (kMulti) hin = cur.gh;  // wavefront 0: from the block below (or nothing)
+    // what enters the wavefront's first column from the left: for the lattice's own first
+    // column (u = 0) nothing, which is -inf while its cells are inside the lattice (:49-52 adds
+    // nothing there, so a -inf blank score must come out as -inf) and kOutside once they are
+    // past the last frame (the idle lane's pair is then (kOutside, -inf) again)
+    float4 hin;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) f4set(hin, j, (first_column && 4 * g + j < Tb) ? kNegInf : kOutside);
+    if constexpr (kMulti) {
+      if (gin) hin = cur.gh;  // wavefront 0: from the block below
+    }
     if (W > 1 && wave > 0) {
       wait_for(4 * g + 3);  // the scores entering steps 4g .. 4g+3 left steps 4g-1 .. 4g+2
       hin = *reinterpret_cast<const float4*>(hand_in + 4 * g);
@@ -357,8 +372,7 @@ __global__ __launch_bounds__(64 * W) void alpha_kernel(Planes p, const int* __re
       const int s = 4 * g + j;
       if constexpr (kMulti) gsend[j] = kOutside;
       if (kWhole || s < nsteps) {  // uniform; a step past the last must not touch the scores
-        float from_left = wave_shr1(emit[C - 1], kOutside);
-        if (W > 1 || kMulti) from_left = (lane == 0) ? f4get(hin, j) : from_left;
+        const float from_left = wave_shr1(emit[C - 1], f4get(hin, j));  // lane 0: hin
 #pragma unroll
         for (int c = C - 1; c >= 0; --c) {
           const float left = (c == 0) ? from_left : emit[c - 1];
@@ -375,7 +389,7 @@ __global__ __launch_bounds__(64 * W) void alpha_kernel(Planes p, const int* __re
           // outside the utterance never enters a log-sum-exp (where it would cost the whole
           // wavefront the library path).
           const bool inside = (unsigned)(s - (u0 + c)) < tlim[c];
-          stay[c] = inside ? sb : kOutside;
+          stay[c] = inside ? sb : kNegInf;
           emit[c] = inside ? se : kOutside;
           f4set(aout[c], j, a);
         }

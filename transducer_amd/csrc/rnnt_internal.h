@@ -283,6 +283,14 @@ int launch_pgrads(const float* E, const float* P, const float* mE, const float* 
 
 
 // ---------------------------------------------------------------- launchers (rnnt_grads.hip)
+// Both dense gradients from one walk over the frames (each row of E read once); needs the
+// blank / label terms folded into both write-outs.
+bool grads_fused_possible(const Dims& d);  // the kernel can take this shape
+bool grads_fused_pays(const Dims& d);      // ... and is expected to beat the two contractions
+int launch_grads_fused(const float* E, const float* P, const float* mE, const float* mP,
+                       const float* Wn, const float* Wt, const float* deltas, float* egrads,
+                       float* pgrads, const int* inLen, const int* labLen, const Dims& d,
+                       const SparseTerms& sp, const SparsePTerms& spp, hipStream_t s);
 // Whether one launch covers the label axis.  A longer axis goes slice by slice, the slices adding
 // up in the output array; 16-bit gradients then go through `wide` (fp32 scratch of wide_bytes,
 // at least 32 frames of B * V values), a window of frames at a time, so that each value is still
