@@ -440,10 +440,6 @@ def main():
     ap.add_argument("--maxplus-mode", type=int, default=0, choices=(0, 1, 2),
                     help="best-path workloads: how the table of best labels is built "
                          "(rnnt_hip_set_maxplus_mode: 0 default, 1 every column, 2 lists)")
-    ap.add_argument("--fused-grads", type=int, default=1, choices=(0, 1),
-                    help="loss workloads: both dense gradients from one kernel where the shape "
-                         "allows (1, the library's default) or always the two separate "
-                         "contractions (0); rnnt_hip_set_fused_grads")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one plain elementwise copy of the emissions array (B*T*V*4 "
                          "bytes read, as many written) so that a counter run can scale "
@@ -465,7 +461,6 @@ def main():
     if opt.get("kind") == "viterbi":
         return viterbi_main(args, args.workload, cfg, opt, capi, d, device)
 
-    capi.load().rnnt_hip_set_fused_grads(args.fused_grads)
     B, T, U1, V = cfg.B, cfg.T, cfg.U + 1, cfg.V
     il, ll = d["input_lengths"], d["label_lengths"]
     E = torch.from_numpy(d["emissions"]).to(device)
@@ -586,7 +581,7 @@ def main():
         "dtype": "f32 arithmetic on %s scores, %s gradients" % (io, io) if io else "f32",
         "data": "synthetic",
         "config": {"workload": describe(args.workload, cfg, opt), "seed": args.seed,
-                   "valid_lattice_cells": int(cells), "fused_grads": args.fused_grads},
+                   "valid_lattice_cells": int(cells)},
         "roofline": roofline,
         "whole_step_frac_of_mfma_roofline": round(
             (flops_all / (PEAK_FP32_MATRIX_TFLOPS * 1e12)) / (ms_per_step * 1e-3), 4),

@@ -211,15 +211,13 @@ int rnnt_hip_set_spin_limit(int trips);
  * The labels returned are the same in every mode; the setting is process-wide.  No counterpart
  * in the reference. */
 int rnnt_hip_set_maxplus_mode(int mode);
-/* How rnnt_hip_loss_backward forms the two dense gradients:
- *   1 (default): where the shape allows it and it is expected to pay (2 to 112 label positions,
- *      a vocabulary of 512 or more, at least 192 tiles of 128 columns over the batch) ONE
- *      kernel walks the frames once, reads each row of the emissions once and produces both
- *      gradients from it;
- *   0: always the two separate contractions (each reads the emissions);
- *   2: the one kernel wherever the shape allows it (for tests, which run small shapes).
- * Returns the previous setting; process-wide.  For tests and A/B timings; no counterpart in
- * the reference (which leaves both products to torch.bmm, transducer/torch_binding.py:85-89). */
+/* rnnt_hip_loss_backward forms the two dense gradients with two kernels, each of which reads
+ * the emissions.  A one-kernel form that reads them once (both gradients from one walk over
+ * the frames, transducer_amd/csrc/rnnt_fused.hip) exists for 2 to 112 label positions but is
+ * SWITCHED OFF: it measured level with the two kernels and then faulted at the headline shape
+ * for a reason not yet found.  mode 0 (the two kernels) returns the previous setting, 0; any
+ * other mode is refused with -1 and changes nothing.  No counterpart in the reference (which
+ * leaves both products to torch.bmm, transducer/torch_binding.py:85-89). */
 int rnnt_hip_set_fused_grads(int mode);
 /* 1 if a best-path call of this shape starts on the list path under the current mode (it may
  * still turn back after looking at a sample of the cells), else 0. */

@@ -14,7 +14,13 @@ from transducer_amd import capi
 from transducer_amd.synthetic import make_inputs, small_config
 from util import DeviceCase, assert_close, assert_same_bits, gpu_log_norms, gpu_loss, violations
 
-pytestmark = pytest.mark.gpu
+# Switched off with the code path: at the headline shape the fused kernel left NaN entries in
+# pgrads on one input and made an illegal memory access on another (these small shapes passed),
+# and the cause has not been found.  rnnt_hip_set_fused_grads refuses every mode but 0; the tests
+# stay for the day the kernel is switched on again.
+pytestmark = [pytest.mark.gpu,
+              pytest.mark.skip(reason="fused gradient kernel switched off: unexplained GPU "
+                                      "fault at the headline shape")]
 
 KEYS = ("emissions", "predictions", "labels", "input_lengths", "label_lengths")
 
@@ -56,9 +62,11 @@ def test_fused_walk_equals_the_two_contractions_and_the_oracle(shape):
     costs0, eg0, pg0 = loss_in_mode(c, 0, deltas)
     costs2, eg2, pg2 = loss_in_mode(c, 2, deltas)
     assert_same_bits(costs2, costs0, what="costs")
-    if V >= 512:
+    if V >= 512 and len(np.unique(labels[0])) == labels.shape[1]:
         assert_same_bits(eg2, eg0, what="egrads, fused against separate")
     else:
+        # (a label that repeats inside an utterance puts two terms on one entry, which the two
+        # forms add in a different order)
         # (below 512 columns the separate path adds the blank / label terms after the dense
         # kernel, delta * dense + delta * term instead of delta * (dense + term): those entries
         # round differently)
@@ -70,7 +78,7 @@ def test_fused_walk_equals_the_two_contractions_and_the_oracle(shape):
     # rounding of the dense part: the scale is the row's largest entry)
     err = np.abs(pg2.astype(np.float64) - pg0)
     scale = np.abs(pg0).max(axis=-1, keepdims=True)
-    assert (err <= 4 * np.spacing(np.abs(pg0)) + 1e-6 * scale).all(), \
+    assert (err <= 4 * np.spacing(np.abs(pg0)) + 1e-5 * scale).all(), \
         "pgrads: fused %g from separate at worst" % err.max()
     want = oracle_on_device_log_norms(E, P, labels, il, ll, c)
     sc = deltas[:, None, None]

@@ -17,7 +17,7 @@ CSRC = os.path.join(HERE, "csrc")
 INCLUDE = os.path.join(ROOT, "include")
 
 HIP_SOURCES = ["rnnt_capi.hip", "rnnt_dp.hip", "rnnt_prep.hip", "rnnt_grads.hip", "rnnt_lse.hip",
-               "rnnt_cand.hip"]
+               "rnnt_cand.hip", "rnnt_fused.hip"]
 
 # -ffp-contract=off: the lattice recursions must round like the reference's scalar code.
 # packed-fp32 instructions are disabled for the device pass (the host pass does not know the

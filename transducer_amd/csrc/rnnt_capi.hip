@@ -179,6 +179,7 @@ int log_norms_stages(const float* E, const float* P, float* mE, float* mP, float
 struct LossWorkspace {
   Planes planes;
   float *mE, *mP, *LN, *Wn, *Wt, *bsum;
+  WImages img;  // shares its memory with Wn / Wt: a backward call writes one form or the other
   void* lse_scratch;
   void* psplit;  // pgrads_split_bytes(d) bytes, or null
 };
@@ -198,14 +199,23 @@ size_t loss_workspace_layout(const Dims& d, void* base, LossWorkspace* w) {
   float* mE = take(sizeof(float) * (size_t)d.B * d.T);
   float* mP = take(sizeof(float) * (size_t)d.B * d.U);
   float* LN = take(btu);
-  const size_t wb = sizeof(float) * (size_t)d.B * wplane_tw(d.T) * wplane_up(d.U);
-  float* Wn = take(wb);
-  float* Wt = take(wb);
+  // W for the gradient kernels: two fp32 planes, or (fused kernel) the two slab images of bf16
+  // pieces, in the same memory
+  const size_t wb = align_up(sizeof(float) * (size_t)d.B * wplane_tw(d.T) * wplane_up(d.U));
+  const bool images = grads_fused_possible(d);
+  const size_t ie = images ? align_up(WImages::e_bytes(d.B, wplane_tw(d.T))) : 0;
+  const size_t ip = images ? align_up(WImages::p_bytes(d.B, wplane_tw(d.T))) : 0;
+  float* Wn = take(2 * wb > ie + ip ? 2 * wb : ie + ip);
+  float* Wt = Wn ? reinterpret_cast<float*>(reinterpret_cast<char*>(Wn) + wb) : nullptr;
   float* bsum = take(sizeof(float) * (size_t)d.B * d.T);
   void* ys = take(lse_scratch_bytes(d));  // forward only
   void* ps = take(pgrads_split_bytes(d));  // backward only
   if (base) {
     w->mE = mE; w->mP = mP; w->LN = LN; w->Wn = Wn; w->Wt = Wt; w->bsum = bsum;
+    if (images) {
+      w->img.e = reinterpret_cast<unsigned*>(Wn);
+      w->img.p = reinterpret_cast<unsigned*>(reinterpret_cast<char*>(Wn) + ie);
+    }
     w->lse_scratch = lse_scratch_bytes(d) ? ys : nullptr;
     w->psplit = pgrads_split_bytes(d) ? ps : nullptr;
   }
@@ -546,7 +556,8 @@ int rnnt_hip_maxplus_tries_lists(int B, int T, int U, int V) {
 }
 
 int rnnt_hip_set_fused_grads(int mode) {
-  return g_fused_grads.exchange(mode < 0 ? 0 : (mode > 2 ? 2 : mode));
+  if (mode != 0) return -1;  // switched off, see rnnt_hip_loss_backward
+  return g_fused_grads.exchange(0);
 }
 
 int rnnt_hip_set_maxplus_mode(int mode) {
@@ -793,12 +804,17 @@ int rnnt_hip_loss_backward(const float* E, const float* P, const int* labels, co
   // scattered; from V=1000 on folding is level or ahead)
   // (and not with more than 1024 labels: the dense kernel's per-wavefront match list holds
   // that many)
+  // The one-kernel form of the two gradients (rnnt_fused.hip) is switched off: at the headline
+  // shape it left NaN entries in pgrads on one input and made an illegal memory access on
+  // another, and the cause has not been found.  rnnt_hip_set_fused_grads refuses to switch it
+  // on, so use_fused is always false here.
   const int fused_mode = g_fused_grads.load();
   const bool use_fused = labels != nullptr && grads_fused_possible(d) &&
                          (fused_mode == 2 || (fused_mode == 1 && grads_fused_pays(d)));
   const bool fold = labels != nullptr && (d.V >= 512 || use_fused) && d.U - 1 <= 1024;
   RNNT_STAGE(kWplanes, launch_post_beta(w.planes, w.mE, w.mP, w.Wn, w.Wt,
-                                        fold ? w.bsum : nullptr, labels, inLen, labLen, d, s));
+                                        fold ? w.bsum : nullptr, labels, inLen, labLen, d, s,
+                                        use_fused ? w.img : WImages()));
   SparseTerms sp;
   if (fold) { sp.dS = w.planes.dS; sp.wE = w.planes.wE; sp.bsum = w.bsum; sp.labels = labels; }
   // pgrads always takes its blank / label totals in its write-out (the same two fp32 operations
@@ -807,7 +823,7 @@ int rnnt_hip_loss_backward(const float* E, const float* P, const int* labels, co
   spp.gB = w.planes.gB; spp.gL = w.planes.gL; spp.labels = labels;
   if (use_fused) {
     // one walk over the frames for both gradients: each row of E is read once
-    RNNT_STAGE(kGrads, launch_grads_fused(E, P, w.mE, w.mP, w.Wn, w.Wt, deltas, egrads, pgrads,
+    RNNT_STAGE(kGrads, launch_grads_fused(E, P, w.mE, w.mP, w.img, deltas, egrads, pgrads,
                                           inLen, labLen, d, sp, spp, s));
     return kOk;
   }

@@ -18,6 +18,7 @@
 
 #include "rnnt_internal.h"
 #include "rnnt_libm.h"
+#include "rnnt_split.h"
 
 namespace rnnt {
 
@@ -827,11 +828,13 @@ __device__ __forceinline__ void blank_sums_block(const Planes& p, float* __restr
 
 // The same from the skewed planes the lattice kernels leave behind (dalpha and LN stored
 // [u][t+u]): no un-skewed copy of dalpha is needed first.  Same arithmetic, same bits.
+// With `img` the block leaves its 64 frames x 64 label positions of W as bf16 pieces instead, in
+// the two slab images the fused gradient kernel copies into LDS as they are (WImages).
 __device__ __forceinline__ void wplanes_skewed_block(
     const float* __restrict__ dS, const float* __restrict__ lnS, const float* __restrict__ mE,
     const float* __restrict__ mP, float* __restrict__ Wn, float* __restrict__ Wt,
     const int* __restrict__ inLen, const int* __restrict__ labLen, const Dims& d, int Up, int Tw,
-    float (*tile)[65], int bx, int by, int b) {
+    float (*tile)[65], int bx, int by, int b, const WImages& img) {
   const int t0 = bx * 64, u0 = by * 64;
   int Tb, Ub;
   utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
@@ -844,14 +847,49 @@ __device__ __forceinline__ void wplanes_skewed_block(
       const size_t o = plane_row(d, b, u) + t + u;
       w = dS[o] * expf((mE[(size_t)b * d.T + t] + mP[(size_t)b * d.U + u]) - lnS[o]);
     }
-    tile[ty + 4 * i][tx] = w;
-    if (t < Tw && u < Up) Wt[((size_t)b * Up + u) * Tw + t] = w;
+    tile[ty + 4 * i][tx] = w;  // [label position][frame]
+    if (!img.e && t < Tw && u < Up) Wt[((size_t)b * Up + u) * Tw + t] = w;
   }
   __syncthreads();
+  if (!img.e) {
 #pragma unroll
-  for (int i = 0; i < 16; ++i) {
-    const int t = t0 + ty + 4 * i, u = u0 + tx;
-    if (t < Tw && u < Up) Wn[((size_t)b * Tw + t) * Up + u] = tile[tx][ty + 4 * i];
+    for (int i = 0; i < 16; ++i) {
+      const int t = t0 + ty + 4 * i, u = u0 + tx;
+      if (t < Tw && u < Up) Wn[((size_t)b * Tw + t) * Up + u] = tile[tx][ty + 4 * i];
+    }
+    return;
+  }
+  const int ntile = Tw >> 5;
+  // frames x label positions (the egrads operand): pairs of neighbouring label positions
+#pragma unroll
+  for (int k = 0; k < 8; ++k) {
+    const int id = k * 256 + threadIdx.x, tl = id >> 5, j = id & 31;
+    const int u = u0 + 2 * j;
+    if (u < WImages::kCols) {
+      unsigned ph, pm, pl;
+      split_pair(tile[2 * j][tl], tile[2 * j + 1][tl], ph, pm, pl);
+      unsigned* dst = img.e + ((size_t)b * ntile + ((t0 + tl) >> 5)) * (3 * WImages::kEPlane) +
+                      ((t0 + tl) & 31) * (WImages::kCols / 2) + (u >> 1);
+      dst[0] = ph;
+      dst[WImages::kEPlane] = pm;
+      dst[2 * WImages::kEPlane] = pl;
+    }
+  }
+  // label positions x frames (the pgrads operand), the frames of a slab in the order the fused
+  // kernel feeds them to the matrix instruction: slot = frame with bits 2 and 3 swapped (its own
+  // inverse; pairs of neighbouring frames stay pairs)
+#pragma unroll
+  for (int k = 0; k < 8; ++k) {
+    const int id = k * 256 + threadIdx.x, ul = id >> 5, q = id & 31;
+    const int sel = q >> 4, slot = 2 * (q & 15);
+    const int f = (slot & 16) | ((slot & 4) << 1) | ((slot & 8) >> 1) | (slot & 2);
+    unsigned ph, pm, pl;
+    split_pair(tile[ul][32 * sel + f], tile[ul][32 * sel + f + 1], ph, pm, pl);
+    unsigned* dst = img.p + ((size_t)b * ntile + (t0 >> 5) + sel) * (3 * WImages::kPPlane) +
+                    (u0 + ul) * 16 + (slot >> 1);
+    dst[0] = ph;
+    dst[WImages::kPPlane] = pm;
+    dst[2 * WImages::kPPlane] = pl;
   }
 }
 
@@ -869,13 +907,13 @@ __global__ __launch_bounds__(256) void post_beta_kernel(Planes p, const float* _
                                                         const int* __restrict__ inLen,
                                                         const int* __restrict__ labLen, Dims d,
                                                         int Up, int Tw, int wx, int wy, int nw,
-                                                        int sx) {
+                                                        int sx, WImages img) {
   __shared__ float tile[64][65];
   const int n = blockIdx.x;
   if (n < nw) {
     const int b = n / (wx * wy), r = n - b * (wx * wy);
     wplanes_skewed_block(p.dS, p.lnS, mE, mP, Wn, Wt, inLen, labLen, d, Up, Tw, tile, r % wx,
-                         r / wx, b);
+                         r / wx, b, img);
   } else {
     const int m = n - nw;
     blank_sums_block(p, bsum, labels, inLen, labLen, d, m % sx, m / sx);
@@ -1648,13 +1686,15 @@ int launch_sparse(const Planes& p, float* egrads, float* pgrads, const int* labe
 
 int launch_post_beta(const Planes& p, const float* mE, const float* mP, float* Wn, float* Wt,
                      float* bsum, const int* labels, const int* inLen, const int* labLen,
-                     const Dims& d, hipStream_t s) {
+                     const Dims& d, hipStream_t s, const WImages& img) {
   if (d.B == 0 || d.T == 0 || d.U == 0) return kOk;
   const int Up = wplane_up(d.U), Tw = wplane_tw(d.T);
+  if (img.e && Up > WImages::kCols)
+    return fail(kInvalid, "W images hold at most %d label positions", WImages::kCols);
   const int wx = Tw / 64, wy = (Up + 63) / 64, nw = wx * wy * d.B;
   const int sx = (d.T + 255) / 256, ns = bsum ? sx * d.B : 0;
   hipLaunchKernelGGL(post_beta_kernel, dim3(nw + ns), dim3(256), 0, s, p, mE, mP, Wn, Wt, bsum,
-                     labels, inLen, labLen, d, Up, Tw, wx, wy, nw, sx);
+                     labels, inLen, labLen, d, Up, Tw, wx, wy, nw, sx, img);
   RNNT_LAUNCH_CHECK("post_beta_kernel");
   return kOk;
 }

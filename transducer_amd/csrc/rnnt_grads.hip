@@ -22,38 +22,14 @@
 #include "rnnt_internal.h"
 #include "rnnt_io.h"
 #include "rnnt_split.h"
+#include "rnnt_grads.h"
 
 namespace rnnt {
 
 namespace {
 
-constexpr float kNegInf = -__builtin_huge_valf();
-constexpr float kLog2e = 1.44269504088896340736f;
-
-// exp(e - m) for a reference m that is used for many e: m comes in already multiplied by log2(e)
-// (once per frame, as the slab is staged), so an exponential is one fused multiply-add and one
-// v_exp_f32 instead of a subtraction, a multiplication and the v_exp_f32.  Against exp(e - m) the
-// result carries one more relative error of 2^-24 |m log2 e| ln 2, the same for every e that
-// shares m: 2e-7 at |m| = 4, far inside the gradients' tolerance.
-__device__ inline float exp_minus_scaled(float e, float m_log2e) {
-  return __builtin_amdgcn_exp2f(__builtin_fmaf(e, kLog2e, -m_log2e));
-}
-
-
-__device__ inline float f4at(const float4& v, int q) {
-  return q == 0 ? v.x : (q == 1 ? v.y : (q == 2 ? v.z : v.w));
-}
 
 // ------------------------------------------------------------------ egrads
-constexpr int kEsMaxS = 7;               // steps of 16 label positions kept in registers
-constexpr int kEsPitch = 16 * kEsMaxS + 8;  // LDS row pitch of a W-slab plane in halfwords (240 B:
-                                            // 16-byte reads of 8 consecutive rows spread over all banks)
-constexpr int kEsPlane = 32 * kEsPitch;
-constexpr int kEsPrefetch = 2;          // labels per 32-column block whose sparse terms are prefetched
-constexpr int kMaxLabels = 1024;        // labels whose terms the egrads write-out can fold in
-
-// Row of the 32x32 output block that register r of lane-half h holds.
-__device__ inline int mfma_row(int r, int h) { return 8 * (r >> 2) + 4 * h + (r & 3); }
 
 // Which of two register sets a tile of the egrads walk works on (chosen at compile time).
 __device__ __forceinline__ float (&pick_set(std::true_type, float (&a)[16], float (&)[16]))[16] {
@@ -411,17 +387,6 @@ __global__ __launch_bounds__(256, 2) void egrads_stream_kernel(
 }
 
 // ------------------------------------------------------------------ pgrads
-// W^T slab in LDS: three bf16 planes of 128 rows (u) x 32 frames, row pitch 40 halfwords (80 B:
-// the 16-byte fragment reads of 8 consecutive rows fall into distinct bank groups).
-constexpr int kPsPitch = 40;
-constexpr int kPsPlane = 128 * kPsPitch;
-constexpr int kPsFlush = 8;  // slabs of 32 frames between two flushes of the running sums
-
-// Blank / label terms of the 128 rows of one tile, staged in LDS for the write-out.
-struct PRowTerms {
-  float gB[128], gL[128];
-  int label[128];
-};
 
 // Splitting a tile's frames over several workgroups (small grids: one utterance with a small
 // vocabulary is a single tile, whose workgroup would walk all frames alone).  Workgroup c of
@@ -697,426 +662,6 @@ __global__ __launch_bounds__(256, 2) void pgrads_stream_kernel(
 #undef RNNT_PG_TILE
 }
 
-// ------------------------------------------------------------------ egrads + pgrads in one walk
-// The two contractions above give a wavefront the same unit of work -- 32 columns v of one
-// utterance, all of its frames, 32 at a time -- and both need X = exp(E - mE) of the 32 x 32 slab
-// of E they just loaded.  Here one wavefront does both: the slab of E is read once and turned
-// into X once; X scales the finished egrads block on its way out (lane = column, registers = the
-// block's rows) and, split into its three pieces, is the B operand of the pgrads products.  The
-// matrix instruction sums over k in any order as long as both operands agree on it, so the
-// frames of a slab are fed to the pgrads products in the order the egrads block holds them
-// (slot 16 s + 8 h + i of the k axis = frame 16 s + 8 (i >> 2) + 4 h + (i & 3)) and the W^T slab
-// is laid out in LDS in that same order: X is never exchanged between lanes.
-// Nothing is shared between wavefronts beyond what the two kernels above share (the two W slabs
-// in LDS, one barrier per slab).  Registers: the Y pieces (84), pgrads sums at both levels (128),
-// the egrads block, X and the staging: one wavefront per SIMD with the whole register file; a
-// slab's emissions are requested one slab ahead to make up for the second wavefront.
-// Same additions as the two kernels above (six piece products per block, pgrads' running sums
-// moved into the second level every kPsFlush slabs).
-struct FusedLds {
-  unsigned short Ae[2][3][kEsPlane];     // W slab, frames x label positions (egrads' A operand)
-  unsigned short Ap[2][3][kPsPlane];     // W^T slab, label positions x frames (pgrads' A operand)
-  float Ms[2][32];                       // mE * log2(e) of the slab's frames
-  float Strip[4][32];                    // per wavefront: sparse terms of egrads
-  unsigned short Match[4][kMaxLabels];   // per wavefront: label positions whose label is one of
-                                         // its 32 columns
-  PRowTerms Rt;
-};
-
-// slot of frame f (0..31 inside a slab) on the k axis of the pgrads products
-__device__ inline int fused_slot(int f) {
-  return (f & 16) | ((f & 4) << 1) | ((f & 8) >> 1) | (f & 3);
-}
-
-template <int NS, int NMB, typename TIO>
-__device__ __forceinline__ void fused_walk(
-    const TIO* __restrict__ E, const TIO* __restrict__ P, const float* __restrict__ mE,
-    const float* __restrict__ mP, const float* __restrict__ Wn, const float* __restrict__ Wt,
-    const float* __restrict__ deltas, TIO* __restrict__ egrads, TIO* __restrict__ pgrads,
-    FusedLds& L, const Dims& d, int Up, int Tw, int b, int Tb, int Ub, const SparseTerms& sp,
-    int nmatch) {
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, h = lane >> 5;
-  const int wave_col0 = blockIdx.x * 128 + wave * 32;
-  const int vcol = wave_col0 + l32;
-  const bool vok = vcol < d.V;
-  const int vc = vok ? vcol : d.V - 1;
-  const bool cols_full = wave_col0 + 32 <= d.V;
-  const unsigned short* match = L.Match[wave];
-  const int blank_lane = (d.blank >= wave_col0 && d.blank < wave_col0 + 32) ? d.blank - wave_col0 : -1;
-  const int ntiles = (d.T + 31) >> 5;
-  const int tile_valid = (Tb + 31) >> 5;  // >= 1: utterances without frames never get here
-  const float delta = deltas ? deltas[b] : 1.0f;
-  const TIO* Eb = E + (size_t)b * d.T * d.V;
-  TIO* eout = egrads + (size_t)b * d.T * d.V;
-  const float* mEb = mE + (size_t)b * d.T;
-  const TIO* Pb = P + (size_t)b * d.U * d.V;
-  const float* mPb = mP + (size_t)b * d.U;
-
-  // Y fragments (egrads' B operand): step s holds label positions 16 s + 8 h + i
-  Frag3 Yf[NS];
-  {
-    float praw[NS][8], mraw[NS][8];
-#pragma unroll
-    for (int s = 0; s < NS; ++s)
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const int u = 16 * s + 8 * h + i;
-        const int uc = u < Ub ? u : 0;
-        praw[s][i] = ldf(Pb + (size_t)uc * d.V + vc);
-        mraw[s][i] = mPb[uc];
-      }
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int s = 0; s < NS; ++s) {
-      float y[8];
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const int u = 16 * s + 8 * h + i;
-        const float e = __expf(praw[s][i] - mraw[s][i]);
-        y[i] = (u < Ub && vok) ? e : 0.0f;
-      }
-      Yf[s] = split8(y);
-    }
-  }
-
-  // staging of the two W slabs of a frame tile (each split into pieces on its way into LDS)
-  const int up4 = Up >> 2, cw4 = min(Up, 16 * kEsMaxS) >> 2;
-  const int nvec = 32 * cw4;
-  int e_lds[4], e_src[4];
-  bool e_ok[4];
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int idx = tid + 256 * i;
-    e_ok[i] = idx < nvec;
-    const int ic = e_ok[i] ? idx : nvec - 1;
-    e_src[i] = (ic / cw4) * up4 + ic % cw4;
-    e_lds[i] = e_ok[i] ? (idx / cw4) * kEsPitch + 4 * (idx % cw4) : 0;
-  }
-  const int arow = tid >> 3, ac4 = tid & 7;  // W^T rows arow + 32 i, frames 4 ac4 .. 4 ac4 + 3
-  const int p_lds = arow * kPsPitch + fused_slot(4 * ac4);
-  const float* p_src[NMB];
-#pragma unroll
-  for (int i = 0; i < NMB; ++i)
-    p_src[i] = Wt + ((size_t)b * Up + min(arow + 32 * i, Up - 1)) * Tw + 4 * ac4;
-  struct Staged {
-    float4 e[4];
-    float4 p[NMB];
-    float m;
-  };
-  auto fetch = [&](int ti) -> Staged {
-    Staged s;
-    const float4* src =
-        reinterpret_cast<const float4*>(Wn + ((size_t)b * Tw + (size_t)ti * 32) * Up);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) s.e[i] = src[e_src[i]];
-#pragma unroll
-    for (int i = 0; i < NMB; ++i) s.p[i] = *reinterpret_cast<const float4*>(p_src[i] + ti * 32);
-    s.m = mEb[min(ti * 32 + (tid & 31), Tb - 1)];
-    return s;
-  };
-  auto stage = [&](int buf, const Staged& s) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      uint2 ph, pm, pl;
-      split_pair(s.e[i].x, s.e[i].y, ph.x, pm.x, pl.x);
-      split_pair(s.e[i].z, s.e[i].w, ph.y, pm.y, pl.y);
-      if (e_ok[i]) {
-        *reinterpret_cast<uint2*>(&L.Ae[buf][0][e_lds[i]]) = ph;
-        *reinterpret_cast<uint2*>(&L.Ae[buf][1][e_lds[i]]) = pm;
-        *reinterpret_cast<uint2*>(&L.Ae[buf][2][e_lds[i]]) = pl;
-      }
-    }
-#pragma unroll
-    for (int i = 0; i < NMB; ++i) {
-      uint2 ph, pm, pl;
-      split_pair(s.p[i].x, s.p[i].y, ph.x, pm.x, pl.x);
-      split_pair(s.p[i].z, s.p[i].w, ph.y, pm.y, pl.y);
-      const int o = p_lds + 32 * i * kPsPitch;
-      *reinterpret_cast<uint2*>(&L.Ap[buf][0][o]) = ph;
-      *reinterpret_cast<uint2*>(&L.Ap[buf][1][o]) = pm;
-      *reinterpret_cast<uint2*>(&L.Ap[buf][2][o]) = pl;
-    }
-    if (tid < 32) L.Ms[buf][tid] = s.m * kLog2e;
-  };
-
-  // the first kEsPrefetch matches of the folded label terms, resolved once
-  int mu[kEsPrefetch], mc[kEsPrefetch];
-#pragma unroll
-  for (int i = 0; i < kEsPrefetch; ++i) {
-    mu[i] = i < nmatch ? match[i] : 0;
-    mc[i] = i < nmatch ? label_at(sp.labels, d, b, mu[i]) - wave_col0 : -1;
-  }
-
-  const unsigned lane_off = (unsigned)(4 * h) * (unsigned)d.V + (unsigned)vcol;
-  auto load_e = [&](int ti, float (&e)[16]) __attribute__((always_inline)) {
-    const int t0 = ti * 32;
-    if (cols_full && (t0 + 32 <= Tb)) {
-      const TIO* Etile = Eb + (size_t)t0 * d.V;
-#pragma unroll
-      for (int r = 0; r < 16; ++r)
-        e[r] = ldf(Etile + (lane_off + (unsigned)(8 * (r >> 2) + (r & 3)) * (unsigned)d.V));
-    } else {
-      // rows past the utterance are read from its last frame: masked on the way out of egrads,
-      // multiplied by the zeros of W^T in pgrads
-#pragma unroll
-      for (int r = 0; r < 16; ++r)
-        e[r] = ldf(Eb + (size_t)min(t0 + mfma_row(r, h), Tb - 1) * d.V + vc);
-    }
-  };
-
-  floatx16 pacc[NMB], ptot[NMB];
-#pragma unroll
-  for (int mb = 0; mb < NMB; ++mb)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) pacc[mb][r] = ptot[mb][r] = 0.0f;
-
-  int cur = 0;
-  stage(0, fetch(0));
-  __syncthreads();
-
-  // One frame tile: `evc` holds its emissions, `evn` receives the next tile's.
-  auto tile = [&](int ti, float (&evc)[16], float (&evn)[16]) __attribute__((always_inline)) {
-    const int t0 = ti * 32;
-    const int tnext = min(ti + 1, tile_valid - 1);
-    const Staged nxt = fetch(tnext);  // (the last tile re-reads its own: no branch around loads)
-    load_e(tnext, evn);
-    const bool interior = cols_full && (t0 + 32 <= Tb);
-    TIO* Otile = eout + (size_t)t0 * d.V;
-    float sd[kEsPrefetch], sw[kEsPrefetch], sbl = 0.0f;
-    if (nmatch > 0 || blank_lane >= 0) {
-      const int tr = min(t0 + l32, Tb - 1);
-#pragma unroll
-      for (int i = 0; i < kEsPrefetch; ++i) {
-        const size_t o = plane_row(d, b, mu[i]) + tr + mu[i];
-        sd[i] = sp.dS[o + d.Dp + 1];
-        sw[i] = sp.wE[o];
-      }
-      if (blank_lane >= 0) sbl = sp.bsum[(size_t)b * d.T + tr];
-    }
-    // X of this tile: register r = frame mfma_row(r, h) of column l32
-    float x[16];
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      const float4 m4 = *reinterpret_cast<const float4*>(&L.Ms[cur][8 * g + 4 * h]);
-#pragma unroll
-      for (int k = 0; k < 4; ++k) x[4 * g + k] = exp_minus_scaled(evc[4 * g + k], f4at(m4, k));
-    }
-    Frag3 xb[2];
-    {
-      float lo[8], hi[8];
-#pragma unroll
-      for (int i = 0; i < 8; ++i) { lo[i] = x[i]; hi[i] = x[8 + i]; }
-      xb[0] = split8(lo);
-      xb[1] = split8(hi);
-    }
-    floatx16 acc, acc2;
-#pragma unroll
-    for (int r = 0; r < 16; ++r) acc[r] = acc2[r] = 0.0f;
-    __builtin_amdgcn_sched_barrier(0);
-    {
-      // egrads: W slab (rows = frames) x Y
-      const unsigned short* arow_e = &L.Ae[cur][0][l32 * kEsPitch + 8 * h];
-#pragma unroll
-      for (int s = 0; s < NS; ++s) {
-        const uint4 ah = *reinterpret_cast<const uint4*>(arow_e + 16 * s);
-        const uint4 am = *reinterpret_cast<const uint4*>(arow_e + kEsPlane + 16 * s);
-        const uint4 al = *reinterpret_cast<const uint4*>(arow_e + 2 * kEsPlane + 16 * s);
-        acc = mfma_bf16(al, Yf[s].h, acc);
-        acc2 = mfma_bf16(ah, Yf[s].l, acc2);
-        acc = mfma_bf16(am, Yf[s].m, acc);
-        acc2 = mfma_bf16(am, Yf[s].h, acc2);
-        acc = mfma_bf16(ah, Yf[s].m, acc);
-        acc2 = mfma_bf16(ah, Yf[s].h, acc2);
-      }
-      // pgrads: W^T slab (rows = label positions) x X
-#pragma unroll
-      for (int s = 0; s < 2; ++s) {
-        uint4 ah[NMB], am[NMB], al[NMB];
-#pragma unroll
-        for (int mb = 0; mb < NMB; ++mb) {
-          const int o = (32 * mb + l32) * kPsPitch + 16 * s + 8 * h;
-          ah[mb] = *reinterpret_cast<const uint4*>(&L.Ap[cur][0][o]);
-          am[mb] = *reinterpret_cast<const uint4*>(&L.Ap[cur][1][o]);
-          al[mb] = *reinterpret_cast<const uint4*>(&L.Ap[cur][2][o]);
-        }
-#pragma unroll
-        for (int mb = 0; mb < NMB; ++mb) pacc[mb] = mfma_bf16(al[mb], xb[s].h, pacc[mb]);
-#pragma unroll
-        for (int mb = 0; mb < NMB; ++mb) pacc[mb] = mfma_bf16(ah[mb], xb[s].l, pacc[mb]);
-#pragma unroll
-        for (int mb = 0; mb < NMB; ++mb) pacc[mb] = mfma_bf16(am[mb], xb[s].m, pacc[mb]);
-#pragma unroll
-        for (int mb = 0; mb < NMB; ++mb) pacc[mb] = mfma_bf16(am[mb], xb[s].h, pacc[mb]);
-#pragma unroll
-        for (int mb = 0; mb < NMB; ++mb) pacc[mb] = mfma_bf16(ah[mb], xb[s].m, pacc[mb]);
-#pragma unroll
-        for (int mb = 0; mb < NMB; ++mb) pacc[mb] = mfma_bf16(ah[mb], xb[s].h, pacc[mb]);
-      }
-    }
-    float v[16];
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const float y = x[r] * (acc[r] + acc2[r]);
-      v[r] = (interior || t0 + mfma_row(r, h) < Tb) ? y : 0.0f;
-    }
-    if (nmatch > 0 || blank_lane >= 0) {  // uniform per wavefront, and rare
-      const bool row_ok = t0 + l32 < Tb;
-      float* strip = &L.Strip[wave][0];
-      auto apply = [&](float term, int col, float sign) {
-        if (h == 0) strip[l32] = term;
-        if (l32 == col) {
-#pragma unroll
-          for (int g = 0; g < 4; ++g) {
-            const float4 q = *reinterpret_cast<const float4*>(&strip[8 * g + 4 * h]);
-            v[4 * g + 0] += sign * q.x;
-            v[4 * g + 1] += sign * q.y;
-            v[4 * g + 2] += sign * q.z;
-            v[4 * g + 3] += sign * q.w;
-          }
-        }
-      };
-#pragma unroll
-      for (int i = 0; i < kEsPrefetch; ++i)
-        if (i < nmatch) apply(row_ok ? sd[i] * sw[i] : 0.0f, mc[i], -1.0f);
-      for (int i = kEsPrefetch; i < nmatch; ++i) {
-        const int u = match[i];
-        const size_t o = plane_row(d, b, u) + min(t0 + l32, Tb - 1) + u;
-        apply(row_ok ? sp.dS[o + d.Dp + 1] * sp.wE[o] : 0.0f,
-              label_at(sp.labels, d, b, u) - wave_col0, -1.0f);
-      }
-      if (blank_lane >= 0) apply(row_ok ? sbl : 0.0f, blank_lane, 1.0f);
-    }
-    if (interior) {
-#pragma unroll
-      for (int r = 0; r < 16; ++r)
-        stf(Otile + (lane_off + (unsigned)(8 * (r >> 2) + (r & 3)) * (unsigned)d.V), delta * v[r]);
-    } else {
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int t = t0 + mfma_row(r, h);
-        if (t < d.T && vok) stf(eout + (size_t)t * d.V + vcol, delta * v[r]);
-      }
-    }
-    if ((ti + 1) % kPsFlush == 0) {
-#pragma unroll
-      for (int mb = 0; mb < NMB; ++mb)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) { ptot[mb][r] += pacc[mb][r]; pacc[mb][r] = 0.0f; }
-    }
-    stage(cur ^ 1, nxt);
-    __syncthreads();
-    cur ^= 1;
-  };
-  float evA[16], evB[16];
-  load_e(0, evA);
-  for (int ti = 0; ti < tile_valid; ti += 2) {
-    tile(ti, evA, evB);
-    if (ti + 1 < tile_valid) tile(ti + 1, evB, evA);
-  }
-
-  // frames past the utterance: egrads is exactly zero there
-  for (int ti = tile_valid; ti < ntiles; ++ti) {
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int t = ti * 32 + mfma_row(r, h);
-      if (t < d.T && vok) stf(eout + (size_t)t * d.V + vcol, 0.0f);
-    }
-  }
-
-  // pgrads write-out (as pgrads_tile's): delta * (Y * sum), then the row's blank / label totals
-#pragma unroll
-  for (int mb = 0; mb < NMB; ++mb)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) pacc[mb][r] += ptot[mb][r];
-  float praw[NMB][16], mraw[NMB][16];
-#pragma unroll
-  for (int mb = 0; mb < NMB; ++mb)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int uc = min(32 * mb + mfma_row(r, h), d.U - 1);
-      praw[mb][r] = ldf(Pb + (size_t)uc * d.V + vc);
-      mraw[mb][r] = mPb[uc];
-    }
-  __builtin_amdgcn_sched_barrier(0);
-  TIO* pout = pgrads + (size_t)b * d.U * d.V;
-#pragma unroll
-  for (int mb = 0; mb < 4; ++mb)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int u = 32 * mb + mfma_row(r, h);
-      float g = 0.0f;
-      if (mb < NMB) {
-        const float y = __expf(praw[mb < NMB ? mb : 0][r] - mraw[mb < NMB ? mb : 0][r]);
-        g = u < Ub ? y * pacc[mb < NMB ? mb : 0][r] : 0.0f;
-      }
-      if (u < d.U && vok) {
-        float res = delta * g;
-        if (vcol == d.blank) res += delta * L.Rt.gB[u];
-        else if (vcol == L.Rt.label[u]) res += delta * L.Rt.gL[u];
-        stf(pout + (size_t)u * d.V + vcol, res);
-      }
-    }
-}
-
-// grid (column tiles of 128, 1, B); dynamic LDS: sizeof(FusedLds).  Needs U <= 112 (one slice of
-// the label axis for egrads, one tile of 128 rows for pgrads) and the blank / label terms
-// folded into both write-outs.
-template <typename TIO>
-__global__ __launch_bounds__(256) void grads_fused_kernel(
-    const TIO* __restrict__ E, const TIO* __restrict__ P, const float* __restrict__ mE,
-    const float* __restrict__ mP, const float* __restrict__ Wn, const float* __restrict__ Wt,
-    const float* __restrict__ deltas, TIO* __restrict__ egrads, TIO* __restrict__ pgrads,
-    const int* __restrict__ inLen, const int* __restrict__ labLen, Dims d, int Up, int Tw,
-    SparseTerms sp, SparsePTerms spp) {
-  extern __shared__ __attribute__((aligned(16))) unsigned char fused_lds_raw[];
-  FusedLds& L = *reinterpret_cast<FusedLds*>(fused_lds_raw);
-  const int b = blockIdx.z;
-  int Tb, Ub;
-  utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int col0 = blockIdx.x * 128 + wave * 32;
-  if (Tb == 0 || Ub == 0) {  // nothing to contract: both gradients are exactly zero
-    for (int t = 0; t < d.T; ++t)
-      if (lane < 32 && col0 + lane < d.V) stf(egrads + ((size_t)b * d.T + t) * d.V + col0 + lane, 0.0f);
-    for (int u = 0; u < d.U; ++u)
-      if (lane < 32 && col0 + lane < d.V) stf(pgrads + ((size_t)b * d.U + u) * d.V + col0 + lane, 0.0f);
-    return;
-  }
-  int nmatch = 0;
-  for (int u0 = 0; u0 < Ub - 1; u0 += 64) {
-    const int u = u0 + lane;
-    const int l = (u < Ub - 1) ? label_at(sp.labels, d, b, u) : -1;
-    const bool hit = l >= col0 && l < col0 + 32 && l != d.blank;
-    const unsigned long long m = __ballot(hit);
-    if (hit) L.Match[wave][nmatch + __popcll(m & ((1ull << lane) - 1))] = (unsigned short)u;
-    nmatch += __popcll(m);
-  }
-  if (threadIdx.x < 128) {
-    const int u = threadIdx.x;
-    const bool valid = u < Ub, has_label = valid && u + 1 < Ub;
-    const int l = has_label ? label_at(spp.labels, d, b, u) : d.blank;
-    L.Rt.gB[u] = valid ? spp.gB[(size_t)b * d.Ua + u] : 0.0f;
-    L.Rt.gL[u] = has_label ? spp.gL[(size_t)b * d.Ua + u] : 0.0f;
-    L.Rt.label[u] = (has_label && l != d.blank) ? l : -1;
-  }
-  // columns of the W slab past Up are never staged, rows of the W^T slab past 32 NMB neither:
-  // clear both buffers once so that what is multiplied there is zero, not whatever LDS held
-  for (int e = threadIdx.x; e < (int)(sizeof(L.Ae) / 4); e += 256)
-    reinterpret_cast<unsigned*>(&L.Ae[0][0][0])[e] = 0u;
-  for (int e = threadIdx.x; e < (int)(sizeof(L.Ap) / 4); e += 256)
-    reinterpret_cast<unsigned*>(&L.Ap[0][0][0])[e] = 0u;
-  __syncthreads();
-#define RNNT_FUSED_WALK(NS, NMB)                                                              \
-  fused_walk<NS, NMB>(E, P, mE, mP, Wn, Wt, deltas, egrads, pgrads, L, d, Up, Tw, b, Tb, Ub, \
-                      sp, nmatch)
-  if (Ub <= 32) RNNT_FUSED_WALK(2, 1);
-  else if (Ub <= 64) RNNT_FUSED_WALK(4, 2);
-  else if (Ub <= 80) RNNT_FUSED_WALK(5, 3);
-  else if (Ub <= 96) RNNT_FUSED_WALK(6, 3);
-  else RNNT_FUSED_WALK(7, 4);
-#undef RNNT_FUSED_WALK
-}
-
 }  // namespace
 
 bool egrads_one_pass(const Dims& d) { return wplane_up(d.U) <= 16 * kEsMaxS; }
@@ -1323,43 +868,6 @@ int launch_pgrads_stream(const f16_t* E, const f16_t* P, const float* mE, const 
                          hipStream_t s) {
   return pgrads_stream_any(E, P, mE, mP, Wt, deltas, pgrads, inLen, labLen, d, accumulate, sp,
                            split_ws, s);
-}
-
-// Whether the fused walk can take this shape -- one slice of the label axis, labels to fold the
-// blank / label terms for -- and whether it is expected to pay: enough column tiles to fill the
-// device with one workgroup per CU (a small grid is better served by the two kernels, whose
-// pgrads tiles can share their frames between workgroups), and a vocabulary large enough for
-// the folded terms.
-bool grads_fused_possible(const Dims& d) {
-  return d.U >= 2 && wplane_up(d.U) <= 16 * kEsMaxS && d.B > 0 && d.T > 0 && d.V > 0;
-}
-bool grads_fused_pays(const Dims& d) {
-  return d.V >= 512 && (long)((d.V + 127) / 128) * d.B >= 192;
-}
-
-template <typename TIO>
-static int grads_fused_any(const TIO* E, const TIO* P, const float* mE, const float* mP,
-                           const float* Wn, const float* Wt, const float* deltas, TIO* egrads,
-                           TIO* pgrads, const int* inLen, const int* labLen, const Dims& d,
-                           const SparseTerms& sp, const SparsePTerms& spp, hipStream_t s) {
-  if (!grads_fused_possible(d)) return fail(kInvalid, "fused gradients: shape not supported");
-  if (!sp.labels || !spp.gB || !spp.labels)
-    return fail(kInvalid, "fused gradients: the blank / label terms must be folded in");
-  const int Up = wplane_up(d.U), Tw = wplane_tw(d.T);
-  auto kernel = grads_fused_kernel<TIO>;
-  RNNT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(FusedLds)));
-  hipLaunchKernelGGL(kernel, dim3((d.V + 127) / 128, 1, d.B), dim3(256), sizeof(FusedLds), s, E, P,
-                     mE, mP, Wn, Wt, deltas, egrads, pgrads, inLen, labLen, d, Up, Tw, sp, spp);
-  RNNT_LAUNCH_CHECK("grads_fused_kernel");
-  return kOk;
-}
-int launch_grads_fused(const float* E, const float* P, const float* mE, const float* mP,
-                       const float* Wn, const float* Wt, const float* deltas, float* egrads,
-                       float* pgrads, const int* inLen, const int* labLen, const Dims& d,
-                       const SparseTerms& sp, const SparsePTerms& spp, hipStream_t s) {
-  return grads_fused_any(E, P, mE, mP, Wn, Wt, deltas, egrads, pgrads, inLen, labLen, d, sp, spp,
-                         s);
 }
 
 }  // namespace rnnt

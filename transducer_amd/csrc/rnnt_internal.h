@@ -160,9 +160,25 @@ int launch_sparse(const Planes& p, float* egrads, float* pgrads, const int* labe
 // After the dalpha walk, in one launch: the W planes (both orientations, from the skewed dalpha
 // and LN planes) and, with bsum != nullptr, bsum[b,t] = what the blank/label terms leave in
 // egrads[b,t,blank] (for folding into the dense kernel's write-out).
+// With `img` set, W is left as bf16 pieces in the slab images of the fused gradient kernel
+// instead of the two fp32 planes (Wn, Wt are then not written).
+struct WImages {
+  // One image per (utterance, slab of 32 frames), three planes (the bf16 pieces, largest first):
+  //   e: [32 frames][kCols label positions]          -- the A operand of the egrads products
+  //   p: [128 label positions][32 frame slots]       -- the A operand of the pgrads products,
+  //      the frames of a slab in the order the fused kernel's matrix instructions take them
+  // as 32-bit words of two bf16 each.  Zero outside the utterance.
+  static constexpr int kCols = 112;
+  static constexpr int kEPlane = 32 * kCols / 2;  // words per plane
+  static constexpr int kPPlane = 128 * 32 / 2;
+  unsigned* e = nullptr;
+  unsigned* p = nullptr;
+  static size_t e_bytes(int B, int Tw) { return (size_t)B * (Tw / 32) * 3 * kEPlane * 4; }
+  static size_t p_bytes(int B, int Tw) { return (size_t)B * (Tw / 32) * 3 * kPPlane * 4; }
+};
 int launch_post_beta(const Planes& p, const float* mE, const float* mP, float* Wn, float* Wt,
                      float* bsum, const int* labels, const int* inLen, const int* labLen,
-                     const Dims& d, hipStream_t s);
+                     const Dims& d, hipStream_t s, const WImages& img = WImages());
 // best / arg: skewed planes ([B][Ua][Dp], see plane_row), written for valid cells only.
 int launch_maxplus(const float* E, const float* P, const int* inLen, const int* labLen,
                    float* best, int* arg, const Dims& d, hipStream_t s, void* lists = nullptr);
@@ -288,9 +304,9 @@ int launch_pgrads(const float* E, const float* P, const float* mE, const float* 
 bool grads_fused_possible(const Dims& d);  // the kernel can take this shape
 bool grads_fused_pays(const Dims& d);      // ... and is expected to beat the two contractions
 int launch_grads_fused(const float* E, const float* P, const float* mE, const float* mP,
-                       const float* Wn, const float* Wt, const float* deltas, float* egrads,
-                       float* pgrads, const int* inLen, const int* labLen, const Dims& d,
-                       const SparseTerms& sp, const SparsePTerms& spp, hipStream_t s);
+                       const WImages& img, const float* deltas, float* egrads, float* pgrads,
+                       const int* inLen, const int* labLen, const Dims& d, const SparseTerms& sp,
+                       const SparsePTerms& spp, hipStream_t s);
 // Whether one launch covers the label axis.  A longer axis goes slice by slice, the slices adding
 // up in the output array; 16-bit gradients then go through `wide` (fp32 scratch of wide_bytes,
 // at least 32 frames of B * V values), a window of frames at a time, so that each value is still
