@@ -48,7 +48,14 @@ int rnnt_hip_forward(const float* emissions, const float* predictions, float* co
 
 /* Replaces cuda::backward (transducer/transducer_cuda.h:29-44, transducer_cuda.cu:309-347):
  * zero-fills egrads, pgrads and lngrads, then writes lngrads = d cost / d log_norms and the
- * sparse blank/label terms of egrads and pgrads. */
+ * sparse blank/label terms of egrads and pgrads.
+ * Like the reference it clears its outputs with memset operations (hipMemsetAsync) and, like
+ * rnnt_hip_forward, rnnt_hip_viterbi, rnnt_hip_log_norms, rnnt_hip_dense_grads and
+ * rnnt_hip_viterbi_decode*, takes its scratch from the stream-ordered allocator
+ * (hipMallocAsync / hipFreeAsync on `stream`): none of these calls can be captured into a HIP
+ * graph.  The capturable entry points are rnnt_hip_loss_forward / rnnt_hip_loss_backward and
+ * their _bf16 / _f16 forms (kernels only, all memory in the caller's workspace), and
+ * rnnt_hip_viterbi_decode_static (kernels only, built-in scratch). */
 int rnnt_hip_backward(const float* emissions, const float* predictions, float* egrads,
                       float* pgrads, float* lngrads, const float* alphas, const float* log_norms,
                       const int* labels, const int* input_lengths, const int* label_lengths,
@@ -159,7 +166,7 @@ int rnnt_hip_viterbi_decode(const float* emissions, const float* predictions,
  * (rnnt_hip_static_scratch_bytes() bytes, held on every GPU the library runs on until the
  * process ends), and the call makes no hipMalloc / hipFree / hipMemset of any kind.  A problem
  * whose scratch does not fit is refused with RNNT_WORKSPACE_TOO_SMALL (one utterance of the
- * headline shape, T=2000 U=101 V=10000, needs 11 MB of the 64).  Every call on a GPU uses that
+ * headline shape, T=2000 U=101 V=10000, needs 16 MB of the 64).  Every call on a GPU uses that
  * GPU's one array: calls that overlap on one GPU (two streams, two threads) race; calls queued
  * on one stream do not.  The array's address is looked up on the first call on each device, so
  * make that first call outside any graph capture. */

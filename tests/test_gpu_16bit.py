@@ -167,6 +167,29 @@ def test_16bit_against_the_fp32_entry_points_and_the_oracle(B, T, U, V, kind):
 
 
 @pytest.mark.parametrize("kind", KIND_NAMES)
+@pytest.mark.parametrize("off_e,off_p", [(200.0, -90.0), (-250.0, 0.0)])
+def test_16bit_scores_far_from_zero(off_e, off_p, kind):
+    """The same inputs with a large common offset (un-normalised logits; fp16 holds them up to
+    65504, with a spacing of 0.125 at 200, which the oracle sees too since it is given the
+    upcast arrays): the per-frame reference of the gradient kernels is then large, and the
+    rounding of its product with log2(e) must not show in the gradients."""
+    LOWP_RTOL = RTOL + KINDS[kind][2]
+    E, P, labels, il, ll = draw(2, 80, 17, 640, seed=int(abs(off_e)), kind=kind)
+    E = (E.float() + off_e).to(E.dtype)
+    P = (P.float() + off_p).to(P.dtype)
+    costs, eg, pg = loss_16bit(E, P, labels, il, ll)
+    c32, e32, p32 = loss_fp32(E, P, labels, il, ll)
+    assert torch.equal(costs, c32)
+    assert_rounds_the_fp32_result(eg, e32, "egrads", 0.999)
+    assert_rounds_the_fp32_result(pg, p32, "pgrads", 0.999)
+    want = oracle.loss_and_grads(E.float().cpu().numpy(), P.float().cpu().numpy(),
+                                 labels.cpu().numpy(), il, ll, precision="f64")
+    for got, ref, what in ((eg, want["egrads"], "egrads"), (pg, want["pgrads"], "pgrads")):
+        frac, worst = violations(got.float().cpu().numpy(), ref, rtol=LOWP_RTOL + 2e-4, atol=ATOL)
+        assert frac == 0.0, "%s: %.4g%% outside (max abs err %g)" % (what, 100 * frac, worst)
+
+
+@pytest.mark.parametrize("kind", KIND_NAMES)
 def test_16bit_blank_not_zero_and_repeated_labels(kind):
     LOWP_RTOL = RTOL + KINDS[kind][2]
     B, T, U, V = 2, 40, 7, 24

@@ -234,7 +234,7 @@ def test_default_mode_in_the_range_where_lists_are_tried(dist, U, V):
     # back to every column, normal ones pass at once; a third utterance is outside the sample
     # either way.
     rng = np.random.default_rng(21)
-    B, T = 3, 37
+    B, T = 3, 130  # (the sample must hold a thousand cells to count: two utterances x 9 frames x U)
     assert capi.load().rnnt_hip_maxplus_tries_lists(B, T, U, V) == 1
     if dist == "normal":
         E, P = rng.standard_normal((B, T, V)), rng.standard_normal((B, U, V))
@@ -244,6 +244,21 @@ def test_default_mode_in_the_range_where_lists_are_tried(dist, U, V):
         E, P = rng.integers(0, 5, (B, T, V)) * 0.5, rng.integers(0, 5, (B, U, V)) * 0.25
     il, ll = np.array([T, T - 5, T - 1], np.int32), np.array([U - 1, U - 3, U - 2], np.int32)
     check(E, P, il, ll, 0, modes=(0,))
+
+
+@pytest.mark.parametrize("dist", ["normal", "uniform"])
+def test_default_mode_when_the_sampled_utterances_are_empty_or_short(dist):
+    # The sample takes utterances 0 and B/2.  With no frames (or a handful) in both, the sample
+    # says nothing about the scores: the call then goes over every column instead of trusting
+    # lists it has no evidence for.  Either way the table is the reference's.
+    rng = np.random.default_rng(5)
+    B, T, U, V = 4, 60, 70, 8192
+    assert capi.load().rnnt_hip_maxplus_tries_lists(B, T, U, V) == 1
+    E = rng.standard_normal((B, T, V)) if dist == "normal" else rng.random((B, T, V))
+    P = rng.standard_normal((B, U, V)) if dist == "normal" else rng.random((B, U, V))
+    for il in ([0, T, 0, T - 7], [3, T, 1, T]):
+        check(E, P, np.array(il, np.int32), np.array([U - 1, U - 2, 5, U - 1], np.int32), 0,
+              modes=(0,))
 
 
 @pytest.mark.parametrize("shape", [(2, 60, 14, 2100), (2, 40, 80, 3200)],

@@ -424,6 +424,33 @@ def test_log_norms_reference_moves_late_in_the_row():
     assert np.abs(got - truth).max() < 4e-6 * max(1.0, np.abs(truth).max())
 
 
+@pytest.mark.parametrize("off_e,off_p", [(300.0, 0.0), (-300.0, 150.0), (120.0, -400.0)])
+@pytest.mark.parametrize("V", [200, 700])
+def test_gradients_of_scores_far_from_zero(off_e, off_p, V):
+    """Scores with a large common offset (un-normalised logits).  The gradient kernels subtract a
+    per-frame reference that they have multiplied by log2(e) beforehand; the rounding of that
+    product grows with the reference's size (6e-6 relative at 100, past the tolerance from about
+    1700) and is taken out again through the W planes.  Costs and both gradients against the
+    oracle on the device's log_norms, every entry inside rel 1e-4 / abs 1e-5; the worst entry is
+    printed in units of that tolerance."""
+    cfg = small_config(2, 90, 20, V, ragged=True)
+    E, P, labels, il, ll = (a.copy() for a in unpack(make_inputs(cfg, seed=int(abs(off_e)) + V)))
+    E += np.float32(off_e)
+    P += np.float32(off_p)
+    c = DeviceCase(E, P, labels, il, ll)
+    costs, eg, pg = gpu_loss(c)
+    LN = gpu_log_norms(c)
+    oc, oa = oracle.forward(E, P, LN, labels, il, ll)
+    oeg, opg, olng = oracle.backward(E, P, np.nan_to_num(oa), LN, labels, il, ll)
+    deg, dpg = oracle.accumulate_grads(E, P, oeg, opg, olng, LN, il, ll)
+    assert_close(costs, oc, what="costs")
+    for got, ref, name in ((eg, deg, "egrads"), (pg, dpg, "pgrads")):
+        ratio = np.abs(got.astype(np.float64) - ref) / (1e-5 + 1e-4 * np.abs(ref))
+        print("offsets %+g / %+g, V=%d: %s worst entry at %.3f of the tolerance"
+              % (off_e, off_p, V, name, ratio.max()))
+        assert_close(got, ref, what=name)
+
+
 def test_log_norms_wide_dynamic_range():
     # maxima of the two operands at different v: the separable shift must not lose the sum
     rng = np.random.default_rng(0)

@@ -75,6 +75,8 @@ constexpr int kCdTileLimit = 128;  // flagged cells a tile may hold and still be
 constexpr int kCdCellGroups = 2048;  // workgroups (of four wavefronts) that share the flagged cells
 constexpr int kCdStats = 8;       // ints of CandScratch::stats
 constexpr int kCdSampleOdds = 150; // lists go on if at most one sampled cell in this many was flagged
+constexpr int kCdSampleMin = 1000; // ... and the sample held at least this many cells (two empty or
+                                   // very short utterances say nothing about the scores)
 constexpr int kNone = 0x7fffffff;
 static_assert(kCdCap % kCdBatch == 0 && kCdDepth % kCdBatch == 0 && kCdBatch % 4 == 0 &&
                   kCdSeg % 4 == 0 && kCdGather % 4 == 0 && (kCdGather & (kCdGather - 1)) == 0 &&
@@ -736,13 +738,17 @@ __global__ __launch_bounds__(256) void cand_cells_kernel(const TIO* __restrict__
 // the call to every column.
 __global__ void cand_decide_kernel(int* stats, int force, int stage, int* tile_fail,
                                    int tiles_per_utterance, int first, int second) {
-  const bool few = (long long)stats[0] * kCdSampleOdds <= (long long)stats[1];
+  const bool enough = stats[1] >= kCdSampleMin;
+  const bool few = enough && (long long)stats[0] * kCdSampleOdds <= (long long)stats[1];
   if (stage == 1) {
     const bool ok = force || few;
     stats[2] = ok ? 1 : 0;
-    stats[3] = ok ? 0 : 1;
-    if (!ok) {  // the second sample starts from nothing: it redoes and flags the same cells
+    // (a sample too small to judge by sends the call to every column at once: longer lists
+    // would be judged by the same few cells)
+    stats[3] = (ok || !enough) ? 0 : 1;
+    if (!ok) {  // the second sample redoes and flags the same cells: their first entries go
       stats[0] = stats[1] = 0;
+      stats[4] = 0;
       for (int i = 0; i < tiles_per_utterance; ++i) {
         tile_fail[(size_t)first * tiles_per_utterance + i] = 0;
         if (second >= 0) tile_fail[(size_t)second * tiles_per_utterance + i] = 0;

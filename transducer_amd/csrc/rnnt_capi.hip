@@ -198,7 +198,9 @@ size_t loss_workspace_layout(const Dims& d, void* base, LossWorkspace* w) {
   const size_t btu = sizeof(float) * (size_t)d.B * d.T * d.U;
   float* mE = take(sizeof(float) * (size_t)d.B * d.T);
   float* mP = take(sizeof(float) * (size_t)d.B * d.U);
-  float* LN = take(btu);
+  // (row-major LN: only when the log-normaliser cannot write it into the lattice plane itself,
+  // i.e. with more labels than its pick list holds)
+  float* LN = d.U - 1 > 1024 ? take(btu) : nullptr;
   // W for the gradient kernels: two fp32 planes, or (fused kernel) the two slab images of bf16
   // pieces, in the same memory
   const size_t wb = align_up(sizeof(float) * (size_t)d.B * wplane_tw(d.T) * wplane_up(d.U));
@@ -273,7 +275,8 @@ size_t viterbi_scratch_bytes(const Dims& d, bool lists) {
 template <typename TIO>
 int viterbi_impl(const TIO* E, const TIO* P, const float* LN, int* labels,
                         const int* inLen, const int* labLen, const Dims& d, Scratch& scratch,
-                        hipStream_t s, bool with_lists, const Planes* ready = nullptr) {
+                        hipStream_t s, int plan, const Planes* ready = nullptr) {
+  const bool with_lists = plan != 0;
   const size_t plane = sizeof(float) * (size_t)d.B * d.Ua * d.Dp + 64;
   Planes p;
   if (ready) p = *ready;
@@ -284,7 +287,7 @@ int viterbi_impl(const TIO* E, const TIO* P, const float* LN, int* labels,
       static_cast<unsigned long long*>(scratch.take(viterbi_bits_bytes(d)));
   void* lists = with_lists ? scratch.take(maxplus_lists_bytes(d)) : nullptr;
   RNNT_STAGE(kMaxplus, launch_maxplus(E, P, inLen, labLen, bestS, reinterpret_cast<int*>(argS), d,
-                                      s, lists));
+                                      s, lists, plan == 2));
   if (!ready) {
     RNNT_STAGE(kSkew, launch_skew(LN, p.lnS, inLen, labLen, d, s));
     // blank scores only: the label planes of the gather are not needed here
@@ -401,7 +404,8 @@ int lowp_viterbi_decode(const TIO* E, const TIO* P, const int* inLen, const int*
   if (!lse_stream_supported(E, d)) return fail(kInvalid, "%s: B*T*U too large", who);
   Scratch scratch(s);
   const size_t yb = lse_scratch_bytes(d);
-  const bool with_lists = maxplus_uses_lists(d);
+  const int plan = maxplus_plan(d);
+  const bool with_lists = plan != 0;
   RNNT_TRY(scratch.reserve(align_up(sizeof(float) * (size_t)B * T) +
                            align_up(sizeof(float) * (size_t)B * U) + align_up(yb) +
                            viterbi_scratch_bytes(d, with_lists)));
@@ -415,7 +419,7 @@ int lowp_viterbi_decode(const TIO* E, const TIO* P, const int* inLen, const int*
   RNNT_STAGE(kYplanes, launch_yplanes(P, mP, ys, labLen, d, s));
   RNNT_STAGE(kLse, launch_lse_stream(E, mE, mP, nullptr, ys, inLen, labLen, d, s, nullptr, p.elS,
                                      p.eb, p.lnS));
-  return viterbi_impl(E, P, nullptr, labels, inLen, labLen, d, scratch, s, with_lists, &p);
+  return viterbi_impl(E, P, nullptr, labels, inLen, labLen, d, scratch, s, plan, &p);
 }
 
 // The best-path decode on fp32 scores; `scratch` decides where its device scratch comes from.
@@ -431,7 +435,8 @@ int decode_fp32(const float* E, const float* P, const int* inLen, const int* lab
   const Dims d = make_dims(B, T, U, V, blank);
   if (!lse_stream_supported(E, d)) return fail(kInvalid, "%s: B*T*U too large", who);
   const size_t yb = lse_scratch_bytes(d);
-  const bool with_lists = maxplus_uses_lists(d);
+  const int plan = maxplus_plan(d);
+  const bool with_lists = plan != 0;
   // LN and the blank scores go straight into the lattice planes, as in the whole-loss path
   // (no row-major LN, no transposing copy, no gather)
   RNNT_TRY(scratch.reserve(align_up(sizeof(float) * (size_t)B * T) +
@@ -446,7 +451,7 @@ int decode_fp32(const float* E, const float* P, const int* inLen, const int* lab
   RNNT_TRY(log_norms_stages(E, P, mE, mP, nullptr, ys, inLen, labLen, d, s, &p, nullptr,
                             &ln_in_plane));
   if (!ln_in_plane) return fail(kInvalid, "%s: log-normaliser left no plane", who);
-  return viterbi_impl(E, P, nullptr, labels, inLen, labLen, d, scratch, s, with_lists, &p);
+  return viterbi_impl(E, P, nullptr, labels, inLen, labLen, d, scratch, s, plan, &p);
 }
 
 // ---------------------------------------------------------------- built-in scratch
@@ -539,20 +544,21 @@ int rnnt_hip_maxplus_table(const float* E, const float* P, const int* inLen, con
   hipStream_t s = static_cast<hipStream_t>(stream);
   const Dims d = make_dims(B, T, U, V, blank);
   const size_t plane = sizeof(float) * (size_t)d.B * d.Ua * d.Dp + 64;
-  const bool with_lists = maxplus_uses_lists(d);
+  const int plan = maxplus_plan(d);
+  const bool with_lists = plan != 0;
   Scratch scratch(s);
   RNNT_TRY(scratch.reserve(2 * align_up(plane) +
                            (with_lists ? align_up(maxplus_lists_bytes(d)) : 0)));
   float* bestS = static_cast<float*>(scratch.take(plane));
   int* argS = static_cast<int*>(scratch.take(plane));
   void* lists = with_lists ? scratch.take(maxplus_lists_bytes(d)) : nullptr;
-  RNNT_STAGE(kMaxplus, launch_maxplus(E, P, inLen, labLen, bestS, argS, d, s, lists));
+  RNNT_STAGE(kMaxplus, launch_maxplus(E, P, inLen, labLen, bestS, argS, d, s, lists, plan == 2));
   return launch_table_out(bestS, argS, inLen, labLen, best, arg, d, s);
 }
 
 int rnnt_hip_maxplus_tries_lists(int B, int T, int U, int V) {
   if (B <= 0 || T <= 0 || U <= 0 || V <= 0) return 0;
-  return maxplus_uses_lists(make_dims(B, T, U, V, 0)) ? 1 : 0;
+  return maxplus_plan(make_dims(B, T, U, V, 0)) != 0 ? 1 : 0;
 }
 
 int rnnt_hip_set_fused_grads(int mode) {
@@ -685,9 +691,10 @@ int rnnt_hip_viterbi(const float* E, const float* P, const float* LN, int* label
   const Dims d = make_dims(B, T, U, V, blank);
   hipStream_t s = static_cast<hipStream_t>(stream);
   Scratch scratch(s);
-  const bool with_lists = maxplus_uses_lists(d);
+  const int plan = maxplus_plan(d);
+  const bool with_lists = plan != 0;
   RNNT_TRY(scratch.reserve(viterbi_scratch_bytes(d, with_lists)));
-  return viterbi_impl(E, P, LN, labels, inLen, labLen, d, scratch, s, with_lists);
+  return viterbi_impl(E, P, LN, labels, inLen, labLen, d, scratch, s, plan);
 }
 
 int rnnt_hip_log_norms(const float* E, const float* P, float* LN, const int* inLen,

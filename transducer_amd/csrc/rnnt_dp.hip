@@ -845,7 +845,8 @@ __device__ __forceinline__ void wplanes_skewed_block(
     float w = 0.0f;
     if (t < Tb && u < Ub) {
       const size_t o = plane_row(d, b, u) + t + u;
-      w = dS[o] * expf((mE[(size_t)b * d.T + t] + mP[(size_t)b * d.U + u]) - lnS[o]);
+      const float me = mE[(size_t)b * d.T + t];
+      w = dS[o] * expf((me + mP[(size_t)b * d.U + u]) - lnS[o]) * frame_exp_correction(me);
     }
     tile[ty + 4 * i][tx] = w;  // [label position][frame]
     if (!img.e && t < Tw && u < Up) Wt[((size_t)b * Up + u) * Tw + t] = w;
@@ -1703,21 +1704,22 @@ int launch_post_beta(const Planes& p, const float* mE, const float* mP, float* W
 // column for every cell; 2: lists wherever the shape allows (tests run small shapes through them)
 static std::atomic<int> g_maxplus_mode{0};
 void set_maxplus_mode(int mode) { g_maxplus_mode.store(mode); }
-bool maxplus_uses_lists(const Dims& d) {
-  const int mode = g_maxplus_mode.load();
-  if (mode == 1 || !maxplus_lists_possible(d)) return false;
-  return mode == 2 || maxplus_lists_pay(d);
+int maxplus_plan(const Dims& d) {
+  const int mode = g_maxplus_mode.load();  // read once per call: the plan is what the call follows
+  if (mode == 1 || !maxplus_lists_possible(d)) return 0;
+  if (mode == 2) return 2;
+  return maxplus_lists_pay(d) ? 1 : 0;
 }
 
 template <typename TIO>
 static int maxplus_any(const TIO* E, const TIO* P, const int* inLen, const int* labLen,
-                       float* best, int* arg, const Dims& d, hipStream_t s, void* lists) {
+                       float* best, int* arg, const Dims& d, hipStream_t s, void* lists,
+                       bool force) {
   if (d.B == 0 || d.T == 0 || d.U == 0) return kOk;
   static_assert(kMpT == 128 && kMpU == 64, "the list pass counts failures per tile of this kernel");
   const int *tile_fail = nullptr, *lists_on = nullptr;
-  if (lists && maxplus_uses_lists(d)) {
-    RNNT_TRY(launch_maxplus_lists(E, P, inLen, labLen, best, arg, d, lists,
-                                  g_maxplus_mode.load() == 2, s));
+  if (lists) {  // (the caller made the plan, and reserved `lists` if it says lists)
+    RNNT_TRY(launch_maxplus_lists(E, P, inLen, labLen, best, arg, d, lists, force, s));
     maxplus_lists_counters(lists, d, &tile_fail, &lists_on);
   }
   const dim3 grid((d.T + kMpT - 1) / kMpT, (d.U + kMpU - 1) / kMpU, d.B);
@@ -1735,16 +1737,16 @@ static int maxplus_any(const TIO* E, const TIO* P, const int* inLen, const int* 
   return kOk;
 }
 int launch_maxplus(const float* E, const float* P, const int* inLen, const int* labLen,
-                   float* best, int* arg, const Dims& d, hipStream_t s, void* lists) {
-  return maxplus_any(E, P, inLen, labLen, best, arg, d, s, lists);
+                   float* best, int* arg, const Dims& d, hipStream_t s, void* lists, bool force) {
+  return maxplus_any(E, P, inLen, labLen, best, arg, d, s, lists, force);
 }
 int launch_maxplus(const bf16_t* E, const bf16_t* P, const int* inLen, const int* labLen,
-                   float* best, int* arg, const Dims& d, hipStream_t s, void* lists) {
-  return maxplus_any(E, P, inLen, labLen, best, arg, d, s, lists);
+                   float* best, int* arg, const Dims& d, hipStream_t s, void* lists, bool force) {
+  return maxplus_any(E, P, inLen, labLen, best, arg, d, s, lists, force);
 }
 int launch_maxplus(const f16_t* E, const f16_t* P, const int* inLen, const int* labLen,
-                   float* best, int* arg, const Dims& d, hipStream_t s, void* lists) {
-  return maxplus_any(E, P, inLen, labLen, best, arg, d, s, lists);
+                   float* best, int* arg, const Dims& d, hipStream_t s, void* lists, bool force) {
+  return maxplus_any(E, P, inLen, labLen, best, arg, d, s, lists, force);
 }
 
 // 32-step words per column of the decision table (one spare)

@@ -12,9 +12,9 @@ constexpr float kLog2e = 1.44269504088896340736f;
 
 // exp(e - m) for a reference m that is used for many e: m comes in already multiplied by log2(e)
 // (once per frame, as the slab is staged), so an exponential is one fused multiply-add and one
-// v_exp_f32 instead of a subtraction, a multiplication and the v_exp_f32.  Against exp(e - m) the
-// result carries one more relative error of 2^-24 |m log2 e| ln 2, the same for every e that
-// shares m: 2e-7 at |m| = 4, far inside the gradients' tolerance.
+// v_exp_f32 instead of a subtraction, a multiplication and the v_exp_f32.  The rounding of that
+// product scales every exponential of the frame by one common factor, which the W planes carry
+// the inverse of (frame_exp_correction, rnnt_internal.h).
 __device__ inline float exp_minus_scaled(float e, float m_log2e) {
   return __builtin_amdgcn_exp2f(__builtin_fmaf(e, kLog2e, -m_log2e));
 }

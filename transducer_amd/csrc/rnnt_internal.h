@@ -181,17 +181,23 @@ int launch_post_beta(const Planes& p, const float* mE, const float* mP, float* W
                      const Dims& d, hipStream_t s, const WImages& img = WImages());
 // best / arg: skewed planes ([B][Ua][Dp], see plane_row), written for valid cells only.
 int launch_maxplus(const float* E, const float* P, const int* inLen, const int* labLen,
-                   float* best, int* arg, const Dims& d, hipStream_t s, void* lists = nullptr);
+                   float* best, int* arg, const Dims& d, hipStream_t s, void* lists = nullptr,
+                   bool force = false);
 int launch_maxplus(const bf16_t* E, const bf16_t* P, const int* inLen, const int* labLen,
-                   float* best, int* arg, const Dims& d, hipStream_t s, void* lists = nullptr);
+                   float* best, int* arg, const Dims& d, hipStream_t s, void* lists = nullptr,
+                   bool force = false);
 int launch_maxplus(const f16_t* E, const f16_t* P, const int* inLen, const int* labLen,
-                   float* best, int* arg, const Dims& d, hipStream_t s, void* lists = nullptr);
-// `lists`: maxplus_lists_bytes(d) bytes of scratch, or null.  With it, and where
-// maxplus_uses_lists(d) says so, most cells are settled from short candidate lists
+                   float* best, int* arg, const Dims& d, hipStream_t s, void* lists = nullptr,
+                   bool force = false);
+// `lists`: maxplus_lists_bytes(d) bytes of scratch, or null (plan 0); force: plan 2.  With it, and where
+// maxplus_plan(d) says so, most cells are settled from short candidate lists
 // (rnnt_cand.hip) and only the cells whose bound test fails are evaluated over every column.
 bool maxplus_lists_possible(const Dims& d);
 bool maxplus_lists_pay(const Dims& d);
-bool maxplus_uses_lists(const Dims& d);
+// How a call of this shape builds its table under the current mode, decided ONCE per call (the
+// mode is process-wide and another thread may change it): 0 over every column, 1 from lists if
+// the sample of cells agrees, 2 from lists unconditionally.
+int maxplus_plan(const Dims& d);
 size_t maxplus_lists_bytes(const Dims& d);
 void set_maxplus_mode(int mode);
 int maxplus_tile_limit();
@@ -216,6 +222,18 @@ int launch_viterbi(const Planes& p, const float* bestS, const float* argS,
 size_t viterbi_bits_bytes(const Dims& d);
 
 // ---------------------------------------------------------------- launchers (rnnt_prep.hip)
+// The gradient kernels form exp(E[t,v] - mE[t]) as exp2(fma(E, log2 e, -fl(mE log2 e))): one
+// fused multiply-add and one v_exp_f32 per element.  The rounding of the product mE log2 e makes
+// every exponential of frame t too large by the same factor 2^r, r = mE log2 e - fl(mE log2 e)
+// (up to 2^-24 |mE log2 e|: 2e-7 at |mE| = 4, but 6e-6 at 100 and past the gradients' tolerance
+// from |mE| of about 1700).  Both gradients are linear in W[t,u] x exp(E[t,v] - mE[t]), so the
+// kernels that write W multiply it by 2^-r of its frame and the hot loops stay as they are.
+constexpr float kLog2eF = 1.44269504088896340736f;
+__device__ inline float frame_exp_correction(float mE) {
+  const float hi = mE * kLog2eF;  // (rounded: what the gradient kernels subtract)
+  const float r = __builtin_fmaf(mE, kLog2eF, -hi);
+  return __builtin_amdgcn_exp2f(-r);
+}
 int wplane_up(int U);  // label-axis pitch of the W planes (multiple of 8)
 int wplane_tw(int T);  // frame-axis pitch of the W planes (multiple of 64)
 // Row maxima of a [rows, V] array.  With `lengths`, rows at or past lengths[item] + extra inside

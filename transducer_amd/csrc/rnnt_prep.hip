@@ -148,7 +148,8 @@ __global__ __launch_bounds__(256) void wplanes_kernel(const float* __restrict__ 
     float w = 0.0f;
     if (t < Tb && u < Ub) {
       const size_t o = ((size_t)b * d.T + t) * d.U + u;
-      w = lngrads[o] * expf((mE[(size_t)b * d.T + t] + mP[(size_t)b * d.U + u]) - LN[o]);
+      const float me = mE[(size_t)b * d.T + t];
+      w = lngrads[o] * expf((me + mP[(size_t)b * d.U + u]) - LN[o]) * frame_exp_correction(me);
     }
     tile[ty + 4 * i][tx] = w;
     if (t < Tw && u < Up) Wn[((size_t)b * Tw + t) * Up + u] = w;
