@@ -66,7 +66,6 @@ constexpr int kCdBisect = 16;    // halvings of the key interval
 constexpr int kCdFrames = 8;     // frames per workgroup of cand_rows_kernel (16: 5 % slower, more utterances'
                                  // transposed P in flight per die; 4: level; 2: 3 % slower)
 constexpr int kCdSampleEvery = 16;  // the sample takes one frame in this many (a multiple of kCdFrames)
-constexpr int kCdGather = 4;     // frames whose results a lane stores together
 constexpr int kCdAheadShort = 10;  // 16-byte pieces of the next row a thread holds while a row is
 constexpr int kCdAheadLong = 17;   // evaluated: rows of up to 10240 / 17408 columns
 constexpr int kCdBatch = 8;      // candidates per batch (two batches in flight)
@@ -79,7 +78,7 @@ constexpr int kCdSampleMin = 1000; // ... and the sample held at least this many
                                    // very short utterances say nothing about the scores)
 constexpr int kNone = 0x7fffffff;
 static_assert(kCdCap % kCdBatch == 0 && kCdDepth % kCdBatch == 0 && kCdBatch % 4 == 0 &&
-                  kCdSeg % 4 == 0 && kCdGather % 4 == 0 && (kCdGather & (kCdGather - 1)) == 0 &&
+                  kCdSeg % 4 == 0 &&
                   kCdSampleEvery % kCdFrames == 0,
               "whole batches, read four entries at a time");
 
@@ -445,16 +444,9 @@ __global__ __launch_bounds__(kCdThreads) void cand_rows_kernel(const TIO* __rest
   for (int s = 1; s < 64; s <<= 1) nmax_first = max(nmax_first, __shfl_xor(nmax_first, s, 64));
   nmax_first = __builtin_amdgcn_readfirstlane(nmax_first);
 
-  // The results of kCdGather consecutive frames leave together, 16 bytes at a time (with at most
-  // 128 label positions, where a lane meets one cell per frame): a cell's neighbours in memory
-  // are the same label position's cells of the next frames, and a 4-byte store per frame would
-  // reach L2 as a sector of its own each time (measured: eight times the planes' bytes written
-  // back; gathering all of a workgroup's frames instead of four changes nothing further).
-  const bool gathered = Ub <= 2 * 64;
-  float qtop[kCdGather];
-  int qarg[kCdGather];
-#pragma unroll
-  for (int k = 0; k < kCdGather; ++k) { qtop[k] = 0.0f; qarg[k] = 0; }
+  // A cell's result is stored as it is found, 4 bytes per plane: in the skewed planes the cells a
+  // wavefront finishes together (64 label positions of one frame) lie within a dozen cache lines,
+  // and the next three frames fill the same lines.
   QuarterBits<kPieces, TIO> ahead;
   if (tid == 0) L->bad[0] = L->bad[1] = 0;
   fetch_quarter<kVec, kPieces>(Eb + (size_t)t_lo * d.V, d.V, ahead);
@@ -616,34 +608,8 @@ __global__ __launch_bounds__(kCdThreads) void cand_rows_kernel(const TIO* __rest
         const float bound =
             tau + (ub == 0 ? ptau_first : (valid ? w.ptau[(size_t)b * d.U + u] : 0.0f));
         const bool ok = !bad && top > bound;
-        if (gathered) {
-          const int slot = (t - t_lo) & (kCdGather - 1);  // uniform
-#pragma unroll
-          for (int k = 0; k < kCdGather; ++k) {
-            qtop[k] = slot == k ? top : qtop[k];
-            qarg[k] = slot == k ? (ok ? at : -1) : qarg[k];
-          }
-          if (valid && (slot == kCdGather - 1 || t == t_hi - 1)) {
-            typedef int int4_align4 __attribute__((ext_vector_type(4), aligned(4)));
-            const size_t o = plane_row(d, b, u) + (t - slot) + u;
-#pragma unroll
-            for (int g = 0; g < kCdGather; g += 4) {
-              if (g + 3 <= slot) {
-                float4_align4 qt;
-                int4_align4 qa;
-                qt.x = qtop[g]; qt.y = qtop[g + 1]; qt.z = qtop[g + 2]; qt.w = qtop[g + 3];
-                qa.x = qarg[g]; qa.y = qarg[g + 1]; qa.z = qarg[g + 2]; qa.w = qarg[g + 3];
-                *reinterpret_cast<float4_align4*>(best + o + g) = qt;
-                *reinterpret_cast<int4_align4*>(arg + o + g) = qa;
-              } else {
-#pragma unroll
-                for (int k = g; k < g + 3; ++k)
-                  if (k <= slot) { best[o + k] = qtop[k]; arg[o + k] = qarg[k]; }
-              }
-            }
-          }
-        } else if (valid) {
-          const size_t o = plane_row(d, b, u) + t + u;
+        if (valid) {
+          const size_t o = plane_at(d, b, u, t + u);
           best[o] = top;
           arg[o] = ok ? at : -1;
         }
@@ -726,7 +692,7 @@ __global__ __launch_bounds__(256) void cand_cells_kernel(const TIO* __restrict__
       if (ot > top || (ot == top && oa < at)) { top = ot; at = oa; }
     }
     if (lane == 0) {
-      const size_t o = plane_row(d, b, u) + t + u;
+      const size_t o = plane_at(d, b, u, t + u);
       best[o] = top;
       arg[o] = at == kNone ? 0 : at;  // :160 nothing beat -inf: index 0 stays
     }
@@ -777,7 +743,7 @@ __global__ __launch_bounds__(256) void table_out_kernel(const float* __restrict_
   int Tb, Ub;
   utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
   const bool cell = t < Tb && u < Ub;
-  const size_t o = plane_row(d, b, u) + t + u, q = ((size_t)b * d.T + t) * d.U + u;
+  const size_t o = plane_at(d, b, u, t + u), q = ((size_t)b * d.T + t) * d.U + u;
   best[q] = cell ? bestS[o] : kNegInf;
   arg[q] = cell ? argS[o] : -1;
 }

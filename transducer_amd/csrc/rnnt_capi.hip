@@ -178,7 +178,7 @@ int log_norms_stages(const float* E, const float* P, float* mE, float* mP, float
 
 struct LossWorkspace {
   Planes planes;
-  float *mE, *mP, *LN, *Wn, *Wt, *bsum;
+  float *mE, *mP, *LN, *Wn, *Wt, *bsum, *emT;
   WImages img;  // shares its memory with Wn / Wt: a backward call writes one form or the other
   void* lse_scratch;
   void* psplit;  // pgrads_split_bytes(d) bytes, or null
@@ -210,10 +210,11 @@ size_t loss_workspace_layout(const Dims& d, void* base, LossWorkspace* w) {
   float* Wn = take(2 * wb > ie + ip ? 2 * wb : ie + ip);
   float* Wt = Wn ? reinterpret_cast<float*>(reinterpret_cast<char*>(Wn) + wb) : nullptr;
   float* bsum = take(sizeof(float) * (size_t)d.B * d.T);
+  float* emT = take(btu);  // label-move terms of egrads, [B][U][T]
   void* ys = take(lse_scratch_bytes(d));  // forward only
   void* ps = take(pgrads_split_bytes(d));  // backward only
   if (base) {
-    w->mE = mE; w->mP = mP; w->LN = LN; w->Wn = Wn; w->Wt = Wt; w->bsum = bsum;
+    w->mE = mE; w->mP = mP; w->LN = LN; w->Wn = Wn; w->Wt = Wt; w->bsum = bsum; w->emT = emT;
     if (images) {
       w->img.e = reinterpret_cast<unsigned*>(Wn);
       w->img.p = reinterpret_cast<unsigned*>(reinterpret_cast<char*>(Wn) + ie);
@@ -372,10 +373,10 @@ int lowp_loss_backward(const TIO* E, const TIO* P, const int* labels, const int*
   // U == 1 there are no labels; the kernels then never read the list, but its pointer is what
   // switches the folding on, so any valid device pointer serves.
   const int* lab = labels ? labels : inLen;
-  RNNT_STAGE(kWplanes, launch_post_beta(w.planes, w.mE, w.mP, w.Wn, w.Wt, w.bsum, lab, inLen,
+  RNNT_STAGE(kWplanes, launch_post_beta(w.planes, w.mE, w.mP, w.Wn, w.Wt, w.bsum, w.emT, lab, inLen,
                                         labLen, d, s));
   SparseTerms sp;
-  sp.dS = w.planes.dS; sp.wE = w.planes.wE; sp.bsum = w.bsum; sp.labels = lab;
+  sp.emT = w.emT; sp.bsum = w.bsum; sp.labels = lab;
   SparsePTerms spp;
   spp.gB = w.planes.gB; spp.gL = w.planes.gL; spp.labels = lab;
   // a label axis of more than one slice: the slices add up in fp32, in the part of the workspace
@@ -820,10 +821,11 @@ int rnnt_hip_loss_backward(const float* E, const float* P, const int* labels, co
                          (fused_mode == 2 || (fused_mode == 1 && grads_fused_pays(d)));
   const bool fold = labels != nullptr && (d.V >= 512 || use_fused) && d.U - 1 <= 1024;
   RNNT_STAGE(kWplanes, launch_post_beta(w.planes, w.mE, w.mP, w.Wn, w.Wt,
-                                        fold ? w.bsum : nullptr, labels, inLen, labLen, d, s,
+                                        fold ? w.bsum : nullptr, fold ? w.emT : nullptr, labels,
+                                        inLen, labLen, d, s,
                                         use_fused ? w.img : WImages()));
   SparseTerms sp;
-  if (fold) { sp.dS = w.planes.dS; sp.wE = w.planes.wE; sp.bsum = w.bsum; sp.labels = labels; }
+  if (fold) { sp.emT = w.emT; sp.bsum = w.bsum; sp.labels = labels; }
   // pgrads always takes its blank / label totals in its write-out (the same two fp32 operations
   // the scatter kernel would do afterwards, so the same bits, and no extra launch)
   SparsePTerms spp;

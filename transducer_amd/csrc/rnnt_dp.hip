@@ -72,9 +72,13 @@ __device__ inline float softplus_fast(float d) { return log1p_unit(exp_neg(d)); 
 // evaluations (a few ulp of lf), the second the rounding of d * log2(e) ahead of v_exp_f32,
 // whose effect on the result grows with |d|.  The bound is not taken from data sheets: the
 // fast value is compared with the exact one for EVERY float d <= 0 (rnnt_hip_lse_bound_check,
-// run by the tests), where it holds with a factor of two to spare.
-constexpr float kFastRelA = 5.0f * 0x1p-23f;
-constexpr float kFastRelB = 1.25f * 0x1p-23f;
+// run by the tests on the device itself).  Measured on gfx950, in units of 2^-23 lf: at most 2.2
+// for |d| <= 1.5, 3.9 up to 4, 6.8 up to 8, 0.46 (5 + 1.25 |d|) beyond; the constants leave an
+// eighth on top of that everywhere.  They are what decides how often a wavefront of the alpha
+// walk takes the library path (its chance per lane is bound / half the sum's spacing), so they
+// are not rounder than that: with 5 and 1.25 the walk of B=32 T=2000 U=100 was a tenth slower.
+constexpr float kFastRelA = 2.75f * 0x1p-23f;
+constexpr float kFastRelB = 0.65f * 0x1p-23f;
 // The bound for fast value lf at argument d.  The clamp keeps 0 * inf out of it at d = -inf;
 // the added 2^-125 covers d below -87.3, where the library's value is a subnormal number and
 // the hardware units return 0.
@@ -101,7 +105,7 @@ __device__ inline float lse2_libm(float a, float b, const unsigned long long* ta
 //   floats on the narrower side of r (the spacing at the float just below |r|: halves when r is
 //   a power of two).
 // Where |hi| < lf the remainder is not exact, but then |r| < 2 lf, the half spacing is below
-// 2^-23 lf and bound(lf) >= 5 * 2^-23 lf alone exceeds it: the test fails by itself.  r = 0, NaN
+// 2^-23 lf and bound(lf) >= 2.75 * 2^-23 lf alone exceeds it: the test fails by itself.  r = 0, NaN
 // operands and two operands of -inf (inf - inf) fail it too.  Lanes that fail take the library
 // path; a wavefront skips it when none does (Ziv's strategy).  Either way the result is the
 // library's, bit for bit.
@@ -180,7 +184,7 @@ __global__ __launch_bounds__(256) void skew_kernel(const float* __restrict__ src
 #pragma unroll
   for (int i = 0; i < 16; ++i) {
     const int u = u0 + ty + 4 * i, t = t0 + tx;
-    if (t < Tb && u < Ub) dstS[plane_row(d, b, u) + t + u] = tile[tx][ty + 4 * i];
+    if (t < Tb && u < Ub) dstS[plane_at(d, b, u, t + u)] = tile[tx][ty + 4 * i];
   }
 }
 
@@ -198,7 +202,7 @@ __global__ __launch_bounds__(256) void unskew_kernel(const float* __restrict__ s
   for (int i = 0; i < 16; ++i) {
     const int u = u0 + ty + 4 * i, t = t0 + tx;
     tile[ty + 4 * i][tx] =
-        (t < Tb && u < Ub) ? srcS[plane_row(d, b, u) + t + u] : 0.0f;
+        (t < Tb && u < Ub) ? srcS[plane_at(d, b, u, t + u)] : 0.0f;
   }
   __syncthreads();
   float* o = dst + (size_t)b * d.T * d.U;
@@ -228,7 +232,7 @@ __global__ __launch_bounds__(256) void gather_kernel(const TIO* __restrict__ E,
   const int l = has_label ? label_at(labels, d, b, u) : d.blank;
   const TIO* Eb = E + (size_t)b * d.T * d.V;
   if (t < Tb) {
-    if (has_label) p.elS[plane_row(d, b, u) + t + u] = ldf(Eb + (size_t)t * d.V + l);
+    if (has_label) p.elS[plane_at(d, b, u, t + u)] = ldf(Eb + (size_t)t * d.V + l);
     if (u == 0) p.eb[(size_t)b * d.Tp + d.Eo + t] = ldf(Eb + (size_t)t * d.V + d.blank);
   }
   if (blockIdx.x == 0 && threadIdx.x == 0) {
@@ -285,6 +289,7 @@ __global__ __launch_bounds__(64 * W) void alpha_kernel(Planes p, const int* __re
   const int nsteps = Tb + Ub - 1;
   const int ngroups = (nsteps + 3) >> 2;
   const int u0 = u_base + (wave * 64 + lane) * C;
+  const int gstride = plane_group_stride(d);
   const bool first_column = u_base == 0 && wave == 0;  // lane 0 owns the lattice's column u = 0
   const float* gin = (kMulti && ghin) ? ghin + (size_t)b * hand_stride : nullptr;
   float* gout = (kMulti && ghout) ? ghout + (size_t)b * hand_stride : nullptr;
@@ -309,7 +314,7 @@ __global__ __launch_bounds__(64 * W) void alpha_kernel(Planes p, const int* __re
 #pragma unroll
   for (int c = 0; c < C; ++c) {
     tlim[c] = (u0 + c < Ub) ? (unsigned)Tb : 0u;
-    const size_t row = plane_row(d, b, u0 + c);  // u0 + c < Ua always
+    const size_t row = plane_group0(d, b, u0 + c);  // u0 + c < Ua always
     lnp[c] = p.lnS + row;
     elp[c] = p.elS + row;
     ap[c] = p.aS + row;
@@ -329,8 +334,8 @@ __global__ __launch_bounds__(64 * W) void alpha_kernel(Planes p, const int* __re
     Group r;
 #pragma unroll
     for (int c = 0; c < C; ++c) {
-      r.ln[c] = *reinterpret_cast<const float4*>(lnp[c] + 4 * g);
-      r.el[c] = *reinterpret_cast<const float4*>(elp[c] + 4 * g);
+      r.ln[c] = *reinterpret_cast<const float4*>(lnp[c] + (size_t)g * gstride);
+      r.el[c] = *reinterpret_cast<const float4*>(elp[c] + (size_t)g * gstride);
     }
 #pragma unroll
     for (int k = 0; k < C + 3; ++k) r.eb[k] = ebl[4 * g + k - (C - 1)];
@@ -400,7 +405,7 @@ __global__ __launch_bounds__(64 * W) void alpha_kernel(Planes p, const int* __re
         hout[j] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(emit[C - 1]), 63));
     }
 #pragma unroll
-    for (int c = 0; c < C; ++c) *reinterpret_cast<float4*>(ap[c] + 4 * g) = aout[c];
+    for (int c = 0; c < C; ++c) *reinterpret_cast<float4*>(ap[c] + (size_t)g * gstride) = aout[c];
     if constexpr (kMulti) {
       if (gout && wave == W - 1 && lane == 63) {  // entries 4g+1 .. 4g+4 for the block above
 #pragma unroll
@@ -457,28 +462,34 @@ __global__ __launch_bounds__(256) void weights_kernel(Planes p, const int* __res
   __shared__ unsigned long long etab[32];  // expf's table (rnnt_libm.h)
   exp2_table_to_lds(etab);
   __syncthreads();
-  const int b = blockIdx.z, u = blockIdx.y;
-  const int dg = blockIdx.x * 256 + threadIdx.x;
-  if (dg >= d.Dp) return;
+  // one thread per plane entry, in memory order: entry i of the utterance's plane is
+  // anti-diagonal 4 (i / 4Ua) + i % 4 of label position (i % 4Ua) / 4 (Ua is a power of two)
+  const int b = blockIdx.z;
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= d.Ua * d.Dp) return;
+  const int per_group = 4 * d.Ua;  // a power of two
+  const int u = (i & (per_group - 1)) >> 2;
+  const int dg = 4 * (i >> (31 - __clz(per_group))) + (i & 3);
   int Tb, Ub;
   utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
   const int t = dg - u;
-  const size_t o = plane_row(d, b, u) + dg;
+  const size_t o = (size_t)b * d.Ua * d.Dp + i;  // = plane_at(d, b, u, dg)
   float wb = 0.0f, we = 0.0f;
   if (u < Ub && t >= 0 && t < Tb) {
     const float a = p.aS[o], ln = p.lnS[o];
+    const size_t o1 = plane_at(d, b, u, dg + 1);
     if (t + 1 < Tb) {
       float x = a + p.eb[(size_t)b * d.Tp + d.Eo + t];
       x = x + p.pb[(size_t)b * d.Ua + u];
       x = x - ln;
-      x = x - p.aS[o + 1];
+      x = x - p.aS[o1];
       wb = expf_glibc(x, etab);
     }
     if (u + 1 < Ub) {
       float x = a + p.elS[o];
       x = x + p.pl[(size_t)b * d.Ua + u];
       x = x - ln;
-      x = x - p.aS[o + d.Dp + 1];
+      x = x - p.aS[o1 + 4];
       we = expf_glibc(x, etab);
     }
   }
@@ -491,13 +502,16 @@ __global__ __launch_bounds__(256) void weights_kernel(Planes p, const int* __res
 // dalpha[t,u] = dalpha[t+1,u]*wB[t,u] + dalpha[t,u+1]*wE[t,u], walked from the last diagonal
 // back to the first; the last cell is seeded with 1 (:95) before the walk.  Each lane also
 // keeps the running sums that the reference subtracts from pgrads[u,blank] and pgrads[u,l_u],
-// in the reference's own order (t descending).  Operands are prefetched two groups of four
-// steps ahead through three rotating register sets.
+// in the reference's own order (t descending).  Operands are prefetched beta_depth(C) groups
+// of four steps ahead through as many rotating register sets.
 // A label axis longer than 64 C positions is walked block by block (u_base = first position of
 // the block), HIGHEST block first: what crosses a boundary here is dalpha of the upper block's
 // first column, one value per diagonal, left in `ghout` ([B][hand_stride], entry s = its dalpha
 // on diagonal s; null for the lowest block) and read by the block below from `ghin` (null for
 // the highest block).
+// register sets of the dalpha walk's prefetch: eight where a set is small, three (the first
+// version's) where a lane owns so many label positions that more sets would spill
+constexpr int beta_depth(int C) { return C <= 4 ? 4 : 3; }
 template <int C, bool kMulti>
 __global__ __launch_bounds__(64) void beta_kernel(Planes p, const int* __restrict__ labels,
                                                   const int* __restrict__ inLen,
@@ -513,6 +527,7 @@ __global__ __launch_bounds__(64) void beta_kernel(Planes p, const int* __restric
   const int nsteps = Tb + Ub - 1;
   const int last = nsteps - 1;  // diagonal of the last cell
   const int u0 = u_base + lane * C;
+  const int gstride = plane_group_stride(d);
   // the block above exists for this utterance only if its first column does
   const float* gin =
       (kMulti && ghin && u_base + 64 * C < Ub) ? ghin + (size_t)b * hand_stride : nullptr;
@@ -526,7 +541,7 @@ __global__ __launch_bounds__(64) void beta_kernel(Planes p, const int* __restric
 #pragma unroll
   for (int c = 0; c < C; ++c) {
     const int u = u0 + c;
-    const size_t row = plane_row(d, b, u);
+    const size_t row = plane_group0(d, b, u);
     wbp[c] = p.wB + row;
     wep[c] = p.wE + row;
     dp[c] = p.dS + row;
@@ -545,8 +560,8 @@ __global__ __launch_bounds__(64) void beta_kernel(Planes p, const int* __restric
     const int gc = g > 0 ? g : 0;
 #pragma unroll
     for (int c = 0; c < C; ++c) {
-      r.wb[c] = *reinterpret_cast<const float4*>(wbp[c] + 4 * gc);
-      r.we[c] = *reinterpret_cast<const float4*>(wep[c] + 4 * gc);
+      r.wb[c] = *reinterpret_cast<const float4*>(wbp[c] + (size_t)gc * gstride);
+      r.we[c] = *reinterpret_cast<const float4*>(wep[c] + (size_t)gc * gstride);
     }
     if constexpr (kMulti) {
 #pragma unroll
@@ -559,14 +574,18 @@ __global__ __launch_bounds__(64) void beta_kernel(Planes p, const int* __restric
   // with_fold: some position of this wavefront has the blank as its label, whose two sums then
   // share one accumulator.  Real transcripts have none, and the walk without the two selects per
   // cell is a fifth shorter (x - 0 is x, so the sums come out the same bits either way).
-  auto run_group = [&](int g, const Group& w, auto with_fold) {
+  // seeded: the group that holds the last diagonal (the first one run).  Every other group has
+  // all four of its steps below `last`, and is compiled without the test per step (a scalar
+  // compare, two mask moves and two branches: eight of the walk's sixteen instructions a step).
+  auto run_group = [&](int g, const Group& w, auto with_fold, auto seeded) {
     constexpr bool kFold = decltype(with_fold)::value;
+    constexpr bool kSeeded = decltype(seeded)::value;
     float4 dout[C];
     float gsend[4];  // dalpha of this lane's first column after each step
 #pragma unroll
     for (int j = 3; j >= 0; --j) {
       const int s = 4 * g + j;
-      if (s >= last) {  // uniform; only in the first group run
+      if (kSeeded && s >= last) {  // uniform
 #pragma unroll
         for (int c = 0; c < C; ++c) f4set(dout[c], j, s == last ? dcol[c] : 0.0f);
         if constexpr (kMulti) gsend[j] = s == last ? dcol[0] : 0.0f;
@@ -596,7 +615,7 @@ __global__ __launch_bounds__(64) void beta_kernel(Planes p, const int* __restric
       }
     }
 #pragma unroll
-    for (int c = 0; c < C; ++c) *reinterpret_cast<float4*>(dp[c] + 4 * g) = dout[c];
+    for (int c = 0; c < C; ++c) *reinterpret_cast<float4*>(dp[c] + (size_t)g * gstride) = dout[c];
     if constexpr (kMulti) {
       if (gout && lane == 0) {
 #pragma unroll
@@ -605,19 +624,37 @@ __global__ __launch_bounds__(64) void beta_kernel(Planes p, const int* __restric
     }
   };
 
+  // beta_depth(C) register sets rotate (no copies): a group's weights are requested that many
+  // groups ahead.  A step of this walk is a dozen instructions, so eight groups are 32 steps or
+  // about a microsecond -- what a load that misses L2 takes; with two groups ahead (the first
+  // version) the walk waited for its weights at nearly every group: 78 ns a step at U = 101.
   auto walk = [&](auto with_fold) __attribute__((always_inline)) {
+    constexpr int kBetaDepth = beta_depth(C);
     int g = last >> 2;  // the group that holds the seed
-    Group x = load_group(g), y = load_group(g - 1), z = load_group(g - 2);
-    for (; g >= 2; g -= 3) {
-      run_group(g, x, with_fold);
-      x = load_group(g - 3);
-      run_group(g - 1, y, with_fold);
-      y = load_group(g - 4);
-      run_group(g - 2, z, with_fold);
-      z = load_group(g - 5);
+    Group q[kBetaDepth];
+#pragma unroll
+    for (int i = 0; i < kBetaDepth; ++i) q[i] = load_group(g - i);
+    // the first round, whose first group holds the seed (a short lattice may end inside it)
+    const std::true_type seeded;
+    const std::false_type plain;
+    run_group(g, q[0], with_fold, seeded);
+    q[0] = load_group(g - kBetaDepth);
+#pragma unroll
+    for (int i = 1; i < kBetaDepth; ++i) {
+      if (g - i >= 0) run_group(g - i, q[i], with_fold, plain);
+      q[i] = load_group(g - i - kBetaDepth);
     }
-    if (g >= 0) run_group(g, x, with_fold);
-    if (g >= 1) run_group(g - 1, y, with_fold);
+    g -= kBetaDepth;
+    for (; g >= kBetaDepth - 1; g -= kBetaDepth) {
+#pragma unroll
+      for (int i = 0; i < kBetaDepth; ++i) {
+        run_group(g - i, q[i], with_fold, plain);
+        q[i] = load_group(g - i - kBetaDepth);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < kBetaDepth - 1; ++i)
+      if (g - i >= 0) run_group(g - i, q[i], with_fold, plain);
   };
   bool any_fold = false;
 #pragma unroll
@@ -671,11 +708,11 @@ __global__ __launch_bounds__(256) void sparse_e_kernel(Planes p, float* __restri
     for (int k = 0; k < kChunk; ++k) {
       const int u = uhi - k;
       const int uc = u > 0 ? u : 0;
-      const size_t o = plane_row(d, b, uc) + t + uc;
+      const size_t o = plane_at(d, b, uc, t + uc), o1 = plane_at(d, b, uc, t + uc + 1);
       // loads are unconditional (the planes are readable one past the utterance); what they
       // return there is discarded by the selects
-      const float ne = dS[o + 1] * wB[o];
-      const float em = dS[o + d.Dp + 1] * wE[o];
+      const float ne = dS[o1] * wB[o];      // dalpha[t+1,u]
+      const float em = dS[o1 + 4] * wE[o];  // dalpha[t,u+1]
       c.ne[k] = has_stay ? ne : 0.0f;
       c.em[k] = (u + 1 < Ub) ? em : 0.0f;
     }
@@ -740,9 +777,9 @@ __global__ __launch_bounds__(64) void sparse_e_rows_kernel(Planes p, float* __re
 #pragma unroll
     for (int k = 0; k < kChunk; ++k) {
       const int u = uhi - k, uc = u > 0 ? u : 0;
-      const size_t o = plane_row(d, b, uc) + t + uc;
-      ne[k] = dS[o + 1] * wB[o];
-      em[k] = dS[o + d.Dp + 1] * wE[o];
+      const size_t o = plane_at(d, b, uc, t + uc), o1 = plane_at(d, b, uc, t + uc + 1);
+      ne[k] = dS[o1] * wB[o];
+      em[k] = dS[o1 + 4] * wE[o];
     }
 #pragma unroll
     for (int k = 0; k < kChunk; ++k) {
@@ -778,63 +815,187 @@ __global__ __launch_bounds__(64) void sparse_e_rows_kernel(Planes p, float* __re
   }
 }
 
-// Per-frame total of everything the reference subtracts from egrads[t, blank]
-// (transducer/transducer_cpu.cpp:96,106,138 and the label moves whose label is the blank): the
-// value sparse_e_kernel would leave in that column.  Used when the label-column terms are folded
-// into the dense egrads kernel instead of being scattered afterwards.
-__device__ __forceinline__ void blank_sums_block(const Planes& p, float* __restrict__ bsum,
-                                                 const int* __restrict__ labels,
-                                                 const int* __restrict__ inLen,
-                                                 const int* __restrict__ labLen, const Dims& d,
-                                                 int bx, int b) {
-  const int t = bx * 256 + threadIdx.x;
+// What the reference subtracts from egrads besides the dense part, per lattice cell
+// (transducer/transducer_cpu.cpp:96,106,138), in the form the dense egrads kernel folds into its
+// write-out:
+//   bsum[b][t]    the total that lands in column `blank` of frame t: -1 for the last frame (:96),
+//                 every blank move's dalpha[t+1,u] wB[t,u], and the label moves whose label is the
+//                 blank -- the value sparse_e_kernel would leave in that column;
+//   emT[b][u][t]  the label move's dalpha[t,u+1] wE[t,u] of every cell ([B][U][T]: the kernel that
+//                 folds them in reads one label position's frames in a row).
+// One lane per frame subtracts its frame's terms in the reference's order, label positions last
+// to first; a wavefront takes 64 frames and works alone (no workgroup barrier).  The operands
+// come through LDS: for eight label positions at a time the wavefront copies the groups of
+// anti-diagonals its 64 frames meet there -- 128 contiguous bytes a group and plane -- with
+// 16-byte loads, requested one chunk ahead, and each lane then picks its own cells (read straight
+// from the planes, the 64 frames would touch 17 cache lines per load).
+constexpr int kBsFrames = 64, kBsPos = 8;
+constexpr int kBsGroups = (kBsFrames + kBsPos + 3) / 4 + 1;  // groups of four anti-diagonals a chunk meets
+// floats per staged group; the pitches put the 16-byte pieces of consecutive groups on different banks
+constexpr int kBsPitch = 4 * kBsPos + 4;         // wB, wE: eight positions
+constexpr int kBsPitchD = 4 * (kBsPos + 1) + 8;  // dalpha: nine (a cell's label move enters position u+1)
+constexpr int kBsPieces = (kBsGroups * kBsPos + 63) / 64;         // 16-byte pieces a lane copies per plane
+constexpr int kBsPiecesD = (kBsGroups * (kBsPos + 1) + 63) / 64;
+constexpr int kBsWave = kBsGroups * (2 * kBsPitch + kBsPitchD);   // floats of LDS a wavefront stages in
+constexpr int kPostBetaLds = 4 * kBsWave > 64 * 65 ? 4 * kBsWave : 64 * 65;  // floats: either kind of block
+__device__ __forceinline__ void frame_terms_block(const Planes& p, float* __restrict__ bsum,
+                                                  float* __restrict__ emT,
+                                                  const int* __restrict__ labels,
+                                                  const int* __restrict__ inLen,
+                                                  const int* __restrict__ labLen, const Dims& d,
+                                                  int bx, int b, float* __restrict__ lds) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int t0 = (4 * bx + wave) * kBsFrames, t = t0 + lane;
   int Tb, Ub;
   utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
-  if (Ub == 0 || t >= Tb) return;
+  if (Ub == 0 || t0 >= Tb) return;  // the whole wavefront
+  const bool active = t < Tb;
   const int* __restrict__ lab = labels + (size_t)b * (d.U - 1);
   const float* __restrict__ dS = p.dS;
   const float* __restrict__ wB = p.wB;
   const float* __restrict__ wE = p.wE;
+  float* stW = lds + wave * kBsWave;        // wB of anti-diagonal groups gbase ..
+  float* stE = stW + kBsGroups * kBsPitch;  // wE
+  float* stD = stE + kBsGroups * kBsPitch;  // dalpha
+  const size_t plane_b = (size_t)b * d.Ua * d.Dp;
+  const int ngroups_plane = d.Dp >> 2;
   const bool has_stay = t + 1 < Tb;
   float acc = (t == Tb - 1) ? -1.0f : 0.0f;
-  // eight label positions per trip: their sixteen loads are requested together, the
-  // subtractions keep the reference's order
-  int u = Ub - 1;
-  for (; u >= 7; u -= 8) {
-    float ne[8];
+  // cell (t,u) reads the weights on anti-diagonal t+u and dalpha on t+u+1: positions ua .. ua+7
+  // of the wavefront's frames meet groups (t0 + ua) / 4 .. (t0 + ua + 64 + 7) / 4
+  struct Pieces { float4 w[kBsPieces], e[kBsPieces], d[kBsPiecesD]; };
+  const float4 zero4 = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+  auto request = [&](int ua) -> Pieces {
+    Pieces r;
+    const int gbase = (t0 + max(ua, 0)) >> 2;
 #pragma unroll
-    for (int k = 0; k < 8; ++k) {
-      const size_t o = plane_row(d, b, u - k) + t + (u - k);
-      ne[k] = dS[o + 1] * wB[o];
+    for (int i = 0; i < kBsPieces; ++i) {
+      const int f = 64 * i + lane, g = gbase + f / kBsPos, ul = f % kBsPos;
+      r.w[i] = zero4;
+      r.e[i] = zero4;
+      if (ua >= 0 && f < kBsGroups * kBsPos && g < ngroups_plane) {  // (ua + ul < Ua: a multiple of 64)
+        const size_t o = plane_b + ((size_t)g * d.Ua + ua + ul) * 4;
+        r.w[i] = *reinterpret_cast<const float4*>(wB + o);
+        r.e[i] = *reinterpret_cast<const float4*>(wE + o);
+      }
     }
 #pragma unroll
-    for (int k = 0; k < 8; ++k) {
-      acc -= has_stay ? ne[k] : 0.0f;
-      const int uu = u - k;
-      if (uu + 1 < Ub && clampi(lab[uu], 0, d.V - 1) == d.blank) {
-        const size_t o = plane_row(d, b, uu) + t + uu;
-        acc -= dS[o + d.Dp + 1] * wE[o];
+    for (int i = 0; i < kBsPiecesD; ++i) {
+      const int f = 64 * i + lane, g = gbase + f / (kBsPos + 1), ul = f % (kBsPos + 1);
+      r.d[i] = zero4;
+      // (position ua + 8 may be Ua itself: the address is then position 0 of the next group,
+      // inside the plane since g + 1 groups exist, and no cell uses the value)
+      if (ua >= 0 && f < kBsGroups * (kBsPos + 1) && g + 1 < ngroups_plane)
+        r.d[i] = *reinterpret_cast<const float4*>(dS + plane_b + ((size_t)g * d.Ua + ua + ul) * 4);
+    }
+    return r;
+  };
+  const int ua_first = (Ub - 1) & ~(kBsPos - 1);
+  Pieces cur = request(ua_first);
+  for (int ua = ua_first; ua >= 0; ua -= kBsPos) {
+    const int gbase = (t0 + ua) >> 2;
+    // (LDS serves a wavefront's accesses in order; the fences only hold the compiler to it)
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int i = 0; i < kBsPieces; ++i) {
+      const int f = 64 * i + lane;
+      if (f < kBsGroups * kBsPos) {
+        *reinterpret_cast<float4*>(stW + (f / kBsPos) * kBsPitch + 4 * (f % kBsPos)) = cur.w[i];
+        *reinterpret_cast<float4*>(stE + (f / kBsPos) * kBsPitch + 4 * (f % kBsPos)) = cur.e[i];
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < kBsPiecesD; ++i) {
+      const int f = 64 * i + lane;
+      if (f < kBsGroups * (kBsPos + 1))
+        *reinterpret_cast<float4*>(stD + (f / (kBsPos + 1)) * kBsPitchD + 4 * (f % (kBsPos + 1))) =
+            cur.d[i];
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    cur = request(ua - kBsPos);
+    if (active) {
+#pragma unroll
+      for (int k = kBsPos - 1; k >= 0; --k) {
+        const int u = ua + k;
+        if (u < Ub) {  // uniform
+          const int dd = t + u;
+          const int here = ((dd >> 2) - gbase) * kBsPitch + 4 * k + (dd & 3);
+          const int next = (((dd + 1) >> 2) - gbase) * kBsPitchD + 4 * k + ((dd + 1) & 3);
+          const float ne = stD[next] * stW[here];      // dalpha[t+1,u] wB[t,u]
+          const float em = stD[next + 4] * stE[here];  // dalpha[t,u+1] wE[t,u]
+          acc -= has_stay ? ne : 0.0f;
+          const bool has_label = u + 1 < Ub;
+          if (has_label && clampi(lab[u], 0, d.V - 1) == d.blank) acc -= em;
+          emT[((size_t)b * d.U + u) * d.T + t] = has_label ? em : 0.0f;
+        }
       }
     }
   }
-  for (; u >= 0; --u) {
-    const size_t o = plane_row(d, b, u) + t + u;
-    const float ne = dS[o + 1] * wB[o];
-    acc -= has_stay ? ne : 0.0f;
-    if (u + 1 < Ub && clampi(lab[u], 0, d.V - 1) == d.blank) acc -= dS[o + d.Dp + 1] * wE[o];
-  }
-  bsum[(size_t)b * d.T + t] = acc;
+  if (active) bsum[(size_t)b * d.T + t] = acc;
 }
 
-// The same from the skewed planes the lattice kernels leave behind (dalpha and LN stored
-// [u][t+u]): no un-skewed copy of dalpha is needed first.  Same arithmetic, same bits.
-// With `img` the block leaves its 64 frames x 64 label positions of W as bf16 pieces instead, in
-// the two slab images the fused gradient kernel copies into LDS as they are (WImages).
+// W from the skewed planes the lattice kernels leave behind (dalpha and LN): no un-skewed copy of
+// dalpha is needed first.  A block takes 64 label positions x 64 anti-diagonals (16 groups of
+// four: 1 KB of contiguous memory a group and plane, read with 16-byte loads), forms W of those
+// cells, and writes them to both orientations through an LDS tile.  Its frames are the 127
+// t = dd - u; the blocks (64 by, 64 bx) over all anti-diagonals below Tw + Up tile the planes.
+// Same arithmetic per cell as wplanes_kernel, same bits.
 __device__ __forceinline__ void wplanes_skewed_block(
     const float* __restrict__ dS, const float* __restrict__ lnS, const float* __restrict__ mE,
     const float* __restrict__ mP, float* __restrict__ Wn, float* __restrict__ Wt,
     const int* __restrict__ inLen, const int* __restrict__ labLen, const Dims& d, int Up, int Tw,
-    float (*tile)[65], int bx, int by, int b, const WImages& img) {
+    float (*tile)[65], int bx, int by, int b) {
+  const int dd0 = bx * 64, u0 = by * 64;
+  int Tb, Ub;
+  utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
+  const size_t plane_b = (size_t)b * d.Ua * d.Dp;
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const int f = k * 256 + threadIdx.x, gl = f >> 6, ul = f & 63;
+    const int u = u0 + ul, g = (dd0 >> 2) + gl;
+    const int tq = 4 * g - u;  // frame of the group's first anti-diagonal
+    float w[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (u < Ub && tq + 3 >= 0 && tq < Tb) {  // (so 4g < T + U: the group lies inside the plane)
+      const size_t o = plane_b + ((size_t)g * d.Ua + u) * 4;
+      const float4 d4 = *reinterpret_cast<const float4*>(dS + o);
+      const float4 l4 = *reinterpret_cast<const float4*>(lnS + o);
+      const float mp = mP[(size_t)b * d.U + u];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int t = tq + j;
+        if (t >= 0 && t < Tb) {
+          const float me = mE[(size_t)b * d.T + t];
+          w[j] = f4get(d4, j) * expf((me + mp) - f4get(l4, j)) * frame_exp_correction(me);
+        }
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) tile[ul][4 * gl + j] = w[j];  // [label position][anti-diagonal]
+  }
+  __syncthreads();
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {  // rows of Wt: one label position, 64 consecutive frames
+    const int ul = ty + 4 * i, u = u0 + ul, t = dd0 + tx - u;
+    if (t >= 0 && t < Tw && u < Up) Wt[((size_t)b * Up + u) * Tw + t] = tile[ul][tx];
+  }
+  for (int i = 0; i < 32; ++i) {  // rows of Wn: one frame, the label positions it has in the tile
+    const int r = ty + 4 * i;     // frame dd0 - u0 - 63 + r meets position u0 + tx on dd0 + tx + r - 63
+    const int t = dd0 - u0 - 63 + r, u = u0 + tx, c = tx + r - 63;
+    if (c >= 0 && c < 64 && t >= 0 && t < Tw && u < Up)
+      Wn[((size_t)b * Tw + t) * Up + u] = tile[tx][c];
+  }
+}
+
+// W of 64 frames x 64 label positions as bf16 pieces, in the two slab images the fused gradient
+// kernel copies into LDS as they are (WImages).  Same arithmetic per cell as above.
+__device__ __forceinline__ void wimages_block(
+    const float* __restrict__ dS, const float* __restrict__ lnS, const float* __restrict__ mE,
+    const float* __restrict__ mP, const int* __restrict__ inLen, const int* __restrict__ labLen,
+    const Dims& d, int Tw, float (*tile)[65], int bx, int by, int b, const WImages& img) {
   const int t0 = bx * 64, u0 = by * 64;
   int Tb, Ub;
   utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
@@ -844,22 +1005,13 @@ __device__ __forceinline__ void wplanes_skewed_block(
     const int u = u0 + ty + 4 * i, t = t0 + tx;
     float w = 0.0f;
     if (t < Tb && u < Ub) {
-      const size_t o = plane_row(d, b, u) + t + u;
+      const size_t o = plane_at(d, b, u, t + u);
       const float me = mE[(size_t)b * d.T + t];
       w = dS[o] * expf((me + mP[(size_t)b * d.U + u]) - lnS[o]) * frame_exp_correction(me);
     }
     tile[ty + 4 * i][tx] = w;  // [label position][frame]
-    if (!img.e && t < Tw && u < Up) Wt[((size_t)b * Up + u) * Tw + t] = w;
   }
   __syncthreads();
-  if (!img.e) {
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const int t = t0 + ty + 4 * i, u = u0 + tx;
-      if (t < Tw && u < Up) Wn[((size_t)b * Tw + t) * Up + u] = tile[tx][ty + 4 * i];
-    }
-    return;
-  }
   const int ntile = Tw >> 5;
   // frames x label positions (the egrads operand): pairs of neighbouring label positions
 #pragma unroll
@@ -897,27 +1049,36 @@ __device__ __forceinline__ void wplanes_skewed_block(
 
 // W planes and per-frame blank totals in one launch: both only need the finished dalpha plane and
 // neither needs the other, so the blocks of the second fill the device beside the first's
-// instead of waiting behind a kernel boundary.  Blocks [0, nw) form W (tile bx, by of utterance
-// b), the rest the blank totals (bsum == nullptr: none).
+// instead of waiting behind a kernel boundary.  The last nw blocks form W (tile bx, by of
+// utterance b; with `img` the tiles are 64 frames x 64 label positions and go to the slab images
+// instead), the blocks before them the per-frame terms bsum and emT (bsum == nullptr: none).
 __global__ __launch_bounds__(256) void post_beta_kernel(Planes p, const float* __restrict__ mE,
                                                         const float* __restrict__ mP,
                                                         float* __restrict__ Wn,
                                                         float* __restrict__ Wt,
                                                         float* __restrict__ bsum,
+                                                        float* __restrict__ emT,
                                                         const int* __restrict__ labels,
                                                         const int* __restrict__ inLen,
                                                         const int* __restrict__ labLen, Dims d,
                                                         int Up, int Tw, int wx, int wy, int nw,
                                                         int sx, WImages img) {
-  __shared__ float tile[64][65];
-  const int n = blockIdx.x;
-  if (n < nw) {
+  __shared__ __attribute__((aligned(16))) float lds[kPostBetaLds];
+  float (*tile)[65] = reinterpret_cast<float (*)[65]>(lds);
+  // the per-frame blocks come first in the grid: each runs longer than a W tile, and started
+  // last they would be the kernel's tail
+  const int ns = gridDim.x - nw;
+  if ((int)blockIdx.x >= ns) {
+    const int n = blockIdx.x - ns;
     const int b = n / (wx * wy), r = n - b * (wx * wy);
-    wplanes_skewed_block(p.dS, p.lnS, mE, mP, Wn, Wt, inLen, labLen, d, Up, Tw, tile, r % wx,
-                         r / wx, b, img);
+    if (img.e)
+      wimages_block(p.dS, p.lnS, mE, mP, inLen, labLen, d, Tw, tile, r % wx, r / wx, b, img);
+    else
+      wplanes_skewed_block(p.dS, p.lnS, mE, mP, Wn, Wt, inLen, labLen, d, Up, Tw, tile, r % wx,
+                           r / wx, b);
   } else {
-    const int m = n - nw;
-    blank_sums_block(p, bsum, labels, inLen, labLen, d, m % sx, m / sx);
+    const int m = blockIdx.x;
+    frame_terms_block(p, bsum, emT, labels, inLen, labLen, d, m % sx, m / sx, lds);
   }
 }
 
@@ -1146,9 +1307,8 @@ __global__ __launch_bounds__(kMpThreads) void maxplus_kernel(const TIO* __restri
         }
       }
       if (cell) {
-        // straight into the skewed planes the lattice walk reads (consecutive frames of one
-        // label position are neighbours there)
-        const size_t o = plane_row(d, b, u) + t + u;
+        // straight into the skewed planes the lattice walk reads
+        const size_t o = plane_at(d, b, u, t + u);
         best[o] = top[i][r];
         arg[o] = at;
       }
@@ -1219,6 +1379,7 @@ __global__ __launch_bounds__(64 * W) void viterbi_kernel(Planes p, const float* 
   // E[t,blank] for the cells of step s sits at ebl[s - u]; column c at step 4g+j reads
   // ebl[4g + j - c], so one run of C+3 values serves all columns of a group
   const float* ebl = p.eb + (size_t)b * d.Tp + d.Eo - u0;
+  const int gstride = plane_group_stride(d);
 
   float stay[C], emit[C], pbv[C];
   unsigned wbits[C];
@@ -1227,7 +1388,7 @@ __global__ __launch_bounds__(64 * W) void viterbi_kernel(Planes p, const float* 
 #pragma unroll
   for (int c = 0; c < C; ++c) {
     const int u = u0 + c, uc = u < d.U ? u : d.U - 1;
-    const size_t row = plane_row(d, b, uc);
+    const size_t row = plane_group0(d, b, uc);
     lnp[c] = p.lnS + row;
     bsp[c] = bestS + row;
     pbv[c] = p.pb[(size_t)b * d.Ua + uc];
@@ -1244,8 +1405,8 @@ __global__ __launch_bounds__(64 * W) void viterbi_kernel(Planes p, const float* 
     Group r;
 #pragma unroll
     for (int c = 0; c < C; ++c) {
-      r.ln[c] = *reinterpret_cast<const float4*>(lnp[c] + 4 * g);
-      r.bs[c] = *reinterpret_cast<const float4*>(bsp[c] + 4 * g);
+      r.ln[c] = *reinterpret_cast<const float4*>(lnp[c] + (size_t)g * gstride);
+      r.bs[c] = *reinterpret_cast<const float4*>(bsp[c] + (size_t)g * gstride);
     }
 #pragma unroll
     for (int k = 0; k < C + 3; ++k) r.eb[k] = ebl[4 * g + k - (C - 1)];
@@ -1361,7 +1522,7 @@ __global__ __launch_bounds__(64 * W) void viterbi_kernel(Planes p, const float* 
     const int st = taken[u1];
     // (a label is never taken at step 0 on a lattice that was walked; the clamp keeps the read
     // inside the plane whatever the decision bits hold)
-    if (st >= 0) out[u1] = argI[plane_row(d, b, u1) + max(st - 1, 0)];
+    if (st >= 0) out[u1] = argI[plane_at(d, b, u1, max(st - 1, 0))];
   }
 }
 
@@ -1601,9 +1762,13 @@ int launch_alpha(const Planes& p, const int* inLen, const int* labLen, float* co
   // array (one float per step and boundary) fits LDS
   const int cpl = block_cells_per_lane(d), nblocks = label_blocks(d);
   const int stride = d.Dp;
-  // (two wavefronts, not four: every lane reads its own plane row, 64 cache lines per load
-  // instruction, and with four wavefronts the CU's vector memory pipeline becomes the limit)
-  const int W = (cpl >= 2 && stride * sizeof(float) <= 48 * 1024) ? 2 : 1;
+  // (two wavefronts up to 256 label positions, where a lane then owns one or two of them; from
+  // eight positions a lane on -- 257 label positions and more in one block -- four wavefronts, if
+  // their three hand-over arrays fit LDS: a step costs a wavefront one log-sum-exp per position
+  // it owns, and the step is what a lattice is bound by)
+  const bool single_block = nblocks == 1;
+  const int W = (single_block && cpl >= 8 && 3 * stride * sizeof(float) <= 144 * 1024) ? 4
+                : (cpl >= 2 && stride * sizeof(float) <= 48 * 1024) ? 2 : 1;
   const size_t lds = W > 1 ? sizeof(float) * (size_t)(W - 1) * stride : 0;
   int* trouble = nullptr;
   RNNT_TRY(trouble_flag(&trouble));
@@ -1614,12 +1779,16 @@ int launch_alpha(const Planes& p, const int* inLen, const int* labLen, float* co
     switch ((nblocks > 1 ? 10000 : 0) + cpl / W * 100 + W) {
 #define CASE(C, W, M)                                                                        \
   case (M ? 10000 : 0) + C * 100 + W:                                                        \
+    if (lds > 64 * 1024)                                                                     \
+      RNNT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(alpha_kernel<C, W, M>),     \
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));   \
     hipLaunchKernelGGL((alpha_kernel<C, W, M>), dim3(d.B), dim3(64 * W), lds, s, p, inLen,  \
                        labLen, costs, d, stride, g_spin_limit, trouble, u_base, ghin,        \
                        ghout);                                                               \
     break;
       CASE(1, 1, false) CASE(2, 1, false) CASE(4, 1, false) CASE(8, 1, false) CASE(16, 1, false)
       CASE(1, 2, false) CASE(2, 2, false) CASE(4, 2, false) CASE(8, 2, false)
+      CASE(2, 4, false) CASE(4, 4, false)
       CASE(16, 1, true) CASE(8, 2, true)  // several blocks: always 1024 positions each
 #undef CASE
       default:
@@ -1633,7 +1802,7 @@ int launch_alpha(const Planes& p, const int* inLen, const int* labLen, float* co
 int launch_weights(const Planes& p, const int* inLen, const int* labLen, const Dims& d,
                    hipStream_t s) {
   if (d.B == 0 || d.T == 0 || d.U == 0) return kOk;
-  hipLaunchKernelGGL(weights_kernel, dim3((d.Dp + 255) / 256, d.Ua, d.B), dim3(256), 0, s, p,
+  hipLaunchKernelGGL(weights_kernel, dim3((d.Ua * d.Dp + 255) / 256, 1, d.B), dim3(256), 0, s, p,
                      inLen, labLen, d);
   RNNT_LAUNCH_CHECK("weights_kernel");
   return kOk;
@@ -1686,16 +1855,20 @@ int launch_sparse(const Planes& p, float* egrads, float* pgrads, const int* labe
 }
 
 int launch_post_beta(const Planes& p, const float* mE, const float* mP, float* Wn, float* Wt,
-                     float* bsum, const int* labels, const int* inLen, const int* labLen,
-                     const Dims& d, hipStream_t s, const WImages& img) {
+                     float* bsum, float* emT, const int* labels, const int* inLen,
+                     const int* labLen, const Dims& d, hipStream_t s, const WImages& img) {
   if (d.B == 0 || d.T == 0 || d.U == 0) return kOk;
   const int Up = wplane_up(d.U), Tw = wplane_tw(d.T);
   if (img.e && Up > WImages::kCols)
     return fail(kInvalid, "W images hold at most %d label positions", WImages::kCols);
-  const int wx = Tw / 64, wy = (Up + 63) / 64, nw = wx * wy * d.B;
-  const int sx = (d.T + 255) / 256, ns = bsum ? sx * d.B : 0;
+  // W tiles: 64 label positions x 64 anti-diagonals (all anti-diagonals below Tw + Up), or for
+  // the images 64 label positions x 64 frames
+  const int wx = img.e ? Tw / 64 : (Tw + Up + 62) / 64, wy = (Up + 63) / 64, nw = wx * wy * d.B;
+  if ((bsum == nullptr) != (emT == nullptr))
+    return fail(kInvalid, "post_beta: the blank totals and the label-move terms come together");
+  const int sx = (d.T + 4 * kBsFrames - 1) / (4 * kBsFrames), ns = bsum ? sx * d.B : 0;
   hipLaunchKernelGGL(post_beta_kernel, dim3(nw + ns), dim3(256), 0, s, p, mE, mP, Wn, Wt, bsum,
-                     labels, inLen, labLen, d, Up, Tw, wx, wy, nw, sx, img);
+                     emT, labels, inLen, labLen, d, Up, Tw, wx, wy, nw, sx, img);
   RNNT_LAUNCH_CHECK("post_beta_kernel");
   return kOk;
 }

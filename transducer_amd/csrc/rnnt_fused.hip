@@ -280,14 +280,12 @@ __device__ __forceinline__ void fused_walk(
     // names how many requests may still be out): this tile's blank / label terms, the next
     // tile's W slabs (stored to LDS at the end of this tile), the next tile's emissions (not
     // needed before the next tile).
-    float sd[kEsPrefetch], sw[kEsPrefetch], sbl = 0.0f;
+    float sd[kEsPrefetch], sbl = 0.0f;
     if (nmatch > 0 || blank_lane >= 0) {
       const int tr = min(t0 + l32, Tb - 1);
 #pragma unroll
       for (int i = 0; i < kEsPrefetch; ++i) {
-        const size_t o = plane_row(d, b, mu[i]) + tr + mu[i];
-        sd[i] = sp.dS[o + d.Dp + 1];
-        sw[i] = sp.wE[o];
+        sd[i] = sp.emT[((size_t)b * d.U + mu[i]) * d.T + tr];
       }
       if (blank_lane >= 0) sbl = sp.bsum[(size_t)b * d.T + tr];
     }
@@ -429,11 +427,10 @@ __device__ __forceinline__ void fused_walk(
       };
 #pragma unroll
       for (int i = 0; i < kEsPrefetch; ++i)
-        if (i < nmatch) apply(row_ok ? sd[i] * sw[i] : 0.0f, mc[i], -1.0f);
+        if (i < nmatch) apply(row_ok ? sd[i] : 0.0f, mc[i], -1.0f);
       for (int i = kEsPrefetch; i < nmatch; ++i) {
         const int u = match[i];
-        const size_t o = plane_row(d, b, u) + min(t0 + l32, Tb - 1) + u;
-        apply(row_ok ? sp.dS[o + d.Dp + 1] * sp.wE[o] : 0.0f,
+        apply(row_ok ? sp.emT[((size_t)b * d.U + u) * d.T + min(t0 + l32, Tb - 1)] : 0.0f,
               label_at(sp.labels, d, b, u) - wave_col0, -1.0f);
       }
       if (blank_lane >= 0) apply(row_ok ? sbl : 0.0f, blank_lane, 1.0f);
@@ -471,19 +468,17 @@ __device__ __forceinline__ void fused_walk(
   // only two places of the tile with a branch (a branch in the middle would cut the tile into
   // basic blocks, and the compiler moves arithmetic into the block that uses its result).
   const bool folding = nmatch > 0 || blank_lane >= 0;  // uniform per wavefront
-  struct FoldRaw { float sd[kEsPrefetch], sw[kEsPrefetch], sbl; };
+  struct FoldRaw { float sd[kEsPrefetch], sbl; };
   auto fold_request = [&](int ti) -> FoldRaw {
     FoldRaw f;
 #pragma unroll
-    for (int i = 0; i < kEsPrefetch; ++i) f.sd[i] = f.sw[i] = 0.0f;
+    for (int i = 0; i < kEsPrefetch; ++i) f.sd[i] = 0.0f;
     f.sbl = 0.0f;
     if (folding) {
       const int tr = ti * 32 + l32;
 #pragma unroll
       for (int i = 0; i < kEsPrefetch; ++i) {
-        const size_t o = plane_row(d, b, mu[i]) + tr + mu[i];
-        f.sd[i] = sp.dS[o + d.Dp + 1];
-        f.sw[i] = sp.wE[o];
+        f.sd[i] = sp.emT[((size_t)b * d.U + mu[i]) * d.T + tr];
       }
       if (blank_lane >= 0) f.sbl = sp.bsum[(size_t)b * d.T + tr];
     }
@@ -509,7 +504,7 @@ __device__ __forceinline__ void fused_walk(
       };
 #pragma unroll
       for (int i = 0; i < kEsPrefetch; ++i)
-        if (i < nmatch) take(f.sd[i] * f.sw[i], mc[i], -1.0f);
+        if (i < nmatch) take(f.sd[i], mc[i], -1.0f);
       if (blank_lane >= 0) take(f.sbl, blank_lane, 1.0f);
     }
   };

@@ -214,14 +214,12 @@ __device__ __forceinline__ void egrads_walk(
     }
     // sparse terms of this tile for up to kEsPrefetch labels that fall into this wavefront's
     // columns: one coalesced load per plane, requested here so it arrives under the matrix work
-    float sd[kEsPrefetch], sw[kEsPrefetch], sbl = 0.0f;
+    float sd[kEsPrefetch], sbl = 0.0f;
     if (!kAccumulate && (nmatch > 0 || blank_lane >= 0)) {
       const int tr = min(t0 + l32, Tb - 1);
 #pragma unroll
       for (int i = 0; i < kEsPrefetch; ++i) {
-        const size_t o = plane_row(d, b, mu[i]) + tr + mu[i];
-        sd[i] = sp.dS[o + d.Dp + 1];
-        sw[i] = sp.wE[o];
+        sd[i] = sp.emT[((size_t)b * d.U + mu[i]) * d.T + tr];
       }
       if (blank_lane >= 0) sbl = sp.bsum[(size_t)b * d.T + tr];
     }
@@ -283,11 +281,10 @@ __device__ __forceinline__ void egrads_walk(
       };
 #pragma unroll
       for (int i = 0; i < kEsPrefetch; ++i)
-        if (i < nmatch) apply(row_ok ? sd[i] * sw[i] : 0.0f, mc[i], -1.0f);
+        if (i < nmatch) apply(row_ok ? sd[i] : 0.0f, mc[i], -1.0f);
       for (int i = kEsPrefetch; i < nmatch; ++i) {  // more labels in one 32-column block
         const int u = match[i];
-        const size_t o = plane_row(d, b, u) + min(t0 + l32, Tb - 1) + u;
-        apply(row_ok ? sp.dS[o + d.Dp + 1] * sp.wE[o] : 0.0f,
+        apply(row_ok ? sp.emT[((size_t)b * d.U + u) * d.T + min(t0 + l32, Tb - 1)] : 0.0f,
               label_at(sp.labels, d, b, u) - wave_col0, -1.0f);
       }
       if (blank_lane >= 0) apply(row_ok ? sbl : 0.0f, blank_lane, 1.0f);

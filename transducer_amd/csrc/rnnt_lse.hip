@@ -247,8 +247,9 @@ __global__ __launch_bounds__(64 * kWaves, kWaves / 2) void lse_stream_kernel(
       r.x[i] = kVec ? load8(px[i], k0 + 8 * c8, d.V) : load8_any(px[i], k0 + 8 * c8, d.V);
     return r;
   };
-  // copies column `col` (which lies in the slab held in r) of this thread's rows to dst[t]
-  auto pick = [&](const XRegs& r, int col, float* dst) {
+  // copies column `col` (which lies in the slab held in r) of this thread's rows to the blank
+  // vector (nu_plane < 0: dst[t]) or to label position nu_plane of the skewed plane dst
+  auto pick = [&](const XRegs& r, int col, float* dst, int nu_plane) {
     if (c8 != ((col & 31) >> 3)) return;
     const int e = col & 7;  // uniform
 #pragma unroll
@@ -266,13 +267,13 @@ __global__ __launch_bounds__(64 * kWaves, kWaves / 2) void lse_stream_kernel(
           (__float_as_uint(x[4]) & k4) | (__float_as_uint(x[5]) & k5) |
           (__float_as_uint(x[6]) & k6) | (__float_as_uint(x[7]) & k7));
       const int t = t0 + srow + (kThreads / 4) * i;
-      if (t < Tb) dst[t] = v;
+      if (t < Tb) dst[nu_plane < 0 ? (size_t)t : plane_at(d, b, nu_plane, t + nu_plane)] = v;
     }
   };
   auto picks = [&](const XRegs& r, int kslab) {
     while ((ncol >> 5) == kslab) {  // uniform
-      if (nu == nlab) pick(r, ncol, ebv + (size_t)b * d.Tp + d.Eo);
-      else pick(r, ncol, elS + plane_row(d, b, nu) + nu);
+      if (nu == nlab) pick(r, ncol, ebv + (size_t)b * d.Tp + d.Eo, -1);
+      else pick(r, ncol, elS, nu);
       ++cursor;
       next_pick();
     }
@@ -497,7 +498,7 @@ __global__ __launch_bounds__(64 * kWaves, kWaves / 2) void lse_stream_kernel(
         if (t < Tb && u < Ub)
           v = add3(logf(tot[m][r] + acc[m][r]), mfin[row], mu, reference_shift(mfin[row]));
         if (lnS == nullptr) LNb[(size_t)t * d.U + u] = v;
-        else if (t < Tb && u < Ub) lnS[plane_row(d, b, u) + t + u] = v;
+        else if (t < Tb && u < Ub) lnS[plane_at(d, b, u, t + u)] = v;
       }
     }
 }
