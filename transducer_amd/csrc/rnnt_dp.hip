@@ -511,23 +511,54 @@ __global__ __launch_bounds__(256) void weights_kernel(Planes p, const int* __res
 // the highest block).
 // register sets of the dalpha walk's prefetch: eight where a set is small, three (the first
 // version's) where a lane owns so many label positions that more sets would spill
-constexpr int beta_depth(int C) { return C <= 4 ? 4 : 3; }
-template <int C, bool kMulti>
-__global__ __launch_bounds__(64) void beta_kernel(Planes p, const int* __restrict__ labels,
-                                                  const int* __restrict__ inLen,
-                                                  const int* __restrict__ labLen, Dims d,
-                                                  int hand_stride, int u_base,
-                                                  const float* __restrict__ ghin,
-                                                  float* __restrict__ ghout) {
-  const int b = blockIdx.x, lane = threadIdx.x;
+constexpr int beta_depth(int C) { return C <= 2 ? 8 : C <= 4 ? 4 : 3; }
+// W wavefronts (one launch covering the whole label axis only): wavefront w owns positions
+// (64 w + lane) C .. + C-1, so the HIGHEST wavefront leads.  Each but the lowest leaves dalpha of
+// its first column in LDS, one value per diagonal, and counts the groups it has finished; the
+// wavefront below reads them one group later (the same hand-over as between blocks, with the
+// bounded wait of alpha_kernel).  Every wavefront runs all groups, past the utterance's labels
+// too (zeros), so nobody waits for a wavefront that has left.
+template <int C, int W, bool kMulti>
+__global__ __launch_bounds__(64 * W) void beta_kernel(Planes p, const int* __restrict__ labels,
+                                                      const int* __restrict__ inLen,
+                                                      const int* __restrict__ labLen, Dims d,
+                                                      int hand_stride, int u_base,
+                                                      const float* __restrict__ ghin,
+                                                      float* __restrict__ ghout, int spin_limit,
+                                                      int* __restrict__ trouble) {
+  static_assert(W == 1 || !kMulti, "several wavefronts only when one launch covers the label axis");
+  extern __shared__ __attribute__((aligned(16))) float hand[];  // [W-1][hand_stride]: entry s =
+                                                                // dalpha on diagonal s
+  __shared__ int done[W];  // groups a wavefront has published
+  const int b = blockIdx.x, lane = threadIdx.x & 63;
+  const int wave = W > 1 ? __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) : 0;
   int Tb, Ub;
   utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
   if (Tb == 0 || Ub == 0) return;  // :92-94
   if (u_base >= Ub) return;        // a block past this utterance's labels
+  if (W > 1) {
+    if (threadIdx.x < W) done[threadIdx.x] = 0;
+    __syncthreads();
+  }
   const int nsteps = Tb + Ub - 1;
   const int last = nsteps - 1;  // diagonal of the last cell
-  const int u0 = u_base + lane * C;
+  // kSpread: a lane's C positions are 64 apart (u0 + 64 c), so that the 64 lanes of a load or
+  // store touch neighbouring 16-byte pieces of the plane, whole cache lines together; the price
+  // is a lane-to-scalar move per position and step (lane 63's right neighbour is lane 0's next
+  // position).  With two positions a lane next to each other (u0 + c) a load still fills half
+  // of every line it touches, and the walk of up to 128 label positions is faster that way
+  // (B=32 T=2000 U=100: 38.6 against 45.4 ns a step; two wavefronts of one position: 52.5).
+  constexpr bool kSpread = W > 1 || C > 2;
+  constexpr int kApart = kSpread ? 64 : 1;
+  const int u0 = u_base + wave * 64 * C + (kSpread ? lane : lane * C);
   const int gstride = plane_group_stride(d);
+  float* hand_out = hand + (wave > 0 ? wave - 1 : 0) * hand_stride;  // wave > 0
+  const float* hand_in = hand + wave * hand_stride;                  // wave < W-1
+  const int g_first = last >> 2;  // the group that holds the seed: the first one run
+  int avail = 0;                  // groups the wavefront above is known to have published
+  auto wait_for = [&](int need) {
+    avail = bounded_wait(&done[wave + 1], avail, need, spin_limit, trouble);
+  };
   // the block above exists for this utterance only if its first column does
   const float* gin =
       (kMulti && ghin && u_base + 64 * C < Ub) ? ghin + (size_t)b * hand_stride : nullptr;
@@ -540,7 +571,7 @@ __global__ __launch_bounds__(64) void beta_kernel(Planes p, const int* __restric
   float* dp[C];
 #pragma unroll
   for (int c = 0; c < C; ++c) {
-    const int u = u0 + c;
+    const int u = u0 + kApart * c;
     const size_t row = plane_group0(d, b, u);
     wbp[c] = p.wB + row;
     wep[c] = p.wE + row;
@@ -582,23 +613,44 @@ __global__ __launch_bounds__(64) void beta_kernel(Planes p, const int* __restric
     constexpr bool kSeeded = decltype(seeded)::value;
     float4 dout[C];
     float gsend[4];  // dalpha of this lane's first column after each step
+    float hh[4] = {0.0f, 0.0f, 0.0f, 0.0f};  // dalpha of the wavefront above's first column on
+                                             // diagonals 4g+1 .. 4g+4
+    if (W > 1 && wave < W - 1) {
+      wait_for(g_first - g + 1);  // diagonals 4g+1 .. 4g+3 are of its group g
+#pragma unroll
+      for (int j = 0; j < 4; ++j) hh[j] = hand_in[4 * g + 1 + j];  // uniform
+    }
 #pragma unroll
     for (int j = 3; j >= 0; --j) {
       const int s = 4 * g + j;
       if (kSeeded && s >= last) {  // uniform
 #pragma unroll
         for (int c = 0; c < C; ++c) f4set(dout[c], j, s == last ? dcol[c] : 0.0f);
-        if constexpr (kMulti) gsend[j] = s == last ? dcol[0] : 0.0f;
+        if constexpr (kMulti || W > 1) gsend[j] = s == last ? dcol[0] : 0.0f;
       } else {
-        float from_right = wave_shl1(dcol[0], 0.0f);
-        // the column right of lane 63's last one belongs to the block above: its dalpha on the
-        // diagonal just done, s + 1
-        if constexpr (kMulti) from_right = (gin && lane == 63) ? w.gh[j] : from_right;
+        // dalpha of the position to the right on the diagonal just done, s + 1: the next lane's,
+        // and for lane 63 lane 0's next position -- or, right of the wavefront's last position,
+        // what the block or the wavefront above handed over (nothing above: 0)
+        float right[C];
+        float above = 0.0f;  // right of the wavefront's last position
+        if constexpr (kMulti) above = gin ? w.gh[j] : 0.0f;
+        if (W > 1) above = wave < W - 1 ? hh[j] : 0.0f;
+        if constexpr (kSpread) {
+#pragma unroll
+          for (int c = 0; c < C; ++c) {
+            const float past =  // what lane 63 receives
+                c < C - 1 ? __int_as_float(__builtin_amdgcn_readlane(__float_as_int(dcol[c + 1]), 0))
+                          : above;
+            right[c] = wave_shl1(dcol[c], past);
+          }
+        } else {
+#pragma unroll
+          for (int c = 0; c < C; ++c) right[c] = c < C - 1 ? dcol[c + 1] : wave_shl1(dcol[0], above);
+        }
 #pragma unroll
         for (int c = 0; c < C; ++c) {
-          const float right = (c == C - 1) ? from_right : dcol[c + 1];
           const float ne = dcol[c] * f4get(w.wb[c], j);
-          const float em = right * f4get(w.we[c], j);
+          const float em = right[c] * f4get(w.we[c], j);
           const float dn = ne + em;
           if constexpr (kFold) {
             const float em_b = fold[c] ? em : 0.0f, em_l = fold[c] ? 0.0f : em;
@@ -611,7 +663,7 @@ __global__ __launch_bounds__(64) void beta_kernel(Planes p, const int* __restric
           dcol[c] = dn;
           f4set(dout[c], j, dn);
         }
-        if constexpr (kMulti) gsend[j] = dcol[0];
+        if constexpr (kMulti || W > 1) gsend[j] = dcol[0];
       }
     }
 #pragma unroll
@@ -622,6 +674,13 @@ __global__ __launch_bounds__(64) void beta_kernel(Planes p, const int* __restric
         for (int j = 0; j < 4; ++j) gout[4 * g + j] = gsend[j];
       }
     }
+    if (W > 1 && wave > 0 && lane == 0) {  // entries 4g .. 4g+3, then the progress
+#pragma unroll
+      for (int j = 0; j < 4; ++j) hand_out[4 * g + j] = gsend[j];
+      asm volatile("" ::: "memory");  // (LDS serves a wavefront's requests in order)
+      __hip_atomic_store(&done[wave], g_first - g + 1, __ATOMIC_RELAXED,
+                         __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
   };
 
   // beta_depth(C) register sets rotate (no copies): a group's weights are requested that many
@@ -630,10 +689,13 @@ __global__ __launch_bounds__(64) void beta_kernel(Planes p, const int* __restric
   // version) the walk waited for its weights at nearly every group: 78 ns a step at U = 101.
   auto walk = [&](auto with_fold) __attribute__((always_inline)) {
     constexpr int kBetaDepth = beta_depth(C);
-    int g = last >> 2;  // the group that holds the seed
+    int g = g_first;
     Group q[kBetaDepth];
 #pragma unroll
     for (int i = 0; i < kBetaDepth; ++i) q[i] = load_group(g - i);
+    // fall a few groups behind the wavefront above, so that the wait per group finds its
+    // counter there already
+    if (W > 1 && wave < W - 1) wait_for(min(g_first + 1, 8 * (W - 1 - wave)));
     // the first round, whose first group holds the seed (a short lattice may end inside it)
     const std::true_type seeded;
     const std::false_type plain;
@@ -664,7 +726,7 @@ __global__ __launch_bounds__(64) void beta_kernel(Planes p, const int* __restric
 
 #pragma unroll
   for (int c = 0; c < C; ++c) {
-    const int u = u0 + c;
+    const int u = u0 + kApart * c;
     if (u < Ub) {
       p.gB[(size_t)b * d.Ua + u] = accB[c];
       p.gL[(size_t)b * d.Ua + u] = accL[c];
@@ -1812,18 +1874,35 @@ int launch_beta(const Planes& p, const int* labels, const int* inLen, const int*
                 const Dims& d, hipStream_t s) {
   if (d.B == 0 || d.T == 0 || d.U == 0) return kOk;
   const int cpl = block_cells_per_lane(d), nblocks = label_blocks(d);
+  // wavefronts: one up to 128 label positions (a step of this walk is a handful of
+  // instructions a position, and the hand-over would cost as much again), two up to 256, four
+  // beyond, if their hand-over arrays fit LDS; one per block when the axis takes several launches
+  const int stride = d.Dp;
+  const bool single_block = nblocks == 1;
+  const int W = !single_block ? 1
+                : (cpl >= 8 && 3 * stride * sizeof(float) <= 144 * 1024) ? 4
+                : (cpl >= 4 && stride * sizeof(float) <= 48 * 1024) ? 2 : 1;
+  const size_t lds = W > 1 ? sizeof(float) * (size_t)(W - 1) * stride : 0;
+  int* trouble = nullptr;
+  RNNT_TRY(trouble_flag(&trouble));
   for (int k = nblocks - 1; k >= 0; --k) {  // highest block first
     const float* ghin = k == nblocks - 1 ? nullptr : p.hand[(k + 1) & 1];
     float* ghout = k == 0 ? nullptr : p.hand[k & 1];
     const int u_base = k * 64 * cpl;
-    switch ((nblocks > 1 ? 100 : 0) + cpl) {
-#define CASE(C, M)                                                                           \
-  case (M ? 100 : 0) + C:                                                                    \
-    hipLaunchKernelGGL((beta_kernel<C, M>), dim3(d.B), dim3(64), 0, s, p, labels, inLen,    \
-                       labLen, d, d.Dp, u_base, ghin, ghout);                                \
+    switch ((nblocks > 1 ? 10000 : 0) + cpl / W * 100 + W) {
+#define CASE(C, W, M)                                                                       \
+  case (M ? 10000 : 0) + C * 100 + W:                                                       \
+    if (lds > 64 * 1024)                                                                    \
+      RNNT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(beta_kernel<C, W, M>),     \
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));  \
+    hipLaunchKernelGGL((beta_kernel<C, W, M>), dim3(d.B), dim3(64 * W), lds, s, p, labels, \
+                       inLen, labLen, d, stride, u_base, ghin, ghout, g_spin_limit,        \
+                       trouble);                                                            \
     break;
-      CASE(1, false) CASE(2, false) CASE(4, false) CASE(8, false) CASE(16, false)
-      CASE(16, true)
+      CASE(1, 1, false) CASE(2, 1, false) CASE(4, 1, false) CASE(8, 1, false) CASE(16, 1, false)
+      CASE(2, 2, false) CASE(4, 2, false) CASE(8, 2, false)
+      CASE(2, 4, false) CASE(4, 4, false)
+      CASE(16, 1, true)
 #undef CASE
       default:
         return fail(kInvalid, "dalpha: no kernel for %d label positions per lane", cpl);
