@@ -291,6 +291,51 @@ def test_headline_table_of_best_labels_is_the_same_however_it_is_built(near_ties
     assert np.array_equal(tables[0][0][b, t, :ub].cpu().numpy(), s.max(axis=1)[:ub])
 
 
+def test_table_when_the_sample_passes_and_the_rest_of_the_batch_does_not_suit_lists():
+    # The dearest case of the default mode: the two sampled utterances (0 and B/2) have normal
+    # scores, so the call goes on with lists, but every other utterance's scores are quantised
+    # (five levels: ties everywhere, empty lists, every cell fails its exactness test).  Their
+    # tiles are then redone over every column; the list pass gives a tile up once it holds more
+    # flagged cells than are redone one by one, a frame or two into each workgroup's eight.
+    # Same table as over every column, and at most 1.5 times its time (measured: 1.33; 1.46
+    # when the list pass ran over all frames for nothing).
+    c = DeviceBatch(CONFIGS["cfg5"], seed=8)
+    B, T, U, V = c.dims
+    for b in range(B):
+        if b not in (0, B // 2):
+            c.E[b] = torch.randint(0, 5, (T, V), device="cuda:0").float() * 0.5
+            c.P[b] = torch.randint(0, 5, (U, V), device="cuda:0").float() * 0.25
+    assert capi.load().rnnt_hip_maxplus_tries_lists(B, T, U, V) == 1
+    best = torch.empty((B, T, U), device="cuda:0")
+    arg = torch.empty((B, T, U), dtype=torch.int32, device="cuda:0")
+
+    def build(mode, repeats):
+        capi.call("rnnt_hip_set_maxplus_mode", mode)
+        try:
+            start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            ms = []
+            for _ in range(repeats):
+                best.fill_(float("nan"))
+                arg.fill_(-7)
+                start.record()
+                capi.call("rnnt_hip_maxplus_table", ptr(c.E), ptr(c.P), ptr(c.il), ptr(c.ll),
+                          ptr(best), ptr(arg), B, T, U, V, 0, None)
+                stop.record()
+                torch.cuda.synchronize()
+                ms.append(start.elapsed_time(stop))
+        finally:
+            capi.call("rnnt_hip_set_maxplus_mode", 0)
+        return min(ms[1:]), best.clone(), arg.clone()
+
+    every_ms, every_best, every_arg = build(1, 4)
+    lists_ms, lists_best, lists_arg = build(0, 4)
+    print("table, sample passes but 30 of 32 utterances are quantised: %.2f ms by default, "
+          "%.2f ms over every column" % (lists_ms, every_ms))
+    assert torch.equal(lists_arg, every_arg)
+    assert torch.equal(lists_best.view(torch.int32), every_best.view(torch.int32))
+    assert lists_ms <= 1.5 * every_ms
+
+
 # ------------------------------------------------------------------ the smaller configurations, whole
 # Fraction of gradient entries outside rel 1e-4 / abs 1e-5 end to end, each side with its own
 # log-normaliser: about three times what was measured, per configuration (egrads, pgrads).

@@ -109,6 +109,7 @@ struct RowLists {
   int n[kCdWaves];                // entries of each quarter (without the padding)
   float tau[kCdWaves];            // each wavefront's threshold for its own sub-maxima
   int bad[2];                     // a quarter did not fit: the list is not the whole set (by frame parity)
+  int quit[2];                    // every tile this frame's cells lie in is redone whole anyway
   float mtop[2][2][64];           // what the second wavefront of a block of label positions
   int marg[2][2][64];             // found, for the first one to merge ([parity][block][lane])
 };
@@ -448,15 +449,34 @@ __global__ __launch_bounds__(kCdThreads) void cand_rows_kernel(const TIO* __rest
   // wavefront finishes together (64 label positions of one frame) lie within a dozen cache lines,
   // and the next three frames fill the same lines.
   QuarterBits<kPieces, TIO> ahead;
-  if (tid == 0) L->bad[0] = L->bad[1] = 0;
+  // Once every tile (128 frames x 64 label positions) that a frame's cells lie in holds more
+  // flagged cells than are redone one by one, maxplus_kernel redoes all of them over every
+  // column whatever is found here: the workgroup then stops (the counters only grow).  An
+  // utterance whose scores do not suit lists -- while the sample's did -- so costs a frame or
+  // two per tile instead of the whole list pass.  One thread looks, a frame ahead; everybody
+  // reads its answer after the barrier in between.
+  auto tiles_lost = [&](int t) -> int {
+    if (phase == 0) return 0;
+    const int* tf = w.tile_fail + ((size_t)b * tiles_t + t / kCdTileT) * tiles_u;
+    for (int k = 0; 64 * k < Ub; ++k)
+      if (__hip_atomic_load(tf + k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) <= kCdTileLimit)
+        return 0;
+    return 1;
+  };
+  if (tid == 0) {
+    L->bad[0] = L->bad[1] = 0;
+    L->quit[0] = tiles_lost(t_lo);
+  }
   fetch_quarter<kVec, kPieces>(Eb + (size_t)t_lo * d.V, d.V, ahead);
   __syncthreads();
   int parity = 0;
   for (int t = t_lo; t < t_hi; ++t) {
     // this frame's row is in registers; the next one's is requested before the evaluation
     const int fp = (t - t_lo) & 1;
+    if (L->quit[fp]) break;  // uniform
     commit_quarter<kVec, kPieces>(ahead, d.V, d.blank, pitch, rank, fp, row, L);
     if (t + 1 < t_hi) fetch_quarter<kVec, kPieces>(Eb + (size_t)(t + 1) * d.V, d.V, ahead);
+    if (tid == 0) L->quit[fp ^ 1] = t + 1 < t_hi ? tiles_lost(t + 1) : 0;
     __syncthreads();
     if (tid == 0) L->bad[fp ^ 1] = 0;  // the next frame's flag: nobody sets it before the hand-over barrier
     const float tau = fmaxf(fmaxf(L->tau[0], L->tau[1]), fmaxf(L->tau[2], L->tau[3]));
