@@ -445,9 +445,15 @@ __global__ __launch_bounds__(kCdThreads) void cand_rows_kernel(const TIO* __rest
   for (int s = 1; s < 64; s <<= 1) nmax_first = max(nmax_first, __shfl_xor(nmax_first, s, 64));
   nmax_first = __builtin_amdgcn_readfirstlane(nmax_first);
 
-  // A cell's result is stored as it is found, 4 bytes per plane: in the skewed planes the cells a
-  // wavefront finishes together (64 label positions of one frame) lie within a dozen cache lines,
-  // and the next three frames fill the same lines.
+  // With at most 128 label positions (a lane meets one cell per frame) a lane keeps its results
+  // until a group of four anti-diagonals is complete -- its cells of consecutive frames are
+  // neighbours in the skewed planes -- and stores the group as one aligned 16-byte piece per plane:
+  // a 4-byte store per frame reaches memory as a sector of its own more often than not.  The
+  // group a lane is in depends on its label position, so a quarter of the lanes store per frame;
+  // what a workgroup's run of frames leaves incomplete at either end goes cell by cell.
+  const bool gathered = Ub <= 2 * 64;
+  float qtop[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+  int qarg[4] = {0, 0, 0, 0};
   QuarterBits<kPieces, TIO> ahead;
   // Once every tile (128 frames x 64 label positions) that a frame's cells lie in holds more
   // flagged cells than are redone one by one, maxplus_kernel redoes all of them over every
@@ -474,9 +480,12 @@ __global__ __launch_bounds__(kCdThreads) void cand_rows_kernel(const TIO* __rest
     // this frame's row is in registers; the next one's is requested before the evaluation
     const int fp = (t - t_lo) & 1;
     if (L->quit[fp]) break;  // uniform
+    // (asked before the next row is requested: loads return in order, and waiting for this
+    // answer behind the row's loads would wait for the row)
+    const int lost_next = (tid == 0 && t + 1 < t_hi) ? tiles_lost(t + 1) : 0;
     commit_quarter<kVec, kPieces>(ahead, d.V, d.blank, pitch, rank, fp, row, L);
     if (t + 1 < t_hi) fetch_quarter<kVec, kPieces>(Eb + (size_t)(t + 1) * d.V, d.V, ahead);
-    if (tid == 0) L->quit[fp ^ 1] = t + 1 < t_hi ? tiles_lost(t + 1) : 0;
+    if (tid == 0) L->quit[fp ^ 1] = lost_next;
     __syncthreads();
     if (tid == 0) L->bad[fp ^ 1] = 0;  // the next frame's flag: nobody sets it before the hand-over barrier
     const float tau = fmaxf(fmaxf(L->tau[0], L->tau[1]), fmaxf(L->tau[2], L->tau[3]));
@@ -628,7 +637,26 @@ __global__ __launch_bounds__(kCdThreads) void cand_rows_kernel(const TIO* __rest
         const float bound =
             tau + (ub == 0 ? ptau_first : (valid ? w.ptau[(size_t)b * d.U + u] : 0.0f));
         const bool ok = !bad && top > bound;
-        if (valid) {
+        if (gathered) {
+          const int dd = t + u, ph = dd & 3;  // per lane
+#pragma unroll
+          for (int k = 0; k < 4; ++k) {
+            qtop[k] = ph == k ? top : qtop[k];
+            qarg[k] = ph == k ? (ok ? at : -1) : qarg[k];
+          }
+          if (valid && (ph == 3 || t == t_hi - 1)) {
+            const int held = min(ph, t - t_lo);  // earlier cells of this group the lane holds
+            const size_t o = plane_at(d, b, u, dd - ph);  // the group's first anti-diagonal: 16-byte aligned
+            if (held == 3) {
+              *reinterpret_cast<float4*>(best + o) = make_float4(qtop[0], qtop[1], qtop[2], qtop[3]);
+              *reinterpret_cast<int4*>(arg + o) = make_int4(qarg[0], qarg[1], qarg[2], qarg[3]);
+            } else {
+#pragma unroll
+              for (int k = 0; k < 4; ++k)
+                if (k <= ph && k >= ph - held) { best[o + k] = qtop[k]; arg[o + k] = qarg[k]; }
+            }
+          }
+        } else if (valid) {
           const size_t o = plane_at(d, b, u, t + u);
           best[o] = top;
           arg[o] = ok ? at : -1;
