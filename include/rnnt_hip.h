@@ -92,7 +92,7 @@ int rnnt_hip_dense_grads(const float* emissions, const float* predictions, float
 
 /* Device bytes rnnt_hip_loss_forward/backward need between them: O(B*T*U) lattice planes,
  * O(B*(T+U)) vectors, and one O(B*U*V) entry -- the bf16 pieces of exp(predictions - row
- * maximum), 1.5 times the bytes of `predictions` with U rounded up to 32 (245 MB of the 535 MB
+ * maximum), 1.5 times the bytes of `predictions` with U rounded up to 32 (245 MB of the 575 MB
  * at B=32, T=2000, U=101, V=10000).  No entry of the size of `emissions`. */
 size_t rnnt_hip_loss_workspace_bytes(int B, int T, int U, int V);
 
