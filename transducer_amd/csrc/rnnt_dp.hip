@@ -9,8 +9,9 @@
 //     emit(t,u) = ((x + E[t,l_u])   + P[u,l_u])   - LN[t,u]   -> consumed by (t,u+1)
 // The hand-over to the next label position stays in registers inside a lane and crosses lanes
 // with one DPP wave shift; there is no barrier and no memory access on the dependent chain.
-// Operands are read from "skewed" planes [u][t+u] so that four steps are one 16-byte load per
-// lane, prefetched a group ahead.  This file is compiled with -ffp-contract=off: the rounding
+// Operands are read from "skewed" planes, indexed by anti-diagonal t+u in groups of four
+// (plane_at in rnnt_internal.h), so that four steps are one 16-byte load per lane and the lanes'
+// loads are neighbours in memory; they are requested several groups ahead.  This file is compiled with -ffp-contract=off: the rounding
 // sequence of every cell must equal the reference's.
 #include <atomic>
 #include <mutex>
@@ -162,29 +163,44 @@ __device__ inline void f4set(float4& v, int j, float x) {
 }
 
 // ------------------------------------------------------------------ skew / unskew
-// row-major [B,T,U] <-> skewed [B,U,Dp]; 64x64 tiles transposed through LDS so both sides
-// move whole cache lines.  Only cells inside the utterance's (T_b, U_b) extent are touched.
+// row-major [B,T,U] <-> skewed planes.  A block takes 64 label positions x 64 anti-diagonals
+// (16 groups of four: 1 KB of contiguous plane memory each) and their 127 frames t = dd - u, and
+// transposes through LDS so that the plane side moves 16-byte pieces next to each other and the
+// row-major side rows of consecutive label positions.  Only cells inside the utterance's
+// (T_b, U_b) extent are touched.  Grid: (anti-diagonal blocks, label blocks, B).
 __global__ __launch_bounds__(256) void skew_kernel(const float* __restrict__ src,
                                                    float* __restrict__ dstS,
                                                    const int* __restrict__ inLen,
                                                    const int* __restrict__ labLen, Dims d) {
-  __shared__ float tile[64][65];
-  const int b = blockIdx.z, t0 = blockIdx.x * 64, u0 = blockIdx.y * 64;
+  __shared__ float tile[64][65];  // [label position][anti-diagonal]
+  const int b = blockIdx.z, dd0 = blockIdx.x * 64, u0 = blockIdx.y * 64;
   int Tb, Ub;
   utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
-  if (t0 >= Tb || u0 >= Ub) return;
+  const int t_first = dd0 - u0 - 63;  // frames t_first .. t_first + 126 meet the tile
+  if (u0 >= Ub || t_first >= Tb || t_first + 126 < 0) return;
   const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
   const float* s = src + (size_t)b * d.T * d.U;
-#pragma unroll
-  for (int i = 0; i < 16; ++i) {
-    const int t = t0 + ty + 4 * i, u = u0 + tx;
-    tile[ty + 4 * i][tx] = (t < Tb && u < Ub) ? s[(size_t)t * d.U + u] : 0.0f;
+  for (int i = 0; i < 32; ++i) {
+    const int r = ty + 4 * i, t = t_first + r, u = u0 + tx, c = tx + r - 63;
+    if (c >= 0 && c < 64)
+      tile[tx][c] = (t >= 0 && t < Tb && u < Ub) ? s[(size_t)t * d.U + u] : 0.0f;
   }
   __syncthreads();
+  const size_t plane_b = (size_t)b * d.Ua * d.Dp;
 #pragma unroll
-  for (int i = 0; i < 16; ++i) {
-    const int u = u0 + ty + 4 * i, t = t0 + tx;
-    if (t < Tb && u < Ub) dstS[plane_at(d, b, u, t + u)] = tile[tx][ty + 4 * i];
+  for (int k = 0; k < 4; ++k) {
+    const int f = k * 256 + threadIdx.x, gl = f >> 6, ul = f & 63;
+    const int u = u0 + ul, g = (dd0 >> 2) + gl, tq = 4 * g - u;  // frame of the group's first cell
+    if (u >= Ub || tq + 3 < 0 || tq >= Tb) continue;
+    float* dst = dstS + plane_b + ((size_t)g * d.Ua + u) * 4;
+    if (tq >= 0 && tq + 3 < Tb) {
+      *reinterpret_cast<float4*>(dst) = make_float4(tile[ul][4 * gl], tile[ul][4 * gl + 1],
+                                                    tile[ul][4 * gl + 2], tile[ul][4 * gl + 3]);
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if (tq + j >= 0 && tq + j < Tb) dst[j] = tile[ul][4 * gl + j];
+    }
   }
 }
 
@@ -192,29 +208,37 @@ __global__ __launch_bounds__(256) void unskew_kernel(const float* __restrict__ s
                                                      float* __restrict__ dst,
                                                      const int* __restrict__ inLen,
                                                      const int* __restrict__ labLen, Dims d) {
-  __shared__ float tile[64][65];
-  const int b = blockIdx.z, t0 = blockIdx.x * 64, u0 = blockIdx.y * 64;
+  __shared__ float tile[64][65];  // [label position][anti-diagonal]
+  const int b = blockIdx.z, dd0 = blockIdx.x * 64, u0 = blockIdx.y * 64;
   int Tb, Ub;
   utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
-  if (t0 >= Tb || u0 >= Ub) return;
-  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  const int t_first = dd0 - u0 - 63;
+  if (u0 >= Ub || t_first >= Tb || t_first + 126 < 0) return;
+  const size_t plane_b = (size_t)b * d.Ua * d.Dp;
 #pragma unroll
-  for (int i = 0; i < 16; ++i) {
-    const int u = u0 + ty + 4 * i, t = t0 + tx;
-    tile[ty + 4 * i][tx] =
-        (t < Tb && u < Ub) ? srcS[plane_at(d, b, u, t + u)] : 0.0f;
+  for (int k = 0; k < 4; ++k) {
+    const int f = k * 256 + threadIdx.x, gl = f >> 6, ul = f & 63;
+    const int u = u0 + ul, g = (dd0 >> 2) + gl, tq = 4 * g - u;
+    float4 v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    // (a group that holds a cell of the lattice lies inside the plane: 4g < T + U)
+    if (u < Ub && tq + 3 >= 0 && tq < Tb)
+      v = *reinterpret_cast<const float4*>(srcS + plane_b + ((size_t)g * d.Ua + u) * 4);
+    tile[ul][4 * gl] = v.x;
+    tile[ul][4 * gl + 1] = v.y;
+    tile[ul][4 * gl + 2] = v.z;
+    tile[ul][4 * gl + 3] = v.w;
   }
   __syncthreads();
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
   float* o = dst + (size_t)b * d.T * d.U;
-#pragma unroll
-  for (int i = 0; i < 16; ++i) {
-    const int t = t0 + ty + 4 * i, u = u0 + tx;
-    if (t < Tb && u < Ub) o[(size_t)t * d.U + u] = tile[tx][ty + 4 * i];
+  for (int i = 0; i < 32; ++i) {
+    const int r = ty + 4 * i, t = t_first + r, u = u0 + tx, c = tx + r - 63;
+    if (c >= 0 && c < 64 && t >= 0 && t < Tb && u < Ub) o[(size_t)t * d.U + u] = tile[tx][c];
   }
 }
 
 // ------------------------------------------------------------------ gather
-// elS[u][t+u] = E[t, label_u]; eb[t] = E[t, blank]; pb[u] = P[u, blank]; pl[u] = P[u, label_u].
+// elS(u, t+u) = E[t, label_u]; eb[t] = E[t, blank]; pb[u] = P[u, blank]; pl[u] = P[u, label_u].
 // grid (ceil(T/256), U, B): a block serves 256 frames of one label position.
 template <typename TIO>
 __global__ __launch_bounds__(256) void gather_kernel(const TIO* __restrict__ E,
@@ -1767,8 +1791,9 @@ void carve_planes(void* base, const Dims& d, Planes* p, bool decode_only) {
 }
 
 // ------------------------------------------------------------------ launchers
+// tiles of 64 anti-diagonals x 64 label positions over all anti-diagonals t + u < T + U
 static dim3 tile_grid(const Dims& d) {
-  return dim3((d.T + 63) / 64, (d.U + 63) / 64, d.B);
+  return dim3((d.T + d.U + 62) / 64, (d.U + 63) / 64, d.B);
 }
 
 int launch_skew(const float* src, float* dstS, const int* inLen, const int* labLen, const Dims& d,
