@@ -176,6 +176,14 @@ int rnnt_hip_viterbi_decode_static(const float* emissions, const float* predicti
                                    rnnt_stream_t stream);
 size_t rnnt_hip_static_scratch_bytes(void);
 
+/* The entry points that take their own scratch (rnnt_hip_forward, _backward, _viterbi,
+ * _log_norms, _dense_grads, _viterbi_decode*, _maxplus_table) allocate it stream-ordered, as the
+ * reference's viterbi does (transducer/transducer_cuda.cu:364-369, 386-387), from a memory pool of
+ * the library's own that keeps freed blocks for the next call: the scratch of the largest call so
+ * far stays reserved on the device.  This hands it back to the driver (current device; call it
+ * when no such call is in flight).  No counterpart in the reference. */
+int rnnt_hip_release_scratch(void);
+
 /* ---- stage timing (diagnostic; no counterpart in the reference, whose only instrumentation
  * is wall-clock loops in transducer/benchmark.cpp:21-34) ---------------------------------- */
 

@@ -112,3 +112,26 @@ def test_chain_latency_floor_is_a_plausible_number_of_nanoseconds():
         assert lo < out.value < hi
     assert lib.rnnt_hip_chain_floor(3, 100, ctypes.byref(out)) == 1
     assert lib.rnnt_hip_chain_floor(0, 0, ctypes.byref(out)) == 1
+
+
+def test_scratch_pool_can_be_released_between_calls():
+    """The allocating entry points take their scratch from a pool that keeps freed blocks;
+    rnnt_hip_release_scratch hands them back to the driver, and the next call allocates afresh
+    with the same results."""
+    from util import DeviceCase, gpu_forward, gpu_log_norms, gpu_viterbi
+    rng = np.random.default_rng(3)
+    B, T, U, V = 2, 40, 9, 50
+    E = rng.standard_normal((B, T, V)).astype(np.float32)
+    P = rng.standard_normal((B, U, V)).astype(np.float32)
+    labels = rng.integers(1, V, (B, U - 1)).astype(np.int32)
+    il, ll = np.array([T, T - 3], np.int32), np.array([U - 1, U - 2], np.int32)
+    c = DeviceCase(E, P, labels, il, ll)
+    lib = capi.load()
+    LN = gpu_log_norms(c)
+    costs, alphas = gpu_forward(c, LN)
+    paths = gpu_viterbi(c, LN)
+    assert lib.rnnt_hip_release_scratch() == 0
+    assert lib.rnnt_hip_release_scratch() == 0   # nothing held: still fine
+    costs2, alphas2 = gpu_forward(c, LN)
+    assert np.array_equal(costs, costs2) and np.array_equal(np.nan_to_num(alphas), np.nan_to_num(alphas2))
+    assert np.array_equal(paths, gpu_viterbi(c, LN))

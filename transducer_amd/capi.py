@@ -29,6 +29,7 @@ SIGNATURES = {
     "rnnt_hip_viterbi_decode": (_I, [_F] * 5 + [_I] * 5 + [_F]),
     "rnnt_hip_viterbi_decode_static": (_I, [_F] * 5 + [_I] * 5 + [_F]),
     "rnnt_hip_static_scratch_bytes": (_Z, []),
+    "rnnt_hip_release_scratch": (_I, []),
     "rnnt_hip_viterbi_decode_bf16": (_I, [_F] * 5 + [_I] * 5 + [_F]),
     "rnnt_hip_viterbi_decode_f16": (_I, [_F] * 5 + [_I] * 5 + [_F]),
     "rnnt_hip_check_kernels": (_I, [_F]),

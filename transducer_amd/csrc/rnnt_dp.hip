@@ -759,12 +759,17 @@ __global__ __launch_bounds__(64 * W) void beta_kernel(Planes p, const int* __res
 }
 
 // ------------------------------------------------------------------ sparse gradient terms
-// The blank/label terms of transducer/transducer_cpu.cpp:95-141.  One thread per frame walks
-// the label positions from last to first, which is the order in which the reference subtracts
-// into a row of egrads, so repeated labels round the same way.  pgrads comes from the sums
-// the dalpha kernel kept.  add == 0: the terms are stored (the arrays were zero-filled);
-// add != 0: scale[b] (1 when scale is null) times the term is added to what the arrays hold.
-__global__ __launch_bounds__(256) void sparse_e_kernel(Planes p, float* __restrict__ egrads,
+// The blank/label terms of transducer/transducer_cpu.cpp:95-141, scattered into egrads from what
+// frame_terms_block (below) leaves: bsum[b][t], the finished value of column `blank` of frame t,
+// and emT[b][u][t], the label move's term of every cell.  One thread per frame walks the label
+// positions from last to first, which is the order in which the reference subtracts into a row
+// of egrads, so repeated labels round the same way; a label position's terms of 256 consecutive
+// frames are 1 KB in a row.  pgrads comes from the sums the dalpha kernel kept.  add == 0: the
+// terms are stored (the arrays were zero-filled); add != 0: scale[b] (1 when scale is null)
+// times the term is added to what the arrays hold.
+__global__ __launch_bounds__(256) void sparse_e_kernel(const float* __restrict__ bsum,
+                                                       const float* __restrict__ emT,
+                                                       float* __restrict__ egrads,
                                                        const int* __restrict__ labels,
                                                        const int* __restrict__ inLen,
                                                        const int* __restrict__ labLen,
@@ -777,55 +782,39 @@ __global__ __launch_bounds__(256) void sparse_e_kernel(Planes p, float* __restri
   if (Ub == 0 || t >= Tb) return;
   float* __restrict__ row = egrads + ((size_t)b * d.T + t) * d.V;
   const int* __restrict__ lab = labels + (size_t)b * (d.U - 1);
-  const float* __restrict__ dS = p.dS;
-  const float* __restrict__ wB = p.wB;
-  const float* __restrict__ wE = p.wE;
+  const float* __restrict__ em = emT + (size_t)b * d.U * d.T + t;
   const float sc = scale ? scale[b] : 1.0f;
-  const bool has_stay = t + 1 < Tb;
-  float blank_acc = (t == Tb - 1) ? -1.0f : 0.0f;
-  // Positions are taken eight at a time, last to first; the products of the next eight are
+  const float blank_total = bsum[(size_t)b * d.T + t];
+  // Positions are taken eight at a time, last to first; the terms of the next eight are
   // requested before the current eight are folded in, so the loop runs at the rate of the
   // memory pipe rather than one round trip per label position.
   constexpr int kChunk = 8;
-  struct Chunk { float ne[kChunk], em[kChunk]; };
+  struct Chunk { float em[kChunk]; };
   auto load_chunk = [&](int uhi) -> Chunk {  // positions uhi, uhi-1, ..., uhi-7 (those >= 0)
     Chunk c;
 #pragma unroll
-    for (int k = 0; k < kChunk; ++k) {
-      const int u = uhi - k;
-      const int uc = u > 0 ? u : 0;
-      const size_t o = plane_at(d, b, uc, t + uc), o1 = plane_at(d, b, uc, t + uc + 1);
-      // loads are unconditional (the planes are readable one past the utterance); what they
-      // return there is discarded by the selects
-      const float ne = dS[o1] * wB[o];      // dalpha[t+1,u]
-      const float em = dS[o1 + 4] * wE[o];  // dalpha[t,u+1]
-      c.ne[k] = has_stay ? ne : 0.0f;
-      c.em[k] = (u + 1 < Ub) ? em : 0.0f;
-    }
+    for (int k = 0; k < kChunk; ++k) c.em[k] = em[(size_t)max(uhi - k, 0) * d.T];
     return c;
   };
-  Chunk cur = load_chunk(Ub - 1);
-  for (int uhi = Ub - 1; uhi >= 0; uhi -= kChunk) {
+  Chunk cur = load_chunk(Ub - 2);  // the last position has no label move
+  for (int uhi = Ub - 2; uhi >= 0; uhi -= kChunk) {
     const Chunk nxt = load_chunk(uhi - kChunk);
 #pragma unroll
     for (int k = 0; k < kChunk; ++k) {
       const int u = uhi - k;
       if (u >= 0) {
-        blank_acc -= cur.ne[k];
-        if (u + 1 < Ub) {
-          const int l = clampi(lab[u], 0, d.V - 1);
-          // Label columns are updated with no-return hardware adds: nothing waits on them,
-          // and since this thread alone touches row t and its requests to one address stay
-          // in order, repeated labels still accumulate in the reference's order.
-          if (l == d.blank) blank_acc -= cur.em[k];
-          else unsafeAtomicAdd(&row[l], add ? sc * (-cur.em[k]) : -cur.em[k]);
-        }
+        const int l = clampi(lab[u], 0, d.V - 1);
+        // Label columns are updated with no-return hardware adds: nothing waits on them,
+        // and since this thread alone touches row t and its requests to one address stay
+        // in order, repeated labels still accumulate in the reference's order.  (A label move
+        // whose label is the blank is already part of the blank total.)
+        if (l != d.blank) unsafeAtomicAdd(&row[l], add ? sc * (-cur.em[k]) : -cur.em[k]);
       }
     }
     cur = nxt;
   }
-  if (add) row[d.blank] += sc * blank_acc;
-  else row[d.blank] = blank_acc;
+  if (add) row[d.blank] += sc * blank_total;
+  else row[d.blank] = blank_total;
 }
 
 // The same terms for a small vocabulary, added (times scale[b]) onto an egrads that holds the
@@ -835,7 +824,9 @@ __global__ __launch_bounds__(256) void sparse_e_kernel(Planes p, float* __restri
 // t, all lanes hit column l together, no conflicts), subtracts the terms there in the
 // reference's order, and then adds the rows to egrads with row-contiguous accesses.
 // Dynamic LDS: 64 * (V | 1) floats.
-__global__ __launch_bounds__(64) void sparse_e_rows_kernel(Planes p, float* __restrict__ egrads,
+__global__ __launch_bounds__(64) void sparse_e_rows_kernel(const float* __restrict__ bsum,
+                                                           const float* __restrict__ emT,
+                                                           float* __restrict__ egrads,
                                                            const int* __restrict__ labels,
                                                            const int* __restrict__ inLen,
                                                            const int* __restrict__ labLen,
@@ -852,35 +843,22 @@ __global__ __launch_bounds__(64) void sparse_e_rows_kernel(Planes p, float* __re
   const int t = min(t0 + lane, Tb - 1);  // lanes past the utterance walk its last frame, unused
   float* mine = rows + lane * pitch;
   const int* __restrict__ lab = labels + (size_t)b * (d.U - 1);
-  const float* __restrict__ dS = p.dS;
-  const float* __restrict__ wB = p.wB;
-  const float* __restrict__ wE = p.wE;
-  const bool has_stay = t + 1 < Tb;
-  float blank_acc = (t == Tb - 1) ? -1.0f : 0.0f;
+  const float* __restrict__ em = emT + (size_t)b * d.U * d.T + t;
   constexpr int kChunk = 16;
-  for (int uhi = Ub - 1; uhi >= 0; uhi -= kChunk) {
-    float ne[kChunk], em[kChunk];
+  for (int uhi = Ub - 2; uhi >= 0; uhi -= kChunk) {
+    float e[kChunk];
 #pragma unroll
-    for (int k = 0; k < kChunk; ++k) {
-      const int u = uhi - k, uc = u > 0 ? u : 0;
-      const size_t o = plane_at(d, b, uc, t + uc), o1 = plane_at(d, b, uc, t + uc + 1);
-      ne[k] = dS[o1] * wB[o];
-      em[k] = dS[o1 + 4] * wE[o];
-    }
+    for (int k = 0; k < kChunk; ++k) e[k] = em[(size_t)max(uhi - k, 0) * d.T];
 #pragma unroll
     for (int k = 0; k < kChunk; ++k) {
       const int u = uhi - k;
       if (u >= 0) {  // uniform
-        blank_acc -= has_stay ? ne[k] : 0.0f;
-        if (u + 1 < Ub) {
-          const int l = clampi(lab[u], 0, d.V - 1);
-          if (l == d.blank) blank_acc -= em[k];
-          else mine[l] -= em[k];
-        }
+        const int l = clampi(lab[u], 0, d.V - 1);
+        if (l != d.blank) mine[l] -= e[k];
       }
     }
   }
-  mine[d.blank] += blank_acc;
+  mine[d.blank] += bsum[(size_t)b * d.T + t];
   __syncthreads();
   const float sc = scale ? scale[b] : 1.0f;
   const int nrows = min(64, Tb - t0);
@@ -1937,18 +1915,19 @@ int launch_beta(const Planes& p, const int* labels, const int* inLen, const int*
   return kOk;
 }
 
-int launch_sparse(const Planes& p, float* egrads, float* pgrads, const int* labels,
-                  const int* inLen, const int* labLen, const float* scale, bool add,
-                  const Dims& d, hipStream_t s) {
+int launch_sparse(const Planes& p, const float* bsum, const float* emT, float* egrads,
+                  float* pgrads, const int* labels, const int* inLen, const int* labLen,
+                  const float* scale, bool add, const Dims& d, hipStream_t s) {
   if (d.B == 0 || d.T == 0 || d.U == 0) return kOk;
+  if (!bsum || !emT) return fail(kInvalid, "sparse terms: the per-frame terms were not formed");
   const size_t rows_bytes = sizeof(float) * 64 * (size_t)(d.V | 1);
   if (add && rows_bytes <= 64 * 1024 && labels != nullptr) {
     hipLaunchKernelGGL(sparse_e_rows_kernel, dim3((d.T + 63) / 64, d.B), dim3(64), rows_bytes, s,
-                       p, egrads, labels, inLen, labLen, scale, d);
+                       bsum, emT, egrads, labels, inLen, labLen, scale, d);
     RNNT_LAUNCH_CHECK("sparse_e_rows_kernel");
   } else {
-    hipLaunchKernelGGL(sparse_e_kernel, dim3((d.T + 255) / 256, d.B), dim3(256), 0, s, p, egrads,
-                       labels, inLen, labLen, scale, add ? 1 : 0, d);
+    hipLaunchKernelGGL(sparse_e_kernel, dim3((d.T + 255) / 256, d.B), dim3(256), 0, s, bsum, emT,
+                       egrads, labels, inLen, labLen, scale, add ? 1 : 0, d);
     RNNT_LAUNCH_CHECK("sparse_e_kernel");
   }
   if (pgrads == nullptr) return kOk;  // the caller adds those terms itself
@@ -1967,10 +1946,13 @@ int launch_post_beta(const Planes& p, const float* mE, const float* mP, float* W
     return fail(kInvalid, "W images hold at most %d label positions", WImages::kCols);
   // W tiles: 64 label positions x 64 anti-diagonals (all anti-diagonals below Tw + Up), or for
   // the images 64 label positions x 64 frames
-  const int wx = img.e ? Tw / 64 : (Tw + Up + 62) / 64, wy = (Up + 63) / 64, nw = wx * wy * d.B;
+  // (Wn == nullptr: no W at all, only the per-frame terms)
+  const int wx = img.e ? Tw / 64 : (Tw + Up + 62) / 64, wy = (Up + 63) / 64;
+  const int nw = (Wn || img.e) ? wx * wy * d.B : 0;
   if ((bsum == nullptr) != (emT == nullptr))
     return fail(kInvalid, "post_beta: the blank totals and the label-move terms come together");
   const int sx = (d.T + 4 * kBsFrames - 1) / (4 * kBsFrames), ns = bsum ? sx * d.B : 0;
+  if (nw + ns == 0) return kOk;
   hipLaunchKernelGGL(post_beta_kernel, dim3(nw + ns), dim3(256), 0, s, p, mE, mP, Wn, Wt, bsum,
                      emT, labels, inLen, labLen, d, Up, Tw, wx, wy, nw, sx, img);
   RNNT_LAUNCH_CHECK("post_beta_kernel");

@@ -164,10 +164,11 @@ int launch_beta(const Planes& p, const int* labels, const int* inLen, const int*
 // Sparse blank/label terms.  add == false: written onto zero-filled egrads/pgrads exactly as
 // the reference's backward leaves them.  add == true: added, times scale[b] (1 when scale is
 // null), onto arrays that already hold the dense part.
-// pgrads == nullptr: only the egrads terms.
-int launch_sparse(const Planes& p, float* egrads, float* pgrads, const int* labels,
-                  const int* inLen, const int* labLen, const float* scale, bool add,
-                  const Dims& d, hipStream_t s);
+// pgrads == nullptr: only the egrads terms.  bsum ([B,T]) and emT ([B,U,T]) are the per-frame
+// terms launch_post_beta forms from the finished dalpha plane.
+int launch_sparse(const Planes& p, const float* bsum, const float* emT, float* egrads,
+                  float* pgrads, const int* labels, const int* inLen, const int* labLen,
+                  const float* scale, bool add, const Dims& d, hipStream_t s);
 // After the dalpha walk, in one launch: the W planes (both orientations, from the skewed dalpha
 // and LN planes) and, with bsum != nullptr, bsum[b,t] = what the blank/label terms leave in
 // egrads[b,t,blank] (for folding into the dense kernel's write-out).
@@ -188,7 +189,8 @@ struct WImages {
   static size_t p_bytes(int B, int Tw) { return (size_t)B * (Tw / 32) * 3 * kPPlane * 4; }
 };
 // bsum ([B,T]) and emT ([B,U,T]): the per-frame blank totals and the per-cell label-move terms
-// the dense egrads kernel folds in (SparseTerms); both null: not formed.
+// that the dense egrads kernel folds in (SparseTerms) or launch_sparse scatters; both null: not
+// formed.  Wn == nullptr (and no images): no W planes, only those terms (mE, mP unused).
 int launch_post_beta(const Planes& p, const float* mE, const float* mP, float* Wn, float* Wt,
                      float* bsum, float* emT, const int* labels, const int* inLen,
                      const int* labLen, const Dims& d, hipStream_t s,
