@@ -438,6 +438,9 @@ def main():
     ap.add_argument("--workload", default="cfg4", choices=sorted(WORKLOADS))
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--graph", action="store_true",
+                    help="also time the step replayed from a captured HIP graph "
+                         "(reported as graph_replay_ms_per_step; loss workloads only)")
     ap.add_argument("--maxplus-mode", type=int, default=0, choices=(0, 1, 2),
                     help="best-path workloads: how the table of best labels is built "
                          "(rnnt_hip_set_maxplus_mode: 0 default, 1 every column, 2 lists)")
@@ -506,6 +509,21 @@ def main():
     # from the workspace the last forward call left
     fwd_ms = time_steps(step_fwd, args.steps)
     bwd_ms = time_steps(step_bwd, args.steps)
+    # the same step replayed from a captured HIP graph (the two entry points allocate nothing and
+    # launch kernels only): what a training loop that captures its step pays per launch less.
+    # Reported beside `value`, which stays the eager figure the reference's script measures.
+    graph_ms = None
+    if args.graph:
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            gs = ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+            capi.call("rnnt_hip_loss_forward" + suffix, p(E), p(P), p(labels), p(d_il), p(d_ll),
+                      p(costs), p(ws), nbytes, B, T, U1, V, 0, gs)
+            capi.call("rnnt_hip_loss_backward" + suffix, p(E), p(P), p(labels), p(d_il), p(d_ll),
+                      p(deltas), p(egrads), p(pgrads), p(ws), nbytes, B, T, U1, V, 0, gs)
+        graph.replay()
+        torch.cuda.synchronize()
+        graph_ms = time_steps(graph.replay, args.steps)
     per_launch, per_step = stage_times(capi, step, args.steps)
     capi.call("rnnt_hip_check_kernels", stream)          # no lattice kernel gave up a wait
     checks = output_checks(costs, egrads, pgrads, il, ll)
@@ -575,6 +593,7 @@ def main():
         "ms_per_step": round(ms_per_step, 4),
         "fwd_ms": round(fwd_ms, 4),
         "bwd_ms": round(bwd_ms, 4),
+        "graph_replay_ms_per_step": round(graph_ms, 4) if graph_ms is not None else None,
         "higher_is_better": False,
         "scaling": "weak",
         "vs_baseline": (round(ms_per_step / opt["published_ms"], 5) if opt.get("published_ms")
