@@ -307,6 +307,35 @@ def test_long_label_axis_uses_more_cells_per_lane():
     assert np.array_equal(gpu_viterbi(c, LN), oracle.viterbi(E, P, LN, il, ll))
 
 
+@pytest.mark.parametrize("T", [1, 6, 45])
+@pytest.mark.parametrize("U", [128, 129, 192, 256, 257, 300, 512, 513, 768, 1000])
+def test_label_axes_dealt_to_several_wavefronts_carry_the_reference_bits(T, U):
+    """From 65 label positions the alpha walk and from 129 the dalpha walk deal the label axis to
+    two or four wavefronts of one workgroup, which hand the boundary column's score on through
+    LDS and wait for each other's progress counters (four from 257 positions; there a lane's
+    positions of the dalpha walk are 64 apart).  U counts the rows of predictions and sits on
+    either side of every change of that split; T = 1 and 6 leave most wavefronts with less than
+    one or two groups of four steps, 45 lets them fall the few groups behind that they run at.
+    Same bars as everywhere: the reference's bits in every alpha, dalpha and sparse term, the
+    exact path."""
+    cfg = small_config(3, T, U - 1, 6, ragged=True)
+    E, P, labels, il, ll = unpack(make_inputs(cfg, seed=1000 * T + U))
+    il[0], ll[0] = T, U - 1          # one utterance uses every wavefront
+    il[1], ll[1] = max(T - 2, 1), (U - 1) // 2   # one ends inside the label axis
+    c = DeviceCase(E, P, labels, il, ll)
+    LN = oracle.log_norms_naive(E, P, il, ll)
+    costs_o, alphas_o = oracle.forward(E, P, LN, labels, il, ll)
+    costs, alphas = gpu_forward(c, LN)
+    assert_same_bits(costs, costs_o, what="costs")
+    assert_same_bits(alphas, alphas_o, what="alphas")
+    eg, pg, lng = gpu_backward(c, alphas, LN)
+    eg_o, pg_o, lng_o = oracle.backward(E, P, np.nan_to_num(alphas_o), LN, labels, il, ll)
+    assert_same_bits(lng, lng_o, what="lngrads")
+    assert_same_bits(eg, eg_o, what="egrads (sparse)")
+    assert_same_bits(pg, pg_o, what="pgrads (sparse)")
+    assert np.array_equal(gpu_viterbi(c, LN), oracle.viterbi(E, P, LN, il, ll))
+
+
 @pytest.mark.parametrize("T,U,V", [(40, 1024, 9), (30, 1025, 9), (50, 1500, 7), (24, 2100, 520),
                                    (300, 1300, 5)])
 def test_label_axis_longer_than_one_block_of_1024_positions(T, U, V):
