@@ -1827,12 +1827,13 @@ int launch_alpha(const Planes& p, const int* inLen, const int* labLen, float* co
   // array (one float per step and boundary) fits LDS
   const int cpl = block_cells_per_lane(d), nblocks = label_blocks(d);
   const int stride = d.Dp;
-  // (two wavefronts up to 256 label positions, where a lane then owns one or two of them; from
-  // eight positions a lane on -- 257 label positions and more in one block -- four wavefronts, if
-  // their three hand-over arrays fit LDS: a step costs a wavefront one log-sum-exp per position
-  // it owns, and the step is what a lattice is bound by)
+  // (two wavefronts up to 128 label positions, four beyond -- one, two or four positions a lane
+  // -- if their three hand-over arrays fit LDS: a step costs a wavefront one log-sum-exp per
+  // position it owns, and the step is what a lattice is bound by.  B=8 T=2000, 129..256 label
+  // positions: 262 ns a step with two wavefronts of two positions, 160 with four of one, what
+  // 101 positions on two wavefronts take)
   const bool single_block = nblocks == 1;
-  const int W = (single_block && cpl >= 8 && 3 * stride * sizeof(float) <= 144 * 1024) ? 4
+  const int W = (single_block && cpl >= 4 && 3 * stride * sizeof(float) <= 144 * 1024) ? 4
                 : (cpl >= 2 && stride * sizeof(float) <= 48 * 1024) ? 2 : 1;
   const size_t lds = W > 1 ? sizeof(float) * (size_t)(W - 1) * stride : 0;
   int* trouble = nullptr;
@@ -1853,7 +1854,7 @@ int launch_alpha(const Planes& p, const int* inLen, const int* labLen, float* co
     break;
       CASE(1, 1, false) CASE(2, 1, false) CASE(4, 1, false) CASE(8, 1, false) CASE(16, 1, false)
       CASE(1, 2, false) CASE(2, 2, false) CASE(4, 2, false) CASE(8, 2, false)
-      CASE(2, 4, false) CASE(4, 4, false)
+      CASE(1, 4, false) CASE(2, 4, false) CASE(4, 4, false)
       CASE(16, 1, true) CASE(8, 2, true)  // several blocks: always 1024 positions each
 #undef CASE
       default:
@@ -1878,12 +1879,14 @@ int launch_beta(const Planes& p, const int* labels, const int* inLen, const int*
   if (d.B == 0 || d.T == 0 || d.U == 0) return kOk;
   const int cpl = block_cells_per_lane(d), nblocks = label_blocks(d);
   // wavefronts: one up to 128 label positions (a step of this walk is a handful of
-  // instructions a position, and the hand-over would cost as much again), two up to 256, four
-  // beyond, if their hand-over arrays fit LDS; one per block when the axis takes several launches
+  // instructions a position, and the hand-over would cost as much again), four beyond (two if
+  // only their hand-over array fits LDS); one per block when the axis takes several launches.
+  // (129..256 label positions, B=8 T=2000: 70 ns a step with two wavefronts of two positions, 57
+  // with four of one)
   const int stride = d.Dp;
   const bool single_block = nblocks == 1;
   const int W = !single_block ? 1
-                : (cpl >= 8 && 3 * stride * sizeof(float) <= 144 * 1024) ? 4
+                : (cpl >= 4 && 3 * stride * sizeof(float) <= 144 * 1024) ? 4
                 : (cpl >= 4 && stride * sizeof(float) <= 48 * 1024) ? 2 : 1;
   const size_t lds = W > 1 ? sizeof(float) * (size_t)(W - 1) * stride : 0;
   int* trouble = nullptr;
@@ -1904,7 +1907,7 @@ int launch_beta(const Planes& p, const int* labels, const int* inLen, const int*
     break;
       CASE(1, 1, false) CASE(2, 1, false) CASE(4, 1, false) CASE(8, 1, false) CASE(16, 1, false)
       CASE(2, 2, false) CASE(4, 2, false) CASE(8, 2, false)
-      CASE(2, 4, false) CASE(4, 4, false)
+      CASE(1, 4, false) CASE(2, 4, false) CASE(4, 4, false)
       CASE(16, 1, true)
 #undef CASE
       default:
