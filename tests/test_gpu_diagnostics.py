@@ -18,9 +18,13 @@ from transducer_amd.synthetic import make_inputs, small_config  # noqa: E402
 KEYS = ("emissions", "predictions", "labels", "input_lengths", "label_lengths")
 
 
-def test_a_wait_that_runs_out_raises_the_flag_and_the_kernel_still_finishes():
+@pytest.mark.parametrize("U", [100, 400])
+def test_a_wait_that_runs_out_raises_the_flag_and_the_kernel_still_finishes(U):
+    """101 label positions: two wavefronts of one workgroup wait for each other; 401: the alpha
+    walk also runs the two halves of the label axis as two workgroups side by side, the upper
+    one waiting (with the same bound) for the scores the lower one writes to memory."""
     lib = capi.load()
-    d = make_inputs(small_config(2, 300, 100, 16, ragged=False), seed=9)  # 101 positions: two wavefronts
+    d = make_inputs(small_config(2, 300, U, 16, ragged=False), seed=9)
     E, P, labels, il, ll = (d[k] for k in KEYS)
     LN = oracle.log_norms_naive(E, P, il, ll)
     want_costs, _ = oracle.forward(E, P, LN, labels, il, ll)

@@ -336,6 +336,32 @@ def test_label_axes_dealt_to_several_wavefronts_carry_the_reference_bits(T, U):
     assert np.array_equal(gpu_viterbi(c, LN), oracle.viterbi(E, P, LN, il, ll))
 
 
+@pytest.mark.parametrize("B,T,U", [(11, 300, 400), (3, 700, 258), (17, 150, 512), (96, 40, 300),
+                                   (97, 40, 300)])
+def test_two_halves_of_a_label_axis_walked_side_by_side_carry_the_reference_bits(B, T, U):
+    """257 .. 512 label positions in a batch of at most 96 utterances: the alpha walk runs the two
+    halves of the label axis as two workgroups at the same time; the scores of the boundary
+    column cross through memory, each with the number of its step beside it, and the upper half
+    asks again for what was not there yet.  Long enough lattices that the upper half runs its
+    steady state a few groups of steps behind the lower one; batches that fill the last eight
+    workgroup slots only partly; 97 utterances take the one-workgroup walk again.  U counts the
+    rows of predictions."""
+    cfg = small_config(B, T, U - 1, 5, ragged=True)
+    E, P, labels, il, ll = unpack(make_inputs(cfg, seed=B * 1000 + U))
+    il[0], ll[0] = T, U - 1                  # one utterance uses both halves to the end
+    il[1], ll[1] = max(T // 3, 1), 255       # one ends at the boundary: 256 positions
+    il[2], ll[2] = T, 256                    # one puts a single position into the upper half
+    c = DeviceCase(E, P, labels, il, ll)
+    LN = oracle.log_norms_naive(E, P, il, ll)
+    costs_o, alphas_o = oracle.forward(E, P, LN, labels, il, ll)
+    for _ in range(2):                       # the second call finds the first one's entries
+        costs, alphas = gpu_forward(c, LN)
+        assert_same_bits(costs, costs_o, what="costs")
+        assert_same_bits(alphas, alphas_o, what="alphas")
+    from transducer_amd import capi
+    assert capi.load().rnnt_hip_check_kernels(None) == 0
+
+
 @pytest.mark.parametrize("T,U,V", [(40, 1024, 9), (30, 1025, 9), (50, 1500, 7), (24, 2100, 520),
                                    (300, 1300, 5)])
 def test_label_axis_longer_than_one_block_of_1024_positions(T, U, V):

@@ -289,19 +289,41 @@ __global__ __launch_bounds__(256) void gather_kernel(const TIO* __restrict__ E,
 // null for the last block) and the next one reads them from `ghin` (null for the first block).
 // kMulti: this launch is one of several blocks (the hand-over code is compiled in only then: in
 // the single-block kernel even an unused hand-over load costs the walk its prefetch distance).
-template <int C, int W, bool kMulti>
+// kLive (with kMulti): the two blocks of a label axis of up to 128 C W positions run at the same
+// time, as two workgroups on two CUs of one XCD (with few utterances and many label positions
+// one CU's wavefronts are what holds the walk).  The boundary column's scores then cross in
+// `live` ([B][hand_stride] 64-bit words, zero before the launch): entry s is the score entering
+// step s with s + 1 in its upper half, so that a reader can tell a written entry by itself --
+// one store, no fence, no separate counter.  The upper block asks for its entries four groups
+// ahead like every other operand (lane j for entry 4g + j), checks the tags when it comes to
+// use them, and asks again (bounded, like the waits inside a workgroup) if the lower block has
+// not got there yet; it starts kLiveLag groups behind, so that in the steady state what it asks
+// for has long been written.  Workgroups are dispatched in launch order and an utterance's
+// lower block has the smaller index, so the block that is waited for is always running or done.
+constexpr int kLiveLag = 12;
+constexpr int kLiveWaveLag = 2;  // groups between the wavefronts of a live block at the start (8 elsewhere)
+template <int C, int W, bool kMulti, bool kLive = false>
 __global__ __launch_bounds__(64 * W) void alpha_kernel(Planes p, const int* __restrict__ inLen,
                                                        const int* __restrict__ labLen,
                                                        float* __restrict__ costs, Dims d,
                                                        int hand_stride, int spin_limit,
                                                        int* __restrict__ trouble, int u_base,
                                                        const float* __restrict__ ghin,
-                                                       float* __restrict__ ghout) {
+                                                       float* __restrict__ ghout,
+                                                       unsigned long long* __restrict__ live) {
+  static_assert(kMulti || !kLive, "live blocks are blocks");
   extern __shared__ __attribute__((aligned(16))) float hand[];  // [W-1][hand_stride]: entry s =
                                                                 // score handed to step s
   __shared__ int done[W];          // steps a wavefront has published
   __shared__ unsigned long long etab[32];  // expf's table (rnnt_libm.h)
-  const int b = blockIdx.x, lane = threadIdx.x & 63;
+  // live blocks: workgroups go round the 8 XCDs in launch order; ids i and i + 8 share one, and
+  // with it the L2 the boundary scores cross in
+  const int live_half = kLive ? (blockIdx.x >> 3) & 1 : 0;
+  const int b = kLive ? (blockIdx.x >> 4) * 8 + (blockIdx.x & 7) : blockIdx.x, lane = threadIdx.x & 63;
+  if (kLive) {
+    if (b >= d.B) return;
+    u_base = live_half * 64 * C * W;
+  }
   const int wave = W > 1 ? __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) : 0;
   int Tb, Ub;
   utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
@@ -315,9 +337,33 @@ __global__ __launch_bounds__(64 * W) void alpha_kernel(Planes p, const int* __re
   const int u0 = u_base + (wave * 64 + lane) * C;
   const int gstride = plane_group_stride(d);
   const bool first_column = u_base == 0 && wave == 0;  // lane 0 owns the lattice's column u = 0
-  const float* gin = (kMulti && ghin) ? ghin + (size_t)b * hand_stride : nullptr;
-  float* gout = (kMulti && ghout) ? ghout + (size_t)b * hand_stride : nullptr;
+  const float* gin = (kMulti && !kLive && ghin) ? ghin + (size_t)b * hand_stride : nullptr;
+  float* gout = (kMulti && !kLive && ghout) ? ghout + (size_t)b * hand_stride : nullptr;
   if (kMulti && gout && threadIdx.x == 0) gout[0] = kOutside;  // nothing enters step 0
+  // live blocks: block 0 writes the entries, block 1 reads them
+  unsigned long long* lrow = kLive ? live + (size_t)b * hand_stride : nullptr;
+  const bool live_in = kLive && live_half == 1, live_out = kLive && live_half == 0;
+  auto live_entry = [](int s, float x) -> unsigned long long {
+    return ((unsigned long long)(unsigned)(s + 1) << 32) | (unsigned long long)__float_as_uint(x);
+  };
+  auto live_load = [&](int s) -> unsigned long long {
+    return __hip_atomic_load(lrow + s, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  };
+  // Asking again for an entry that was not there yet: the load and its wait are one opaque
+  // statement, so that the compiler's count of the loads in flight in the walk's main loop (the
+  // operands of the next four groups) stays exact -- a loop around a load it knows of makes it
+  // wait for all of them at every use.
+  auto live_reload = [&](int s) -> unsigned long long {
+    unsigned long long e;
+    const unsigned long long* q = lrow + s;
+    asm volatile("global_load_dwordx2 %0, %1, off sc1\n\ts_waitcnt vmcnt(0)"
+                 : "=&v"(e)
+                 : "v"(q)
+                 : "memory");
+    return e;
+  };
+  if (live_out && threadIdx.x == 0)  // nothing enters step 0
+    __hip_atomic_store(lrow, live_entry(0, kOutside), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   exp2_table_to_lds(etab);
   if (W > 1) {
     if (threadIdx.x < W) done[threadIdx.x] = 0;
@@ -353,6 +399,7 @@ __global__ __launch_bounds__(64 * W) void alpha_kernel(Planes p, const int* __re
     float4 ln[C], el[C];
     float eb[C + 3];
     float4 gh;  // scores entering the block's first column from the block below
+    unsigned long long lv;  // the same, tagged, from the block running beside this one: lane j holds entry 4g + j
   };
   auto load_group = [&](int g) -> Group {
     Group r;
@@ -366,10 +413,18 @@ __global__ __launch_bounds__(64 * W) void alpha_kernel(Planes p, const int* __re
     if constexpr (kMulti) {
       r.gh = make_float4(kOutside, kOutside, kOutside, kOutside);
       if (gin) r.gh = *reinterpret_cast<const float4*>(gin + 4 * g);  // uniform
+      if constexpr (kLive) {
+        // every wavefront of both blocks asks (only wavefront 0 of the upper block takes the
+        // answer): a load under a condition would have its result copied, hence waited for,
+        // right where it is asked for -- and so would a load from an address all lanes share,
+        // which the compiler moves to scalar registers at once
+        r.lv = live_load(4 * g + (lane & 3));
+      }
     }
     return r;
   };
 
+  unsigned live_sink = 0;
   int avail = 0;  // steps the wavefront below is known to have published
   auto wait_for = [&](int need) {
     // LDS serves a wavefront's requests in order, so no hardware fence is needed on either
@@ -390,6 +445,30 @@ __global__ __launch_bounds__(64 * W) void alpha_kernel(Planes p, const int* __re
     for (int j = 0; j < 4; ++j) f4set(hin, j, (first_column && 4 * g + j < Tb) ? kNegInf : kOutside);
     if constexpr (kMulti) {
       if (gin) hin = cur.gh;  // wavefront 0: from the block below
+      if constexpr (kLive) {
+        // Wavefront 0 of the upper block takes what it asked for: lanes 0 .. 3 hold the four
+        // entries and check their tags.  Every other wavefront folds the answer into a word
+        // that is looked at once, at the very end: a result nobody reads would have its
+        // registers reused at once, and that reuse waits for the load.
+        if (live_in && wave == 0) {  // uniform
+          unsigned long long e = cur.lv;
+          int spins = 0;
+          while (__builtin_amdgcn_ballot_w64(lane < 4 &&
+                                             (unsigned)(e >> 32) != (unsigned)(4 * g + lane + 1))) {
+            if (spins++ >= spin_limit) {  // an entry was not written when it was asked for
+              if (lane == 0) *reinterpret_cast<volatile int*>(trouble) = 1;
+              break;
+            }
+            __builtin_amdgcn_s_sleep(2);
+            e = live_reload(4 * g + (lane & 3));
+          }
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            f4set(hin, j, __int_as_float(__builtin_amdgcn_readlane((int)(unsigned)e, j)));
+        } else {
+          live_sink ^= (unsigned)cur.lv;
+        }
+      }
     }
     if (W > 1 && wave > 0) {
       wait_for(4 * g + 3);  // the scores entering steps 4g .. 4g+3 left steps 4g-1 .. 4g+2
@@ -435,6 +514,14 @@ __global__ __launch_bounds__(64 * W) void alpha_kernel(Planes p, const int* __re
 #pragma unroll
         for (int j = 0; j < 4; ++j) gout[4 * g + 1 + j] = gsend[j];
       }
+      if constexpr (kLive) {
+        if (live_out && wave == W - 1 && lane == 63) {
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            __hip_atomic_store(lrow + 4 * g + 1 + j, live_entry(4 * g + 1 + j, gsend[j]),
+                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+      }
     }
     if (W > 1 && wave < W - 1 && lane == 0) {  // entries 4g+1 .. 4g+4, then the progress
 #pragma unroll
@@ -446,9 +533,22 @@ __global__ __launch_bounds__(64 * W) void alpha_kernel(Planes p, const int* __re
   // four register sets rotate (no copies): a group's loads are requested four groups (16
   // steps, more than a microsecond) ahead -- the planes of a long batch do not fit L2
   auto clamp_g = [&](int g) { return g < ngroups ? g : ngroups - 1; };
+  if constexpr (kLive) {
+    if (live_in && wave == 0) {  // the upper block starts kLiveLag groups behind (or when the lower is done)
+      const int far = min(4 * ngroups, 4 * kLiveLag);
+      int spins = 0;
+      while ((unsigned)(live_load(far) >> 32) != (unsigned)(far + 1)) {
+        if (spins++ >= spin_limit) {
+          if (lane == 0) *reinterpret_cast<volatile int*>(trouble) = 1;
+          break;
+        }
+        __builtin_amdgcn_s_sleep(8);
+      }
+    }
+  }
   Group q0 = load_group(0), q1 = load_group(clamp_g(1)), q2 = load_group(clamp_g(2)),
         q3 = load_group(clamp_g(3));
-  if (W > 1 && wave > 0) wait_for(min(4 * ngroups, 4 * 8 * wave));  // fall a few groups behind
+  if (W > 1 && wave > 0) wait_for(min(4 * ngroups, 4 * (kLive ? kLiveWaveLag : 8) * wave));  // fall a few groups behind
   const std::true_type whole;
   const std::false_type partial;
   const int nwhole = nsteps >> 2;  // groups with all four steps
@@ -473,6 +573,9 @@ __global__ __launch_bounds__(64 * W) void alpha_kernel(Planes p, const int* __re
 #pragma unroll
   for (int c = 0; c < C; ++c)
     if (u0 + c == Ub - 1) costs[b] = -stay[c];
+  if constexpr (kLive) {
+    if (spin_limit < 0 && live_sink == 1u) *reinterpret_cast<volatile int*>(trouble) = 1;  // never
+  }
 }
 
 
@@ -1820,6 +1923,17 @@ static int label_blocks(const Dims& d) {
   return (d.U + width - 1) / width;
 }
 
+__global__ void clear_words_kernel(int* x, int n) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i < n) x[i] = 0;
+}
+
+// Whether the alpha walk takes a label axis as two blocks running side by side (the two
+// hand-over vectors of the planes then hold one array of 64-bit entries).
+static bool alpha_live_blocks(const Dims& d) {
+  return d.Ua == 512 && d.B <= 96 && label_blocks(d) == 1;
+}
+
 int launch_alpha(const Planes& p, const int* inLen, const int* labLen, float* costs,
                  const Dims& d, hipStream_t s) {
   if (d.B == 0) return kOk;
@@ -1838,6 +1952,25 @@ int launch_alpha(const Planes& p, const int* inLen, const int* labLen, float* co
   const size_t lds = W > 1 ? sizeof(float) * (size_t)(W - 1) * stride : 0;
   int* trouble = nullptr;
   RNNT_TRY(trouble_flag(&trouble));
+  // 257 .. 512 label positions and few enough utterances that the device has CUs to spare: two
+  // blocks of 256 positions side by side on two CUs, four wavefronts of one position a lane each
+  // (B=8 T=10000, 401 positions: 176 ns a step against 235 on one CU; from about a hundred
+  // utterances on the planes' traffic holds both forms, B=128 T=2000: 241 ns)
+  if (alpha_live_blocks(d) && W == 4) {
+    unsigned long long* live = reinterpret_cast<unsigned long long*>(p.hand[0]);
+    const int words = 2 * d.B * stride;
+    hipLaunchKernelGGL(clear_words_kernel, dim3((words + 255) / 256), dim3(256), 0, s,
+                       reinterpret_cast<int*>(live), words);
+    RNNT_LAUNCH_CHECK("clear_words_kernel");
+    if (lds > 64 * 1024)
+      RNNT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(alpha_kernel<1, 4, true, true>),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    hipLaunchKernelGGL((alpha_kernel<1, 4, true, true>), dim3(16 * ((d.B + 7) / 8)), dim3(256), lds, s, p,
+                       inLen, labLen, costs, d, stride, g_spin_limit, trouble, 0, nullptr, nullptr,
+                       live);
+    RNNT_LAUNCH_CHECK("alpha_kernel (live blocks)");
+    return kOk;
+  }
   for (int k = 0; k < nblocks; ++k) {  // lowest block first
     const float* ghin = k == 0 ? nullptr : p.hand[(k - 1) & 1];
     float* ghout = k == nblocks - 1 ? nullptr : p.hand[k & 1];
@@ -1850,7 +1983,7 @@ int launch_alpha(const Planes& p, const int* inLen, const int* labLen, float* co
                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));   \
     hipLaunchKernelGGL((alpha_kernel<C, W, M>), dim3(d.B), dim3(64 * W), lds, s, p, inLen,  \
                        labLen, costs, d, stride, g_spin_limit, trouble, u_base, ghin,        \
-                       ghout);                                                               \
+                       ghout, nullptr);                                                      \
     break;
       CASE(1, 1, false) CASE(2, 1, false) CASE(4, 1, false) CASE(8, 1, false) CASE(16, 1, false)
       CASE(1, 2, false) CASE(2, 2, false) CASE(4, 2, false) CASE(8, 2, false)
