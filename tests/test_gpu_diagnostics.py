@@ -6,7 +6,7 @@ import ctypes
 import numpy as np
 import pytest
 
-from util import DeviceCase, gpu_forward, gpu_viterbi
+from util import DeviceCase, gpu_backward, gpu_forward, gpu_viterbi
 
 pytestmark = pytest.mark.gpu
 
@@ -32,8 +32,11 @@ def test_a_wait_that_runs_out_raises_the_flag_and_the_kernel_still_finishes(U):
     assert lib.rnnt_hip_check_kernels(None) == 0
     before = lib.rnnt_hip_set_spin_limit(0)
     try:
-        gpu_forward(c, LN)          # returns: the walk finishes on whatever it finds
+        _, alphas = gpu_forward(c, LN)          # returns: the walk finishes on whatever it finds
         gpu_viterbi(c, LN)
+        if U > 256:                             # the dalpha walk of two halves waits the same way
+            assert lib.rnnt_hip_check_kernels(None) == 2
+            gpu_backward(c, np.nan_to_num(alphas, posinf=0.0, neginf=0.0), LN)
         assert lib.rnnt_hip_check_kernels(None) == 2
         assert b"gave up waiting" in lib.rnnt_hip_last_error()
         assert lib.rnnt_hip_check_kernels(None) == 0   # reading the flag clears it

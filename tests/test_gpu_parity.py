@@ -339,11 +339,11 @@ def test_label_axes_dealt_to_several_wavefronts_carry_the_reference_bits(T, U):
 @pytest.mark.parametrize("B,T,U", [(11, 300, 400), (3, 700, 258), (17, 150, 512), (96, 40, 300),
                                    (97, 40, 300)])
 def test_two_halves_of_a_label_axis_walked_side_by_side_carry_the_reference_bits(B, T, U):
-    """257 .. 512 label positions in a batch of at most 96 utterances: the alpha walk runs the two
-    halves of the label axis as two workgroups at the same time; the scores of the boundary
-    column cross through memory, each with the number of its step beside it, and the upper half
-    asks again for what was not there yet.  Long enough lattices that the upper half runs its
-    steady state a few groups of steps behind the lower one; batches that fill the last eight
+    """257 .. 512 label positions in a batch of at most 96 utterances: the alpha and the dalpha
+    walk run the two halves of the label axis as two workgroups at the same time; the values of
+    the boundary column cross through memory, each with the number of its step beside it, and
+    the half that follows asks again for what was not there yet.  Long enough lattices that it
+    runs its steady state a few groups of steps behind the half that leads; batches that fill the last eight
     workgroup slots only partly; 97 utterances take the one-workgroup walk again.  U counts the
     rows of predictions."""
     cfg = small_config(B, T, U - 1, 5, ragged=True)
@@ -354,10 +354,15 @@ def test_two_halves_of_a_label_axis_walked_side_by_side_carry_the_reference_bits
     c = DeviceCase(E, P, labels, il, ll)
     LN = oracle.log_norms_naive(E, P, il, ll)
     costs_o, alphas_o = oracle.forward(E, P, LN, labels, il, ll)
+    eg_o, pg_o, lng_o = oracle.backward(E, P, np.nan_to_num(alphas_o), LN, labels, il, ll)
     for _ in range(2):                       # the second call finds the first one's entries
         costs, alphas = gpu_forward(c, LN)
         assert_same_bits(costs, costs_o, what="costs")
         assert_same_bits(alphas, alphas_o, what="alphas")
+        eg, pg, lng = gpu_backward(c, alphas, LN)
+        assert_same_bits(lng, lng_o, what="lngrads")
+        assert_same_bits(eg, eg_o, what="egrads (sparse)")
+        assert_same_bits(pg, pg_o, what="pgrads (sparse)")
     from transducer_amd import capi
     assert capi.load().rnnt_hip_check_kernels(None) == 0
 

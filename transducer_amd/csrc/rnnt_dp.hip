@@ -132,6 +132,16 @@ __device__ inline float lse2(float a, float b) {
   return (hi == kNegInf) ? kNegInf : r;
 }
 
+// Raises the device's trouble flag.  A store to GLOBAL memory by its address space: through a
+// generic pointer it would be a flat instruction, which may go to LDS as well, and with one of
+// those possibly in flight the compiler waits for every load in flight at the next use of any
+// loaded value -- on the walk's fast path too, where the branch that raises the flag is never
+// taken.
+__device__ inline void raise_trouble(int* trouble) {
+  typedef __attribute__((address_space(1))) int global_int;
+  __hip_atomic_store((global_int*)trouble, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 // The wait of an upper wavefront for the progress counter of the one below it (LDS, same
 // workgroup).  The lower wavefront never waits for an upper one, so the counter always gets
 // there; the trip bound only turns a logic slip of a future edit into an error report instead
@@ -146,7 +156,7 @@ __device__ inline int bounded_wait(const int* counter, int have, int need, int s
     asm volatile("" ::: "memory");
     if (have < need) {
       if (spins++ >= spin_limit) {
-        if ((threadIdx.x & 63) == 0) *reinterpret_cast<volatile int*>(trouble) = 1;
+        if ((threadIdx.x & 63) == 0) raise_trouble(trouble);
         return 0x7fffffff;
       }
       __builtin_amdgcn_s_sleep(1);
@@ -301,6 +311,7 @@ __global__ __launch_bounds__(256) void gather_kernel(const TIO* __restrict__ E,
 // for has long been written.  Workgroups are dispatched in launch order and an utterance's
 // lower block has the smaller index, so the block that is waited for is always running or done.
 constexpr int kLiveLag = 12;
+constexpr int kBetaLiveLag = 24;  // (the dalpha walk asks eight groups ahead, not four)
 constexpr int kLiveWaveLag = 2;  // groups between the wavefronts of a live block at the start (8 elsewhere)
 template <int C, int W, bool kMulti, bool kLive = false>
 __global__ __launch_bounds__(64 * W) void alpha_kernel(Planes p, const int* __restrict__ inLen,
@@ -452,15 +463,22 @@ __global__ __launch_bounds__(64 * W) void alpha_kernel(Planes p, const int* __re
         // registers reused at once, and that reuse waits for the load.
         if (live_in && wave == 0) {  // uniform
           unsigned long long e = cur.lv;
-          int spins = 0;
-          while (__builtin_amdgcn_ballot_w64(lane < 4 &&
-                                             (unsigned)(e >> 32) != (unsigned)(4 * g + lane + 1))) {
-            if (spins++ >= spin_limit) {  // an entry was not written when it was asked for
-              if (lane == 0) *reinterpret_cast<volatile int*>(trouble) = 1;
-              break;
-            }
-            __builtin_amdgcn_s_sleep(2);
-            e = live_reload(4 * g + (lane & 3));
+          if (__builtin_amdgcn_ballot_w64(lane < 4 &&
+                                          (unsigned)(e >> 32) != (unsigned)(4 * g + lane + 1))) {
+            // An entry was not written when it was asked for: the lower block is closer than it
+            // should be.  Let it get kLiveLag groups ahead again (or finish) before going on --
+            // asking only for what is missing would leave this block right behind it, late at
+            // every group.  Lanes 0 .. 3 ask for their entries again, the others for the far one.
+            const int mine = lane < 4 ? 4 * g + lane : min(4 * ngroups, 4 * (g + kLiveLag));
+            int spins = 0;
+            do {
+              if (spins++ >= spin_limit) {
+                if (lane == 0) raise_trouble(trouble);
+                break;
+              }
+              __builtin_amdgcn_s_sleep(4);
+              e = live_reload(mine);
+            } while (__builtin_amdgcn_ballot_w64((unsigned)(e >> 32) != (unsigned)(mine + 1)));
           }
 #pragma unroll
           for (int j = 0; j < 4; ++j)
@@ -539,7 +557,7 @@ __global__ __launch_bounds__(64 * W) void alpha_kernel(Planes p, const int* __re
       int spins = 0;
       while ((unsigned)(live_load(far) >> 32) != (unsigned)(far + 1)) {
         if (spins++ >= spin_limit) {
-          if (lane == 0) *reinterpret_cast<volatile int*>(trouble) = 1;
+          if (lane == 0) raise_trouble(trouble);
           break;
         }
         __builtin_amdgcn_s_sleep(8);
@@ -574,7 +592,7 @@ __global__ __launch_bounds__(64 * W) void alpha_kernel(Planes p, const int* __re
   for (int c = 0; c < C; ++c)
     if (u0 + c == Ub - 1) costs[b] = -stay[c];
   if constexpr (kLive) {
-    if (spin_limit < 0 && live_sink == 1u) *reinterpret_cast<volatile int*>(trouble) = 1;  // never
+    if (spin_limit < 0 && live_sink == 1u) raise_trouble(trouble);  // never
   }
 }
 
@@ -645,20 +663,37 @@ constexpr int beta_depth(int C) { return C <= 2 ? 8 : C <= 4 ? 4 : 3; }
 // wavefront below reads them one group later (the same hand-over as between blocks, with the
 // bounded wait of alpha_kernel).  Every wavefront runs all groups, past the utterance's labels
 // too (zeros), so nobody waits for a wavefront that has left.
-template <int C, int W, bool kMulti>
+// kLive: the two halves of a label axis of up to 128 C W positions as two workgroups running at
+// the same time, as in alpha_kernel with the directions turned round: the UPPER half leads (and
+// has the smaller workgroup index, so it is dispatched first), lane 0 of its wavefront 0 leaves
+// dalpha of the half's first column in `live` (entry s: the value on diagonal s, s + 1 in the
+// upper word; zero before the launch), and the highest wavefront of the lower half asks for
+// them, lane j for entry 4g + 1 + j, with its weights, checks the tags when it uses them and
+// asks again, bounded, for what was not there yet.  An utterance whose labels end in the lower
+// half has no upper half: that workgroup leaves at once and nothing is taken from `live`.
+template <int C, int W, bool kMulti, bool kLive = false>
 __global__ __launch_bounds__(64 * W) void beta_kernel(Planes p, const int* __restrict__ labels,
                                                       const int* __restrict__ inLen,
                                                       const int* __restrict__ labLen, Dims d,
                                                       int hand_stride, int u_base,
                                                       const float* __restrict__ ghin,
                                                       float* __restrict__ ghout, int spin_limit,
-                                                      int* __restrict__ trouble) {
+                                                      int* __restrict__ trouble,
+                                                      unsigned long long* __restrict__ live) {
   static_assert(W == 1 || !kMulti, "several wavefronts only when one launch covers the label axis");
+  static_assert(!kLive || (!kMulti && W > 1), "live halves are dealt to several wavefronts");
   extern __shared__ __attribute__((aligned(16))) float hand[];  // [W-1][hand_stride]: entry s =
                                                                 // dalpha on diagonal s
   __shared__ int done[W];  // groups a wavefront has published
-  const int b = blockIdx.x, lane = threadIdx.x & 63;
+  // live halves: workgroups go round the 8 XCDs in launch order; indices i and i + 8 share one
+  const int live_half = kLive ? 1 - ((blockIdx.x >> 3) & 1) : 0;  // the upper half comes first
+  const int b = kLive ? (blockIdx.x >> 4) * 8 + (blockIdx.x & 7) : blockIdx.x;
+  const int lane = threadIdx.x & 63;
   const int wave = W > 1 ? __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) : 0;
+  if (kLive) {
+    if (b >= d.B) return;
+    u_base = live_half * 64 * C * W;
+  }
   int Tb, Ub;
   utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
   if (Tb == 0 || Ub == 0) return;  // :92-94
@@ -690,6 +725,25 @@ __global__ __launch_bounds__(64 * W) void beta_kernel(Planes p, const int* __res
   const float* gin =
       (kMulti && ghin && u_base + 64 * C < Ub) ? ghin + (size_t)b * hand_stride : nullptr;
   float* gout = (kMulti && ghout) ? ghout + (size_t)b * hand_stride : nullptr;
+  // live halves: the upper one writes the entries; the highest wavefront of the lower one takes
+  // them if the utterance has an upper half at all
+  unsigned long long* lrow = kLive ? live + (size_t)b * hand_stride : nullptr;
+  const bool live_out = kLive && live_half == 1;
+  const bool live_takes = kLive && live_half == 0 && wave == W - 1 && 64 * C * W < Ub;
+  auto live_load = [&](int s) -> unsigned long long {
+    return __hip_atomic_load(lrow + s, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  };
+  // (one opaque statement: see alpha_kernel)
+  auto live_reload = [&](int s) -> unsigned long long {
+    unsigned long long e;
+    const unsigned long long* q = lrow + s;
+    asm volatile("global_load_dwordx2 %0, %1, off sc1\n\ts_waitcnt vmcnt(0)"
+                 : "=&v"(e)
+                 : "v"(q)
+                 : "memory");
+    return e;
+  };
+  unsigned live_sink = 0;
 
   float dcol[C], accB[C], accL[C];
   bool fold[C];  // label of this position equals blank: both sums share one accumulator
@@ -712,6 +766,8 @@ __global__ __launch_bounds__(64 * W) void beta_kernel(Planes p, const int* __res
   struct Group {
     float4 wb[C], we[C];
     float gh[4];  // dalpha of the block above's first column on diagonals 4g+1 .. 4g+4
+    unsigned long long lv;  // the same, tagged, from the half running beside this one: lane j
+                            // holds the entry of diagonal 4g + 1 + j
   };
   auto load_group = [&](int g) -> Group {
     Group r;
@@ -725,6 +781,7 @@ __global__ __launch_bounds__(64 * W) void beta_kernel(Planes p, const int* __res
 #pragma unroll
       for (int j = 0; j < 4; ++j) r.gh[j] = gin ? gin[4 * gc + 1 + j] : 0.0f;  // uniform
     }
+    if constexpr (kLive) r.lv = live_load(4 * gc + 1 + (lane & 3));  // every wavefront asks
     return r;
   };
   // steps last-1 .. 0 are computed; the slot of step `last` receives the seed and the slots
@@ -747,6 +804,33 @@ __global__ __launch_bounds__(64 * W) void beta_kernel(Planes p, const int* __res
 #pragma unroll
       for (int j = 0; j < 4; ++j) hh[j] = hand_in[4 * g + 1 + j];  // uniform
     }
+    if constexpr (kLive) {
+      if (live_takes) {  // uniform
+        // diagonals past the seed's group are never written, and never used either
+        const int top = 4 * g_first + 3;
+        unsigned long long e = w.lv;
+        if (__builtin_amdgcn_ballot_w64(lane < 4 && 4 * g + 1 + lane <= top &&
+                                        (unsigned)(e >> 32) != (unsigned)(4 * g + 2 + lane))) {
+          // (as in alpha_kernel: let the upper half get kBetaLiveLag groups ahead again)
+          const int mine = (lane < 4 && 4 * g + 1 + lane <= top) ? 4 * g + 1 + lane
+                                                                 : 4 * max(g - kBetaLiveLag, 0);
+          int spins = 0;
+          do {
+            if (spins++ >= spin_limit) {
+              if (lane == 0) raise_trouble(trouble);
+              break;
+            }
+            __builtin_amdgcn_s_sleep(4);
+            e = live_reload(mine);
+          } while (__builtin_amdgcn_ballot_w64((unsigned)(e >> 32) != (unsigned)(mine + 1)));
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          hh[j] = __int_as_float(__builtin_amdgcn_readlane((int)(unsigned)e, j));
+      } else {
+        live_sink ^= (unsigned)w.lv;  // (kept until the end: see alpha_kernel)
+      }
+    }
 #pragma unroll
     for (int j = 3; j >= 0; --j) {
       const int s = 4 * g + j;
@@ -761,7 +845,7 @@ __global__ __launch_bounds__(64 * W) void beta_kernel(Planes p, const int* __res
         float right[C];
         float above = 0.0f;  // right of the wavefront's last position
         if constexpr (kMulti) above = gin ? w.gh[j] : 0.0f;
-        if (W > 1) above = wave < W - 1 ? hh[j] : 0.0f;
+        if (W > 1) above = (wave < W - 1 || live_takes) ? hh[j] : 0.0f;
         if constexpr (kSpread) {
 #pragma unroll
           for (int c = 0; c < C; ++c) {
@@ -801,6 +885,16 @@ __global__ __launch_bounds__(64 * W) void beta_kernel(Planes p, const int* __res
         for (int j = 0; j < 4; ++j) gout[4 * g + j] = gsend[j];
       }
     }
+    if constexpr (kLive) {
+      if (live_out && wave == 0 && lane == 0) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          __hip_atomic_store(lrow + 4 * g + j,
+                             ((unsigned long long)(unsigned)(4 * g + j + 1) << 32) |
+                                 (unsigned long long)__float_as_uint(gsend[j]),
+                             __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
     if (W > 1 && wave > 0 && lane == 0) {  // entries 4g .. 4g+3, then the progress
 #pragma unroll
       for (int j = 0; j < 4; ++j) hand_out[4 * g + j] = gsend[j];
@@ -817,12 +911,25 @@ __global__ __launch_bounds__(64 * W) void beta_kernel(Planes p, const int* __res
   auto walk = [&](auto with_fold) __attribute__((always_inline)) {
     constexpr int kBetaDepth = beta_depth(C);
     int g = g_first;
+    if constexpr (kLive) {
+      if (live_takes) {  // start kBetaLiveLag groups behind the upper half (or when it is done)
+        const int far = 4 * max(g_first - kBetaLiveLag, 0);
+        int spins = 0;
+        while ((unsigned)(live_load(far) >> 32) != (unsigned)(far + 1)) {
+          if (spins++ >= spin_limit) {
+            if (lane == 0) raise_trouble(trouble);
+            break;
+          }
+          __builtin_amdgcn_s_sleep(8);
+        }
+      }
+    }
     Group q[kBetaDepth];
 #pragma unroll
     for (int i = 0; i < kBetaDepth; ++i) q[i] = load_group(g - i);
     // fall a few groups behind the wavefront above, so that the wait per group finds its
     // counter there already
-    if (W > 1 && wave < W - 1) wait_for(min(g_first + 1, 8 * (W - 1 - wave)));
+    if (W > 1 && wave < W - 1) wait_for(min(g_first + 1, (kLive ? kLiveWaveLag : 8) * (W - 1 - wave)));
     // the first round, whose first group holds the seed (a short lattice may end inside it)
     const std::true_type seeded;
     const std::false_type plain;
@@ -858,6 +965,9 @@ __global__ __launch_bounds__(64 * W) void beta_kernel(Planes p, const int* __res
       p.gB[(size_t)b * d.Ua + u] = accB[c];
       p.gL[(size_t)b * d.Ua + u] = accL[c];
     }
+  }
+  if constexpr (kLive) {
+    if (spin_limit < 0 && live_sink == 1u) raise_trouble(trouble);  // never
   }
 }
 
@@ -2024,6 +2134,23 @@ int launch_beta(const Planes& p, const int* labels, const int* inLen, const int*
   const size_t lds = W > 1 ? sizeof(float) * (size_t)(W - 1) * stride : 0;
   int* trouble = nullptr;
   RNNT_TRY(trouble_flag(&trouble));
+  // 257 .. 512 label positions in few enough utterances: the two halves side by side on two
+  // CUs, four wavefronts of one position a lane each (as in launch_alpha)
+  if (alpha_live_blocks(d) && W == 4) {
+    unsigned long long* live = reinterpret_cast<unsigned long long*>(p.hand[0]);
+    const int words = 2 * d.B * stride;
+    hipLaunchKernelGGL(clear_words_kernel, dim3((words + 255) / 256), dim3(256), 0, s,
+                       reinterpret_cast<int*>(live), words);
+    RNNT_LAUNCH_CHECK("clear_words_kernel");
+    if (lds > 64 * 1024)
+      RNNT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(beta_kernel<1, 4, false, true>),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    hipLaunchKernelGGL((beta_kernel<1, 4, false, true>), dim3(16 * ((d.B + 7) / 8)), dim3(256),
+                       lds, s, p, labels, inLen, labLen, d, stride, 0, nullptr, nullptr,
+                       g_spin_limit, trouble, live);
+    RNNT_LAUNCH_CHECK("beta_kernel (live halves)");
+    return kOk;
+  }
   for (int k = nblocks - 1; k >= 0; --k) {  // highest block first
     const float* ghin = k == nblocks - 1 ? nullptr : p.hand[(k + 1) & 1];
     float* ghout = k == 0 ? nullptr : p.hand[k & 1];
@@ -2036,7 +2163,7 @@ int launch_beta(const Planes& p, const int* labels, const int* inLen, const int*
                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));  \
     hipLaunchKernelGGL((beta_kernel<C, W, M>), dim3(d.B), dim3(64 * W), lds, s, p, labels, \
                        inLen, labLen, d, stride, u_base, ghin, ghout, g_spin_limit,        \
-                       trouble);                                                            \
+                       trouble, nullptr);                                                   \
     break;
       CASE(1, 1, false) CASE(2, 1, false) CASE(4, 1, false) CASE(8, 1, false) CASE(16, 1, false)
       CASE(2, 2, false) CASE(4, 2, false) CASE(8, 2, false)
