@@ -198,10 +198,10 @@ int rnnt_hip_profile_read(double* total_ms, int* launches, int n);
 
 /* ---- diagnostics of the lattice walks (no counterpart in the reference) ------------------ */
 
-/* The alpha and best-path walks deal a long label axis to two wavefronts of a workgroup; the
- * upper one waits, with a trip bound, for the lower one's progress counter.  Should the bound
- * ever run out the kernel still finishes, with invalid results, and raises a flag on its
- * device.  This call waits for `stream`, reads the current device's flag and clears it:
+/* The lattice walks deal a long label axis to several wavefronts of a workgroup (from 257
+ * label positions in a small batch the alpha and dalpha walks also to two workgroups); each
+ * waits, with a trip bound, for what its neighbour hands over.  Should the bound ever run out
+ * the kernel still finishes, with invalid results, and raises a flag on its device.  This call waits for `stream`, reads the current device's flag and clears it:
  * RNNT_OK if no kernel gave up since the last check, else RNNT_HIP_FAILURE with a message.
  * (The reference's kernels synchronise with __syncthreads and cannot hang this way,
  * transducer/transducer_cuda.cu:65-90.) */
