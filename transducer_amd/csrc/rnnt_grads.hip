@@ -55,7 +55,14 @@ struct EgradsWindow {
 // (a template parameter, so the matrix instructions of a tile form one straight-line block).
 // Label positions past the utterance contribute exact zeros: their Y rows are masked and the
 // W slab is zero there.
-template <int NS, bool kAccumulate, typename TIO, typename TOUT>
+// kMode: what a launch does with the sums of its slice of the label axis.
+//   kEgWhole    out = delta (X sums + sparse terms)         the only slice
+//   kEgAdd      out = delta (out + X sums)                  onto what the caller's array holds
+//   kEgPartial  out = sums (first slice) or out + sums      a slice but the last of several:
+//                                                           no emissions read, no exponentials
+//   kEgFinal    out = delta (X (out + sums) + sparse terms) the last of several slices
+constexpr int kEgWhole = 0, kEgAdd = 1, kEgPartial = 2, kEgFinal = 3;
+template <int NS, int kMode, typename TIO, typename TOUT>
 __device__ __forceinline__ void egrads_walk(
     const TIO* __restrict__ E, const TIO* __restrict__ P, const float* __restrict__ mE,
     const float* __restrict__ mP, const float* __restrict__ Wn, const float* __restrict__ deltas,
@@ -69,6 +76,10 @@ __device__ __forceinline__ void egrads_walk(
   const int vc = vok ? vcol : d.V - 1;  // always readable
   const bool cols_full = wave_col0 + 32 <= d.V;
   // lane that owns the blank column, if it is one of this wavefront's and terms are folded in
+  constexpr bool kSparse = kMode == kEgWhole || kMode == kEgFinal;  // may fold sparse terms in
+  constexpr bool kScores = kMode != kEgPartial;                     // reads the emissions
+  // reads what the output holds (a first partial slice starts from nothing)
+  const bool reads_out = kMode == kEgAdd || kMode == kEgFinal || (kMode == kEgPartial && u_lo > 0);
   const int blank_lane = (sp.labels && d.blank >= wave_col0 && d.blank < wave_col0 + 32)
                              ? d.blank - wave_col0 : -1;
   const int tile_lo = win.tile_begin + blockIdx.y * tiles_per_chunk;
@@ -199,7 +210,8 @@ __device__ __forceinline__ void egrads_walk(
     TOUT* Otile = out + (size_t)(t0 - win.t_base) * d.V;
     float evl[16];
     float (&ev)[16] = pick_set(ahead, evc, evl);
-    if constexpr (decltype(ahead)::value) {
+    if constexpr (!kScores) {
+    } else if constexpr (decltype(ahead)::value) {
       load_e(min(ti + 1, tile_valid - 1), evn);
     } else if (interior) {
       // the emissions of this tile, requested before the matrix work so they arrive under it
@@ -212,10 +224,30 @@ __device__ __forceinline__ void egrads_walk(
       for (int r = 0; r < 16; ++r)
         ev[r] = ldf(Eb + (size_t)min(t0 + mfma_row(r, h), Tb - 1) * d.V + vc);
     }
+    // a later slice of a long label axis adds to what the earlier ones left: requested here
+    // too (asked for at the store, every tile waited a memory round trip for them: 0.44 ms a
+    // slice of 112 label positions at B=8 T=10000 V=1000, where the first slice takes 0.30)
+    float ov[16];
+    if constexpr (kMode != kEgWhole) {
+      if (!reads_out) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) ov[r] = 0.0f;
+      } else if (interior) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          ov[r] = ldf(Otile + (lane_off + (unsigned)(8 * (r >> 2) + (r & 3)) * (unsigned)d.V));
+      } else {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int t = t0 + mfma_row(r, h);
+          ov[r] = (t < d.T && vok) ? ldf(out + (size_t)(t - win.t_base) * d.V + vcol) : 0.0f;
+        }
+      }
+    }
     // sparse terms of this tile for up to kEsPrefetch labels that fall into this wavefront's
     // columns: one coalesced load per plane, requested here so it arrives under the matrix work
     float sd[kEsPrefetch], sbl = 0.0f;
-    if (!kAccumulate && (nmatch > 0 || blank_lane >= 0)) {
+    if (kSparse && (nmatch > 0 || blank_lane >= 0)) {
       const int tr = min(t0 + l32, Tb - 1);
 #pragma unroll
       for (int i = 0; i < kEsPrefetch; ++i) {
@@ -256,11 +288,14 @@ __device__ __forceinline__ void egrads_walk(
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
         const int r = 4 * g + k;
-        const float x = exp_minus_scaled(ev[r], f4at(m4, k)) * acc[r];
+        float x;
+        if constexpr (kMode == kEgPartial) x = ov[r] + acc[r];
+        else if constexpr (kMode == kEgFinal) x = exp_minus_scaled(ev[r], f4at(m4, k)) * (ov[r] + acc[r]);
+        else x = exp_minus_scaled(ev[r], f4at(m4, k)) * acc[r];
         v[r] = (interior || t0 + mfma_row(r, h) < Tb) ? x : 0.0f;
       }
     }
-    if (!kAccumulate && (nmatch > 0 || blank_lane >= 0)) {  // uniform per wavefront, and rare
+    if (kSparse && (nmatch > 0 || blank_lane >= 0)) {  // uniform per wavefront, and rare
       // Lane l32 holds the term of frame t0+l32 (fetched before the matrix block).  The terms go
       // through a per-wavefront LDS strip; the two lanes that own the target column read their
       // 16 frames back as four 16-byte loads.
@@ -282,10 +317,22 @@ __device__ __forceinline__ void egrads_walk(
 #pragma unroll
       for (int i = 0; i < kEsPrefetch; ++i)
         if (i < nmatch) apply(row_ok ? sd[i] : 0.0f, mc[i], -1.0f);
-      for (int i = kEsPrefetch; i < nmatch; ++i) {  // more labels in one 32-column block
-        const int u = match[i];
-        apply(row_ok ? sp.emT[((size_t)b * d.U + u) * d.T + min(t0 + l32, Tb - 1)] : 0.0f,
-              label_at(sp.labels, d, b, u) - wave_col0, -1.0f);
+      // more labels in one 32-column block (long transcripts over a small vocabulary: 400 labels
+      // and 1000 columns put a dozen into every block): their terms are asked for four at a
+      // time, so that a tile waits one memory round trip per four, not one per label
+      constexpr int kBatch = 4;
+      for (int i0 = kEsPrefetch; i0 < nmatch; i0 += kBatch) {
+        float term[kBatch];
+        int col[kBatch];
+#pragma unroll
+        for (int k = 0; k < kBatch; ++k) {
+          const int u = match[min(i0 + k, nmatch - 1)];
+          term[k] = sp.emT[((size_t)b * d.U + u) * d.T + min(t0 + l32, Tb - 1)];
+          col[k] = label_at(sp.labels, d, b, u) - wave_col0;
+        }
+#pragma unroll
+        for (int k = 0; k < kBatch; ++k)
+          if (i0 + k < nmatch) apply(row_ok ? term[k] : 0.0f, col[k], -1.0f);
       }
       if (blank_lane >= 0) apply(row_ok ? sbl : 0.0f, blank_lane, 1.0f);
     }
@@ -293,7 +340,9 @@ __device__ __forceinline__ void egrads_walk(
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         TOUT* o = Otile + (lane_off + (unsigned)(8 * (r >> 2) + (r & 3)) * (unsigned)d.V);
-        stf(o, delta * (kAccumulate ? ldf(o) + v[r] : v[r]));
+        if constexpr (kMode == kEgAdd) stf(o, delta * (ov[r] + v[r]));
+        else if constexpr (kMode == kEgPartial) stf(o, v[r]);
+        else stf(o, delta * v[r]);
       }
     } else {
 #pragma unroll
@@ -301,7 +350,9 @@ __device__ __forceinline__ void egrads_walk(
         const int t = t0 + mfma_row(r, h);
         if (t < d.T && vok) {
           TOUT* o = out + (size_t)(t - win.t_base) * d.V + vcol;
-          stf(o, delta * (kAccumulate ? ldf(o) + v[r] : v[r]));
+          if constexpr (kMode == kEgAdd) stf(o, delta * (ov[r] + v[r]));
+          else if constexpr (kMode == kEgPartial) stf(o, v[r]);
+          else stf(o, delta * v[r]);
         }
       }
     }
@@ -310,7 +361,7 @@ __device__ __forceinline__ void egrads_walk(
     cur ^= 1;
   };
   float evA[16], evB[16];
-  if constexpr (kAhead) {
+  if constexpr (kAhead && kScores) {
     // two tiles per trip, the two register sets swapping roles (a copy from one set to the other
     // would wait for the requests a tile too early)
     if (tile_lo < tile_valid) load_e(tile_lo, evA);
@@ -322,20 +373,23 @@ __device__ __forceinline__ void egrads_walk(
     for (int ti = tile_lo; ti < tile_valid; ++ti) tile(ti, evA, evB, std::false_type());
   }
 
-  // frames past the utterance: the dense part is exactly zero
-  for (int ti = max(tile_lo, tile_valid); ti < tile_hi; ++ti) {
+  // frames past the utterance: the dense part is exactly zero (of several slices the first
+  // writes the zeros and the later ones leave them)
+  if (kMode == kEgWhole || kMode == kEgAdd || (kMode == kEgPartial && u_lo == 0)) {
+    for (int ti = max(tile_lo, tile_valid); ti < tile_hi; ++ti) {
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int t = ti * 32 + mfma_row(r, h);
-      if (t < d.T && vok) {
-        TOUT* o = out + (size_t)(t - win.t_base) * d.V + vcol;
-        stf(o, kAccumulate ? delta * ldf(o) : 0.0f);
+      for (int r = 0; r < 16; ++r) {
+        const int t = ti * 32 + mfma_row(r, h);
+        if (t < d.T && vok) {
+          TOUT* o = out + (size_t)(t - win.t_base) * d.V + vcol;
+          stf(o, kMode == kEgAdd ? delta * ldf(o) : 0.0f);
+        }
       }
     }
   }
 }
 
-template <bool kAccumulate, typename TIO, typename TOUT>
+template <int kMode, typename TIO, typename TOUT>
 __global__ __launch_bounds__(256, 2) void egrads_stream_kernel(
     const TIO* __restrict__ E, const TIO* __restrict__ P, const float* __restrict__ mE,
     const float* __restrict__ mP, const float* __restrict__ Wn, const float* __restrict__ deltas,
@@ -350,8 +404,9 @@ __global__ __launch_bounds__(256, 2) void egrads_stream_kernel(
   int Tb, Ub;
   utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
   // a later slice of the label axis that lies past this utterance adds nothing; only the last
-  // slice (the one that is given the factors) still has to scale what is there
-  if (kAccumulate && u_lo > 0 && u_lo >= Ub && deltas == nullptr) return;
+  // slice (the one that is given the factors) still has to finish what is there
+  if (kMode == kEgPartial && u_lo > 0 && u_lo >= Ub) return;
+  if (kMode == kEgAdd && u_lo > 0 && u_lo >= Ub && deltas == nullptr) return;
   int nmatch = 0;
   if (sp.labels) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -372,7 +427,7 @@ __global__ __launch_bounds__(256, 2) void egrads_stream_kernel(
   __syncthreads();
   const int nsteps = (min(max(Ub - u_lo, 0), 16 * kEsMaxS) + 15) >> 4;
 #define RNNT_EG_WALK(NS)                                                                      \
-  egrads_walk<NS, kAccumulate>(E, P, mE, mP, Wn, deltas, egrads, As, Ms, d, Up, Tw,          \
+  egrads_walk<NS, kMode>(E, P, mE, mP, Wn, deltas, egrads, As, Ms, d, Up, Tw,                \
                                tiles_per_chunk, u_lo, b, Tb, Ub, sp, Match[threadIdx.x >> 6], \
                                nmatch, &Strip[threadIdx.x >> 6], win)
   if (nsteps <= 2) RNNT_EG_WALK(2);
@@ -681,22 +736,27 @@ static int egrads_window(const TIO* E, const TIO* P, const float* mE, const floa
   const int per = (ntiles + chunks - 1) / chunks;
   chunks = (ntiles + per - 1) / per;
   // A launch contracts 16 * kEsMaxS label positions (what a wavefront keeps of Y in registers);
-  // a longer label axis goes slice by slice, each later slice adding to what the earlier ones
-  // left in the output.  Only the last slice is given the factors, and scales the whole sum.
+  // a longer label axis goes slice by slice.  Into an array of the caller's that is added to,
+  // every slice adds X times its sums and the last one scales the whole.  Otherwise the slices
+  // but the last leave their bare sums in the output -- no emissions read, no exponentials --
+  // and the last one finishes them: X times the total, the sparse terms, the factor (B=8
+  // T=10000 U=400 V=1000, four slices: 1.91 ms with every slice adding X times its sums and
+  // asking for the output where it is stored, 1.49 asking for it at the start of a tile).
   const SparseTerms none;
-  for (int u_lo = 0; u_lo < Up; u_lo += 16 * kEsMaxS) {
-    const bool last = u_lo + 16 * kEsMaxS >= Up;
-    const float* dl = last ? deltas : nullptr;
-    if (accumulate || u_lo > 0)
-      hipLaunchKernelGGL((egrads_stream_kernel<true, TIO, TOUT>), dim3(vtiles, chunks, d.B),
-                         dim3(256), 0, s, E, P, mE, mP, Wn, dl, out, inLen, labLen, d, Up, Tw,
-                         per, u_lo, none, win);
-    else
-      hipLaunchKernelGGL((egrads_stream_kernel<false, TIO, TOUT>), dim3(vtiles, chunks, d.B),
-                         dim3(256), 0, s, E, P, mE, mP, Wn, dl, out, inLen, labLen, d, Up, Tw,
-                         per, u_lo, sparse, win);
+  const int slice = 16 * kEsMaxS;
+#define RNNT_EG_LAUNCH(MODE, DL, SP)                                                          \
+  hipLaunchKernelGGL((egrads_stream_kernel<MODE, TIO, TOUT>), dim3(vtiles, chunks, d.B),      \
+                     dim3(256), 0, s, E, P, mE, mP, Wn, DL, out, inLen, labLen, d, Up, Tw,    \
+                     per, u_lo, SP, win)
+  for (int u_lo = 0; u_lo < Up; u_lo += slice) {
+    const bool last = u_lo + slice >= Up;
+    if (accumulate) RNNT_EG_LAUNCH(kEgAdd, (last ? deltas : nullptr), none);
+    else if (Up <= slice) RNNT_EG_LAUNCH(kEgWhole, deltas, sparse);
+    else if (!last) RNNT_EG_LAUNCH(kEgPartial, nullptr, none);
+    else RNNT_EG_LAUNCH(kEgFinal, deltas, sparse);
     RNNT_LAUNCH_CHECK("egrads_stream_kernel");
   }
+#undef RNNT_EG_LAUNCH
   return kOk;
 }
 
