@@ -312,8 +312,9 @@ def test_long_label_axis_uses_more_cells_per_lane():
 def test_label_axes_dealt_to_several_wavefronts_carry_the_reference_bits(T, U):
     """From 65 label positions the alpha walk and from 129 the dalpha walk deal the label axis to
     two or four wavefronts of one workgroup, which hand the boundary column's score on through
-    LDS and wait for each other's progress counters (four from 257 positions; there a lane's
-    positions of the dalpha walk are 64 apart).  U counts the rows of predictions and sits on
+    LDS and wait for each other's progress counters (four from 129 positions; from 257 a small
+    batch like this one is walked as two halves side by side, and past 512 a lane owns two to
+    four positions, those of the dalpha walk 64 apart).  U counts the rows of predictions and sits on
     either side of every change of that split; T = 1 and 6 leave most wavefronts with less than
     one or two groups of four steps, 45 lets them fall the few groups behind that they run at.
     Same bars as everywhere: the reference's bits in every alpha, dalpha and sparse term, the
