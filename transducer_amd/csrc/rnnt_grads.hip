@@ -62,7 +62,9 @@ struct EgradsWindow {
 //                                                           no emissions read, no exponentials
 //   kEgFinal    out = delta (X (out + sums) + sparse terms) the last of several slices
 constexpr int kEgWhole = 0, kEgAdd = 1, kEgPartial = 2, kEgFinal = 3;
-template <int NS, int kMode, typename TIO, typename TOUT>
+// kManyLabels: compiled for transcripts that put more than two labels into most blocks of 32
+// columns (the launcher decides by U * 32 > 2 V); see where the terms are fetched.
+template <int NS, int kMode, bool kManyLabels, typename TIO, typename TOUT>
 __device__ __forceinline__ void egrads_walk(
     const TIO* __restrict__ E, const TIO* __restrict__ P, const float* __restrict__ mE,
     const float* __restrict__ mP, const float* __restrict__ Wn, const float* __restrict__ deltas,
@@ -317,22 +319,33 @@ __device__ __forceinline__ void egrads_walk(
 #pragma unroll
       for (int i = 0; i < kEsPrefetch; ++i)
         if (i < nmatch) apply(row_ok ? sd[i] : 0.0f, mc[i], -1.0f);
-      // more labels in one 32-column block (long transcripts over a small vocabulary: 400 labels
-      // and 1000 columns put a dozen into every block): their terms are asked for four at a
-      // time, so that a tile waits one memory round trip per four, not one per label
-      constexpr int kBatch = 4;
-      for (int i0 = kEsPrefetch; i0 < nmatch; i0 += kBatch) {
-        float term[kBatch];
-        int col[kBatch];
+      // more labels in one 32-column block
+      if constexpr (kManyLabels) {
+        // long transcripts over a small vocabulary (400 labels and 1000 columns put a dozen into
+        // every block): their terms are asked for four at a time, so that a tile waits one
+        // memory round trip per four, not one per label (B=8 T=10000 U=400 V=1000: 1.21 ->
+        // 1.02 ms).  A kernel of its own: compiled into the kernel of the large vocabularies,
+        // where it hardly ever runs, it cost that one 1 % (B=32 T=2000 U=100 V=10000).
+        constexpr int kBatch = 4;
+        for (int i0 = kEsPrefetch; i0 < nmatch; i0 += kBatch) {
+          float term[kBatch];
+          int col[kBatch];
 #pragma unroll
-        for (int k = 0; k < kBatch; ++k) {
-          const int u = match[min(i0 + k, nmatch - 1)];
-          term[k] = sp.emT[((size_t)b * d.U + u) * d.T + min(t0 + l32, Tb - 1)];
-          col[k] = label_at(sp.labels, d, b, u) - wave_col0;
+          for (int k = 0; k < kBatch; ++k) {
+            const int u = match[min(i0 + k, nmatch - 1)];
+            term[k] = sp.emT[((size_t)b * d.U + u) * d.T + min(t0 + l32, Tb - 1)];
+            col[k] = label_at(sp.labels, d, b, u) - wave_col0;
+          }
+#pragma unroll
+          for (int k = 0; k < kBatch; ++k)
+            if (i0 + k < nmatch) apply(row_ok ? term[k] : 0.0f, col[k], -1.0f);
         }
-#pragma unroll
-        for (int k = 0; k < kBatch; ++k)
-          if (i0 + k < nmatch) apply(row_ok ? term[k] : 0.0f, col[k], -1.0f);
+      } else {
+        for (int i = kEsPrefetch; i < nmatch; ++i) {
+          const int u = match[i];
+          apply(row_ok ? sp.emT[((size_t)b * d.U + u) * d.T + min(t0 + l32, Tb - 1)] : 0.0f,
+                label_at(sp.labels, d, b, u) - wave_col0, -1.0f);
+        }
       }
       if (blank_lane >= 0) apply(row_ok ? sbl : 0.0f, blank_lane, 1.0f);
     }
@@ -389,7 +402,7 @@ __device__ __forceinline__ void egrads_walk(
   }
 }
 
-template <int kMode, typename TIO, typename TOUT>
+template <int kMode, bool kManyLabels, typename TIO, typename TOUT>
 __global__ __launch_bounds__(256, 2) void egrads_stream_kernel(
     const TIO* __restrict__ E, const TIO* __restrict__ P, const float* __restrict__ mE,
     const float* __restrict__ mP, const float* __restrict__ Wn, const float* __restrict__ deltas,
@@ -427,7 +440,7 @@ __global__ __launch_bounds__(256, 2) void egrads_stream_kernel(
   __syncthreads();
   const int nsteps = (min(max(Ub - u_lo, 0), 16 * kEsMaxS) + 15) >> 4;
 #define RNNT_EG_WALK(NS)                                                                      \
-  egrads_walk<NS, kMode>(E, P, mE, mP, Wn, deltas, egrads, As, Ms, d, Up, Tw,                \
+  egrads_walk<NS, kMode, kManyLabels>(E, P, mE, mP, Wn, deltas, egrads, As, Ms, d, Up, Tw,   \
                                tiles_per_chunk, u_lo, b, Tb, Ub, sp, Match[threadIdx.x >> 6], \
                                nmatch, &Strip[threadIdx.x >> 6], win)
   if (nsteps <= 2) RNNT_EG_WALK(2);
@@ -744,10 +757,21 @@ static int egrads_window(const TIO* E, const TIO* P, const float* mE, const floa
   // asking for the output where it is stored, 1.49 asking for it at the start of a tile).
   const SparseTerms none;
   const int slice = 16 * kEsMaxS;
-#define RNNT_EG_LAUNCH(MODE, DL, SP)                                                          \
-  hipLaunchKernelGGL((egrads_stream_kernel<MODE, TIO, TOUT>), dim3(vtiles, chunks, d.B),      \
+  const bool many = (long)d.U * 32 > 2 * (long)d.V;  // labels per block of 32 columns
+#define RNNT_EG_LAUNCH_(MODE, MANY, DL, SP)                                                   \
+  hipLaunchKernelGGL((egrads_stream_kernel<MODE, MANY, TIO, TOUT>), dim3(vtiles, chunks, d.B), \
                      dim3(256), 0, s, E, P, mE, mP, Wn, DL, out, inLen, labLen, d, Up, Tw,    \
                      per, u_lo, SP, win)
+  // (only the kernels that fold sparse terms in come in both forms)
+#define RNNT_EG_LAUNCH(MODE, DL, SP)                                                          \
+  do {                                                                                        \
+    if constexpr (MODE == kEgWhole || MODE == kEgFinal) {                                     \
+      if (many) RNNT_EG_LAUNCH_(MODE, true, DL, SP);                                          \
+      else RNNT_EG_LAUNCH_(MODE, false, DL, SP);                                              \
+    } else {                                                                                  \
+      RNNT_EG_LAUNCH_(MODE, false, DL, SP);                                                   \
+    }                                                                                         \
+  } while (0)
   for (int u_lo = 0; u_lo < Up; u_lo += slice) {
     const bool last = u_lo + slice >= Up;
     if (accumulate) RNNT_EG_LAUNCH(kEgAdd, (last ? deltas : nullptr), none);
@@ -757,6 +781,7 @@ static int egrads_window(const TIO* E, const TIO* P, const float* mE, const floa
     RNNT_LAUNCH_CHECK("egrads_stream_kernel");
   }
 #undef RNNT_EG_LAUNCH
+#undef RNNT_EG_LAUNCH_
   return kOk;
 }
 
