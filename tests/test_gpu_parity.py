@@ -368,6 +368,36 @@ def test_two_halves_of_a_label_axis_walked_side_by_side_carry_the_reference_bits
     assert capi.load().rnnt_hip_check_kernels(None) == 0
 
 
+def test_two_halves_side_by_side_keep_their_bits_while_the_device_is_busy():
+    """How far the half that follows runs behind the half that leads depends on when their two
+    workgroups get their CUs; with matrix products on a second stream keeping every CU busy the
+    follower meets entries that are not written yet and takes its bounded wait.  Whatever the
+    timing: the reference's bits, call after call, and no wait given up."""
+    import torch
+    from transducer_amd import capi
+    B, T, U = 24, 600, 400
+    cfg = small_config(B, T, U - 1, 4, ragged=True)
+    E, P, labels, il, ll = unpack(make_inputs(cfg, seed=77))
+    il[0], ll[0] = T, U - 1
+    c = DeviceCase(E, P, labels, il, ll)
+    LN = oracle.log_norms_naive(E, P, il, ll)
+    costs_o, alphas_o = oracle.forward(E, P, LN, labels, il, ll)
+    _, _, lng_o = oracle.backward(E, P, np.nan_to_num(alphas_o), LN, labels, il, ll)
+    side = torch.cuda.Stream()
+    X = torch.randn(4096, 4096, device=c.E.device)
+    for _ in range(8):
+        with torch.cuda.stream(side):
+            for _ in range(4):
+                X @ X
+        costs, alphas = gpu_forward(c, LN)
+        _, _, lng = gpu_backward(c, alphas, LN)
+        assert_same_bits(costs, costs_o, what="costs")
+        assert_same_bits(alphas, alphas_o, what="alphas")
+        assert_same_bits(lng, lng_o, what="lngrads")
+    torch.cuda.synchronize()
+    assert capi.load().rnnt_hip_check_kernels(None) == 0
+
+
 @pytest.mark.parametrize("T,U,V", [(40, 1024, 9), (30, 1025, 9), (50, 1500, 7), (24, 2100, 520),
                                    (300, 1300, 5)])
 def test_label_axis_longer_than_one_block_of_1024_positions(T, U, V):
