@@ -199,7 +199,7 @@ int rnnt_hip_profile_read(double* total_ms, int* launches, int n);
 /* ---- diagnostics of the lattice walks (no counterpart in the reference) ------------------ */
 
 /* The lattice walks deal a long label axis to several wavefronts of a workgroup (from 257
- * label positions in a small batch the alpha and dalpha walks also to two workgroups); each
+ * label positions in a small batch the alpha and dalpha walks also to several workgroups); each
  * waits, with a trip bound, for what its neighbour hands over.  Should the bound ever run out
  * the kernel still finishes, with invalid results, and raises a flag on its device.  This call waits for `stream`, reads the current device's flag and clears it:
  * RNNT_OK if no kernel gave up since the last check, else RNNT_HIP_FAILURE with a message.

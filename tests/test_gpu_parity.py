@@ -368,6 +368,36 @@ def test_two_halves_of_a_label_axis_walked_side_by_side_carry_the_reference_bits
     assert capi.load().rnnt_hip_check_kernels(None) == 0
 
 
+@pytest.mark.parametrize("B,T,U", [(5, 200, 513), (9, 120, 700), (3, 60, 1000), (4, 90, 1025),
+                                   (2, 40, 2100), (70, 6, 600), (40, 5, 1025), (12, 4, 4200)])
+def test_label_axis_as_a_chain_of_blocks_side_by_side_and_where_it_is_not(B, T, U):
+    """From 513 label positions the alpha and dalpha walks run three and more blocks of 256
+    positions side by side, each following the one before it through its own array of tagged
+    entries -- as long as the batch leaves the device the CUs for it (utterances x blocks at
+    most 192, blocks at most 16).  70 x 3 and 40 x 5 workgroups are too many and 17 blocks too
+    long: those take one workgroup per utterance again, a lane owning several positions, or a
+    launch per 1024 positions.  Either way the reference's bits.  U counts the rows of
+    predictions; ragged batches, so that some utterances end blocks below the top one."""
+    cfg = small_config(B, T, U - 1, 4, ragged=True)
+    E, P, labels, il, ll = unpack(make_inputs(cfg, seed=B * 7 + U))
+    il[0], ll[0] = T, U - 1
+    il[1], ll[1] = max(T // 2, 1), 256        # one position in the second block
+    c = DeviceCase(E, P, labels, il, ll)
+    LN = oracle.log_norms_naive(E, P, il, ll)
+    costs_o, alphas_o = oracle.forward(E, P, LN, labels, il, ll)
+    eg_o, pg_o, lng_o = oracle.backward(E, P, np.nan_to_num(alphas_o), LN, labels, il, ll)
+    for _ in range(2):
+        costs, alphas = gpu_forward(c, LN)
+        assert_same_bits(costs, costs_o, what="costs")
+        assert_same_bits(alphas, alphas_o, what="alphas")
+        eg, pg, lng = gpu_backward(c, alphas, LN)
+        assert_same_bits(lng, lng_o, what="lngrads")
+        assert_same_bits(eg, eg_o, what="egrads (sparse)")
+        assert_same_bits(pg, pg_o, what="pgrads (sparse)")
+    from transducer_amd import capi
+    assert capi.load().rnnt_hip_check_kernels(None) == 0
+
+
 def test_two_halves_side_by_side_keep_their_bits_while_the_device_is_busy():
     """How far the half that follows runs behind the half that leads depends on when their two
     workgroups get their CUs; with matrix products on a second stream keeping every CU busy the

@@ -299,17 +299,18 @@ __global__ __launch_bounds__(256) void gather_kernel(const TIO* __restrict__ E,
 // null for the last block) and the next one reads them from `ghin` (null for the first block).
 // kMulti: this launch is one of several blocks (the hand-over code is compiled in only then: in
 // the single-block kernel even an unused hand-over load costs the walk its prefetch distance).
-// kLive (with kMulti): the two blocks of a label axis of up to 128 C W positions run at the same
-// time, as two workgroups on two CUs of one XCD (with few utterances and many label positions
-// one CU's wavefronts are what holds the walk).  The boundary column's scores then cross in
-// `live` ([B][hand_stride] 64-bit words, zero before the launch): entry s is the score entering
-// step s with s + 1 in its upper half, so that a reader can tell a written entry by itself --
-// one store, no fence, no separate counter.  The upper block asks for its entries four groups
-// ahead like every other operand (lane j for entry 4g + j), checks the tags when it comes to
-// use them, and asks again (bounded, like the waits inside a workgroup) if the lower block has
-// not got there yet; it starts kLiveLag groups behind, so that in the steady state what it asks
-// for has long been written.  Workgroups are dispatched in launch order and an utterance's
-// lower block has the smaller index, so the block that is waited for is always running or done.
+// kLive (with kMulti): the live_n blocks of 64 C W positions of a label axis run at the same
+// time, as live_n workgroups on as many CUs of one XCD (with few utterances and many label
+// positions one CU's wavefronts are what holds the walk).  The scores of a boundary column then
+// cross in `live` (live_n - 1 arrays of [B][hand_stride] 64-bit words, zero before the launch):
+// entry s is the score entering step s with s + 1 in its upper half, so that a reader can tell
+// a written entry by itself -- one store, no fence, no separate counter.  A block asks for the
+// entries of the block below it four groups ahead like every other operand (lane j for entry
+// 4g + j), checks the tags when it comes to use them, and asks again (bounded, like the waits
+// inside a workgroup) if the block below has not got there yet; it starts kLiveLag groups
+// behind it, so that in the steady state what it asks for has long been written.  Workgroups
+// are dispatched in launch order and a block has a smaller index than the block above it, so
+// the block that is waited for is always running or done.
 constexpr int kLiveLag = 12;
 constexpr int kBetaLiveLag = 24;  // (the dalpha walk asks eight groups ahead, not four)
 constexpr int kLiveWaveLag = 2;  // groups between the wavefronts of a live block at the start (8 elsewhere)
@@ -321,19 +322,22 @@ __global__ __launch_bounds__(64 * W) void alpha_kernel(Planes p, const int* __re
                                                        int* __restrict__ trouble, int u_base,
                                                        const float* __restrict__ ghin,
                                                        float* __restrict__ ghout,
-                                                       unsigned long long* __restrict__ live) {
+                                                       unsigned long long* __restrict__ live,
+                                                       int live_n) {
   static_assert(kMulti || !kLive, "live blocks are blocks");
   extern __shared__ __attribute__((aligned(16))) float hand[];  // [W-1][hand_stride]: entry s =
                                                                 // score handed to step s
   __shared__ int done[W];          // steps a wavefront has published
   __shared__ unsigned long long etab[32];  // expf's table (rnnt_libm.h)
-  // live blocks: workgroups go round the 8 XCDs in launch order; ids i and i + 8 share one, and
-  // with it the L2 the boundary scores cross in
-  const int live_half = kLive ? (blockIdx.x >> 3) & 1 : 0;
-  const int b = kLive ? (blockIdx.x >> 4) * 8 + (blockIdx.x & 7) : blockIdx.x, lane = threadIdx.x & 63;
+  // live blocks: workgroups go round the 8 XCDs in launch order; ids i, i + 8, i + 16 .. share
+  // one, and with it the L2 the boundary scores cross in.  Eight utterances take 8 live_n
+  // consecutive ids, block by block, lowest block first.
+  const int live_block = kLive ? (int)(blockIdx.x >> 3) % live_n : 0;
+  const int b = kLive ? (int)(blockIdx.x / (8 * live_n)) * 8 + (blockIdx.x & 7) : blockIdx.x;
+  const int lane = threadIdx.x & 63;
   if (kLive) {
     if (b >= d.B) return;
-    u_base = live_half * 64 * C * W;
+    u_base = live_block * 64 * C * W;
   }
   const int wave = W > 1 ? __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) : 0;
   int Tb, Ub;
@@ -351,9 +355,15 @@ __global__ __launch_bounds__(64 * W) void alpha_kernel(Planes p, const int* __re
   const float* gin = (kMulti && !kLive && ghin) ? ghin + (size_t)b * hand_stride : nullptr;
   float* gout = (kMulti && !kLive && ghout) ? ghout + (size_t)b * hand_stride : nullptr;
   if (kMulti && gout && threadIdx.x == 0) gout[0] = kOutside;  // nothing enters step 0
-  // live blocks: block 0 writes the entries, block 1 reads them
-  unsigned long long* lrow = kLive ? live + (size_t)b * hand_stride : nullptr;
-  const bool live_in = kLive && live_half == 1, live_out = kLive && live_half == 0;
+  // live blocks: block h reads the entries of boundary h - 1 and writes those of boundary h
+  // (live_n - 1 arrays of [B][hand_stride] entries; the lowest block asks at its own boundary,
+  // for nothing)
+  const bool live_in = kLive && live_block > 0, live_out = kLive && live_block < live_n - 1;
+  const unsigned long long* lrow =
+      kLive ? live + ((size_t)max(live_block - 1, 0) * d.B + b) * hand_stride : nullptr;
+  unsigned long long* lrow_out =
+      kLive ? live + ((size_t)min(live_block, max(live_n - 2, 0)) * d.B + b) * hand_stride
+            : nullptr;
   auto live_entry = [](int s, float x) -> unsigned long long {
     return ((unsigned long long)(unsigned)(s + 1) << 32) | (unsigned long long)__float_as_uint(x);
   };
@@ -374,7 +384,8 @@ __global__ __launch_bounds__(64 * W) void alpha_kernel(Planes p, const int* __re
     return e;
   };
   if (live_out && threadIdx.x == 0)  // nothing enters step 0
-    __hip_atomic_store(lrow, live_entry(0, kOutside), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(lrow_out, live_entry(0, kOutside), __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
   exp2_table_to_lds(etab);
   if (W > 1) {
     if (threadIdx.x < W) done[threadIdx.x] = 0;
@@ -536,7 +547,7 @@ __global__ __launch_bounds__(64 * W) void alpha_kernel(Planes p, const int* __re
         if (live_out && wave == W - 1 && lane == 63) {
 #pragma unroll
           for (int j = 0; j < 4; ++j)
-            __hip_atomic_store(lrow + 4 * g + 1 + j, live_entry(4 * g + 1 + j, gsend[j]),
+            __hip_atomic_store(lrow_out + 4 * g + 1 + j, live_entry(4 * g + 1 + j, gsend[j]),
                                __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
       }
@@ -663,14 +674,14 @@ constexpr int beta_depth(int C) { return C <= 2 ? 8 : C <= 4 ? 4 : 3; }
 // wavefront below reads them one group later (the same hand-over as between blocks, with the
 // bounded wait of alpha_kernel).  Every wavefront runs all groups, past the utterance's labels
 // too (zeros), so nobody waits for a wavefront that has left.
-// kLive: the two halves of a label axis of up to 128 C W positions as two workgroups running at
-// the same time, as in alpha_kernel with the directions turned round: the UPPER half leads (and
-// has the smaller workgroup index, so it is dispatched first), lane 0 of its wavefront 0 leaves
-// dalpha of the half's first column in `live` (entry s: the value on diagonal s, s + 1 in the
-// upper word; zero before the launch), and the highest wavefront of the lower half asks for
-// them, lane j for entry 4g + 1 + j, with its weights, checks the tags when it uses them and
-// asks again, bounded, for what was not there yet.  An utterance whose labels end in the lower
-// half has no upper half: that workgroup leaves at once and nothing is taken from `live`.
+// kLive: the live_n blocks of 64 C W positions of a label axis as live_n workgroups running at
+// the same time, as in alpha_kernel with the directions turned round: the HIGHEST block leads
+// (and has the smallest workgroup index, so it is dispatched first), lane 0 of a block's
+// wavefront 0 leaves dalpha of the block's first column in `live` (entry s: the value on
+// diagonal s, s + 1 in the upper word; zero before the launch), and the highest wavefront of the
+// block below asks for them, lane j for entry 4g + 1 + j, with its weights, checks the tags when
+// it uses them and asks again, bounded, for what was not there yet.  A block above an
+// utterance's last label leaves at once, and the utterance's highest block takes nothing.
 template <int C, int W, bool kMulti, bool kLive = false>
 __global__ __launch_bounds__(64 * W) void beta_kernel(Planes p, const int* __restrict__ labels,
                                                       const int* __restrict__ inLen,
@@ -679,20 +690,21 @@ __global__ __launch_bounds__(64 * W) void beta_kernel(Planes p, const int* __res
                                                       const float* __restrict__ ghin,
                                                       float* __restrict__ ghout, int spin_limit,
                                                       int* __restrict__ trouble,
-                                                      unsigned long long* __restrict__ live) {
+                                                      unsigned long long* __restrict__ live,
+                                                      int live_n) {
   static_assert(W == 1 || !kMulti, "several wavefronts only when one launch covers the label axis");
   static_assert(!kLive || (!kMulti && W > 1), "live halves are dealt to several wavefronts");
   extern __shared__ __attribute__((aligned(16))) float hand[];  // [W-1][hand_stride]: entry s =
                                                                 // dalpha on diagonal s
   __shared__ int done[W];  // groups a wavefront has published
-  // live halves: workgroups go round the 8 XCDs in launch order; indices i and i + 8 share one
-  const int live_half = kLive ? 1 - ((blockIdx.x >> 3) & 1) : 0;  // the upper half comes first
-  const int b = kLive ? (blockIdx.x >> 4) * 8 + (blockIdx.x & 7) : blockIdx.x;
+  // live blocks: as in alpha_kernel, the highest block first
+  const int live_block = kLive ? live_n - 1 - (int)(blockIdx.x >> 3) % live_n : 0;
+  const int b = kLive ? (int)(blockIdx.x / (8 * live_n)) * 8 + (blockIdx.x & 7) : blockIdx.x;
   const int lane = threadIdx.x & 63;
   const int wave = W > 1 ? __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) : 0;
   if (kLive) {
     if (b >= d.B) return;
-    u_base = live_half * 64 * C * W;
+    u_base = live_block * 64 * C * W;
   }
   int Tb, Ub;
   utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
@@ -727,9 +739,16 @@ __global__ __launch_bounds__(64 * W) void beta_kernel(Planes p, const int* __res
   float* gout = (kMulti && ghout) ? ghout + (size_t)b * hand_stride : nullptr;
   // live halves: the upper one writes the entries; the highest wavefront of the lower one takes
   // them if the utterance has an upper half at all
-  unsigned long long* lrow = kLive ? live + (size_t)b * hand_stride : nullptr;
-  const bool live_out = kLive && live_half == 1;
-  const bool live_takes = kLive && live_half == 0 && wave == W - 1 && 64 * C * W < Ub;
+  // block h writes the entries of boundary h - 1 and takes those of boundary h, if the utterance
+  // has a block above it at all (the highest block asks at its own boundary, for nothing)
+  const unsigned long long* lrow =
+      kLive ? live + ((size_t)min(live_block, max(live_n - 2, 0)) * d.B + b) * hand_stride
+            : nullptr;
+  unsigned long long* lrow_out =
+      kLive ? live + ((size_t)max(live_block - 1, 0) * d.B + b) * hand_stride : nullptr;
+  const bool live_out = kLive && live_block > 0;
+  const bool live_takes = kLive && live_block < live_n - 1 && wave == W - 1 &&
+                          u_base + 64 * C * W < Ub;
   auto live_load = [&](int s) -> unsigned long long {
     return __hip_atomic_load(lrow + s, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   };
@@ -889,7 +908,7 @@ __global__ __launch_bounds__(64 * W) void beta_kernel(Planes p, const int* __res
       if (live_out && wave == 0 && lane == 0) {
 #pragma unroll
         for (int j = 0; j < 4; ++j)
-          __hip_atomic_store(lrow + 4 * g + j,
+          __hip_atomic_store(lrow_out + 4 * g + j,
                              ((unsigned long long)(unsigned)(4 * g + j + 1) << 32) |
                                  (unsigned long long)__float_as_uint(gsend[j]),
                              __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -1957,11 +1976,28 @@ int trouble_flag(int** out) {
 // ------------------------------------------------------------------ workspace layout
 static size_t align_up(size_t x) { return (x + 255) & ~(size_t)255; }
 
+// Blocks of 256 label positions that the alpha and dalpha walks run side by side, one workgroup
+// each: 0 where one workgroup takes the label axis (up to 256 positions), where the batch would
+// need more workgroups than the device has CUs to spare, or where a block's three hand-over
+// arrays do not fit LDS.
+int live_blocks(const Dims& d) {
+  const int n = (d.U + 255) / 256;
+  if (n < 2 || n > 16 || d.B * n > 192) return 0;
+  if (3 * sizeof(float) * (size_t)d.Dp > 144 * 1024) return 0;
+  return n;
+}
+// The two hand-over vectors of the planes hold the walks' tagged 64-bit entries as well: one
+// array of [B][Dp] entries per boundary between live blocks.  In units of [B][Dp] floats each.
+static int hand_arrays(const Dims& d) {
+  const int n = live_blocks(d);
+  return n > 2 ? n - 1 : 1;
+}
+
 size_t planes_bytes(const Dims& d, bool decode_only) {
   const size_t plane = align_up(sizeof(float) * (size_t)d.B * d.Ua * d.Dp + 64);
   return (decode_only ? 1 : 6) * plane + align_up(sizeof(float) * (size_t)d.B * d.Tp) +
          4 * align_up(sizeof(float) * (size_t)d.B * d.Ua) +
-         2 * align_up(sizeof(float) * (size_t)d.B * d.Dp);
+         2 * align_up(sizeof(float) * (size_t)d.B * d.Dp * hand_arrays(d));
 }
 
 void carve_planes(void* base, const Dims& d, Planes* p, bool decode_only) {
@@ -1977,7 +2013,7 @@ void carve_planes(void* base, const Dims& d, Planes* p, bool decode_only) {
   p->eb = take(align_up(sizeof(float) * (size_t)d.B * d.Tp));
   const size_t bu = align_up(sizeof(float) * (size_t)d.B * d.Ua);
   p->pb = take(bu); p->pl = take(bu); p->gB = take(bu); p->gL = take(bu);
-  const size_t bh = align_up(sizeof(float) * (size_t)d.B * d.Dp);
+  const size_t bh = align_up(sizeof(float) * (size_t)d.B * d.Dp * hand_arrays(d));
   p->hand[0] = take(bh); p->hand[1] = take(bh);
 }
 
@@ -2038,10 +2074,24 @@ __global__ void clear_words_kernel(int* x, int n) {
   if (i < n) x[i] = 0;
 }
 
-// Whether the alpha walk takes a label axis as two blocks running side by side (the two
-// hand-over vectors of the planes then hold one array of 64-bit entries).
-static bool alpha_live_blocks(const Dims& d) {
-  return d.Ua == 512 && d.B <= 96 && label_blocks(d) == 1;
+// Launches the side-by-side form of a walk (K: its kernel, four wavefronts of one position a
+// lane) for live_blocks(d) blocks: clears the tagged entries, then one workgroup per utterance
+// and block, eight utterances' blocks in consecutive indices.
+template <typename K, typename... Args>
+static int launch_live(K kernel, const Planes& p, const Dims& d, int n,
+                       hipStream_t s, Args... args) {
+  unsigned long long* live = reinterpret_cast<unsigned long long*>(p.hand[0]);
+  const size_t lds = sizeof(float) * 3 * (size_t)d.Dp;
+  const int words = 2 * d.B * d.Dp * (n - 1);
+  hipLaunchKernelGGL(clear_words_kernel, dim3((words + 255) / 256), dim3(256), 0, s,
+                     reinterpret_cast<int*>(live), words);
+  RNNT_LAUNCH_CHECK("clear_words_kernel");
+  if (lds > 64 * 1024)
+    RNNT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+  hipLaunchKernelGGL(kernel, dim3(8 * n * ((d.B + 7) / 8)), dim3(256), lds, s, args..., live, n);
+  RNNT_LAUNCH_CHECK("lattice walk (blocks side by side)");
+  return kOk;
 }
 
 int launch_alpha(const Planes& p, const int* inLen, const int* labLen, float* costs,
@@ -2062,25 +2112,15 @@ int launch_alpha(const Planes& p, const int* inLen, const int* labLen, float* co
   const size_t lds = W > 1 ? sizeof(float) * (size_t)(W - 1) * stride : 0;
   int* trouble = nullptr;
   RNNT_TRY(trouble_flag(&trouble));
-  // 257 .. 512 label positions and few enough utterances that the device has CUs to spare: two
-  // blocks of 256 positions side by side on two CUs, four wavefronts of one position a lane each
-  // (B=8 T=10000, 401 positions: 176 ns a step against 235 on one CU; from about a hundred
-  // utterances on the planes' traffic holds both forms, B=128 T=2000: 241 ns)
-  if (alpha_live_blocks(d) && W == 4) {
-    unsigned long long* live = reinterpret_cast<unsigned long long*>(p.hand[0]);
-    const int words = 2 * d.B * stride;
-    hipLaunchKernelGGL(clear_words_kernel, dim3((words + 255) / 256), dim3(256), 0, s,
-                       reinterpret_cast<int*>(live), words);
-    RNNT_LAUNCH_CHECK("clear_words_kernel");
-    if (lds > 64 * 1024)
-      RNNT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(alpha_kernel<1, 4, true, true>),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    hipLaunchKernelGGL((alpha_kernel<1, 4, true, true>), dim3(16 * ((d.B + 7) / 8)), dim3(256), lds, s, p,
-                       inLen, labLen, costs, d, stride, g_spin_limit, trouble, 0, nullptr, nullptr,
-                       live);
-    RNNT_LAUNCH_CHECK("alpha_kernel (live blocks)");
-    return kOk;
-  }
+  // From 257 label positions, with few enough utterances that the device has the CUs: blocks
+  // of 256 positions side by side on as many CUs, four wavefronts of one position a lane each
+  // (B=8 T=10000, 401 positions: 176 ns a step against 235 on one CU; B=8 T=2000, 513 .. 1024
+  // positions: 523 .. 539 ns on one CU with two to four positions a lane; from about a hundred
+  // utterances on the planes' traffic holds every form, B=128 T=2000: 241 ns)
+  if (const int n = live_blocks(d))
+    return launch_live(alpha_kernel<1, 4, true, true>, p, d, n, s,
+                       p, inLen, labLen, costs, d, stride, g_spin_limit, trouble, 0,
+                       (const float*)nullptr, (float*)nullptr);
   for (int k = 0; k < nblocks; ++k) {  // lowest block first
     const float* ghin = k == 0 ? nullptr : p.hand[(k - 1) & 1];
     float* ghout = k == nblocks - 1 ? nullptr : p.hand[k & 1];
@@ -2093,7 +2133,7 @@ int launch_alpha(const Planes& p, const int* inLen, const int* labLen, float* co
                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));   \
     hipLaunchKernelGGL((alpha_kernel<C, W, M>), dim3(d.B), dim3(64 * W), lds, s, p, inLen,  \
                        labLen, costs, d, stride, g_spin_limit, trouble, u_base, ghin,        \
-                       ghout, nullptr);                                                      \
+                       ghout, nullptr, 0);                                                   \
     break;
       CASE(1, 1, false) CASE(2, 1, false) CASE(4, 1, false) CASE(8, 1, false) CASE(16, 1, false)
       CASE(1, 2, false) CASE(2, 2, false) CASE(4, 2, false) CASE(8, 2, false)
@@ -2134,23 +2174,12 @@ int launch_beta(const Planes& p, const int* labels, const int* inLen, const int*
   const size_t lds = W > 1 ? sizeof(float) * (size_t)(W - 1) * stride : 0;
   int* trouble = nullptr;
   RNNT_TRY(trouble_flag(&trouble));
-  // 257 .. 512 label positions in few enough utterances: the two halves side by side on two
-  // CUs, four wavefronts of one position a lane each (as in launch_alpha)
-  if (alpha_live_blocks(d) && W == 4) {
-    unsigned long long* live = reinterpret_cast<unsigned long long*>(p.hand[0]);
-    const int words = 2 * d.B * stride;
-    hipLaunchKernelGGL(clear_words_kernel, dim3((words + 255) / 256), dim3(256), 0, s,
-                       reinterpret_cast<int*>(live), words);
-    RNNT_LAUNCH_CHECK("clear_words_kernel");
-    if (lds > 64 * 1024)
-      RNNT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(beta_kernel<1, 4, false, true>),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    hipLaunchKernelGGL((beta_kernel<1, 4, false, true>), dim3(16 * ((d.B + 7) / 8)), dim3(256),
-                       lds, s, p, labels, inLen, labLen, d, stride, 0, nullptr, nullptr,
-                       g_spin_limit, trouble, live);
-    RNNT_LAUNCH_CHECK("beta_kernel (live halves)");
-    return kOk;
-  }
+  // from 257 label positions in few enough utterances: blocks of 256 positions side by side
+  // (as in launch_alpha)
+  if (const int n = live_blocks(d))
+    return launch_live(beta_kernel<1, 4, false, true>, p, d, n, s,
+                       p, labels, inLen, labLen, d, stride, 0, (const float*)nullptr,
+                       (float*)nullptr, g_spin_limit, trouble);
   for (int k = nblocks - 1; k >= 0; --k) {  // highest block first
     const float* ghin = k == nblocks - 1 ? nullptr : p.hand[(k + 1) & 1];
     float* ghout = k == 0 ? nullptr : p.hand[k & 1];
@@ -2163,7 +2192,7 @@ int launch_beta(const Planes& p, const int* labels, const int* inLen, const int*
                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));  \
     hipLaunchKernelGGL((beta_kernel<C, W, M>), dim3(d.B), dim3(64 * W), lds, s, p, labels, \
                        inLen, labLen, d, stride, u_base, ghin, ghout, g_spin_limit,        \
-                       trouble, nullptr);                                                   \
+                       trouble, nullptr, 0);                                                \
     break;
       CASE(1, 1, false) CASE(2, 1, false) CASE(4, 1, false) CASE(8, 1, false) CASE(16, 1, false)
       CASE(2, 2, false) CASE(4, 2, false) CASE(8, 2, false)
