@@ -369,14 +369,17 @@ def test_two_halves_of_a_label_axis_walked_side_by_side_carry_the_reference_bits
 
 
 @pytest.mark.parametrize("B,T,U", [(5, 200, 513), (9, 120, 700), (3, 60, 1000), (4, 90, 1025),
-                                   (2, 40, 2100), (70, 6, 600), (40, 5, 1025), (12, 4, 4200)])
+                                   (2, 40, 2100), (70, 6, 600), (40, 5, 1025), (12, 4, 4200),
+                                   (300, 3, 1100)])
 def test_label_axis_as_a_chain_of_blocks_side_by_side_and_where_it_is_not(B, T, U):
     """From 513 label positions the alpha and dalpha walks run three and more blocks of 256
     positions side by side, each following the one before it through its own array of tagged
-    entries -- as long as the batch leaves the device the CUs for it (utterances x blocks at
-    most 192, blocks at most 16).  70 x 3 and 40 x 5 workgroups are too many and 17 blocks too
-    long: those take one workgroup per utterance again, a lane owning several positions, or a
-    launch per 1024 positions.  Either way the reference's bits.  U counts the rows of
+    entries -- up to 1024 positions as long as the batch leaves the device the CUs for it
+    (utterances x blocks at most 192), beyond whatever the batch (40 x 5 workgroups, 300 x 5:
+    more than the device runs at once, so later utterances' blocks queue behind earlier ones).
+    70 x 3 workgroups for 600 positions are too many and 17 blocks too long: those take one
+    workgroup per utterance again, a lane owning several positions, or a launch per 1024
+    positions.  Either way the reference's bits.  U counts the rows of
     predictions; ragged batches, so that some utterances end blocks below the top one."""
     cfg = small_config(B, T, U - 1, 4, ragged=True)
     E, P, labels, il, ll = unpack(make_inputs(cfg, seed=B * 7 + U))

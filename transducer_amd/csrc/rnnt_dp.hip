@@ -1977,12 +1977,17 @@ int trouble_flag(int** out) {
 static size_t align_up(size_t x) { return (x + 255) & ~(size_t)255; }
 
 // Blocks of 256 label positions that the alpha and dalpha walks run side by side, one workgroup
-// each: 0 where one workgroup takes the label axis (up to 256 positions), where the batch would
-// need more workgroups than the device has CUs to spare, or where a block's three hand-over
-// arrays do not fit LDS.
+// each: 0 where one workgroup takes the label axis (up to 256 positions), where a block's three
+// hand-over arrays do not fit LDS, and, up to 1024 positions, where the batch would need more
+// workgroups than the device has CUs to spare (one workgroup per utterance is then as good:
+// with that many utterances the planes' traffic holds the walks either way).  Past 1024
+// positions the blocks go side by side whatever the batch: workgroups are dispatched in order,
+// a block after the block it follows, so more workgroups than CUs only queue -- and the other
+// way there, a launch per 1024 positions with sixteen positions a lane, is many times slower.
 int live_blocks(const Dims& d) {
   const int n = (d.U + 255) / 256;
-  if (n < 2 || n > 16 || d.B * n > 192) return 0;
+  if (n < 2 || n > 16) return 0;
+  if (d.B * n > 192 && d.U <= 1024) return 0;
   if (3 * sizeof(float) * (size_t)d.Dp > 144 * 1024) return 0;
   return n;
 }
