@@ -2316,8 +2316,11 @@ int launch_viterbi(const Planes& p, const float* bestS, const float* argS,
   const int cpl = block_cells_per_lane(d), nblocks = label_blocks(d);
   const int stride = d.Dp;
   const int nw = viterbi_words(d);
-  const int W = (cpl >= 2 && stride * sizeof(float) <= 16 * 1024) ? 2 : 1;
-  // dynamic LDS: one int per label position, the hand-over array between the two wavefronts,
+  // (four wavefronts from 257 label positions while their hand-over arrays fit: B=8 T=2000,
+  // 209 -> 167 ns a step at 257 positions, 446 -> 254 at 513, 551 -> 340 at 1000)
+  const int W = (nblocks == 1 && cpl >= 4 && 3 * stride * sizeof(float) <= 48 * 1024) ? 4
+                : (cpl >= 2 && stride * sizeof(float) <= 16 * 1024) ? 2 : 1;
+  // dynamic LDS: one int per label position, the hand-over arrays between the wavefronts,
   // and the decision columns when they fit (one block only: with several, every block's columns
   // must be there for the backtrace of the last launch)
   const size_t base_lds = sizeof(int) * (size_t)((d.U + 3) & ~3) +
@@ -2354,6 +2357,7 @@ int launch_viterbi(const Planes& p, const float* bestS, const float* argS,
     break;
       CASE(1, 1) CASE(2, 1) CASE(4, 1) CASE(8, 1) CASE(16, 1)
       CASE(1, 2) CASE(2, 2) CASE(4, 2) CASE(8, 2)
+      CASE(1, 4) CASE(2, 4) CASE(4, 4)
       CASE_MULTI(16, 1) CASE_MULTI(8, 2)  // several blocks: always 1024 positions each
 #undef CASE
 #undef CASE_MULTI
