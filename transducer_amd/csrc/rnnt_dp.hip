@@ -2316,7 +2316,7 @@ int launch_viterbi(const Planes& p, const float* bestS, const float* argS,
   const int cpl = block_cells_per_lane(d), nblocks = label_blocks(d);
   const int stride = d.Dp;
   const int nw = viterbi_words(d);
-  // (four wavefronts from 257 label positions while their hand-over arrays fit: B=8 T=2000,
+  // (four wavefronts from 129 label positions while their hand-over arrays fit: B=8 T=2000,
   // 209 -> 167 ns a step at 257 positions, 446 -> 254 at 513, 551 -> 340 at 1000)
   const int W = (nblocks == 1 && cpl >= 4 && 3 * stride * sizeof(float) <= 48 * 1024) ? 4
                 : (cpl >= 2 && stride * sizeof(float) <= 16 * 1024) ? 2 : 1;
