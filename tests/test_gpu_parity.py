@@ -434,11 +434,14 @@ def test_two_halves_side_by_side_keep_their_bits_while_the_device_is_busy():
 @pytest.mark.parametrize("T,U,V", [(40, 1024, 9), (30, 1025, 9), (50, 1500, 7), (24, 2100, 520),
                                    (300, 1300, 5)])
 def test_label_axis_longer_than_one_block_of_1024_positions(T, U, V):
-    """The lattice walks give a lane at most 16 label positions: 1024 per launch.  A longer axis
-    is walked block by block (alpha and the best path upwards, dalpha downwards), the scores of
-    the boundary column handed on through memory; the reference strides its loop instead
-    (transducer_cuda.cu:74,150,220).  U counts the rows of predictions: 1024 is the last single
-    block, 1025 the first double one, 2100 takes three; V = 520 also takes the whole loss
+    """A workgroup of the lattice walks takes at most 1024 label positions.  A longer axis is
+    walked in blocks, the scores of the boundary column handed on through memory: the best path
+    a launch per 1024 positions, lowest block first; alpha and dalpha as blocks of 256 positions
+    side by side (a batch this small; the other form of theirs is covered by
+    test_label_axis_as_a_chain_of_blocks_side_by_side_and_where_it_is_not).  The reference
+    strides its loop instead (transducer_cuda.cu:74,150,220).  U counts the rows of predictions:
+    for the best path 1024 is the last single block, 1025 the first double one, 2100 takes
+    three; V = 520 also takes the whole loss
     through the scattered blank / label terms (the folded ones stop at 1024 labels).  Same bars
     as everywhere: the reference's bits at the boundary, the oracle's tolerance for the loss,
     the exact path."""
