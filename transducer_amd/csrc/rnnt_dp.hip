@@ -2218,9 +2218,12 @@ int launch_sparse(const Planes& p, const float* bsum, const float* emT, float* e
   if (d.B == 0 || d.T == 0 || d.U == 0) return kOk;
   if (!bsum || !emT) return fail(kInvalid, "sparse terms: the per-frame terms were not formed");
   const size_t rows_bytes = sizeof(float) * 64 * (size_t)(d.V | 1);
-  if (add && rows_bytes <= 64 * 1024 && labels != nullptr) {
+  // (a small vocabulary also when the terms are to be stored: the arrays are zero-filled then,
+  // and adding to zeros leaves the same bits -- B=8 T=10000 U=400 V=32: 1.67 ms with one
+  // hardware add per term, all of them into 128 bytes a frame)
+  if (rows_bytes <= 64 * 1024 && labels != nullptr) {
     hipLaunchKernelGGL(sparse_e_rows_kernel, dim3((d.T + 63) / 64, d.B), dim3(64), rows_bytes, s,
-                       bsum, emT, egrads, labels, inLen, labLen, scale, d);
+                       bsum, emT, egrads, labels, inLen, labLen, add ? scale : nullptr, d);
     RNNT_LAUNCH_CHECK("sparse_e_rows_kernel");
   } else {
     hipLaunchKernelGGL(sparse_e_kernel, dim3((d.T + 255) / 256, d.B), dim3(256), 0, s, bsum, emT,
@@ -2318,8 +2321,12 @@ int launch_viterbi(const Planes& p, const float* bestS, const float* argS,
   const int nw = viterbi_words(d);
   // (four wavefronts from 129 label positions while their hand-over arrays fit: B=8 T=2000,
   // 209 -> 167 ns a step at 257 positions, 446 -> 254 at 513, 551 -> 340 at 1000)
-  const int W = (nblocks == 1 && cpl >= 4 && 3 * stride * sizeof(float) <= 48 * 1024) ? 4
-                : (cpl >= 2 && stride * sizeof(float) <= 16 * 1024) ? 2 : 1;
+  // (B=8 T=10000 U=400, the reference's kernel benchmark: 3.5 ms with one wavefront of eight
+  // positions a lane, which is what 64 KB of LDS allowed)
+  const size_t taken_lds = sizeof(int) * (size_t)((d.U + 3) & ~3);
+  const int W = (nblocks == 1 && cpl >= 4 &&
+                 taken_lds + 3 * stride * sizeof(float) <= 144 * 1024) ? 4
+                : (cpl >= 2 && taken_lds + stride * sizeof(float) <= 48 * 1024) ? 2 : 1;
   // dynamic LDS: one int per label position, the hand-over arrays between the wavefronts,
   // and the decision columns when they fit (one block only: with several, every block's columns
   // must be there for the backtrace of the last launch)
@@ -2328,7 +2335,7 @@ int launch_viterbi(const Planes& p, const float* bestS, const float* argS,
   const size_t cols_lds = sizeof(unsigned) * (size_t)64 * cpl * nw;
   const bool use_lds = nblocks == 1 && base_lds + cols_lds <= 60 * 1024;
   const size_t lds = base_lds + (use_lds ? cols_lds : 0);
-  if (lds > 64 * 1024)
+  if (lds > 150 * 1024)
     return fail(kInvalid, "viterbi: %d label positions and %d steps need %zu bytes of LDS", d.U,
                 stride, lds);
   int* trouble = nullptr;
@@ -2344,10 +2351,15 @@ int launch_viterbi(const Planes& p, const float* bestS, const float* argS,
       hipLaunchKernelGGL((viterbi_kernel<C, W, true, false>), dim3(d.B), dim3(64 * W), lds,   \
                          s, p, bestS, argS, inLen, labLen, gcols, labels_out, d, stride, nw,   \
                          g_spin_limit, trouble, u_base, ghin, ghout, traces);                  \
-    else                                                                                       \
+    else {                                                                                     \
+      if (lds > 64 * 1024)                                                                     \
+        RNNT_HIP(hipFuncSetAttribute(                                                          \
+            reinterpret_cast<const void*>(viterbi_kernel<C, W, false, false>),                 \
+            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));                            \
       hipLaunchKernelGGL((viterbi_kernel<C, W, false, false>), dim3(d.B), dim3(64 * W), lds,  \
                          s, p, bestS, argS, inLen, labLen, gcols, labels_out, d, stride, nw,   \
                          g_spin_limit, trouble, u_base, ghin, ghout, traces);                  \
+    }                                                                                          \
     break;
 #define CASE_MULTI(C, W)                                                                       \
   case 10000 + C * 100 + W:                                                                    \
