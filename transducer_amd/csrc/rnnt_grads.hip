@@ -24,6 +24,14 @@
 #include "rnnt_split.h"
 #include "rnnt_grads.h"
 
+// This file is compiled in six parts side by side (-DRNNT_GRADS_PART=0..5: egrads then pgrads,
+// each for fp32, bf16 and fp16 scores; a part instantiates only its own kernels), or whole when
+// the macro is not given.
+#ifndef RNNT_GRADS_PART
+#define RNNT_GRADS_PART -1
+#endif
+#define RNNT_IN_PART(n) (RNNT_GRADS_PART < 0 || RNNT_GRADS_PART == (n))
+
 namespace rnnt {
 
 namespace {
@@ -729,7 +737,9 @@ __global__ __launch_bounds__(256, 2) void pgrads_stream_kernel(
 
 }  // namespace
 
+#if RNNT_IN_PART(0)
 bool egrads_one_pass(const Dims& d) { return wplane_up(d.U) <= 16 * kEsMaxS; }
+#endif
 
 // One pass of the egrads kernels over the frames of `win` (all slices of the label axis), into
 // `out` (the caller's array, or a wide copy of a window of it).
@@ -765,7 +775,10 @@ static int egrads_window(const TIO* E, const TIO* P, const float* mE, const floa
   // (only the kernels that fold sparse terms in come in both forms)
 #define RNNT_EG_LAUNCH(MODE, DL, SP)                                                          \
   do {                                                                                        \
-    if constexpr (MODE == kEgWhole || MODE == kEgFinal) {                                     \
+    if constexpr (sizeof(TOUT) == 2 && MODE != kEgWhole) {                                    \
+      /* 16-bit gradients of several slices add up in a wide window: never reached */        \
+      return fail(kInvalid, "egrads: slices of 16-bit gradients need a wide window");        \
+    } else if constexpr (MODE == kEgWhole || MODE == kEgFinal) {                              \
       if (many) RNNT_EG_LAUNCH_(MODE, true, DL, SP);                                          \
       else RNNT_EG_LAUNCH_(MODE, false, DL, SP);                                              \
     } else {                                                                                  \
@@ -833,6 +846,7 @@ static int egrads_stream_any(const TIO* E, const TIO* P, const float* mE, const 
   }
   return kOk;
 }
+#if RNNT_IN_PART(0)
 int launch_egrads_stream(const float* E, const float* P, const float* mE, const float* mP,
                          const float* Wn, const float* deltas, float* egrads, const int* inLen,
                          const int* labLen, const Dims& d, bool accumulate,
@@ -840,6 +854,8 @@ int launch_egrads_stream(const float* E, const float* P, const float* mE, const 
   return egrads_stream_any(E, P, mE, mP, Wn, deltas, egrads, inLen, labLen, d, accumulate, sparse,
                            s);
 }
+#endif
+#if RNNT_IN_PART(1)
 int launch_egrads_stream(const bf16_t* E, const bf16_t* P, const float* mE, const float* mP,
                          const float* Wn, const float* deltas, bf16_t* egrads, const int* inLen,
                          const int* labLen, const Dims& d, bool accumulate,
@@ -848,6 +864,8 @@ int launch_egrads_stream(const bf16_t* E, const bf16_t* P, const float* mE, cons
   return egrads_stream_any(E, P, mE, mP, Wn, deltas, egrads, inLen, labLen, d, accumulate, sparse,
                            s, wide, wide_bytes);
 }
+#endif
+#if RNNT_IN_PART(2)
 int launch_egrads_stream(const f16_t* E, const f16_t* P, const float* mE, const float* mP,
                          const float* Wn, const float* deltas, f16_t* egrads, const int* inLen,
                          const int* labLen, const Dims& d, bool accumulate,
@@ -856,6 +874,7 @@ int launch_egrads_stream(const f16_t* E, const f16_t* P, const float* mE, const 
   return egrads_stream_any(E, P, mE, mP, Wn, deltas, egrads, inLen, labLen, d, accumulate, sparse,
                            s, wide, wide_bytes);
 }
+#endif
 
 // Whether the workgroups of a tile share its frames.  A chunk is always kPsFlush slabs, the
 // period at which the unsplit walk moves its running sum into the second-level sum: the
@@ -872,6 +891,7 @@ static void pgrads_split_plan(const Dims& d, int& chunks, int& per) {
   if (chunks < 2 || tiles * chunks > 256) chunks = 1;
 }
 
+#if RNNT_IN_PART(3)
 size_t pgrads_split_bytes(const Dims& d) {
   if (d.B == 0 || d.T == 0 || d.U == 0 || d.V == 0) return 0;
   int chunks, per;
@@ -880,8 +900,9 @@ size_t pgrads_split_bytes(const Dims& d) {
   const size_t tiles = (size_t)((d.V + 127) / 128) * ((d.U + 127) / 128) * d.B;
   return tiles * chunks * kPsPartialFloats * sizeof(float) + ((tiles * sizeof(int) + 255) & ~(size_t)255);
 }
+#endif
 
-__global__ void zero_ints_kernel(int* x, int n) {
+static __global__ void zero_ints_kernel(int* x, int n) {
   const int i = blockIdx.x * 256 + threadIdx.x;
   if (i < n) x[i] = 0;
 }
@@ -927,6 +948,7 @@ static int pgrads_stream_any(const TIO* E, const TIO* P, const float* mE, const 
   RNNT_LAUNCH_CHECK("pgrads_stream_kernel");
   return kOk;
 }
+#if RNNT_IN_PART(3)
 int launch_pgrads_stream(const float* E, const float* P, const float* mE, const float* mP,
                          const float* Wt, const float* deltas, float* pgrads, const int* inLen,
                          const int* labLen, const Dims& d, bool accumulate,
@@ -935,6 +957,8 @@ int launch_pgrads_stream(const float* E, const float* P, const float* mE, const 
   return pgrads_stream_any(E, P, mE, mP, Wt, deltas, pgrads, inLen, labLen, d, accumulate, sp,
                            split_ws, s);
 }
+#endif
+#if RNNT_IN_PART(4)
 int launch_pgrads_stream(const bf16_t* E, const bf16_t* P, const float* mE, const float* mP,
                          const float* Wt, const float* deltas, bf16_t* pgrads, const int* inLen,
                          const int* labLen, const Dims& d, bool accumulate,
@@ -943,6 +967,8 @@ int launch_pgrads_stream(const bf16_t* E, const bf16_t* P, const float* mE, cons
   return pgrads_stream_any(E, P, mE, mP, Wt, deltas, pgrads, inLen, labLen, d, accumulate, sp,
                            split_ws, s);
 }
+#endif
+#if RNNT_IN_PART(5)
 int launch_pgrads_stream(const f16_t* E, const f16_t* P, const float* mE, const float* mP,
                          const float* Wt, const float* deltas, f16_t* pgrads, const int* inLen,
                          const int* labLen, const Dims& d, bool accumulate,
@@ -951,5 +977,6 @@ int launch_pgrads_stream(const f16_t* E, const f16_t* P, const float* mE, const 
   return pgrads_stream_any(E, P, mE, mP, Wt, deltas, pgrads, inLen, labLen, d, accumulate, sp,
                            split_ws, s);
 }
+#endif
 
 }  // namespace rnnt
