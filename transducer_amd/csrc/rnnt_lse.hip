@@ -40,9 +40,8 @@ namespace rnnt {
 
 namespace {
 
-constexpr int kRows = 128;    // frames per workgroup tile
+constexpr int kRowsMax = 128;  // frames per workgroup tile (64 where the grid would be small)
 constexpr int kSlice = 32;    // v per LDS slab (two matrix-instruction steps)
-constexpr int kSlots = kRows * 4;  // 16-byte slots per piece plane: 4 per row
 constexpr int kFlush = 8;     // slabs between two flushes of the running sums
 constexpr float kSlack = 40.0f;  // a row's reference moves when a value tops it by more than this
 constexpr float kLowest = -1.0e30f;  // stands in for a reference of -inf (a slab of -inf scores)
@@ -142,12 +141,15 @@ __global__ __launch_bounds__(256) void yplanes_kernel(const TIO* __restrict__ P,
 }
 
 // ------------------------------------------------------------------ contraction
-// kWaves = 4: a wavefront owns one block of 32 label positions and all 128 frames (four
-// accumulators).  kWaves = 8: two wavefronts share a block, 64 frames each (two accumulators,
-// half the registers, twice the wavefronts to hide each other's staging).
+// kRows frames x 128 label positions per workgroup.  kWaves = 4: a wavefront owns one block of
+// 32 label positions and all kRows frames (four accumulators at 128 frames, two at 64).
+// kWaves = 8: two wavefronts share a block, half the frames each (half the registers, twice the
+// wavefronts to hide each other's staging).  64 frames for grids that 128 would leave below one
+// workgroup per CU (each workgroup walks all columns, so a small grid is a long walk on a few
+// CUs: B=32 T=400 U=101 V=4096 0.25 -> 0.18 ms, B=8 T=2000 U=101 V=2000 0.147 -> 0.096).
 // kVec: rows start 16-byte aligned and hold a multiple of the vector width, so a thread's eight
 // values are one or two 16-byte loads; otherwise they are fetched one by one.
-template <int kWaves, typename TIO, bool kVec>
+template <int kWaves, typename TIO, bool kVec, int kRows>
 __global__ __launch_bounds__(64 * kWaves, kWaves / 2) void lse_stream_kernel(
     const TIO* __restrict__ E, float* __restrict__ mE, const float* __restrict__ mP,
     const uint4* __restrict__ Yp, float* __restrict__ LN, const int* __restrict__ inLen,
@@ -155,8 +157,10 @@ __global__ __launch_bounds__(64 * kWaves, kWaves / 2) void lse_stream_kernel(
     const int* __restrict__ labels, float* __restrict__ elS, float* __restrict__ ebv,
     float* __restrict__ lnS) {
   constexpr int kThreads = 64 * kWaves;
-  constexpr int MB = 16 / kWaves;          // 32-frame blocks per wavefront
-  constexpr int NR = 512 / kThreads;       // (row, eight v) items a thread stages per slab
+  constexpr int MB = kRows / 8 / kWaves;   // 32-frame blocks per wavefront
+  constexpr int NR = 4 * kRows / kThreads;  // (row, eight v) items a thread stages per slab
+  constexpr int kSlots = kRows * 4;        // 16-byte slots per piece plane: 4 per row
+  static_assert(MB >= 1 && NR >= 1, "a tile gives every wavefront a frame block and every thread a row");
   __shared__ uint4 Xs[2][3][kSlots];
   __shared__ float scale[kRows];  // pending factor for a row's sums (1 when its reference stood)
   __shared__ float mfin[kRows];   // final references, for the write-out
@@ -508,7 +512,7 @@ __global__ __launch_bounds__(64 * kWaves, kWaves / 2) void lse_stream_kernel(
 template <typename TIO>
 static bool lse_stream_ok(const TIO* E, const Dims& d) {
   (void)E;
-  const long total = (long)((d.T + kRows - 1) / kRows) * ((d.U + 127) / 128) * d.B;
+  const long total = (long)((d.T + 63) / 64) * ((d.U + 127) / 128) * d.B;
   return d.V >= 1 && total < (1l << 30);
 }
 bool lse_stream_supported(const float* E, const Dims& d) { return lse_stream_ok(E, d); }
@@ -549,20 +553,28 @@ static int lse_stream_any(const TIO* E, float* mE, const float* mP, float* LN,
                           const Dims& d, hipStream_t s, const int* labels, float* elS,
                           float* eb, float* lnS) {
   const int nub = y_ublocks(d), nks = y_steps(d);
-  const int ttiles = (d.T + kRows - 1) / kRows, utiles = (d.U + 127) / 128;
+  // Tiles of 128 frames; of 64 where those would not give every CU a workgroup (short or few
+  // utterances: B=32 T=400 U=101 V=4096 is 128 tiles of 128 frames, each walking all columns on
+  // a CU of its own while half the device idles).
+  const int utiles = (d.U + 127) / 128;
+  const bool low = (long)((d.T + 127) / 128) * utiles * d.B < 256;
+  const int rows = low ? 64 : kRowsMax;
+  const int ttiles = (d.T + rows - 1) / rows;
   const long total = (long)ttiles * utiles * d.B;
   const int grid = (int)((total + 7) / 8 * 8);
   constexpr int kWaves = 4;
   constexpr int kA = RowAlign<TIO>::kElems;
   const bool vec = d.V % kA == 0 && d.V >= kA && (reinterpret_cast<uintptr_t>(E) & 15) == 0;
-  if (vec)
-    hipLaunchKernelGGL((lse_stream_kernel<kWaves, TIO, true>), dim3(grid), dim3(64 * kWaves), 0,
-                       s, E, mE, mP, static_cast<const uint4*>(scratch), LN, inLen, labLen, d,
-                       ttiles, utiles, (int)total, nub, nks, labels, elS, eb, lnS);
-  else
-    hipLaunchKernelGGL((lse_stream_kernel<kWaves, TIO, false>), dim3(grid), dim3(64 * kWaves), 0,
-                       s, E, mE, mP, static_cast<const uint4*>(scratch), LN, inLen, labLen, d,
-                       ttiles, utiles, (int)total, nub, nks, labels, elS, eb, lnS);
+#define RNNT_LSE_LAUNCH(VEC, ROWS)                                                            \
+  hipLaunchKernelGGL((lse_stream_kernel<kWaves, TIO, VEC, ROWS>), dim3(grid),                 \
+                     dim3(64 * kWaves), 0, s, E, mE, mP, static_cast<const uint4*>(scratch),  \
+                     LN, inLen, labLen, d, ttiles, utiles, (int)total, nub, nks, labels, elS, \
+                     eb, lnS)
+  if (vec && low) RNNT_LSE_LAUNCH(true, 64);
+  else if (vec) RNNT_LSE_LAUNCH(true, kRowsMax);
+  else if (low) RNNT_LSE_LAUNCH(false, 64);
+  else RNNT_LSE_LAUNCH(false, kRowsMax);
+#undef RNNT_LSE_LAUNCH
   RNNT_LAUNCH_CHECK("lse_stream_kernel");
   return kOk;
 }
