@@ -401,6 +401,28 @@ def test_label_axis_as_a_chain_of_blocks_side_by_side_and_where_it_is_not(B, T, 
     assert capi.load().rnnt_hip_check_kernels(None) == 0
 
 
+@pytest.mark.parametrize("B,T,U", [(2, 13000, 70), (2, 12500, 200), (1, 20000, 300), (3, 12400, 129)])
+def test_very_long_utterances_keep_their_wavefronts(B, T, U):
+    """Past about 12000 anti-diagonals the three hand-over arrays of four wavefronts no longer fit
+    LDS: the walks then deal the label axis to workgroups of two wavefronts (one array, good for
+    36000 anti-diagonals), up to 128 positions one workgroup, beyond blocks of 128 side by side.
+    The reference's bits and the exact path, as everywhere."""
+    cfg = small_config(B, T, U - 1, 4, ragged=True)
+    E, P, labels, il, ll = unpack(make_inputs(cfg, seed=T + U))
+    il[0], ll[0] = T, U - 1
+    c = DeviceCase(E, P, labels, il, ll)
+    LN = oracle.log_norms_naive(E, P, il, ll)
+    costs_o, alphas_o = oracle.forward(E, P, LN, labels, il, ll)
+    costs, alphas = gpu_forward(c, LN)
+    assert_same_bits(costs, costs_o, what="costs")
+    assert_same_bits(alphas, alphas_o, what="alphas")
+    eg, pg, lng = gpu_backward(c, alphas, LN)
+    eg_o, pg_o, lng_o = oracle.backward(E, P, np.nan_to_num(alphas_o), LN, labels, il, ll)
+    assert_same_bits(lng, lng_o, what="lngrads")
+    assert_same_bits(eg, eg_o, what="egrads (sparse)")
+    assert np.array_equal(gpu_viterbi(c, LN), oracle.viterbi(E, P, LN, il, ll))
+
+
 def test_two_halves_side_by_side_keep_their_bits_while_the_device_is_busy():
     """How far the half that follows runs behind the half that leads depends on when their two
     workgroups get their CUs; with matrix products on a second stream keeping every CU busy the

@@ -2054,25 +2054,30 @@ int trouble_flag(int** out) {
 // ------------------------------------------------------------------ workspace layout
 static size_t align_up(size_t x) { return (x + 255) & ~(size_t)255; }
 
-// Blocks of 256 label positions that the alpha and dalpha walks run side by side, one workgroup
-// each: 0 where one workgroup takes the label axis (up to 256 positions), where a block's three
-// hand-over arrays do not fit LDS, and, up to 1024 positions, where the batch would need more
-// workgroups than the device has CUs to spare (one workgroup per utterance is then as good:
-// with that many utterances the planes' traffic holds the walks either way).  Past 1024
+// Blocks of label positions that the alpha and dalpha walks run side by side, one workgroup of
+// `waves` wavefronts (one position a lane) each: four wavefronts, 256 positions, while their
+// three hand-over arrays fit LDS (up to about 12000 anti-diagonals); two wavefronts, 128
+// positions, with their one array up to about 36000.  0 blocks where one workgroup takes the
+// label axis as well or better: up to 256 positions on four wavefronts, up to 128 on two; and,
+// up to 1024 positions, where the batch would need more workgroups than the device has CUs to
+// spare (with that many utterances the planes' traffic holds the walks either way).  Past 1024
 // positions the blocks go side by side whatever the batch: workgroups are dispatched in order,
 // a block after the block it follows, so more workgroups than CUs only queue -- and the other
 // way there, a launch per 1024 positions with sixteen positions a lane, is many times slower.
-int live_blocks(const Dims& d) {
-  const int n = (d.U + 255) / 256;
+int live_blocks(const Dims& d, int* waves) {
+  const size_t one = sizeof(float) * (size_t)d.Dp;
+  const int W = 3 * one <= 144 * 1024 ? 4 : one <= 144 * 1024 ? 2 : 0;
+  if (waves) *waves = W;
+  if (W == 0) return 0;
+  const int n = (d.U + 64 * W - 1) / (64 * W);
   if (n < 2 || n > 16) return 0;
   if (d.B * n > 192 && d.U <= 1024) return 0;
-  if (3 * sizeof(float) * (size_t)d.Dp > 144 * 1024) return 0;
   return n;
 }
 // The two hand-over vectors of the planes hold the walks' tagged 64-bit entries as well: one
 // array of [B][Dp] entries per boundary between live blocks.  In units of [B][Dp] floats each.
 static int hand_arrays(const Dims& d) {
-  const int n = live_blocks(d);
+  const int n = live_blocks(d, nullptr);
   return n > 2 ? n - 1 : 1;
 }
 
@@ -2161,14 +2166,14 @@ __global__ void clear_words_kernel(int* x, int n) {
   if (i < n) x[i] = 0;
 }
 
-// Launches the side-by-side form of a walk (K: its kernel, four wavefronts of one position a
-// lane) for live_blocks(d) blocks: clears the tagged entries, then one workgroup per utterance
-// and block, eight utterances' blocks in consecutive indices.
+// Launches the side-by-side form of a walk (K: its kernel, W wavefronts of one position a lane)
+// for n blocks: clears the tagged entries, then one workgroup per utterance and block, eight
+// utterances' blocks in consecutive indices.
 template <typename K, typename... Args>
-static int launch_live(K kernel, const Planes& p, const Dims& d, int n,
+static int launch_live(K kernel, const Planes& p, const Dims& d, int n, int W,
                        hipStream_t s, Args... args) {
   unsigned long long* live = reinterpret_cast<unsigned long long*>(p.hand[0]);
-  const size_t lds = sizeof(float) * 3 * (size_t)d.Dp;
+  const size_t lds = sizeof(float) * (size_t)(W - 1) * d.Dp;
   const int words = 2 * d.B * d.Dp * (n - 1);
   hipLaunchKernelGGL(clear_words_kernel, dim3((words + 255) / 256), dim3(256), 0, s,
                      reinterpret_cast<int*>(live), words);
@@ -2176,7 +2181,8 @@ static int launch_live(K kernel, const Planes& p, const Dims& d, int n,
   if (lds > 64 * 1024)
     RNNT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-  hipLaunchKernelGGL(kernel, dim3(8 * n * ((d.B + 7) / 8)), dim3(256), lds, s, args..., live, n);
+  hipLaunchKernelGGL(kernel, dim3(8 * n * ((d.B + 7) / 8)), dim3(64 * W), lds, s, args..., live,
+                     n);
   RNNT_LAUNCH_CHECK("lattice walk (blocks side by side)");
   return kOk;
 }
@@ -2195,7 +2201,7 @@ int launch_alpha(const Planes& p, const int* inLen, const int* labLen, float* co
   // 101 positions on two wavefronts take)
   const bool single_block = nblocks == 1;
   const int W = (single_block && cpl >= 4 && 3 * stride * sizeof(float) <= 144 * 1024) ? 4
-                : (cpl >= 2 && stride * sizeof(float) <= 48 * 1024) ? 2 : 1;
+                : (cpl >= 2 && stride * sizeof(float) <= 144 * 1024) ? 2 : 1;
   const size_t lds = W > 1 ? sizeof(float) * (size_t)(W - 1) * stride : 0;
   int* trouble = nullptr;
   RNNT_TRY(trouble_flag(&trouble));
@@ -2204,10 +2210,15 @@ int launch_alpha(const Planes& p, const int* inLen, const int* labLen, float* co
   // (B=8 T=10000, 401 positions: 176 ns a step against 235 on one CU; B=8 T=2000, 513 .. 1024
   // positions: 523 .. 539 ns on one CU with two to four positions a lane; from about a hundred
   // utterances on the planes' traffic holds every form, B=128 T=2000: 241 ns)
-  if (const int n = live_blocks(d))
-    return launch_live(alpha_kernel<1, 4, true, true>, p, d, n, s,
-                       p, inLen, labLen, costs, d, stride, g_spin_limit, trouble, 0,
-                       (const float*)nullptr, (float*)nullptr);
+  int live_w = 0;
+  if (const int n = live_blocks(d, &live_w)) {
+    if (live_w == 4)
+      return launch_live(alpha_kernel<1, 4, true, true>, p, d, n, 4, s, p, inLen, labLen, costs,
+                         d, stride, g_spin_limit, trouble, 0, (const float*)nullptr,
+                         (float*)nullptr);
+    return launch_live(alpha_kernel<1, 2, true, true>, p, d, n, 2, s, p, inLen, labLen, costs, d,
+                       stride, g_spin_limit, trouble, 0, (const float*)nullptr, (float*)nullptr);
+  }
   for (int k = 0; k < nblocks; ++k) {  // lowest block first
     const float* ghin = k == 0 ? nullptr : p.hand[(k - 1) & 1];
     float* ghout = k == nblocks - 1 ? nullptr : p.hand[k & 1];
@@ -2257,16 +2268,21 @@ int launch_beta(const Planes& p, const int* labels, const int* inLen, const int*
   const bool single_block = nblocks == 1;
   const int W = !single_block ? 1
                 : (cpl >= 4 && 3 * stride * sizeof(float) <= 144 * 1024) ? 4
-                : (cpl >= 4 && stride * sizeof(float) <= 48 * 1024) ? 2 : 1;
+                : (cpl >= 4 && stride * sizeof(float) <= 144 * 1024) ? 2 : 1;
   const size_t lds = W > 1 ? sizeof(float) * (size_t)(W - 1) * stride : 0;
   int* trouble = nullptr;
   RNNT_TRY(trouble_flag(&trouble));
   // from 257 label positions in few enough utterances: blocks of 256 positions side by side
   // (as in launch_alpha)
-  if (const int n = live_blocks(d))
-    return launch_live(beta_kernel<1, 4, false, true>, p, d, n, s,
-                       p, labels, inLen, labLen, d, stride, 0, (const float*)nullptr,
-                       (float*)nullptr, g_spin_limit, trouble);
+  int live_w = 0;
+  if (const int n = live_blocks(d, &live_w)) {
+    if (live_w == 4)
+      return launch_live(beta_kernel<1, 4, false, true>, p, d, n, 4, s, p, labels, inLen, labLen,
+                         d, stride, 0, (const float*)nullptr, (float*)nullptr, g_spin_limit,
+                         trouble);
+    return launch_live(beta_kernel<1, 2, false, true>, p, d, n, 2, s, p, labels, inLen, labLen, d,
+                       stride, 0, (const float*)nullptr, (float*)nullptr, g_spin_limit, trouble);
+  }
   for (int k = nblocks - 1; k >= 0; --k) {  // highest block first
     const float* ghin = k == nblocks - 1 ? nullptr : p.hand[(k + 1) & 1];
     float* ghout = k == 0 ? nullptr : p.hand[k & 1];
@@ -2408,7 +2424,7 @@ int launch_viterbi(const Planes& p, const float* bestS, const float* argS,
   const size_t taken_lds = sizeof(int) * (size_t)((d.U + 3) & ~3);
   const int W = (nblocks == 1 && cpl >= 4 &&
                  taken_lds + 3 * stride * sizeof(float) <= 144 * 1024) ? 4
-                : (cpl >= 2 && taken_lds + stride * sizeof(float) <= 48 * 1024) ? 2 : 1;
+                : (cpl >= 2 && taken_lds + stride * sizeof(float) <= 144 * 1024) ? 2 : 1;
   // dynamic LDS: one int per label position, the hand-over arrays between the wavefronts,
   // and the decision columns when they fit (one block only: with several, every block's columns
   // must be there for the backtrace of the last launch)
@@ -2445,6 +2461,10 @@ int launch_viterbi(const Planes& p, const float* bestS, const float* argS,
     break;
 #define CASE_MULTI(C, W)                                                                       \
   case 10000 + C * 100 + W:                                                                    \
+    if (lds > 64 * 1024)                                                                       \
+      RNNT_HIP(hipFuncSetAttribute(                                                            \
+          reinterpret_cast<const void*>(viterbi_kernel<C, W, false, true>),                    \
+          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));                              \
     hipLaunchKernelGGL((viterbi_kernel<C, W, false, true>), dim3(d.B), dim3(64 * W), lds, s,  \
                        p, bestS, argS, inLen, labLen, gcols, labels_out, d, stride, nw,        \
                        g_spin_limit, trouble, u_base, ghin, ghout, traces);                    \
