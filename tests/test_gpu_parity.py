@@ -530,8 +530,11 @@ def test_label_axis_longer_than_one_block_of_1024_positions(T, U, V):
 # ------------------------------------------------------------------ log-normaliser
 @pytest.mark.parametrize("B,T,U,V,sigma", [(2, 70, 9, 31, 1.0), (1, 200, 101, 1000, 2.0),
                                            (3, 129, 130, 257, 1.0), (1, 64, 17, 4099, 3.0),
-                                           (1, 64, 17, 4100, 3.0), (2, 150, 40, 10000, 1.0)])
+                                           (1, 64, 17, 4100, 3.0), (2, 150, 40, 10000, 1.0),
+                                           (70, 500, 9, 33, 1.0), (45, 300, 130, 24, 1.0)])
 def test_log_norms_against_fp64(B, T, U, V, sigma):
+    # (the last two give at least 256 tiles of 128 frames and so take the kernel with tiles of
+    # that height; the smaller grids take tiles of 64 frames)
     cfg = small_config(B, T, U - 1, V, sigma=sigma, ragged=True)
     E, P, labels, il, ll = unpack(make_inputs(cfg, seed=V))
     c = DeviceCase(E, P, labels, il, ll)
