@@ -187,8 +187,12 @@ def test_loss_on_a_side_stream_matches_the_default_stream():
 
 
 # the second shape has 19 slabs of frames on few tiles: the prediction-gradient walk splits over
-# frames there, and its arrival counters must be cleared again inside every replay
-@pytest.mark.parametrize("shape", [(3, 150, 20, 260), (2, 600, 20, 1024)])
+# frames there, and its arrival counters must be cleared again inside every replay; the last two
+# have 300 and 700 labels: the lattice walks run blocks of the label axis side by side, whose
+# tagged entries must be cleared inside every replay too (and the emission gradients of 700
+# labels add up over several launches)
+@pytest.mark.parametrize("shape", [(3, 150, 20, 260), (2, 600, 20, 1024), (2, 150, 300, 40),
+                                   (2, 60, 700, 24)])
 def test_fused_entry_points_replay_from_a_captured_graph(shape):
     """rnnt_hip_loss_forward / rnnt_hip_loss_backward allocate nothing and use kernels only, so
     a caller may capture them; every replay (with eager work and synchronisation in between)
