@@ -401,11 +401,13 @@ def test_label_axis_as_a_chain_of_blocks_side_by_side_and_where_it_is_not(B, T, 
     assert capi.load().rnnt_hip_check_kernels(None) == 0
 
 
-@pytest.mark.parametrize("B,T,U", [(2, 13000, 70), (2, 12500, 200), (1, 20000, 300), (3, 12400, 129)])
+@pytest.mark.parametrize("B,T,U", [(2, 13000, 70), (2, 12500, 200), (1, 20000, 300), (3, 12400, 129),
+                                   (1, 40000, 30), (1, 37000, 150)])
 def test_very_long_utterances_keep_their_wavefronts(B, T, U):
     """Past about 12000 anti-diagonals the three hand-over arrays of four wavefronts no longer fit
     LDS: the walks then deal the label axis to workgroups of two wavefronts (one array, good for
-    36000 anti-diagonals), up to 128 positions one workgroup, beyond blocks of 128 side by side.
+    36000 anti-diagonals), up to 128 positions one workgroup, beyond blocks of 128 side by side;
+    past 36000 anti-diagonals one wavefront per utterance walks the whole label axis.
     The reference's bits and the exact path, as everywhere."""
     cfg = small_config(B, T, U - 1, 4, ragged=True)
     E, P, labels, il, ll = unpack(make_inputs(cfg, seed=T + U))
