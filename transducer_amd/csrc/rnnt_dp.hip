@@ -1707,7 +1707,11 @@ __global__ __launch_bounds__(kMpThreads) void maxplus_kernel(const TIO* __restri
 // afterwards.
 // Dynamic LDS: one int per label position (steps at which labels were taken), the hand-over
 // array (W > 1), the columns (kLdsBits; else they live in global memory).
-template <int C, int W, bool kLdsBits, bool kMulti>
+// kLive (with kMulti, columns in global memory): live_n blocks of 64 C W label positions side by
+// side, one workgroup each, the boundary column's scores crossing in tagged 64-bit entries as in
+// alpha_kernel (same order of workgroups, same bounded waits).  Such a launch only walks; the
+// path is traced by a launch of its own afterwards (traces != 0, u_base past every label).
+template <int C, int W, bool kLdsBits, bool kMulti, bool kLive = false>
 __global__ __launch_bounds__(64 * W) void viterbi_kernel(Planes p, const float* __restrict__ bestS,
                                                          const float* __restrict__ argS,
                                                          const int* __restrict__ inLen,
@@ -1718,11 +1722,20 @@ __global__ __launch_bounds__(64 * W) void viterbi_kernel(Planes p, const float* 
                                                          int* __restrict__ trouble, int u_base,
                                                          const float* __restrict__ ghin,
                                                          float* __restrict__ ghout,
-                                                         int traces) {
+                                                         int traces,
+                                                         unsigned long long* __restrict__ live,
+                                                         int live_n) {
+  static_assert(!kLive || (kMulti && !kLdsBits), "live blocks keep their columns in global memory");
   extern __shared__ __attribute__((aligned(16))) int dyn[];
   __shared__ int done[W];  // steps a wavefront has published
-  const int b = blockIdx.x, lane = threadIdx.x & 63, tidx = threadIdx.x;
+  const int live_block = kLive ? (int)(blockIdx.x >> 3) % live_n : 0;
+  const int b = kLive ? (int)(blockIdx.x / (8 * live_n)) * 8 + (blockIdx.x & 7) : blockIdx.x;
+  const int lane = threadIdx.x & 63, tidx = threadIdx.x;
   const int wave = W > 1 ? __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) : 0;
+  if (kLive) {
+    if (b >= d.B) return;
+    u_base = live_block * 64 * C * W;
+  }
   int Tb, Ub;
   utt_extent(inLen, labLen, b, d.T, d.U, Tb, Ub);
   if (Tb == 0 || Ub == 0) return;  // :152-154
@@ -1733,23 +1746,53 @@ __global__ __launch_bounds__(64 * W) void viterbi_kernel(Planes p, const float* 
   if (!walks && !traces) return;
   const int nsteps = Tb + Ub - 1;
   const int ngroups = (nsteps + 3) >> 2;
-  int* taken = dyn;                                                   // [U rounded up to 4]
-  float* hand = reinterpret_cast<float*>(dyn + ((d.U + 3) & ~3));     // [W-1][hand_stride]
+  int* taken = dyn;                             // [U rounded up to 4] (not in a live launch)
+  float* hand = reinterpret_cast<float*>(dyn + (kLive ? 0 : (d.U + 3) & ~3));  // [W-1][hand_stride]
   unsigned* cols = kLdsBits
       ? reinterpret_cast<unsigned*>(hand + (W - 1) * hand_stride)     // [64 C W][nw]
       : gcols + (size_t)b * d.Ua * nw;                                // [Ua][nw]
-  const float* gin = (kMulti && ghin) ? ghin + (size_t)b * hand_stride : nullptr;
-  float* gout = (kMulti && ghout && walks) ? ghout + (size_t)b * hand_stride : nullptr;
+  const float* gin = (kMulti && !kLive && ghin) ? ghin + (size_t)b * hand_stride : nullptr;
+  float* gout = (kMulti && !kLive && ghout && walks) ? ghout + (size_t)b * hand_stride : nullptr;
   if (kMulti && gout && tidx == 0) gout[0] = kNegInf;  // nothing enters step 0
+  // live blocks: block h reads the entries of boundary h - 1 and writes those of boundary h
+  const bool live_in = kLive && live_block > 0, live_out = kLive && live_block < live_n - 1;
+  const unsigned long long* lrow =
+      kLive ? live + ((size_t)max(live_block - 1, 0) * d.B + b) * hand_stride : nullptr;
+  unsigned long long* lrow_out =
+      kLive ? live + ((size_t)min(live_block, max(live_n - 2, 0)) * d.B + b) * hand_stride
+            : nullptr;
+  auto live_entry = [](int s, float x) -> unsigned long long {
+    return ((unsigned long long)(unsigned)(s + 1) << 32) | (unsigned long long)__float_as_uint(x);
+  };
+  auto live_load = [&](int s) -> unsigned long long {
+    return __hip_atomic_load(lrow + s, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  };
+  // (one opaque statement: see alpha_kernel)
+  auto live_reload = [&](int s) -> unsigned long long {
+    unsigned long long e;
+    const unsigned long long* q = lrow + s;
+    asm volatile("global_load_dwordx2 %0, %1, off sc1\n\ts_waitcnt vmcnt(0)"
+                 : "=&v"(e)
+                 : "v"(q)
+                 : "memory");
+    return e;
+  };
+  unsigned live_sink = 0;
+  if (live_out && tidx == 0)  // nothing enters step 0
+    __hip_atomic_store(lrow_out, live_entry(0, kNegInf), __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
   if (W > 1) {
     if (tidx < W) done[tidx] = 0;
     if (tidx < W - 1) hand[tidx * hand_stride] = kNegInf;  // nothing enters step 0
   }
-  for (int u = tidx; u < Ub; u += 64 * W) taken[u] = -1;
+  if (!kLive)
+    for (int u = tidx; u < Ub; u += 64 * W) taken[u] = -1;
   __syncthreads();
   float* hand_out = hand + wave * hand_stride;                            // wave < W-1
   const float* hand_in = hand + (wave > 0 ? wave - 1 : 0) * hand_stride;  // wave > 0
-  const int u0 = u_base + (wave * 64 + lane) * C;
+  // (a launch that only traces asks for its first groups' operands like any other, and never
+  // uses them: it asks where the lowest block would, inside the arrays)
+  const int u0 = (walks ? u_base : 0) + (wave * 64 + lane) * C;
   // E[t,blank] for the cells of step s sits at ebl[s - u]; column c at step 4g+j reads
   // ebl[4g + j - c], so one run of C+3 values serves all columns of a group
   const float* ebl = p.eb + (size_t)b * d.Tp + d.Eo - u0;
@@ -1774,6 +1817,8 @@ __global__ __launch_bounds__(64 * W) void viterbi_kernel(Planes p, const float* 
     float4 ln[C], bs[C];
     float eb[C + 3];
     float4 gh;  // scores entering the block's first column from the block below
+    unsigned long long lv;  // the same, tagged, from the block running beside this one: lane j
+                            // holds entry 4g + j
   };
   auto load_group = [&](int g) -> Group {
     Group r;
@@ -1787,6 +1832,7 @@ __global__ __launch_bounds__(64 * W) void viterbi_kernel(Planes p, const float* 
     if constexpr (kMulti) {
       r.gh = make_float4(kNegInf, kNegInf, kNegInf, kNegInf);
       if (gin) r.gh = *reinterpret_cast<const float4*>(gin + 4 * g);  // uniform
+      if constexpr (kLive) r.lv = live_load(4 * g + (lane & 3));  // every wavefront asks
     }
     return r;
   };
@@ -1799,6 +1845,29 @@ __global__ __launch_bounds__(64 * W) void viterbi_kernel(Planes p, const float* 
   auto run_group = [&](int g, const Group& cur) {
     float4 hin = {kNegInf, kNegInf, kNegInf, kNegInf};
     if constexpr (kMulti) hin = cur.gh;  // wavefront 0: from the block below (or nothing)
+    if constexpr (kLive) {
+      if (live_in && wave == 0) {  // uniform; as in alpha_kernel
+        unsigned long long e = cur.lv;
+        if (__builtin_amdgcn_ballot_w64(lane < 4 &&
+                                        (unsigned)(e >> 32) != (unsigned)(4 * g + lane + 1))) {
+          const int mine = lane < 4 ? 4 * g + lane : min(4 * ngroups, 4 * (g + kLiveLag));
+          int spins = 0;
+          do {
+            if (spins++ >= spin_limit) {
+              if (lane == 0) raise_trouble(trouble);
+              break;
+            }
+            __builtin_amdgcn_s_sleep(4);
+            e = live_reload(mine);
+          } while (__builtin_amdgcn_ballot_w64((unsigned)(e >> 32) != (unsigned)(mine + 1)));
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          f4set(hin, j, __int_as_float(__builtin_amdgcn_readlane((int)(unsigned)e, j)));
+      } else {
+        live_sink ^= (unsigned)cur.lv;
+      }
+    }
     if (W > 1 && wave > 0) {
       wait_for(4 * g + 3);
       hin = *reinterpret_cast<const float4*>(hand_in + 4 * g);
@@ -1837,6 +1906,14 @@ __global__ __launch_bounds__(64 * W) void viterbi_kernel(Planes p, const float* 
 #pragma unroll
         for (int j = 0; j < 4; ++j) gout[4 * g + 1 + j] = gsend[j];
       }
+      if constexpr (kLive) {
+        if (live_out && wave == W - 1 && lane == 63) {
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            __hip_atomic_store(lrow_out + 4 * g + 1 + j, live_entry(4 * g + 1 + j, gsend[j]),
+                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+      }
     }
     if ((g & 7) == 7 || g == ngroups - 1) {  // uniform: a word of 32 steps is complete
 #pragma unroll
@@ -1854,10 +1931,24 @@ __global__ __launch_bounds__(64 * W) void viterbi_kernel(Planes p, const float* 
   };
   // four register sets rotate (no copies): a group's loads are requested four groups ahead
   auto clamp_g = [&](int g) { return g < ngroups ? g : ngroups - 1; };
+  if constexpr (kLive) {
+    if (live_in && wave == 0) {  // start kLiveLag groups behind the block below (or when it is done)
+      const int far = min(4 * ngroups, 4 * kLiveLag);
+      int spins = 0;
+      while ((unsigned)(live_load(far) >> 32) != (unsigned)(far + 1)) {
+        if (spins++ >= spin_limit) {
+          if (lane == 0) raise_trouble(trouble);
+          break;
+        }
+        __builtin_amdgcn_s_sleep(8);
+      }
+    }
+  }
   Group q0 = load_group(0), q1 = load_group(clamp_g(1)), q2 = load_group(clamp_g(2)),
         q3 = load_group(clamp_g(3));
   const int nwalk = walks ? ngroups : 0;  // a block past the utterance's labels only traces
-  if (W > 1 && wave > 0 && walks) wait_for(min(4 * ngroups, 4 * 8 * wave));  // fall a few groups behind
+  if (W > 1 && wave > 0 && walks)
+    wait_for(min(4 * ngroups, 4 * (kLive ? kLiveWaveLag : 8) * wave));  // fall a few groups behind
   for (int g = 0; g < nwalk; g += 4) {
     run_group(g, q0);
     q0 = load_group(clamp_g(g + 4));
@@ -1867,6 +1958,9 @@ __global__ __launch_bounds__(64 * W) void viterbi_kernel(Planes p, const float* 
     q2 = load_group(clamp_g(g + 6));
     if (g + 3 < ngroups) run_group(g + 3, q3);
     q3 = load_group(clamp_g(g + 7));
+  }
+  if constexpr (kLive) {
+    if (spin_limit < 0 && live_sink == 1u) raise_trouble(trouble);  // never
   }
   if (!kLdsBits) __threadfence();  // the columns in global memory, before another lane reads them
   __syncthreads();
@@ -2438,6 +2532,22 @@ int launch_viterbi(const Planes& p, const float* bestS, const float* argS,
                 stride, lds);
   int* trouble = nullptr;
   RNNT_TRY(trouble_flag(&trouble));
+  // Blocks of 256 label positions side by side where alpha_kernel takes them so (four wavefronts
+  // whose hand-over arrays fit LDS), then one launch that only traces the path (B=8 T=10000
+  // U=400: 1.65 ms for the walk on one CU, four wavefronts of two positions a lane).
+  int live_w = 0;
+  if (const int n = live_blocks(d, &live_w); n && live_w == 4) {
+    RNNT_TRY(launch_live(viterbi_kernel<1, 4, false, true, true>, p, d, n, 4, s, p, bestS, argS,
+                         inLen, labLen, gcols, labels_out, d, stride, nw, g_spin_limit, trouble, 0,
+                         (const float*)nullptr, (float*)nullptr, 0));
+    const size_t trace_lds = sizeof(int) * (size_t)((d.U + 3) & ~3);
+    hipLaunchKernelGGL((viterbi_kernel<1, 1, false, true>), dim3(d.B), dim3(64), trace_lds, s, p,
+                       bestS, argS, inLen, labLen, gcols, labels_out, d, stride, nw, g_spin_limit,
+                       trouble, d.Ua, (const float*)nullptr, (float*)nullptr, 1,
+                       (unsigned long long*)nullptr, 0);
+    RNNT_LAUNCH_CHECK("viterbi_kernel (trace)");
+    return kOk;
+  }
   for (int k = 0; k < nblocks; ++k) {  // lowest block first; the last launch traces the path
     const float* ghin = k == 0 ? nullptr : p.hand[(k - 1) & 1];
     float* ghout = k == nblocks - 1 ? nullptr : p.hand[k & 1];
@@ -2448,7 +2558,7 @@ int launch_viterbi(const Planes& p, const float* bestS, const float* argS,
     if (use_lds)                                                                               \
       hipLaunchKernelGGL((viterbi_kernel<C, W, true, false>), dim3(d.B), dim3(64 * W), lds,   \
                          s, p, bestS, argS, inLen, labLen, gcols, labels_out, d, stride, nw,   \
-                         g_spin_limit, trouble, u_base, ghin, ghout, traces);                  \
+                         g_spin_limit, trouble, u_base, ghin, ghout, traces, nullptr, 0);      \
     else {                                                                                     \
       if (lds > 64 * 1024)                                                                     \
         RNNT_HIP(hipFuncSetAttribute(                                                          \
@@ -2456,7 +2566,7 @@ int launch_viterbi(const Planes& p, const float* bestS, const float* argS,
             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));                            \
       hipLaunchKernelGGL((viterbi_kernel<C, W, false, false>), dim3(d.B), dim3(64 * W), lds,  \
                          s, p, bestS, argS, inLen, labLen, gcols, labels_out, d, stride, nw,   \
-                         g_spin_limit, trouble, u_base, ghin, ghout, traces);                  \
+                         g_spin_limit, trouble, u_base, ghin, ghout, traces, nullptr, 0);      \
     }                                                                                          \
     break;
 #define CASE_MULTI(C, W)                                                                       \
@@ -2467,7 +2577,7 @@ int launch_viterbi(const Planes& p, const float* bestS, const float* argS,
           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));                              \
     hipLaunchKernelGGL((viterbi_kernel<C, W, false, true>), dim3(d.B), dim3(64 * W), lds, s,  \
                        p, bestS, argS, inLen, labLen, gcols, labels_out, d, stride, nw,        \
-                       g_spin_limit, trouble, u_base, ghin, ghout, traces);                    \
+                       g_spin_limit, trouble, u_base, ghin, ghout, traces, nullptr, 0);        \
     break;
       CASE(1, 1) CASE(2, 1) CASE(4, 1) CASE(8, 1) CASE(16, 1)
       CASE(1, 2) CASE(2, 2) CASE(4, 2) CASE(8, 2)
